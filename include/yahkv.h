@@ -1,0 +1,162 @@
+/* yahkv: paged, block-quantized KV cache for one attention layer on one MI355X (gfx950).
+ *
+ * C ABI of the shared library libyahkv.so. Every entry point takes plain pointers and sizes; device
+ * pointers are raw HIP device addresses, `stream` is a hipStream_t passed as void*. Entry points return
+ * 0 on success or a negative yahkv_status; they never throw, never synchronize the device and, except
+ * for yahkv_pagepool_*, never allocate.
+ *
+ * The entry points replace, for this path, the reference engine's kernel dispatches
+ * (LoomDevice::Dispatch, engine/model/loom_runtime.hpp:372-376) issued by LoomDecoder::Step
+ * (engine/model/loom_decoder.hpp:253-268) and by the prefill attention block
+ * (engine/model/loom_prefill.hpp:3341-3410).
+ *
+ * ---------------------------------------------------------------------------------------------
+ * Formats. A block is 32 consecutive head dimensions of one token of one kv head.
+ *   q8_0: f16 scale d, 32 int8 codes, value = d * code   (engine/core/gguf_quant.cpp:72-75,310-320)
+ *   q4_0: f16 scale d, 32 4-bit codes n in 0..15, value = d * (n - 8); byte j of the 16 code bytes holds
+ *         element j in its low nibble and element j + 16 in its high nibble
+ *         (engine/core/gguf_quant.cpp:48-51)
+ *
+ * Pools (the reference keeps codes and scales of K and V in four buffers per layer as well:
+ * LoomDecoderState::kq/ks/vq/vs, engine/model/loom_decoder.hpp:43-51). With PT = page_tokens,
+ * H = n_kv_heads, D = head_dim, NB = D / 32, all arrays C-order, one page after the other:
+ *   q8_0  kq  int8 [n_pages][H][NB][PT][32]   codes of block (token t, block b) are 32 contiguous bytes
+ *         ks  f16  [n_pages][H][PT][NB]
+ *         vq  int8 [n_pages][H][D][PT]        V is stored transposed inside the page (token fastest), as the
+ *                                             reference stores V^T tiles (gen_decode_attn.py:4-6)
+ *         vs  f16  [n_pages][H][NB][PT]
+ *   q4_0  kq  u8   [n_pages][H][NB][PT][16]   the 16 code bytes of a block, ggml nibble order
+ *         ks  f16  [n_pages][H][PT][NB]
+ *         vq  u8   [n_pages][H][NB][16][PT]   byte (b, j, t) = code(t, 32 b + j) | code(t, 32 b + 16 + j) << 4
+ *         vs  f16  [n_pages][H][NB][PT]
+ * The (scale, codes) pairs are bit-identical to the 34-byte / 18-byte ggml blocks; yahkv_gather_blocks
+ * writes them back out in that array-of-blocks form.
+ *
+ * Page table: int32 [n_seqs][page_table_stride], entry [s][p] is the physical page that holds tokens
+ * p * PT .. p * PT + PT - 1 of sequence s (engine/gpu/loom/tools/gen_kvq.py:48-71 for one sequence).
+ * Lengths and positions are device-resident int32 so that steps queue without a host round trip
+ * (engine/model/loom_decoder.hpp:119,131-133,239). Kernels clamp what they read from device memory
+ * (positions to the table's extent, page numbers to the pool) as the reference's do
+ * (gen_decode_attn.py:59-72); validate tables on the host with yahkv_validate_page_table.
+ */
+#ifndef YAHKV_H_
+#define YAHKV_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum yahkv_status {
+  YAHKV_OK = 0,
+  YAHKV_ERR_ARG = -1,        /* null pointer, non-positive count, misaligned pointer */
+  YAHKV_ERR_SHAPE = -2,      /* geometry this build has no kernel for */
+  YAHKV_ERR_PAGE = -3,       /* page table entry outside the pool, or a page used twice */
+  YAHKV_ERR_WORKSPACE = -4,  /* workspace smaller than yahkv_*_workspace_bytes */
+  YAHKV_ERR_NOMEM = -5,      /* page pool exhausted */
+  YAHKV_ERR_LAUNCH = -6      /* the HIP runtime refused the launch */
+} yahkv_status;
+
+/* "kv q KB VB" of the reference's decode.txt (loom_decoder.hpp:76-79): K and V share one format here. */
+typedef enum yahkv_format { YAHKV_Q4_0 = 4, YAHKV_Q8_0 = 8 } yahkv_format;
+typedef enum yahkv_dtype { YAHKV_F32 = 0, YAHKV_F16 = 1, YAHKV_BF16 = 2 } yahkv_dtype;
+
+typedef struct yahkv_geometry {
+  int32_t format;       /* yahkv_format */
+  int32_t n_q_heads;    /* a multiple of n_kv_heads; at most 8 query heads per kv head */
+  int32_t n_kv_heads;
+  int32_t head_dim;     /* 128 or 256 */
+  int32_t page_tokens;  /* 16, 32 or 64 */
+  int32_t n_pages;      /* pages in each of the four pools */
+} yahkv_geometry;
+
+/* Device addresses of one layer's pools, each at least yahkv_*_bytes long and 256-byte aligned. */
+typedef struct yahkv_pools {
+  void* kq;
+  void* ks;
+  void* vq;
+  void* vs;
+} yahkv_pools;
+
+/* Library version string and the gfx target the kernels were compiled for. */
+const char* yahkv_version(void);
+/* Text for a yahkv_status. */
+const char* yahkv_strerror(int status);
+/* 0 if this build has kernels for the geometry, else YAHKV_ERR_SHAPE / YAHKV_ERR_ARG. */
+int yahkv_check_geometry(const yahkv_geometry* g);
+
+/* Pool sizes in bytes. Replace LoomDecoder::KqBytes/KsBytes/VqBytes/VsBytes (loom_decoder.hpp:151-154). */
+size_t yahkv_kq_bytes(const yahkv_geometry* g);
+size_t yahkv_ks_bytes(const yahkv_geometry* g);
+size_t yahkv_vq_bytes(const yahkv_geometry* g);
+size_t yahkv_vs_bytes(const yahkv_geometry* g);
+/* KV bytes one token occupies in the pools (all kv heads, K and V, codes and scales); the figure the
+ * reference's memory plan uses per layer (engine/model/memory_plan.hpp:55). */
+size_t yahkv_bytes_per_token(const yahkv_geometry* g);
+
+/* Host check of a page table before upload: every entry of the first ceil(len[s] / PT) entries of each row
+ * is in [0, n_pages) and no physical page appears twice. Replaces the loop at loom_prefill.hpp:1314-1316.
+ * `table` and `seq_len` are host pointers. */
+int yahkv_validate_page_table(const yahkv_geometry* g, const int32_t* table, int32_t page_table_stride,
+                              const int32_t* seq_len, int32_t n_seqs);
+
+/* Append: quantize `n_new` tokens per sequence and scatter them into their pages.
+ * Token i of sequence s goes to position start_pos[s] + i. k_src / v_src are [n_seqs][n_new][H][D] of
+ * src_dtype (F32, F16 or BF16) on the device. n_valid (device int32 [n_seqs], or NULL for "all n_new")
+ * gives the real rows of a padded chunk: rows at or past n_valid[s] are not written.
+ * Replaces yah_dattn_kappend / yah_dattn_vappend (gen_decode_attn.py:1043-1107, 436-573) for n_new = 1 and
+ * yah_kq8 / yah_vq8 (gen_kvq.py:166-285, 474-660) for a prefill chunk. */
+int yahkv_append(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
+                 int32_t page_table_stride, const int32_t* start_pos, const int32_t* n_valid, int32_t n_seqs,
+                 int32_t n_new, const void* k_src, const void* v_src, int32_t src_dtype, void* stream);
+
+/* Decode attention: one query token per sequence against keys 0 .. seq_len[s] - 1.
+ *   q    [n_seqs][n_q_heads][D] of q_dtype (F16 or BF16)
+ *   gate [n_seqs][n_q_heads][D] f32 or NULL; with a gate, out = ctx * sigmoid(gate) (gen_decode_attn.py:402-407)
+ *   out  [n_seqs][n_q_heads][D] f32
+ * max_seq_len is a host-side upper bound of seq_len[] (it sizes the grid and the workspace); seq_len
+ * values above it are clamped. A sequence of length 0 yields zeros.
+ * Replaces yah_dattn_part_q + yah_dattn_reduce (gen_decode_attn.py:576-1040, 338-411). */
+size_t yahkv_decode_workspace_bytes(const yahkv_geometry* g, int32_t n_seqs, int32_t max_seq_len);
+int yahkv_decode_attend(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
+                        int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs, int32_t max_seq_len,
+                        const void* q, int32_t q_dtype, float softmax_scale, const float* gate, float* out,
+                        void* workspace, size_t workspace_bytes, void* stream);
+
+/* Chunked-prefill attention: query t of sequence s (t < chunk_len) sees keys 0 .. prefix_len[s] + t, which
+ * must already be in the pools (append the chunk first).
+ *   q    [n_seqs][chunk_len][n_q_heads][D] bf16
+ *   out  [n_seqs][chunk_len][n_q_heads][D] bf16
+ * prefix_len is device int32 [n_seqs]; max_prefix_len is its host-side upper bound.
+ * Replaces yah_attn_wmma with its quantized staging (gen_attn_fa.py:1589-1595, 2664-2779). */
+int yahkv_prefill_attend(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
+                         int32_t page_table_stride, const int32_t* prefix_len, int32_t n_seqs,
+                         int32_t max_prefix_len, int32_t chunk_len, const void* q, float softmax_scale,
+                         const float* gate, void* out, void* stream);
+
+/* Gather the blocks of tokens [0, n_tokens) of one sequence back into ggml array-of-blocks order:
+ * dst_k / dst_v are device buffers [n_tokens][H][NB][34 or 18 bytes]. `table_row` is that sequence's row of
+ * the device page table. Test and export helper; shows the pool bytes equal the ggml blocks. */
+int yahkv_gather_blocks(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* table_row,
+                        int32_t n_tokens, void* dst_k, void* dst_v, void* stream);
+
+/* Host page allocator with a free list. The reference has none (its table is the identity,
+ * loom_decoder.hpp:175-179); sequences own pages, freed pages are handed out again, lowest id first. */
+typedef struct yahkv_pagepool yahkv_pagepool;
+yahkv_pagepool* yahkv_pagepool_create(int32_t n_pages);
+void yahkv_pagepool_destroy(yahkv_pagepool* p);
+int32_t yahkv_pagepool_free_count(const yahkv_pagepool* p);
+/* Takes n pages; writes their ids to out. YAHKV_ERR_NOMEM (and takes none) if fewer than n are free. */
+int yahkv_pagepool_alloc(yahkv_pagepool* p, int32_t n, int32_t* out);
+/* Returns n pages. YAHKV_ERR_PAGE (and frees none) if an id is out of range or already free. */
+int yahkv_pagepool_free(yahkv_pagepool* p, const int32_t* pages, int32_t n);
+/* Hands out the free pages in the order of a seeded Fisher-Yates shuffle from now on (tests and benches use
+ * it for a scrambled table, as gen_decode_attn's checker does, dattn_q_check.py:151). */
+void yahkv_pagepool_shuffle(yahkv_pagepool* p, uint64_t seed);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* YAHKV_H_ */

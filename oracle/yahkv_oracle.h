@@ -1,0 +1,91 @@
+/* TEST INFRASTRUCTURE, NOT PRODUCT CODE.
+ *
+ * CPU restatement of the reference's algorithm for the paged quantized KV path. Only tests, the smoke check
+ * and the benchmark's CPU-baseline leg may call it, and only as the checker; the library under test never
+ * links or loads it.
+ *
+ * Pinning status of each function (what proves the restatement is right):
+ *   orc_quantize_q8_0      bit-exact against the reference's own yah::core::QuantizeQ8_0 compiled from its
+ *                          source (oracle/_ref) and against committed golden vectors made with it
+ *   orc_dequantize_q8_0/4_0  bit-exact against the reference's yah::core::Dequantize (oracle/_ref) + golden vectors
+ *   orc_f16 / bf16 conversions  brute force over all 65536 bit patterns and directed f32 cases against numpy
+ *   orc_quantize_q4_0      PARITY UNPINNED against the reference: it has no q4_0 quantizer. Restates ggml's
+ *                          published quantize_row_q4_0_ref (llama.cpp ggml-quants.c, the file
+ *                          engine/core/gguf_quant.cpp:1 cites; not vendored, no version pinned by the
+ *                          reference); checked by invariants only
+ *   orc_append / orc_gather_blocks  page scatter: gather-through-table == contiguous quantize, poison-fill
+ *                          proves untouched bytes, brute force on tiny inputs
+ *   orc_decode_attend      float64 closed-form softmax over dequantized K/V (what
+ *                          engine/gpu/loom/tools/dattn_q_check.py:193-203 does) and special cases
+ *   orc_prefill_attend     same closed form with the causal mask; chunk of 1 == decode
+ */
+#ifndef YAHKV_ORACLE_H_
+#define YAHKV_ORACLE_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct orc_geometry {
+  int32_t format;      /* 8 = q8_0, 4 = q4_0 */
+  int32_t n_q_heads;
+  int32_t n_kv_heads;
+  int32_t head_dim;
+  int32_t page_tokens;
+  int32_t n_pages;
+} orc_geometry;
+
+typedef struct orc_pools {
+  uint8_t* kq;
+  uint16_t* ks;
+  uint8_t* vq;
+  uint16_t* vs;
+} orc_pools;
+
+uint16_t orc_f32_to_f16(float f);
+float orc_f16_to_f32(uint16_t h);
+uint16_t orc_f32_to_bf16(float f);
+float orc_bf16_to_f32(uint16_t h);
+/* element-wise over arrays, for the brute-force tests */
+void orc_f32_to_f16_n(const float* x, uint64_t n, uint16_t* y);
+void orc_f16_to_f32_n(const uint16_t* x, uint64_t n, float* y);
+void orc_f32_to_bf16_n(const float* x, uint64_t n, uint16_t* y);
+void orc_bf16_to_f32_n(const uint16_t* x, uint64_t n, float* y);
+
+/* n elements (a multiple of 32) to 34-byte / 18-byte ggml blocks and back. */
+void orc_quantize_q8_0(const float* x, uint64_t n, uint8_t* dst);
+void orc_quantize_q4_0(const float* x, uint64_t n, uint8_t* dst);
+void orc_dequantize_q8_0(const uint8_t* src, uint64_t n, float* y);
+void orc_dequantize_q4_0(const uint8_t* src, uint64_t n, float* y);
+
+size_t orc_kq_bytes(const orc_geometry* g);
+size_t orc_ks_bytes(const orc_geometry* g);
+size_t orc_vq_bytes(const orc_geometry* g);
+size_t orc_vs_bytes(const orc_geometry* g);
+
+/* k_src / v_src: f32 [n_seqs][n_new][H][D] (f16 / bf16 sources are widened by the caller, which is exact). */
+void orc_append(const orc_geometry* g, const orc_pools* pools, const int32_t* table, int32_t stride,
+                const int32_t* start_pos, const int32_t* n_valid, int32_t n_seqs, int32_t n_new,
+                const float* k_src, const float* v_src);
+/* tokens [0, n_tokens) of one sequence as ggml blocks [n_tokens][H][NB][34|18]. */
+void orc_gather_blocks(const orc_geometry* g, const orc_pools* pools, const int32_t* table_row, int32_t n_tokens,
+                       uint8_t* dst_k, uint8_t* dst_v);
+/* q f32 [n_seqs][n_q_heads][D]; gate f32 or NULL; out f32. */
+void orc_decode_attend(const orc_geometry* g, const orc_pools* pools, const int32_t* table, int32_t stride,
+                       const int32_t* seq_len, int32_t n_seqs, const float* q, float softmax_scale,
+                       const float* gate, float* out);
+/* q f32 [n_seqs][chunk_len][n_q_heads][D]; out f32 same shape. bf16_operands != 0 rounds the dequantized K and V
+ * and the softmax numerators to bf16 before they are multiplied, which is what a bf16 matrix unit sees. */
+void orc_prefill_attend(const orc_geometry* g, const orc_pools* pools, const int32_t* table, int32_t stride,
+                        const int32_t* prefix_len, int32_t n_seqs, int32_t chunk_len, const float* q,
+                        float softmax_scale, const float* gate, float* out, int32_t bf16_operands);
+/* worker threads the attend functions use */
+int32_t orc_threads(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
