@@ -1,0 +1,225 @@
+#!/usr/bin/env python3
+"""Benchmark of the paged q8_0 KV decode step on one MI355X: append one token per sequence, then paged GQA decode
+attention, on the batched ragged configuration (64 sequences, context lengths uniform in [1024, 65536], 24 Q / 4 KV
+heads, head_dim 256, 64-token pages from one shared shuffled pool sized to fit exactly).
+
+Prints ONE JSON line. `value` is the algorithmic KV bytes of a step (sum of context lengths x 2176 B) over the wall
+time of a step with everything resident in HBM; `roofline` is the same bytes over the split-K kernel's own duration,
+measured with HIP events on the launch stream; `cpu_baseline` is the CPU oracle's decode attention on a bounded
+sample of the same sequences, on this box's host cores.
+"""
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+HBM_PEAK_GBS = 8000.0
+
+WORKLOADS = {
+    # name: (format, batch, lo, hi, outlier channels)
+    "ragged_b64_q8_0": dict(fmt=8, batch=64, lo=1024, hi=65536, seed=4),
+    "b1_ctx32k_q8_0": dict(fmt=8, batch=1, lo=32768, hi=32768, seed=4),
+    "b16_ctx128k_q4_0": dict(fmt=4, batch=16, lo=131072, hi=131072, seed=4, outliers=8),
+}
+NQ, NKV, HD, PT = 24, 4, 256, 64
+
+
+def fnv1a(b):
+    h = 0xCBF29CE484222325
+    for x in np.frombuffer(b, np.uint8)[:65536]:
+        h = ((h ^ int(x)) * 0x100000001B3) & 0xFFFFFFFFFFFFFFFF
+    return f"{h:016x}"
+
+
+def build_state(yahkv, torch, wl, total_steps):
+    rng = np.random.default_rng(wl["seed"])
+    lens = rng.integers(wl["lo"], wl["hi"] + 1, wl["batch"]).astype(np.int32)
+    pages = (lens + total_steps + PT - 1) // PT
+    n_pages = int(pages.sum())                       # the pool fits the job exactly
+    g = yahkv.geometry(wl["fmt"], NQ, NKV, HD, PT, n_pages)
+    alloc = yahkv.PagePool(n_pages)
+    alloc.shuffle(12345)
+    table = np.zeros((wl["batch"], int(pages.max())), np.int32)
+    for s, n in enumerate(pages):
+        table[s, :n] = alloc.alloc(int(n))
+    assert alloc.free_count == 0
+    yahkv.validate_page_table(g, table, lens + total_steps)
+    pools = yahkv.DevicePools(g)
+    t_table = torch.from_numpy(table).cuda()
+    gen = torch.Generator(device="cuda").manual_seed(wl["seed"])
+    chunk = 8192
+    outl = None
+    if wl.get("outliers"):
+        outl = torch.ones(NKV, HD, device="cuda")
+        for h in range(NKV):
+            outl[h, torch.from_numpy(rng.permutation(HD)[:wl["outliers"]]).cuda()] = 20.0
+    for s in range(wl["batch"]):                     # fill the prefix through the library's own append
+        for o in range(0, int(lens[s]), chunk):
+            n = min(chunk, int(lens[s]) - o)
+            k = torch.randn((1, n, NKV, HD), generator=gen, device="cuda", dtype=torch.float32)
+            if outl is not None:
+                k = k * outl
+            v = torch.randn((1, n, NKV, HD), generator=gen, device="cuda", dtype=torch.float32)
+            yahkv.append(pools, t_table[s:s + 1], torch.tensor([o], dtype=torch.int32, device="cuda"),
+                         k.to(torch.bfloat16), v.to(torch.bfloat16))
+    torch.cuda.synchronize()
+    return g, pools, lens, table, t_table, gen
+
+
+def parity_check(yahkv, torch, g, pools, t_table, lens, q, out, scale, rows):
+    """Closed-form float64 attention on the library's own gathered blocks, for a few sequences, before timing."""
+    import oracle
+    worst = 0.0
+    for s in rows:
+        n = int(lens[s])
+        k, v = yahkv.gather_blocks(pools, t_table[s], n)
+        bb = k.shape[-1]
+        deq = oracle.dequantize_q8_0 if g.format == 8 else oracle.dequantize_q4_0
+        Kd = deq(k.cpu().numpy().reshape(-1, bb)).reshape(n, NKV, HD).astype(np.float64)
+        Vd = deq(v.cpu().numpy().reshape(-1, bb)).reshape(n, NKV, HD).astype(np.float64)
+        qs = q[s].float().cpu().numpy().astype(np.float64)
+        want = np.zeros((NQ, HD))
+        for h in range(NQ):
+            sc = Kd[:, h // (NQ // NKV)] @ qs[h] * scale
+            p = np.exp(sc - sc.max())
+            want[h] = (p / p.sum()) @ Vd[:, h // (NQ // NKV)]
+        got = out[s].cpu().numpy()
+        worst = max(worst, float(np.abs(got - want).max() / np.abs(want).max()))
+    return worst
+
+
+def cpu_baseline(wl, lens, scale, budget_tokens=150000):
+    """The CPU oracle (a port: the reference has no CPU paged attention) on the first sequences of the batch whose
+    lengths add up to about budget_tokens, all host cores."""
+    import oracle
+    take, tot = [], 0
+    for s, n in enumerate(lens):
+        if take and tot + int(n) > budget_tokens:
+            break
+        take.append(s)
+        tot += int(n)
+    rng = np.random.default_rng(99)
+    sub = lens[take]
+    pages = (sub + PT - 1) // PT
+    g = oracle.geometry(wl["fmt"], NQ, NKV, HD, PT, int(pages.sum()))
+    perm = rng.permutation(g.n_pages).astype(np.int32)
+    table = np.zeros((len(take), int(pages.max())), np.int32)
+    o = 0
+    for i, n in enumerate(pages):
+        table[i, :n] = perm[o:o + n]
+        o += n
+    host = oracle.HostPools(g)
+    t0 = time.perf_counter()
+    for i, n in enumerate(sub):
+        oracle.append(host, table[i:i + 1], [0], None, rng.standard_normal((1, int(n), NKV, HD), np.float32),
+                      rng.standard_normal((1, int(n), NKV, HD), np.float32))
+    t_quant = time.perf_counter() - t0
+    q = rng.standard_normal((len(take), NQ, HD)).astype(np.float32)
+    oracle.decode_attend(host, table, sub, q, scale)          # warm-up
+    times = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        oracle.decode_attend(host, table, sub, q, scale)
+        times.append(time.perf_counter() - t0)
+    t = float(np.median(times))
+    bpt = 2 * NKV * (HD // 32) * ((32 if wl["fmt"] == 8 else 16) + 2)
+    return {"value": round(tot * bpt / t / 1e9, 3), "unit": "GB/s", "cores": oracle.threads(), "kind": "port",
+            "sample": f"oracle decode attention on the first {len(take)} sequences of the batch ({tot} tokens, "
+                      f"{tot * bpt / 1e6:.0f} MB of KV), median of 3 after a warm-up",
+            "tok_per_s": round(len(take) / t, 2),
+            "append_blocks_per_s": round(tot * 2 * NKV * (HD // 32) / t_quant, 0),
+            "append_note": "oracle scalar block quantizer + page scatter, 1 thread"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="ragged_b64_q8_0", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        raise SystemExit("bench.py: this build runs on ONE GPU (the path has no cross-GPU exchange); use --gpus 1")
+    import torch
+    yahkv = importlib.import_module("yet-another-halo-engine_amd")
+    torch.cuda.set_device(0)
+    wl = WORKLOADS[a.workload]
+    total = a.warmup + a.steps + 1
+    g, pools, lens, table, t_table, gen = build_state(yahkv, torch, wl, total)
+    B = wl["batch"]
+    scale = 1.0 / float(np.sqrt(HD))
+    max_len = int(lens.max()) + total
+    seq_len = torch.from_numpy(lens.copy()).cuda()
+    q = torch.randn((B, NQ, HD), generator=gen, device="cuda").to(torch.bfloat16)
+    knew = torch.randn((total, B, 1, NKV, HD), generator=gen, device="cuda").to(torch.bfloat16)
+    vnew = torch.randn((total, B, 1, NKV, HD), generator=gen, device="cuda").to(torch.bfloat16)
+    out = torch.empty((B, NQ, HD), dtype=torch.float32, device="cuda")
+    ws = torch.empty(yahkv.decode_workspace_bytes(g, B, max_len), dtype=torch.uint8, device="cuda")
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(a.steps)]
+
+    def step(i, pair=None):
+        yahkv.append(pools, t_table, seq_len, knew[i], vnew[i])       # position = current length (device-resident)
+        seq_len.add_(1)
+        if pair:
+            pair[0].record()
+        yahkv.decode_part(pools, t_table, seq_len, max_len, q, scale, ws)
+        if pair:
+            pair[1].record()
+        yahkv.decode_reduce(g, t_table.shape[1], seq_len, B, max_len, out, ws)
+
+    # parity before timing: first step, a few sequences against the float64 closed form
+    step(0)
+    torch.cuda.synchronize()
+    first_hash = fnv1a(out.cpu().numpy().tobytes())
+    order = np.argsort(lens)
+    rows = [int(order[0]), int(order[len(order) // 4])] if B > 1 else [0]
+    err = parity_check(yahkv, torch, g, pools, t_table, lens + 1, q, out, scale, rows)
+    if not err < 2e-3:
+        raise SystemExit(f"bench.py: parity check failed before timing: max relative error {err:.3e}")
+
+    for i in range(a.warmup):
+        step(1 + i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(a.steps):
+        step(1 + a.warmup + i, ev[i])
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+
+    bpt = yahkv.lib.yahkv_bytes_per_token(g)
+    # context lengths seen by timed step i: lens + 1 (parity step) + warmup + i + 1
+    tokens = [int(lens.sum()) + B * (2 + a.warmup + i) for i in range(a.steps)]
+    kv_bytes = float(np.mean(tokens)) * bpt
+    ms = dt / a.steps * 1e3
+    kern_ms = float(np.mean([p[0].elapsed_time(p[1]) for p in ev]))
+    gbs = kv_bytes / (ms * 1e-3) / 1e9
+    kgbs = kv_bytes / (kern_ms * 1e-3) / 1e9
+    res = {
+        "metric": "paged q8 KV decode-attn HBM GB/s (% of peak) + tok/s, B=64 ragged ctx",
+        "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "u8" if wl["fmt"] == 8 else "u4", "data": "synthetic",
+        "config": {"workload": a.workload, "batch": B, "ctx_min": int(lens.min()), "ctx_max": int(lens.max()),
+                   "ctx_sum": int(lens.sum()), "n_q_heads": NQ, "n_kv_heads": NKV, "head_dim": HD, "page_tokens": PT,
+                   "n_pages": g.n_pages, "kv_format": "q8_0" if wl["fmt"] == 8 else "q4_0",
+                   "step": "append 1 token/seq + paged decode attention"},
+        "pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2), "tok_per_s": round(B / (ms * 1e-3), 1),
+        "kv_bytes_per_step": int(kv_bytes), "parity_max_rel_err": float(f"{err:.3e}"), "out_fnv1a": first_hash,
+        "roofline": {"bound": "hbm", "achieved": round(kgbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(kgbs / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "DattnPart",
+                     "kernel_ms": round(kern_ms, 4)},
+    }
+    if not a.no_cpu_baseline:
+        res["cpu_baseline"] = cpu_baseline(wl, lens, scale)
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

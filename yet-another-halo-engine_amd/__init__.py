@@ -1,0 +1,248 @@
+"""Python binding of libyahkv.so (the C ABI of include/yahkv.h) for tests and benchmarks.
+
+PyTorch only provides device memory and streams here: every call passes raw device pointers and torch's current HIP
+stream to the library. There is no CPU fallback: without the built library the import fails.
+"""
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libyahkv.so")
+
+Q8_0, Q4_0 = 8, 4
+F32, F16, BF16 = 0, 1, 2
+
+
+class YahkvError(RuntimeError):
+    def __init__(self, status, what):
+        super().__init__(f"{what}: {status_text(status)} ({status})")
+        self.status = status
+
+
+class Geometry(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in ("format", "n_q_heads", "n_kv_heads", "head_dim", "page_tokens", "n_pages")]
+
+
+class Pools(C.Structure):
+    _fields_ = [("kq", C.c_void_p), ("ks", C.c_void_p), ("vq", C.c_void_p), ("vs", C.c_void_p)]
+
+
+def _load():
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(f"{LIB_PATH} is not built: run `python __graft_entry__.py build` (hipcc, gfx950)")
+    # torch ships its own HIP runtime (same soname as /opt/rocm's). It must be in the process first, so that the
+    # library binds to that one: two runtimes in one process do not share streams or device memory.
+    import torch  # noqa: F401
+    lib = C.CDLL(LIB_PATH)
+    G, P, vp, i32, i32p = C.POINTER(Geometry), C.POINTER(Pools), C.c_void_p, C.c_int32, C.c_void_p
+    lib.yahkv_version.restype = C.c_char_p
+    lib.yahkv_strerror.restype = C.c_char_p
+    lib.yahkv_strerror.argtypes = [C.c_int]
+    lib.yahkv_check_geometry.argtypes = [G]
+    for n in ("yahkv_kq_bytes", "yahkv_ks_bytes", "yahkv_vq_bytes", "yahkv_vs_bytes", "yahkv_bytes_per_token"):
+        getattr(lib, n).restype = C.c_size_t
+        getattr(lib, n).argtypes = [G]
+    lib.yahkv_validate_page_table.argtypes = [G, i32p, i32, i32p, i32]
+    lib.yahkv_append.argtypes = [G, P, i32p, i32, i32p, i32p, i32, i32, vp, vp, i32, vp]
+    lib.yahkv_decode_workspace_bytes.restype = C.c_size_t
+    lib.yahkv_decode_workspace_bytes.argtypes = [G, i32, i32]
+    lib.yahkv_decode_part.argtypes = [G, P, i32p, i32, i32p, i32, i32, vp, i32, C.c_float, vp, C.c_size_t, vp]
+    lib.yahkv_decode_reduce.argtypes = [G, i32, i32p, i32, i32, vp, vp, vp, C.c_size_t, vp]
+    lib.yahkv_decode_attend.argtypes = [G, P, i32p, i32, i32p, i32, i32, vp, i32, C.c_float, vp, vp, vp, C.c_size_t, vp]
+    if hasattr(lib, "yahkv_prefill_attend"):
+        lib.yahkv_prefill_attend.argtypes = [G, P, i32p, i32, i32p, i32, i32, i32, vp, C.c_float, vp, vp, vp]
+    lib.yahkv_gather_blocks.argtypes = [G, P, i32p, i32, vp, vp, vp]
+    lib.yahkv_pagepool_create.restype = C.c_void_p
+    lib.yahkv_pagepool_create.argtypes = [i32]
+    lib.yahkv_pagepool_destroy.argtypes = [vp]
+    lib.yahkv_pagepool_free_count.argtypes = [vp]
+    lib.yahkv_pagepool_alloc.argtypes = [vp, i32, i32p]
+    lib.yahkv_pagepool_free.argtypes = [vp, i32p, i32]
+    lib.yahkv_pagepool_shuffle.argtypes = [vp, C.c_uint64]
+    return lib
+
+
+lib = _load()
+
+
+def status_text(status):
+    return lib.yahkv_strerror(int(status)).decode()
+
+
+def _check(status, what):
+    if status != 0:
+        raise YahkvError(status, what)
+
+
+def geometry(fmt, n_q_heads, n_kv_heads, head_dim, page_tokens, n_pages):
+    g = Geometry(fmt, n_q_heads, n_kv_heads, head_dim, page_tokens, n_pages)
+    _check(lib.yahkv_check_geometry(C.byref(g)), "geometry")
+    return g
+
+
+def pool_bytes(g):
+    r = C.byref(g)
+    return {"kq": lib.yahkv_kq_bytes(r), "ks": lib.yahkv_ks_bytes(r), "vq": lib.yahkv_vq_bytes(r),
+            "vs": lib.yahkv_vs_bytes(r)}
+
+
+def validate_page_table(g, table, seq_len):
+    """table: numpy int32 [n_seqs][stride]; seq_len: numpy int32 [n_seqs]. Raises YahkvError on a bad table."""
+    import numpy as np
+    table = np.ascontiguousarray(table, np.int32)
+    seq_len = np.ascontiguousarray(seq_len, np.int32)
+    _check(lib.yahkv_validate_page_table(C.byref(g), table.ctypes.data, table.shape[1], seq_len.ctypes.data,
+                                         len(seq_len)), "page table")
+
+
+class PagePool:
+    """Host page allocator with a free list (yahkv_pagepool_*)."""
+
+    def __init__(self, n_pages):
+        self._p = lib.yahkv_pagepool_create(n_pages)
+        if not self._p:
+            raise YahkvError(-1, "pagepool_create")
+
+    def close(self):
+        if self._p:
+            lib.yahkv_pagepool_destroy(self._p)
+            self._p = None
+
+    __del__ = close
+
+    @property
+    def free_count(self):
+        return lib.yahkv_pagepool_free_count(self._p)
+
+    def alloc(self, n):
+        out = (C.c_int32 * max(n, 1))()
+        _check(lib.yahkv_pagepool_alloc(self._p, n, C.cast(out, C.c_void_p)), "pagepool_alloc")
+        return list(out[:n])
+
+    def free(self, pages):
+        arr = (C.c_int32 * max(len(pages), 1))(*pages)
+        _check(lib.yahkv_pagepool_free(self._p, C.cast(arr, C.c_void_p), len(pages)), "pagepool_free")
+
+    def shuffle(self, seed):
+        lib.yahkv_pagepool_shuffle(self._p, seed)
+
+
+# ---- device side (torch supplies memory and the stream) --------------------------------------------------------------
+
+def _stream():
+    import torch
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _dp(t):
+    return None if t is None else C.c_void_p(t.data_ptr())
+
+
+def _dtype_code(t):
+    import torch
+    return {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}[t.dtype]
+
+
+class DevicePools:
+    """One layer's four pools on the GPU (LoomDecoderState's kq / ks / vq / vs)."""
+
+    def __init__(self, g, fill=0, device="cuda:0"):
+        import torch
+        self.geom = g
+        b = pool_bytes(g)
+        self.kq = torch.full((b["kq"],), fill, dtype=torch.uint8, device=device)
+        self.ks = torch.full((b["ks"],), fill, dtype=torch.uint8, device=device)
+        self.vq = torch.full((b["vq"],), fill, dtype=torch.uint8, device=device)
+        self.vs = torch.full((b["vs"],), fill, dtype=torch.uint8, device=device)
+
+    def struct(self):
+        return Pools(self.kq.data_ptr(), self.ks.data_ptr(), self.vq.data_ptr(), self.vs.data_ptr())
+
+    def numpy(self):
+        import numpy as np
+        return {"kq": self.kq.cpu().numpy(), "ks": self.ks.cpu().numpy().view(np.uint16),
+                "vq": self.vq.cpu().numpy(), "vs": self.vs.cpu().numpy().view(np.uint16)}
+
+    def load(self, arrays):
+        """Upload host pools (numpy arrays keyed kq / ks / vq / vs)."""
+        import numpy as np
+        import torch
+        for name in ("kq", "ks", "vq", "vs"):
+            src = torch.from_numpy(np.ascontiguousarray(arrays[name]).view(np.uint8).reshape(-1))
+            getattr(self, name).copy_(src)
+
+
+def append(pools, table, start_pos, k_src, v_src, n_valid=None):
+    """k_src / v_src: [n_seqs][n_new][H][D] f32 / f16 / bf16 cuda tensors; table int32 [n_seqs][stride]."""
+    g = pools.geom
+    assert k_src.is_contiguous() and v_src.is_contiguous() and table.is_contiguous() and k_src.dtype == v_src.dtype
+    n_seqs, n_new = k_src.shape[0], k_src.shape[1]
+    assert tuple(k_src.shape) == (n_seqs, n_new, g.n_kv_heads, g.head_dim) and k_src.shape == v_src.shape
+    st = pools.struct()
+    _check(lib.yahkv_append(C.byref(g), C.byref(st), _dp(table), table.shape[1], _dp(start_pos), _dp(n_valid),
+                            n_seqs, n_new, _dp(k_src), _dp(v_src), _dtype_code(k_src), _stream()), "append")
+
+
+def decode_workspace_bytes(g, n_seqs, max_seq_len):
+    return lib.yahkv_decode_workspace_bytes(C.byref(g), n_seqs, max_seq_len)
+
+
+def decode_attend(pools, table, seq_len, max_seq_len, q, scale, gate=None, out=None, workspace=None):
+    """q: [n_seqs][n_q_heads][D] f16 / bf16 / f32; returns out f32 of the same shape."""
+    import torch
+    g = pools.geom
+    n_seqs = q.shape[0]
+    assert q.is_contiguous() and table.is_contiguous() and tuple(q.shape) == (n_seqs, g.n_q_heads, g.head_dim)
+    if out is None:
+        out = torch.empty(q.shape, dtype=torch.float32, device=q.device)
+    need = decode_workspace_bytes(g, n_seqs, max_seq_len)
+    if workspace is None:
+        workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
+    st = pools.struct()
+    _check(lib.yahkv_decode_attend(C.byref(g), C.byref(st), _dp(table), table.shape[1], _dp(seq_len), n_seqs,
+                                   max_seq_len, _dp(q), _dtype_code(q), scale, _dp(gate), _dp(out), _dp(workspace),
+                                   workspace.numel(), _stream()), "decode_attend")
+    return out
+
+
+def decode_part(pools, table, seq_len, max_seq_len, q, scale, workspace):
+    """First dispatch of decode_attend: partials into the workspace."""
+    g = pools.geom
+    st = pools.struct()
+    _check(lib.yahkv_decode_part(C.byref(g), C.byref(st), _dp(table), table.shape[1], _dp(seq_len), q.shape[0],
+                                 max_seq_len, _dp(q), _dtype_code(q), scale, _dp(workspace), workspace.numel(),
+                                 _stream()), "decode_part")
+
+
+def decode_reduce(g, table_stride, seq_len, n_seqs, max_seq_len, out, workspace, gate=None):
+    """Second dispatch of decode_attend: merge the partials into out."""
+    _check(lib.yahkv_decode_reduce(C.byref(g), table_stride, _dp(seq_len), n_seqs, max_seq_len, _dp(gate), _dp(out),
+                                   _dp(workspace), workspace.numel(), _stream()), "decode_reduce")
+
+
+def prefill_attend(pools, table, prefix_len, max_prefix_len, q, scale, gate=None, out=None):
+    """q: [n_seqs][chunk][n_q_heads][D] bf16; returns out bf16 of the same shape."""
+    import torch
+    g = pools.geom
+    assert q.is_contiguous() and q.dtype == torch.bfloat16
+    if out is None:
+        out = torch.empty_like(q)
+    st = pools.struct()
+    _check(lib.yahkv_prefill_attend(C.byref(g), C.byref(st), _dp(table), table.shape[1], _dp(prefix_len), q.shape[0],
+                                    max_prefix_len, q.shape[1], _dp(q), scale, _dp(gate), _dp(out), _stream()),
+           "prefill_attend")
+    return out
+
+
+def gather_blocks(pools, table_row, n_tokens):
+    """Blocks of tokens [0, n_tokens) of one sequence in ggml order: two uint8 tensors [n][H][NB][34 | 18]."""
+    import torch
+    g = pools.geom
+    bb = 34 if g.format == Q8_0 else 18
+    shape = (n_tokens, g.n_kv_heads, g.head_dim // 32, bb)
+    k = torch.zeros(shape, dtype=torch.uint8, device=table_row.device)
+    v = torch.zeros(shape, dtype=torch.uint8, device=table_row.device)
+    st = pools.struct()
+    _check(lib.yahkv_gather_blocks(C.byref(g), C.byref(st), _dp(table_row), n_tokens, _dp(k), _dp(v), _stream()),
+           "gather_blocks")
+    return k, v
