@@ -1,11 +1,17 @@
-// Paged GQA decode attention over block-quantized K/V: split-K over 64-token tiles, then a merge.
+// Paged GQA decode attention over block-quantized K/V: split-K over slices of the context, then a merge.
 //
 // Structure follows the reference's decode attention (engine/gpu/loom/tools/gen_decode_attn.py): `part` computes one
 // partial (M, l, acc) per slice of the context for the query heads of one kv head (:97-335, quantized :576-1040),
 // `reduce` merges the partials: out = (sum_s e^(M_s - M) acc_s) / (sum_s e^(M_s - M) l_s) * sigmoid(gate) (:338-411).
 // Keys at or past the sequence length are masked (key < pos + 1, :145,167); the "minus infinity" is the finite
 // -FLT_MAX the reference uses (:357), so that no inf - inf can appear.
+//
+// The reference launches one workgroup per 256-key page of its single sequence. Here lengths are ragged and live on
+// the device, so a small `plan` kernel first cuts every sequence into items of equal size (a run of 64-key tiles) and
+// writes one record per item; `part` runs one wavefront per (item, kv head). Equal items keep 256 CUs evenly loaded
+// whatever the mix of lengths, and no workgroup is launched for work that does not exist except at the grid's end.
 #include <algorithm>
+#include <cstdlib>
 
 #include "common.hpp"
 
@@ -13,9 +19,9 @@ namespace yahkv {
 namespace {
 
 constexpr float kNegMax = -3.4028234663852886e+38f;
-constexpr int kTile = 64;     // tokens per tile: one wavefront, one token per lane in the score phase
-constexpr int kWaves = 4;
+constexpr int kTile = 64;     // keys per tile: one wavefront, one key per lane in the score phase
 constexpr int kMaxGroup = 8;  // query heads per kv head
+constexpr int kPlanThreads = 256;
 
 struct DecodeArgs {
   Geom g;
@@ -23,16 +29,71 @@ struct DecodeArgs {
   const int32_t* table;
   int32_t stride;
   const int32_t* seq_len;
-  int32_t n_seqs, max_len;  // max_len already clamped to stride * PT
+  int32_t n_seqs, max_len;  // max_len: host bound, already clamped to stride * PT
   const void* q;
   int32_t q_dtype;
   float scale;
   const float* gate;
   float* out;
-  float* acc;  // [n_seqs][H][n_splits][G][D]
-  float* ml;   // [n_seqs][H][n_splits][G][2]
-  int32_t n_splits, tiles_per_split;
+  // workspace
+  int32_t* header;   // [0] chunks in use, [1] tiles per item
+  int32_t* prefix;   // [n_seqs + 1] first chunk of each sequence
+  int4* items;       // [max_chunks] {sequence or -1, first tile, end tile, length}
+  float* ml;         // [max_chunks * H][G][2]
+  float* acc;        // [max_chunks * H][G][D]
+  int32_t max_chunks, min_tiles_per_item, target_items;
 };
+
+// ---- plan -------------------------------------------------------------------------------------------------------------
+
+// One workgroup. Reads the lengths, picks the item size (tiles per item: at least the host's lower bound, which sized
+// the workspace, and large enough that there are about target_items items), and writes prefix[] and items[].
+__global__ __launch_bounds__(kPlanThreads) void DattnPlan(const DecodeArgs a) {
+  __shared__ int part_sum[kPlanThreads];
+  __shared__ int tpi_s;
+  const int t = threadIdx.x;
+  const int per = (a.n_seqs + kPlanThreads - 1) / kPlanThreads;
+  const int s0 = min(t * per, a.n_seqs), s1 = min(s0 + per, a.n_seqs);
+  auto tiles_of = [&](int s) { return (min(max(a.seq_len[s], 0), a.max_len) + kTile - 1) / kTile; };
+  int sum = 0;
+  for (int s = s0; s < s1; ++s) sum += tiles_of(s);
+  part_sum[t] = sum;
+  __syncthreads();
+  if (t == 0) {
+    long long total = 0;
+    for (int i = 0; i < kPlanThreads; ++i) total += part_sum[i];
+    const long long want = (total * a.g.n_kv + a.target_items - 1) / a.target_items;
+    tpi_s = static_cast<int>(max(static_cast<long long>(a.min_tiles_per_item), want));
+  }
+  __syncthreads();
+  const int tpi = tpi_s;
+  sum = 0;
+  for (int s = s0; s < s1; ++s) sum += (tiles_of(s) + tpi - 1) / tpi;
+  __syncthreads();
+  part_sum[t] = sum;
+  __syncthreads();
+  int base = 0;
+  for (int i = 0; i < t; ++i) base += part_sum[i];
+  for (int s = s0; s < s1; ++s) {
+    const int len = min(max(a.seq_len[s], 0), a.max_len), nt = (len + kTile - 1) / kTile;
+    const int nc = (nt + tpi - 1) / tpi;
+    a.prefix[s] = base;
+    for (int c = 0; c < nc; ++c)
+      if (base + c < a.max_chunks) a.items[base + c] = int4{s, c * tpi, min(c * tpi + tpi, nt), len};
+    base += nc;
+  }
+  if (t == kPlanThreads - 1) {
+    a.prefix[a.n_seqs] = base;
+    a.header[0] = min(base, a.max_chunks);
+    a.header[1] = tpi;
+  }
+  __syncthreads();
+  int total = 0;
+  for (int i = 0; i < kPlanThreads; ++i) total += part_sum[i];
+  for (int c = total + t; c < a.max_chunks; c += kPlanThreads) a.items[c] = int4{-1, 0, 0, 0};  // unused records
+}
+
+// ---- shared pieces ----------------------------------------------------------------------------------------------------
 
 __device__ __forceinline__ float WaveMax(float v) {
 #pragma unroll
@@ -44,39 +105,44 @@ __device__ __forceinline__ float WaveSum(float v) {
   for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
   return v;
 }
+__device__ __forceinline__ float HalfMax32(float v) {  // over the 32 lanes of a wave half
+#pragma unroll
+  for (int o = 16; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+__device__ __forceinline__ float HalfSum32(float v) {
+#pragma unroll
+  for (int o = 16; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
 
-// Dimension k (< D / 64) of lane `lane`: q8_0 keeps a lane's dims contiguous; q4_0 pairs dim j with j + 16 of a block
-// because one V byte holds both.
-template <int FMT>
-__device__ __forceinline__ int LaneDim(int lane, int k, int dpl) {
-  if (FMT == 8) return lane * dpl + k;
+// ---- q4_0: scalar-ALU part ----------------------------------------------------------------------------------------------
+
+// Dimension k (< D / 64) of lane `lane`: dim j is paired with j + 16 of its block because one V byte holds both.
+__device__ __forceinline__ int LaneDimQ4(int lane, int k, int dpl) {
   const int pair = lane * (dpl / 2) + k / 2;
   return (pair / 16) * 32 + pair % 16 + 16 * (k & 1);
 }
 
-// One workgroup per (split, kv head, sequence); wave w takes tiles split * tps + w, + 4, ... A lane owns one token for
-// the scores and D / 64 dims for P.V. G query heads share every K and V byte read.
-template <int FMT, int D>
-__global__ __launch_bounds__(256) void DattnPartScalar(const DecodeArgs a) {
-  constexpr int NB = D / 32, DPL = D / 64, CB = FMT == 8 ? 32 : 16;
+// One wavefront per (item, kv head). A lane owns one key for the scores and D / 64 dims for P.V.
+template <int D>
+__global__ __launch_bounds__(64) void DattnPartQ4(const DecodeArgs a) {
+  constexpr int NB = D / 32, DPL = D / 64, CB = 16;
   const Geom g = a.g;
   const int G = g.group(), H = g.n_kv, PT = g.pt;
-  const int s = blockIdx.z, h = blockIdx.y, split = blockIdx.x;
-  const int len = min(max(a.seq_len[s], 0), a.max_len);
-  const int n_tiles = (len + kTile - 1) / kTile;
-  const int tile0 = split * a.tiles_per_split;
-  if (tile0 >= n_tiles) return;
-  const int tile1 = min(tile0 + a.tiles_per_split, n_tiles);
-  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  const int item = blockIdx.x, h = item % H;
+  const int4 rec = a.items[item / H];
+  if (rec.x < 0) return;
+  const int s = rec.x, tile0 = rec.y, tile1 = rec.z, len = rec.w;
+  const int lane = threadIdx.x;
 
   __shared__ float qs[kMaxGroup][D];
-  __shared__ float ps[kWaves][kMaxGroup][kTile];
-  __shared__ float wm[kWaves][kMaxGroup], wl[kWaves][kMaxGroup];
-  __shared__ float wacc[kWaves][kMaxGroup][D];
-
-  for (int i = threadIdx.x; i < G * D; i += 256)
+  __shared__ float ps[kMaxGroup][kTile];
+  for (int i = lane; i < G * D; i += 64)
     qs[i / D][i % D] = LoadSrc(a.q, (size_t(s) * g.n_q + size_t(h) * G) * D + i, a.q_dtype);
-  __syncthreads();
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
   float m[kMaxGroup], l[kMaxGroup], acc[kMaxGroup][DPL];
 #pragma unroll
@@ -87,8 +153,7 @@ __global__ __launch_bounds__(256) void DattnPartScalar(const DecodeArgs a) {
   }
   const int32_t* row = a.table + int64_t(s) * a.stride;
 
-  for (int tile = tile0 + wave; tile < tile1; tile += kWaves) {
-    // ---- scores: lane = token
+  for (int tile = tile0; tile < tile1; ++tile) {
     const int tok = tile * kTile + lane;
     const bool valid = tok < len;
     float sc[kMaxGroup];
@@ -99,38 +164,26 @@ __global__ __launch_bounds__(256) void DattnPartScalar(const DecodeArgs a) {
       const int t = tok % PT;
       for (int b = 0; b < NB; ++b) {
         const float d = WidenF16(a.pools.ks[(ph * PT + t) * NB + b]);
-        const uint4* cp = reinterpret_cast<const uint4*>(a.pools.kq + ((ph * NB + b) * PT + t) * CB);
+        const uint4 v = *reinterpret_cast<const uint4*>(a.pools.kq + ((ph * NB + b) * PT + t) * CB);
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
         float part[kMaxGroup];
 #pragma unroll
         for (int gi = 0; gi < kMaxGroup; ++gi) part[gi] = 0.0f;
 #pragma unroll
-        for (int c = 0; c < CB / 16; ++c) {
-          const uint4 v = cp[c];
-          const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+        for (int j = 0; j < 16; ++j) {
+          const uint32_t byte = (w[j / 4] >> (8 * (j % 4))) & 0xFF;
+          const float x0 = static_cast<float>(int(byte & 0xF) - 8), x1 = static_cast<float>(int(byte >> 4) - 8);
 #pragma unroll
-          for (int j = 0; j < 16; ++j) {
-            const uint32_t byte = (w[j / 4] >> (8 * (j % 4))) & 0xFF;
-            if (FMT == 8) {
-              const float x = static_cast<float>(static_cast<int8_t>(byte));
-#pragma unroll
-              for (int gi = 0; gi < kMaxGroup; ++gi)
-                if (gi < G) part[gi] = __builtin_fmaf(qs[gi][b * 32 + c * 16 + j], x, part[gi]);
-            } else {
-              const float x0 = static_cast<float>(int(byte & 0xF) - 8), x1 = static_cast<float>(int(byte >> 4) - 8);
-#pragma unroll
-              for (int gi = 0; gi < kMaxGroup; ++gi)
-                if (gi < G) {
-                  part[gi] = __builtin_fmaf(qs[gi][b * 32 + j], x0, part[gi]);
-                  part[gi] = __builtin_fmaf(qs[gi][b * 32 + 16 + j], x1, part[gi]);
-                }
+          for (int gi = 0; gi < kMaxGroup; ++gi)
+            if (gi < G) {
+              part[gi] = __builtin_fmaf(qs[gi][b * 32 + j], x0, part[gi]);
+              part[gi] = __builtin_fmaf(qs[gi][b * 32 + 16 + j], x1, part[gi]);
             }
-          }
         }
 #pragma unroll
         for (int gi = 0; gi < kMaxGroup; ++gi) sc[gi] = __builtin_fmaf(d, part[gi], sc[gi]);
       }
     }
-    // ---- online softmax per head, across the wave's 64 tokens
 #pragma unroll
     for (int gi = 0; gi < kMaxGroup; ++gi) {
       if (gi < G) {
@@ -142,74 +195,48 @@ __global__ __launch_bounds__(256) void DattnPartScalar(const DecodeArgs a) {
 #pragma unroll
         for (int k = 0; k < DPL; ++k) acc[gi][k] *= alpha;
         m[gi] = mn;
-        ps[wave][gi][lane] = p;
+        ps[gi][lane] = p;
       }
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    // ---- P.V: lane = D / 64 dims, loop over the tile's pages and tokens
     for (int sp = 0; sp < kTile / PT; ++sp) {
       const int base = tile * kTile + sp * PT;
       if (base >= len) break;
       const int nt = min(PT, len - base);
       const size_t ph = size_t(ClampPage(row[base / PT], g.n_pages)) * H + h;
 #pragma unroll
-      for (int k = 0; k < DPL; k += (FMT == 8 ? 1 : 2)) {
-        const int d0 = LaneDim<FMT>(lane, k, DPL);
+      for (int k = 0; k < DPL; k += 2) {
+        const int d0 = LaneDimQ4(lane, k, DPL);
         const int b = d0 / 32;
         const uint16_t* sp16 = a.pools.vs + (ph * NB + b) * PT;
-        const uint8_t* cp = FMT == 8 ? a.pools.vq + (ph * D + d0) * PT
-                                     : a.pools.vq + ((ph * NB + b) * 16 + d0 % 32) * PT;
+        const uint8_t* cp = a.pools.vq + ((ph * NB + b) * 16 + d0 % 32) * PT;
         for (int t = 0; t < nt; ++t) {
           const float d = WidenF16(sp16[t]);
           const uint32_t byte = cp[t];
-          if (FMT == 8) {
-            const float v = d * static_cast<float>(static_cast<int8_t>(byte));
+          const float v0 = d * static_cast<float>(int(byte & 0xF) - 8), v1 = d * static_cast<float>(int(byte >> 4) - 8);
 #pragma unroll
-            for (int gi = 0; gi < kMaxGroup; ++gi)
-              if (gi < G) acc[gi][k] = __builtin_fmaf(ps[wave][gi][sp * PT + t], v, acc[gi][k]);
-          } else {
-            const float v0 = d * static_cast<float>(int(byte & 0xF) - 8), v1 = d * static_cast<float>(int(byte >> 4) - 8);
-#pragma unroll
-            for (int gi = 0; gi < kMaxGroup; ++gi)
-              if (gi < G) {
-                const float p = ps[wave][gi][sp * PT + t];
-                acc[gi][k] = __builtin_fmaf(p, v0, acc[gi][k]);
-                acc[gi][k + 1] = __builtin_fmaf(p, v1, acc[gi][k + 1]);
-              }
-          }
+          for (int gi = 0; gi < kMaxGroup; ++gi)
+            if (gi < G) {
+              const float p = ps[gi][sp * PT + t];
+              acc[gi][k] = __builtin_fmaf(p, v0, acc[gi][k]);
+              acc[gi][k + 1] = __builtin_fmaf(p, v1, acc[gi][k + 1]);
+            }
         }
       }
     }
     __builtin_amdgcn_wave_barrier();  // ps is rewritten by the next tile
   }
 
-  // ---- merge the four waves, write the split's partial
+  const size_t part = size_t(item) * G;
 #pragma unroll
   for (int gi = 0; gi < kMaxGroup; ++gi) {
     if (gi < G) {
-      if (lane == 0) wm[wave][gi] = m[gi], wl[wave][gi] = l[gi];
+      if (lane == 0) a.ml[(part + gi) * 2] = m[gi], a.ml[(part + gi) * 2 + 1] = l[gi];
 #pragma unroll
-      for (int k = 0; k < DPL; ++k) wacc[wave][gi][LaneDim<FMT>(lane, k, DPL)] = acc[gi][k];
+      for (int k = 0; k < DPL; ++k) a.acc[(part + gi) * D + LaneDimQ4(lane, k, DPL)] = acc[gi][k];
     }
-  }
-  __syncthreads();
-  const size_t part = ((size_t(s) * H + h) * a.n_splits + split) * G;
-  for (int i = threadIdx.x; i < G * D; i += 256) {
-    const int gi = i / D, d = i % D;
-    float M = kNegMax;
-#pragma unroll
-    for (int w = 0; w < kWaves; ++w) M = fmaxf(M, wm[w][gi]);
-    float L = 0.0f, A = 0.0f;
-#pragma unroll
-    for (int w = 0; w < kWaves; ++w) {
-      const float e = __expf(wm[w][gi] - M);
-      L = __builtin_fmaf(e, wl[w][gi], L);
-      A = __builtin_fmaf(e, wacc[w][gi][d], A);
-    }
-    a.acc[(part + gi) * D + d] = A;
-    if (d == 0) a.ml[(part + gi) * 2] = M, a.ml[(part + gi) * 2 + 1] = L;
   }
 }
 
@@ -218,13 +245,13 @@ __global__ __launch_bounds__(256) void DattnPartScalar(const DecodeArgs a) {
 // A scalar-ALU version of this kernel needs 7 lane operations per KV byte (one convert and one multiply-add per query
 // head of the group): at 5.6 TB/s that is every VALU issue slot of the chip. So the two contractions go to MFMA, whose
 // f16 rate leaves both at a few percent of peak, and the VALU only converts codes (about 1.5 operations per byte):
-//   scores  S[head][token] = sum_block ks[token][block] * (Q_block . codes_block)   v_mfma_f32_32x32x16_f16, one
+//   scores  S[head][key] = sum_block ks[key][block] * (Q_block . codes_block)       v_mfma_f32_32x32x16_f16, one
 //           32-dim block per pair of instructions (K = 16 each), so the block scale is applied to the f32 result and
 //           the products themselves are exact (int8 codes and f16 queries are exact in f16)
-//   output  O[head][dim] += sum_token P[head][token] * (vs[token][block] * codes)   v_mfma_f32_16x16x32_f16; the scale
+//   output  O[head][dim] += sum_key P[head][key] * (vs[key][block] * codes)          v_mfma_f32_16x16x32_f16; the scale
 //           varies along the contraction here, so V is dequantized to f16 (one rounding, 2^-12 relative)
-// The page layouts are chosen for these operand shapes: a lane's 16-byte load is 16 dims of one key (K, [block][token]
-// [32]) or 16 keys of one dim (V^T, [dim][token]); each wave-wide load is 1 KB contiguous.
+// The page layouts are chosen for these operand shapes: a lane's 16-byte load is 16 dims of one key (K, [block][key]
+// [32]) or 16 keys of one dim (V^T, [dim][key]); each wave-wide load is 1 KB contiguous.
 typedef _Float16 h2v __attribute__((ext_vector_type(2)));
 typedef _Float16 h8v __attribute__((ext_vector_type(8)));
 typedef float f4v __attribute__((ext_vector_type(4)));
@@ -262,103 +289,91 @@ __device__ __forceinline__ h8v LoadQ8(const void* q, size_t i, int dt) {
   return r;
 }
 
-__device__ __forceinline__ float HalfMax32(float v) {  // over the 32 lanes of a wave half
-#pragma unroll
-  for (int o = 16; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-  return v;
-}
-__device__ __forceinline__ float HalfSum32(float v) {
-#pragma unroll
-  for (int o = 16; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-  return v;
-}
-
-// One workgroup per (split, kv head, sequence), four waves, each with its own tiles of 64 keys and its own online
-// softmax; merged through LDS at the end. Loads run one tile ahead of the arithmetic: V of the tile is in flight while
-// its scores are computed, K of the wave's next tile while P.V is. Page numbers come through scalar loads (they are
-// the same for the whole wave), so waiting for them does not drain the vector-memory queue.
+// One wavefront per (item, kv head), alone in its workgroup: no workgroup barriers anywhere. The wave walks its tiles
+// of 64 keys with an online softmax. Registers hold half a tile of K (32 keys) and half a tile of V (half the dims) at
+// a time, which keeps the kernel under 256 registers, i.e. two waves per SIMD; the four load phases of a tile are
+// rotated against the four arithmetic phases so that every load has arithmetic between its issue and its first use:
+//   scores(keys 0-31)   | load K keys 32-63
+//   P.V(dims D/2.., previous tile) | load V dims 0..D/2 of this tile
+//   scores(keys 32-63)  | load K keys 0-31 of the next tile
+//   softmax, P.V(dims 0..D/2)      | load V dims D/2.. of this tile
+// Page numbers come through scalar loads (they are the same for the whole wave).
 template <int D, int PT>
-__global__ __launch_bounds__(256) void DattnPartQ8(const DecodeArgs a) {
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void DattnPartQ8(const DecodeArgs a) {
   constexpr int NB = D / 32, NT = D / 16, PPT = kTile / PT;
   constexpr float kLog2e = 1.4426950408889634f, kLn2 = 0.6931471805599453f;
   const Geom g = a.g;
   const int G = g.group(), H = g.n_kv;
-  const int s = blockIdx.z, h = blockIdx.y, split = blockIdx.x;
-  const int len = min(max(a.seq_len[s], 0), a.max_len);
-  const int n_tiles = (len + kTile - 1) / kTile;
-  const int tile0 = split * a.tiles_per_split;
-  if (tile0 >= n_tiles) return;
-  const int tile1 = min(tile0 + a.tiles_per_split, n_tiles);
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64), lane = threadIdx.x % 64;
+  const int item = blockIdx.x, h = item % H;
+  const int4 rec = a.items[item / H];
+  if (rec.x < 0) return;
+  const int s = rec.x, tile0 = rec.y, tile1 = rec.z, len = rec.w;
+  const int lane = threadIdx.x;
   const int n32 = lane % 32, half = lane / 32;  // score layout: lane = key (mod 32), registers = heads 4 * half + r
   const int n16 = lane % 16, kg = lane / 16;    // P.V layout: lane = dim (mod 16), 16 keys per lane group
 
-  __shared__ __align__(16) _Float16 lq[NB][2][64][8];  // query A-operands, [block][K half][lane]
-  __shared__ __align__(16) _Float16 lp[kWaves][kMaxGroup][kTile];
-  __shared__ __align__(16) _Float16 lvs[kWaves][NB][kTile];
-  __shared__ float wm[kWaves][kMaxGroup], wl[kWaves][kMaxGroup];
-  __shared__ float wacc[kWaves][kMaxGroup][D];
-
-  // Query operands: row m of the 32-row A matrix is head m of the group (rows past G are zero); lane (m, half) holds
-  // dims 32 b + 16 half + 8 sub + 0..7 for the (b, sub) instruction, matching the 16 code bytes a key lane loads.
-  for (int i = threadIdx.x; i < NB * 2 * 64; i += 256) {
-    const int b = i / 128, sub = (i / 64) % 2, l = i % 64;
+  // Query A-operands [block][K half of the block's instruction pair][lane half][head row]: 8 f16 each. Row m of the
+  // 32-row A matrix is head m; only rows 0-7 exist here and lanes of rows 8-31 re-read them (their output rows are
+  // never looked at). Entry (b, sub, hf, row) holds dims 32 b + 16 hf + 8 sub + 0..7, the dims of the 8 code bytes a
+  // key lane of that half feeds to instruction `sub`.
+  __shared__ __align__(16) _Float16 lq[NB][2][2][8][8];
+  __shared__ __align__(16) _Float16 lp[kMaxGroup][kTile];
+  __shared__ __align__(16) _Float16 lvs[NB][kTile];
+  for (int i = lane; i < NB * 32; i += 64) {
+    const int b = i / 32, sub = (i / 16) % 2, hf = (i / 8) % 2, rw = i % 8;
     h8v v = {0, 0, 0, 0, 0, 0, 0, 0};
-    if (l % 32 < G)
-      v = LoadQ8(a.q, (size_t(s) * g.n_q + size_t(h) * G + l % 32) * D + b * 32 + 16 * (l / 32) + 8 * sub, a.q_dtype);
-    *reinterpret_cast<h8v*>(&lq[b][sub][l][0]) = v;
+    if (rw < G)
+      v = LoadQ8(a.q, (size_t(s) * g.n_q + size_t(h) * G + rw) * D + b * 32 + 16 * hf + 8 * sub, a.q_dtype);
+    *reinterpret_cast<h8v*>(&lq[b][sub][hf][rw][0]) = v;
   }
-  __syncthreads();
 
   const int32_t* row = a.table + int64_t(s) * a.stride;
-  // (page, kv head) index of the key `tok_in_tile` of a tile; page numbers are wave-uniform loads.
-  auto page_head = [&](const int (&pg)[PPT], int tok_in_tile) -> size_t {
+  auto load_pages = [&](int tile, int (&pg)[PPT]) {
+#pragma unroll
+    for (int j = 0; j < PPT; ++j) pg[j] = ClampPage(row[min(tile * PPT + j, a.stride - 1)], g.n_pages);
+  };
+  auto page_head = [&](const int (&pg)[PPT], int tok_in_tile) -> size_t {  // (page, kv head) index of a key of the tile
     int p = pg[0];
 #pragma unroll
     for (int j = 1; j < PPT; ++j) p = tok_in_tile / PT == j ? pg[j] : p;
     return size_t(p) * H + h;
   };
-  auto load_pages = [&](int tile, int (&pg)[PPT]) {
-#pragma unroll
-    for (int j = 0; j < PPT; ++j) pg[j] = ClampPage(row[min(tile * PPT + j, a.stride - 1)], g.n_pages);
-  };
 
-  uint4 kb[NB][2];   // [block][32-key half of the tile]: 16 codes of this lane's key
-  uint4 ksc[2];      // the key's NB block scales (f16)
-  uint4 vb[NT];      // [16-dim tile]: 16 keys of this lane's dim
+  uint4 kb[NB];      // [block]: 16 codes of this lane's key (one 32-key half of the tile at a time)
+  uint4 ksc;         // that key's NB block scales (f16)
+  uint4 vb[NT / 2];  // [16-dim tile]: 16 keys of this lane's dim (one half of the dims at a time)
   uint4 vsr;         // staging of the tile's V scales: 8 keys of one block per lane
-  auto load_k = [&](const int (&pg)[PPT]) {
+  auto load_k = [&](int tt, const int (&pg)[PPT]) {
+    const int tk = 32 * tt + n32;
+    const size_t ph = page_head(pg, tk);
+    const int t = tk % PT;
 #pragma unroll
-    for (int tt = 0; tt < 2; ++tt) {
-      const int tk = 32 * tt + n32;
-      const size_t ph = page_head(pg, tk);
-      const int t = tk % PT;
-#pragma unroll
-      for (int b = 0; b < NB; ++b)
-        kb[b][tt] = *reinterpret_cast<const uint4*>(a.pools.kq + ((ph * NB + b) * PT + t) * 32 + 16 * half);
-      const uint16_t* sp = a.pools.ks + (ph * PT + t) * NB;
-      if (NB == 8) {
-        ksc[tt] = *reinterpret_cast<const uint4*>(sp);
-      } else {
-        const uint2 v = *reinterpret_cast<const uint2*>(sp);
-        ksc[tt] = uint4{v.x, v.y, 0u, 0u};
-      }
+    for (int b = 0; b < NB; ++b)
+      kb[b] = *reinterpret_cast<const uint4*>(a.pools.kq + ((ph * NB + b) * PT + t) * 32 + 16 * half);
+    const uint16_t* sp = a.pools.ks + (ph * PT + t) * NB;
+    if (NB == 8) {
+      ksc = *reinterpret_cast<const uint4*>(sp);
+    } else {
+      const uint2 v = *reinterpret_cast<const uint2*>(sp);
+      ksc = uint4{v.x, v.y, 0u, 0u};
     }
   };
-  auto load_v = [&](const int (&pg)[PPT]) {
+  auto load_v = [&](int hf, const int (&pg)[PPT]) {
     const size_t ph = page_head(pg, 16 * kg);
     const int t0 = (16 * kg) % PT;
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt)
-      vb[nt] = *reinterpret_cast<const uint4*>(a.pools.vq + (ph * D + 16 * nt + n16) * PT + t0);
-    const int b = lane / 8, chunk = lane % 8;  // V scales: lane = (block, 8 keys)
-    if (b < NB) {
-      const size_t ps = page_head(pg, 8 * chunk);
-      vsr = *reinterpret_cast<const uint4*>(a.pools.vs + (ps * NB + b) * PT + (8 * chunk) % PT);
+    for (int j = 0; j < NT / 2; ++j)
+      vb[j] = *reinterpret_cast<const uint4*>(a.pools.vq + (ph * D + 16 * (hf * (NT / 2) + j) + n16) * PT + t0);
+    if (hf == 0) {  // with the first half come the tile's V scales: lane = (block, 8 keys)
+      const int b = lane / 8, chunk = lane % 8;
+      if (b < NB) {
+        const size_t ps = page_head(pg, 8 * chunk);
+        vsr = *reinterpret_cast<const uint4*>(a.pools.vs + (ps * NB + b) * PT + (8 * chunk) % PT);
+      }
     }
   };
 
-  float m[4], lsum[4];
+  float m[4], lsum[4], sc[2][4];
   f4v o[NT];
 #pragma unroll
   for (int r = 0; r < 4; ++r) m[r] = kNegMax, lsum[r] = 0.0f;
@@ -369,47 +384,68 @@ __global__ __launch_bounds__(256) void DattnPartQ8(const DecodeArgs a) {
   // the heads whose running maximum it already holds (lanes 0-15: heads 0-3, lanes 32-47: heads 4-7).
   const int prow = n16 < 4 ? n16 : (n16 >= 8 && n16 < 12 ? n16 - 4 : 0);
 
-  int tile = tile0 + wave;
-  int pg[PPT];
-  if (tile < tile1) {
-    load_pages(tile, pg);
-    load_k(pg);
-    load_v(pg);
-  }
-  for (; tile < tile1; tile += kWaves) {
-    const int next = tile + kWaves;
-    if (next < tile1) load_pages(next, pg);
-    // ---- scores
-    float sc[2][4];
+  // scores of the 32 keys in kb against all heads: two blocks (two accumulator chains) at a time
+  auto scores = [&](int tt) {
 #pragma unroll
-    for (int tt = 0; tt < 2; ++tt)
+    for (int r = 0; r < 4; ++r) sc[tt][r] = 0.0f;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) sc[tt][r] = 0.0f;
-#pragma unroll
-    for (int b = 0; b < NB; ++b) {
-      const h8v q0 = *reinterpret_cast<const h8v*>(&lq[b][0][lane][0]);
-      const h8v q1 = *reinterpret_cast<const h8v*>(&lq[b][1][lane][0]);
+    for (int b = 0; b < NB; b += 2) {
+      const h8v qa0 = *reinterpret_cast<const h8v*>(&lq[b][0][half][n32 % 8][0]);
+      const h8v qa1 = *reinterpret_cast<const h8v*>(&lq[b][1][half][n32 % 8][0]);
+      const h8v qb0 = *reinterpret_cast<const h8v*>(&lq[b + 1][0][half][n32 % 8][0]);
+      const h8v qb1 = *reinterpret_cast<const h8v*>(&lq[b + 1][1][half][n32 % 8][0]);
       f16v c0 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}, c1 = c0;
-      c0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(q0, Codes8(kb[b][0].x, kb[b][0].y), c0, 0, 0, 0);
-      c1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(q0, Codes8(kb[b][1].x, kb[b][1].y), c1, 0, 0, 0);
-      c0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(q1, Codes8(kb[b][0].z, kb[b][0].w), c0, 0, 0, 0);
-      c1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(q1, Codes8(kb[b][1].z, kb[b][1].w), c1, 0, 0, 0);
-      const uint32_t w0 = b < 2 ? ksc[0].x : b < 4 ? ksc[0].y : b < 6 ? ksc[0].z : ksc[0].w;
-      const uint32_t w1 = b < 2 ? ksc[1].x : b < 4 ? ksc[1].y : b < 6 ? ksc[1].z : ksc[1].w;
-      const float d0 = WidenF16(static_cast<uint16_t>(w0 >> (16 * (b % 2)))) * qk_scale;
-      const float d1 = WidenF16(static_cast<uint16_t>(w1 >> (16 * (b % 2)))) * qk_scale;
+      c0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(qa0, Codes8(kb[b].x, kb[b].y), c0, 0, 0, 0);
+      c1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(qb0, Codes8(kb[b + 1].x, kb[b + 1].y), c1, 0, 0, 0);
+      c0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(qa1, Codes8(kb[b].z, kb[b].w), c0, 0, 0, 0);
+      c1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(qb1, Codes8(kb[b + 1].z, kb[b + 1].w), c1, 0, 0, 0);
+      const uint32_t w = b < 2 ? ksc.x : b < 4 ? ksc.y : b < 6 ? ksc.z : ksc.w;  // scales of blocks b, b + 1
+      const float d0 = WidenF16(static_cast<uint16_t>(w & 0xFFFF)) * qk_scale;
+      const float d1 = WidenF16(static_cast<uint16_t>(w >> 16)) * qk_scale;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        sc[0][r] = __builtin_fmaf(c0[r], d0, sc[0][r]);
-        sc[1][r] = __builtin_fmaf(c1[r], d1, sc[1][r]);
-      }
-      // One block (two independent accumulator chains) at a time: more only multiplies live 32x32 accumulators.
-      // The empty asm pins the scaled sums here, so the accumulators die before the next block starts.
-      asm volatile("" : "+v"(sc[0][0]), "+v"(sc[0][1]), "+v"(sc[0][2]), "+v"(sc[0][3]), "+v"(sc[1][0]), "+v"(sc[1][1]),
-                        "+v"(sc[1][2]), "+v"(sc[1][3]));
+      for (int r = 0; r < 4; ++r) sc[tt][r] = __builtin_fmaf(c1[r], d1, __builtin_fmaf(c0[r], d0, sc[tt][r]));
+      // The empty asm pins the scaled sums here, so the 32x32 accumulators die before the next pair of blocks starts
+      // (otherwise every pair's accumulators stay live to the end and the kernel spills).
+      asm volatile("" : "+v"(sc[tt][0]), "+v"(sc[tt][1]), "+v"(sc[tt][2]), "+v"(sc[tt][3]));
       __builtin_amdgcn_sched_barrier(0);
     }
-    if (next < tile1) load_k(pg);
+  };
+  // P.V for one half of the dims, from vb, lp and lvs
+  auto pv = [&](int hf) {
+    const h8v pa0 = *reinterpret_cast<const h8v*>(&lp[prow][16 * kg]);
+    const h8v pa1 = *reinterpret_cast<const h8v*>(&lp[prow][16 * kg + 8]);
+#pragma unroll
+    for (int bb = 0; bb < NB / 2; ++bb) {
+      const int b = hf * (NB / 2) + bb;
+      const h8v s0 = *reinterpret_cast<const h8v*>(&lvs[b][16 * kg]);
+      const h8v s1 = *reinterpret_cast<const h8v*>(&lvs[b][16 * kg + 8]);
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const uint4 w = vb[2 * bb + j];
+        const int nt = 2 * b + j;
+        const h8v v0 = Codes8(w.x, w.y) * s0, v1 = Codes8(w.z, w.w) * s1;
+        o[nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa0, v0, o[nt], 0, 0, 0);
+        o[nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa1, v1, o[nt], 0, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  int pgc[PPT], pgn[PPT];
+  load_pages(tile0, pgc);
+  load_k(0, pgc);
+  load_v(0, pgc);
+  for (int tile = tile0; tile < tile1; ++tile) {
+    const bool has_next = tile + 1 < tile1;
+    if (has_next) load_pages(tile + 1, pgn);
+    scores(0);
+    load_k(1, pgc);
+    if (tile > tile0) {
+      pv(1);  // second half of the previous tile's P.V: lp and lvs still hold that tile
+      load_v(0, pgc);
+    }
+    scores(1);
+    if (has_next) load_k(0, pgn);
     // ---- online softmax (base 2); keys at or past len are masked by select, so stale scales cannot leak
     float alpha[4];
 #pragma unroll
@@ -425,8 +461,8 @@ __global__ __launch_bounds__(256) void DattnPartQ8(const DecodeArgs a) {
       m[r] = mn;
       const float p0 = __builtin_amdgcn_exp2f(sc[0][r] - mn), p1 = __builtin_amdgcn_exp2f(sc[1][r] - mn);
       lsum[r] = __builtin_fmaf(lsum[r], alpha[r], p0 + p1);  // per lane; summed over the lanes at the end
-      lp[wave][4 * half + r][n32] = static_cast<_Float16>(p0);
-      lp[wave][4 * half + r][32 + n32] = static_cast<_Float16>(p1);
+      lp[4 * half + r][n32] = static_cast<_Float16>(p0);
+      lp[4 * half + r][32 + n32] = static_cast<_Float16>(p1);
     }
     {  // V scales of the tile to LDS; scales of keys at or past len become 0, which makes their V rows 0
       const int b = lane / 8, chunk = lane % 8;
@@ -438,7 +474,7 @@ __global__ __launch_bounds__(256) void DattnPartQ8(const DecodeArgs a) {
           for (int j = 0; j < 8; ++j)
             if (k0 + j >= len) w[j / 2] &= j % 2 ? 0x0000FFFFu : 0xFFFF0000u;
         }
-        *reinterpret_cast<uint4*>(&lvs[wave][b][8 * chunk]) = uint4{w[0], w[1], w[2], w[3]};
+        *reinterpret_cast<uint4*>(&lvs[b][8 * chunk]) = uint4{w[0], w[1], w[2], w[3]};
       }
     }
 #pragma unroll
@@ -448,56 +484,34 @@ __global__ __launch_bounds__(256) void DattnPartQ8(const DecodeArgs a) {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    // ---- P.V
-    const h8v pa0 = *reinterpret_cast<const h8v*>(&lp[wave][prow][16 * kg]);
-    const h8v pa1 = *reinterpret_cast<const h8v*>(&lp[wave][prow][16 * kg + 8]);
+    pv(0);
+    load_v(1, pgc);
 #pragma unroll
-    for (int b = 0; b < NB; ++b) {
-      const h8v s0 = *reinterpret_cast<const h8v*>(&lvs[wave][b][16 * kg]);
-      const h8v s1 = *reinterpret_cast<const h8v*>(&lvs[wave][b][16 * kg + 8]);
-#pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        const int nt = 2 * b + j;
-        const h8v v0 = Codes8(vb[nt].x, vb[nt].y) * s0, v1 = Codes8(vb[nt].z, vb[nt].w) * s1;
-        o[nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa0, v0, o[nt], 0, 0, 0);
-        o[nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa1, v1, o[nt], 0, 0, 0);
-      }
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    __builtin_amdgcn_wave_barrier();  // lp / lvs are rewritten by the next tile
-    if (next < tile1) load_v(pg);
+    for (int j = 0; j < PPT; ++j) pgc[j] = pgn[j];
   }
+  pv(1);
 
-  // ---- merge the four waves (natural-log units, as the reduce expects), write the split's partial
+  // ---- the item's partial, straight from registers (natural-log units, as the reduce expects)
+  const size_t part = size_t(item) * G;
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     const float l = HalfSum32(lsum[r]);
-    if (n32 == 0) wm[wave][4 * half + r] = m[r] * kLn2, wl[wave][4 * half + r] = l;
+    const int head = 4 * half + r;
+    if (n32 == 0 && head < G) a.ml[(part + head) * 2] = m[r] * kLn2, a.ml[(part + head) * 2 + 1] = l;
   }
   if (kg == 0 || kg == 2) {
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt)
+    for (int r = 0; r < 4; ++r) {
+      const int head = 2 * kg + r;
+      if (head < G) {
 #pragma unroll
-      for (int r = 0; r < 4; ++r) wacc[wave][2 * kg + r][16 * nt + n16] = o[nt][r];
-  }
-  __syncthreads();
-  const size_t part = ((size_t(s) * H + h) * a.n_splits + split) * G;
-  for (int i = threadIdx.x; i < G * D; i += 256) {
-    const int gi = i / D, d = i % D;
-    float M = kNegMax;
-#pragma unroll
-    for (int w = 0; w < kWaves; ++w) M = fmaxf(M, wm[w][gi]);
-    float L = 0.0f, A = 0.0f;
-#pragma unroll
-    for (int w = 0; w < kWaves; ++w) {
-      const float e = __expf(wm[w][gi] - M);
-      L = __builtin_fmaf(e, wl[w][gi], L);
-      A = __builtin_fmaf(e, wacc[w][gi][d], A);
+        for (int nt = 0; nt < NT; ++nt) a.acc[(part + head) * D + 16 * nt + n16] = o[nt][r];
+      }
     }
-    a.acc[(part + gi) * D + d] = A;
-    if (d == 0) a.ml[(part + gi) * 2] = M, a.ml[(part + gi) * 2 + 1] = L;
   }
 }
+
+// ---- reduce -------------------------------------------------------------------------------------------------------------
 
 // One workgroup per (query head, sequence), thread = dim (gen_decode_attn.py:338-411).
 __global__ void DattnReduce(const DecodeArgs a) {
@@ -505,20 +519,17 @@ __global__ void DattnReduce(const DecodeArgs a) {
   const int G = g.group(), H = g.n_kv, D = g.hd;
   const int hq = blockIdx.x, s = blockIdx.y, d = threadIdx.x;
   const int h = hq / G, gi = hq % G;
-  const int len = min(max(a.seq_len[s], 0), a.max_len);
   const size_t o = (size_t(s) * g.n_q + hq) * D + d;
-  if (len == 0) {
+  const int c0 = min(a.prefix[s], a.max_chunks), c1 = min(a.prefix[s + 1], a.max_chunks);
+  if (c0 >= c1) {  // length 0
     a.out[o] = 0.0f;
     return;
   }
-  const int n_tiles = (len + kTile - 1) / kTile;
-  const int ns = (n_tiles + a.tiles_per_split - 1) / a.tiles_per_split;
-  const size_t part = (size_t(s) * H + h) * a.n_splits * G + gi;
   float M = kNegMax;
-  for (int sp = 0; sp < ns; ++sp) M = fmaxf(M, a.ml[(part + size_t(sp) * G) * 2]);
+  for (int c = c0; c < c1; ++c) M = fmaxf(M, a.ml[((size_t(c) * H + h) * G + gi) * 2]);
   float L = 0.0f, A = 0.0f;
-  for (int sp = 0; sp < ns; ++sp) {
-    const size_t p = part + size_t(sp) * G;
+  for (int c = c0; c < c1; ++c) {
+    const size_t p = (size_t(c) * H + h) * G + gi;
     const float w = __expf(a.ml[p * 2] - M);
     L = __builtin_fmaf(w, a.ml[p * 2 + 1], L);
     A = __builtin_fmaf(w, a.acc[p * D + d], A);
@@ -528,21 +539,56 @@ __global__ void DattnReduce(const DecodeArgs a) {
   a.out[o] = v;
 }
 
-// Slices of the context: enough workgroups to fill 256 CUs several times over, at least one tile per wave.
+// ---- host side ----------------------------------------------------------------------------------------------------------
+
+// Workspace layout and item sizing from the host's bounds alone (the lengths themselves are on the device).
 struct Plan {
-  int32_t max_len, n_splits, tiles_per_split;
+  int32_t max_len, max_chunks, min_tiles_per_item, target_items;
+  size_t off_prefix, off_items, off_ml, off_acc, bytes;
 };
+size_t Align(size_t x) { return (x + 255) & ~size_t(255); }
 Plan MakePlan(const Geom& g, int32_t n_seqs, int32_t max_seq_len) {
   Plan p;
   p.max_len = std::max(max_seq_len, 1);
   const int64_t max_tiles = (int64_t(p.max_len) + kTile - 1) / kTile;
-  const int64_t want_wgs = 2048;
-  int64_t tps = (max_tiles * g.n_kv * n_seqs + want_wgs - 1) / want_wgs;
-  tps = std::max<int64_t>(tps, kWaves);
-  tps = (tps + kWaves - 1) / kWaves * kWaves;
-  p.tiles_per_split = static_cast<int32_t>(tps);
-  p.n_splits = static_cast<int32_t>((max_tiles + tps - 1) / tps);
+  // About six items per wave slot (256 CUs x 8 waves) when the batch is large; never more than 16384 records.
+  p.target_items = 12288;
+  if (const char* e = std::getenv("YAHKV_DECODE_TARGET_ITEMS")) p.target_items = std::max(1, std::atoi(e));
+  int64_t tpi = (max_tiles * n_seqs * g.n_kv + 16383) / 16384;
+  if (const char* e = std::getenv("YAHKV_DECODE_MIN_TILES_PER_ITEM")) tpi = std::max<int64_t>(tpi, std::atoll(e));
+  p.min_tiles_per_item = static_cast<int32_t>(std::max<int64_t>(tpi, 2));
+  p.max_chunks = static_cast<int32_t>(n_seqs * ((max_tiles + p.min_tiles_per_item - 1) / p.min_tiles_per_item));
+  const size_t items = size_t(p.max_chunks) * g.n_kv;
+  p.off_prefix = 256;
+  p.off_items = Align(p.off_prefix + sizeof(int32_t) * (size_t(n_seqs) + 1));
+  p.off_ml = Align(p.off_items + sizeof(int4) * size_t(p.max_chunks));
+  p.off_acc = Align(p.off_ml + sizeof(float) * items * g.group() * 2);
+  p.bytes = Align(p.off_acc + sizeof(float) * items * g.group() * g.hd);
   return p;
+}
+
+// Fills the launch arguments all dispatches share; returns a status.
+int Prepare(const yahkv_geometry* g, int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs,
+            int32_t max_seq_len, const void* workspace, size_t workspace_bytes, DecodeArgs* a) {
+  if (const int st = CheckGeometry(g)) return st;
+  if (seq_len == nullptr || workspace == nullptr) return YAHKV_ERR_ARG;
+  if (n_seqs <= 0 || max_seq_len <= 0 || page_table_stride <= 0) return YAHKV_ERR_ARG;
+  if (reinterpret_cast<uintptr_t>(workspace) & 15) return YAHKV_ERR_ARG;
+  const Geom m = MakeGeom(*g);
+  const Plan p = MakePlan(m, n_seqs, max_seq_len);
+  if (workspace_bytes < p.bytes) return YAHKV_ERR_WORKSPACE;
+  *a = DecodeArgs{};
+  a->g = m, a->stride = page_table_stride, a->seq_len = seq_len, a->n_seqs = n_seqs;
+  // lengths read on the device are clamped to the host's bound and to the table's extent
+  a->max_len = static_cast<int32_t>(std::min<int64_t>(p.max_len, int64_t(page_table_stride) * m.pt));
+  char* ws = static_cast<char*>(const_cast<void*>(workspace));
+  a->header = reinterpret_cast<int32_t*>(ws);
+  a->prefix = reinterpret_cast<int32_t*>(ws + p.off_prefix);
+  a->items = reinterpret_cast<int4*>(ws + p.off_items);
+  a->ml = reinterpret_cast<float*>(ws + p.off_ml);
+  a->acc = reinterpret_cast<float*>(ws + p.off_acc);
+  a->max_chunks = p.max_chunks, a->min_tiles_per_item = p.min_tiles_per_item, a->target_items = p.target_items;
+  return YAHKV_OK;
 }
 
 }  // namespace
@@ -552,34 +598,8 @@ using namespace yahkv;
 
 extern "C" size_t yahkv_decode_workspace_bytes(const yahkv_geometry* g, int32_t n_seqs, int32_t max_seq_len) {
   if (CheckGeometry(g) || n_seqs <= 0 || max_seq_len <= 0) return 0;
-  const Geom m = MakeGeom(*g);
-  const Plan p = MakePlan(m, n_seqs, max_seq_len);
-  return size_t(n_seqs) * m.n_kv * p.n_splits * m.group() * (m.hd + 2) * sizeof(float);
+  return MakePlan(MakeGeom(*g), n_seqs, max_seq_len).bytes;
 }
-
-namespace {
-
-// Fills the launch arguments both dispatches share; returns a status.
-int Prepare(const yahkv_geometry* g, int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs,
-            int32_t max_seq_len, const void* workspace, size_t workspace_bytes, DecodeArgs* a) {
-  if (const int st = CheckGeometry(g)) return st;
-  if (seq_len == nullptr || workspace == nullptr) return YAHKV_ERR_ARG;
-  if (n_seqs <= 0 || max_seq_len <= 0 || page_table_stride <= 0) return YAHKV_ERR_ARG;
-  if (reinterpret_cast<uintptr_t>(workspace) & 15) return YAHKV_ERR_ARG;
-  if (workspace_bytes < yahkv_decode_workspace_bytes(g, n_seqs, max_seq_len)) return YAHKV_ERR_WORKSPACE;
-  const Geom m = MakeGeom(*g);
-  const Plan p = MakePlan(m, n_seqs, max_seq_len);
-  *a = DecodeArgs{};
-  a->g = m, a->stride = page_table_stride, a->seq_len = seq_len, a->n_seqs = n_seqs;
-  // lengths read on the device are clamped to the host's bound and to the table's extent
-  a->max_len = static_cast<int32_t>(std::min<int64_t>(p.max_len, int64_t(page_table_stride) * m.pt));
-  a->acc = static_cast<float*>(const_cast<void*>(workspace));
-  a->ml = a->acc + size_t(n_seqs) * m.n_kv * p.n_splits * m.group() * m.hd;
-  a->n_splits = p.n_splits, a->tiles_per_split = p.tiles_per_split;
-  return YAHKV_OK;
-}
-
-}  // namespace
 
 extern "C" int yahkv_decode_part(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
                                  int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs,
@@ -593,14 +613,17 @@ extern "C" int yahkv_decode_part(const yahkv_geometry* g, const yahkv_pools* poo
     return YAHKV_ERR_ARG;
   if (q_dtype != YAHKV_F32 && q_dtype != YAHKV_F16 && q_dtype != YAHKV_BF16) return YAHKV_ERR_ARG;
   if ((reinterpret_cast<uintptr_t>(pools->kq) | reinterpret_cast<uintptr_t>(pools->vq) |
-       reinterpret_cast<uintptr_t>(pools->ks) | reinterpret_cast<uintptr_t>(pools->vs)) & 15)
+       reinterpret_cast<uintptr_t>(pools->ks) | reinterpret_cast<uintptr_t>(pools->vs) |
+       reinterpret_cast<uintptr_t>(q)) & 15)
     return YAHKV_ERR_ARG;
   a.pools = MakePools(*pools), a.table = page_table, a.q = q, a.q_dtype = q_dtype, a.scale = softmax_scale;
   const Geom& m = a.g;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  const dim3 grid(a.n_splits, m.n_kv, n_seqs);
+  hipLaunchKernelGGL(DattnPlan, dim3(1), dim3(kPlanThreads), 0, st, a);
+  if (const int ls = LaunchStatus()) return ls;
+  const dim3 grid(static_cast<unsigned>(a.max_chunks) * m.n_kv);
   if (m.format == 8) {
-#define YAHKV_LAUNCH_Q8(DD, PP) hipLaunchKernelGGL((DattnPartQ8<DD, PP>), grid, dim3(256), 0, st, a)
+#define YAHKV_LAUNCH_Q8(DD, PP) hipLaunchKernelGGL((DattnPartQ8<DD, PP>), grid, dim3(64), 0, st, a)
     if (m.hd == 256 && m.pt == 64) YAHKV_LAUNCH_Q8(256, 64);
     else if (m.hd == 256 && m.pt == 32) YAHKV_LAUNCH_Q8(256, 32);
     else if (m.hd == 256) YAHKV_LAUNCH_Q8(256, 16);
@@ -609,9 +632,9 @@ extern "C" int yahkv_decode_part(const yahkv_geometry* g, const yahkv_pools* poo
     else YAHKV_LAUNCH_Q8(128, 16);
 #undef YAHKV_LAUNCH_Q8
   } else if (m.hd == 256) {
-    hipLaunchKernelGGL((DattnPartScalar<4, 256>), grid, dim3(256), 0, st, a);
+    hipLaunchKernelGGL((DattnPartQ4<256>), grid, dim3(64), 0, st, a);
   } else {
-    hipLaunchKernelGGL((DattnPartScalar<4, 128>), grid, dim3(256), 0, st, a);
+    hipLaunchKernelGGL((DattnPartQ4<128>), grid, dim3(64), 0, st, a);
   }
   return LaunchStatus();
 }
