@@ -7,9 +7,12 @@
 // -FLT_MAX the reference uses (:357), so that no inf - inf can appear.
 //
 // The reference launches one workgroup per 256-key page of its single sequence. Here lengths are ragged and live on
-// the device, so a small `plan` kernel first cuts every sequence into items of equal size (a run of 64-key tiles) and
-// writes one record per item; `part` runs one wavefront per (item, kv head). Equal items keep 256 CUs evenly loaded
-// whatever the mix of lengths, and no workgroup is launched for work that does not exist except at the grid's end.
+// the device, so the work is cut stream-K style: all (sequence, kv head) pairs are laid end to end on one line of
+// 64-key tiles and the line is cut into chunks. The first chunks are long and equal, one per wavefront slot of the chip
+// (every wave starts with the same amount of work whatever the mix of lengths); the last part of the line is cut into
+// short chunks that waves take from a counter as they finish, because waves do not run at one speed (the XCDs do not
+// all see the same bandwidth). A wave leaves one partial per (chunk, pair) it touches. A small `plan` kernel computes
+// the cut from the device-resident lengths.
 #include <algorithm>
 #include <cstdlib>
 
@@ -22,6 +25,7 @@ constexpr float kNegMax = -3.4028234663852886e+38f;
 constexpr int kTile = 64;     // keys per tile: one wavefront, one key per lane in the score phase
 constexpr int kMaxGroup = 8;  // query heads per kv head
 constexpr int kPlanThreads = 256;
+constexpr int kMaxSeqs = 8191;
 
 struct DecodeArgs {
   Geom g;
@@ -36,61 +40,104 @@ struct DecodeArgs {
   const float* gate;
   float* out;
   // workspace
-  int32_t* header;   // [0] chunks in use, [1] tiles per item
-  int32_t* prefix;   // [n_seqs + 1] first chunk of each sequence
-  int4* items;       // [max_chunks] {sequence or -1, first tile, end tile, length}
-  float* ml;         // [max_chunks * H][G][2]
-  float* acc;        // [max_chunks * H][G][D]
-  int32_t max_chunks, min_tiles_per_item, target_items;
+  int32_t* header;   // [0] tiles on the line, [1] tiles per long chunk, [2] tiles per short chunk, [3] ticket counter
+  int32_t* tprefix;  // [n_seqs + 1] tiles of all earlier sequences (one kv head's worth)
+  int4* chunks;      // [max_chunks] {sequence or -1, kv head, first tile within the pair, tiles in the chunk}
+  float* ml;         // [max_chunks + n_seqs * H][G][2]   partial of (chunk k, pair p) is number k + p
+  float* acc;        // [max_chunks + n_seqs * H][G][D]
+  int32_t n_long, max_chunks;    // long chunks = wavefronts launched; records in `chunks`
+  int32_t min_long_tiles, short_tiles, short_permille;
 };
+
+__device__ __forceinline__ int ClampLen(const DecodeArgs& a, int s) { return min(max(a.seq_len[s], 0), a.max_len); }
 
 // ---- plan -------------------------------------------------------------------------------------------------------------
 
-// One workgroup. Reads the lengths, picks the item size (tiles per item: at least the host's lower bound, which sized
-// the workspace, and large enough that there are about target_items items), and writes prefix[] and items[].
+// Every workgroup recomputes the prefix sums of the sequences' tile counts in LDS (a few hundred integers), then each
+// thread writes one chunk record. Workgroup 0 also publishes the prefix sums, the chunk sizes and a zeroed ticket
+// counter. Chunk k < n_long covers tiles [k A, (k + 1) A) of the line, chunk n_long + i covers
+// [n_long A + i c, n_long A + (i + 1) c), both clipped to the line's length.
 __global__ __launch_bounds__(kPlanThreads) void DattnPlan(const DecodeArgs a) {
+  extern __shared__ int lpre[];  // [n_seqs + 1]
   __shared__ int part_sum[kPlanThreads];
-  __shared__ int tpi_s;
-  const int t = threadIdx.x;
+  const int t = threadIdx.x, H = a.g.n_kv;
   const int per = (a.n_seqs + kPlanThreads - 1) / kPlanThreads;
   const int s0 = min(t * per, a.n_seqs), s1 = min(s0 + per, a.n_seqs);
-  auto tiles_of = [&](int s) { return (min(max(a.seq_len[s], 0), a.max_len) + kTile - 1) / kTile; };
   int sum = 0;
-  for (int s = s0; s < s1; ++s) sum += tiles_of(s);
+  for (int s = s0; s < s1; ++s) sum += (ClampLen(a, s) + kTile - 1) / kTile;
   part_sum[t] = sum;
   __syncthreads();
-  if (t == 0) {
-    long long total = 0;
-    for (int i = 0; i < kPlanThreads; ++i) total += part_sum[i];
-    const long long want = (total * a.g.n_kv + a.target_items - 1) / a.target_items;
-    tpi_s = static_cast<int>(max(static_cast<long long>(a.min_tiles_per_item), want));
+  int base = 0, total = 0;
+  for (int i = 0; i < kPlanThreads; ++i) {
+    if (i < t) base += part_sum[i];
+    total += part_sum[i];
   }
-  __syncthreads();
-  const int tpi = tpi_s;
-  sum = 0;
-  for (int s = s0; s < s1; ++s) sum += (tiles_of(s) + tpi - 1) / tpi;
-  __syncthreads();
-  part_sum[t] = sum;
-  __syncthreads();
-  int base = 0;
-  for (int i = 0; i < t; ++i) base += part_sum[i];
   for (int s = s0; s < s1; ++s) {
-    const int len = min(max(a.seq_len[s], 0), a.max_len), nt = (len + kTile - 1) / kTile;
-    const int nc = (nt + tpi - 1) / tpi;
-    a.prefix[s] = base;
-    for (int c = 0; c < nc; ++c)
-      if (base + c < a.max_chunks) a.items[base + c] = int4{s, c * tpi, min(c * tpi + tpi, nt), len};
-    base += nc;
+    lpre[s] = base;
+    base += (ClampLen(a, s) + kTile - 1) / kTile;
   }
-  if (t == kPlanThreads - 1) {
-    a.prefix[a.n_seqs] = base;
-    a.header[0] = min(base, a.max_chunks);
-    a.header[1] = tpi;
-  }
+  if (t == 0) lpre[a.n_seqs] = total;
   __syncthreads();
-  int total = 0;
-  for (int i = 0; i < kPlanThreads; ++i) total += part_sum[i];
-  for (int c = total + t; c < a.max_chunks; c += kPlanThreads) a.items[c] = int4{-1, 0, 0, 0};  // unused records
+  const long long line = static_cast<long long>(total) * H;  // tiles on the line
+  // long chunks share (1 - short_permille / 1000) of the line, but a short line is not cut finer than min_long_tiles
+  long long A = line * (1000 - a.short_permille) / 1000 / a.n_long;
+  if (A < 4LL * a.short_tiles) A = (line + a.n_long - 1) / a.n_long;  // too little work to bother with a tail
+  A = max(A, static_cast<long long>(a.min_long_tiles));
+  const long long long_end = A * a.n_long;
+  const int c = a.short_tiles;
+  if (blockIdx.x == 0) {
+    for (int s = t; s <= a.n_seqs; s += kPlanThreads) a.tprefix[s] = lpre[s];
+    if (t == 0) {
+      a.header[0] = static_cast<int>(min(line, 0x7fffffffLL));
+      a.header[1] = static_cast<int>(A), a.header[2] = c, a.header[3] = 0;
+    }
+  }
+  const int k = blockIdx.x * kPlanThreads + t;
+  if (k >= a.max_chunks) return;
+  const long long start = k < a.n_long ? k * A : long_end + static_cast<long long>(k - a.n_long) * c;
+  const long long size = k < a.n_long ? A : c;
+  if (start >= line) {
+    a.chunks[k] = int4{-1, 0, 0, 0};
+    return;
+  }
+  int lo = 0, hi = a.n_seqs;  // largest s with H * prefix[s] <= start (then sequence s is not empty)
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) / 2;
+    if (static_cast<long long>(lpre[mid]) * H <= start) lo = mid; else hi = mid;
+  }
+  const int ts = lpre[lo + 1] - lpre[lo];
+  const int r = static_cast<int>(start - static_cast<long long>(lpre[lo]) * H);
+  a.chunks[k] = int4{lo, r / ts, r % ts, static_cast<int>(min(size, line - start))};
+}
+
+// The chunks of one wavefront: first the long chunk of its own number, then short chunks by ticket until none is
+// left. Calls piece(s, h, first tile, end tile, length, partial number) for every pair a chunk touches. Every wave
+// leaves the loop: tickets only grow and records past the line's end are marked.
+template <typename F>
+__device__ __forceinline__ void WalkChunks(const DecodeArgs& a, F&& piece) {
+  const int H = a.g.n_kv;
+  int k = blockIdx.x;
+  while (k < a.max_chunks) {
+    const int4 rec = a.chunks[k];
+    if (rec.x < 0) break;
+    int ticket = 0;  // taken now, used after the chunk: its latency hides behind the chunk's work
+    if (threadIdx.x == 0) ticket = __hip_atomic_fetch_add(a.header + 3, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    int s = rec.x, h = rec.y, tile = rec.z, left = rec.w;
+    while (left > 0) {
+      const int ts = a.tprefix[s + 1] - a.tprefix[s];
+      if (ts > 0) {
+        const int run = min(left, ts - tile);
+        piece(s, h, tile, tile + run, ClampLen(a, s), k + s * H + h);
+        left -= run;
+      } else {
+        h = H - 1;  // empty sequence: skip all its heads
+      }
+      tile = 0;
+      if (++h == H) h = 0, ++s;
+      if (s >= a.n_seqs) break;
+    }
+    k = a.n_long + __builtin_amdgcn_readfirstlane(ticket);
+  }
 }
 
 // ---- shared pieces ----------------------------------------------------------------------------------------------------
@@ -124,20 +171,17 @@ __device__ __forceinline__ int LaneDimQ4(int lane, int k, int dpl) {
   return (pair / 16) * 32 + pair % 16 + 16 * (k & 1);
 }
 
-// One wavefront per (item, kv head). A lane owns one key for the scores and D / 64 dims for P.V.
+// One wavefront per long chunk. A lane owns one key for the scores and D / 64 dims for P.V.
 template <int D>
 __global__ __launch_bounds__(64) void DattnPartQ4(const DecodeArgs a) {
   constexpr int NB = D / 32, DPL = D / 64, CB = 16;
   const Geom g = a.g;
   const int G = g.group(), H = g.n_kv, PT = g.pt;
-  const int item = blockIdx.x, h = item % H;
-  const int4 rec = a.items[item / H];
-  if (rec.x < 0) return;
-  const int s = rec.x, tile0 = rec.y, tile1 = rec.z, len = rec.w;
   const int lane = threadIdx.x;
-
   __shared__ float qs[kMaxGroup][D];
   __shared__ float ps[kMaxGroup][kTile];
+  WalkChunks(a, [&](int s, int h, int tile0, int tile1, int len, int pid) {
+  __builtin_amdgcn_wave_barrier();  // the previous piece is done with qs
   for (int i = lane; i < G * D; i += 64)
     qs[i / D][i % D] = LoadSrc(a.q, (size_t(s) * g.n_q + size_t(h) * G) * D + i, a.q_dtype);
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -229,7 +273,7 @@ __global__ __launch_bounds__(64) void DattnPartQ4(const DecodeArgs a) {
     __builtin_amdgcn_wave_barrier();  // ps is rewritten by the next tile
   }
 
-  const size_t part = size_t(item) * G;
+  const size_t part = size_t(pid) * G;
 #pragma unroll
   for (int gi = 0; gi < kMaxGroup; ++gi) {
     if (gi < G) {
@@ -238,6 +282,7 @@ __global__ __launch_bounds__(64) void DattnPartQ4(const DecodeArgs a) {
       for (int k = 0; k < DPL; ++k) a.acc[(part + gi) * D + LaneDimQ4(lane, k, DPL)] = acc[gi][k];
     }
   }
+  });
 }
 
 // ---- q8_0 on the matrix cores -----------------------------------------------------------------------------------------
@@ -289,8 +334,8 @@ __device__ __forceinline__ h8v LoadQ8(const void* q, size_t i, int dt) {
   return r;
 }
 
-// One wavefront per (item, kv head), alone in its workgroup: no workgroup barriers anywhere. The wave walks its tiles
-// of 64 keys with an online softmax. Registers hold half a tile of K (32 keys) and half a tile of V (half the dims) at
+// One wavefront per long chunk, alone in its workgroup: no workgroup barriers anywhere. For each (sequence, kv head)
+// pair a chunk of it touches, the wave walks that pair's tiles of 64 keys with an online softmax. Registers hold half a tile of K (32 keys) and half a tile of V (half the dims) at
 // a time, which keeps the kernel under 256 registers, i.e. two waves per SIMD; the four load phases of a tile are
 // rotated against the four arithmetic phases so that every load has arithmetic between its issue and its first use:
 //   scores(keys 0-31)   | load K keys 32-63
@@ -304,10 +349,6 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void Da
   constexpr float kLog2e = 1.4426950408889634f, kLn2 = 0.6931471805599453f;
   const Geom g = a.g;
   const int G = g.group(), H = g.n_kv;
-  const int item = blockIdx.x, h = item % H;
-  const int4 rec = a.items[item / H];
-  if (rec.x < 0) return;
-  const int s = rec.x, tile0 = rec.y, tile1 = rec.z, len = rec.w;
   const int lane = threadIdx.x;
   const int n32 = lane % 32, half = lane / 32;  // score layout: lane = key (mod 32), registers = heads 4 * half + r
   const int n16 = lane % 16, kg = lane / 16;    // P.V layout: lane = dim (mod 16), 16 keys per lane group
@@ -319,12 +360,16 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void Da
   __shared__ __align__(16) _Float16 lq[NB][2][2][8][8];
   __shared__ __align__(16) _Float16 lp[kMaxGroup][kTile];
   __shared__ __align__(16) _Float16 lvs[NB][kTile];
-  for (int i = lane; i < NB * 32; i += 64) {
-    const int b = i / 32, sub = (i / 16) % 2, hf = (i / 8) % 2, rw = i % 8;
-    h8v v = {0, 0, 0, 0, 0, 0, 0, 0};
+  WalkChunks(a, [&](int s, int h, int tile0, int tile1, int len, int pid) {
+  // The piece's query rows, in flight while the first K and V loads are issued below.
+  constexpr int QE = NB * 32 / 64;  // lq entries per lane
+  h8v qreg[QE];
+#pragma unroll
+  for (int e = 0; e < QE; ++e) {
+    const int i = lane + 64 * e, b = i / 32, sub = (i / 16) % 2, hf = (i / 8) % 2, rw = i % 8;
+    qreg[e] = h8v{0, 0, 0, 0, 0, 0, 0, 0};
     if (rw < G)
-      v = LoadQ8(a.q, (size_t(s) * g.n_q + size_t(h) * G + rw) * D + b * 32 + 16 * hf + 8 * sub, a.q_dtype);
-    *reinterpret_cast<h8v*>(&lq[b][sub][hf][rw][0]) = v;
+      qreg[e] = LoadQ8(a.q, (size_t(s) * g.n_q + size_t(h) * G + rw) * D + b * 32 + 16 * hf + 8 * sub, a.q_dtype);
   }
 
   const int32_t* row = a.table + int64_t(s) * a.stride;
@@ -435,6 +480,12 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void Da
   load_pages(tile0, pgc);
   load_k(0, pgc);
   load_v(0, pgc);
+  __builtin_amdgcn_wave_barrier();  // the previous piece is done with lq
+#pragma unroll
+  for (int e = 0; e < QE; ++e) {
+    const int i = lane + 64 * e;
+    *reinterpret_cast<h8v*>(&lq[i / 32][(i / 16) % 2][(i / 8) % 2][i % 8][0]) = qreg[e];
+  }
   for (int tile = tile0; tile < tile1; ++tile) {
     const bool has_next = tile + 1 < tile1;
     if (has_next) load_pages(tile + 1, pgn);
@@ -491,8 +542,8 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void Da
   }
   pv(1);
 
-  // ---- the item's partial, straight from registers (natural-log units, as the reduce expects)
-  const size_t part = size_t(item) * G;
+  // ---- the piece's partial, straight from registers (natural-log units, as the reduce expects)
+  const size_t part = size_t(pid) * G;
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     const float l = HalfSum32(lsum[r]);
@@ -509,27 +560,36 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void Da
       }
     }
   }
+  });
 }
 
 // ---- reduce -------------------------------------------------------------------------------------------------------------
 
-// One workgroup per (query head, sequence), thread = dim (gen_decode_attn.py:338-411).
+// One workgroup per (query head, sequence), thread = dim (gen_decode_attn.py:338-411). The pair's partials are those
+// of the chunks its stretch of the line overlaps.
 __global__ void DattnReduce(const DecodeArgs a) {
   const Geom g = a.g;
   const int G = g.group(), H = g.n_kv, D = g.hd;
   const int hq = blockIdx.x, s = blockIdx.y, d = threadIdx.x;
   const int h = hq / G, gi = hq % G;
   const size_t o = (size_t(s) * g.n_q + hq) * D + d;
-  const int c0 = min(a.prefix[s], a.max_chunks), c1 = min(a.prefix[s + 1], a.max_chunks);
-  if (c0 >= c1) {  // length 0
+  const int ts = a.tprefix[s + 1] - a.tprefix[s];
+  if (ts <= 0) {  // length 0
     a.out[o] = 0.0f;
     return;
   }
+  const int A_ = a.header[1], c = a.header[2], pair = s * H + h;
+  const long long long_end = static_cast<long long>(A_) * a.n_long;
+  const long long first = static_cast<long long>(a.tprefix[s]) * H + static_cast<long long>(h) * ts, last = first + ts - 1;
+  auto chunk_of = [&](long long pos) {
+    return static_cast<int>(pos < long_end ? pos / A_ : a.n_long + (pos - long_end) / c);
+  };
+  const int k0 = chunk_of(first), k1 = chunk_of(last);
   float M = kNegMax;
-  for (int c = c0; c < c1; ++c) M = fmaxf(M, a.ml[((size_t(c) * H + h) * G + gi) * 2]);
+  for (int k = k0; k <= k1; ++k) M = fmaxf(M, a.ml[(size_t(k + pair) * G + gi) * 2]);
   float L = 0.0f, A = 0.0f;
-  for (int c = c0; c < c1; ++c) {
-    const size_t p = (size_t(c) * H + h) * G + gi;
+  for (int k = k0; k <= k1; ++k) {
+    const size_t p = size_t(k + pair) * G + gi;
     const float w = __expf(a.ml[p * 2] - M);
     L = __builtin_fmaf(w, a.ml[p * 2 + 1], L);
     A = __builtin_fmaf(w, a.acc[p * D + d], A);
@@ -541,29 +601,47 @@ __global__ void DattnReduce(const DecodeArgs a) {
 
 // ---- host side ----------------------------------------------------------------------------------------------------------
 
-// Workspace layout and item sizing from the host's bounds alone (the lengths themselves are on the device).
+// Workspace layout and chunk counts, from the host's bounds alone (the lengths are on the device).
 struct Plan {
-  int32_t max_len, max_chunks, min_tiles_per_item, target_items;
-  size_t off_prefix, off_items, off_ml, off_acc, bytes;
+  int32_t max_len, n_long, max_chunks, min_long_tiles, short_tiles, short_permille;
+  size_t off_tprefix, off_chunks, off_ml, off_acc, bytes;
 };
 size_t Align(size_t x) { return (x + 255) & ~size_t(255); }
+int WaveSlots() {  // wavefronts the chip holds at two per SIMD
+  static const int slots = [] {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+      cus = 256;
+    return cus * 8;
+  }();
+  return slots;
+}
+int EnvInt(const char* name, int fallback, int lo, int hi) {
+  const char* e = std::getenv(name);
+  return e == nullptr ? fallback : std::min(hi, std::max(lo, std::atoi(e)));
+}
 Plan MakePlan(const Geom& g, int32_t n_seqs, int32_t max_seq_len) {
   Plan p;
   p.max_len = std::max(max_seq_len, 1);
   const int64_t max_tiles = (int64_t(p.max_len) + kTile - 1) / kTile;
-  // About six items per wave slot (256 CUs x 8 waves) when the batch is large; never more than 16384 records.
-  p.target_items = 12288;
-  if (const char* e = std::getenv("YAHKV_DECODE_TARGET_ITEMS")) p.target_items = std::max(1, std::atoi(e));
-  int64_t tpi = (max_tiles * n_seqs * g.n_kv + 16383) / 16384;
-  if (const char* e = std::getenv("YAHKV_DECODE_MIN_TILES_PER_ITEM")) tpi = std::max<int64_t>(tpi, std::atoll(e));
-  p.min_tiles_per_item = static_cast<int32_t>(std::max<int64_t>(tpi, 2));
-  p.max_chunks = static_cast<int32_t>(n_seqs * ((max_tiles + p.min_tiles_per_item - 1) / p.min_tiles_per_item));
-  const size_t items = size_t(p.max_chunks) * g.n_kv;
-  p.off_prefix = 256;
-  p.off_items = Align(p.off_prefix + sizeof(int32_t) * (size_t(n_seqs) + 1));
-  p.off_ml = Align(p.off_items + sizeof(int4) * size_t(p.max_chunks));
-  p.off_acc = Align(p.off_ml + sizeof(float) * items * g.group() * 2);
-  p.bytes = Align(p.off_acc + sizeof(float) * items * g.group() * g.hd);
+  // Tuning knobs (environment overrides are for experiments): a short line is not cut finer than min_long_tiles per
+  // wave, because each piece costs a partial (G x (D + 2) floats); the last short_permille / 1000 of the line goes
+  // out in chunks of short_tiles.
+  p.min_long_tiles = EnvInt("YAHKV_DECODE_MIN_LONG_TILES", 2, 1, 1 << 20);
+  p.short_tiles = EnvInt("YAHKV_DECODE_SHORT_TILES", 8, 1, 1 << 20);
+  p.short_permille = EnvInt("YAHKV_DECODE_SHORT_PERMILLE", 0, 0, 900);  // measured: no gain on the ragged batch
+  const int slots = EnvInt("YAHKV_DECODE_WAVES", WaveSlots(), 1, 1 << 20);
+  const int64_t line_max = max_tiles * n_seqs * g.n_kv;
+  p.n_long = static_cast<int32_t>(std::min<int64_t>(slots, (line_max + p.min_long_tiles - 1) / p.min_long_tiles));
+  const int64_t short_max = (line_max * p.short_permille / 1000 + p.short_tiles - 1) / p.short_tiles + 1;
+  p.max_chunks = static_cast<int32_t>(p.n_long + short_max);
+  const size_t parts = size_t(p.max_chunks) + size_t(n_seqs) * g.n_kv;
+  p.off_tprefix = 256;
+  p.off_chunks = Align(p.off_tprefix + sizeof(int32_t) * (size_t(n_seqs) + 1));
+  p.off_ml = Align(p.off_chunks + sizeof(int4) * size_t(p.max_chunks));
+  p.off_acc = Align(p.off_ml + sizeof(float) * parts * g.group() * 2);
+  p.bytes = Align(p.off_acc + sizeof(float) * parts * g.group() * g.hd);
   return p;
 }
 
@@ -573,6 +651,7 @@ int Prepare(const yahkv_geometry* g, int32_t page_table_stride, const int32_t* s
   if (const int st = CheckGeometry(g)) return st;
   if (seq_len == nullptr || workspace == nullptr) return YAHKV_ERR_ARG;
   if (n_seqs <= 0 || max_seq_len <= 0 || page_table_stride <= 0) return YAHKV_ERR_ARG;
+  if (n_seqs > kMaxSeqs) return YAHKV_ERR_SHAPE;  // the plan kernel keeps one integer per sequence in LDS
   if (reinterpret_cast<uintptr_t>(workspace) & 15) return YAHKV_ERR_ARG;
   const Geom m = MakeGeom(*g);
   const Plan p = MakePlan(m, n_seqs, max_seq_len);
@@ -583,11 +662,12 @@ int Prepare(const yahkv_geometry* g, int32_t page_table_stride, const int32_t* s
   a->max_len = static_cast<int32_t>(std::min<int64_t>(p.max_len, int64_t(page_table_stride) * m.pt));
   char* ws = static_cast<char*>(const_cast<void*>(workspace));
   a->header = reinterpret_cast<int32_t*>(ws);
-  a->prefix = reinterpret_cast<int32_t*>(ws + p.off_prefix);
-  a->items = reinterpret_cast<int4*>(ws + p.off_items);
+  a->tprefix = reinterpret_cast<int32_t*>(ws + p.off_tprefix);
+  a->chunks = reinterpret_cast<int4*>(ws + p.off_chunks);
   a->ml = reinterpret_cast<float*>(ws + p.off_ml);
   a->acc = reinterpret_cast<float*>(ws + p.off_acc);
-  a->max_chunks = p.max_chunks, a->min_tiles_per_item = p.min_tiles_per_item, a->target_items = p.target_items;
+  a->n_long = p.n_long, a->max_chunks = p.max_chunks;
+  a->min_long_tiles = p.min_long_tiles, a->short_tiles = p.short_tiles, a->short_permille = p.short_permille;
   return YAHKV_OK;
 }
 
@@ -619,9 +699,10 @@ extern "C" int yahkv_decode_part(const yahkv_geometry* g, const yahkv_pools* poo
   a.pools = MakePools(*pools), a.table = page_table, a.q = q, a.q_dtype = q_dtype, a.scale = softmax_scale;
   const Geom& m = a.g;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  hipLaunchKernelGGL(DattnPlan, dim3(1), dim3(kPlanThreads), 0, st, a);
+  hipLaunchKernelGGL(DattnPlan, dim3((a.max_chunks + kPlanThreads - 1) / kPlanThreads), dim3(kPlanThreads),
+                     sizeof(int) * (size_t(n_seqs) + 1), st, a);
   if (const int ls = LaunchStatus()) return ls;
-  const dim3 grid(static_cast<unsigned>(a.max_chunks) * m.n_kv);
+  const dim3 grid(static_cast<unsigned>(a.n_long));
   if (m.format == 8) {
 #define YAHKV_LAUNCH_Q8(DD, PP) hipLaunchKernelGGL((DattnPartQ8<DD, PP>), grid, dim3(64), 0, st, a)
     if (m.hd == 256 && m.pt == 64) YAHKV_LAUNCH_Q8(256, 64);
