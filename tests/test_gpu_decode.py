@@ -81,7 +81,8 @@ def test_config1_tiny(yahkv, torch_gpu):
 
 
 @pytest.mark.parametrize("fmt,n_q,n_kv,hd,pt", [(8, 24, 4, 256, 64), (4, 24, 4, 256, 64), (8, 8, 2, 128, 16),
-                                                 (4, 8, 2, 128, 16), (8, 8, 1, 256, 32), (8, 4, 4, 128, 64)])
+                                                 (4, 8, 2, 128, 16), (8, 8, 1, 256, 32), (8, 4, 4, 128, 64), (8, 16, 2, 256, 16),
+                                                 (8, 24, 4, 128, 32)])
 def test_ragged_batch_with_gate(yahkv, torch_gpu, fmt, n_q, n_kv, hd, pt):
     torch = torch_gpu
     lens = [1, pt - 1, pt, pt + 1, 63, 64, 65, 5 * 64 + 17, 1500, 0, 257]

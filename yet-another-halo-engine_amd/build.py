@@ -9,6 +9,7 @@ SOURCES = ["host.cpp", "append.hip", "decode.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",   # no packed-FP32 VALU forms
+         "-mllvm", "--disable-promote-alloca-to-lds",                   # small private arrays stay out of LDS
          "-x", "hip"]
 
 

@@ -8,11 +8,14 @@
 //
 // The reference launches one workgroup per 256-key page of its single sequence. Here lengths are ragged and live on
 // the device, so the work is cut stream-K style: all (sequence, kv head) pairs are laid end to end on one line of
-// 64-key tiles and the line is cut into chunks. The first chunks are long and equal, one per wavefront slot of the chip
-// (every wave starts with the same amount of work whatever the mix of lengths); the last part of the line is cut into
-// short chunks that waves take from a counter as they finish, because waves do not run at one speed (the XCDs do not
-// all see the same bandwidth). A wave leaves one partial per (chunk, pair) it touches. A small `plan` kernel computes
-// the cut from the device-resident lengths.
+// 64-key tiles and the line is cut into equal chunks, one per workgroup, one workgroup per CU: every CU gets the same
+// number of tiles whatever the mix of lengths, in a single round. Inside a workgroup the waves take the chunk's tiles
+// one by one from an LDS counter, because waves of one CU do not run at one speed (the older wave of a SIMD wins the
+// issue arbitration); each wave keeps its own online softmax and leaves one partial per pair it worked on. A small
+// `plan` kernel computes the cut from the device-resident lengths.
+// (Measured and dropped: finishing the line with short chunks or single tiles handed out dynamically, by a counter in
+// global memory or by the dispatcher, to even out the XCDs, which finish up to 10 % apart. Every variant was slower:
+// each change of pair costs a wave a pipeline fill, and the XCDs that finish first leave their bandwidth to the rest.)
 #include <algorithm>
 #include <cstdlib>
 
@@ -26,6 +29,7 @@ constexpr int kTile = 64;     // keys per tile: one wavefront, one key per lane 
 constexpr int kMaxGroup = 8;  // query heads per kv head
 constexpr int kPlanThreads = 256;
 constexpr int kMaxSeqs = 8191;
+constexpr int kWavesPerGroup = 8;  // q8_0 kernel: one workgroup fills a CU at two waves per SIMD
 
 struct DecodeArgs {
   Geom g;
@@ -40,13 +44,13 @@ struct DecodeArgs {
   const float* gate;
   float* out;
   // workspace
-  int32_t* header;   // [0] tiles on the line, [1] tiles per long chunk, [2] tiles per short chunk, [3] ticket counter
+  int32_t* header;   // [0] tiles on the line, [1] tiles per chunk
   int32_t* tprefix;  // [n_seqs + 1] tiles of all earlier sequences (one kv head's worth)
-  int4* chunks;      // [max_chunks] {sequence or -1, kv head, first tile within the pair, tiles in the chunk}
-  float* ml;         // [max_chunks + n_seqs * H][G][2]   partial of (chunk k, pair p) is number k + p
-  float* acc;        // [max_chunks + n_seqs * H][G][D]
-  int32_t n_long, max_chunks;    // long chunks = wavefronts launched; records in `chunks`
-  int32_t min_long_tiles, short_tiles, short_permille;
+  int4* chunks;      // [n_chunks] {sequence or -1, kv head, first tile within the pair, tiles in the chunk}
+  float* ml;         // [(n_chunks + n_seqs * H) * wpc][G][2]   partial of (chunk k, wave w, pair p): (k + p) * wpc + w
+  float* acc;        // [(n_chunks + n_seqs * H) * wpc][G][D]
+  int32_t n_chunks, wpc;  // chunks = workgroups launched; waves per chunk
+  int32_t min_chunk_tiles;
 };
 
 __device__ __forceinline__ int ClampLen(const DecodeArgs& a, int s) { return min(max(a.seq_len[s], 0), a.max_len); }
@@ -54,9 +58,8 @@ __device__ __forceinline__ int ClampLen(const DecodeArgs& a, int s) { return min
 // ---- plan -------------------------------------------------------------------------------------------------------------
 
 // Every workgroup recomputes the prefix sums of the sequences' tile counts in LDS (a few hundred integers), then each
-// thread writes one chunk record. Workgroup 0 also publishes the prefix sums, the chunk sizes and a zeroed ticket
-// counter. Chunk k < n_long covers tiles [k A, (k + 1) A) of the line, chunk n_long + i covers
-// [n_long A + i c, n_long A + (i + 1) c), both clipped to the line's length.
+// thread writes one chunk record. Workgroup 0 also publishes the prefix sums and the chunk size. Chunk k covers tiles
+// [k A, (k + 1) A) of the line, clipped to the line's length.
 __global__ __launch_bounds__(kPlanThreads) void DattnPlan(const DecodeArgs a) {
   extern __shared__ int lpre[];  // [n_seqs + 1]
   __shared__ int part_sum[kPlanThreads];
@@ -79,23 +82,15 @@ __global__ __launch_bounds__(kPlanThreads) void DattnPlan(const DecodeArgs a) {
   if (t == 0) lpre[a.n_seqs] = total;
   __syncthreads();
   const long long line = static_cast<long long>(total) * H;  // tiles on the line
-  // long chunks share (1 - short_permille / 1000) of the line, but a short line is not cut finer than min_long_tiles
-  long long A = line * (1000 - a.short_permille) / 1000 / a.n_long;
-  if (A < 4LL * a.short_tiles) A = (line + a.n_long - 1) / a.n_long;  // too little work to bother with a tail
-  A = max(A, static_cast<long long>(a.min_long_tiles));
-  const long long long_end = A * a.n_long;
-  const int c = a.short_tiles;
+  // a short line is not cut finer than min_chunk_tiles: each piece costs a partial (G x (D + 2) floats)
+  const long long A = max((line + a.n_chunks - 1) / a.n_chunks, static_cast<long long>(a.min_chunk_tiles));
   if (blockIdx.x == 0) {
     for (int s = t; s <= a.n_seqs; s += kPlanThreads) a.tprefix[s] = lpre[s];
-    if (t == 0) {
-      a.header[0] = static_cast<int>(min(line, 0x7fffffffLL));
-      a.header[1] = static_cast<int>(A), a.header[2] = c, a.header[3] = 0;
-    }
+    if (t == 0) a.header[0] = static_cast<int>(min(line, 0x7fffffffLL)), a.header[1] = static_cast<int>(A);
   }
   const int k = blockIdx.x * kPlanThreads + t;
-  if (k >= a.max_chunks) return;
-  const long long start = k < a.n_long ? k * A : long_end + static_cast<long long>(k - a.n_long) * c;
-  const long long size = k < a.n_long ? A : c;
+  if (k >= a.n_chunks) return;
+  const long long start = k * A;
   if (start >= line) {
     a.chunks[k] = int4{-1, 0, 0, 0};
     return;
@@ -107,37 +102,34 @@ __global__ __launch_bounds__(kPlanThreads) void DattnPlan(const DecodeArgs a) {
   }
   const int ts = lpre[lo + 1] - lpre[lo];
   const int r = static_cast<int>(start - static_cast<long long>(lpre[lo]) * H);
-  a.chunks[k] = int4{lo, r / ts, r % ts, static_cast<int>(min(size, line - start))};
+  a.chunks[k] = int4{lo, r / ts, r % ts, static_cast<int>(min(A, line - start))};
 }
 
-// The chunks of one wavefront: first the long chunk of its own number, then short chunks by ticket until none is
-// left. Calls piece(s, h, first tile, end tile, length, partial number) for every pair a chunk touches. Every wave
-// leaves the loop: tickets only grow and records past the line's end are marked.
-template <typename F>
-__device__ __forceinline__ void WalkChunks(const DecodeArgs& a, F&& piece) {
-  const int H = a.g.n_kv;
-  int k = blockIdx.x;
-  while (k < a.max_chunks) {
-    const int4 rec = a.chunks[k];
-    if (rec.x < 0) break;
-    int ticket = 0;  // taken now, used after the chunk: its latency hides behind the chunk's work
-    if (threadIdx.x == 0) ticket = __hip_atomic_fetch_add(a.header + 3, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    int s = rec.x, h = rec.y, tile = rec.z, left = rec.w;
-    while (left > 0) {
-      const int ts = a.tprefix[s + 1] - a.tprefix[s];
-      if (ts > 0) {
-        const int run = min(left, ts - tile);
-        piece(s, h, tile, tile + run, ClampLen(a, s), k + s * H + h);
-        left -= run;
-      } else {
-        h = H - 1;  // empty sequence: skip all its heads
-      }
-      tile = 0;
-      if (++h == H) h = 0, ++s;
-      if (s >= a.n_seqs) break;
-    }
-    k = a.n_long + __builtin_amdgcn_readfirstlane(ticket);
-  }
+// Position of a wave on its chunk: the pair (s, h) it stands on, which of the chunk's tiles belong to that pair
+// ([base, base + n) in chunk numbering, starting at the pair's tile `first`), and that sequence's length.
+struct PairCursor {
+  int s, h, first, base, n, len;
+};
+__device__ __forceinline__ PairCursor FirstPair(const DecodeArgs& a, const int4 rec) {
+  const int ts = a.tprefix[rec.x + 1] - a.tprefix[rec.x];
+  return PairCursor{rec.x, rec.y, rec.z, 0, min(ts - rec.z, rec.w), ClampLen(a, rec.x)};
+}
+// Next pair of the chunk; false when the chunk (of chunk_n tiles) ends with the current pair.
+__device__ __forceinline__ bool NextPair(const DecodeArgs& a, int chunk_n, PairCursor* c) {
+  if (c->base + c->n >= chunk_n) return false;
+  c->base += c->n, c->first = 0;
+  int ts = 0;
+  do {  // empty sequences have no tiles on the line
+    if (++c->h == a.g.n_kv) c->h = 0, ++c->s;
+    if (c->s >= a.n_seqs) return false;
+    ts = a.tprefix[c->s + 1] - a.tprefix[c->s];
+    if (ts == 0) c->h = a.g.n_kv - 1;
+  } while (ts == 0);
+  c->n = min(ts, chunk_n - c->base), c->len = ClampLen(a, c->s);
+  return true;
+}
+__device__ __forceinline__ size_t PartialIndex(const DecodeArgs& a, int chunk, int wave, const PairCursor& c) {
+  return (size_t(chunk) + size_t(c.s) * a.g.n_kv + c.h) * a.wpc + wave;
 }
 
 // ---- shared pieces ----------------------------------------------------------------------------------------------------
@@ -171,7 +163,7 @@ __device__ __forceinline__ int LaneDimQ4(int lane, int k, int dpl) {
   return (pair / 16) * 32 + pair % 16 + 16 * (k & 1);
 }
 
-// One wavefront per long chunk. A lane owns one key for the scores and D / 64 dims for P.V.
+// One wavefront per chunk. A lane owns one key for the scores and D / 64 dims for P.V.
 template <int D>
 __global__ __launch_bounds__(64) void DattnPartQ4(const DecodeArgs a) {
   constexpr int NB = D / 32, DPL = D / 64, CB = 16;
@@ -180,8 +172,12 @@ __global__ __launch_bounds__(64) void DattnPartQ4(const DecodeArgs a) {
   const int lane = threadIdx.x;
   __shared__ float qs[kMaxGroup][D];
   __shared__ float ps[kMaxGroup][kTile];
-  WalkChunks(a, [&](int s, int h, int tile0, int tile1, int len, int pid) {
-  __builtin_amdgcn_wave_barrier();  // the previous piece is done with qs
+  const int4 rec = a.chunks[blockIdx.x];
+  if (rec.x < 0) return;
+  PairCursor cur = FirstPair(a, rec);
+  do {
+  const int s = cur.s, h = cur.h, tile0 = cur.first, tile1 = cur.first + cur.n, len = cur.len;
+  __builtin_amdgcn_wave_barrier();  // the previous pair is done with qs
   for (int i = lane; i < G * D; i += 64)
     qs[i / D][i % D] = LoadSrc(a.q, (size_t(s) * g.n_q + size_t(h) * G) * D + i, a.q_dtype);
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -273,7 +269,7 @@ __global__ __launch_bounds__(64) void DattnPartQ4(const DecodeArgs a) {
     __builtin_amdgcn_wave_barrier();  // ps is rewritten by the next tile
   }
 
-  const size_t part = size_t(pid) * G;
+  const size_t part = PartialIndex(a, blockIdx.x, 0, cur) * G;
 #pragma unroll
   for (int gi = 0; gi < kMaxGroup; ++gi) {
     if (gi < G) {
@@ -282,7 +278,7 @@ __global__ __launch_bounds__(64) void DattnPartQ4(const DecodeArgs a) {
       for (int k = 0; k < DPL; ++k) a.acc[(part + gi) * D + LaneDimQ4(lane, k, DPL)] = acc[gi][k];
     }
   }
-  });
+  } while (NextPair(a, rec.w, &cur));
 }
 
 // ---- q8_0 on the matrix cores -----------------------------------------------------------------------------------------
@@ -334,22 +330,27 @@ __device__ __forceinline__ h8v LoadQ8(const void* q, size_t i, int dt) {
   return r;
 }
 
-// One wavefront per long chunk, alone in its workgroup: no workgroup barriers anywhere. For each (sequence, kv head)
-// pair a chunk of it touches, the wave walks that pair's tiles of 64 keys with an online softmax. Registers hold half a tile of K (32 keys) and half a tile of V (half the dims) at
-// a time, which keeps the kernel under 256 registers, i.e. two waves per SIMD; the four load phases of a tile are
-// rotated against the four arithmetic phases so that every load has arithmetic between its issue and its first use:
-//   scores(keys 0-31)   | load K keys 32-63
+// One workgroup of eight waves per chunk, one workgroup per CU (two waves per SIMD). The waves share nothing but the
+// LDS counter that hands out the chunk's tiles; after the first barrier no wave waits for another. A wave takes tiles
+// in increasing order, so it meets the chunk's (sequence, kv head) pairs in order; for each pair it worked on it keeps
+// an online softmax over its tiles and leaves one partial, for a pair it got no tile of it leaves l = 0.
+//
+// Registers hold half a tile of K (32 keys) and half a tile of V (half the dims) at a time, which keeps the kernel at
+// 256 registers; the four load phases of a tile are rotated against the four arithmetic phases so that every load has
+// arithmetic between its issue and its first use:
+//   scores(keys 0-31)              | load K keys 32-63
 //   P.V(dims D/2.., previous tile) | load V dims 0..D/2 of this tile
-//   scores(keys 32-63)  | load K keys 0-31 of the next tile
+//   scores(keys 32-63)             | load K keys 0-31 of the wave's next tile
 //   softmax, P.V(dims 0..D/2)      | load V dims D/2.. of this tile
 // Page numbers come through scalar loads (they are the same for the whole wave).
 template <int D, int PT>
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void DattnPartQ8(const DecodeArgs a) {
+__global__ __launch_bounds__(64 * kWavesPerGroup) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void DattnPartQ8(const DecodeArgs a) {
   constexpr int NB = D / 32, NT = D / 16, PPT = kTile / PT;
   constexpr float kLog2e = 1.4426950408889634f, kLn2 = 0.6931471805599453f;
   const Geom g = a.g;
   const int G = g.group(), H = g.n_kv;
-  const int lane = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64), lane = threadIdx.x % 64;
   const int n32 = lane % 32, half = lane / 32;  // score layout: lane = key (mod 32), registers = heads 4 * half + r
   const int n16 = lane % 16, kg = lane / 16;    // P.V layout: lane = dim (mod 16), 16 keys per lane group
 
@@ -357,22 +358,38 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void Da
   // 32-row A matrix is head m; only rows 0-7 exist here and lanes of rows 8-31 re-read them (their output rows are
   // never looked at). Entry (b, sub, hf, row) holds dims 32 b + 16 hf + 8 sub + 0..7, the dims of the 8 code bytes a
   // key lane of that half feeds to instruction `sub`.
-  __shared__ __align__(16) _Float16 lq[NB][2][2][8][8];
-  __shared__ __align__(16) _Float16 lp[kMaxGroup][kTile];
-  __shared__ __align__(16) _Float16 lvs[NB][kTile];
-  WalkChunks(a, [&](int s, int h, int tile0, int tile1, int len, int pid) {
-  // The piece's query rows, in flight while the first K and V loads are issued below.
-  constexpr int QE = NB * 32 / 64;  // lq entries per lane
-  h8v qreg[QE];
-#pragma unroll
-  for (int e = 0; e < QE; ++e) {
-    const int i = lane + 64 * e, b = i / 32, sub = (i / 16) % 2, hf = (i / 8) % 2, rw = i % 8;
-    qreg[e] = h8v{0, 0, 0, 0, 0, 0, 0, 0};
-    if (rw < G)
-      qreg[e] = LoadQ8(a.q, (size_t(s) * g.n_q + size_t(h) * G + rw) * D + b * 32 + 16 * hf + 8 * sub, a.q_dtype);
-  }
+  __shared__ __align__(16) _Float16 lq_all[kWavesPerGroup][NB][2][2][8][8];
+  __shared__ __align__(16) _Float16 lp_all[kWavesPerGroup][kMaxGroup][kTile];
+  __shared__ __align__(16) _Float16 lvs_all[kWavesPerGroup][NB][kTile];
+  __shared__ int next_tile;
+  auto& lq = lq_all[wave];
+  auto& lp = lp_all[wave];
+  auto& lvs = lvs_all[wave];
 
-  const int32_t* row = a.table + int64_t(s) * a.stride;
+  const int4 rec = a.chunks[blockIdx.x];
+  if (rec.x < 0) return;
+  const int chunk_n = rec.w;
+  if (threadIdx.x == 0) next_tile = 0;
+  __syncthreads();
+  auto take = [&]() -> int {  // the next tile of the chunk nobody has taken yet (>= chunk_n: none left)
+    int v = 0;
+    if (lane == 0) v = __hip_atomic_fetch_add(&next_tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    return __builtin_amdgcn_readfirstlane(v);
+  };
+
+  uint4 kb[NB];      // [block]: 16 codes of this lane's key (one 32-key half of the tile at a time)
+  uint4 ksc;         // that key's NB block scales (f16)
+  uint4 vb[NT / 2];  // [16-dim tile]: 16 keys of this lane's dim (one half of the dims at a time)
+  uint4 vsr;         // staging of the tile's V scales: 8 keys of one block per lane
+  float m[4], lsum[4], sc[2][4];
+  f4v o[NT];
+  const float qk_scale = a.scale * kLog2e;  // softmax in base 2
+  // P rows read back as A-matrix rows: rows 0-3 are heads 0-3, rows 8-11 heads 4-7, so that a lane's output rows are
+  // the heads whose running maximum it already holds (lanes 0-15: heads 0-3, lanes 32-47: heads 4-7).
+  const int prow = n16 < 4 ? n16 : (n16 >= 8 && n16 < 12 ? n16 - 4 : 0);
+
+  PairCursor cur = FirstPair(a, rec);
+  const int32_t* row = nullptr;
   auto load_pages = [&](int tile, int (&pg)[PPT]) {
 #pragma unroll
     for (int j = 0; j < PPT; ++j) pg[j] = ClampPage(row[min(tile * PPT + j, a.stride - 1)], g.n_pages);
@@ -381,13 +398,8 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void Da
     int p = pg[0];
 #pragma unroll
     for (int j = 1; j < PPT; ++j) p = tok_in_tile / PT == j ? pg[j] : p;
-    return size_t(p) * H + h;
+    return size_t(p) * H + cur.h;
   };
-
-  uint4 kb[NB];      // [block]: 16 codes of this lane's key (one 32-key half of the tile at a time)
-  uint4 ksc;         // that key's NB block scales (f16)
-  uint4 vb[NT / 2];  // [16-dim tile]: 16 keys of this lane's dim (one half of the dims at a time)
-  uint4 vsr;         // staging of the tile's V scales: 8 keys of one block per lane
   auto load_k = [&](int tt, const int (&pg)[PPT]) {
     const int tk = 32 * tt + n32;
     const size_t ph = page_head(pg, tk);
@@ -417,18 +429,6 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void Da
       }
     }
   };
-
-  float m[4], lsum[4], sc[2][4];
-  f4v o[NT];
-#pragma unroll
-  for (int r = 0; r < 4; ++r) m[r] = kNegMax, lsum[r] = 0.0f;
-#pragma unroll
-  for (int nt = 0; nt < NT; ++nt) o[nt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
-  const float qk_scale = a.scale * kLog2e;  // softmax in base 2
-  // P rows read back as A-matrix rows: rows 0-3 are heads 0-3, rows 8-11 heads 4-7, so that a lane's output rows are
-  // the heads whose running maximum it already holds (lanes 0-15: heads 0-3, lanes 32-47: heads 4-7).
-  const int prow = n16 < 4 ? n16 : (n16 >= 8 && n16 < 12 ? n16 - 4 : 0);
-
   // scores of the 32 keys in kb against all heads: two blocks (two accumulator chains) at a time
   auto scores = [&](int tt) {
 #pragma unroll
@@ -475,92 +475,141 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void Da
       __builtin_amdgcn_sched_barrier(0);
     }
   };
-
-  int pgc[PPT], pgn[PPT];
-  load_pages(tile0, pgc);
-  load_k(0, pgc);
-  load_v(0, pgc);
-  __builtin_amdgcn_wave_barrier();  // the previous piece is done with lq
-#pragma unroll
-  for (int e = 0; e < QE; ++e) {
-    const int i = lane + 64 * e;
-    *reinterpret_cast<h8v*>(&lq[i / 32][(i / 16) % 2][(i / 8) % 2][i % 8][0]) = qreg[e];
-  }
-  for (int tile = tile0; tile < tile1; ++tile) {
-    const bool has_next = tile + 1 < tile1;
-    if (has_next) load_pages(tile + 1, pgn);
-    scores(0);
-    load_k(1, pgc);
-    if (tile > tile0) {
-      pv(1);  // second half of the previous tile's P.V: lp and lvs still hold that tile
-      load_v(0, pgc);
-    }
-    scores(1);
-    if (has_next) load_k(0, pgn);
-    // ---- online softmax (base 2); keys at or past len are masked by select, so stale scales cannot leak
-    float alpha[4];
-#pragma unroll
-    for (int tt = 0; tt < 2; ++tt) {
-      const bool valid = tile * kTile + 32 * tt + n32 < len;
-#pragma unroll
-      for (int r = 0; r < 4; ++r) sc[tt][r] = valid ? sc[tt][r] : kNegMax;
-    }
+  // l = 0 for a pair this wave got no tile of (the reduce then skips it)
+  auto leave_empty = [&]() {
+    const size_t part = PartialIndex(a, blockIdx.x, wave, cur) * G;
+    if (lane < G) a.ml[(part + lane) * 2] = kNegMax, a.ml[(part + lane) * 2 + 1] = 0.0f;
+  };
+  // the pair's partial, straight from registers (natural-log units, as the reduce expects)
+  auto leave_partial = [&]() {
+    const size_t part = PartialIndex(a, blockIdx.x, wave, cur) * G;
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      const float mn = fmaxf(m[r], HalfMax32(fmaxf(sc[0][r], sc[1][r])));
-      alpha[r] = __builtin_amdgcn_exp2f(m[r] - mn);
-      m[r] = mn;
-      const float p0 = __builtin_amdgcn_exp2f(sc[0][r] - mn), p1 = __builtin_amdgcn_exp2f(sc[1][r] - mn);
-      lsum[r] = __builtin_fmaf(lsum[r], alpha[r], p0 + p1);  // per lane; summed over the lanes at the end
-      lp[4 * half + r][n32] = static_cast<_Float16>(p0);
-      lp[4 * half + r][32 + n32] = static_cast<_Float16>(p1);
+      const float l = HalfSum32(lsum[r]);
+      const int head = 4 * half + r;
+      if (n32 == 0 && head < G) a.ml[(part + head) * 2] = m[r] * kLn2, a.ml[(part + head) * 2 + 1] = l;
     }
-    {  // V scales of the tile to LDS; scales of keys at or past len become 0, which makes their V rows 0
-      const int b = lane / 8, chunk = lane % 8;
-      if (b < NB) {
-        uint32_t w[4] = {vsr.x, vsr.y, vsr.z, vsr.w};
-        const int k0 = tile * kTile + 8 * chunk;
-        if (k0 + 8 > len) {
+    if (kg == 0 || kg == 2) {
 #pragma unroll
-          for (int j = 0; j < 8; ++j)
-            if (k0 + j >= len) w[j / 2] &= j % 2 ? 0x0000FFFFu : 0xFFFF0000u;
+      for (int r = 0; r < 4; ++r) {
+        const int head = 2 * kg + r;
+        if (head < G) {
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt) a.acc[(part + head) * D + 16 * nt + n16] = o[nt][r];
         }
-        *reinterpret_cast<uint4*>(&lvs[b][8 * chunk]) = uint4{w[0], w[1], w[2], w[3]};
       }
     }
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) o[nt][r] *= alpha[r];
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    pv(0);
-    load_v(1, pgc);
-#pragma unroll
-    for (int j = 0; j < PPT; ++j) pgc[j] = pgn[j];
-  }
-  pv(1);
+  };
 
-  // ---- the piece's partial, straight from registers (natural-log units, as the reduce expects)
-  const size_t part = size_t(pid) * G;
-#pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    const float l = HalfSum32(lsum[r]);
-    const int head = 4 * half + r;
-    if (n32 == 0 && head < G) a.ml[(part + head) * 2] = m[r] * kLn2, a.ml[(part + head) * 2 + 1] = l;
-  }
-  if (kg == 0 || kg == 2) {
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const int head = 2 * kg + r;
-      if (head < G) {
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt) a.acc[(part + head) * D + 16 * nt + n16] = o[nt][r];
-      }
+  int idx = take();
+  bool worked = false;  // this wave has worked on the pair `cur`
+  while (true) {
+    // ---- move to the pair of tile idx; pairs passed without a tile get an empty partial
+    bool more = idx < chunk_n;
+    while (more && idx >= cur.base + cur.n) {
+      if (!worked) leave_empty();
+      worked = false;
+      more = NextPair(a, chunk_n, &cur);
     }
+    if (!more) break;
+    // ---- first tile of this wave in the pair: query rows, empty state, first loads
+    constexpr int QE = NB * 32 / 64;  // lq entries per lane
+    h8v qreg[QE];
+#pragma unroll
+    for (int e = 0; e < QE; ++e) {
+      const int i = lane + 64 * e, b = i / 32, sub = (i / 16) % 2, hf = (i / 8) % 2, rw = i % 8;
+      qreg[e] = h8v{0, 0, 0, 0, 0, 0, 0, 0};
+      if (rw < G)
+        qreg[e] = LoadQ8(a.q, (size_t(cur.s) * g.n_q + size_t(cur.h) * G + rw) * D + b * 32 + 16 * hf + 8 * sub,
+                         a.q_dtype);
+    }
+    row = a.table + int64_t(cur.s) * a.stride;
+    int tile = cur.first + (idx - cur.base);
+    int pgc[PPT], pgn[PPT];
+    load_pages(tile, pgc);
+    load_k(0, pgc);
+    load_v(0, pgc);
+#pragma unroll
+    for (int e = 0; e < QE; ++e) {
+      const int i = lane + 64 * e;
+      *reinterpret_cast<h8v*>(&lq[i / 32][(i / 16) % 2][(i / 8) % 2][i % 8][0]) = qreg[e];
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) m[r] = kNegMax, lsum[r] = 0.0f;
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) o[nt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
+    worked = true;
+    bool first = true;
+    // ---- this wave's tiles of the pair
+    while (true) {
+      const int nidx = take();
+      const bool has_next = nidx < cur.base + cur.n;  // the wave's next tile is in the same pair
+      const int ntile = cur.first + (nidx - cur.base);
+      if (has_next) load_pages(ntile, pgn);
+      scores(0);
+      load_k(1, pgc);
+      if (!first) {
+        pv(1);  // second half of the previous tile's P.V: lp and lvs still hold that tile
+        load_v(0, pgc);
+      }
+      first = false;
+      scores(1);
+      if (has_next) load_k(0, pgn);
+      // ---- online softmax (base 2); keys at or past len are masked by select, so stale scales cannot leak
+      float alpha[4];
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt) {
+        const bool valid = tile * kTile + 32 * tt + n32 < cur.len;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) sc[tt][r] = valid ? sc[tt][r] : kNegMax;
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float mn = fmaxf(m[r], HalfMax32(fmaxf(sc[0][r], sc[1][r])));
+        alpha[r] = __builtin_amdgcn_exp2f(m[r] - mn);
+        m[r] = mn;
+        const float p0 = __builtin_amdgcn_exp2f(sc[0][r] - mn), p1 = __builtin_amdgcn_exp2f(sc[1][r] - mn);
+        lsum[r] = __builtin_fmaf(lsum[r], alpha[r], p0 + p1);  // per lane; summed over the lanes at the end
+        lp[4 * half + r][n32] = static_cast<_Float16>(p0);
+        lp[4 * half + r][32 + n32] = static_cast<_Float16>(p1);
+      }
+      {  // V scales of the tile to LDS; scales of keys at or past len become 0, which makes their V rows 0
+        const int b = lane / 8, chunk = lane % 8;
+        if (b < NB) {
+          uint32_t w[4] = {vsr.x, vsr.y, vsr.z, vsr.w};
+          const int k0 = tile * kTile + 8 * chunk;
+          if (k0 + 8 > cur.len) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+              if (k0 + j >= cur.len) w[j / 2] &= j % 2 ? 0x0000FFFFu : 0xFFFF0000u;
+          }
+          *reinterpret_cast<uint4*>(&lvs[b][8 * chunk]) = uint4{w[0], w[1], w[2], w[3]};
+        }
+      }
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o[nt][r] *= alpha[r];
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      pv(0);
+      load_v(1, pgc);
+      idx = nidx;
+      if (!has_next) break;
+      tile = ntile;
+#pragma unroll
+      for (int j = 0; j < PPT; ++j) pgc[j] = pgn[j];
+    }
+    pv(1);
+    leave_partial();
+    __builtin_amdgcn_wave_barrier();  // lq, lp and lvs are rewritten for the next pair
   }
-  });
+  // pairs of the chunk after this wave's last tile
+  do {
+    if (!worked) leave_empty();
+    worked = false;
+  } while (NextPair(a, chunk_n, &cur));
 }
 
 // ---- reduce -------------------------------------------------------------------------------------------------------------
@@ -578,21 +627,22 @@ __global__ void DattnReduce(const DecodeArgs a) {
     a.out[o] = 0.0f;
     return;
   }
-  const int A_ = a.header[1], c = a.header[2], pair = s * H + h;
-  const long long long_end = static_cast<long long>(A_) * a.n_long;
-  const long long first = static_cast<long long>(a.tprefix[s]) * H + static_cast<long long>(h) * ts, last = first + ts - 1;
-  auto chunk_of = [&](long long pos) {
-    return static_cast<int>(pos < long_end ? pos / A_ : a.n_long + (pos - long_end) / c);
-  };
-  const int k0 = chunk_of(first), k1 = chunk_of(last);
+  const int A_ = a.header[1], pair = s * H + h;
+  const long long first = static_cast<long long>(a.tprefix[s]) * H + static_cast<long long>(h) * ts;
+  const int k0 = static_cast<int>(first / A_), k1 = static_cast<int>((first + ts - 1) / A_);
+  const size_t p0 = size_t(k0 + pair) * a.wpc, p1 = size_t(k1 + pair + 1) * a.wpc;
+  // waves that got no tile of this pair left l = 0 (and no acc)
   float M = kNegMax;
-  for (int k = k0; k <= k1; ++k) M = fmaxf(M, a.ml[(size_t(k + pair) * G + gi) * 2]);
+  for (size_t p = p0; p < p1; ++p)
+    if (a.ml[(p * G + gi) * 2 + 1] > 0.0f) M = fmaxf(M, a.ml[(p * G + gi) * 2]);
   float L = 0.0f, A = 0.0f;
-  for (int k = k0; k <= k1; ++k) {
-    const size_t p = size_t(k + pair) * G + gi;
-    const float w = __expf(a.ml[p * 2] - M);
-    L = __builtin_fmaf(w, a.ml[p * 2 + 1], L);
-    A = __builtin_fmaf(w, a.acc[p * D + d], A);
+  for (size_t p = p0; p < p1; ++p) {
+    const float l = a.ml[(p * G + gi) * 2 + 1];
+    if (l > 0.0f) {
+      const float w = __expf(a.ml[(p * G + gi) * 2] - M);
+      L = __builtin_fmaf(w, l, L);
+      A = __builtin_fmaf(w, a.acc[(p * G + gi) * D + d], A);
+    }
   }
   float v = A / L;
   if (a.gate != nullptr) v *= 1.0f / (1.0f + __expf(-a.gate[o]));
@@ -601,21 +651,21 @@ __global__ void DattnReduce(const DecodeArgs a) {
 
 // ---- host side ----------------------------------------------------------------------------------------------------------
 
-// Workspace layout and chunk counts, from the host's bounds alone (the lengths are on the device).
+// Workspace layout and chunk count, from the host's bounds alone (the lengths are on the device).
 struct Plan {
-  int32_t max_len, n_long, max_chunks, min_long_tiles, short_tiles, short_permille;
+  int32_t max_len, n_chunks, wpc, min_chunk_tiles;
   size_t off_tprefix, off_chunks, off_ml, off_acc, bytes;
 };
 size_t Align(size_t x) { return (x + 255) & ~size_t(255); }
-int WaveSlots() {  // wavefronts the chip holds at two per SIMD
-  static const int slots = [] {
-    int dev = 0, cus = 0;
+int ComputeUnits() {
+  static const int cus = [] {
+    int dev = 0, n = 0;
     if (hipGetDevice(&dev) != hipSuccess ||
-        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
-      cus = 256;
-    return cus * 8;
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      n = 256;
+    return n;
   }();
-  return slots;
+  return cus;
 }
 int EnvInt(const char* name, int fallback, int lo, int hi) {
   const char* e = std::getenv(name);
@@ -625,21 +675,23 @@ Plan MakePlan(const Geom& g, int32_t n_seqs, int32_t max_seq_len) {
   Plan p;
   p.max_len = std::max(max_seq_len, 1);
   const int64_t max_tiles = (int64_t(p.max_len) + kTile - 1) / kTile;
-  // Tuning knobs (environment overrides are for experiments): a short line is not cut finer than min_long_tiles per
-  // wave, because each piece costs a partial (G x (D + 2) floats); the last short_permille / 1000 of the line goes
-  // out in chunks of short_tiles.
-  p.min_long_tiles = EnvInt("YAHKV_DECODE_MIN_LONG_TILES", 2, 1, 1 << 20);
-  p.short_tiles = EnvInt("YAHKV_DECODE_SHORT_TILES", 8, 1, 1 << 20);
-  p.short_permille = EnvInt("YAHKV_DECODE_SHORT_PERMILLE", 0, 0, 900);  // measured: no gain on the ragged batch
-  const int slots = EnvInt("YAHKV_DECODE_WAVES", WaveSlots(), 1, 1 << 20);
   const int64_t line_max = max_tiles * n_seqs * g.n_kv;
-  p.n_long = static_cast<int32_t>(std::min<int64_t>(slots, (line_max + p.min_long_tiles - 1) / p.min_long_tiles));
-  const int64_t short_max = (line_max * p.short_permille / 1000 + p.short_tiles - 1) / p.short_tiles + 1;
-  p.max_chunks = static_cast<int32_t>(p.n_long + short_max);
-  const size_t parts = size_t(p.max_chunks) + size_t(n_seqs) * g.n_kv;
+  // Tuning knobs; the environment overrides are for experiments.
+  if (g.format == 8) {  // one 8-wave workgroup per CU (two waves per SIMD)
+    p.wpc = kWavesPerGroup;
+    p.min_chunk_tiles = EnvInt("YAHKV_DECODE_MIN_CHUNK_TILES", 2 * kWavesPerGroup, 1, 1 << 20);
+    p.n_chunks = EnvInt("YAHKV_DECODE_CHUNKS", ComputeUnits(), 1, 1 << 20);
+  } else {  // scalar q4_0 kernel: one wave per chunk, 16 waves per CU
+    p.wpc = 1;
+    p.min_chunk_tiles = 2;
+    p.n_chunks = ComputeUnits() * 16;
+  }
+  p.n_chunks =
+      static_cast<int32_t>(std::min<int64_t>(p.n_chunks, (line_max + p.min_chunk_tiles - 1) / p.min_chunk_tiles));
+  const size_t parts = (size_t(p.n_chunks) + size_t(n_seqs) * g.n_kv) * p.wpc;
   p.off_tprefix = 256;
   p.off_chunks = Align(p.off_tprefix + sizeof(int32_t) * (size_t(n_seqs) + 1));
-  p.off_ml = Align(p.off_chunks + sizeof(int4) * size_t(p.max_chunks));
+  p.off_ml = Align(p.off_chunks + sizeof(int4) * size_t(p.n_chunks));
   p.off_acc = Align(p.off_ml + sizeof(float) * parts * g.group() * 2);
   p.bytes = Align(p.off_acc + sizeof(float) * parts * g.group() * g.hd);
   return p;
@@ -666,8 +718,7 @@ int Prepare(const yahkv_geometry* g, int32_t page_table_stride, const int32_t* s
   a->chunks = reinterpret_cast<int4*>(ws + p.off_chunks);
   a->ml = reinterpret_cast<float*>(ws + p.off_ml);
   a->acc = reinterpret_cast<float*>(ws + p.off_acc);
-  a->n_long = p.n_long, a->max_chunks = p.max_chunks;
-  a->min_long_tiles = p.min_long_tiles, a->short_tiles = p.short_tiles, a->short_permille = p.short_permille;
+  a->n_chunks = p.n_chunks, a->wpc = p.wpc, a->min_chunk_tiles = p.min_chunk_tiles;
   return YAHKV_OK;
 }
 
@@ -699,12 +750,12 @@ extern "C" int yahkv_decode_part(const yahkv_geometry* g, const yahkv_pools* poo
   a.pools = MakePools(*pools), a.table = page_table, a.q = q, a.q_dtype = q_dtype, a.scale = softmax_scale;
   const Geom& m = a.g;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  hipLaunchKernelGGL(DattnPlan, dim3((a.max_chunks + kPlanThreads - 1) / kPlanThreads), dim3(kPlanThreads),
+  hipLaunchKernelGGL(DattnPlan, dim3((a.n_chunks + kPlanThreads - 1) / kPlanThreads), dim3(kPlanThreads),
                      sizeof(int) * (size_t(n_seqs) + 1), st, a);
   if (const int ls = LaunchStatus()) return ls;
-  const dim3 grid(static_cast<unsigned>(a.n_long));
+  const dim3 grid(static_cast<unsigned>(a.n_chunks));
   if (m.format == 8) {
-#define YAHKV_LAUNCH_Q8(DD, PP) hipLaunchKernelGGL((DattnPartQ8<DD, PP>), grid, dim3(64), 0, st, a)
+#define YAHKV_LAUNCH_Q8(DD, PP) hipLaunchKernelGGL((DattnPartQ8<DD, PP>), grid, dim3(64 * kWavesPerGroup), 0, st, a)
     if (m.hd == 256 && m.pt == 64) YAHKV_LAUNCH_Q8(256, 64);
     else if (m.hd == 256 && m.pt == 32) YAHKV_LAUNCH_Q8(256, 32);
     else if (m.hd == 256) YAHKV_LAUNCH_Q8(256, 16);
