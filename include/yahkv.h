@@ -139,13 +139,15 @@ int yahkv_decode_attend(const yahkv_geometry* g, const yahkv_pools* pools, const
 /* Chunked-prefill attention: query t of sequence s (t < chunk_len) sees keys 0 .. prefix_len[s] + t, which
  * must already be in the pools (append the chunk first).
  *   q    [n_seqs][chunk_len][n_q_heads][D] bf16
- *   out  [n_seqs][chunk_len][n_q_heads][D] bf16
- * prefix_len is device int32 [n_seqs]; max_prefix_len is its host-side upper bound.
+ *   gate [n_seqs][chunk_len][n_q_heads][D] f32 or NULL
+ *   out  [n_seqs][chunk_len][n_q_heads][D] of out_dtype (F32, F16 or BF16)
+ * prefix_len is device int32 [n_seqs]; max_prefix_len is its host-side upper bound. K, V and the softmax
+ * numerators enter the matrix unit as bf16 (round to nearest even), sums are f32. q8_0 pools only in this build.
  * Replaces yah_attn_wmma with its quantized staging (gen_attn_fa.py:1589-1595, 2664-2779). */
 int yahkv_prefill_attend(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
                          int32_t page_table_stride, const int32_t* prefix_len, int32_t n_seqs,
                          int32_t max_prefix_len, int32_t chunk_len, const void* q, float softmax_scale,
-                         const float* gate, void* out, void* stream);
+                         const float* gate, void* out, int32_t out_dtype, void* stream);
 
 /* Gather the blocks of tokens [0, n_tokens) of one sequence back into ggml array-of-blocks order:
  * dst_k / dst_v are device buffers [n_tokens][H][NB][34 or 18 bytes]. `table_row` is that sequence's row of

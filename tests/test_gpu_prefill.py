@@ -1,0 +1,105 @@
+"""GPU chunked-prefill attention against the CPU oracle that models the bf16 operands of the matrix unit (K, V and the
+softmax numerators rounded to bf16, f32 sums): tolerance 2e-3 max relative error, max |got - want| / max |want|. The
+error against the exact closed form on the dequantized K / V is reported and bounded more loosely: bf16 operands
+alone carry 2^-9 relative error each, which short contexts do not average out."""
+import numpy as np
+import pytest
+
+import oracle
+from helpers import bf16_bits, closed_form, dequant, logical_blocks, make_tables, rel_err, to_bf16_f32
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-3
+
+
+def build(yahkv, torch, fmt, n_q, n_kv, hd, pt, prefix, chunk, seed, fill=0):
+    rng = np.random.default_rng(seed)
+    lens = [p + chunk for p in prefix]
+    pages = [(n + pt - 1) // pt for n in lens]
+    g = oracle.geometry(fmt, n_q, n_kv, hd, pt, sum(pages) + 2)
+    table = make_tables(rng, pages, g.n_pages)
+    host = oracle.HostPools(g, fill=fill)
+    dev = yahkv.DevicePools(yahkv.geometry(fmt, n_q, n_kv, hd, pt, g.n_pages), fill=fill)
+    t_table = torch.from_numpy(table).cuda()
+    to_t = lambda x: torch.from_numpy(bf16_bits(x).view(np.int16)).cuda().view(torch.bfloat16)
+    for s, p in enumerate(prefix):                       # the prefix, then the chunk, both through the GPU append
+        for start, n in ((0, p), (p, chunk)):
+            if n == 0:
+                continue
+            k = to_bf16_f32(rng.standard_normal((1, n, n_kv, hd)))
+            v = to_bf16_f32(rng.standard_normal((1, n, n_kv, hd)))
+            oracle.append(host, table[s:s + 1], [start], None, k, v)
+            yahkv.append(dev, t_table[s:s + 1], torch.tensor([start], dtype=torch.int32, device="cuda"), to_t(k), to_t(v))
+    got = dev.numpy()
+    for name, want in host.arrays().items():
+        assert np.array_equal(got[name], want), name
+    return g, table, host, dev, t_table, rng, to_t
+
+
+@pytest.mark.parametrize("fmt,n_q,n_kv,hd,pt,prefix,chunk", [
+    (8, 24, 4, 256, 64, [100, 0, 64 * 3 + 5], 70),
+    (8, 24, 4, 256, 64, [1000], 256),
+    (8, 8, 2, 128, 16, [37, 0, 64], 21),
+    (8, 6, 2, 256, 32, [31, 500], 64),
+    (8, 10, 2, 128, 64, [129], 130),
+])
+def test_prefill_against_oracle(yahkv, torch_gpu, fmt, n_q, n_kv, hd, pt, prefix, chunk):
+    torch = torch_gpu
+    g, table, host, dev, t_table, rng, to_t = build(yahkv, torch, fmt, n_q, n_kv, hd, pt, prefix, chunk,
+                                                    seed=hd + pt + chunk, fill=0x7F)
+    q = to_bf16_f32(rng.standard_normal((len(prefix), chunk, n_q, hd)))
+    gate = rng.standard_normal(q.shape).astype(np.float32)
+    scale = 1 / np.sqrt(hd)
+    t_prefix = torch.tensor(prefix, dtype=torch.int32, device="cuda")
+    for gt in (None, gate):
+        tg = None if gt is None else torch.from_numpy(gt).cuda()
+        out = yahkv.prefill_attend(dev, t_table, t_prefix, max(prefix), to_t(q), scale, gate=tg)
+        torch.cuda.synchronize()
+        got = out.cpu().numpy()
+        assert np.all(np.isfinite(got))
+        want = oracle.prefill_attend(host, table, prefix, q, scale, gt, bf16_operands=True)
+        assert rel_err(got, want) < TOL
+        exact = oracle.prefill_attend(host, table, prefix, q, scale, gt)
+        assert rel_err(got, exact) < 3 * 2.0 ** -9
+    # bf16 output: the same numbers rounded once more
+    out16 = yahkv.prefill_attend(dev, t_table, t_prefix, max(prefix), to_t(q), scale, out_dtype=torch.bfloat16)
+    assert rel_err(out16.float().cpu().numpy(), oracle.prefill_attend(host, table, prefix, q, scale, None, True)) < 2 * 2.0 ** -9
+
+
+def test_prefill_special_cases(yahkv, torch_gpu):
+    """Closed-form checks: the first query of a sequence without prefix returns its own V row; a chunk of one query
+    equals decode attention at that length; independent float64 closed form for a few rows."""
+    torch = torch_gpu
+    prefix, chunk = [0, 77], 40
+    g, table, host, dev, t_table, rng, to_t = build(yahkv, torch, 8, 24, 4, 256, 64, prefix, chunk, seed=5)
+    q = to_bf16_f32(rng.standard_normal((2, chunk, 24, 256)))
+    t_prefix = torch.tensor(prefix, dtype=torch.int32, device="cuda")
+    got = yahkv.prefill_attend(dev, t_table, t_prefix, 77, to_t(q), 0.0625).cpu().numpy()
+    (ks, kc), (vs, vc) = logical_blocks(host.arrays(), g, table[0], chunk)
+    Kd, Vd = dequant(ks, kc), dequant(vs, vc)
+    assert rel_err(got[0, 0], np.repeat(to_bf16_f32(Vd[0]), 6, 0)) < 1e-6       # one visible key: out = bf16(V row)
+    for t in (1, 17, chunk - 1):
+        assert rel_err(got[0, t], closed_form(Kd[:t + 1], Vd[:t + 1], q[0, t], 0.0625)) < 3 * 2.0 ** -9
+    lens = [p + chunk for p in prefix]
+    one = yahkv.prefill_attend(dev, t_table, torch.tensor([l - 1 for l in lens], dtype=torch.int32, device="cuda"),
+                               max(lens), to_t(q[:, -1:]), 0.0625).cpu().numpy()
+    dec = yahkv.decode_attend(dev, t_table, torch.tensor(lens, dtype=torch.int32, device="cuda"), max(lens),
+                              to_t(q[:, -1]), 0.0625).cpu().numpy()
+    assert rel_err(one[:, 0], dec) < 3 * 2.0 ** -9
+    assert rel_err(one[:, 0], got[:, -1]) < 1e-6                                 # same query, same keys, same kernel
+
+
+def test_prefill_rejects_bad_arguments(yahkv, torch_gpu):
+    import ctypes as C
+    torch = torch_gpu
+    g = yahkv.geometry(4, 24, 4, 256, 64, 8)
+    dev = yahkv.DevicePools(g)
+    table = torch.zeros((1, 4), dtype=torch.int32, device="cuda")
+    q = torch.zeros((1, 8, 24, 256), dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(yahkv.YahkvError) as e:                                    # q4_0 prefill is not built
+        yahkv.prefill_attend(dev, table, torch.zeros(1, dtype=torch.int32, device="cuda"), 0, q, 0.0625)
+    assert e.value.status == -2
+    g8 = yahkv.geometry(8, 24, 4, 256, 64, 8)
+    st = yahkv.DevicePools(g8).struct()
+    rc = yahkv.lib.yahkv_prefill_attend(C.byref(g8), C.byref(st), None, 4, None, 1, 0, 8, None, 0.0625, None, None, 0, None)
+    assert rc == -1

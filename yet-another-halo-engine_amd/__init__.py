@@ -49,8 +49,7 @@ def _load():
     lib.yahkv_decode_part.argtypes = [G, P, i32p, i32, i32p, i32, i32, vp, i32, C.c_float, vp, C.c_size_t, vp]
     lib.yahkv_decode_reduce.argtypes = [G, i32, i32p, i32, i32, vp, vp, vp, C.c_size_t, vp]
     lib.yahkv_decode_attend.argtypes = [G, P, i32p, i32, i32p, i32, i32, vp, i32, C.c_float, vp, vp, vp, C.c_size_t, vp]
-    if hasattr(lib, "yahkv_prefill_attend"):
-        lib.yahkv_prefill_attend.argtypes = [G, P, i32p, i32, i32p, i32, i32, i32, vp, C.c_float, vp, vp, vp]
+    lib.yahkv_prefill_attend.argtypes = [G, P, i32p, i32, i32p, i32, i32, i32, vp, C.c_float, vp, vp, i32, vp]
     lib.yahkv_gather_blocks.argtypes = [G, P, i32p, i32, vp, vp, vp]
     lib.yahkv_pagepool_create.restype = C.c_void_p
     lib.yahkv_pagepool_create.argtypes = [i32]
@@ -220,17 +219,17 @@ def decode_reduce(g, table_stride, seq_len, n_seqs, max_seq_len, out, workspace,
                                    _dp(workspace), workspace.numel(), _stream()), "decode_reduce")
 
 
-def prefill_attend(pools, table, prefix_len, max_prefix_len, q, scale, gate=None, out=None):
-    """q: [n_seqs][chunk][n_q_heads][D] bf16; returns out bf16 of the same shape."""
+def prefill_attend(pools, table, prefix_len, max_prefix_len, q, scale, gate=None, out=None, out_dtype=None):
+    """q: [n_seqs][chunk][n_q_heads][D] bf16; returns out (f32 unless out / out_dtype say otherwise), same shape."""
     import torch
     g = pools.geom
-    assert q.is_contiguous() and q.dtype == torch.bfloat16
+    assert q.is_contiguous() and q.dtype == torch.bfloat16 and table.is_contiguous()
     if out is None:
-        out = torch.empty_like(q)
+        out = torch.empty(q.shape, dtype=out_dtype or torch.float32, device=q.device)
     st = pools.struct()
     _check(lib.yahkv_prefill_attend(C.byref(g), C.byref(st), _dp(table), table.shape[1], _dp(prefix_len), q.shape[0],
-                                    max_prefix_len, q.shape[1], _dp(q), scale, _dp(gate), _dp(out), _stream()),
-           "prefill_attend")
+                                    max_prefix_len, q.shape[1], _dp(q), scale, _dp(gate), _dp(out), _dtype_code(out),
+                                    _stream()), "prefill_attend")
     return out
 
 

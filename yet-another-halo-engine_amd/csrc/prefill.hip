@@ -1,0 +1,351 @@
+// Chunked-prefill attention over the paged, block-quantized prefix: a FlashAttention-style kernel on bf16 MFMA.
+//
+// Semantics follow the reference's prefill attention (engine/gpu/loom/tools/gen_attn_fa.py:1-21, launch signature
+// :1589-1595): query t of the chunk sees keys 0 .. prefix + t, which the caller has already appended to the pools;
+// online softmax in base 2 (:1614), output o / l, times sigmoid(gate) if a gate is given (:4230). Quantized K / V are
+// decoded while they are staged into LDS (:2664-2779), here to bf16: value = bf16(d * code), round to nearest even.
+//
+// Shape of the computation (everything is transposed so that keys run along MFMA rows and queries along lanes):
+//   S^T[key][q] = sum_dim K[key][dim] Q[q][dim]     A = K tile from LDS (16 keys x 32 dims), B = Q^T (registers)
+//   O^T[dim][q] += sum_key V^T[dim][key] P^T[key][q]  A = V^T tile from LDS (16 dims x 32 keys), B = P^T (registers)
+// v_mfma_f32_16x16x32_bf16 leaves S^T with one query per lane and keys down the registers, which is exactly the
+// B-operand shape of the second product: P never leaves the registers, the row maximum needs two cross-lane steps, and
+// the rescaling factor of a lane's accumulators is the lane's own.
+// A workgroup (4 waves) owns 64 consecutive chunk positions of one sequence for two query heads of one kv head: eight
+// row blocks of 16 queries, two per wave (three per wave would let all six heads of a group share a tile, but the
+// accumulators of three blocks at head_dim 256, 192 registers, leave too little room and the kernel spills). Every
+// K / V tile is fetched and decoded once per workgroup and used by all eight blocks (the reference decodes once per
+// layer into an f16 pool for the same reason, :4648-4861).
+#include "common.hpp"
+
+namespace yahkv {
+namespace {
+
+constexpr int kKeys = 64;    // keys per tile
+constexpr int kQueries = 64; // chunk positions per workgroup
+constexpr int kHeadsPerGroup = 2;  // query heads per workgroup
+constexpr int RB = 2;        // row blocks (16 queries of one head) per wave
+constexpr float kNegBig = -3.4028234663852886e+38f;
+
+typedef __bf16 b8v __attribute__((ext_vector_type(8)));
+typedef float f4v __attribute__((ext_vector_type(4)));
+
+struct PrefillArgs {
+  Geom g;
+  Pools pools;
+  const int32_t* table;
+  int32_t stride;
+  const int32_t* prefix_len;
+  int32_t n_seqs, max_prefix, chunk_len;
+  const uint16_t* q;  // bf16 [n_seqs][chunk_len][n_q][D]
+  float scale;
+  const float* gate;
+  void* out;
+  int32_t out_dtype;
+};
+
+__device__ __forceinline__ uint32_t PackBf16(float a, float b) {  // round to nearest even
+  typedef __bf16 b2v __attribute__((ext_vector_type(2)));
+  const b2v v = {static_cast<__bf16>(a), static_cast<__bf16>(b)};
+  return __builtin_bit_cast(uint32_t, v);
+}
+
+// Sixteen int8 codes times one scale, as sixteen bf16 (two 16-byte halves).
+__device__ __forceinline__ void Decode16(const uint4 c, float d, uint4* lo, uint4* hi) {
+  const uint32_t w[4] = {c.x ^ 0x80808080u, c.y ^ 0x80808080u, c.z ^ 0x80808080u, c.w ^ 0x80808080u};
+  const float off = -128.0f * d;
+  uint32_t o[8];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {  // v_cvt_f32_ubyteN on code + 128, then one fma brings it back and scales it
+    const float f0 = __builtin_fmaf(static_cast<float>(w[i] & 0xFF), d, off);
+    const float f1 = __builtin_fmaf(static_cast<float>((w[i] >> 8) & 0xFF), d, off);
+    const float f2 = __builtin_fmaf(static_cast<float>((w[i] >> 16) & 0xFF), d, off);
+    const float f3 = __builtin_fmaf(static_cast<float>(w[i] >> 24), d, off);
+    o[2 * i] = PackBf16(f0, f1), o[2 * i + 1] = PackBf16(f2, f3);
+  }
+  *lo = uint4{o[0], o[1], o[2], o[3]}, *hi = uint4{o[4], o[5], o[6], o[7]};
+}
+// Sixteen int8 codes of one dim, sixteen keys, each with its own scale.
+__device__ __forceinline__ void Decode16V(const uint4 c, const uint4 s0, const uint4 s1, uint4* lo, uint4* hi) {
+  const uint32_t w[4] = {c.x ^ 0x80808080u, c.y ^ 0x80808080u, c.z ^ 0x80808080u, c.w ^ 0x80808080u};
+  const uint32_t sw[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+  uint32_t o[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const float d0 = WidenF16(static_cast<uint16_t>(sw[i] & 0xFFFF)), d1 = WidenF16(static_cast<uint16_t>(sw[i] >> 16));
+    const uint32_t b0 = (w[i / 2] >> (16 * (i % 2))) & 0xFF, b1 = (w[i / 2] >> (16 * (i % 2) + 8)) & 0xFF;
+    o[i] = PackBf16(__builtin_fmaf(static_cast<float>(b0), d0, -128.0f * d0),
+                    __builtin_fmaf(static_cast<float>(b1), d1, -128.0f * d1));
+  }
+  *lo = uint4{o[0], o[1], o[2], o[3]}, *hi = uint4{o[4], o[5], o[6], o[7]};
+}
+
+template <int D, int PT>
+__global__ __launch_bounds__(256) void PrefillAttendQ8(const PrefillArgs a) {
+  constexpr int NB = D / 32, NDT = D / 16, KS = D / 32;  // blocks, 16-dim tiles, 32-dim steps of the first product
+  constexpr int KSTR = D + 8, VSTR = kKeys + 8;          // LDS row strides (bf16), padded against bank conflicts
+  constexpr int KCH = kKeys * D / 16 / 256;              // 16-code chunks of a tile per thread
+  const Geom g = a.g;
+  const int G = g.group(), H = g.n_kv;
+  const int n_qt = (a.chunk_len + kQueries - 1) / kQueries, n_hp = (G + kHeadsPerGroup - 1) / kHeadsPerGroup;
+  // Workgroups of one (sequence, kv head) pair run on one XCD (they stream the same K / V through that XCD's L2),
+  // longest query tile first.
+  const int bid = blockIdx.x, xcd = bid % 8, local = bid / 8, per_pair = n_qt * n_hp;
+  const int pair = xcd + 8 * (local / per_pair), qt = n_qt - 1 - (local % per_pair) / n_hp, hp = local % n_hp;
+  if (pair >= a.n_seqs * H) return;
+  const int s = pair / H, h = pair % H;
+  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+  const int qn = lane % 16, jg = lane / 16;  // lane = query (mod 16); lane group = rows 4 jg .. 4 jg + 3 of a tile
+  const int prefix = min(max(a.prefix_len[s], 0), min(a.max_prefix, a.stride * g.pt - a.chunk_len));
+  const int q0 = qt * kQueries;              // first chunk position of this workgroup
+  const int n_keys = min(prefix + q0 + kQueries, prefix + a.chunk_len);
+  const int n_tiles = (n_keys + kKeys - 1) / kKeys;
+
+  __shared__ __align__(16) __bf16 lk[kKeys][KSTR];  // K tile, [key][dim]
+  __shared__ __align__(16) __bf16 lv[D][VSTR];      // V^T tile, [dim][key]
+  __shared__ __align__(16) uint16_t lvs[NB][kKeys]; // V scales of the tile (f16 bits), [block][key]
+
+  // ---- this wave's row blocks: rb = RB * wave + i -> head 2 hp + rb / 4, queries q0 + 16 (rb % 4) + 0..15
+  b8v qb[RB][KS];
+  int qpos[RB];   // chunk position of this lane's query in block i (may be >= chunk_len: then it is never stored)
+  int head[RB];   // head within the group (may be >= G: then the block is never stored)
+#pragma unroll
+  for (int i = 0; i < RB; ++i) {
+    const int rb = RB * wave + i;
+    head[i] = kHeadsPerGroup * hp + rb / 4;
+    qpos[i] = q0 + 16 * (rb % 4) + qn;
+    const int t = min(qpos[i], a.chunk_len - 1), hd = min(head[i], G - 1);
+    const uint16_t* qp = a.q + ((size_t(s) * a.chunk_len + t) * g.n_q + size_t(h) * G + hd) * D;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qb[i][ks] = *reinterpret_cast<const b8v*>(qp + 32 * ks + 8 * jg);
+  }
+  f4v o[RB][NDT];
+  float m[RB], lsum[RB];
+#pragma unroll
+  for (int i = 0; i < RB; ++i) {
+    m[i] = kNegBig, lsum[i] = 0.0f;
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt) o[i][dt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
+  }
+  const float sscale = a.scale * 1.4426950408889634f;
+  const int32_t* row = a.table + int64_t(s) * a.stride;
+  auto page_head = [&](int key) -> size_t {  // (page, kv head) index of a key of the sequence
+    return size_t(ClampPage(row[min(key / PT, a.stride - 1)], g.n_pages)) * H + h;
+  };
+
+  // staging registers: this thread's chunks of the next K tile or V tile
+  uint4 craw[KCH];
+  uint16_t ksr[KCH];
+  uint4 vsr;  // threads 0 .. NB * 8 - 1: eight V scales of one block
+  auto fetch_k = [&](int tile) {  // chunk c: block c / 128, key (c % 128) / 2, half c % 2
+#pragma unroll
+    for (int j = 0; j < KCH; ++j) {
+      const int c = tid + 256 * j, b = c / 128, key = (c % 128) / 2, hf = c % 2;
+      const int kk = min(tile * kKeys + key, a.stride * PT - 1);
+      const size_t ph = page_head(kk);
+      craw[j] = *reinterpret_cast<const uint4*>(a.pools.kq + ((ph * NB + b) * PT + kk % PT) * 32 + 16 * hf);
+      ksr[j] = a.pools.ks[(ph * PT + kk % PT) * NB + b];
+    }
+  };
+  auto stage_k = [&]() {
+#pragma unroll
+    for (int j = 0; j < KCH; ++j) {
+      const int c = tid + 256 * j, b = c / 128, key = (c % 128) / 2, hf = c % 2;
+      uint4 lo, hi;
+      Decode16(craw[j], WidenF16(ksr[j]), &lo, &hi);
+      uint4* dst = reinterpret_cast<uint4*>(&lk[key][32 * b + 16 * hf]);
+      dst[0] = lo, dst[1] = hi;
+    }
+  };
+  auto fetch_v = [&](int tile) {  // chunk c: dim c / 4, keys 16 (c % 4) .. + 15
+#pragma unroll
+    for (int j = 0; j < KCH; ++j) {
+      const int c = tid + 256 * j, d = c / 4, k0 = 16 * (c % 4);
+      const int kk = min(tile * kKeys + k0, a.stride * PT - 16);
+      craw[j] = *reinterpret_cast<const uint4*>(a.pools.vq + (page_head(kk) * D + d) * PT + kk % PT);
+    }
+    if (tid < NB * 8) {  // the tile's V scales: thread = (block, 8 keys)
+      const int b = tid / 8, kk = min(tile * kKeys + 8 * (tid % 8), a.stride * PT - 8);
+      vsr = *reinterpret_cast<const uint4*>(a.pools.vs + (page_head(kk) * NB + b) * PT + kk % PT);
+    }
+  };
+  // V scales to LDS; keys past the end get scale 0, so stale bytes decode to 0 and 0 * P stays 0
+  auto stage_vs = [&](int tile) {
+    if (tid < NB * 8) {
+      uint32_t sw[4] = {vsr.x, vsr.y, vsr.z, vsr.w};
+      const int kbase = tile * kKeys + 8 * (tid % 8);
+      if (kbase + 8 > n_keys) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (kbase + e >= n_keys) sw[e / 2] &= e % 2 ? 0x0000FFFFu : 0xFFFF0000u;
+      }
+      *reinterpret_cast<uint4*>(&lvs[tid / 8][8 * (tid % 8)]) = uint4{sw[0], sw[1], sw[2], sw[3]};
+    }
+  };
+  auto stage_v = [&]() {
+#pragma unroll
+    for (int j = 0; j < KCH; ++j) {
+      const int c = tid + 256 * j, d = c / 4, k0 = 16 * (c % 4);
+      const uint4* sp = reinterpret_cast<const uint4*>(&lvs[d / 32][k0]);
+      uint4 lo, hi;
+      Decode16V(craw[j], sp[0], sp[1], &lo, &hi);
+      uint4* dst = reinterpret_cast<uint4*>(&lv[d][k0]);
+      dst[0] = lo, dst[1] = hi;
+    }
+  };
+
+  fetch_k(0);
+  for (int tile = 0; tile < n_tiles; ++tile) {
+    __syncthreads();  // the previous tile's products are done with lk and lv
+    stage_k();
+    __syncthreads();
+    fetch_v(tile);
+    // ---- S^T = K Q^T, keys 16 kt + 4 jg + r down the registers
+    f4v st[RB][4];
+#pragma unroll
+    for (int i = 0; i < RB; ++i)
+#pragma unroll
+      for (int kt = 0; kt < 4; ++kt) st[i][kt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int kt = 0; kt < 4; ++kt) {
+        const b8v ka = *reinterpret_cast<const b8v*>(&lk[16 * kt + qn][32 * ks + 8 * jg]);
+#pragma unroll
+        for (int i = 0; i < RB; ++i) st[i][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qb[i][ks], st[i][kt], 0, 0, 0);
+        if (kt % 2 == 1) __builtin_amdgcn_sched_barrier(0);  // keep LDS reads close to their use: registers are scarce
+      }
+    // ---- online softmax per query (= per lane); the row maximum crosses the four lane groups
+    const bool diag = (tile + 1) * kKeys > prefix + q0 + 1;  // some key of the tile is masked for some query
+    uint32_t pb[RB][2][4];                                   // P^T B-operands: [32-key step][packed pairs]
+#pragma unroll
+    for (int i = 0; i < RB; ++i) {
+      float mx = kNegBig;
+#pragma unroll
+      for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          float v = st[i][kt][r] * sscale;
+          if (diag && tile * kKeys + 16 * kt + 4 * jg + r > prefix + qpos[i]) v = kNegBig;
+          st[i][kt][r] = v;
+          mx = fmaxf(mx, v);
+        }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float mn = fmaxf(m[i], mx);
+      const float alpha = __builtin_amdgcn_exp2f(m[i] - mn);
+      m[i] = mn;
+      float psum = 0.0f;
+#pragma unroll
+      for (int kt = 0; kt < 4; ++kt) {
+        float p[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) p[r] = __builtin_amdgcn_exp2f(st[i][kt][r] - mn), psum += p[r];
+        // step kt / 2 takes keys 32 (kt / 2) + {4 jg + r} from its even tile and + 16 + {4 jg + r} from its odd one
+        pb[i][kt / 2][2 * (kt % 2)] = PackBf16(p[0], p[1]);
+        pb[i][kt / 2][2 * (kt % 2) + 1] = PackBf16(p[2], p[3]);
+      }
+      lsum[i] = __builtin_fmaf(lsum[i], alpha, psum);
+      if (alpha != 1.0f) {
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) o[i][dt][r] *= alpha;
+      }
+    }
+    stage_vs(tile);
+    __syncthreads();  // V scales are in place (and every wave is done with lk)
+    stage_v();
+    __syncthreads();
+    if (tile + 1 < n_tiles) fetch_k(tile + 1);
+    // ---- O^T += V^T P^T; the A operand's key slots follow pb: 4 keys at 32 s2 + 4 jg, 4 at 32 s2 + 16 + 4 jg
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) {
+        const uint2 v0 = *reinterpret_cast<const uint2*>(&lv[16 * dt + qn][32 * s2 + 4 * jg]);
+        const uint2 v1 = *reinterpret_cast<const uint2*>(&lv[16 * dt + qn][32 * s2 + 16 + 4 * jg]);
+        const b8v va = __builtin_bit_cast(b8v, uint4{v0.x, v0.y, v1.x, v1.y});
+#pragma unroll
+        for (int i = 0; i < RB; ++i) {
+          const b8v pv = __builtin_bit_cast(b8v, uint4{pb[i][s2][0], pb[i][s2][1], pb[i][s2][2], pb[i][s2][3]});
+          o[i][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pv, o[i][dt], 0, 0, 0);
+        }
+        if (s2 == 1) __builtin_amdgcn_sched_barrier(0);
+      }
+  }
+
+  // ---- out = o / l (* sigmoid(gate)); lane (query, group jg) holds dims 16 dt + 4 jg + r
+#pragma unroll
+  for (int i = 0; i < RB; ++i) {
+    float l = lsum[i];
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    if (head[i] >= G || qpos[i] >= a.chunk_len) continue;
+    const float inv = 1.0f / l;
+    const size_t base = ((size_t(s) * a.chunk_len + qpos[i]) * g.n_q + size_t(h) * G + head[i]) * D;
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt) {
+      float v[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        v[r] = o[i][dt][r] * inv;
+        if (a.gate != nullptr) v[r] *= 1.0f / (1.0f + __expf(-a.gate[base + 16 * dt + 4 * jg + r]));
+      }
+      const size_t e = base + 16 * dt + 4 * jg;
+      if (a.out_dtype == YAHKV_F32) {
+        *reinterpret_cast<float4*>(static_cast<float*>(a.out) + e) = float4{v[0], v[1], v[2], v[3]};
+      } else if (a.out_dtype == YAHKV_BF16) {
+        *reinterpret_cast<uint2*>(static_cast<uint16_t*>(a.out) + e) = uint2{PackBf16(v[0], v[1]), PackBf16(v[2], v[3])};
+      } else {
+        typedef _Float16 h2v __attribute__((ext_vector_type(2)));
+        const h2v x = {static_cast<_Float16>(v[0]), static_cast<_Float16>(v[1])};
+        const h2v y = {static_cast<_Float16>(v[2]), static_cast<_Float16>(v[3])};
+        *reinterpret_cast<uint2*>(static_cast<uint16_t*>(a.out) + e) =
+            uint2{__builtin_bit_cast(uint32_t, x), __builtin_bit_cast(uint32_t, y)};
+      }
+    }
+  }
+}
+
+}  // namespace
+}  // namespace yahkv
+
+using namespace yahkv;
+
+extern "C" int yahkv_prefill_attend(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
+                                    int32_t page_table_stride, const int32_t* prefix_len, int32_t n_seqs,
+                                    int32_t max_prefix_len, int32_t chunk_len, const void* q, float softmax_scale,
+                                    const float* gate, void* out, int32_t out_dtype, void* stream) {
+  if (const int st = CheckGeometry(g)) return st;
+  if (pools == nullptr || pools->kq == nullptr || pools->ks == nullptr || pools->vq == nullptr ||
+      pools->vs == nullptr || page_table == nullptr || prefix_len == nullptr || q == nullptr || out == nullptr)
+    return YAHKV_ERR_ARG;
+  if (n_seqs <= 0 || chunk_len <= 0 || max_prefix_len < 0 || page_table_stride <= 0) return YAHKV_ERR_ARG;
+  if (out_dtype != YAHKV_F32 && out_dtype != YAHKV_F16 && out_dtype != YAHKV_BF16) return YAHKV_ERR_ARG;
+  if ((reinterpret_cast<uintptr_t>(pools->kq) | reinterpret_cast<uintptr_t>(pools->vq) |
+       reinterpret_cast<uintptr_t>(pools->ks) | reinterpret_cast<uintptr_t>(pools->vs) |
+       reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(out)) & 15)
+    return YAHKV_ERR_ARG;
+  const Geom m = MakeGeom(*g);
+  if (m.format != 8) return YAHKV_ERR_SHAPE;      // q4_0 prefill: not built yet
+  if (int64_t(page_table_stride) * m.pt < chunk_len) return YAHKV_ERR_ARG;
+  PrefillArgs a{};
+  a.g = m, a.pools = MakePools(*pools), a.table = page_table, a.stride = page_table_stride, a.prefix_len = prefix_len;
+  a.n_seqs = n_seqs, a.max_prefix = max_prefix_len, a.chunk_len = chunk_len;
+  a.q = static_cast<const uint16_t*>(q), a.scale = softmax_scale, a.gate = gate, a.out = out, a.out_dtype = out_dtype;
+  const int n_qt = (chunk_len + kQueries - 1) / kQueries;
+  const int n_hp = (m.group() + kHeadsPerGroup - 1) / kHeadsPerGroup;
+  const int pairs = n_seqs * m.n_kv, pair_slots = (pairs + 7) / 8 * 8;
+  const dim3 grid(static_cast<unsigned>(pair_slots) * n_qt * n_hp);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+#define YAHKV_LAUNCH_PF(DD, PP) hipLaunchKernelGGL((PrefillAttendQ8<DD, PP>), grid, dim3(256), 0, st, a)
+  if (m.hd == 256 && m.pt == 64) YAHKV_LAUNCH_PF(256, 64);
+  else if (m.hd == 256 && m.pt == 32) YAHKV_LAUNCH_PF(256, 32);
+  else if (m.hd == 256) YAHKV_LAUNCH_PF(256, 16);
+  else if (m.pt == 64) YAHKV_LAUNCH_PF(128, 64);
+  else if (m.pt == 32) YAHKV_LAUNCH_PF(128, 32);
+  else YAHKV_LAUNCH_PF(128, 16);
+#undef YAHKV_LAUNCH_PF
+  return LaunchStatus();
+}
