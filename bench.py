@@ -144,19 +144,31 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="ragged_b64_q8_0", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="only run plain device copies of 1 GiB (to scale rocprofv3's FETCH_SIZE / WRITE_SIZE)")
     a = ap.parse_args()
     if a.gpus != 1:
         raise SystemExit("bench.py: this build runs on ONE GPU (the path has no cross-GPU exchange); use --gpus 1")
     import torch
     yahkv = importlib.import_module("yet-another-halo-engine_amd")
     torch.cuda.set_device(0)
+    if a.copy_calibration:
+        src = torch.ones(1 << 30, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_calibration": {"bytes_read": 1 << 30, "bytes_written": 1 << 30, "copies": 5}}))
+        return
     wl = WORKLOADS[a.workload]
     total = a.warmup + a.steps + 1
     g, pools, lens, table, t_table, gen = build_state(yahkv, torch, wl, total)
     B = wl["batch"]
     scale = 1.0 / float(np.sqrt(HD))
     max_len = int(lens.max()) + total
-    seq_len = torch.from_numpy(lens.copy()).cuda()
+    # Lengths live on the device, one row per step, as the reference preloads its position array
+    # (engine/model/loom_decoder.hpp:131-133): no kernel is spent on incrementing them.
+    len_rows = torch.from_numpy(lens[None, :] + np.arange(total + 1, dtype=np.int32)[:, None]).cuda()
     q = torch.randn((B, NQ, HD), generator=gen, device="cuda").to(torch.bfloat16)
     knew = torch.randn((total, B, 1, NKV, HD), generator=gen, device="cuda").to(torch.bfloat16)
     vnew = torch.randn((total, B, 1, NKV, HD), generator=gen, device="cuda").to(torch.bfloat16)
@@ -165,8 +177,9 @@ def main():
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(a.steps)]
 
     def step(i, pair=None):
-        yahkv.append(pools, t_table, seq_len, knew[i], vnew[i])       # position = current length (device-resident)
-        seq_len.add_(1)
+        seq_len = len_rows[i + 1]
+        yahkv.append(pools, t_table, len_rows[i], knew[i], vnew[i])    # position = current length (device-resident)
+        yahkv.decode_plan(g, t_table.shape[1], seq_len, B, max_len, ws)
         if pair:
             pair[0].record()
         yahkv.decode_part(pools, t_table, seq_len, max_len, q, scale, ws)

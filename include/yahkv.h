@@ -120,9 +120,13 @@ int yahkv_append(const yahkv_geometry* g, const yahkv_pools* pools, const int32_
  * values above it are clamped. A sequence of length 0 yields zeros.
  * Replaces yah_dattn_part_q + yah_dattn_reduce (gen_decode_attn.py:576-1040, 338-411). */
 size_t yahkv_decode_workspace_bytes(const yahkv_geometry* g, int32_t n_seqs, int32_t max_seq_len);
-/* The two dispatches of a decode attention on their own, as LoomDecoder::Step issues them (loom_decoder.hpp:259-268):
- * `part` leaves one partial (M, l, acc) per slice of the context in the workspace, `reduce` merges them into out.
- * Both must be given the same geometry, n_seqs, max_seq_len, page_table_stride and workspace. */
+/* The dispatches of a decode attention on their own, as LoomDecoder::Step issues its own (loom_decoder.hpp:259-268):
+ * `plan` cuts the batch into equal pieces of work from the device-resident lengths (the reference needs none: it has
+ * one sequence and launches one workgroup per page in use), `part` leaves partials (M, l, acc) per piece in the
+ * workspace, `reduce` merges them into out. All three must be given the same geometry, n_seqs, max_seq_len,
+ * page_table_stride and workspace, in this order on one stream; the lengths must not change in between. */
+int yahkv_decode_plan(const yahkv_geometry* g, int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs,
+                      int32_t max_seq_len, void* workspace, size_t workspace_bytes, void* stream);
 int yahkv_decode_part(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
                       int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs, int32_t max_seq_len,
                       const void* q, int32_t q_dtype, float softmax_scale, void* workspace, size_t workspace_bytes,
@@ -130,7 +134,7 @@ int yahkv_decode_part(const yahkv_geometry* g, const yahkv_pools* pools, const i
 int yahkv_decode_reduce(const yahkv_geometry* g, int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs,
                         int32_t max_seq_len, const float* gate, float* out, const void* workspace,
                         size_t workspace_bytes, void* stream);
-/* part, then reduce. */
+/* plan, part, reduce. */
 int yahkv_decode_attend(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
                         int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs, int32_t max_seq_len,
                         const void* q, int32_t q_dtype, float softmax_scale, const float* gate, float* out,

@@ -1,0 +1,107 @@
+"""Host-side checks that need no GPU: the C ABI library loads and exports every entry point include/yahkv.h declares,
+geometry and size functions, page-table validation (the reference throws on an out-of-range entry,
+engine/model/loom_prefill.hpp:1314-1316) and the page allocator's invariants."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "yahkv.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(yahkv_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_entry_point(yahkv):
+    names = declared_functions()
+    assert len(names) >= 20 and "yahkv_append" in names and "yahkv_prefill_attend" in names
+    for n in names:
+        assert hasattr(yahkv.lib, n), f"{n} is declared in include/yahkv.h but not exported by libyahkv.so"
+    assert yahkv.lib.yahkv_version().startswith(b"yahkv")
+    assert yahkv.status_text(0) == "ok" and "geometry" in yahkv.status_text(-2)
+
+
+def test_geometry_and_pool_sizes(yahkv):
+    g = yahkv.geometry(yahkv.Q8_0, 24, 4, 256, 64, 1024)
+    b = yahkv.pool_bytes(g)
+    assert b == {"kq": 1024 * 4 * 256 * 64, "ks": 1024 * 4 * 64 * 8 * 2, "vq": 1024 * 4 * 256 * 64, "vs": 1024 * 4 * 64 * 8 * 2}
+    assert yahkv.lib.yahkv_bytes_per_token(C.byref(g)) == 2176           # 2 x 4 heads x 8 blocks x 34 B
+    g4 = yahkv.geometry(yahkv.Q4_0, 24, 4, 256, 64, 1024)
+    assert yahkv.lib.yahkv_bytes_per_token(C.byref(g4)) == 1152          # 18-byte blocks
+    assert yahkv.pool_bytes(g4)["kq"] == b["kq"] // 2 and yahkv.pool_bytes(g4)["ks"] == b["ks"]
+    assert sum(b.values()) == 1024 * 64 * 2176
+    for bad in [(8, 24, 4, 192, 64, 8), (8, 24, 5, 256, 64, 8), (8, 36, 4, 256, 64, 8), (8, 24, 4, 256, 48, 8), (5, 24, 4, 256, 64, 8)]:
+        with pytest.raises(yahkv.YahkvError) as e:
+            yahkv.geometry(*bad)
+        assert e.value.status == -2
+    with pytest.raises(yahkv.YahkvError) as e:
+        yahkv.geometry(8, 24, 4, 256, 64, 0)
+    assert e.value.status == -1
+    assert yahkv.decode_workspace_bytes(g, 64, 65536) > 0
+    assert yahkv.decode_workspace_bytes(g, 64, 65536) >= yahkv.decode_workspace_bytes(g, 1, 1024)
+    assert yahkv.decode_workspace_bytes(g, 0, 10) == 0
+
+
+def test_validate_page_table(yahkv):
+    g = yahkv.geometry(yahkv.Q8_0, 8, 2, 128, 16, 10)
+    table = np.array([[0, 1, 2, 9], [3, 4, 5, 6]], np.int32)
+    yahkv.validate_page_table(g, table, [64, 33])
+    for bad, lens in [(np.array([[0, 1, 2, 10], [3, 4, 5, 6]]), [64, 33]),      # out of range
+                      (np.array([[0, 1, 2, -1], [3, 4, 5, 6]]), [64, 33]),      # negative
+                      (np.array([[0, 1, 2, 3], [3, 4, 5, 6]]), [64, 33]),       # page 3 used twice
+                      (table, [65, 33])]:                                       # longer than the table's extent
+        with pytest.raises(yahkv.YahkvError) as e:
+            yahkv.validate_page_table(g, bad, lens)
+        assert e.value.status == -3
+    yahkv.validate_page_table(g, np.array([[0, 1, 2, 77], [3, 4, 5, 6]], np.int32), [48, 33])   # unused entries are free
+    with pytest.raises(yahkv.YahkvError):
+        yahkv.validate_page_table(g, table, [-1, 3])
+
+
+def test_page_allocator_invariants(yahkv):
+    n = 97
+    pool = yahkv.PagePool(n)
+    assert pool.free_count == n
+    a = pool.alloc(10)
+    assert a == list(range(10))                                 # lowest id first
+    b = pool.alloc(n - 10)
+    assert sorted(a + b) == list(range(n)) and pool.free_count == 0       # no page handed out twice, pool used up
+    with pytest.raises(yahkv.YahkvError) as e:
+        pool.alloc(1)
+    assert e.value.status == -5 and pool.free_count == 0
+    pool.free([5, 50, 7])
+    assert pool.free_count == 3
+    assert pool.alloc(2) == [5, 7]                              # freed pages are handed out again
+    for bad in ([50], [n], [-1], [60, 60], [61, 50]):           # already free / out of range / listed twice
+        before = pool.free_count
+        with pytest.raises(yahkv.YahkvError) as e:
+            pool.free(bad)
+        assert e.value.status == -3 and pool.free_count == before      # and nothing was freed
+    pool.close()
+    # a shuffled pool still hands out every page exactly once ("pool sized to fit exactly")
+    pool = yahkv.PagePool(1000)
+    pool.shuffle(12345)
+    got = pool.alloc(1000)
+    assert sorted(got) == list(range(1000)) and got != list(range(1000))
+    other = yahkv.PagePool(1000)
+    other.shuffle(12345)
+    assert other.alloc(1000) == got                             # seeded: reproducible
+    rng = np.random.default_rng(0)                              # random alloc / free: allocated + free == pool
+    pool = yahkv.PagePool(64)
+    held = []
+    for _ in range(300):
+        if held and rng.random() < 0.5:
+            k = int(rng.integers(1, len(held) + 1))
+            idx = rng.permutation(len(held))[:k]
+            pool.free([held[i] for i in idx])
+            held = [p for i, p in enumerate(held) if i not in set(idx.tolist())]
+        else:
+            k = int(rng.integers(0, 9))
+            if k <= pool.free_count:
+                held += pool.alloc(k)
+        assert len(set(held)) == len(held) and len(held) + pool.free_count == 64 and all(0 <= p < 64 for p in held)

@@ -46,6 +46,7 @@ def _load():
     lib.yahkv_append.argtypes = [G, P, i32p, i32, i32p, i32p, i32, i32, vp, vp, i32, vp]
     lib.yahkv_decode_workspace_bytes.restype = C.c_size_t
     lib.yahkv_decode_workspace_bytes.argtypes = [G, i32, i32]
+    lib.yahkv_decode_plan.argtypes = [G, i32, i32p, i32, i32, vp, C.c_size_t, vp]
     lib.yahkv_decode_part.argtypes = [G, P, i32p, i32, i32p, i32, i32, vp, i32, C.c_float, vp, C.c_size_t, vp]
     lib.yahkv_decode_reduce.argtypes = [G, i32, i32p, i32, i32, vp, vp, vp, C.c_size_t, vp]
     lib.yahkv_decode_attend.argtypes = [G, P, i32p, i32, i32p, i32, i32, vp, i32, C.c_float, vp, vp, vp, C.c_size_t, vp]
@@ -204,8 +205,14 @@ def decode_attend(pools, table, seq_len, max_seq_len, q, scale, gate=None, out=N
     return out
 
 
+def decode_plan(g, table_stride, seq_len, n_seqs, max_seq_len, workspace):
+    """First dispatch of decode_attend: cut the batch into pieces of work."""
+    _check(lib.yahkv_decode_plan(C.byref(g), table_stride, _dp(seq_len), n_seqs, max_seq_len, _dp(workspace),
+                                 workspace.numel(), _stream()), "decode_plan")
+
+
 def decode_part(pools, table, seq_len, max_seq_len, q, scale, workspace):
-    """First dispatch of decode_attend: partials into the workspace."""
+    """Second dispatch of decode_attend: partials into the workspace."""
     g = pools.geom
     st = pools.struct()
     _check(lib.yahkv_decode_part(C.byref(g), C.byref(st), _dp(table), table.shape[1], _dp(seq_len), q.shape[0],
@@ -214,7 +221,7 @@ def decode_part(pools, table, seq_len, max_seq_len, q, scale, workspace):
 
 
 def decode_reduce(g, table_stride, seq_len, n_seqs, max_seq_len, out, workspace, gate=None):
-    """Second dispatch of decode_attend: merge the partials into out."""
+    """Third dispatch of decode_attend: merge the partials into out."""
     _check(lib.yahkv_decode_reduce(C.byref(g), table_stride, _dp(seq_len), n_seqs, max_seq_len, _dp(gate), _dp(out),
                                    _dp(workspace), workspace.numel(), _stream()), "decode_reduce")
 

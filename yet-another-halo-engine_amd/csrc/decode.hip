@@ -62,18 +62,26 @@ __device__ __forceinline__ int ClampLen(const DecodeArgs& a, int s) { return min
 // [k A, (k + 1) A) of the line, clipped to the line's length.
 __global__ __launch_bounds__(kPlanThreads) void DattnPlan(const DecodeArgs a) {
   extern __shared__ int lpre[];  // [n_seqs + 1]
-  __shared__ int part_sum[kPlanThreads];
+  __shared__ int part_sum[kPlanThreads / 64];
   const int t = threadIdx.x, H = a.g.n_kv;
   const int per = (a.n_seqs + kPlanThreads - 1) / kPlanThreads;
   const int s0 = min(t * per, a.n_seqs), s1 = min(s0 + per, a.n_seqs);
   int sum = 0;
   for (int s = s0; s < s1; ++s) sum += (ClampLen(a, s) + kTile - 1) / kTile;
-  part_sum[t] = sum;
+  // exclusive prefix of the threads' sums: inclusive scan inside each wave, then the waves' totals
+  int incl = sum;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const int v = __shfl_up(incl, o, 64);
+    if (t % 64 >= o) incl += v;
+  }
+  if (t % 64 == 63) part_sum[t / 64] = incl;
   __syncthreads();
-  int base = 0, total = 0;
-  for (int i = 0; i < kPlanThreads; ++i) {
-    if (i < t) base += part_sum[i];
-    total += part_sum[i];
+  int base = incl - sum, total = 0;
+#pragma unroll
+  for (int w = 0; w < kPlanThreads / 64; ++w) {
+    if (w < t / 64) base += part_sum[w];
+    total += part_sum[w];
   }
   for (int s = s0; s < s1; ++s) {
     lpre[s] = base;
@@ -615,7 +623,9 @@ void DattnPartQ8(const DecodeArgs a) {
 // ---- reduce -------------------------------------------------------------------------------------------------------------
 
 // One workgroup per (query head, sequence), thread = dim (gen_decode_attn.py:338-411). The pair's partials are those
-// of the chunks its stretch of the line overlaps.
+// of the waves of the chunks its stretch of the line overlaps; their weights e^(M_p - M) are computed once per
+// workgroup, by one thread each, so that the sum over partials is a loop of independent loads.
+constexpr int kReduceBatch = 256;  // partial slots weighed at a time
 __global__ void DattnReduce(const DecodeArgs a) {
   const Geom g = a.g;
   const int G = g.group(), H = g.n_kv, D = g.hd;
@@ -631,17 +641,32 @@ __global__ void DattnReduce(const DecodeArgs a) {
   const long long first = static_cast<long long>(a.tprefix[s]) * H + static_cast<long long>(h) * ts;
   const int k0 = static_cast<int>(first / A_), k1 = static_cast<int>((first + ts - 1) / A_);
   const size_t p0 = size_t(k0 + pair) * a.wpc, p1 = size_t(k1 + pair + 1) * a.wpc;
-  // waves that got no tile of this pair left l = 0 (and no acc)
+  __shared__ float wgt[kReduceBatch];
+  __shared__ float red[4];
+  // waves that got no tile of this pair left l = 0 (and no acc): they weigh nothing
   float M = kNegMax;
-  for (size_t p = p0; p < p1; ++p)
+  for (size_t p = p0 + d; p < p1; p += D)
     if (a.ml[(p * G + gi) * 2 + 1] > 0.0f) M = fmaxf(M, a.ml[(p * G + gi) * 2]);
+  M = WaveMax(M);
+  if (d % 64 == 0) red[d / 64] = M;
+  __syncthreads();
+  M = red[0];
+  for (int w = 1; w < D / 64; ++w) M = fmaxf(M, red[w]);
   float L = 0.0f, A = 0.0f;
-  for (size_t p = p0; p < p1; ++p) {
-    const float l = a.ml[(p * G + gi) * 2 + 1];
-    if (l > 0.0f) {
-      const float w = __expf(a.ml[(p * G + gi) * 2] - M);
-      L = __builtin_fmaf(w, l, L);
-      A = __builtin_fmaf(w, a.acc[(p * G + gi) * D + d], A);
+  for (size_t b0 = p0; b0 < p1; b0 += kReduceBatch) {
+    const int nb = static_cast<int>(min(p1 - b0, size_t(kReduceBatch)));
+    __syncthreads();
+    for (int i = d; i < nb; i += D) {
+      const float l = a.ml[((b0 + i) * G + gi) * 2 + 1];
+      wgt[i] = l > 0.0f ? __expf(a.ml[((b0 + i) * G + gi) * 2] - M) : 0.0f;
+    }
+    __syncthreads();
+    for (int i = 0; i < nb; ++i) {
+      const float w = wgt[i];
+      if (w > 0.0f) {  // uniform over the workgroup
+        L = __builtin_fmaf(w, a.ml[((b0 + i) * G + gi) * 2 + 1], L);
+        A = __builtin_fmaf(w, a.acc[((b0 + i) * G + gi) * D + d], A);
+      }
     }
   }
   float v = A / L;
@@ -732,6 +757,17 @@ extern "C" size_t yahkv_decode_workspace_bytes(const yahkv_geometry* g, int32_t 
   return MakePlan(MakeGeom(*g), n_seqs, max_seq_len).bytes;
 }
 
+extern "C" int yahkv_decode_plan(const yahkv_geometry* g, int32_t page_table_stride, const int32_t* seq_len,
+                                 int32_t n_seqs, int32_t max_seq_len, void* workspace, size_t workspace_bytes,
+                                 void* stream) {
+  DecodeArgs a;
+  if (const int st = Prepare(g, page_table_stride, seq_len, n_seqs, max_seq_len, workspace, workspace_bytes, &a))
+    return st;
+  hipLaunchKernelGGL(DattnPlan, dim3((a.n_chunks + kPlanThreads - 1) / kPlanThreads), dim3(kPlanThreads),
+                     sizeof(int) * (size_t(n_seqs) + 1), static_cast<hipStream_t>(stream), a);
+  return LaunchStatus();
+}
+
 extern "C" int yahkv_decode_part(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
                                  int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs,
                                  int32_t max_seq_len, const void* q, int32_t q_dtype, float softmax_scale,
@@ -750,9 +786,6 @@ extern "C" int yahkv_decode_part(const yahkv_geometry* g, const yahkv_pools* poo
   a.pools = MakePools(*pools), a.table = page_table, a.q = q, a.q_dtype = q_dtype, a.scale = softmax_scale;
   const Geom& m = a.g;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  hipLaunchKernelGGL(DattnPlan, dim3((a.n_chunks + kPlanThreads - 1) / kPlanThreads), dim3(kPlanThreads),
-                     sizeof(int) * (size_t(n_seqs) + 1), st, a);
-  if (const int ls = LaunchStatus()) return ls;
   const dim3 grid(static_cast<unsigned>(a.n_chunks));
   if (m.format == 8) {
 #define YAHKV_LAUNCH_Q8(DD, PP) hipLaunchKernelGGL((DattnPartQ8<DD, PP>), grid, dim3(64 * kWavesPerGroup), 0, st, a)
@@ -789,6 +822,9 @@ extern "C" int yahkv_decode_attend(const yahkv_geometry* g, const yahkv_pools* p
                                    const float* gate, float* out, void* workspace, size_t workspace_bytes,
                                    void* stream) {
   if (out == nullptr) return YAHKV_ERR_ARG;
+  if (const int st = yahkv_decode_plan(g, page_table_stride, seq_len, n_seqs, max_seq_len, workspace, workspace_bytes,
+                                       stream))
+    return st;
   if (const int st = yahkv_decode_part(g, pools, page_table, page_table_stride, seq_len, n_seqs, max_seq_len, q,
                                        q_dtype, softmax_scale, workspace, workspace_bytes, stream))
     return st;
