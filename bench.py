@@ -28,6 +28,10 @@ WORKLOADS = {
     "b16_ctx128k_q4_0": dict(fmt=4, batch=16, lo=131072, hi=131072, seed=4, outliers=8),
 }
 NQ, NKV, HD, PT = 24, 4, 256, 64
+# HBM bytes per launch of the split-K kernel from rocprofv3 counters (FETCH_SIZE + WRITE_SIZE, each scaled by what the
+# counter reads for a plain 1 GiB copy); a measurement made outside this script, recorded with its summary.
+TRAFFIC = {"ragged_b64_q8_0": 5.381e9}
+TRAFFIC_SOURCE = "profiles/decode_part_q8_0_ragged_b64.md"
 
 
 def fnv1a(b):
@@ -226,8 +230,9 @@ def main():
         "pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2), "tok_per_s": round(B / (ms * 1e-3), 1),
         "kv_bytes_per_step": int(kv_bytes), "parity_max_rel_err": float(f"{err:.3e}"), "out_fnv1a": first_hash,
         "roofline": {"bound": "hbm", "achieved": round(kgbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(kgbs / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "DattnPart",
-                     "kernel_ms": round(kern_ms, 4)},
+                     "frac": round(kgbs / HBM_PEAK_GBS, 4), "traffic": TRAFFIC.get(a.workload),
+                     "traffic_source": TRAFFIC_SOURCE if a.workload in TRAFFIC else None,
+                     "kernel": "DattnPartQ8" if wl["fmt"] == 8 else "DattnPartQ4", "kernel_ms": round(kern_ms, 4)},
     }
     if not a.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline(wl, lens, scale)
