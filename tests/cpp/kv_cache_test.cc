@@ -1,0 +1,161 @@
+// GPU test of the C++ host classes (csrc/kv_cache.hpp) against the CPU oracle: a chunked prefill of three sequences,
+// then decode steps, with pages from the allocator; pools bit-exact, attention within 2e-3; and the host checks that
+// throw where the reference's LoomDecoder throws (engine/model/loom_decoder.hpp:186-203,229-235).
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <random>
+#include <vector>
+
+#include "kv_cache.hpp"
+#include "yahkv_oracle.h"
+
+using namespace yahkv_host;
+
+namespace {
+
+uint16_t Bf16(float f) { return orc_f32_to_bf16(f); }
+float Widen(uint16_t h) { return orc_bf16_to_f32(h); }
+
+struct Fail : std::runtime_error {
+  using std::runtime_error::runtime_error;
+};
+void Expect(bool ok, const char* what) {
+  if (!ok) throw Fail(what);
+}
+template <typename F>
+void ExpectThrow(F&& f, const char* what) {
+  try {
+    f();
+  } catch (const KvError&) {
+    return;
+  }
+  throw Fail(what);
+}
+double RelErr(const std::vector<float>& got, const std::vector<float>& want) {
+  double d = 0, m = 0;
+  for (size_t i = 0; i < got.size(); ++i) d = std::max(d, std::fabs(double(got[i]) - want[i])), m = std::max(m, std::fabs(double(want[i])));
+  return d / m;
+}
+
+}  // namespace
+
+int main() {
+  try {
+    const yahkv_geometry g{YAHKV_Q8_0, 8, 2, 128, 16, 40};
+    const orc_geometry og{8, 8, 2, 128, 16, 40};
+    const int B = 3, T = 200, chunk = 37, steps = 5, H = 2, D = 128, NQ = 8;
+    std::mt19937 rng(7);
+    std::normal_distribution<float> nd;
+    auto randn_bf16 = [&](size_t n, std::vector<uint16_t>* bits, std::vector<float>* f) {
+      bits->resize(n), f->resize(n);
+      for (size_t i = 0; i < n; ++i) (*bits)[i] = Bf16(nd(rng)), (*f)[i] = Widen((*bits)[i]);
+    };
+
+    KvDecoder dec(g, B, T);
+    ExpectThrow([&] { dec.Step(B, nullptr, nullptr, YAHKV_BF16, nullptr, YAHKV_BF16, 1.0f, nullptr, nullptr); },
+                "Step before Bind must throw");
+    KvDecoderState st = dec.OwnState(/*shuffle_seed=*/99);
+    {
+      KvDecoderState small = st;
+      small.kq.length -= 1;
+      ExpectThrow([&] { dec.Bind(small); }, "Bind must reject a pool smaller than the geometry");
+      small = st, small.ptab.length = 4;
+      ExpectThrow([&] { dec.Bind(small); }, "Bind must reject a short page table");
+    }
+    dec.Bind(st);
+    Expect(dec.KqBytes() == size_t(40) * 2 * 128 * 16 && dec.KsBytes() == size_t(40) * 2 * 16 * 4 * 2, "pool byte formulas");
+    Expect(dec.free_pages() == 40, "fresh pool");
+
+    // ---- prefill chunk
+    std::vector<uint16_t> kb, vb, qb;
+    std::vector<float> kf, vf, qf;
+    randn_bf16(size_t(B) * chunk * H * D, &kb, &kf);
+    randn_bf16(size_t(B) * chunk * H * D, &vb, &vf);
+    randn_bf16(size_t(B) * chunk * NQ * D, &qb, &qf);
+    DeviceBuffer dk(kb.size() * 2), dv(vb.size() * 2), dq(qb.size() * 2), dout(qb.size() * 4);
+    CheckHip(hipMemcpy(dk.get(), kb.data(), kb.size() * 2, hipMemcpyHostToDevice), "h2d");
+    CheckHip(hipMemcpy(dv.get(), vb.data(), vb.size() * 2, hipMemcpyHostToDevice), "h2d");
+    CheckHip(hipMemcpy(dq.get(), qb.data(), qb.size() * 2, hipMemcpyHostToDevice), "h2d");
+    KvPrefill pre(dec);
+    const float scale = 1.0f / std::sqrt(float(D));
+    pre.RunChunk(B, chunk, dk.get(), dv.get(), YAHKV_BF16, dq.get(), scale, nullptr, dout.get(), YAHKV_F32);
+    CheckHip(hipDeviceSynchronize(), "sync");
+    Expect(dec.length(0) == chunk && dec.pages(1).size() == 3 && dec.free_pages() == 40 - 9, "pages after the chunk");
+
+    // oracle mirror with the decoder's own page tables
+    const int stride = dec.page_table_stride();
+    std::vector<int32_t> table(size_t(B) * stride, 0), zero(B, 0), pre_len(B, 0);
+    auto refresh_table = [&] {
+      for (int s = 0; s < B; ++s)
+        for (size_t p = 0; p < dec.pages(s).size(); ++p) table[size_t(s) * stride + p] = dec.pages(s)[p];
+    };
+    refresh_table();
+    std::vector<uint8_t> hkq(orc_kq_bytes(&og), 0), hvq(orc_vq_bytes(&og), 0);
+    std::vector<uint16_t> hks(orc_ks_bytes(&og) / 2, 0), hvs(orc_vs_bytes(&og) / 2, 0);
+    const orc_pools op{hkq.data(), hks.data(), hvq.data(), hvs.data()};
+    orc_append(&og, &op, table.data(), stride, zero.data(), nullptr, B, chunk, kf.data(), vf.data());
+    std::vector<float> want(qf.size()), got(qf.size());
+    orc_prefill_attend(&og, &op, table.data(), stride, pre_len.data(), B, chunk, qf.data(), scale, nullptr, want.data(), 1);
+    CheckHip(hipMemcpy(got.data(), dout.get(), got.size() * 4, hipMemcpyDeviceToHost), "d2h");
+    const double e1 = RelErr(got, want);
+    Expect(e1 < 2e-3, "prefill attention differs from the oracle");
+
+    // ---- decode steps
+    double e2 = 0;
+    for (int i = 0; i < steps; ++i) {
+      std::vector<uint16_t> k1, v1, q1;
+      std::vector<float> k1f, v1f, q1f;
+      randn_bf16(size_t(B) * H * D, &k1, &k1f);
+      randn_bf16(size_t(B) * H * D, &v1, &v1f);
+      randn_bf16(size_t(B) * NQ * D, &q1, &q1f);
+      CheckHip(hipMemcpy(dk.get(), k1.data(), k1.size() * 2, hipMemcpyHostToDevice), "h2d");
+      CheckHip(hipMemcpy(dv.get(), v1.data(), v1.size() * 2, hipMemcpyHostToDevice), "h2d");
+      CheckHip(hipMemcpy(dq.get(), q1.data(), q1.size() * 2, hipMemcpyHostToDevice), "h2d");
+      std::vector<int32_t> pos(B), len(B);
+      for (int s = 0; s < B; ++s) pos[s] = dec.length(s), len[s] = pos[s] + 1;
+      dec.Step(B, dk.get(), dv.get(), YAHKV_BF16, dq.get(), YAHKV_BF16, scale, nullptr, static_cast<float*>(dout.get()));
+      CheckHip(hipDeviceSynchronize(), "sync");
+      refresh_table();
+      orc_append(&og, &op, table.data(), stride, pos.data(), nullptr, B, 1, k1f.data(), v1f.data());
+      std::vector<float> w(q1f.size()), o(q1f.size());
+      orc_decode_attend(&og, &op, table.data(), stride, len.data(), B, q1f.data(), scale, nullptr, w.data());
+      CheckHip(hipMemcpy(o.data(), dout.get(), o.size() * 4, hipMemcpyDeviceToHost), "d2h");
+      e2 = std::max(e2, RelErr(o, w));
+    }
+    Expect(e2 < 2e-3, "decode attention differs from the oracle");
+    // pool contents bit-exact: every sequence's blocks, gathered through the page table, against the oracle's
+    const yahkv_pools dp{st.kq.ptr, st.ks.ptr, st.vq.ptr, st.vs.ptr};
+    for (int s = 0; s < B; ++s) {
+      const size_t bytes = size_t(dec.length(s)) * H * (D / 32) * 34;
+      std::vector<uint8_t> gk(bytes), gv(bytes), wk(bytes), wv(bytes);
+      DeviceBuffer bk(bytes), bv(bytes);
+      Check(yahkv_gather_blocks(&g, &dp, static_cast<const int32_t*>(st.ptab.ptr) + size_t(s) * stride, dec.length(s),
+                                bk.get(), bv.get(), nullptr), "gather");
+      CheckHip(hipMemcpy(gk.data(), bk.get(), bytes, hipMemcpyDeviceToHost), "d2h");
+      CheckHip(hipMemcpy(gv.data(), bv.get(), bytes, hipMemcpyDeviceToHost), "d2h");
+      orc_gather_blocks(&og, &op, table.data() + size_t(s) * stride, dec.length(s), wk.data(), wv.data());
+      Expect(gk == wk && gv == wv, "pool blocks differ from the oracle");
+    }
+
+    // ---- host checks
+    Expect(dec.length(2) == chunk + steps, "lengths after the steps");
+    ExpectThrow([&] { dec.Reserve(0, T + 1); }, "Reserve past the context must throw");
+    const int before = dec.free_pages();
+    dec.Release(1);
+    Expect(dec.free_pages() == before + 3 && dec.length(1) == 0, "Release returns the pages");
+    ExpectThrow([&] { dec.Reserve(1, 16 * (dec.free_pages() + 1)); }, "an exhausted pool must throw");
+    dec.ResumeAt(1, 20);
+    Expect(dec.length(1) == 20 && dec.pages(1).size() == 2, "ResumeAt reserves the pages below pos");
+    KvDecoder tiny(g, 1, 16);
+    tiny.Bind(tiny.OwnState());
+    tiny.ResumeAt(0, 16);
+    ExpectThrow([&] { tiny.Step(1, dk.get(), dv.get(), YAHKV_BF16, dq.get(), YAHKV_BF16, scale, nullptr, static_cast<float*>(dout.get())); },
+                "Step past the context must throw");
+    std::printf("kv_cache_test: ok (prefill %.2e, decode %.2e max relative error)\n", e1, e2);
+    return 0;
+  } catch (const std::exception& e) {
+    std::fprintf(stderr, "kv_cache_test: FAILED: %s\n", e.what());
+    return 1;
+  }
+}
