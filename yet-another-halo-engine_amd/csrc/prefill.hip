@@ -133,8 +133,8 @@ __global__ __launch_bounds__(256) void PrefillAttendQ8(const PrefillArgs a) {
     return size_t(ClampPage(row[min(key / PT, a.stride - 1)], g.n_pages)) * H + h;
   };
 
-  // staging registers: this thread's chunks of the next K tile or V tile
-  uint4 craw[KCH];
+  // staging registers: this thread's chunks of the K tile and of the V tile that come next (fetched one tile ahead)
+  uint4 kraw[KCH], vraw[KCH];
   uint16_t ksr[KCH];
   uint4 vsr;  // threads 0 .. NB * 8 - 1: eight V scales of one block
   auto fetch_k = [&](int tile) {  // chunk c: block c / 128, key (c % 128) / 2, half c % 2
@@ -143,28 +143,27 @@ __global__ __launch_bounds__(256) void PrefillAttendQ8(const PrefillArgs a) {
       const int c = tid + 256 * j, b = c / 128, key = (c % 128) / 2, hf = c % 2;
       const int kk = min(tile * kKeys + key, a.stride * PT - 1);
       const size_t ph = page_head(kk);
-      craw[j] = *reinterpret_cast<const uint4*>(a.pools.kq + ((ph * NB + b) * PT + kk % PT) * 32 + 16 * hf);
+      kraw[j] = *reinterpret_cast<const uint4*>(a.pools.kq + ((ph * NB + b) * PT + kk % PT) * 32 + 16 * hf);
       ksr[j] = a.pools.ks[(ph * PT + kk % PT) * NB + b];
     }
   };
-  auto stage_k = [&]() {
-#pragma unroll
-    for (int j = 0; j < KCH; ++j) {
-      const int c = tid + 256 * j, b = c / 128, key = (c % 128) / 2, hf = c % 2;
-      uint4 lo, hi;
-      Decode16(craw[j], WidenF16(ksr[j]), &lo, &hi);
-      uint4* dst = reinterpret_cast<uint4*>(&lk[key][32 * b + 16 * hf]);
-      dst[0] = lo, dst[1] = hi;
-    }
+  auto stage_k = [&](int j) {
+    const int c = tid + 256 * j, b = c / 128, key = (c % 128) / 2, hf = c % 2;
+    uint4 lo, hi;
+    Decode16(kraw[j], WidenF16(ksr[j]), &lo, &hi);
+    uint4* dst = reinterpret_cast<uint4*>(&lk[key][32 * b + 16 * hf]);
+    dst[0] = lo, dst[1] = hi;
   };
   auto fetch_v = [&](int tile) {  // chunk c: dim c / 4, keys 16 (c % 4) .. + 15
 #pragma unroll
     for (int j = 0; j < KCH; ++j) {
       const int c = tid + 256 * j, d = c / 4, k0 = 16 * (c % 4);
       const int kk = min(tile * kKeys + k0, a.stride * PT - 16);
-      craw[j] = *reinterpret_cast<const uint4*>(a.pools.vq + (page_head(kk) * D + d) * PT + kk % PT);
+      vraw[j] = *reinterpret_cast<const uint4*>(a.pools.vq + (page_head(kk) * D + d) * PT + kk % PT);
     }
-    if (tid < NB * 8) {  // the tile's V scales: thread = (block, 8 keys)
+  };
+  auto fetch_vs = [&](int tile) {  // the tile's V scales: thread = (block, 8 keys)
+    if (tid < NB * 8) {
       const int b = tid / 8, kk = min(tile * kKeys + 8 * (tid % 8), a.stride * PT - 8);
       vsr = *reinterpret_cast<const uint4*>(a.pools.vs + (page_head(kk) * NB + b) * PT + kk % PT);
     }
@@ -182,39 +181,63 @@ __global__ __launch_bounds__(256) void PrefillAttendQ8(const PrefillArgs a) {
       *reinterpret_cast<uint4*>(&lvs[tid / 8][8 * (tid % 8)]) = uint4{sw[0], sw[1], sw[2], sw[3]};
     }
   };
-  auto stage_v = [&]() {
-#pragma unroll
-    for (int j = 0; j < KCH; ++j) {
-      const int c = tid + 256 * j, d = c / 4, k0 = 16 * (c % 4);
-      const uint4* sp = reinterpret_cast<const uint4*>(&lvs[d / 32][k0]);
-      uint4 lo, hi;
-      Decode16V(craw[j], sp[0], sp[1], &lo, &hi);
-      uint4* dst = reinterpret_cast<uint4*>(&lv[d][k0]);
-      dst[0] = lo, dst[1] = hi;
-    }
+  auto stage_v = [&](int j) {
+    const int c = tid + 256 * j, d = c / 4, k0 = 16 * (c % 4);
+    const uint4* sp = reinterpret_cast<const uint4*>(&lvs[d / 32][k0]);
+    uint4 lo, hi;
+    Decode16V(vraw[j], sp[0], sp[1], &lo, &hi);
+    uint4* dst = reinterpret_cast<uint4*>(&lv[d][k0]);
+    dst[0] = lo, dst[1] = hi;
   };
 
+  // Pipeline: while the matrix cores run tile i's K Q^T out of lk, the vector units decode V(i) into lv; while they
+  // run V^T P^T out of lv, K(i + 1) is decoded into lk. Raw bytes are fetched a whole tile before they are decoded.
   fetch_k(0);
+  fetch_vs(0);
+  fetch_v(0);
+#pragma unroll
+  for (int j = 0; j < KCH; ++j) stage_k(j);
+  stage_vs(0);
+  if (n_tiles > 1) fetch_k(1), fetch_vs(1);
+  __syncthreads();
   for (int tile = 0; tile < n_tiles; ++tile) {
-    __syncthreads();  // the previous tile's products are done with lk and lv
-    stage_k();
-    __syncthreads();
-    fetch_v(tile);
     // ---- S^T = K Q^T, keys 16 kt + 4 jg + r down the registers
     f4v st[RB][4];
 #pragma unroll
     for (int i = 0; i < RB; ++i)
 #pragma unroll
       for (int kt = 0; kt < 4; ++kt) st[i][kt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
+    {
+      // A operands are read one 32-dim step ahead of the products that use them; the scheduling groups spread the
+      // vector work of the V decode between the matrix instructions (one wave per SIMD: nothing else hides latency).
+      b8v ka[2][4];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks)
+      for (int kt = 0; kt < 4; ++kt) ka[0][kt] = *reinterpret_cast<const b8v*>(&lk[16 * kt + qn][8 * jg]);
 #pragma unroll
-      for (int kt = 0; kt < 4; ++kt) {
-        const b8v ka = *reinterpret_cast<const b8v*>(&lk[16 * kt + qn][32 * ks + 8 * jg]);
+      for (int ks = 0; ks < KS; ++ks) {
+        if (ks + 1 < KS) {
 #pragma unroll
-        for (int i = 0; i < RB; ++i) st[i][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qb[i][ks], st[i][kt], 0, 0, 0);
-        if (kt % 2 == 1) __builtin_amdgcn_sched_barrier(0);  // keep LDS reads close to their use: registers are scarce
+          for (int kt = 0; kt < 4; ++kt)
+            ka[(ks + 1) % 2][kt] = *reinterpret_cast<const b8v*>(&lk[16 * kt + qn][32 * (ks + 1) + 8 * jg]);
+        }
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+          for (int i = 0; i < RB; ++i)
+            st[i][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[ks % 2][kt], qb[i][ks], st[i][kt], 0, 0, 0);
+        if (ks % (KS / KCH) == KS / KCH - 1) {
+          stage_v(ks / (KS / KCH));
+#pragma unroll
+          for (int n = 0; n < 8; ++n) {
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
+            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // two matrix instructions
+            __builtin_amdgcn_sched_group_barrier(0x002, 10, 0); // ten vector instructions
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
       }
+    }
+    if (tile + 1 < n_tiles) fetch_v(tile + 1);
     // ---- online softmax per query (= per lane); the row maximum crosses the four lane groups
     const bool diag = (tile + 1) * kKeys > prefix + q0 + 1;  // some key of the tile is masked for some query
     uint32_t pb[RB][2][4];                                   // P^T B-operands: [32-key step][packed pairs]
@@ -253,26 +276,49 @@ __global__ __launch_bounds__(256) void PrefillAttendQ8(const PrefillArgs a) {
           for (int r = 0; r < 4; ++r) o[i][dt][r] *= alpha;
       }
     }
-    stage_vs(tile);
-    __syncthreads();  // V scales are in place (and every wave is done with lk)
-    stage_v();
-    __syncthreads();
-    if (tile + 1 < n_tiles) fetch_k(tile + 1);
+    __syncthreads();  // every wave is done with lk, and V(tile) is complete in lv
     // ---- O^T += V^T P^T; the A operand's key slots follow pb: 4 keys at 32 s2 + 4 jg, 4 at 32 s2 + 16 + 4 jg
-#pragma unroll
-    for (int dt = 0; dt < NDT; ++dt)
-#pragma unroll
-      for (int s2 = 0; s2 < 2; ++s2) {
+    {
+      auto read_v = [&](int dt, int s2) -> b8v {
         const uint2 v0 = *reinterpret_cast<const uint2*>(&lv[16 * dt + qn][32 * s2 + 4 * jg]);
         const uint2 v1 = *reinterpret_cast<const uint2*>(&lv[16 * dt + qn][32 * s2 + 16 + 4 * jg]);
-        const b8v va = __builtin_bit_cast(b8v, uint4{v0.x, v0.y, v1.x, v1.y});
+        return __builtin_bit_cast(b8v, uint4{v0.x, v0.y, v1.x, v1.y});
+      };
+      b8v pv[RB][2];
 #pragma unroll
-        for (int i = 0; i < RB; ++i) {
-          const b8v pv = __builtin_bit_cast(b8v, uint4{pb[i][s2][0], pb[i][s2][1], pb[i][s2][2], pb[i][s2][3]});
-          o[i][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pv, o[i][dt], 0, 0, 0);
+      for (int i = 0; i < RB; ++i)
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2)
+          pv[i][s2] = __builtin_bit_cast(b8v, uint4{pb[i][s2][0], pb[i][s2][1], pb[i][s2][2], pb[i][s2][3]});
+      b8v va[3][2];  // read two 16-dim tiles ahead
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) va[0][s2] = read_v(0, s2), va[1][s2] = read_v(1, s2);
+#pragma unroll
+      for (int dt = 0; dt < NDT; ++dt) {
+        if (dt + 2 < NDT) {
+#pragma unroll
+          for (int s2 = 0; s2 < 2; ++s2) va[(dt + 2) % 3][s2] = read_v(dt + 2, s2);
         }
-        if (s2 == 1) __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+          for (int i = 0; i < RB; ++i)
+            o[i][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[dt % 3][s2], pv[i][s2], o[i][dt], 0, 0, 0);
+        if (dt % (NDT / KCH) == NDT / KCH - 1) {
+          stage_k(dt / (NDT / KCH));  // K(tile + 1), or stale bytes after the last tile
+#pragma unroll
+          for (int n = 0; n < 8; ++n) {
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
       }
+    }
+    stage_vs(tile + 1);
+    if (tile + 2 < n_tiles) fetch_k(tile + 2), fetch_vs(tile + 2);
+    __syncthreads();  // every wave is done with lv; K(tile + 1) and its V scales are in place
   }
 
   // ---- out = o / l (* sigmoid(gate)); lane (query, group jg) holds dims 16 dt + 4 jg + r
