@@ -232,7 +232,7 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(kgbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(kgbs / HBM_PEAK_GBS, 4), "traffic": TRAFFIC.get(a.workload),
                      "traffic_source": TRAFFIC_SOURCE if a.workload in TRAFFIC else None,
-                     "kernel": "DattnPartQ8" if wl["fmt"] == 8 else "DattnPartQ4", "kernel_ms": round(kern_ms, 4)},
+                     "kernel": "DattnPart<%d, %d, %d>" % (wl["fmt"], HD, PT), "kernel_ms": round(kern_ms, 4)},
     }
     if not a.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline(wl, lens, scale)

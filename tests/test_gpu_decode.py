@@ -82,7 +82,8 @@ def test_config1_tiny(yahkv, torch_gpu):
 
 @pytest.mark.parametrize("fmt,n_q,n_kv,hd,pt", [(8, 24, 4, 256, 64), (4, 24, 4, 256, 64), (8, 8, 2, 128, 16),
                                                  (4, 8, 2, 128, 16), (8, 8, 1, 256, 32), (8, 4, 4, 128, 64), (8, 16, 2, 256, 16),
-                                                 (8, 24, 4, 128, 32)])
+                                                 (8, 24, 4, 128, 32), (4, 8, 1, 256, 32), (4, 16, 2, 256, 16),
+                                                 (4, 24, 4, 128, 32), (4, 4, 4, 128, 64)])
 def test_ragged_batch_with_gate(yahkv, torch_gpu, fmt, n_q, n_kv, hd, pt):
     torch = torch_gpu
     lens = [1, pt - 1, pt, pt + 1, 63, 64, 65, 5 * 64 + 17, 1500, 0, 257]
@@ -121,11 +122,12 @@ def test_special_cases(yahkv, torch_gpu):
     assert np.abs(out[1, 7] - Vd[117, 1]).max() < 2e-3 * np.abs(Vd[117, 1]).max()   # one huge score: that V row
 
 
-def test_stale_bytes_past_the_length_are_masked(yahkv, torch_gpu):
+@pytest.mark.parametrize("fmt", [8, 4])
+def test_stale_bytes_past_the_length_are_masked(yahkv, torch_gpu, fmt):
     """Slots past seq_len hold poison (NaN scales, 0x7F codes): they must not reach the output."""
     torch = torch_gpu
     lens = [70, 3]
-    g, table, host, dev, rng = setup(yahkv, torch, 8, 24, 4, 256, 64, lens, seed=10, fill=0x7F)  # f16 0x7F7F is NaN
+    g, table, host, dev, rng = setup(yahkv, torch, fmt, 24, 4, 256, 64, lens, seed=10, fill=0x7F)  # f16 0x7F7F is NaN
     q = to_bf16_f32(rng.standard_normal((2, 24, 256)))
     got = gpu_attend(yahkv, torch, dev, table, lens, q, 0.0625)
     assert np.all(np.isfinite(got))

@@ -29,7 +29,7 @@ constexpr int kTile = 64;     // keys per tile: one wavefront, one key per lane 
 constexpr int kMaxGroup = 8;  // query heads per kv head
 constexpr int kPlanThreads = 256;
 constexpr int kMaxSeqs = 8191;
-constexpr int kWavesPerGroup = 8;  // q8_0 kernel: one workgroup fills a CU at two waves per SIMD
+constexpr int kWavesPerGroup = 8;  // one workgroup fills a CU at two waves per SIMD
 
 struct DecodeArgs {
   Geom g;
@@ -147,11 +147,6 @@ __device__ __forceinline__ float WaveMax(float v) {
   for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
   return v;
 }
-__device__ __forceinline__ float WaveSum(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-  return v;
-}
 __device__ __forceinline__ float HalfMax32(float v) {  // over the 32 lanes of a wave half
 #pragma unroll
   for (int o = 16; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
@@ -163,144 +158,21 @@ __device__ __forceinline__ float HalfSum32(float v) {
   return v;
 }
 
-// ---- q4_0: scalar-ALU part ----------------------------------------------------------------------------------------------
-
-// Dimension k (< D / 64) of lane `lane`: dim j is paired with j + 16 of its block because one V byte holds both.
-__device__ __forceinline__ int LaneDimQ4(int lane, int k, int dpl) {
-  const int pair = lane * (dpl / 2) + k / 2;
-  return (pair / 16) * 32 + pair % 16 + 16 * (k & 1);
-}
-
-// One wavefront per chunk. A lane owns one key for the scores and D / 64 dims for P.V.
-template <int D>
-__global__ __launch_bounds__(64) void DattnPartQ4(const DecodeArgs a) {
-  constexpr int NB = D / 32, DPL = D / 64, CB = 16;
-  const Geom g = a.g;
-  const int G = g.group(), H = g.n_kv, PT = g.pt;
-  const int lane = threadIdx.x;
-  __shared__ float qs[kMaxGroup][D];
-  __shared__ float ps[kMaxGroup][kTile];
-  const int4 rec = a.chunks[blockIdx.x];
-  if (rec.x < 0) return;
-  PairCursor cur = FirstPair(a, rec);
-  do {
-  const int s = cur.s, h = cur.h, tile0 = cur.first, tile1 = cur.first + cur.n, len = cur.len;
-  __builtin_amdgcn_wave_barrier();  // the previous pair is done with qs
-  for (int i = lane; i < G * D; i += 64)
-    qs[i / D][i % D] = LoadSrc(a.q, (size_t(s) * g.n_q + size_t(h) * G) * D + i, a.q_dtype);
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-
-  float m[kMaxGroup], l[kMaxGroup], acc[kMaxGroup][DPL];
-#pragma unroll
-  for (int gi = 0; gi < kMaxGroup; ++gi) {
-    m[gi] = kNegMax, l[gi] = 0.0f;
-#pragma unroll
-    for (int k = 0; k < DPL; ++k) acc[gi][k] = 0.0f;
-  }
-  const int32_t* row = a.table + int64_t(s) * a.stride;
-
-  for (int tile = tile0; tile < tile1; ++tile) {
-    const int tok = tile * kTile + lane;
-    const bool valid = tok < len;
-    float sc[kMaxGroup];
-#pragma unroll
-    for (int gi = 0; gi < kMaxGroup; ++gi) sc[gi] = 0.0f;
-    if (valid) {
-      const size_t ph = size_t(ClampPage(row[tok / PT], g.n_pages)) * H + h;
-      const int t = tok % PT;
-      for (int b = 0; b < NB; ++b) {
-        const float d = WidenF16(a.pools.ks[(ph * PT + t) * NB + b]);
-        const uint4 v = *reinterpret_cast<const uint4*>(a.pools.kq + ((ph * NB + b) * PT + t) * CB);
-        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-        float part[kMaxGroup];
-#pragma unroll
-        for (int gi = 0; gi < kMaxGroup; ++gi) part[gi] = 0.0f;
-#pragma unroll
-        for (int j = 0; j < 16; ++j) {
-          const uint32_t byte = (w[j / 4] >> (8 * (j % 4))) & 0xFF;
-          const float x0 = static_cast<float>(int(byte & 0xF) - 8), x1 = static_cast<float>(int(byte >> 4) - 8);
-#pragma unroll
-          for (int gi = 0; gi < kMaxGroup; ++gi)
-            if (gi < G) {
-              part[gi] = __builtin_fmaf(qs[gi][b * 32 + j], x0, part[gi]);
-              part[gi] = __builtin_fmaf(qs[gi][b * 32 + 16 + j], x1, part[gi]);
-            }
-        }
-#pragma unroll
-        for (int gi = 0; gi < kMaxGroup; ++gi) sc[gi] = __builtin_fmaf(d, part[gi], sc[gi]);
-      }
-    }
-#pragma unroll
-    for (int gi = 0; gi < kMaxGroup; ++gi) {
-      if (gi < G) {
-        const float sv = valid ? sc[gi] * a.scale : kNegMax;
-        const float mn = fmaxf(m[gi], WaveMax(sv));
-        const float alpha = __expf(m[gi] - mn);
-        const float p = valid ? __expf(sv - mn) : 0.0f;
-        l[gi] = l[gi] * alpha + WaveSum(p);
-#pragma unroll
-        for (int k = 0; k < DPL; ++k) acc[gi][k] *= alpha;
-        m[gi] = mn;
-        ps[gi][lane] = p;
-      }
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    for (int sp = 0; sp < kTile / PT; ++sp) {
-      const int base = tile * kTile + sp * PT;
-      if (base >= len) break;
-      const int nt = min(PT, len - base);
-      const size_t ph = size_t(ClampPage(row[base / PT], g.n_pages)) * H + h;
-#pragma unroll
-      for (int k = 0; k < DPL; k += 2) {
-        const int d0 = LaneDimQ4(lane, k, DPL);
-        const int b = d0 / 32;
-        const uint16_t* sp16 = a.pools.vs + (ph * NB + b) * PT;
-        const uint8_t* cp = a.pools.vq + ((ph * NB + b) * 16 + d0 % 32) * PT;
-        for (int t = 0; t < nt; ++t) {
-          const float d = WidenF16(sp16[t]);
-          const uint32_t byte = cp[t];
-          const float v0 = d * static_cast<float>(int(byte & 0xF) - 8), v1 = d * static_cast<float>(int(byte >> 4) - 8);
-#pragma unroll
-          for (int gi = 0; gi < kMaxGroup; ++gi)
-            if (gi < G) {
-              const float p = ps[gi][sp * PT + t];
-              acc[gi][k] = __builtin_fmaf(p, v0, acc[gi][k]);
-              acc[gi][k + 1] = __builtin_fmaf(p, v1, acc[gi][k + 1]);
-            }
-        }
-      }
-    }
-    __builtin_amdgcn_wave_barrier();  // ps is rewritten by the next tile
-  }
-
-  const size_t part = PartialIndex(a, blockIdx.x, 0, cur) * G;
-#pragma unroll
-  for (int gi = 0; gi < kMaxGroup; ++gi) {
-    if (gi < G) {
-      if (lane == 0) a.ml[(part + gi) * 2] = m[gi], a.ml[(part + gi) * 2 + 1] = l[gi];
-#pragma unroll
-      for (int k = 0; k < DPL; ++k) a.acc[(part + gi) * D + LaneDimQ4(lane, k, DPL)] = acc[gi][k];
-    }
-  }
-  } while (NextPair(a, rec.w, &cur));
-}
-
-// ---- q8_0 on the matrix cores -----------------------------------------------------------------------------------------
+// ---- the part kernel, on the matrix cores -----------------------------------------------------------------------------
 //
-// A scalar-ALU version of this kernel needs 7 lane operations per KV byte (one convert and one multiply-add per query
-// head of the group): at 5.6 TB/s that is every VALU issue slot of the chip. So the two contractions go to MFMA, whose
-// f16 rate leaves both at a few percent of peak, and the VALU only converts codes (about 1.5 operations per byte):
+// A scalar-ALU version of this kernel needs 7 lane operations per q8_0 byte (one convert and one multiply-add per
+// query head of the group): at 5.6 TB/s that is every VALU issue slot of the chip. So the two contractions go to MFMA,
+// whose f16 rate leaves both at a few percent of peak, and the VALU only converts codes (about 1.5 operations per
+// q8_0 byte, 3 per q4_0 byte):
 //   scores  S[head][key] = sum_block ks[key][block] * (Q_block . codes_block)       v_mfma_f32_32x32x16_f16, one
 //           32-dim block per pair of instructions (K = 16 each), so the block scale is applied to the f32 result and
-//           the products themselves are exact (int8 codes and f16 queries are exact in f16)
+//           the products themselves are exact (codes and f16 queries are exact in f16)
 //   output  O[head][dim] += sum_key P[head][key] * (vs[key][block] * codes)          v_mfma_f32_16x16x32_f16; the scale
 //           varies along the contraction here, so V is dequantized to f16 (one rounding, 2^-12 relative)
-// The page layouts are chosen for these operand shapes: a lane's 16-byte load is 16 dims of one key (K, [block][key]
-// [32]) or 16 keys of one dim (V^T, [dim][key]); each wave-wide load is 1 KB contiguous.
+// The page layouts are chosen for these operand shapes. q8_0: a lane's 16-byte load is 16 dims of one key (K, [block]
+// [key][32]) or 16 keys of one dim (V^T, [dim][key]). q4_0: a lane's 8-byte K load is half a block of one key (low
+// nibbles dims 8 h + 0..7, high nibbles dims 16 + 8 h + 0..7, [block][key][16]); its 16-byte V load is 16 keys of the
+// byte row that holds dims j and j + 16 of a block ([block][16][key]), which feeds two 16-dim output tiles.
 typedef _Float16 h2v __attribute__((ext_vector_type(2)));
 typedef _Float16 h8v __attribute__((ext_vector_type(8)));
 typedef float f4v __attribute__((ext_vector_type(4)));
@@ -314,6 +186,28 @@ __device__ __forceinline__ h8v Codes8(uint32_t w0, uint32_t w1) {
   const h2v b = __builtin_bit_cast(h2v, __builtin_amdgcn_perm(0x64646464u, x0, 0x04030402u)) + off;
   const h2v c = __builtin_bit_cast(h2v, __builtin_amdgcn_perm(0x64646464u, x1, 0x04010400u)) + off;
   const h2v d = __builtin_bit_cast(h2v, __builtin_amdgcn_perm(0x64646464u, x1, 0x04030402u)) + off;
+  return h8v{a[0], a[1], b[0], b[1], c[0], c[1], d[0], d[1]};
+}
+
+// Eight nibbles of two dwords as eight f16 holding (nibble - 8), exact. Low nibbles: 0x6400 | n is 1024 + n. High
+// nibbles stay in place: 0x6400 | (n << 4) is 1024 + 16 n, and one fused multiply-add takes it to n - 8.
+__device__ __forceinline__ h8v NibblesLo8(uint32_t w0, uint32_t w1) {
+  const h2v off = {static_cast<_Float16>(-1032.0f), static_cast<_Float16>(-1032.0f)};
+  const uint32_t x0 = w0 & 0x0F0F0F0Fu, x1 = w1 & 0x0F0F0F0Fu;
+  const h2v a = __builtin_bit_cast(h2v, __builtin_amdgcn_perm(0x64646464u, x0, 0x04010400u)) + off;
+  const h2v b = __builtin_bit_cast(h2v, __builtin_amdgcn_perm(0x64646464u, x0, 0x04030402u)) + off;
+  const h2v c = __builtin_bit_cast(h2v, __builtin_amdgcn_perm(0x64646464u, x1, 0x04010400u)) + off;
+  const h2v d = __builtin_bit_cast(h2v, __builtin_amdgcn_perm(0x64646464u, x1, 0x04030402u)) + off;
+  return h8v{a[0], a[1], b[0], b[1], c[0], c[1], d[0], d[1]};
+}
+__device__ __forceinline__ h8v NibblesHi8(uint32_t w0, uint32_t w1) {
+  const h2v mul = {static_cast<_Float16>(0.0625f), static_cast<_Float16>(0.0625f)};
+  const h2v off = {static_cast<_Float16>(-72.0f), static_cast<_Float16>(-72.0f)};
+  const uint32_t x0 = w0 & 0xF0F0F0F0u, x1 = w1 & 0xF0F0F0F0u;
+  const h2v a = __builtin_elementwise_fma(__builtin_bit_cast(h2v, __builtin_amdgcn_perm(0x64646464u, x0, 0x04010400u)), mul, off);
+  const h2v b = __builtin_elementwise_fma(__builtin_bit_cast(h2v, __builtin_amdgcn_perm(0x64646464u, x0, 0x04030402u)), mul, off);
+  const h2v c = __builtin_elementwise_fma(__builtin_bit_cast(h2v, __builtin_amdgcn_perm(0x64646464u, x1, 0x04010400u)), mul, off);
+  const h2v d = __builtin_elementwise_fma(__builtin_bit_cast(h2v, __builtin_amdgcn_perm(0x64646464u, x1, 0x04030402u)), mul, off);
   return h8v{a[0], a[1], b[0], b[1], c[0], c[1], d[0], d[1]};
 }
 
@@ -351,10 +245,13 @@ __device__ __forceinline__ h8v LoadQ8(const void* q, size_t i, int dt) {
 //   scores(keys 32-63)             | load K keys 0-31 of the wave's next tile
 //   softmax, P.V(dims 0..D/2)      | load V dims D/2.. of this tile
 // Page numbers come through scalar loads (they are the same for the whole wave).
-template <int D, int PT>
+template <int FMT, int D, int PT>
 __global__ __launch_bounds__(64 * kWavesPerGroup) __attribute__((amdgpu_waves_per_eu(2, 2)))
-void DattnPartQ8(const DecodeArgs a) {
+void DattnPart(const DecodeArgs a) {
   constexpr int NB = D / 32, NT = D / 16, PPT = kTile / PT;
+  constexpr bool Q8 = FMT == 8;
+  constexpr int KW = Q8 ? 4 : 2;             // dwords of K codes per lane and block
+  constexpr int NVB = Q8 ? NT / 2 : NB / 2;  // 16-byte V loads per lane and half of the dims
   constexpr float kLog2e = 1.4426950408889634f, kLn2 = 0.6931471805599453f;
   const Geom g = a.g;
   const int G = g.group(), H = g.n_kv;
@@ -364,8 +261,9 @@ void DattnPartQ8(const DecodeArgs a) {
 
   // Query A-operands [block][K half of the block's instruction pair][lane half][head row]: 8 f16 each. Row m of the
   // 32-row A matrix is head m; only rows 0-7 exist here and lanes of rows 8-31 re-read them (their output rows are
-  // never looked at). Entry (b, sub, hf, row) holds dims 32 b + 16 hf + 8 sub + 0..7, the dims of the 8 code bytes a
-  // key lane of that half feeds to instruction `sub`.
+  // never looked at). Entry (b, sub, hf, row) holds the dims of the 8 codes a key lane of that half feeds to
+  // instruction `sub`: 32 b + 16 hf + 8 sub + 0..7 for q8_0 (bytes 8 sub .. of its 16), 32 b + 16 sub + 8 hf + 0..7
+  // for q4_0 (low nibbles, then high nibbles, of its 8 bytes).
   __shared__ __align__(16) _Float16 lq_all[kWavesPerGroup][NB][2][2][8][8];
   __shared__ __align__(16) _Float16 lp_all[kWavesPerGroup][kMaxGroup][kTile];
   __shared__ __align__(16) _Float16 lvs_all[kWavesPerGroup][NB][kTile];
@@ -385,9 +283,9 @@ void DattnPartQ8(const DecodeArgs a) {
     return __builtin_amdgcn_readfirstlane(v);
   };
 
-  uint4 kb[NB];      // [block]: 16 codes of this lane's key (one 32-key half of the tile at a time)
-  uint4 ksc;         // that key's NB block scales (f16)
-  uint4 vb[NT / 2];  // [16-dim tile]: 16 keys of this lane's dim (one half of the dims at a time)
+  uint32_t kb[NB][KW];  // [block]: 16 codes of this lane's key (one 32-key half of the tile at a time)
+  uint4 ksc;            // that key's NB block scales (f16)
+  uint4 vb[NVB];        // 16 keys of this lane's dim, or pair of dims (one half of the dims at a time)
   uint4 vsr;         // staging of the tile's V scales: 8 keys of one block per lane
   float m[4], lsum[4], sc[2][4];
   f4v o[NT];
@@ -413,8 +311,15 @@ void DattnPartQ8(const DecodeArgs a) {
     const size_t ph = page_head(pg, tk);
     const int t = tk % PT;
 #pragma unroll
-    for (int b = 0; b < NB; ++b)
-      kb[b] = *reinterpret_cast<const uint4*>(a.pools.kq + ((ph * NB + b) * PT + t) * 32 + 16 * half);
+    for (int b = 0; b < NB; ++b) {
+      if constexpr (Q8) {
+        const uint4 v = *reinterpret_cast<const uint4*>(a.pools.kq + ((ph * NB + b) * PT + t) * 32 + 16 * half);
+        kb[b][0] = v.x, kb[b][1] = v.y, kb[b][2] = v.z, kb[b][3] = v.w;
+      } else {
+        const uint2 v = *reinterpret_cast<const uint2*>(a.pools.kq + ((ph * NB + b) * PT + t) * 16 + 8 * half);
+        kb[b][0] = v.x, kb[b][1] = v.y;
+      }
+    }
     const uint16_t* sp = a.pools.ks + (ph * PT + t) * NB;
     if (NB == 8) {
       ksc = *reinterpret_cast<const uint4*>(sp);
@@ -427,8 +332,12 @@ void DattnPartQ8(const DecodeArgs a) {
     const size_t ph = page_head(pg, 16 * kg);
     const int t0 = (16 * kg) % PT;
 #pragma unroll
-    for (int j = 0; j < NT / 2; ++j)
-      vb[j] = *reinterpret_cast<const uint4*>(a.pools.vq + (ph * D + 16 * (hf * (NT / 2) + j) + n16) * PT + t0);
+    for (int j = 0; j < NVB; ++j) {
+      if constexpr (Q8)
+        vb[j] = *reinterpret_cast<const uint4*>(a.pools.vq + (ph * D + 16 * (hf * NVB + j) + n16) * PT + t0);
+      else
+        vb[j] = *reinterpret_cast<const uint4*>(a.pools.vq + ((ph * NB + hf * NVB + j) * 16 + n16) * PT + t0);
+    }
     if (hf == 0) {  // with the first half come the tile's V scales: lane = (block, 8 keys)
       const int b = lane / 8, chunk = lane % 8;
       if (b < NB) {
@@ -436,6 +345,11 @@ void DattnPartQ8(const DecodeArgs a) {
         vsr = *reinterpret_cast<const uint4*>(a.pools.vs + (ps * NB + b) * PT + (8 * chunk) % PT);
       }
     }
+  };
+  // the 8 codes of block b this lane feeds to instruction `sub` of the block's pair
+  auto kcodes = [&](int b, int sub) -> h8v {
+    if constexpr (Q8) return Codes8(kb[b][2 * sub], kb[b][2 * sub + 1]);
+    return sub == 0 ? NibblesLo8(kb[b][0], kb[b][1]) : NibblesHi8(kb[b][0], kb[b][1]);
   };
   // scores of the 32 keys in kb against all heads: two blocks (two accumulator chains) at a time
   auto scores = [&](int tt) {
@@ -448,10 +362,10 @@ void DattnPartQ8(const DecodeArgs a) {
       const h8v qb0 = *reinterpret_cast<const h8v*>(&lq[b + 1][0][half][n32 % 8][0]);
       const h8v qb1 = *reinterpret_cast<const h8v*>(&lq[b + 1][1][half][n32 % 8][0]);
       f16v c0 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}, c1 = c0;
-      c0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(qa0, Codes8(kb[b].x, kb[b].y), c0, 0, 0, 0);
-      c1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(qb0, Codes8(kb[b + 1].x, kb[b + 1].y), c1, 0, 0, 0);
-      c0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(qa1, Codes8(kb[b].z, kb[b].w), c0, 0, 0, 0);
-      c1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(qb1, Codes8(kb[b + 1].z, kb[b + 1].w), c1, 0, 0, 0);
+      c0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(qa0, kcodes(b, 0), c0, 0, 0, 0);
+      c1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(qb0, kcodes(b + 1, 0), c1, 0, 0, 0);
+      c0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(qa1, kcodes(b, 1), c0, 0, 0, 0);
+      c1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(qb1, kcodes(b + 1, 1), c1, 0, 0, 0);
       const uint32_t w = b < 2 ? ksc.x : b < 4 ? ksc.y : b < 6 ? ksc.z : ksc.w;  // scales of blocks b, b + 1
       const float d0 = WidenF16(static_cast<uint16_t>(w & 0xFFFF)) * qk_scale;
       const float d1 = WidenF16(static_cast<uint16_t>(w >> 16)) * qk_scale;
@@ -473,10 +387,17 @@ void DattnPartQ8(const DecodeArgs a) {
       const h8v s0 = *reinterpret_cast<const h8v*>(&lvs[b][16 * kg]);
       const h8v s1 = *reinterpret_cast<const h8v*>(&lvs[b][16 * kg + 8]);
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        const uint4 w = vb[2 * bb + j];
+      for (int j = 0; j < 2; ++j) {  // output tile 2 b + j: dims 32 b + 16 j + 0..15
+        const uint4 w = vb[Q8 ? 2 * bb + j : bb];
         const int nt = 2 * b + j;
-        const h8v v0 = Codes8(w.x, w.y) * s0, v1 = Codes8(w.z, w.w) * s1;
+        h8v v0, v1;
+        if constexpr (Q8) {
+          v0 = Codes8(w.x, w.y) * s0, v1 = Codes8(w.z, w.w) * s1;
+        } else if (j == 0) {
+          v0 = NibblesLo8(w.x, w.y) * s0, v1 = NibblesLo8(w.z, w.w) * s1;
+        } else {
+          v0 = NibblesHi8(w.x, w.y) * s0, v1 = NibblesHi8(w.z, w.w) * s1;
+        }
         o[nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa0, v0, o[nt], 0, 0, 0);
         o[nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa1, v1, o[nt], 0, 0, 0);
       }
@@ -528,8 +449,8 @@ void DattnPartQ8(const DecodeArgs a) {
       const int i = lane + 64 * e, b = i / 32, sub = (i / 16) % 2, hf = (i / 8) % 2, rw = i % 8;
       qreg[e] = h8v{0, 0, 0, 0, 0, 0, 0, 0};
       if (rw < G)
-        qreg[e] = LoadQ8(a.q, (size_t(cur.s) * g.n_q + size_t(cur.h) * G + rw) * D + b * 32 + 16 * hf + 8 * sub,
-                         a.q_dtype);
+        qreg[e] = LoadQ8(a.q, (size_t(cur.s) * g.n_q + size_t(cur.h) * G + rw) * D + b * 32 +
+                                   (Q8 ? 16 * hf + 8 * sub : 16 * sub + 8 * hf), a.q_dtype);
     }
     row = a.table + int64_t(cur.s) * a.stride;
     int tile = cur.first + (idx - cur.base);
@@ -702,15 +623,10 @@ Plan MakePlan(const Geom& g, int32_t n_seqs, int32_t max_seq_len) {
   const int64_t max_tiles = (int64_t(p.max_len) + kTile - 1) / kTile;
   const int64_t line_max = max_tiles * n_seqs * g.n_kv;
   // Tuning knobs; the environment overrides are for experiments.
-  if (g.format == 8) {  // one 8-wave workgroup per CU (two waves per SIMD)
-    p.wpc = kWavesPerGroup;
-    p.min_chunk_tiles = EnvInt("YAHKV_DECODE_MIN_CHUNK_TILES", 2 * kWavesPerGroup, 1, 1 << 20);
-    p.n_chunks = EnvInt("YAHKV_DECODE_CHUNKS", ComputeUnits(), 1, 1 << 20);
-  } else {  // scalar q4_0 kernel: one wave per chunk, 16 waves per CU
-    p.wpc = 1;
-    p.min_chunk_tiles = 2;
-    p.n_chunks = ComputeUnits() * 16;
-  }
+  // one 8-wave workgroup per CU (two waves per SIMD)
+  p.wpc = kWavesPerGroup;
+  p.min_chunk_tiles = EnvInt("YAHKV_DECODE_MIN_CHUNK_TILES", 2 * kWavesPerGroup, 1, 1 << 20);
+  p.n_chunks = EnvInt("YAHKV_DECODE_CHUNKS", ComputeUnits(), 1, 1 << 20);
   p.n_chunks =
       static_cast<int32_t>(std::min<int64_t>(p.n_chunks, (line_max + p.min_chunk_tiles - 1) / p.min_chunk_tiles));
   const size_t parts = (size_t(p.n_chunks) + size_t(n_seqs) * g.n_kv) * p.wpc;
@@ -787,20 +703,22 @@ extern "C" int yahkv_decode_part(const yahkv_geometry* g, const yahkv_pools* poo
   const Geom& m = a.g;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const dim3 grid(static_cast<unsigned>(a.n_chunks));
+#define YAHKV_LAUNCH_PART(FF, DD, PP) \
+  hipLaunchKernelGGL((DattnPart<FF, DD, PP>), grid, dim3(64 * kWavesPerGroup), 0, st, a)
+#define YAHKV_LAUNCH_FMT(FF)                                       \
+  if (m.hd == 256 && m.pt == 64) YAHKV_LAUNCH_PART(FF, 256, 64);      \
+  else if (m.hd == 256 && m.pt == 32) YAHKV_LAUNCH_PART(FF, 256, 32); \
+  else if (m.hd == 256) YAHKV_LAUNCH_PART(FF, 256, 16);               \
+  else if (m.pt == 64) YAHKV_LAUNCH_PART(FF, 128, 64);                \
+  else if (m.pt == 32) YAHKV_LAUNCH_PART(FF, 128, 32);                \
+  else YAHKV_LAUNCH_PART(FF, 128, 16)
   if (m.format == 8) {
-#define YAHKV_LAUNCH_Q8(DD, PP) hipLaunchKernelGGL((DattnPartQ8<DD, PP>), grid, dim3(64 * kWavesPerGroup), 0, st, a)
-    if (m.hd == 256 && m.pt == 64) YAHKV_LAUNCH_Q8(256, 64);
-    else if (m.hd == 256 && m.pt == 32) YAHKV_LAUNCH_Q8(256, 32);
-    else if (m.hd == 256) YAHKV_LAUNCH_Q8(256, 16);
-    else if (m.pt == 64) YAHKV_LAUNCH_Q8(128, 64);
-    else if (m.pt == 32) YAHKV_LAUNCH_Q8(128, 32);
-    else YAHKV_LAUNCH_Q8(128, 16);
-#undef YAHKV_LAUNCH_Q8
-  } else if (m.hd == 256) {
-    hipLaunchKernelGGL((DattnPartQ4<256>), grid, dim3(64), 0, st, a);
+    YAHKV_LAUNCH_FMT(8);
   } else {
-    hipLaunchKernelGGL((DattnPartQ4<128>), grid, dim3(64), 0, st, a);
+    YAHKV_LAUNCH_FMT(4);
   }
+#undef YAHKV_LAUNCH_FMT
+#undef YAHKV_LAUNCH_PART
   return LaunchStatus();
 }
 
