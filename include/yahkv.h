@@ -145,13 +145,20 @@ int yahkv_decode_attend(const yahkv_geometry* g, const yahkv_pools* pools, const
  *   q    [n_seqs][chunk_len][n_q_heads][D] bf16
  *   gate [n_seqs][chunk_len][n_q_heads][D] f32 or NULL
  *   out  [n_seqs][chunk_len][n_q_heads][D] of out_dtype (F32, F16 or BF16)
- * prefix_len is device int32 [n_seqs]; max_prefix_len is its host-side upper bound. K, V and the softmax
- * numerators enter the matrix unit as bf16 (round to nearest even), sums are f32. q8_0 pools only in this build.
- * Replaces yah_attn_wmma with its quantized staging (gen_attn_fa.py:1589-1595, 2664-2779). */
+ * prefix_len is device int32 [n_seqs]; max_prefix_len is its host-side upper bound; softmax_scale > 0. K, V and
+ * the softmax numerators enter the matrix unit as bf16 (round to nearest even), sums are f32.
+ * With a workspace of yahkv_prefill_workspace_bytes() the prefix is decoded to bf16 once per call and the attention
+ * kernel reads the decoded tiles (the reference's yah_kdeq8 / yah_vdeq8 into a 16-bit pool followed by yah_attn_wmma,
+ * gen_attn_fa.py:4648-4861, 1589-1595); q8_0 and q4_0. With workspace NULL the tiles are decoded inside the attention
+ * kernel while they are staged (gen_attn_fa.py:2664-2779): no extra memory, slower, q8_0 only
+ * (q4_0: YAHKV_ERR_WORKSPACE). Both give the same results up to the order of f32 sums. */
+size_t yahkv_prefill_workspace_bytes(const yahkv_geometry* g, int32_t n_seqs, int32_t max_prefix_len,
+                                     int32_t chunk_len);
 int yahkv_prefill_attend(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
                          int32_t page_table_stride, const int32_t* prefix_len, int32_t n_seqs,
                          int32_t max_prefix_len, int32_t chunk_len, const void* q, float softmax_scale,
-                         const float* gate, void* out, int32_t out_dtype, void* stream);
+                         const float* gate, void* out, int32_t out_dtype, void* workspace, size_t workspace_bytes,
+                         void* stream);
 
 /* Gather the blocks of tokens [0, n_tokens) of one sequence back into ggml array-of-blocks order:
  * dst_k / dst_v are device buffers [n_tokens][H][NB][34 or 18 bytes]. `table_row` is that sequence's row of

@@ -36,15 +36,25 @@ def build(yahkv, torch, fmt, n_q, n_kv, hd, pt, prefix, chunk, seed, fill=0):
     return g, table, host, dev, t_table, rng, to_t
 
 
-@pytest.mark.parametrize("fmt,n_q,n_kv,hd,pt,prefix,chunk", [
-    (8, 24, 4, 256, 64, [100, 0, 64 * 3 + 5], 70),
-    (8, 24, 4, 256, 64, [1000], 256),
-    (8, 8, 2, 128, 16, [37, 0, 64], 21),
-    (8, 6, 2, 256, 32, [31, 500], 64),
-    (8, 10, 2, 128, 64, [129], 130),
+# path "images": decode to bf16 tile images in a workspace, then attention; "fused": one kernel, no workspace (q8_0)
+@pytest.mark.parametrize("path,fmt,n_q,n_kv,hd,pt,prefix,chunk", [
+    ("images", 8, 24, 4, 256, 64, [100, 0, 64 * 3 + 5], 70),
+    ("images", 8, 24, 4, 256, 64, [1000], 256),
+    ("images", 8, 8, 2, 128, 16, [37, 0, 64], 21),
+    ("images", 8, 6, 2, 256, 32, [31, 500], 64),
+    ("images", 8, 10, 2, 128, 64, [129], 130),
+    ("images", 4, 24, 4, 256, 64, [100, 0, 64 * 3 + 5], 70),
+    ("images", 4, 8, 2, 128, 16, [37, 0, 64], 21),
+    ("images", 4, 6, 2, 256, 32, [31, 500], 64),
+    ("fused", 8, 24, 4, 256, 64, [100, 0, 64 * 3 + 5], 70),
+    ("fused", 8, 24, 4, 256, 64, [1000], 256),
+    ("fused", 8, 8, 2, 128, 16, [37, 0, 64], 21),
+    ("fused", 8, 6, 2, 256, 32, [31, 500], 64),
+    ("fused", 8, 10, 2, 128, 64, [129], 130),
 ])
-def test_prefill_against_oracle(yahkv, torch_gpu, fmt, n_q, n_kv, hd, pt, prefix, chunk):
+def test_prefill_against_oracle(yahkv, torch_gpu, path, fmt, n_q, n_kv, hd, pt, prefix, chunk):
     torch = torch_gpu
+    ws = None if path == "images" else False
     g, table, host, dev, t_table, rng, to_t = build(yahkv, torch, fmt, n_q, n_kv, hd, pt, prefix, chunk,
                                                     seed=hd + pt + chunk, fill=0x7F)
     q = to_bf16_f32(rng.standard_normal((len(prefix), chunk, n_q, hd)))
@@ -53,7 +63,7 @@ def test_prefill_against_oracle(yahkv, torch_gpu, fmt, n_q, n_kv, hd, pt, prefix
     t_prefix = torch.tensor(prefix, dtype=torch.int32, device="cuda")
     for gt in (None, gate):
         tg = None if gt is None else torch.from_numpy(gt).cuda()
-        out = yahkv.prefill_attend(dev, t_table, t_prefix, max(prefix), to_t(q), scale, gate=tg)
+        out = yahkv.prefill_attend(dev, t_table, t_prefix, max(prefix), to_t(q), scale, gate=tg, workspace=ws)
         torch.cuda.synchronize()
         got = out.cpu().numpy()
         assert np.all(np.isfinite(got))
@@ -62,11 +72,13 @@ def test_prefill_against_oracle(yahkv, torch_gpu, fmt, n_q, n_kv, hd, pt, prefix
         exact = oracle.prefill_attend(host, table, prefix, q, scale, gt)
         assert rel_err(got, exact) < 3 * 2.0 ** -9
     # bf16 output: the same numbers rounded once more
-    out16 = yahkv.prefill_attend(dev, t_table, t_prefix, max(prefix), to_t(q), scale, out_dtype=torch.bfloat16)
+    out16 = yahkv.prefill_attend(dev, t_table, t_prefix, max(prefix), to_t(q), scale, out_dtype=torch.bfloat16,
+                                 workspace=ws)
     assert rel_err(out16.float().cpu().numpy(), oracle.prefill_attend(host, table, prefix, q, scale, None, True)) < 2 * 2.0 ** -9
 
 
-def test_prefill_special_cases(yahkv, torch_gpu):
+@pytest.mark.parametrize("ws", [None, False], ids=["images", "fused"])
+def test_prefill_special_cases(yahkv, torch_gpu, ws):
     """Closed-form checks: the first query of a sequence without prefix returns its own V row; a chunk of one query
     equals decode attention at that length; independent float64 closed form for a few rows."""
     torch = torch_gpu
@@ -74,7 +86,7 @@ def test_prefill_special_cases(yahkv, torch_gpu):
     g, table, host, dev, t_table, rng, to_t = build(yahkv, torch, 8, 24, 4, 256, 64, prefix, chunk, seed=5)
     q = to_bf16_f32(rng.standard_normal((2, chunk, 24, 256)))
     t_prefix = torch.tensor(prefix, dtype=torch.int32, device="cuda")
-    got = yahkv.prefill_attend(dev, t_table, t_prefix, 77, to_t(q), 0.0625).cpu().numpy()
+    got = yahkv.prefill_attend(dev, t_table, t_prefix, 77, to_t(q), 0.0625, workspace=ws).cpu().numpy()
     (ks, kc), (vs, vc) = logical_blocks(host.arrays(), g, table[0], chunk)
     Kd, Vd = dequant(ks, kc), dequant(vs, vc)
     assert rel_err(got[0, 0], np.repeat(to_bf16_f32(Vd[0]), 6, 0)) < 1e-6       # one visible key: out = bf16(V row)
@@ -82,11 +94,26 @@ def test_prefill_special_cases(yahkv, torch_gpu):
         assert rel_err(got[0, t], closed_form(Kd[:t + 1], Vd[:t + 1], q[0, t], 0.0625)) < 3 * 2.0 ** -9
     lens = [p + chunk for p in prefix]
     one = yahkv.prefill_attend(dev, t_table, torch.tensor([l - 1 for l in lens], dtype=torch.int32, device="cuda"),
-                               max(lens), to_t(q[:, -1:]), 0.0625).cpu().numpy()
+                               max(lens), to_t(q[:, -1:]), 0.0625, workspace=ws).cpu().numpy()
     dec = yahkv.decode_attend(dev, t_table, torch.tensor(lens, dtype=torch.int32, device="cuda"), max(lens),
                               to_t(q[:, -1]), 0.0625).cpu().numpy()
     assert rel_err(one[:, 0], dec) < 3 * 2.0 ** -9
     assert rel_err(one[:, 0], got[:, -1]) < 1e-6                                 # same query, same keys, same kernel
+
+
+def test_both_paths_agree(yahkv, torch_gpu):
+    """The two paths feed the matrix unit the same bf16 values; only the order of the f32 sums differs."""
+    torch = torch_gpu
+    prefix, chunk = [300, 5], 100
+    g, table, host, dev, t_table, rng, to_t = build(yahkv, torch, 8, 24, 4, 256, 64, prefix, chunk, seed=6)
+    q = to_t(to_bf16_f32(rng.standard_normal((2, chunk, 24, 256))))
+    t_prefix = torch.tensor(prefix, dtype=torch.int32, device="cuda")
+    a = yahkv.prefill_attend(dev, t_table, t_prefix, 300, q, 0.0625).cpu().numpy()
+    b = yahkv.prefill_attend(dev, t_table, t_prefix, 300, q, 0.0625, workspace=False).cpu().numpy()
+    assert rel_err(a, b) < 1e-3
+    ws = torch.empty(yahkv.prefill_workspace_bytes(dev.geom, 2, 400, chunk), dtype=torch.uint8, device="cuda")
+    c = yahkv.prefill_attend(dev, t_table, t_prefix, 400, q, 0.0625, workspace=ws).cpu().numpy()   # a looser bound
+    assert np.array_equal(a, c)
 
 
 def test_prefill_rejects_bad_arguments(yahkv, torch_gpu):
@@ -96,10 +123,18 @@ def test_prefill_rejects_bad_arguments(yahkv, torch_gpu):
     dev = yahkv.DevicePools(g)
     table = torch.zeros((1, 4), dtype=torch.int32, device="cuda")
     q = torch.zeros((1, 8, 24, 256), dtype=torch.bfloat16, device="cuda")
-    with pytest.raises(yahkv.YahkvError) as e:                                    # q4_0 prefill is not built
-        yahkv.prefill_attend(dev, table, torch.zeros(1, dtype=torch.int32, device="cuda"), 0, q, 0.0625)
-    assert e.value.status == -2
+    zero = torch.zeros(1, dtype=torch.int32, device="cuda")
+    with pytest.raises(yahkv.YahkvError) as e:                                    # q4_0 needs the workspace
+        yahkv.prefill_attend(dev, table, zero, 0, q, 0.0625, workspace=False)
+    assert e.value.status == -4
+    with pytest.raises(yahkv.YahkvError) as e:                                    # workspace too small
+        yahkv.prefill_attend(dev, table, zero, 0, q, 0.0625, workspace=torch.empty(256, dtype=torch.uint8, device="cuda"))
+    assert e.value.status == -4
+    with pytest.raises(yahkv.YahkvError) as e:                                    # scale must be positive
+        yahkv.prefill_attend(dev, table, zero, 0, q, 0.0)
+    assert e.value.status == -1
     g8 = yahkv.geometry(8, 24, 4, 256, 64, 8)
     st = yahkv.DevicePools(g8).struct()
-    rc = yahkv.lib.yahkv_prefill_attend(C.byref(g8), C.byref(st), None, 4, None, 1, 0, 8, None, 0.0625, None, None, 0, None)
+    rc = yahkv.lib.yahkv_prefill_attend(C.byref(g8), C.byref(st), None, 4, None, 1, 0, 8, None, 0.0625, None, None, 0,
+                                        None, 0, None)
     assert rc == -1

@@ -50,7 +50,10 @@ def _load():
     lib.yahkv_decode_part.argtypes = [G, P, i32p, i32, i32p, i32, i32, vp, i32, C.c_float, vp, C.c_size_t, vp]
     lib.yahkv_decode_reduce.argtypes = [G, i32, i32p, i32, i32, vp, vp, vp, C.c_size_t, vp]
     lib.yahkv_decode_attend.argtypes = [G, P, i32p, i32, i32p, i32, i32, vp, i32, C.c_float, vp, vp, vp, C.c_size_t, vp]
-    lib.yahkv_prefill_attend.argtypes = [G, P, i32p, i32, i32p, i32, i32, i32, vp, C.c_float, vp, vp, i32, vp]
+    lib.yahkv_prefill_workspace_bytes.restype = C.c_size_t
+    lib.yahkv_prefill_workspace_bytes.argtypes = [G, i32, i32, i32]
+    lib.yahkv_prefill_attend.argtypes = [G, P, i32p, i32, i32p, i32, i32, i32, vp, C.c_float, vp, vp, i32, vp,
+                                         C.c_size_t, vp]
     lib.yahkv_gather_blocks.argtypes = [G, P, i32p, i32, vp, vp, vp]
     lib.yahkv_pagepool_create.restype = C.c_void_p
     lib.yahkv_pagepool_create.argtypes = [i32]
@@ -226,17 +229,29 @@ def decode_reduce(g, table_stride, seq_len, n_seqs, max_seq_len, out, workspace,
                                    _dp(workspace), workspace.numel(), _stream()), "decode_reduce")
 
 
-def prefill_attend(pools, table, prefix_len, max_prefix_len, q, scale, gate=None, out=None, out_dtype=None):
-    """q: [n_seqs][chunk][n_q_heads][D] bf16; returns out (f32 unless out / out_dtype say otherwise), same shape."""
+def prefill_workspace_bytes(g, n_seqs, max_prefix_len, chunk_len):
+    return lib.yahkv_prefill_workspace_bytes(C.byref(g), n_seqs, max_prefix_len, chunk_len)
+
+
+def prefill_attend(pools, table, prefix_len, max_prefix_len, q, scale, gate=None, out=None, out_dtype=None,
+                   workspace=None):
+    """q: [n_seqs][chunk][n_q_heads][D] bf16; returns out (f32 unless out / out_dtype say otherwise), same shape.
+
+    workspace: a uint8 device tensor of prefill_workspace_bytes() (None: one is allocated for the call) selects the
+    two-pass path, decode to bf16 tile images and then attention; False selects the one-pass kernel (q8_0 only)."""
     import torch
     g = pools.geom
     assert q.is_contiguous() and q.dtype == torch.bfloat16 and table.is_contiguous()
     if out is None:
         out = torch.empty(q.shape, dtype=out_dtype or torch.float32, device=q.device)
+    if workspace is None:
+        workspace = torch.empty(prefill_workspace_bytes(g, q.shape[0], max_prefix_len, q.shape[1]), dtype=torch.uint8,
+                                device=q.device)
+    ws_ptr, ws_bytes = (None, 0) if workspace is False else (_dp(workspace), workspace.numel())
     st = pools.struct()
     _check(lib.yahkv_prefill_attend(C.byref(g), C.byref(st), _dp(table), table.shape[1], _dp(prefix_len), q.shape[0],
                                     max_prefix_len, q.shape[1], _dp(q), scale, _dp(gate), _dp(out), _dtype_code(out),
-                                    _stream()), "prefill_attend")
+                                    ws_ptr, ws_bytes, _stream()), "prefill_attend")
     return out
 
 

@@ -279,14 +279,21 @@ class KvPrefill {
     const int32_t* pre = static_cast<const int32_t*>(prefix_dev_.get());
     Check(yahkv_append(&dec_.geometry(), &pools, ptab, dec_.page_table_stride(), pre, nullptr, n_seqs, chunk_len, k, v,
                        kv_dtype, dec_.stream()), "append");
+    // the decoded prefix (bf16 tile images) lives in a buffer that grows with the longest call so far
+    const size_t need = yahkv_prefill_workspace_bytes(&dec_.geometry(), n_seqs, max_prefix, chunk_len);
+    if (need > images_.size()) {
+      CheckHip(hipStreamSynchronize(dec_.stream()), "prefill workspace");
+      images_ = DeviceBuffer(need);
+    }
     Check(yahkv_prefill_attend(&dec_.geometry(), &pools, ptab, dec_.page_table_stride(), pre, n_seqs, max_prefix,
-                               chunk_len, q, softmax_scale, gate, out, out_dtype, dec_.stream()), "prefill_attend");
+                               chunk_len, q, softmax_scale, gate, out, out_dtype, images_.get(), images_.size(),
+                               dec_.stream()), "prefill_attend");
     for (int32_t s = 0; s < n_seqs; ++s) dec_.SetLength(s, prefix[size_t(s)] + chunk_len);
   }
 
  private:
   KvDecoder& dec_;
-  DeviceBuffer prefix_dev_;
+  DeviceBuffer prefix_dev_, images_;
 };
 
 }  // namespace yahkv_host

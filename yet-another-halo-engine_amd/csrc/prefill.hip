@@ -80,6 +80,44 @@ __device__ __forceinline__ void Decode16V(const uint4 c, const uint4 s0, const u
   *lo = uint4{o[0], o[1], o[2], o[3]}, *hi = uint4{o[4], o[5], o[6], o[7]};
 }
 
+// out = o / l (* sigmoid(gate)); lane (query, lane group jg) holds dims 16 dt + 4 jg + r of its query in each row block
+template <int D>
+__device__ __forceinline__ void StoreRows(const PrefillArgs& a, int s, int h, int G, int jg, const f4v (&o)[RB][D / 16],
+                                          const float (&lsum)[RB], const int (&qpos)[RB], const int (&head)[RB]) {
+  constexpr int NDT = D / 16;
+  const Geom& g = a.g;
+#pragma unroll
+  for (int i = 0; i < RB; ++i) {
+    float l = lsum[i];
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    if (head[i] >= G || qpos[i] >= a.chunk_len) continue;
+    const float inv = 1.0f / l;
+    const size_t base = ((size_t(s) * a.chunk_len + qpos[i]) * g.n_q + size_t(h) * G + head[i]) * D;
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt) {
+      float v[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        v[r] = o[i][dt][r] * inv;
+        if (a.gate != nullptr) v[r] *= 1.0f / (1.0f + __expf(-a.gate[base + 16 * dt + 4 * jg + r]));
+      }
+      const size_t e = base + 16 * dt + 4 * jg;
+      if (a.out_dtype == YAHKV_F32) {
+        *reinterpret_cast<float4*>(static_cast<float*>(a.out) + e) = float4{v[0], v[1], v[2], v[3]};
+      } else if (a.out_dtype == YAHKV_BF16) {
+        *reinterpret_cast<uint2*>(static_cast<uint16_t*>(a.out) + e) = uint2{PackBf16(v[0], v[1]), PackBf16(v[2], v[3])};
+      } else {
+        typedef _Float16 h2v __attribute__((ext_vector_type(2)));
+        const h2v x = {static_cast<_Float16>(v[0]), static_cast<_Float16>(v[1])};
+        const h2v y = {static_cast<_Float16>(v[2]), static_cast<_Float16>(v[3])};
+        *reinterpret_cast<uint2*>(static_cast<uint16_t*>(a.out) + e) =
+            uint2{__builtin_bit_cast(uint32_t, x), __builtin_bit_cast(uint32_t, y)};
+      }
+    }
+  }
+}
+
 template <int D, int PT>
 __global__ __launch_bounds__(256) void PrefillAttendQ8(const PrefillArgs a) {
   constexpr int NB = D / 32, NDT = D / 16, KS = D / 32;  // blocks, 16-dim tiles, 32-dim steps of the first product
@@ -321,37 +359,293 @@ __global__ __launch_bounds__(256) void PrefillAttendQ8(const PrefillArgs a) {
     __syncthreads();  // every wave is done with lv; K(tile + 1) and its V scales are in place
   }
 
-  // ---- out = o / l (* sigmoid(gate)); lane (query, group jg) holds dims 16 dt + 4 jg + r
+  StoreRows<D>(a, s, h, G, jg, o, lsum, qpos, head);
+}
+
+
+// ---- two passes: tile images, then attention on the images ---------------------------------------------------------------
+//
+// The fused kernel above decodes every K / V tile once per workgroup, i.e. once per 64 chunk positions and pair of
+// heads: at 2048 positions and 6 heads per kv head that is 96 times per key, and with one wave per SIMD the decode's
+// vector instructions and the matrix instructions compete for the wave's issue slots. When the caller provides a
+// workspace, the prefix is decoded once per call instead (the reference does the same: yah_kdeq8 / yah_vdeq8 into an
+// f16 pool before yah_attn_wmma, gen_attn_fa.py:4648-4861): `PrefillImages` writes, per (sequence, kv head, tile of
+// 64 keys), the bf16 K tile and V^T tile exactly as the attention kernel wants them in LDS, and `PrefillAttendImg`
+// copies images to LDS with direct global-to-LDS loads (no registers, no vector instructions) one tile ahead.
+//
+// K image: 64 rows (keys) of D bf16; the 16-byte chunk c of row r sits at chunk position c ^ (r % 8).
+// V image: D rows (dims) of 64 bf16; chunk c = 4 s2 + jg of row r holds keys 32 s2 + 4 jg + 0..3 and 32 s2 + 16 +
+// 4 jg + 0..3 (the eight k-slots of lane group jg in step s2 of the second product) and sits at position c ^ (r % 8).
+// With the XOR, the sixteen rows a wave reads at once fall into different banks. Keys at or past the end of the
+// sequence are zero in both images.
+struct ImageArgs {
+  Geom g;
+  Pools pools;
+  const int32_t* table;
+  int32_t stride;
+  const int32_t* prefix_len;
+  int32_t n_seqs, max_prefix, chunk_len;
+  char* img;
+  int32_t tiles_per_pair;
+};
+
+template <int D>
+constexpr int TileImageBytes() { return 2 * kKeys * D * 2; }
+
+__device__ __forceinline__ int ClampPrefix(const int32_t* prefix_len, int s, int max_prefix, int stride, int pt,
+                                           int chunk_len) {
+  return min(max(prefix_len[s], 0), min(max_prefix, stride * pt - chunk_len));
+}
+
+template <int FMT, int D, int PT>
+__global__ __launch_bounds__(256) void PrefillImages(const ImageArgs a) {
+  constexpr int NB = D / 32, CPR = D / 8;  // blocks; 16-byte chunks per K row
+  constexpr bool Q8 = FMT == 8;
+  const Geom g = a.g;
+  const int H = g.n_kv, tile = blockIdx.x, pair = blockIdx.y, s = pair / H, h = pair % H, tid = threadIdx.x;
+  const int n_keys = ClampPrefix(a.prefix_len, s, a.max_prefix, a.stride, g.pt, a.chunk_len) + a.chunk_len;
+  if (tile * kKeys >= n_keys) return;
+  const int32_t* row = a.table + int64_t(s) * a.stride;
+  char* kimg = a.img + (size_t(pair) * a.tiles_per_pair + tile) * TileImageBytes<D>();
+  char* vimg = kimg + kKeys * D * 2;
+  auto page_head = [&](int key) -> size_t {
+    return size_t(ClampPage(row[min(key / PT, a.stride - 1)], g.n_pages)) * H + h;
+  };
+  for (int p = tid; p < kKeys * CPR; p += 256) {  // K: chunk = dims 8 c .. 8 c + 7 of one key
+    const int key = p / CPR, c = (p % CPR) ^ (key % 8), kk = tile * kKeys + key;
+    uint32_t o[4] = {0u, 0u, 0u, 0u};
+    if (kk < n_keys) {
+      const size_t ph = page_head(kk);
+      const int t = kk % PT, b = c / 4, off = (8 * c) % 32;
+      const float d = WidenF16(a.pools.ks[(ph * PT + t) * NB + b]);
+      float v[8];
+      if constexpr (Q8) {
+        const uint2 w = *reinterpret_cast<const uint2*>(a.pools.kq + ((ph * NB + b) * PT + t) * 32 + off);
 #pragma unroll
-  for (int i = 0; i < RB; ++i) {
-    float l = lsum[i];
-    l += __shfl_xor(l, 16, 64);
-    l += __shfl_xor(l, 32, 64);
-    if (head[i] >= G || qpos[i] >= a.chunk_len) continue;
-    const float inv = 1.0f / l;
-    const size_t base = ((size_t(s) * a.chunk_len + qpos[i]) * g.n_q + size_t(h) * G + head[i]) * D;
+        for (int e = 0; e < 8; ++e)
+          v[e] = d * static_cast<float>(static_cast<int8_t>(((e < 4 ? w.x : w.y) >> (8 * (e % 4))) & 0xFF));
+      } else {  // byte j of a block: low nibble dim j, high nibble dim 16 + j
+        const uint2 w = *reinterpret_cast<const uint2*>(a.pools.kq + ((ph * NB + b) * PT + t) * 16 + off % 16);
 #pragma unroll
-    for (int dt = 0; dt < NDT; ++dt) {
+        for (int e = 0; e < 8; ++e)
+          v[e] = d * static_cast<float>(int((((e < 4 ? w.x : w.y) >> (8 * (e % 4))) >> (off / 16 * 4)) & 0xF) - 8);
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = PackBf16(v[2 * e], v[2 * e + 1]);
+    }
+    *reinterpret_cast<uint4*>(kimg + size_t(p) * 16) = uint4{o[0], o[1], o[2], o[3]};
+  }
+  for (int p = tid; p < D * 8; p += 256) {  // V: chunk = 4 + 4 keys of one dim
+    const int dim = p / 8, c = (p % 8) ^ (dim % 8), s2 = c / 4, jg = c % 4, b = dim / 32;
+    uint32_t o[4];
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf) {
+      const int kk = tile * kKeys + 32 * s2 + 16 * hf + 4 * jg;  // four keys, always within one page
+      const size_t ph = page_head(kk);
+      const int t = kk % PT;
+      const uint2 sw = *reinterpret_cast<const uint2*>(a.pools.vs + (ph * NB + b) * PT + t);
+      uint32_t w;
+      int shift = 0;
+      if constexpr (Q8) {
+        w = *reinterpret_cast<const uint32_t*>(a.pools.vq + (ph * D + dim) * PT + t);
+      } else {  // byte row j of a block: low nibble dim j, high nibble dim 16 + j
+        w = *reinterpret_cast<const uint32_t*>(a.pools.vq + ((ph * NB + b) * 16 + dim % 16) * PT + t);
+        shift = dim % 32 / 16 * 4;
+      }
       float v[4];
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        v[r] = o[i][dt][r] * inv;
-        if (a.gate != nullptr) v[r] *= 1.0f / (1.0f + __expf(-a.gate[base + 16 * dt + 4 * jg + r]));
+      for (int e = 0; e < 4; ++e) {
+        const float d = WidenF16(static_cast<uint16_t>((e < 2 ? sw.x : sw.y) >> (16 * (e % 2))));
+        const uint32_t byte = (w >> (8 * e)) & 0xFF;
+        const float code = Q8 ? static_cast<float>(static_cast<int8_t>(byte))
+                              : static_cast<float>(int((byte >> shift) & 0xF) - 8);
+        v[e] = kk + e < n_keys ? d * code : 0.0f;
       }
-      const size_t e = base + 16 * dt + 4 * jg;
-      if (a.out_dtype == YAHKV_F32) {
-        *reinterpret_cast<float4*>(static_cast<float*>(a.out) + e) = float4{v[0], v[1], v[2], v[3]};
-      } else if (a.out_dtype == YAHKV_BF16) {
-        *reinterpret_cast<uint2*>(static_cast<uint16_t*>(a.out) + e) = uint2{PackBf16(v[0], v[1]), PackBf16(v[2], v[3])};
-      } else {
-        typedef _Float16 h2v __attribute__((ext_vector_type(2)));
-        const h2v x = {static_cast<_Float16>(v[0]), static_cast<_Float16>(v[1])};
-        const h2v y = {static_cast<_Float16>(v[2]), static_cast<_Float16>(v[3])};
-        *reinterpret_cast<uint2*>(static_cast<uint16_t*>(a.out) + e) =
-            uint2{__builtin_bit_cast(uint32_t, x), __builtin_bit_cast(uint32_t, y)};
+      o[2 * hf] = PackBf16(v[0], v[1]), o[2 * hf + 1] = PackBf16(v[2], v[3]);
+    }
+    *reinterpret_cast<uint4*>(vimg + size_t(p) * 16) = uint4{o[0], o[1], o[2], o[3]};
+  }
+}
+
+// Maximum over the four lane groups of a wave (lanes n, n + 16, n + 32, n + 48): v_permlane16_swap exchanges the odd
+// rows of one operand with the even rows of the other, v_permlane32_swap the upper half with the lower half; with both
+// operands equal, the maximum of the two results is the maximum over the pair of rows (halves) in every lane.
+__device__ __forceinline__ float MaxOverLaneGroups(float v) {
+  const uint32_t u = __builtin_bit_cast(uint32_t, v);
+  const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  const uint32_t r0 = r[0], r1 = r[1];  // (a bit cast applied to r[1] directly reads r[0] with this compiler)
+  const float w = fmaxf(__builtin_bit_cast(float, r0), __builtin_bit_cast(float, r1));
+  const uint32_t x = __builtin_bit_cast(uint32_t, w);
+  const auto q = __builtin_amdgcn_permlane32_swap(x, x, false, false);
+  const uint32_t q0 = q[0], q1 = q[1];
+  return fmaxf(__builtin_bit_cast(float, q0), __builtin_bit_cast(float, q1));
+}
+
+// Same work split as the fused kernel: 4 waves, 64 chunk positions x 2 heads, two row blocks of 16 queries per wave,
+// everything transposed (keys along MFMA rows, queries along lanes). LDS holds two tile images; the copy of tile
+// i + 1 is issued before the arithmetic of tile i and waited for after it: one barrier per tile.
+template <int D>
+__global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, const char* img, int tiles_per_pair) {
+  constexpr int KS = D / 32, NDT = D / 16;
+  constexpr int KIMG = kKeys * D * 2, TIMG = TileImageBytes<D>();
+  constexpr int kCopies = TIMG / 1024 / 4;  // 1 KB wave-wide copies per wave and tile
+  const Geom g = a.g;
+  const int G = g.group(), H = g.n_kv;
+  const int n_qt = (a.chunk_len + kQueries - 1) / kQueries, n_hp = (G + kHeadsPerGroup - 1) / kHeadsPerGroup;
+  const int bid = blockIdx.x, xcd = bid % 8, local = bid / 8, per_pair = n_qt * n_hp;
+  const int pair = xcd + 8 * (local / per_pair), qt = n_qt - 1 - (local % per_pair) / n_hp, hp = local % n_hp;
+  if (pair >= a.n_seqs * H) return;
+  const int s = pair / H, h = pair % H;
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / 64), lane = tid % 64;
+  const int qn = lane % 16, jg = lane / 16;
+  const int prefix = ClampPrefix(a.prefix_len, s, a.max_prefix, a.stride, g.pt, a.chunk_len);
+  const int q0 = qt * kQueries;
+  const int n_keys = min(prefix + q0 + kQueries, prefix + a.chunk_len);
+  const int n_tiles = (n_keys + kKeys - 1) / kKeys;
+
+  __shared__ __align__(1024) char lds[2][TIMG];
+
+  b8v qb[RB][KS];
+  int qpos[RB], head[RB];
+#pragma unroll
+  for (int i = 0; i < RB; ++i) {
+    const int rb = RB * wave + i;
+    head[i] = kHeadsPerGroup * hp + rb / 4;
+    qpos[i] = q0 + 16 * (rb % 4) + qn;
+    const int t = min(qpos[i], a.chunk_len - 1), hd = min(head[i], G - 1);
+    const uint16_t* qp = a.q + ((size_t(s) * a.chunk_len + t) * g.n_q + size_t(h) * G + hd) * D;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qb[i][ks] = *reinterpret_cast<const b8v*>(qp + 32 * ks + 8 * jg);
+  }
+  f4v o[RB][NDT];
+  float m[RB], lsum[RB];
+#pragma unroll
+  for (int i = 0; i < RB; ++i) {
+    m[i] = kNegBig, lsum[i] = 0.0f;
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt) o[i][dt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
+  }
+  const float sscale = a.scale * 1.4426950408889634f;
+  const char* src = img + size_t(pair) * tiles_per_pair * TIMG + size_t(lane) * 16;
+  auto copy_tile = [&](int tile) {
+    const char* from = src + size_t(tile) * TIMG;
+    char* to = lds[tile % 2];
+#pragma unroll
+    for (int j = 0; j < kCopies; ++j) {
+      const int c = wave + 4 * j;
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(from + c * 1024),
+                                       (__attribute__((address_space(3))) void*)(to + c * 1024), 16, 0, 0);
+    }
+  };
+  // byte offsets of this lane's operand reads within an image; the XOR with qn % 8 undoes the images' swizzle
+  const int sw = qn % 8;
+  const int koff = qn * (2 * D), voff = KIMG + qn * 128;
+
+  copy_tile(0);
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+  __syncthreads();
+  for (int tile = 0; tile < n_tiles; ++tile) {
+    if (tile + 1 < n_tiles) copy_tile(tile + 1);
+    const char* buf = lds[tile % 2];
+    // ---- S^T = K Q^T
+    f4v st[RB][4];
+#pragma unroll
+    for (int i = 0; i < RB; ++i)
+#pragma unroll
+      for (int kt = 0; kt < 4; ++kt) st[i][kt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
+    {
+      auto read_k = [&](int ks, int kt) -> b8v {
+        return *reinterpret_cast<const b8v*>(buf + koff + kt * 16 * (2 * D) + 16 * ((4 * ks + jg) ^ sw));
+      };
+      b8v ka[2][4];
+#pragma unroll
+      for (int kt = 0; kt < 4; ++kt) ka[0][kt] = read_k(0, kt);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        if (ks + 1 < KS) {
+#pragma unroll
+          for (int kt = 0; kt < 4; ++kt) ka[(ks + 1) % 2][kt] = read_k(ks + 1, kt);
+        }
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+          for (int i = 0; i < RB; ++i)
+            st[i][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[ks % 2][kt], qb[i][ks], st[i][kt], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
+    // ---- online softmax per query (= per lane). The accumulators are rescaled only in tiles where some query of the
+    // wave meets a new maximum, which becomes rare as the context grows.
+    const bool diag = (tile + 1) * kKeys > prefix + q0 + 1;
+    uint32_t pb[RB][2][4];
+#pragma unroll
+    for (int i = 0; i < RB; ++i) {
+      if (diag) {
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            if (tile * kKeys + 16 * kt + 4 * jg + r > prefix + qpos[i]) st[i][kt][r] = kNegBig;
+      }
+      float mx = fmaxf(fmaxf(st[i][0][0], st[i][0][1]), fmaxf(st[i][0][2], st[i][0][3]));
+#pragma unroll
+      for (int kt = 1; kt < 4; ++kt)
+        mx = fmaxf(mx, fmaxf(fmaxf(st[i][kt][0], st[i][kt][1]), fmaxf(st[i][kt][2], st[i][kt][3])));
+      mx = MaxOverLaneGroups(mx) * sscale;  // sscale > 0 is required by the entry point
+      if (__builtin_amdgcn_ballot_w64(mx > m[i]) != 0) {
+        const float mn = fmaxf(mx, m[i]);
+        const float alpha = __builtin_amdgcn_exp2f(m[i] - mn);
+        m[i] = mn;
+        lsum[i] *= alpha;
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) o[i][dt][r] *= alpha;
+      }
+      float psum = 0.0f;
+#pragma unroll
+      for (int kt = 0; kt < 4; ++kt) {
+        float p[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          p[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(st[i][kt][r], sscale, -m[i])), psum += p[r];
+        pb[i][kt / 2][2 * (kt % 2)] = PackBf16(p[0], p[1]);
+        pb[i][kt / 2][2 * (kt % 2) + 1] = PackBf16(p[2], p[3]);
+      }
+      lsum[i] += psum;
+    }
+    // ---- O^T += V^T P^T
+    {
+      auto read_v = [&](int dt, int s2) -> b8v {
+        return *reinterpret_cast<const b8v*>(buf + voff + dt * 16 * 128 + 16 * ((4 * s2 + jg) ^ sw));
+      };
+      b8v pv[RB][2];
+#pragma unroll
+      for (int i = 0; i < RB; ++i)
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2)
+          pv[i][s2] = __builtin_bit_cast(b8v, uint4{pb[i][s2][0], pb[i][s2][1], pb[i][s2][2], pb[i][s2][3]});
+      b8v va[3][2];
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) va[0][s2] = read_v(0, s2), va[1][s2] = read_v(1, s2);
+#pragma unroll
+      for (int dt = 0; dt < NDT; ++dt) {
+        if (dt + 2 < NDT) {
+#pragma unroll
+          for (int s2 = 0; s2 < 2; ++s2) va[(dt + 2) % 3][s2] = read_v(dt + 2, s2);
+        }
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+          for (int i = 0; i < RB; ++i)
+            o[i][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[dt % 3][s2], pv[i][s2], o[i][dt], 0, 0, 0);
+        if (dt % 2 == 1) __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's part of the next image has landed
+    __syncthreads();                     // ... and everybody's; everybody is done with this tile's image
   }
+  StoreRows<D>(a, s, h, G, jg, o, lsum, qpos, head);
 }
 
 }  // namespace
@@ -359,22 +653,38 @@ __global__ __launch_bounds__(256) void PrefillAttendQ8(const PrefillArgs a) {
 
 using namespace yahkv;
 
+namespace {
+int32_t TilesPerPair(int32_t max_prefix_len, int32_t chunk_len) {
+  return static_cast<int32_t>((int64_t(max_prefix_len) + chunk_len + kKeys - 1) / kKeys);
+}
+size_t ImageBytes(const Geom& m, int32_t n_seqs, int32_t max_prefix_len, int32_t chunk_len) {
+  return size_t(n_seqs) * m.n_kv * TilesPerPair(max_prefix_len, chunk_len) * (size_t(2) * kKeys * m.hd * 2);
+}
+}  // namespace
+
+extern "C" size_t yahkv_prefill_workspace_bytes(const yahkv_geometry* g, int32_t n_seqs, int32_t max_prefix_len,
+                                                int32_t chunk_len) {
+  if (CheckGeometry(g) || n_seqs <= 0 || max_prefix_len < 0 || chunk_len <= 0) return 0;
+  return ImageBytes(MakeGeom(*g), n_seqs, max_prefix_len, chunk_len);
+}
+
 extern "C" int yahkv_prefill_attend(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
                                     int32_t page_table_stride, const int32_t* prefix_len, int32_t n_seqs,
                                     int32_t max_prefix_len, int32_t chunk_len, const void* q, float softmax_scale,
-                                    const float* gate, void* out, int32_t out_dtype, void* stream) {
+                                    const float* gate, void* out, int32_t out_dtype, void* workspace,
+                                    size_t workspace_bytes, void* stream) {
   if (const int st = CheckGeometry(g)) return st;
   if (pools == nullptr || pools->kq == nullptr || pools->ks == nullptr || pools->vq == nullptr ||
       pools->vs == nullptr || page_table == nullptr || prefix_len == nullptr || q == nullptr || out == nullptr)
     return YAHKV_ERR_ARG;
   if (n_seqs <= 0 || chunk_len <= 0 || max_prefix_len < 0 || page_table_stride <= 0) return YAHKV_ERR_ARG;
+  if (!(softmax_scale > 0.0f)) return YAHKV_ERR_ARG;
   if (out_dtype != YAHKV_F32 && out_dtype != YAHKV_F16 && out_dtype != YAHKV_BF16) return YAHKV_ERR_ARG;
   if ((reinterpret_cast<uintptr_t>(pools->kq) | reinterpret_cast<uintptr_t>(pools->vq) |
        reinterpret_cast<uintptr_t>(pools->ks) | reinterpret_cast<uintptr_t>(pools->vs) |
-       reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(out)) & 15)
+       reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(workspace)) & 15)
     return YAHKV_ERR_ARG;
   const Geom m = MakeGeom(*g);
-  if (m.format != 8) return YAHKV_ERR_SHAPE;      // q4_0 prefill: not built yet
   if (int64_t(page_table_stride) * m.pt < chunk_len) return YAHKV_ERR_ARG;
   PrefillArgs a{};
   a.g = m, a.pools = MakePools(*pools), a.table = page_table, a.stride = page_table_stride, a.prefix_len = prefix_len;
@@ -385,13 +695,42 @@ extern "C" int yahkv_prefill_attend(const yahkv_geometry* g, const yahkv_pools* 
   const int pairs = n_seqs * m.n_kv, pair_slots = (pairs + 7) / 8 * 8;
   const dim3 grid(static_cast<unsigned>(pair_slots) * n_qt * n_hp);
   hipStream_t st = static_cast<hipStream_t>(stream);
+  if (workspace == nullptr) {  // one pass: tiles are decoded inside the attention kernel
+    if (m.format != 8) return YAHKV_ERR_WORKSPACE;  // q4_0 pools are only served through the images
 #define YAHKV_LAUNCH_PF(DD, PP) hipLaunchKernelGGL((PrefillAttendQ8<DD, PP>), grid, dim3(256), 0, st, a)
-  if (m.hd == 256 && m.pt == 64) YAHKV_LAUNCH_PF(256, 64);
-  else if (m.hd == 256 && m.pt == 32) YAHKV_LAUNCH_PF(256, 32);
-  else if (m.hd == 256) YAHKV_LAUNCH_PF(256, 16);
-  else if (m.pt == 64) YAHKV_LAUNCH_PF(128, 64);
-  else if (m.pt == 32) YAHKV_LAUNCH_PF(128, 32);
-  else YAHKV_LAUNCH_PF(128, 16);
+    if (m.hd == 256 && m.pt == 64) YAHKV_LAUNCH_PF(256, 64);
+    else if (m.hd == 256 && m.pt == 32) YAHKV_LAUNCH_PF(256, 32);
+    else if (m.hd == 256) YAHKV_LAUNCH_PF(256, 16);
+    else if (m.pt == 64) YAHKV_LAUNCH_PF(128, 64);
+    else if (m.pt == 32) YAHKV_LAUNCH_PF(128, 32);
+    else YAHKV_LAUNCH_PF(128, 16);
 #undef YAHKV_LAUNCH_PF
+    return LaunchStatus();
+  }
+  if (workspace_bytes < ImageBytes(m, n_seqs, max_prefix_len, chunk_len)) return YAHKV_ERR_WORKSPACE;
+  ImageArgs ia{};
+  ia.g = m, ia.pools = a.pools, ia.table = page_table, ia.stride = page_table_stride, ia.prefix_len = prefix_len;
+  ia.n_seqs = n_seqs, ia.max_prefix = max_prefix_len, ia.chunk_len = chunk_len;
+  ia.img = static_cast<char*>(workspace), ia.tiles_per_pair = TilesPerPair(max_prefix_len, chunk_len);
+  const dim3 igrid(static_cast<unsigned>(ia.tiles_per_pair), static_cast<unsigned>(pairs));
+#define YAHKV_LAUNCH_IMG(FF, DD, PP) hipLaunchKernelGGL((PrefillImages<FF, DD, PP>), igrid, dim3(256), 0, st, ia)
+#define YAHKV_LAUNCH_IMG_FMT(FF)                                     \
+  if (m.hd == 256 && m.pt == 64) YAHKV_LAUNCH_IMG(FF, 256, 64);         \
+  else if (m.hd == 256 && m.pt == 32) YAHKV_LAUNCH_IMG(FF, 256, 32);    \
+  else if (m.hd == 256) YAHKV_LAUNCH_IMG(FF, 256, 16);                  \
+  else if (m.pt == 64) YAHKV_LAUNCH_IMG(FF, 128, 64);                   \
+  else if (m.pt == 32) YAHKV_LAUNCH_IMG(FF, 128, 32);                   \
+  else YAHKV_LAUNCH_IMG(FF, 128, 16)
+  if (m.format == 8) {
+    YAHKV_LAUNCH_IMG_FMT(8);
+  } else {
+    YAHKV_LAUNCH_IMG_FMT(4);
+  }
+#undef YAHKV_LAUNCH_IMG_FMT
+#undef YAHKV_LAUNCH_IMG
+  if (const int rc = LaunchStatus()) return rc;
+  const char* img = static_cast<const char*>(workspace);
+  if (m.hd == 256) hipLaunchKernelGGL((PrefillAttendImg<256>), grid, dim3(256), 0, st, a, img, ia.tiles_per_pair);
+  else hipLaunchKernelGGL((PrefillAttendImg<128>), grid, dim3(256), 0, st, a, img, ia.tiles_per_pair);
   return LaunchStatus();
 }
