@@ -367,12 +367,15 @@ void orc_prefill_attend(const orc_geometry* g, const orc_pools* pools, const int
             sc[k] = dot * softmax_scale;
             if (sc[k] > M) M = sc[k];
           }
+          /* bf16 model: numerators are taken against the maximum rounded up to a whole power of two, so that
+           * where they are rounded does not depend on the order in which a running maximum met the keys */
+          if (bf16_operands) M = ceil(M * 1.4426950408889634) / 1.4426950408889634;
           double l = 0;
           for (int d = 0; d < D; ++d) acc[d] = 0;
           for (int k = 0; k < keys; ++k) {
             const double e = exp(sc[k] - M);
-            l += e;
             const double pe = bf16_operands ? (double)round_bf16((float)e) : e;
+            l += pe; /* the denominator sums what the numerator multiplies */
             for (int d = 0; d < D; ++d) acc[d] += pe * vd[(size_t)k * D + d];
           }
           for (int d = 0; d < D; ++d) {

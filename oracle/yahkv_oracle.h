@@ -78,7 +78,10 @@ void orc_decode_attend(const orc_geometry* g, const orc_pools* pools, const int3
                        const int32_t* seq_len, int32_t n_seqs, const float* q, float softmax_scale,
                        const float* gate, float* out);
 /* q f32 [n_seqs][chunk_len][n_q_heads][D]; out f32 same shape. bf16_operands != 0 rounds the dequantized K and V
- * and the softmax numerators to bf16 before they are multiplied, which is what a bf16 matrix unit sees. */
+ * and the softmax numerators to bf16 before they are multiplied, which is what a bf16 matrix unit sees; the
+ * numerators are then 2^(score * log2 e - ceil(max score * log2 e)): with the maximum a whole power of two, an
+ * online softmax that rescales by powers of two rounds every numerator exactly as this global form does. The
+ * denominator is the sum of the rounded numerators. */
 void orc_prefill_attend(const orc_geometry* g, const orc_pools* pools, const int32_t* table, int32_t stride,
                         const int32_t* prefix_len, int32_t n_seqs, int32_t chunk_len, const float* q,
                         float softmax_scale, const float* gate, float* out, int32_t bf16_operands);

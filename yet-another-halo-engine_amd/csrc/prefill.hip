@@ -44,6 +44,9 @@ struct PrefillArgs {
   int32_t out_dtype;
 };
 
+__device__ __forceinline__ b8v OnesBf16() {  // 1.0 in all eight slots
+  return __builtin_bit_cast(b8v, uint4{0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u});
+}
 __device__ __forceinline__ uint32_t PackBf16(float a, float b) {  // round to nearest even
   typedef __bf16 b2v __attribute__((ext_vector_type(2)));
   const b2v v = {static_cast<__bf16>(a), static_cast<__bf16>(b)};
@@ -80,19 +83,18 @@ __device__ __forceinline__ void Decode16V(const uint4 c, const uint4 s0, const u
   *lo = uint4{o[0], o[1], o[2], o[3]}, *hi = uint4{o[4], o[5], o[6], o[7]};
 }
 
-// out = o / l (* sigmoid(gate)); lane (query, lane group jg) holds dims 16 dt + 4 jg + r of its query in each row block
+// out = o / l (* sigmoid(gate)); lane (query, lane group jg) holds dims 16 dt + 4 jg + r of its query in each row block.
+// The denominators l are the sums of the bf16 numerators, accumulated by the matrix unit against an all-ones operand
+// next to V^T: numerators and denominator then carry the same rounding, and a lone key returns its V row exactly.
 template <int D>
 __device__ __forceinline__ void StoreRows(const PrefillArgs& a, int s, int h, int G, int jg, const f4v (&o)[RB][D / 16],
-                                          const float (&lsum)[RB], const int (&qpos)[RB], const int (&head)[RB]) {
+                                          const f4v (&lacc)[RB], const int (&qpos)[RB], const int (&head)[RB]) {
   constexpr int NDT = D / 16;
   const Geom& g = a.g;
 #pragma unroll
   for (int i = 0; i < RB; ++i) {
-    float l = lsum[i];
-    l += __shfl_xor(l, 16, 64);
-    l += __shfl_xor(l, 32, 64);
     if (head[i] >= G || qpos[i] >= a.chunk_len) continue;
-    const float inv = 1.0f / l;
+    const float inv = 1.0f / lacc[i][0];  // every row of the all-ones product holds the query's denominator
     const size_t base = ((size_t(s) * a.chunk_len + qpos[i]) * g.n_q + size_t(h) * G + head[i]) * D;
 #pragma unroll
     for (int dt = 0; dt < NDT; ++dt) {
@@ -158,10 +160,11 @@ __global__ __launch_bounds__(256) void PrefillAttendQ8(const PrefillArgs a) {
     for (int ks = 0; ks < KS; ++ks) qb[i][ks] = *reinterpret_cast<const b8v*>(qp + 32 * ks + 8 * jg);
   }
   f4v o[RB][NDT];
-  float m[RB], lsum[RB];
+  float m[RB];
+  f4v lacc[RB];
 #pragma unroll
   for (int i = 0; i < RB; ++i) {
-    m[i] = kNegBig, lsum[i] = 0.0f;
+    m[i] = kNegBig, lacc[i] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
     for (int dt = 0; dt < NDT; ++dt) o[i][dt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
   }
@@ -293,21 +296,23 @@ __global__ __launch_bounds__(256) void PrefillAttendQ8(const PrefillArgs a) {
         }
       mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
       mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const float mn = fmaxf(m[i], mx);
+      // The running maximum moves in whole powers of two: rescaling is then exact, so the result does not depend on
+      // the order in which the maximum was met (and it moves less often).
+      const float mn = fmaxf(m[i], __builtin_ceilf(mx));
       const float alpha = __builtin_amdgcn_exp2f(m[i] - mn);
       m[i] = mn;
-      float psum = 0.0f;
 #pragma unroll
       for (int kt = 0; kt < 4; ++kt) {
         float p[4];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) p[r] = __builtin_amdgcn_exp2f(st[i][kt][r] - mn), psum += p[r];
+        for (int r = 0; r < 4; ++r) p[r] = __builtin_amdgcn_exp2f(st[i][kt][r] - mn);
         // step kt / 2 takes keys 32 (kt / 2) + {4 jg + r} from its even tile and + 16 + {4 jg + r} from its odd one
         pb[i][kt / 2][2 * (kt % 2)] = PackBf16(p[0], p[1]);
         pb[i][kt / 2][2 * (kt % 2) + 1] = PackBf16(p[2], p[3]);
       }
-      lsum[i] = __builtin_fmaf(lsum[i], alpha, psum);
       if (alpha != 1.0f) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) lacc[i][r] *= alpha;
 #pragma unroll
         for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
@@ -331,6 +336,11 @@ __global__ __launch_bounds__(256) void PrefillAttendQ8(const PrefillArgs a) {
       b8v va[3][2];  // read two 16-dim tiles ahead
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2) va[0][s2] = read_v(0, s2), va[1][s2] = read_v(1, s2);
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+        for (int i = 0; i < RB; ++i)
+          lacc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(OnesBf16(), pv[i][s2], lacc[i], 0, 0, 0);
 #pragma unroll
       for (int dt = 0; dt < NDT; ++dt) {
         if (dt + 2 < NDT) {
@@ -359,7 +369,7 @@ __global__ __launch_bounds__(256) void PrefillAttendQ8(const PrefillArgs a) {
     __syncthreads();  // every wave is done with lv; K(tile + 1) and its V scales are in place
   }
 
-  StoreRows<D>(a, s, h, G, jg, o, lsum, qpos, head);
+  StoreRows<D>(a, s, h, G, jg, o, lacc, qpos, head);
 }
 
 
@@ -481,14 +491,19 @@ __device__ __forceinline__ float MaxOverLaneGroups(float v) {
   return fmaxf(__builtin_bit_cast(float, q0), __builtin_bit_cast(float, q1));
 }
 
+// s_waitcnt operand: at most n vector memory operations outstanding, the other counters unconstrained
+constexpr int VmCnt(int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); }
+
 // Same work split as the fused kernel: 4 waves, 64 chunk positions x 2 heads, two row blocks of 16 queries per wave,
-// everything transposed (keys along MFMA rows, queries along lanes). LDS holds two tile images; the copy of tile
-// i + 1 is issued before the arithmetic of tile i and waited for after it: one barrier per tile.
+// everything transposed (keys along MFMA rows, queries along lanes). LDS holds two tile images; the copy of image
+// i + 1 is spread over the two products of tile i and waited for after them: one barrier per tile. (Waiting for the
+// V half only before the second product of tile i + 1, with a second barrier there, measured slower.)
 template <int D>
 __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, const char* img, int tiles_per_pair) {
   constexpr int KS = D / 32, NDT = D / 16;
   constexpr int KIMG = kKeys * D * 2, TIMG = TileImageBytes<D>();
   constexpr int kCopies = TIMG / 1024 / 4;  // 1 KB wave-wide copies per wave and tile
+  static_assert(kCopies == KS + NDT / 2, "one copy per step of the first product and per two of the second");
   const Geom g = a.g;
   const int G = g.group(), H = g.n_kv;
   const int n_qt = (a.chunk_len + kQueries - 1) / kQueries, n_hp = (G + kHeadsPerGroup - 1) / kHeadsPerGroup;
@@ -518,34 +533,34 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
     for (int ks = 0; ks < KS; ++ks) qb[i][ks] = *reinterpret_cast<const b8v*>(qp + 32 * ks + 8 * jg);
   }
   f4v o[RB][NDT];
-  float m[RB], lsum[RB];
+  float m[RB];
+  f4v lacc[RB];
 #pragma unroll
   for (int i = 0; i < RB; ++i) {
-    m[i] = kNegBig, lsum[i] = 0.0f;
+    m[i] = kNegBig, lacc[i] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
     for (int dt = 0; dt < NDT; ++dt) o[i][dt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
   }
   const float sscale = a.scale * 1.4426950408889634f;
   const char* src = img + size_t(pair) * tiles_per_pair * TIMG + size_t(lane) * 16;
-  auto copy_tile = [&](int tile) {
-    const char* from = src + size_t(tile) * TIMG;
-    char* to = lds[tile % 2];
-#pragma unroll
-    for (int j = 0; j < kCopies; ++j) {
-      const int c = wave + 4 * j;
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(from + c * 1024),
-                                       (__attribute__((address_space(3))) void*)(to + c * 1024), 16, 0, 0);
-    }
+  // copy j (of kCopies) of this wave's share of a tile image; the copies of tile i + 1 are spread over the two
+  // products of tile i, because the CU's vector memory path takes 16 cycles per KB and a burst of them stalls
+  // every wave
+  auto copy_part = [&](int tile, int j) {
+    const int c = wave + 4 * j;
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + size_t(tile) * TIMG + c * 1024),
+                                     (__attribute__((address_space(3))) void*)(lds[tile % 2] + c * 1024), 16, 0, 0);
   };
   // byte offsets of this lane's operand reads within an image; the XOR with qn % 8 undoes the images' swizzle
   const int sw = qn % 8;
   const int koff = qn * (2 * D), voff = KIMG + qn * 128;
 
-  copy_tile(0);
-  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+#pragma unroll
+  for (int j = 0; j < kCopies; ++j) copy_part(0, j);
+  __builtin_amdgcn_s_waitcnt(VmCnt(0));
   __syncthreads();
   for (int tile = 0; tile < n_tiles; ++tile) {
-    if (tile + 1 < n_tiles) copy_tile(tile + 1);
+    const bool more = tile + 1 < n_tiles;
     const char* buf = lds[tile % 2];
     // ---- S^T = K Q^T
     f4v st[RB][4];
@@ -557,7 +572,7 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
       auto read_k = [&](int ks, int kt) -> b8v {
         return *reinterpret_cast<const b8v*>(buf + koff + kt * 16 * (2 * D) + 16 * ((4 * ks + jg) ^ sw));
       };
-      b8v ka[2][4];
+      b8v ka[2][4];  // operands are read one step ahead of their use
 #pragma unroll
       for (int kt = 0; kt < 4; ++kt) ka[0][kt] = read_k(0, kt);
 #pragma unroll
@@ -571,11 +586,14 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
 #pragma unroll
           for (int i = 0; i < RB; ++i)
             st[i][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[ks % 2][kt], qb[i][ks], st[i][kt], 0, 0, 0);
+        if (more) copy_part(tile + 1, ks);
         __builtin_amdgcn_sched_barrier(0);
       }
     }
-    // ---- online softmax per query (= per lane). The accumulators are rescaled only in tiles where some query of the
-    // wave meets a new maximum, which becomes rare as the context grows.
+    // ---- online softmax per query (= per lane). The reference point m of the numerators 2^(score - m) is a whole
+    // power of two and is only moved when a score exceeds it by more than 2^16: moving it rescales numerators, sums
+    // and accumulators by a power of two, which is exact, so moving it late changes nothing in the result, while
+    // bf16 numerators and f32 sums have room for the factor 2^16. Rescaling is then rare (the first tile, mostly).
     const bool diag = (tile + 1) * kKeys > prefix + q0 + 1;
     uint32_t pb[RB][2][4];
 #pragma unroll
@@ -592,27 +610,38 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
       for (int kt = 1; kt < 4; ++kt)
         mx = fmaxf(mx, fmaxf(fmaxf(st[i][kt][0], st[i][kt][1]), fmaxf(st[i][kt][2], st[i][kt][3])));
       mx = MaxOverLaneGroups(mx) * sscale;  // sscale > 0 is required by the entry point
-      if (__builtin_amdgcn_ballot_w64(mx > m[i]) != 0) {
-        const float mn = fmaxf(mx, m[i]);
+      if (__builtin_expect(__builtin_amdgcn_ballot_w64(mx > m[i] + 16.0f) != 0, 0)) {
+        const b8v zero = {0, 0, 0, 0, 0, 0, 0, 0};
+        const float mn = mx > m[i] + 16.0f ? __builtin_ceilf(mx) : m[i];
         const float alpha = __builtin_amdgcn_exp2f(m[i] - mn);
         m[i] = mn;
-        lsum[i] *= alpha;
+        {
+          f4v t = lacc[i];
+          asm volatile("" : "+a"(t));
 #pragma unroll
-        for (int dt = 0; dt < NDT; ++dt)
+          for (int r = 0; r < 4; ++r) t[r] *= alpha;
+          lacc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(zero, zero, t, 0, 0, 0);
+        }
+        // The rescaled accumulators go back through a matrix instruction with zero factors: that keeps them in
+        // the accumulation registers on this path as on the common one (otherwise the compiler moves all of them to
+        // ordinary registers and back in every tile, rescaled or not).
 #pragma unroll
-          for (int r = 0; r < 4; ++r) o[i][dt][r] *= alpha;
+        for (int dt = 0; dt < NDT; ++dt) {
+          f4v t = o[i][dt];
+          asm volatile("" : "+a"(t));  // the copy out of the accumulation registers stays on this path
+#pragma unroll
+          for (int r = 0; r < 4; ++r) t[r] *= alpha;
+          o[i][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(zero, zero, t, 0, 0, 0);
+        }
       }
-      float psum = 0.0f;
 #pragma unroll
       for (int kt = 0; kt < 4; ++kt) {
         float p[4];
 #pragma unroll
-        for (int r = 0; r < 4; ++r)
-          p[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(st[i][kt][r], sscale, -m[i])), psum += p[r];
+        for (int r = 0; r < 4; ++r) p[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(st[i][kt][r], sscale, -m[i]));
         pb[i][kt / 2][2 * (kt % 2)] = PackBf16(p[0], p[1]);
         pb[i][kt / 2][2 * (kt % 2) + 1] = PackBf16(p[2], p[3]);
       }
-      lsum[i] += psum;
     }
     // ---- O^T += V^T P^T
     {
@@ -625,9 +654,14 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2)
           pv[i][s2] = __builtin_bit_cast(b8v, uint4{pb[i][s2][0], pb[i][s2][1], pb[i][s2][2], pb[i][s2][3]});
-      b8v va[3][2];
+      b8v va[3][2];  // read two 16-dim tiles ahead
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2) va[0][s2] = read_v(0, s2), va[1][s2] = read_v(1, s2);
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+        for (int i = 0; i < RB; ++i)
+          lacc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(OnesBf16(), pv[i][s2], lacc[i], 0, 0, 0);
 #pragma unroll
       for (int dt = 0; dt < NDT; ++dt) {
         if (dt + 2 < NDT) {
@@ -639,13 +673,16 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
 #pragma unroll
           for (int i = 0; i < RB; ++i)
             o[i][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[dt % 3][s2], pv[i][s2], o[i][dt], 0, 0, 0);
-        if (dt % 2 == 1) __builtin_amdgcn_sched_barrier(0);
+        if (dt % 2 == 1) {
+          if (more) copy_part(tile + 1, KS + dt / 2);
+          __builtin_amdgcn_sched_barrier(0);
+        }
       }
     }
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's part of the next image has landed
-    __syncthreads();                     // ... and everybody's; everybody is done with this tile's image
+    __builtin_amdgcn_s_waitcnt(VmCnt(0));  // this wave's part of the next image has landed
+    __syncthreads();                       // ... and everybody's; everybody is done with this tile's image
   }
-  StoreRows<D>(a, s, h, G, jg, o, lsum, qpos, head);
+  StoreRows<D>(a, s, h, G, jg, o, lacc, qpos, head);
 }
 
 }  // namespace
