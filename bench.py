@@ -26,7 +26,10 @@ WORKLOADS = {
     "ragged_b64_q8_0": dict(fmt=8, batch=64, lo=1024, hi=65536, seed=4),
     "b1_ctx32k_q8_0": dict(fmt=8, batch=1, lo=32768, hi=32768, seed=4),
     "b16_ctx128k_q4_0": dict(fmt=4, batch=16, lo=131072, hi=131072, seed=4, outliers=8),
+    # chunked prefill: every sequence holds `lo` tokens and takes a chunk of `chunk` more per step
+    "prefill_b8_ctx16k_chunk2k_q8_0": dict(fmt=8, batch=8, lo=16384, hi=16384, seed=4, chunk=2048),
 }
+MFMA_BF16_PEAK_TFLOPS = 2500.0
 NQ, NKV, HD, PT = 24, 4, 256, 64
 # HBM bytes per launch of the split-K kernel from rocprofv3 counters (FETCH_SIZE + WRITE_SIZE, each scaled by what the
 # counter reads for a plain 1 GiB copy); a measurement made outside this script, recorded with its summary.
@@ -44,6 +47,7 @@ def fnv1a(b):
 def build_state(yahkv, torch, wl, total_steps):
     rng = np.random.default_rng(wl["seed"])
     lens = rng.integers(wl["lo"], wl["hi"] + 1, wl["batch"]).astype(np.int32)
+    total_steps = wl.get("chunk", total_steps)       # prefill: room for one chunk, rewritten by every step
     pages = (lens + total_steps + PT - 1) // PT
     n_pages = int(pages.sum())                       # the pool fits the job exactly
     g = yahkv.geometry(wl["fmt"], NQ, NKV, HD, PT, n_pages)
@@ -141,6 +145,104 @@ def cpu_baseline(wl, lens, scale, budget_tokens=150000):
             "append_note": "oracle scalar block quantizer + page scatter, 1 thread"}
 
 
+def prefill_cpu_baseline(wl, scale, prefix=2048, chunk=64):
+    """The CPU oracle's chunked-prefill attention (f32 operands) on one short sequence, all host cores."""
+    import oracle
+    rng = np.random.default_rng(98)
+    n = prefix + chunk
+    g = oracle.geometry(wl["fmt"], NQ, NKV, HD, PT, (n + PT - 1) // PT)
+    table = rng.permutation(g.n_pages).astype(np.int32)[None]
+    host = oracle.HostPools(g)
+    oracle.append(host, table, [0], None, rng.standard_normal((1, n, NKV, HD), np.float32),
+                  rng.standard_normal((1, n, NKV, HD), np.float32))
+    q = rng.standard_normal((1, chunk, NQ, HD)).astype(np.float32)
+    oracle.prefill_attend(host, table, [prefix], q, scale)
+    times = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        oracle.prefill_attend(host, table, [prefix], q, scale)
+        times.append(time.perf_counter() - t0)
+    t = float(np.median(times))
+    flops = NQ * chunk * (prefix + (chunk + 1) / 2) * HD * 4
+    return {"value": round(flops / t / 1e12, 5), "unit": "TFLOP/s", "cores": oracle.threads(), "kind": "port",
+            "sample": f"oracle prefill attention, 1 sequence, prefix {prefix} + chunk {chunk}, median of 3 after a "
+                      "warm-up", "tok_per_s": round(chunk / t, 1)}
+
+
+def run_prefill(a, wl, torch, yahkv):
+    """A step: quantize + scatter one chunk per sequence, decode prefix + chunk to bf16 tiles, causal attention."""
+    g, pools, lens, table, t_table, gen = build_state(yahkv, torch, wl, 0)
+    B, chunk, prefix = wl["batch"], wl["chunk"], int(lens.max())
+    scale = 1.0 / float(np.sqrt(HD))
+    t_prefix = torch.from_numpy(lens).cuda()
+    q = torch.randn((B, chunk, NQ, HD), generator=gen, device="cuda").to(torch.bfloat16)
+    knew = torch.randn((B, chunk, NKV, HD), generator=gen, device="cuda").to(torch.bfloat16)
+    vnew = torch.randn((B, chunk, NKV, HD), generator=gen, device="cuda").to(torch.bfloat16)
+    out = torch.empty(q.shape, dtype=torch.bfloat16, device="cuda")
+    ws = torch.empty(yahkv.prefill_workspace_bytes(g, B, prefix, chunk), dtype=torch.uint8, device="cuda")
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(a.steps)]
+
+    def step(pair=None):
+        yahkv.append(pools, t_table, t_prefix, knew, vnew)
+        yahkv.prefill_decode_tiles(pools, t_table, t_prefix, prefix, B, chunk, ws)
+        if pair:
+            pair[0].record()
+        yahkv.prefill_attend_tiles(pools, t_table, t_prefix, prefix, q, scale, out, ws)
+        if pair:
+            pair[1].record()
+
+    # parity before timing: float64 closed form on the library's own gathered blocks, a few (query, head) rows;
+    # the bound is what bf16 operands allow against exact arithmetic
+    step()
+    torch.cuda.synchronize()
+    first_hash = fnv1a(out.view(torch.int16).cpu().numpy().tobytes())
+    import oracle
+    n = prefix + chunk
+    k, v = yahkv.gather_blocks(pools, t_table[0], n)
+    Kd = oracle.dequantize_q8_0(k.cpu().numpy().reshape(-1, 34)).reshape(n, NKV, HD).astype(np.float64)
+    Vd = oracle.dequantize_q8_0(v.cpu().numpy().reshape(-1, 34)).reshape(n, NKV, HD).astype(np.float64)
+    err = 0.0
+    for t in (0, chunk // 2, chunk - 1):
+        for h in (0, NQ - 1):
+            sc = Kd[:prefix + t + 1, h // (NQ // NKV)] @ q[0, t, h].float().cpu().numpy().astype(np.float64) * scale
+            p = np.exp(sc - sc.max())
+            want = (p / p.sum()) @ Vd[:prefix + t + 1, h // (NQ // NKV)]
+            got = out[0, t, h].float().cpu().numpy()
+            err = max(err, float(np.abs(got - want).max() / np.abs(want).max()))
+    if not err < 4 * 2.0 ** -9:
+        raise SystemExit(f"bench.py: parity check failed before timing: max relative error {err:.3e}")
+
+    for _ in range(a.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(a.steps):
+        step(ev[i])
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms = dt / a.steps * 1e3
+    kern_ms = float(np.mean([p[0].elapsed_time(p[1]) for p in ev]))
+    flops = float(B) * NQ * chunk * (prefix + (chunk + 1) / 2) * HD * 4   # both products, causal part counted once
+    res = {
+        "metric": "chunked-prefill attention over paged q8 KV, TFLOP/s (bf16 MFMA) + tok/s",
+        "value": round(flops / (ms * 1e-3) / 1e12, 1), "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps,
+        "warmup": a.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": a.workload, "batch": B, "prefix": prefix, "chunk": chunk, "n_q_heads": NQ,
+                   "n_kv_heads": NKV, "head_dim": HD, "page_tokens": PT, "n_pages": g.n_pages, "kv_format": "q8_0",
+                   "step": "append chunk (quantize + scatter) + decode tiles to bf16 + causal attention"},
+        "tok_per_s": round(B * chunk / (ms * 1e-3), 1), "flops_per_step": int(flops),
+        "parity_max_rel_err": float(f"{err:.3e}"), "out_fnv1a": first_hash,
+        "roofline": {"bound": "mfma", "achieved": round(flops / (kern_ms * 1e-3) / 1e12, 1),
+                     "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(flops / (kern_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
+                     "kernel": "PrefillAttendImg<%d>" % HD, "kernel_ms": round(kern_ms, 4)},
+    }
+    if not a.no_cpu_baseline:
+        res["cpu_baseline"] = prefill_cpu_baseline(wl, scale)
+    print(json.dumps(res))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -165,6 +267,8 @@ def main():
         print(json.dumps({"copy_calibration": {"bytes_read": 1 << 30, "bytes_written": 1 << 30, "copies": 5}}))
         return
     wl = WORKLOADS[a.workload]
+    if "chunk" in wl:
+        return run_prefill(a, wl, torch, yahkv)
     total = a.warmup + a.steps + 1
     g, pools, lens, table, t_table, gen = build_state(yahkv, torch, wl, total)
     B = wl["batch"]

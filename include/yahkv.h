@@ -154,6 +154,20 @@ int yahkv_decode_attend(const yahkv_geometry* g, const yahkv_pools* pools, const
  * (q4_0: YAHKV_ERR_WORKSPACE). Both give the same results up to the order of f32 sums. */
 size_t yahkv_prefill_workspace_bytes(const yahkv_geometry* g, int32_t n_seqs, int32_t max_prefix_len,
                                      int32_t chunk_len);
+/* The two dispatches of the workspace path, for callers that queue them separately (as the reference does with
+ * yah_kdeq8 / yah_vdeq8 and yah_attn_wmma, loom_prefill.hpp:3378-3416): decode keys 0 .. prefix_len[s] + chunk_len
+ * of every sequence into bf16 tiles in the workspace; then attention of the chunk's queries over those tiles. The
+ * tiles stay valid for further queries of the same chunk (e.g. another slice of heads) until the pools change. */
+int yahkv_prefill_decode_tiles(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
+                               int32_t page_table_stride, const int32_t* prefix_len, int32_t n_seqs,
+                               int32_t max_prefix_len, int32_t chunk_len, void* workspace, size_t workspace_bytes,
+                               void* stream);
+int yahkv_prefill_attend_tiles(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
+                               int32_t page_table_stride, const int32_t* prefix_len, int32_t n_seqs,
+                               int32_t max_prefix_len, int32_t chunk_len, const void* q, float softmax_scale,
+                               const float* gate, void* out, int32_t out_dtype, const void* workspace,
+                               size_t workspace_bytes, void* stream);
+/* decode_tiles + attend_tiles when workspace is not NULL, else the one-pass kernel. */
 int yahkv_prefill_attend(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
                          int32_t page_table_stride, const int32_t* prefix_len, int32_t n_seqs,
                          int32_t max_prefix_len, int32_t chunk_len, const void* q, float softmax_scale,

@@ -54,6 +54,8 @@ def _load():
     lib.yahkv_prefill_workspace_bytes.argtypes = [G, i32, i32, i32]
     lib.yahkv_prefill_attend.argtypes = [G, P, i32p, i32, i32p, i32, i32, i32, vp, C.c_float, vp, vp, i32, vp,
                                          C.c_size_t, vp]
+    lib.yahkv_prefill_attend_tiles.argtypes = lib.yahkv_prefill_attend.argtypes
+    lib.yahkv_prefill_decode_tiles.argtypes = [G, P, i32p, i32, i32p, i32, i32, i32, vp, C.c_size_t, vp]
     lib.yahkv_gather_blocks.argtypes = [G, P, i32p, i32, vp, vp, vp]
     lib.yahkv_pagepool_create.restype = C.c_void_p
     lib.yahkv_pagepool_create.argtypes = [i32]
@@ -252,6 +254,24 @@ def prefill_attend(pools, table, prefix_len, max_prefix_len, q, scale, gate=None
     _check(lib.yahkv_prefill_attend(C.byref(g), C.byref(st), _dp(table), table.shape[1], _dp(prefix_len), q.shape[0],
                                     max_prefix_len, q.shape[1], _dp(q), scale, _dp(gate), _dp(out), _dtype_code(out),
                                     ws_ptr, ws_bytes, _stream()), "prefill_attend")
+    return out
+
+
+def prefill_decode_tiles(pools, table, prefix_len, max_prefix_len, n_seqs, chunk_len, workspace):
+    """First dispatch of the workspace path of prefill_attend: K / V of prefix + chunk as bf16 tiles in workspace."""
+    g, st = pools.geom, pools.struct()
+    _check(lib.yahkv_prefill_decode_tiles(C.byref(g), C.byref(st), _dp(table), table.shape[1], _dp(prefix_len), n_seqs,
+                                          max_prefix_len, chunk_len, _dp(workspace), workspace.numel(), _stream()),
+           "prefill_decode_tiles")
+
+
+def prefill_attend_tiles(pools, table, prefix_len, max_prefix_len, q, scale, out, workspace, gate=None):
+    """Second dispatch: attention of the chunk's queries over the tiles in workspace."""
+    g, st = pools.geom, pools.struct()
+    _check(lib.yahkv_prefill_attend_tiles(C.byref(g), C.byref(st), _dp(table), table.shape[1], _dp(prefix_len),
+                                          q.shape[0], max_prefix_len, q.shape[1], _dp(q), scale, _dp(gate), _dp(out),
+                                          _dtype_code(out), _dp(workspace), workspace.numel(), _stream()),
+           "prefill_attend_tiles")
     return out
 
 

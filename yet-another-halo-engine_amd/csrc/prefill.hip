@@ -705,51 +705,63 @@ extern "C" size_t yahkv_prefill_workspace_bytes(const yahkv_geometry* g, int32_t
   return ImageBytes(MakeGeom(*g), n_seqs, max_prefix_len, chunk_len);
 }
 
-extern "C" int yahkv_prefill_attend(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
-                                    int32_t page_table_stride, const int32_t* prefix_len, int32_t n_seqs,
-                                    int32_t max_prefix_len, int32_t chunk_len, const void* q, float softmax_scale,
-                                    const float* gate, void* out, int32_t out_dtype, void* workspace,
-                                    size_t workspace_bytes, void* stream) {
+namespace {
+// Checks shared by the prefill entry points and the arguments common to their kernels.
+int PreparePrefill(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
+                   int32_t page_table_stride, const int32_t* prefix_len, int32_t n_seqs, int32_t max_prefix_len,
+                   int32_t chunk_len, PrefillArgs* a) {
   if (const int st = CheckGeometry(g)) return st;
   if (pools == nullptr || pools->kq == nullptr || pools->ks == nullptr || pools->vq == nullptr ||
-      pools->vs == nullptr || page_table == nullptr || prefix_len == nullptr || q == nullptr || out == nullptr)
+      pools->vs == nullptr || page_table == nullptr || prefix_len == nullptr)
     return YAHKV_ERR_ARG;
   if (n_seqs <= 0 || chunk_len <= 0 || max_prefix_len < 0 || page_table_stride <= 0) return YAHKV_ERR_ARG;
-  if (!(softmax_scale > 0.0f)) return YAHKV_ERR_ARG;
-  if (out_dtype != YAHKV_F32 && out_dtype != YAHKV_F16 && out_dtype != YAHKV_BF16) return YAHKV_ERR_ARG;
   if ((reinterpret_cast<uintptr_t>(pools->kq) | reinterpret_cast<uintptr_t>(pools->vq) |
-       reinterpret_cast<uintptr_t>(pools->ks) | reinterpret_cast<uintptr_t>(pools->vs) |
-       reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(workspace)) & 15)
+       reinterpret_cast<uintptr_t>(pools->ks) | reinterpret_cast<uintptr_t>(pools->vs)) & 15)
     return YAHKV_ERR_ARG;
   const Geom m = MakeGeom(*g);
   if (int64_t(page_table_stride) * m.pt < chunk_len) return YAHKV_ERR_ARG;
-  PrefillArgs a{};
-  a.g = m, a.pools = MakePools(*pools), a.table = page_table, a.stride = page_table_stride, a.prefix_len = prefix_len;
-  a.n_seqs = n_seqs, a.max_prefix = max_prefix_len, a.chunk_len = chunk_len;
-  a.q = static_cast<const uint16_t*>(q), a.scale = softmax_scale, a.gate = gate, a.out = out, a.out_dtype = out_dtype;
-  const int n_qt = (chunk_len + kQueries - 1) / kQueries;
-  const int n_hp = (m.group() + kHeadsPerGroup - 1) / kHeadsPerGroup;
-  const int pairs = n_seqs * m.n_kv, pair_slots = (pairs + 7) / 8 * 8;
-  const dim3 grid(static_cast<unsigned>(pair_slots) * n_qt * n_hp);
-  hipStream_t st = static_cast<hipStream_t>(stream);
-  if (workspace == nullptr) {  // one pass: tiles are decoded inside the attention kernel
-    if (m.format != 8) return YAHKV_ERR_WORKSPACE;  // q4_0 pools are only served through the images
-#define YAHKV_LAUNCH_PF(DD, PP) hipLaunchKernelGGL((PrefillAttendQ8<DD, PP>), grid, dim3(256), 0, st, a)
-    if (m.hd == 256 && m.pt == 64) YAHKV_LAUNCH_PF(256, 64);
-    else if (m.hd == 256 && m.pt == 32) YAHKV_LAUNCH_PF(256, 32);
-    else if (m.hd == 256) YAHKV_LAUNCH_PF(256, 16);
-    else if (m.pt == 64) YAHKV_LAUNCH_PF(128, 64);
-    else if (m.pt == 32) YAHKV_LAUNCH_PF(128, 32);
-    else YAHKV_LAUNCH_PF(128, 16);
-#undef YAHKV_LAUNCH_PF
-    return LaunchStatus();
-  }
-  if (workspace_bytes < ImageBytes(m, n_seqs, max_prefix_len, chunk_len)) return YAHKV_ERR_WORKSPACE;
+  *a = PrefillArgs{};
+  a->g = m, a->pools = MakePools(*pools), a->table = page_table, a->stride = page_table_stride;
+  a->prefix_len = prefix_len, a->n_seqs = n_seqs, a->max_prefix = max_prefix_len, a->chunk_len = chunk_len;
+  return YAHKV_OK;
+}
+int PrepareQueries(const void* q, float softmax_scale, const float* gate, void* out, int32_t out_dtype,
+                   PrefillArgs* a) {
+  if (q == nullptr || out == nullptr || !(softmax_scale > 0.0f)) return YAHKV_ERR_ARG;
+  if (out_dtype != YAHKV_F32 && out_dtype != YAHKV_F16 && out_dtype != YAHKV_BF16) return YAHKV_ERR_ARG;
+  if ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(out)) & 15) return YAHKV_ERR_ARG;
+  a->q = static_cast<const uint16_t*>(q), a->scale = softmax_scale, a->gate = gate, a->out = out;
+  a->out_dtype = out_dtype;
+  return YAHKV_OK;
+}
+int CheckWorkspace(const PrefillArgs& a, const void* workspace, size_t workspace_bytes) {
+  if (workspace == nullptr || (reinterpret_cast<uintptr_t>(workspace) & 15)) return YAHKV_ERR_ARG;
+  return workspace_bytes < ImageBytes(a.g, a.n_seqs, a.max_prefix, a.chunk_len) ? YAHKV_ERR_WORKSPACE : YAHKV_OK;
+}
+dim3 AttendGrid(const PrefillArgs& a) {
+  const int n_qt = (a.chunk_len + kQueries - 1) / kQueries;
+  const int n_hp = (a.g.group() + kHeadsPerGroup - 1) / kHeadsPerGroup;
+  const int pair_slots = (a.n_seqs * a.g.n_kv + 7) / 8 * 8;
+  return dim3(static_cast<unsigned>(pair_slots) * n_qt * n_hp);
+}
+}  // namespace
+
+extern "C" int yahkv_prefill_decode_tiles(const yahkv_geometry* g, const yahkv_pools* pools,
+                                          const int32_t* page_table, int32_t page_table_stride,
+                                          const int32_t* prefix_len, int32_t n_seqs, int32_t max_prefix_len,
+                                          int32_t chunk_len, void* workspace, size_t workspace_bytes, void* stream) {
+  PrefillArgs a;
+  if (const int rc = PreparePrefill(g, pools, page_table, page_table_stride, prefix_len, n_seqs, max_prefix_len,
+                                    chunk_len, &a))
+    return rc;
+  if (const int rc = CheckWorkspace(a, workspace, workspace_bytes)) return rc;
+  const Geom& m = a.g;
   ImageArgs ia{};
   ia.g = m, ia.pools = a.pools, ia.table = page_table, ia.stride = page_table_stride, ia.prefix_len = prefix_len;
   ia.n_seqs = n_seqs, ia.max_prefix = max_prefix_len, ia.chunk_len = chunk_len;
   ia.img = static_cast<char*>(workspace), ia.tiles_per_pair = TilesPerPair(max_prefix_len, chunk_len);
-  const dim3 igrid(static_cast<unsigned>(ia.tiles_per_pair), static_cast<unsigned>(pairs));
+  const dim3 igrid(static_cast<unsigned>(ia.tiles_per_pair), static_cast<unsigned>(n_seqs * m.n_kv));
+  hipStream_t st = static_cast<hipStream_t>(stream);
 #define YAHKV_LAUNCH_IMG(FF, DD, PP) hipLaunchKernelGGL((PrefillImages<FF, DD, PP>), igrid, dim3(256), 0, st, ia)
 #define YAHKV_LAUNCH_IMG_FMT(FF)                                     \
   if (m.hd == 256 && m.pt == 64) YAHKV_LAUNCH_IMG(FF, 256, 64);         \
@@ -765,9 +777,59 @@ extern "C" int yahkv_prefill_attend(const yahkv_geometry* g, const yahkv_pools* 
   }
 #undef YAHKV_LAUNCH_IMG_FMT
 #undef YAHKV_LAUNCH_IMG
-  if (const int rc = LaunchStatus()) return rc;
+  return LaunchStatus();
+}
+
+extern "C" int yahkv_prefill_attend_tiles(const yahkv_geometry* g, const yahkv_pools* pools,
+                                          const int32_t* page_table, int32_t page_table_stride,
+                                          const int32_t* prefix_len, int32_t n_seqs, int32_t max_prefix_len,
+                                          int32_t chunk_len, const void* q, float softmax_scale, const float* gate,
+                                          void* out, int32_t out_dtype, const void* workspace, size_t workspace_bytes,
+                                          void* stream) {
+  PrefillArgs a;
+  if (const int rc = PreparePrefill(g, pools, page_table, page_table_stride, prefix_len, n_seqs, max_prefix_len,
+                                    chunk_len, &a))
+    return rc;
+  if (const int rc = PrepareQueries(q, softmax_scale, gate, out, out_dtype, &a)) return rc;
+  if (const int rc = CheckWorkspace(a, workspace, workspace_bytes)) return rc;
   const char* img = static_cast<const char*>(workspace);
-  if (m.hd == 256) hipLaunchKernelGGL((PrefillAttendImg<256>), grid, dim3(256), 0, st, a, img, ia.tiles_per_pair);
-  else hipLaunchKernelGGL((PrefillAttendImg<128>), grid, dim3(256), 0, st, a, img, ia.tiles_per_pair);
+  const int tiles = TilesPerPair(max_prefix_len, chunk_len);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (a.g.hd == 256) hipLaunchKernelGGL((PrefillAttendImg<256>), AttendGrid(a), dim3(256), 0, st, a, img, tiles);
+  else hipLaunchKernelGGL((PrefillAttendImg<128>), AttendGrid(a), dim3(256), 0, st, a, img, tiles);
+  return LaunchStatus();
+}
+
+extern "C" int yahkv_prefill_attend(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
+                                    int32_t page_table_stride, const int32_t* prefix_len, int32_t n_seqs,
+                                    int32_t max_prefix_len, int32_t chunk_len, const void* q, float softmax_scale,
+                                    const float* gate, void* out, int32_t out_dtype, void* workspace,
+                                    size_t workspace_bytes, void* stream) {
+  if (workspace != nullptr) {
+    if (const int rc = yahkv_prefill_decode_tiles(g, pools, page_table, page_table_stride, prefix_len, n_seqs,
+                                                  max_prefix_len, chunk_len, workspace, workspace_bytes, stream))
+      return rc;
+    return yahkv_prefill_attend_tiles(g, pools, page_table, page_table_stride, prefix_len, n_seqs, max_prefix_len,
+                                      chunk_len, q, softmax_scale, gate, out, out_dtype, workspace, workspace_bytes,
+                                      stream);
+  }
+  // one pass: tiles are decoded inside the attention kernel
+  PrefillArgs a;
+  if (const int rc = PreparePrefill(g, pools, page_table, page_table_stride, prefix_len, n_seqs, max_prefix_len,
+                                    chunk_len, &a))
+    return rc;
+  if (const int rc = PrepareQueries(q, softmax_scale, gate, out, out_dtype, &a)) return rc;
+  const Geom& m = a.g;
+  if (m.format != 8) return YAHKV_ERR_WORKSPACE;  // q4_0 pools are only served through the tile images
+  const dim3 grid = AttendGrid(a);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+#define YAHKV_LAUNCH_PF(DD, PP) hipLaunchKernelGGL((PrefillAttendQ8<DD, PP>), grid, dim3(256), 0, st, a)
+  if (m.hd == 256 && m.pt == 64) YAHKV_LAUNCH_PF(256, 64);
+  else if (m.hd == 256 && m.pt == 32) YAHKV_LAUNCH_PF(256, 32);
+  else if (m.hd == 256) YAHKV_LAUNCH_PF(256, 16);
+  else if (m.pt == 64) YAHKV_LAUNCH_PF(128, 64);
+  else if (m.pt == 32) YAHKV_LAUNCH_PF(128, 32);
+  else YAHKV_LAUNCH_PF(128, 16);
+#undef YAHKV_LAUNCH_PF
   return LaunchStatus();
 }
