@@ -43,6 +43,8 @@ def build(yahkv, torch, fmt, n_q, n_kv, hd, pt, prefix, chunk, seed, fill=0):
     ("images", 8, 8, 2, 128, 16, [37, 0, 64], 21),
     ("images", 8, 6, 2, 256, 32, [31, 500], 64),
     ("images", 8, 10, 2, 128, 64, [129], 130),
+    ("images", 8, 12, 4, 128, 64, [70, 300], 100),
+    ("images", 8, 6, 1, 128, 32, [1], 65),
     ("images", 4, 24, 4, 256, 64, [100, 0, 64 * 3 + 5], 70),
     ("images", 4, 8, 2, 128, 16, [37, 0, 64], 21),
     ("images", 4, 6, 2, 256, 32, [31, 500], 64),

@@ -23,8 +23,7 @@ namespace {
 
 constexpr int kKeys = 64;    // keys per tile
 constexpr int kQueries = 64; // chunk positions per workgroup
-constexpr int kHeadsPerGroup = 2;  // query heads per workgroup
-constexpr int RB = 2;        // row blocks (16 queries of one head) per wave
+constexpr int kFusedRowBlocks = 2;  // row blocks (16 queries of one head) per wave of the one-pass kernel
 constexpr float kNegBig = -3.4028234663852886e+38f;
 
 typedef __bf16 b8v __attribute__((ext_vector_type(8)));
@@ -86,7 +85,7 @@ __device__ __forceinline__ void Decode16V(const uint4 c, const uint4 s0, const u
 // out = o / l (* sigmoid(gate)); lane (query, lane group jg) holds dims 16 dt + 4 jg + r of its query in each row block.
 // The denominators l are the sums of the bf16 numerators, accumulated by the matrix unit against an all-ones operand
 // next to V^T: numerators and denominator then carry the same rounding, and a lone key returns its V row exactly.
-template <int D>
+template <int D, int RB>
 __device__ __forceinline__ void StoreRows(const PrefillArgs& a, int s, int h, int G, int jg, const f4v (&o)[RB][D / 16],
                                           const f4v (&lacc)[RB], const int (&qpos)[RB], const int (&head)[RB]) {
   constexpr int NDT = D / 16;
@@ -123,6 +122,7 @@ __device__ __forceinline__ void StoreRows(const PrefillArgs& a, int s, int h, in
 template <int D, int PT>
 __global__ __launch_bounds__(256) void PrefillAttendQ8(const PrefillArgs a) {
   constexpr int NB = D / 32, NDT = D / 16, KS = D / 32;  // blocks, 16-dim tiles, 32-dim steps of the first product
+  constexpr int RB = kFusedRowBlocks, kHeadsPerGroup = RB;  // 4 waves x RB row blocks = 64 positions x RB heads
   constexpr int KSTR = D + 8, VSTR = kKeys + 8;          // LDS row strides (bf16), padded against bank conflicts
   constexpr int KCH = kKeys * D / 16 / 256;              // 16-code chunks of a tile per thread
   const Geom g = a.g;
@@ -369,7 +369,7 @@ __global__ __launch_bounds__(256) void PrefillAttendQ8(const PrefillArgs a) {
     __syncthreads();  // every wave is done with lv; K(tile + 1) and its V scales are in place
   }
 
-  StoreRows<D>(a, s, h, G, jg, o, lacc, qpos, head);
+  StoreRows<D, RB>(a, s, h, G, jg, o, lacc, qpos, head);
 }
 
 
@@ -498,9 +498,9 @@ constexpr int VmCnt(int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); }
 // everything transposed (keys along MFMA rows, queries along lanes). LDS holds two tile images; the copy of image
 // i + 1 is spread over the two products of tile i and waited for after them: one barrier per tile. (Waiting for the
 // V half only before the second product of tile i + 1, with a second barrier there, measured slower.)
-template <int D>
+template <int D, int RB>
 __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, const char* img, int tiles_per_pair) {
-  constexpr int KS = D / 32, NDT = D / 16;
+  constexpr int KS = D / 32, NDT = D / 16, kHeadsPerGroup = RB;
   constexpr int KIMG = kKeys * D * 2, TIMG = TileImageBytes<D>();
   constexpr int kCopies = TIMG / 1024 / 4;  // 1 KB wave-wide copies per wave and tile
   static_assert(kCopies == KS + NDT / 2, "one copy per step of the first product and per two of the second");
@@ -682,7 +682,7 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
     __builtin_amdgcn_s_waitcnt(VmCnt(0));  // this wave's part of the next image has landed
     __syncthreads();                       // ... and everybody's; everybody is done with this tile's image
   }
-  StoreRows<D>(a, s, h, G, jg, o, lacc, qpos, head);
+  StoreRows<D, RB>(a, s, h, G, jg, o, lacc, qpos, head);
 }
 
 }  // namespace
@@ -738,9 +738,10 @@ int CheckWorkspace(const PrefillArgs& a, const void* workspace, size_t workspace
   if (workspace == nullptr || (reinterpret_cast<uintptr_t>(workspace) & 15)) return YAHKV_ERR_ARG;
   return workspace_bytes < ImageBytes(a.g, a.n_seqs, a.max_prefix, a.chunk_len) ? YAHKV_ERR_WORKSPACE : YAHKV_OK;
 }
-dim3 AttendGrid(const PrefillArgs& a) {
+// A workgroup serves 64 chunk positions of `heads_per_group` query heads of one kv head.
+dim3 AttendGrid(const PrefillArgs& a, int heads_per_group) {
   const int n_qt = (a.chunk_len + kQueries - 1) / kQueries;
-  const int n_hp = (a.g.group() + kHeadsPerGroup - 1) / kHeadsPerGroup;
+  const int n_hp = (a.g.group() + heads_per_group - 1) / heads_per_group;
   const int pair_slots = (a.n_seqs * a.g.n_kv + 7) / 8 * 8;
   return dim3(static_cast<unsigned>(pair_slots) * n_qt * n_hp);
 }
@@ -795,8 +796,15 @@ extern "C" int yahkv_prefill_attend_tiles(const yahkv_geometry* g, const yahkv_p
   const char* img = static_cast<const char*>(workspace);
   const int tiles = TilesPerPair(max_prefix_len, chunk_len);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (a.g.hd == 256) hipLaunchKernelGGL((PrefillAttendImg<256>), AttendGrid(a), dim3(256), 0, st, a, img, tiles);
-  else hipLaunchKernelGGL((PrefillAttendImg<128>), AttendGrid(a), dim3(256), 0, st, a, img, tiles);
+  // At head_dim 128, three row blocks per wave (three heads per workgroup) when the GQA group is a multiple of
+  // three: each tile image copied to LDS and each operand read from it then serves half as much arithmetic again.
+  // (At head_dim 256 three blocks' accumulators and query operands do not fit the register file: 140 spills.)
+#define YAHKV_LAUNCH_ATT(DD, RR) \
+  hipLaunchKernelGGL((PrefillAttendImg<DD, RR>), AttendGrid(a, RR), dim3(256), 0, st, a, img, tiles)
+  if (a.g.hd == 256) YAHKV_LAUNCH_ATT(256, 2);
+  else if (a.g.group() % 3 == 0) YAHKV_LAUNCH_ATT(128, 3);
+  else YAHKV_LAUNCH_ATT(128, 2);
+#undef YAHKV_LAUNCH_ATT
   return LaunchStatus();
 }
 
@@ -821,7 +829,7 @@ extern "C" int yahkv_prefill_attend(const yahkv_geometry* g, const yahkv_pools* 
   if (const int rc = PrepareQueries(q, softmax_scale, gate, out, out_dtype, &a)) return rc;
   const Geom& m = a.g;
   if (m.format != 8) return YAHKV_ERR_WORKSPACE;  // q4_0 pools are only served through the tile images
-  const dim3 grid = AttendGrid(a);
+  const dim3 grid = AttendGrid(a, kFusedRowBlocks);
   hipStream_t st = static_cast<hipStream_t>(stream);
 #define YAHKV_LAUNCH_PF(DD, PP) hipLaunchKernelGGL((PrefillAttendQ8<DD, PP>), grid, dim3(256), 0, st, a)
   if (m.hd == 256 && m.pt == 64) YAHKV_LAUNCH_PF(256, 64);
