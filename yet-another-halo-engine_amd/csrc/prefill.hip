@@ -494,10 +494,8 @@ __device__ __forceinline__ float MaxOverLaneGroups(float v) {
 // s_waitcnt operand: at most n vector memory operations outstanding, the other counters unconstrained
 constexpr int VmCnt(int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); }
 
-// Same work split as the fused kernel: 4 waves, 64 chunk positions x 2 heads, two row blocks of 16 queries per wave,
-// everything transposed (keys along MFMA rows, queries along lanes). LDS holds two tile images; the copy of image
-// i + 1 is spread over the two products of tile i and waited for after them: one barrier per tile. (Waiting for the
-// V half only before the second product of tile i + 1, with a second barrier there, measured slower.)
+// Same work split as the fused kernel: 4 waves, 64 chunk positions x RB heads, RB row blocks of 16 queries per wave,
+// everything transposed (keys along MFMA rows, queries along lanes). LDS holds two tile images.
 template <int D, int RB>
 __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, const char* img, int tiles_per_pair) {
   constexpr int KS = D / 32, NDT = D / 16, kHeadsPerGroup = RB;
@@ -543,9 +541,10 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
   }
   const float sscale = a.scale * 1.4426950408889634f;
   const char* src = img + size_t(pair) * tiles_per_pair * TIMG + size_t(lane) * 16;
-  // copy j (of kCopies) of this wave's share of a tile image; the copies of tile i + 1 are spread over the two
-  // products of tile i, because the CU's vector memory path takes 16 cycles per KB and a burst of them stalls
-  // every wave
+  // Copy j (of kCopies) of this wave's share of a tile image into the LDS buffer tile % 2: pieces j < kCopies / 2 are
+  // the K half, the others the V half. Direct global-to-LDS loads: no registers, no vector instructions. The copies
+  // are spread over the arithmetic, because the CU's vector memory path moves about 39 bytes per cycle (measured:
+  // 26 cycles per 1 KB wave-wide load, 1700 cycles per 64 KB image) and a burst of them stalls every wave.
   auto copy_part = [&](int tile, int j) {
     const int c = wave + 4 * j;
     __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + size_t(tile) * TIMG + c * 1024),
@@ -554,133 +553,218 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
   // byte offsets of this lane's operand reads within an image; the XOR with qn % 8 undoes the images' swizzle
   const int sw = qn % 8;
   const int koff = qn * (2 * D), voff = KIMG + qn * 128;
-
+  auto read_k = [&](const char* buf, int ks, int kt) -> b8v {
+    return *reinterpret_cast<const b8v*>(buf + koff + kt * 16 * (2 * D) + 16 * ((4 * ks + jg) ^ sw));
+  };
+  // One 32-dim step of S^T = K Q^T: the A operands of step ks + 1 are read before the products of step ks.
+  auto k_step = [&](const char* buf, int ks, b8v (&ka)[2][4], f4v (&st)[RB][4]) {
+    if (ks + 1 < KS) {
 #pragma unroll
-  for (int j = 0; j < kCopies; ++j) copy_part(0, j);
-  __builtin_amdgcn_s_waitcnt(VmCnt(0));
-  __syncthreads();
-  for (int tile = 0; tile < n_tiles; ++tile) {
-    const bool more = tile + 1 < n_tiles;
-    const char* buf = lds[tile % 2];
-    // ---- S^T = K Q^T
-    f4v st[RB][4];
+      for (int kt = 0; kt < 4; ++kt) ka[(ks + 1) % 2][kt] = read_k(buf, ks + 1, kt);
+    }
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+      for (int i = 0; i < RB; ++i)
+        st[i][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[ks % 2][kt], qb[i][ks], st[i][kt], 0, 0, 0);
+  };
+  auto clear = [&](f4v (&st)[RB][4]) {
 #pragma unroll
     for (int i = 0; i < RB; ++i)
 #pragma unroll
       for (int kt = 0; kt < 4; ++kt) st[i][kt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
-    {
-      auto read_k = [&](int ks, int kt) -> b8v {
-        return *reinterpret_cast<const b8v*>(buf + koff + kt * 16 * (2 * D) + 16 * ((4 * ks + jg) ^ sw));
-      };
-      b8v ka[2][4];  // operands are read one step ahead of their use
+  };
+  // Online softmax per query (= per lane). The reference point m of the numerators 2^(score - m) is a whole power
+  // of two and is only moved when a score exceeds it by more than 2^16: moving it rescales numerators, sums and
+  // accumulators by a power of two, which is exact, so moving it late changes nothing in the result, while bf16
+  // numerators and f32 sums have room for the factor 2^16. Rescaling is then rare (the first tile, mostly).
+  auto row_max = [&](const f4v (&st)[4]) -> float {  // over the 64 keys of the tile, times the softmax scale
+    float mx = fmaxf(fmaxf(st[0][0], st[0][1]), fmaxf(st[0][2], st[0][3]));
 #pragma unroll
-      for (int kt = 0; kt < 4; ++kt) ka[0][kt] = read_k(0, kt);
+    for (int kt = 1; kt < 4; ++kt) mx = fmaxf(mx, fmaxf(fmaxf(st[kt][0], st[kt][1]), fmaxf(st[kt][2], st[kt][3])));
+    return MaxOverLaneGroups(mx) * sscale;  // sscale > 0 is required by the entry point
+  };
+  auto move_reference = [&](int i, float mx) {
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(mx > m[i] + 16.0f) != 0, 0)) {
+      const b8v zero = {0, 0, 0, 0, 0, 0, 0, 0};
+      const float mn = mx > m[i] + 16.0f ? __builtin_ceilf(mx) : m[i];
+      const float alpha = __builtin_amdgcn_exp2f(m[i] - mn);
+      m[i] = mn;
+      // The rescaled accumulators go back through a matrix instruction with zero factors: that keeps them in the
+      // accumulation registers on this path as on the common one (otherwise the compiler moves all of them to
+      // ordinary registers and back in every tile, rescaled or not); the empty asm keeps the copy out of the
+      // accumulation registers on this path.
+      {
+        f4v t = lacc[i];
+        asm volatile("" : "+a"(t));
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        if (ks + 1 < KS) {
+        for (int r = 0; r < 4; ++r) t[r] *= alpha;
+        lacc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(zero, zero, t, 0, 0, 0);
+      }
 #pragma unroll
-          for (int kt = 0; kt < 4; ++kt) ka[(ks + 1) % 2][kt] = read_k(ks + 1, kt);
-        }
+      for (int dt = 0; dt < NDT; ++dt) {
+        f4v t = o[i][dt];
+        asm volatile("" : "+a"(t));
 #pragma unroll
-        for (int kt = 0; kt < 4; ++kt)
+        for (int r = 0; r < 4; ++r) t[r] *= alpha;
+        o[i][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(zero, zero, t, 0, 0, 0);
+      }
+    }
+  };
+  // bf16 numerators of row block i as B operands of the second product: [32-key step] 4 + 4 keys per lane
+  auto numerators = [&](int i, const f4v (&st)[4], b8v (&pv)[2]) {
+    uint32_t w[2][4];
 #pragma unroll
-          for (int i = 0; i < RB; ++i)
-            st[i][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[ks % 2][kt], qb[i][ks], st[i][kt], 0, 0, 0);
-        if (more) copy_part(tile + 1, ks);
+    for (int kt = 0; kt < 4; ++kt) {
+      float p[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) p[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(st[kt][r], sscale, -m[i]));
+      w[kt / 2][2 * (kt % 2)] = PackBf16(p[0], p[1]);
+      w[kt / 2][2 * (kt % 2) + 1] = PackBf16(p[2], p[3]);
+    }
+#pragma unroll
+    for (int s2 = 0; s2 < 2; ++s2) pv[s2] = __builtin_bit_cast(b8v, uint4{w[s2][0], w[s2][1], w[s2][2], w[s2][3]});
+  };
+  // O^T += V^T P^T and the denominators; `v_tile` >= 0: the V half of that image is copied meanwhile
+  auto pv_product = [&](const char* buf, const b8v (&pv)[RB][2], int v_tile) {
+    auto read_v = [&](int dt, int s2) -> b8v {
+      return *reinterpret_cast<const b8v*>(buf + voff + dt * 16 * 128 + 16 * ((4 * s2 + jg) ^ sw));
+    };
+    b8v va[3][2];  // read two 16-dim tiles ahead
+#pragma unroll
+    for (int s2 = 0; s2 < 2; ++s2) va[0][s2] = read_v(0, s2), va[1][s2] = read_v(1, s2);
+#pragma unroll
+    for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+      for (int i = 0; i < RB; ++i)
+        lacc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(OnesBf16(), pv[i][s2], lacc[i], 0, 0, 0);
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt) {
+      if (dt + 2 < NDT) {
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) va[(dt + 2) % 3][s2] = read_v(dt + 2, s2);
+      }
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+        for (int i = 0; i < RB; ++i)
+          o[i][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[dt % 3][s2], pv[i][s2], o[i][dt], 0, 0, 0);
+      if (dt % 2 == 1) {
+        if (v_tile >= 0) copy_part(v_tile, KS + dt / 2);
         __builtin_amdgcn_sched_barrier(0);
       }
     }
-    // ---- online softmax per query (= per lane). The reference point m of the numerators 2^(score - m) is a whole
-    // power of two and is only moved when a score exceeds it by more than 2^16: moving it rescales numerators, sums
-    // and accumulators by a power of two, which is exact, so moving it late changes nothing in the result, while
-    // bf16 numerators and f32 sums have room for the factor 2^16. Rescaling is then rare (the first tile, mostly).
-    const bool diag = (tile + 1) * kKeys > prefix + q0 + 1;
-    uint32_t pb[RB][2][4];
+  };
+
+  // Schedule. Iteration t has the scores S^T(t) in registers, K(t + 1) and V(t) in LDS. It computes S^T(t + 1) on the
+  // matrix cores while the vector units turn S^T(t) into numerators (one wave per SIMD: only instructions of the same
+  // wave can overlap), then V^T P^T(t); meanwhile K(t + 2) and V(t + 1) are copied into the halves of the two LDS
+  // buffers that are free. One barrier per tile. Tiles that need the causal mask (the last one or two) and the last
+  // tile take the plain path below the pipelined loop.
+  const int n_full = min(n_tiles, (prefix + q0 + 1) / kKeys);  // tiles every query of the workgroup sees whole
+  const int n_pipe = min(n_full, n_tiles - 1);
 #pragma unroll
-    for (int i = 0; i < RB; ++i) {
-      if (diag) {
+  for (int j = 0; j < kCopies; ++j) copy_part(0, j);
+#pragma unroll
+  for (int j = 0; j < kCopies / 2; ++j) copy_part(min(1, n_tiles - 1), j);  // K(1) (K(0) again if there is no tile 1)
+  __builtin_amdgcn_s_waitcnt(VmCnt(0));
+  __syncthreads();
+  f4v st[RB][4];
+  clear(st);
+  {
+    b8v ka[2][4];
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt) ka[0][kt] = read_k(lds[0], 0, kt);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      k_step(lds[0], ks, ka, st);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  int tile = 0;
+  constexpr int KA = KS / 4;  // steps of the next tile's first product that run beside the row maxima
+  for (; tile < n_pipe; ++tile) {
+    const char* kbuf = lds[(tile + 1) % 2];
+    const int k_tile = min(tile + 2, n_tiles - 1);  // its K half goes where K(tile) was (again K(last) at the end)
+    f4v sn[RB][4];
+    clear(sn);
+    b8v ka[2][4];
+    float mx[RB];
+    b8v pv[RB][2];
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt) ka[0][kt] = read_k(kbuf, 0, kt);
+#pragma unroll
+    for (int ks = 0; ks < KA; ++ks) {
+      k_step(kbuf, ks, ka, sn);
+      copy_part(k_tile, ks);
+    }
+#pragma unroll
+    for (int i = 0; i < RB; ++i) mx[i] = row_max(st[i]);
+#pragma unroll
+    for (int n = 0; n < KA * 4 * RB; ++n) {  // spread the vector work between the matrix instructions
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < RB; ++i) move_reference(i, mx[i]);
+#pragma unroll
+    for (int ks = KA; ks < KS; ++ks) {
+      k_step(kbuf, ks, ka, sn);
+      copy_part(k_tile, ks);
+    }
+#pragma unroll
+    for (int i = 0; i < RB; ++i) numerators(i, st[i], pv[i]);
+#pragma unroll
+    for (int n = 0; n < (KS - KA) * 4 * RB; ++n) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    pv_product(lds[tile % 2], pv, tile + 1);
+#pragma unroll
+    for (int i = 0; i < RB; ++i)
+#pragma unroll
+      for (int kt = 0; kt < 4; ++kt) st[i][kt] = sn[i][kt];
+    __builtin_amdgcn_s_waitcnt(VmCnt(0));  // this wave's pieces of K(tile + 2) and V(tile + 1) have landed
+    __syncthreads();                       // ... and everybody's; everybody is done with K(tile + 1) and V(tile)
+  }
+  // ---- the last tiles, one phase after the other: masked softmax, second product, then the next tile's scores
+  for (; tile < n_tiles; ++tile) {
+    const bool more = tile + 1 < n_tiles;
+    if ((tile + 1) * kKeys > prefix + q0 + 1) {  // some key of the tile is masked for some query
+#pragma unroll
+      for (int i = 0; i < RB; ++i)
 #pragma unroll
         for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
           for (int r = 0; r < 4; ++r)
             if (tile * kKeys + 16 * kt + 4 * jg + r > prefix + qpos[i]) st[i][kt][r] = kNegBig;
-      }
-      float mx = fmaxf(fmaxf(st[i][0][0], st[i][0][1]), fmaxf(st[i][0][2], st[i][0][3]));
+    }
+    b8v pv[RB][2];
 #pragma unroll
-      for (int kt = 1; kt < 4; ++kt)
-        mx = fmaxf(mx, fmaxf(fmaxf(st[i][kt][0], st[i][kt][1]), fmaxf(st[i][kt][2], st[i][kt][3])));
-      mx = MaxOverLaneGroups(mx) * sscale;  // sscale > 0 is required by the entry point
-      if (__builtin_expect(__builtin_amdgcn_ballot_w64(mx > m[i] + 16.0f) != 0, 0)) {
-        const b8v zero = {0, 0, 0, 0, 0, 0, 0, 0};
-        const float mn = mx > m[i] + 16.0f ? __builtin_ceilf(mx) : m[i];
-        const float alpha = __builtin_amdgcn_exp2f(m[i] - mn);
-        m[i] = mn;
-        {
-          f4v t = lacc[i];
-          asm volatile("" : "+a"(t));
+    for (int i = 0; i < RB; ++i) {
+      move_reference(i, row_max(st[i]));
+      numerators(i, st[i], pv[i]);
+    }
+    pv_product(lds[tile % 2], pv, more ? tile + 1 : -1);
+    if (more) {
+      const char* kbuf = lds[(tile + 1) % 2];
+      clear(st);
+      b8v ka[2][4];
 #pragma unroll
-          for (int r = 0; r < 4; ++r) t[r] *= alpha;
-          lacc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(zero, zero, t, 0, 0, 0);
-        }
-        // The rescaled accumulators go back through a matrix instruction with zero factors: that keeps them in
-        // the accumulation registers on this path as on the common one (otherwise the compiler moves all of them to
-        // ordinary registers and back in every tile, rescaled or not).
+      for (int kt = 0; kt < 4; ++kt) ka[0][kt] = read_k(kbuf, 0, kt);
 #pragma unroll
-        for (int dt = 0; dt < NDT; ++dt) {
-          f4v t = o[i][dt];
-          asm volatile("" : "+a"(t));  // the copy out of the accumulation registers stays on this path
-#pragma unroll
-          for (int r = 0; r < 4; ++r) t[r] *= alpha;
-          o[i][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(zero, zero, t, 0, 0, 0);
-        }
-      }
-#pragma unroll
-      for (int kt = 0; kt < 4; ++kt) {
-        float p[4];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) p[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(st[i][kt][r], sscale, -m[i]));
-        pb[i][kt / 2][2 * (kt % 2)] = PackBf16(p[0], p[1]);
-        pb[i][kt / 2][2 * (kt % 2) + 1] = PackBf16(p[2], p[3]);
+      for (int ks = 0; ks < KS; ++ks) {
+        k_step(kbuf, ks, ka, st);
+        if (tile + 2 < n_tiles) copy_part(tile + 2, ks);
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
-    // ---- O^T += V^T P^T
-    {
-      auto read_v = [&](int dt, int s2) -> b8v {
-        return *reinterpret_cast<const b8v*>(buf + voff + dt * 16 * 128 + 16 * ((4 * s2 + jg) ^ sw));
-      };
-      b8v pv[RB][2];
-#pragma unroll
-      for (int i = 0; i < RB; ++i)
-#pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2)
-          pv[i][s2] = __builtin_bit_cast(b8v, uint4{pb[i][s2][0], pb[i][s2][1], pb[i][s2][2], pb[i][s2][3]});
-      b8v va[3][2];  // read two 16-dim tiles ahead
-#pragma unroll
-      for (int s2 = 0; s2 < 2; ++s2) va[0][s2] = read_v(0, s2), va[1][s2] = read_v(1, s2);
-#pragma unroll
-      for (int s2 = 0; s2 < 2; ++s2)
-#pragma unroll
-        for (int i = 0; i < RB; ++i)
-          lacc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(OnesBf16(), pv[i][s2], lacc[i], 0, 0, 0);
-#pragma unroll
-      for (int dt = 0; dt < NDT; ++dt) {
-        if (dt + 2 < NDT) {
-#pragma unroll
-          for (int s2 = 0; s2 < 2; ++s2) va[(dt + 2) % 3][s2] = read_v(dt + 2, s2);
-        }
-#pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2)
-#pragma unroll
-          for (int i = 0; i < RB; ++i)
-            o[i][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[dt % 3][s2], pv[i][s2], o[i][dt], 0, 0, 0);
-        if (dt % 2 == 1) {
-          if (more) copy_part(tile + 1, KS + dt / 2);
-          __builtin_amdgcn_sched_barrier(0);
-        }
-      }
-    }
-    __builtin_amdgcn_s_waitcnt(VmCnt(0));  // this wave's part of the next image has landed
-    __syncthreads();                       // ... and everybody's; everybody is done with this tile's image
+    __builtin_amdgcn_s_waitcnt(VmCnt(0));
+    __syncthreads();
   }
   StoreRows<D, RB>(a, s, h, G, jg, o, lacc, qpos, head);
 }
