@@ -33,8 +33,9 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 NQ, NKV, HD, PT = 24, 4, 256, 64
 # HBM bytes per launch of the split-K kernel from rocprofv3 counters (FETCH_SIZE + WRITE_SIZE, each scaled by what the
 # counter reads for a plain 1 GiB copy); a measurement made outside this script, recorded with its summary.
-TRAFFIC = {"ragged_b64_q8_0": 5.381e9}
-TRAFFIC_SOURCE = "profiles/decode_part_q8_0_ragged_b64.md"
+TRAFFIC = {"ragged_b64_q8_0": (5.381e9, "profiles/decode_part_q8_0_ragged_b64.md"),
+           "b16_ctx128k_q4_0": (2.435e9, "profiles/decode_part_q4_0_b16_ctx128k.md"),
+           "prefill_b8_ctx16k_chunk2k_q8_0": (2.150e9, "profiles/prefill_attend_q8_0_b8_ctx16k_chunk2k.md")}
 
 
 def fnv1a(b):
@@ -235,8 +236,9 @@ def run_prefill(a, wl, torch, yahkv):
         "parity_max_rel_err": float(f"{err:.3e}"), "out_fnv1a": first_hash,
         "roofline": {"bound": "mfma", "achieved": round(flops / (kern_ms * 1e-3) / 1e12, 1),
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(flops / (kern_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
-                     "kernel": "PrefillAttendImg<%d>" % HD, "kernel_ms": round(kern_ms, 4)},
+                     "frac": round(flops / (kern_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+                     "traffic": TRAFFIC[a.workload][0], "traffic_source": TRAFFIC[a.workload][1],
+                     "kernel": "PrefillAttendImg<%d, 2>" % HD, "kernel_ms": round(kern_ms, 4)},
     }
     if not a.no_cpu_baseline:
         res["cpu_baseline"] = prefill_cpu_baseline(wl, scale)
@@ -334,8 +336,8 @@ def main():
         "pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2), "tok_per_s": round(B / (ms * 1e-3), 1),
         "kv_bytes_per_step": int(kv_bytes), "parity_max_rel_err": float(f"{err:.3e}"), "out_fnv1a": first_hash,
         "roofline": {"bound": "hbm", "achieved": round(kgbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(kgbs / HBM_PEAK_GBS, 4), "traffic": TRAFFIC.get(a.workload),
-                     "traffic_source": TRAFFIC_SOURCE if a.workload in TRAFFIC else None,
+                     "frac": round(kgbs / HBM_PEAK_GBS, 4), "traffic": TRAFFIC.get(a.workload, (None, None))[0],
+                     "traffic_source": TRAFFIC.get(a.workload, (None, None))[1],
                      "kernel": "DattnPart<%d, %d, %d>" % (wl["fmt"], HD, PT), "kernel_ms": round(kern_ms, 4)},
     }
     if not a.no_cpu_baseline:
