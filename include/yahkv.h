@@ -112,6 +112,27 @@ int yahkv_append(const yahkv_geometry* g, const yahkv_pools* pools, const int32_
                  int32_t page_table_stride, const int32_t* start_pos, const int32_t* n_valid, int32_t n_seqs,
                  int32_t n_new, const void* k_src, const void* v_src, int32_t src_dtype, void* stream);
 
+/* Append fused with per-head RMSNorm and NeoX RoPE of K (and of Q on the way, if q_src is given):
+ *   normed[i] = (x[i] * rsqrt(sum x^2 / D + eps)) * weight[i]          (weight NULL = ones)
+ *   pair (p, p + rotary_dim / 2), p < rotary_dim / 2, is rotated by pos / theta^(2 p / rotary_dim)
+ * with pos = start_pos[s] + t; dims at or past rotary_dim are only normalised. The rotated K rows are quantized
+ * into their pages (never written out as f32 unless k_out is given), V rows are quantized as they are.
+ *   q_src / q_out  [n_seqs][n_new][n_q_heads][D] of src_dtype / q_out_dtype, or both NULL
+ *   k_out          [n_seqs][n_new][n_kv_heads][D] f32 or NULL
+ * Replaces yah_fused_qk_rope (engine/gpu/loom/yah_fused_qk_rope_f32.loom:1-10,96-241) followed by the K / V cache
+ * writes, and its paged batched form for prefill chunks (engine/gpu/loom/tools/emit_prefill_pp.py:31-111). */
+typedef struct yahkv_rope {
+  float theta;           /* rope base, e.g. 1e7 (yah_fused_qk_rope_f32.loom:33) */
+  float eps;             /* RMSNorm epsilon */
+  int32_t rotary_dim;    /* a multiple of 8, 8 .. head_dim */
+  const float* k_weight; /* device f32 [D] or NULL */
+  const float* q_weight; /* device f32 [D] or NULL */
+} yahkv_rope;
+int yahkv_append_rope(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
+                      int32_t page_table_stride, const int32_t* start_pos, const int32_t* n_valid, int32_t n_seqs,
+                      int32_t n_new, const void* k_src, const void* v_src, int32_t src_dtype, const yahkv_rope* rope,
+                      const void* q_src, void* q_out, int32_t q_out_dtype, float* k_out, void* stream);
+
 /* Decode attention: one query token per sequence against keys 0 .. seq_len[s] - 1.
  *   q    [n_seqs][n_q_heads][D] of q_dtype (F16 or BF16)
  *   gate [n_seqs][n_q_heads][D] f32 or NULL; with a gate, out = ctx * sigmoid(gate) (gen_decode_attn.py:402-407)

@@ -170,6 +170,19 @@ def append(pools, table, start_pos, n_valid, k_src, v_src):
                      _ptr(n_valid), C.c_int32(n_seqs), C.c_int32(n_new), _ptr(k_src), _ptr(v_src))
 
 
+def norm_rope(x, weight, rotary_dim, theta, eps, pos):
+    """x f32 [..., D] rows; pos int per row (same leading shape); returns the normalised, rotated rows."""
+    x = np.ascontiguousarray(x, np.float32)
+    d = x.shape[-1]
+    rows = x.reshape(-1, d)
+    pos = np.ascontiguousarray(np.broadcast_to(np.asarray(pos, np.int32), x.shape[:-1]).reshape(-1), np.int32)
+    w = None if weight is None else np.ascontiguousarray(weight, np.float32)
+    out = np.empty_like(rows)
+    lib().orc_norm_rope(_ptr(rows), _ptr(w), C.c_int32(rows.shape[0]), C.c_int32(d), C.c_int32(rotary_dim),
+                        C.c_float(theta), C.c_float(eps), _ptr(pos), _ptr(out))
+    return out.reshape(x.shape)
+
+
 def gather_blocks(pools, table_row, n_tokens):
     g = pools.geom
     bb = 34 if g.format == 8 else 18

@@ -331,6 +331,31 @@ void orc_decode_attend(const orc_geometry* g, const orc_pools* pools, const int3
     }
 }
 
+/* engine/gpu/loom/yah_fused_qk_rope_f32.loom:96-146 (Q branch; the K branch :147-214 is the same arithmetic):
+ * sum of squares, mean + eps, rsqrt, (x * inv_rms) * weight, then pairs (p, p + half) rotated by
+ * pos * (1 / powf(theta, 2 p / rotary_dim)); dims at or past rotary_dim are only normalised (:137-146). */
+void orc_norm_rope(const float* x, const float* weight, int32_t n_rows, int32_t head_dim, int32_t rotary_dim,
+                   float theta, float eps, const int32_t* pos, float* out) {
+  const int half = rotary_dim / 2;
+  for (int r = 0; r < n_rows; ++r) {
+    const float* xr = x + (size_t)r * head_dim;
+    float* o = out + (size_t)r * head_dim;
+    float ss = 0;
+    for (int i = 0; i < head_dim; ++i) ss += xr[i] * xr[i];
+    const float inv = 1.0f / sqrtf(ss / (float)head_dim + eps);
+    for (int i = 0; i < head_dim; ++i) o[i] = (xr[i] * inv) * (weight ? weight[i] : 1.0f);
+    const float posf = (float)pos[r];
+    for (int p = 0; p < half; ++p) {
+      const float invfreq = powf(theta, (2.0f * (float)p) / (float)rotary_dim);
+      const float angle = posf * (1.0f / invfreq);
+      const float cv = cosf(angle), sv = sinf(angle);
+      const float n0 = o[p], n1 = o[p + half];
+      o[p] = n0 * cv - n1 * sv;
+      o[p + half] = n0 * sv + n1 * cv;
+    }
+  }
+}
+
 static float round_bf16(float x) { return orc_bf16_to_f32(orc_f32_to_bf16(x)); }
 
 void orc_prefill_attend(const orc_geometry* g, const orc_pools* pools, const int32_t* table, int32_t stride,

@@ -18,6 +18,10 @@
  *   orc_decode_attend      float64 closed-form softmax over dequantized K/V (what
  *                          engine/gpu/loom/tools/dattn_q_check.py:193-203 does) and special cases
  *   orc_prefill_attend     same closed form with the causal mask; chunk of 1 == decode
+ *   orc_norm_rope          the reference holds no vectors for its norm + RoPE kernel; pinned by a hand-computed
+ *                          known answer that tells the half-split pairing from the interleaved one, by pos = 0
+ *                          (rotation is the identity), by the norms of rotated pairs, by the relative-position
+ *                          property of the dot product, and against an independent float64 numpy form
  */
 #ifndef YAHKV_ORACLE_H_
 #define YAHKV_ORACLE_H_
@@ -70,6 +74,10 @@ size_t orc_vs_bytes(const orc_geometry* g);
 void orc_append(const orc_geometry* g, const orc_pools* pools, const int32_t* table, int32_t stride,
                 const int32_t* start_pos, const int32_t* n_valid, int32_t n_seqs, int32_t n_new,
                 const float* k_src, const float* v_src);
+/* Per-row RMSNorm and NeoX (half-split) RoPE, in f32 in the reference's order of operations
+ * (engine/gpu/loom/yah_fused_qk_rope_f32.loom:96-146): x, out [n_rows][D]; pos [n_rows]; weight [D] or NULL. */
+void orc_norm_rope(const float* x, const float* weight, int32_t n_rows, int32_t head_dim, int32_t rotary_dim,
+                   float theta, float eps, const int32_t* pos, float* out);
 /* tokens [0, n_tokens) of one sequence as ggml blocks [n_tokens][H][NB][34|18]. */
 void orc_gather_blocks(const orc_geometry* g, const orc_pools* pools, const int32_t* table_row, int32_t n_tokens,
                        uint8_t* dst_k, uint8_t* dst_v);

@@ -27,6 +27,11 @@ class Pools(C.Structure):
     _fields_ = [("kq", C.c_void_p), ("ks", C.c_void_p), ("vq", C.c_void_p), ("vs", C.c_void_p)]
 
 
+class Rope(C.Structure):
+    _fields_ = [("theta", C.c_float), ("eps", C.c_float), ("rotary_dim", C.c_int32), ("k_weight", C.c_void_p),
+                ("q_weight", C.c_void_p)]
+
+
 def _load():
     if not os.path.exists(LIB_PATH):
         raise ImportError(f"{LIB_PATH} is not built: run `python __graft_entry__.py build` (hipcc, gfx950)")
@@ -44,6 +49,8 @@ def _load():
         getattr(lib, n).argtypes = [G]
     lib.yahkv_validate_page_table.argtypes = [G, i32p, i32, i32p, i32]
     lib.yahkv_append.argtypes = [G, P, i32p, i32, i32p, i32p, i32, i32, vp, vp, i32, vp]
+    lib.yahkv_append_rope.argtypes = [G, P, i32p, i32, i32p, i32p, i32, i32, vp, vp, i32, C.POINTER(Rope), vp, vp, i32,
+                                      vp, vp]
     lib.yahkv_decode_workspace_bytes.restype = C.c_size_t
     lib.yahkv_decode_workspace_bytes.argtypes = [G, i32, i32]
     lib.yahkv_decode_plan.argtypes = [G, i32, i32p, i32, i32, vp, C.c_size_t, vp]
@@ -186,6 +193,31 @@ def append(pools, table, start_pos, k_src, v_src, n_valid=None):
     st = pools.struct()
     _check(lib.yahkv_append(C.byref(g), C.byref(st), _dp(table), table.shape[1], _dp(start_pos), _dp(n_valid),
                             n_seqs, n_new, _dp(k_src), _dp(v_src), _dtype_code(k_src), _stream()), "append")
+
+
+def append_rope(pools, table, start_pos, k_src, v_src, theta, eps, rotary_dim, k_weight=None, q_weight=None, q_src=None,
+                q_out_dtype=None, want_k=False, n_valid=None):
+    """append() with per-head RMSNorm + NeoX RoPE of K fused in (position of token t of sequence s: start_pos[s] + t).
+    q_src [n_seqs][n_new][n_q_heads][D] is normalised and rotated into the returned q_out; want_k also returns the
+    rotated K rows as f32. Returns (q_out or None, k_out or None)."""
+    import torch
+    g = pools.geom
+    assert k_src.is_contiguous() and v_src.is_contiguous() and table.is_contiguous() and k_src.dtype == v_src.dtype
+    n_seqs, n_new = k_src.shape[0], k_src.shape[1]
+    assert tuple(k_src.shape) == (n_seqs, n_new, g.n_kv_heads, g.head_dim) and k_src.shape == v_src.shape
+    q_out = None
+    if q_src is not None:
+        assert q_src.is_contiguous() and q_src.dtype == k_src.dtype
+        assert tuple(q_src.shape) == (n_seqs, n_new, g.n_q_heads, g.head_dim)
+        q_out = torch.empty(q_src.shape, dtype=q_out_dtype or torch.float32, device=q_src.device)
+    k_out = torch.empty(k_src.shape, dtype=torch.float32, device=k_src.device) if want_k else None
+    rope = Rope(theta, eps, rotary_dim, _dp(k_weight), _dp(q_weight))
+    st = pools.struct()
+    _check(lib.yahkv_append_rope(C.byref(g), C.byref(st), _dp(table), table.shape[1], _dp(start_pos), _dp(n_valid),
+                                 n_seqs, n_new, _dp(k_src), _dp(v_src), _dtype_code(k_src), C.byref(rope), _dp(q_src),
+                                 _dp(q_out), _dtype_code(q_out) if q_out is not None else 0, _dp(k_out), _stream()),
+           "append_rope")
+    return q_out, k_out
 
 
 def decode_workspace_bytes(g, n_seqs, max_seq_len):

@@ -6,17 +6,10 @@
 // Placement follows the reference's page mapping (engine/gpu/loom/tools/gen_kvq.py:48-71): token at position p goes
 // to page table[p / PT] (clamped into the pool), slot p % PT.
 #include "common.hpp"
-
-// The quantizers' results are compared bit for bit with code built with -ffp-contract=off (the reference's host
-// flags, engine/build_hrx.sh:26): no multiply-add fusion in this file.
-#pragma clang fp contract(off)
+#include "quant.hpp"
 
 namespace yahkv {
 namespace {
-
-// A code from x * inv as the x86-64 reference computes it: lround, whose result for a non-finite or out-of-range
-// argument converts to the int8 0 there (only reachable when 1 / d overflowed, i.e. amax < 2^-119).
-__device__ __forceinline__ int CodeQ8(float r) { return fabsf(r) <= 128.0f ? static_cast<int>(roundf(r)) : 0; }
 
 struct AppendArgs {
   Geom g;
@@ -61,50 +54,10 @@ __global__ __launch_bounds__(256) void AppendBlocks(const AppendArgs a) {
 #pragma unroll
   for (int j = 0; j < 32; ++j) x[j] = LoadSrc(src, off + j, a.src_dtype);
 
-  uint8_t code[32];
+  alignas(16) uint8_t code[32];
   uint16_t hd;
-  if (FMT == 8) {
-    float amax = 0.0f;
-#pragma unroll
-    for (int j = 0; j < 32; ++j) amax = fmaxf(amax, fabsf(x[j]));
-    const float d = amax / 127.0f;
-    const float inv = d > 0.0f ? 1.0f / d : 0.0f;
-    hd = __builtin_bit_cast(uint16_t, static_cast<_Float16>(d));
-#pragma unroll
-    for (int j = 0; j < 32; ++j) code[j] = static_cast<uint8_t>(static_cast<int8_t>(CodeQ8(x[j] * inv)));
-  } else {
-    float amax = 0.0f, mx = 0.0f;
-#pragma unroll
-    for (int j = 0; j < 32; ++j) {
-      const float av = fabsf(x[j]);
-      if (amax < av) amax = av, mx = x[j];
-    }
-    const float d = mx / -8.0f;
-    const float id = d != 0.0f ? 1.0f / d : 0.0f;
-    hd = __builtin_bit_cast(uint16_t, static_cast<_Float16>(d));
-#pragma unroll
-    for (int j = 0; j < 16; ++j) {
-      const int q0 = min(15, static_cast<int>(static_cast<int8_t>(static_cast<int>(x[j] * id + 8.5f))));
-      const int q1 = min(15, static_cast<int>(static_cast<int8_t>(static_cast<int>(x[j + 16] * id + 8.5f))));
-      code[j] = static_cast<uint8_t>(q0 | (q1 << 4));
-    }
-  }
-
-  constexpr int CB = FMT == 8 ? 32 : 16;
-  const size_t ph = size_t(page) * H + h;
-  if (!is_v) {
-    a.pools.ks[(ph * PT + t) * NB + b] = hd;
-    uint4* dst = reinterpret_cast<uint4*>(a.pools.kq + ((ph * NB + b) * PT + t) * CB);
-    const uint4* c4 = reinterpret_cast<const uint4*>(code);
-#pragma unroll
-    for (int j = 0; j < CB / 16; ++j) dst[j] = c4[j];
-  } else {
-    a.pools.vs[(ph * NB + b) * PT + t] = hd;
-    // q8_0: row (32 b + j) of [D][PT]; q4_0: row (16 b + j) of [NB * 16][PT]
-    uint8_t* dst = a.pools.vq + (ph * NB + b) * CB * PT + t;
-#pragma unroll
-    for (int j = 0; j < CB; ++j) dst[size_t(j) * PT] = code[j];
-  }
+  QuantizeBlock<FMT>(x, code, &hd);
+  StoreBlock<FMT>(g, a.pools, is_v, page, t, h, b, code, hd);
 }
 
 // One thread per (K|V, token, kv head, block): the block back in ggml order (scale, then codes).
