@@ -1,17 +1,26 @@
-// Token append: block-quantize K and V rows and scatter them into their pages; and the inverse gather used by tests.
+// Token append: block-quantize K and V rows and scatter them into their pages, optionally with the head RMSNorm and
+// NeoX RoPE of K (and of the queries) fused in; and the inverse gather used by tests.
 //
-// Arithmetic is the reference's QuantizeQ8_0 (engine/core/gguf_quant.cpp:310-320), bit for bit: amax over the 32
-// elements, d = amax / 127 (IEEE division), inv = d > 0 ? 1 / d : 0, code = lround(x * inv) (halves away from zero),
-// stored scale = f16(d) (round to nearest even). q4_0 follows ggml's quantize_row_q4_0_ref.
 // Placement follows the reference's page mapping (engine/gpu/loom/tools/gen_kvq.py:48-71): token at position p goes
-// to page table[p / PT] (clamped into the pool), slot p % PT.
+// to page table[p / PT] (clamped into the pool), slot p % PT; positions are clamped to the table
+// (gen_decode_attn.py:59-63). The quantizers are in quant.hpp.
+//
+// The fused form follows the reference's decode kernel (engine/gpu/loom/yah_fused_qk_rope_f32.loom:1-10, Q branch
+// :96-146, K branch :147-241) and its batched, paged rewrite for prefill chunks
+// (engine/gpu/loom/tools/emit_prefill_pp.py:31-111): per head
+//   inv_rms = rsqrt(sum_i x[i]^2 / head_dim + eps); normed[i] = (x[i] * inv_rms) * weight[i]
+//   angle(p) = pos * (1 / theta^(2 p / rotary_dim)), p < half = rotary_dim / 2
+//   out[p] = normed[p] cos - normed[p + half] sin; out[p + half] = normed[p] sin + normed[p + half] cos
+// and dims at or past rotary_dim are only normalised. The angle uses the token's position as given; the page slot
+// uses the position clamped to the table, as in the reference (:89-94). What the reference stores as f16 rows is
+// stored here as q8_0 / q4_0 blocks: the rotated K never makes a round trip through memory as f32.
 #include "common.hpp"
 #include "quant.hpp"
 
 namespace yahkv {
 namespace {
 
-struct AppendArgs {
+struct RopeArgs {
   Geom g;
   Pools pools;
   const int32_t* table;
@@ -22,42 +31,169 @@ struct AppendArgs {
   const void* k_src;
   const void* v_src;
   int32_t src_dtype;
+  const float* k_weight;
+  const float* q_weight;
+  float theta, eps;
+  int32_t rotary_dim;
+  const void* q_src;  // [n_seqs][n_new][n_q][D] of src_dtype, or null
+  void* q_out;        // same shape, of q_out_dtype
+  int32_t q_out_dtype;
+  float* k_out;       // [n_seqs][n_new][H][D] f32 or null: the rotated K rows, for callers that want them
 };
 
-// One thread per (K|V, sequence, new token, kv head, block): 64 work items per token at 4 kv heads x 256 dims.
-// The K block is stored as two 16-byte writes; the V block's bytes go to 32 rows of the transposed page.
-template <int FMT>
-__global__ __launch_bounds__(256) void AppendBlocks(const AppendArgs a) {
-  const Geom g = a.g;
-  const int NB = g.nb(), H = g.n_kv, PT = g.pt, D = g.hd;
-  const int64_t per_side = int64_t(a.n_seqs) * a.n_new * H * NB;
-  const int64_t idx = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (idx >= 2 * per_side) return;
-  const bool is_v = idx >= per_side;
-  int64_t r = is_v ? idx - per_side : idx;
-  const int b = int(r % NB);
-  r /= NB;
-  const int h = int(r % H);
-  r /= H;
-  const int i = int(r % a.n_new);
-  const int s = int(r / a.n_new);
-  if (a.n_valid != nullptr && i >= a.n_valid[s]) return;  // padding row of a short chunk
+// Four consecutive elements of a source / destination row (element index a multiple of 4).
+__device__ __forceinline__ float4 Load4(const void* src, size_t i, int dtype) {
+  if (dtype == YAHKV_F32) return *reinterpret_cast<const float4*>(static_cast<const float*>(src) + i);
+  const uint2 w = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(src) + i);
+  const uint16_t h[4] = {static_cast<uint16_t>(w.x & 0xFFFF), static_cast<uint16_t>(w.x >> 16),
+                         static_cast<uint16_t>(w.y & 0xFFFF), static_cast<uint16_t>(w.y >> 16)};
+  if (dtype == YAHKV_F16) return float4{WidenF16(h[0]), WidenF16(h[1]), WidenF16(h[2]), WidenF16(h[3])};
+  return float4{WidenBf16(h[0]), WidenBf16(h[1]), WidenBf16(h[2]), WidenBf16(h[3])};
+}
+__device__ __forceinline__ void Store4(void* dst, size_t i, int dtype, float4 v) {
+  if (dtype == YAHKV_F32) {
+    *reinterpret_cast<float4*>(static_cast<float*>(dst) + i) = v;
+    return;
+  }
+  uint32_t lo, hi;
+  if (dtype == YAHKV_F16) {
+    typedef _Float16 h2v __attribute__((ext_vector_type(2)));
+    lo = __builtin_bit_cast(uint32_t, h2v{static_cast<_Float16>(v.x), static_cast<_Float16>(v.y)});
+    hi = __builtin_bit_cast(uint32_t, h2v{static_cast<_Float16>(v.z), static_cast<_Float16>(v.w)});
+  } else {
+    typedef __bf16 b2v __attribute__((ext_vector_type(2)));
+    lo = __builtin_bit_cast(uint32_t, b2v{static_cast<__bf16>(v.x), static_cast<__bf16>(v.y)});
+    hi = __builtin_bit_cast(uint32_t, b2v{static_cast<__bf16>(v.z), static_cast<__bf16>(v.w)});
+  }
+  *reinterpret_cast<uint2*>(static_cast<uint16_t*>(dst) + i) = uint2{lo, hi};
+}
 
-  int pos = a.start_pos[s] + i;
-  pos = min(max(pos, 0), a.stride * PT - 1);  // gen_decode_attn.py:59-63
+// One workgroup of four wavefronts per token. With ROPE, the token's angles (they depend on the position and the
+// pair, not on the head) are computed once into LDS; without, K rows are quantized as they are (plain append) and
+// there are no query rows. The token's rows of head_dim values (its H K heads, its H V heads, then its
+// query heads) are dealt to the wavefronts in turn; a row lies across a wavefront, four consecutive dims per lane, so
+// every load and store is 16 (or 8) bytes per lane, the sum of squares and the block maxima are DPP reductions, and
+// the partner of a rotated pair comes through one lane shuffle: rows never go through LDS. A wavefront issues the
+// loads of all its rows (up to eight at a time) before it works on the first.
+constexpr int kRopeWaves = 4, kRowsInFlight = 8;
+template <int FMT, bool ROPE>
+__global__ __launch_bounds__(64 * kRopeWaves) void AppendRows(const RopeArgs a) {
+#pragma clang fp contract(off)
+  const Geom g = a.g;
+  const int NB = g.nb(), H = g.n_kv, PT = g.pt, D = g.hd, NQ = a.q_src != nullptr ? g.n_q : 0;
+  const int rows_per_token = 2 * H + NQ;
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  const int i = int(blockIdx.x % a.n_new), s = int(blockIdx.x / a.n_new);
+  if (a.n_valid != nullptr && i >= a.n_valid[s]) return;  // padding row of a short chunk
+  const int pos_raw = a.start_pos[s] + i;
+  const int pos = min(max(pos_raw, 0), a.stride * PT - 1);
   const int page = ClampPage(a.table[int64_t(s) * a.stride + pos / PT], g.n_pages);
   const int t = pos % PT;
 
-  const void* src = is_v ? a.v_src : a.k_src;
-  const size_t off = ((size_t(s) * a.n_new + i) * H + h) * D + size_t(b) * 32;
-  float x[32];
+  __shared__ __align__(16) float cs[128], sn[128];  // rotary_dim / 2 <= 128
+  const int rot = a.rotary_dim, half = rot / 2;
+  const float posf = static_cast<float>(pos_raw);
+  if (ROPE) {
+    for (int p = threadIdx.x; p < half; p += 64 * kRopeWaves) {
+      const float inv_freq = 1.0f / powf(a.theta, (2.0f * static_cast<float>(p)) / static_cast<float>(rot));
+      float sv, cv;
+      sincosf(posf * inv_freq, &sv, &cv);
+      cs[p] = cv, sn[p] = sv;
+    }
+    __syncthreads();
+  }
+  const int d0 = 4 * lane;  // this lane's four dims of every row
+  const bool has = d0 < D;
+  // This lane's part of the rotation, the same for every row: element e = d0 + j is the first of its pair
+  // (e < half: out = x c - partner s, partner = e + half), the second (half <= e < rot: out = partner s + x c,
+  // partner = e - half) or past the rotated dims. rotary_dim / 2 is a multiple of 4 (checked by the entry point), so
+  // the four partners lie in one lane.
+  float c4[4] = {1.0f, 1.0f, 1.0f, 1.0f}, s4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  int partner_lane = lane;
+  if (ROPE && has && d0 < rot) {
+    const bool first = d0 < half;
+    partner_lane = first ? lane + half / 4 : lane - half / 4;
 #pragma unroll
-  for (int j = 0; j < 32; ++j) x[j] = LoadSrc(src, off + j, a.src_dtype);
-
-  alignas(16) uint8_t code[32];
-  uint16_t hd;
-  QuantizeBlock<FMT>(x, code, &hd);
-  StoreBlock<FMT>(g, a.pools, is_v, page, t, h, b, code, hd);
+    for (int j = 0; j < 4; ++j) {
+      const int p = first ? d0 + j : d0 + j - half;
+      c4[j] = cs[p];
+      s4[j] = first ? -sn[p] : sn[p];
+    }
+  }
+  float4 wk = {1.0f, 1.0f, 1.0f, 1.0f}, wq = wk;  // this lane's norm weights
+  if (ROPE && a.k_weight != nullptr && has) wk = *reinterpret_cast<const float4*>(a.k_weight + d0);
+  if (ROPE && a.q_weight != nullptr && has) wq = *reinterpret_cast<const float4*>(a.q_weight + d0);
+  // source of row `row` of the token and its element offset
+  auto source = [&](int row, const void** src, size_t* off) {
+    const size_t tok = size_t(s) * a.n_new + i;
+    if (row < H) *src = a.k_src, *off = (tok * H + row) * D;
+    else if (row < 2 * H) *src = a.v_src, *off = (tok * H + (row - H)) * D;
+    else *src = a.q_src, *off = (tok * g.n_q + (row - 2 * H)) * D;
+  };
+  for (int first_row = wave; first_row < rows_per_token; first_row += kRopeWaves * kRowsInFlight) {
+    float4 x[kRowsInFlight];
+#pragma unroll
+    for (int j = 0; j < kRowsInFlight; ++j) {
+      const int row = first_row + kRopeWaves * j;
+      x[j] = float4{0.0f, 0.0f, 0.0f, 0.0f};
+      if (row < rows_per_token && has) {
+        const void* src;
+        size_t off;
+        source(row, &src, &off);
+        x[j] = Load4(src, off + d0, a.src_dtype);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < kRowsInFlight; ++j) {
+      const int row = first_row + kRopeWaves * j;
+      if (row >= rows_per_token) break;
+      const bool is_v = row >= H && row < 2 * H, is_q = row >= 2 * H;
+      float4 v = x[j];
+      if (ROPE && !is_v) {
+        const float ss = WaveSum(v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w);
+        const float inv_rms = 1.0f / sqrtf(ss / static_cast<float>(D) + a.eps);
+        const float4 w = is_q ? wq : wk;
+        v = float4{(v.x * inv_rms) * w.x, (v.y * inv_rms) * w.y, (v.z * inv_rms) * w.z, (v.w * inv_rms) * w.w};
+        const float px = __shfl(v.x, partner_lane, 64), py = __shfl(v.y, partner_lane, 64);
+        const float pz = __shfl(v.z, partner_lane, 64), pw = __shfl(v.w, partner_lane, 64);
+        // first of a pair: x c - partner s; second: partner s + x c (s4 carries the sign); past rot: c = 1, s = 0
+        v = float4{v.x * c4[0] + px * s4[0], v.y * c4[1] + py * s4[1], v.z * c4[2] + pz * s4[2],
+                   v.w * c4[3] + pw * s4[3]};
+      }
+      const void* src;
+      size_t off;
+      source(row, &src, &off);
+      if (is_q) {
+        if (has) Store4(a.q_out, off + d0, a.q_out_dtype, v);
+        continue;
+      }
+      if (!is_v && a.k_out != nullptr && has) *reinterpret_cast<float4*>(a.k_out + off + d0) = v;
+      // quantize: block b = lanes 8 b .. 8 b + 7
+      const int h = is_v ? row - H : row, b = lane / 8, lb = lane % 8;
+      uint16_t scale;
+      const uint32_t codes = FMT == 8 ? QuantizeLanesQ8(v, &scale) : QuantizeLanesQ4(v, lb, &scale);
+      if (!has) continue;
+      const size_t ph = size_t(page) * H + h;
+      if (!is_v) {
+        if (lb == 0) a.pools.ks[(ph * PT + t) * NB + b] = scale;
+        if (FMT == 8)
+          *reinterpret_cast<uint32_t*>(a.pools.kq + ((ph * NB + b) * PT + t) * 32 + 4 * lb) = codes;
+        else if (lb < 4)
+          *reinterpret_cast<uint32_t*>(a.pools.kq + ((ph * NB + b) * PT + t) * 16 + 4 * lb) = codes;
+      } else {
+        if (lb == 0) a.pools.vs[(ph * NB + b) * PT + t] = scale;
+        if (FMT == 8) {  // row (32 b + 4 lb + e) of [D][PT]
+          uint8_t* dst = a.pools.vq + (ph * D + d0) * PT + t;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) dst[size_t(e) * PT] = static_cast<uint8_t>(codes >> (8 * e));
+        } else if (lb < 4) {  // row (16 b + 4 lb + e) of [NB * 16][PT]
+          uint8_t* dst = a.pools.vq + ((ph * NB + b) * 16 + 4 * lb) * PT + t;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) dst[size_t(e) * PT] = static_cast<uint8_t>(codes >> (8 * e));
+        }
+      }
+    }
+  }
 }
 
 // One thread per (K|V, token, kv head, block): the block back in ggml order (scale, then codes).
@@ -98,26 +234,72 @@ __global__ __launch_bounds__(256) void GatherBlocks(Geom g, Pools pools, const i
 
 using namespace yahkv;
 
-extern "C" int yahkv_append(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
-                            int32_t page_table_stride, const int32_t* start_pos, const int32_t* n_valid,
-                            int32_t n_seqs, int32_t n_new, const void* k_src, const void* v_src, int32_t src_dtype,
-                            void* stream) {
+namespace {
+int CheckAppend(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
+                int32_t page_table_stride, const int32_t* start_pos, int32_t n_seqs, int32_t n_new, const void* k_src,
+                const void* v_src, int32_t src_dtype) {
   if (const int st = CheckGeometry(g)) return st;
   if (pools == nullptr || pools->kq == nullptr || pools->ks == nullptr || pools->vq == nullptr ||
       pools->vs == nullptr || page_table == nullptr || start_pos == nullptr || k_src == nullptr || v_src == nullptr)
     return YAHKV_ERR_ARG;
   if (n_seqs <= 0 || n_new <= 0 || page_table_stride <= 0) return YAHKV_ERR_ARG;
   if (src_dtype != YAHKV_F32 && src_dtype != YAHKV_F16 && src_dtype != YAHKV_BF16) return YAHKV_ERR_ARG;
-  if ((reinterpret_cast<uintptr_t>(pools->kq) | reinterpret_cast<uintptr_t>(pools->vq)) & 15) return YAHKV_ERR_ARG;
-  AppendArgs a{MakeGeom(*g), MakePools(*pools), page_table, page_table_stride, start_pos, n_valid,
-               n_seqs,       n_new,             k_src,      v_src,             src_dtype};
-  const int64_t items = int64_t(2) * n_seqs * n_new * a.g.n_kv * a.g.nb();
-  const unsigned blocks = static_cast<unsigned>((items + 255) / 256);
+  if ((reinterpret_cast<uintptr_t>(pools->kq) | reinterpret_cast<uintptr_t>(pools->vq) |
+       reinterpret_cast<uintptr_t>(k_src) | reinterpret_cast<uintptr_t>(v_src)) & 15)
+    return YAHKV_ERR_ARG;
+  if (int64_t(n_seqs) * n_new > 0x7FFFFFFF) return YAHKV_ERR_SHAPE;
+  return YAHKV_OK;
+}
+}  // namespace
+
+extern "C" int yahkv_append(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
+                            int32_t page_table_stride, const int32_t* start_pos, const int32_t* n_valid,
+                            int32_t n_seqs, int32_t n_new, const void* k_src, const void* v_src, int32_t src_dtype,
+                            void* stream) {
+  if (const int st = CheckAppend(g, pools, page_table, page_table_stride, start_pos, n_seqs, n_new, k_src, v_src,
+                                 src_dtype))
+    return st;
+  RopeArgs a{};
+  a.g = MakeGeom(*g), a.pools = MakePools(*pools), a.table = page_table, a.stride = page_table_stride;
+  a.start_pos = start_pos, a.n_valid = n_valid, a.n_seqs = n_seqs, a.n_new = n_new, a.k_src = k_src, a.v_src = v_src;
+  a.src_dtype = src_dtype, a.rotary_dim = 8, a.theta = 1.0f;
+  const dim3 grid(static_cast<unsigned>(n_seqs) * static_cast<unsigned>(n_new));
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (g->format == YAHKV_Q8_0)
-    hipLaunchKernelGGL(AppendBlocks<8>, dim3(blocks), dim3(256), 0, st, a);
+    hipLaunchKernelGGL((AppendRows<8, false>), grid, dim3(64 * kRopeWaves), 0, st, a);
   else
-    hipLaunchKernelGGL(AppendBlocks<4>, dim3(blocks), dim3(256), 0, st, a);
+    hipLaunchKernelGGL((AppendRows<4, false>), grid, dim3(64 * kRopeWaves), 0, st, a);
+  return LaunchStatus();
+}
+
+extern "C" int yahkv_append_rope(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
+                                 int32_t page_table_stride, const int32_t* start_pos, const int32_t* n_valid,
+                                 int32_t n_seqs, int32_t n_new, const void* k_src, const void* v_src,
+                                 int32_t src_dtype, const yahkv_rope* rope, const void* q_src, void* q_out,
+                                 int32_t q_out_dtype, float* k_out, void* stream) {
+  if (const int st = CheckAppend(g, pools, page_table, page_table_stride, start_pos, n_seqs, n_new, k_src, v_src,
+                                 src_dtype))
+    return st;
+  if (rope == nullptr) return YAHKV_ERR_ARG;
+  if ((q_src == nullptr) != (q_out == nullptr)) return YAHKV_ERR_ARG;
+  if (q_src != nullptr && q_out_dtype != YAHKV_F32 && q_out_dtype != YAHKV_F16 && q_out_dtype != YAHKV_BF16)
+    return YAHKV_ERR_ARG;
+  if ((reinterpret_cast<uintptr_t>(pools->kq) | reinterpret_cast<uintptr_t>(pools->vq)) & 15) return YAHKV_ERR_ARG;
+  const Geom m = MakeGeom(*g);
+  if (rope->rotary_dim < 8 || rope->rotary_dim > m.hd || rope->rotary_dim % 8 != 0) return YAHKV_ERR_ARG;
+  if (!(rope->theta > 0.0f) || !(rope->eps >= 0.0f)) return YAHKV_ERR_ARG;
+  RopeArgs a{};
+  a.g = m, a.pools = MakePools(*pools), a.table = page_table, a.stride = page_table_stride, a.start_pos = start_pos;
+  a.n_valid = n_valid, a.n_seqs = n_seqs, a.n_new = n_new, a.k_src = k_src, a.v_src = v_src, a.src_dtype = src_dtype;
+  a.k_weight = rope->k_weight, a.q_weight = rope->q_weight, a.theta = rope->theta, a.eps = rope->eps;
+  a.rotary_dim = rope->rotary_dim, a.q_src = q_src, a.q_out = q_out, a.q_out_dtype = q_out_dtype, a.k_out = k_out;
+  const int64_t tokens = int64_t(n_seqs) * n_new;
+  if (tokens > 0x7FFFFFFF) return YAHKV_ERR_SHAPE;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (g->format == YAHKV_Q8_0)
+    hipLaunchKernelGGL((AppendRows<8, true>), dim3(static_cast<unsigned>(tokens)), dim3(64 * kRopeWaves), 0, st, a);
+  else
+    hipLaunchKernelGGL((AppendRows<4, true>), dim3(static_cast<unsigned>(tokens)), dim3(64 * kRopeWaves), 0, st, a);
   return LaunchStatus();
 }
 

@@ -1,4 +1,4 @@
-// Block quantizers and the store of one block into its page, shared by the append kernels.
+// Block quantizers of the append kernels.
 //
 // Arithmetic is the reference's QuantizeQ8_0 (engine/core/gguf_quant.cpp:310-320), bit for bit: amax over the 32
 // elements, d = amax / 127 (IEEE division), inv = d > 0 ? 1 / d : 0, code = lround(x * inv) (halves away from zero),
@@ -16,59 +16,78 @@ namespace yahkv {
 // argument converts to the int8 0 there (only reachable when 1 / d overflowed, i.e. amax < 2^-119).
 __device__ __forceinline__ int CodeQ8(float r) { return fabsf(r) <= 128.0f ? static_cast<int>(roundf(r)) : 0; }
 
-// 32 values -> codes (32 bytes for q8_0, 16 bytes for q4_0: element j low nibble, j + 16 high nibble) and f16 scale.
-template <int FMT>
-__device__ __forceinline__ void QuantizeBlock(const float (&x)[32], uint8_t (&code)[32], uint16_t* scale) {
-#pragma clang fp contract(off)
-  if (FMT == 8) {
-    float amax = 0.0f;
-#pragma unroll
-    for (int j = 0; j < 32; ++j) amax = fmaxf(amax, fabsf(x[j]));
-    const float d = amax / 127.0f;
-    const float inv = d > 0.0f ? 1.0f / d : 0.0f;
-    *scale = __builtin_bit_cast(uint16_t, static_cast<_Float16>(d));
-#pragma unroll
-    for (int j = 0; j < 32; ++j) code[j] = static_cast<uint8_t>(static_cast<int8_t>(CodeQ8(x[j] * inv)));
-  } else {
-    float amax = 0.0f, mx = 0.0f;
-#pragma unroll
-    for (int j = 0; j < 32; ++j) {
-      const float av = fabsf(x[j]);
-      if (amax < av) amax = av, mx = x[j];
-    }
-    const float d = mx / -8.0f;
-    const float id = d != 0.0f ? 1.0f / d : 0.0f;
-    *scale = __builtin_bit_cast(uint16_t, static_cast<_Float16>(d));
-#pragma unroll
-    for (int j = 0; j < 16; ++j) {
-      const int q0 = min(15, static_cast<int>(static_cast<int8_t>(static_cast<int>(x[j] * id + 8.5f))));
-      const int q1 = min(15, static_cast<int>(static_cast<int8_t>(static_cast<int>(x[j + 16] * id + 8.5f))));
-      code[j] = static_cast<uint8_t>(q0 | (q1 << 4));
-    }
-  }
+template <int CTRL>
+__device__ __forceinline__ float Dpp(float x) {  // the value of another lane of the row, chosen by a DPP control
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xF, 0xF, false));
+}
+template <int CTRL>
+__device__ __forceinline__ int DppI(int x) { return __builtin_amdgcn_update_dpp(0, x, CTRL, 0xF, 0xF, false); }
+constexpr int kQuadSwap1 = 0xB1, kQuadSwap2 = 0x4E, kHalfMirror = 0x141, kRowMirror = 0x140;
+
+// Sum over the 64 lanes, in every lane: four DPP steps inside each row of 16 lanes, then the two row-swapping
+// instructions of gfx950 across the rows (no LDS round trips).
+__device__ __forceinline__ float WaveSum(float v) {
+  v += Dpp<kQuadSwap1>(v);
+  v += Dpp<kQuadSwap2>(v);
+  v += Dpp<kHalfMirror>(v);
+  v += Dpp<kRowMirror>(v);
+  const uint32_t u = __builtin_bit_cast(uint32_t, v);
+  const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  const uint32_t r0 = r[0], r1 = r[1];
+  const float w = __builtin_bit_cast(float, r0) + __builtin_bit_cast(float, r1);
+  const uint32_t x = __builtin_bit_cast(uint32_t, w);
+  const auto q = __builtin_amdgcn_permlane32_swap(x, x, false, false);
+  const uint32_t q0 = q[0], q1 = q[1];
+  return __builtin_bit_cast(float, q0) + __builtin_bit_cast(float, q1);
 }
 
-// Block b of kv head h of the token in slot t of `page`: the K block is stored as 16-byte writes, the V block's
-// bytes go to 32 (16) rows of the transposed page.
-template <int FMT>
-__device__ __forceinline__ void StoreBlock(const Geom& g, const Pools& pools, bool is_v, int page, int t, int h, int b,
-                                           const uint8_t (&code)[32], uint16_t scale) {
-  constexpr int CB = FMT == 8 ? 32 : 16;
-  const int NB = g.nb(), H = g.n_kv, PT = g.pt;
-  const size_t ph = size_t(page) * H + h;
-  if (!is_v) {
-    pools.ks[(ph * PT + t) * NB + b] = scale;
-    uint4* dst = reinterpret_cast<uint4*>(pools.kq + ((ph * NB + b) * PT + t) * CB);
-    const uint4* c4 = reinterpret_cast<const uint4*>(code);
+// A block of 32 values lies in 8 consecutive lanes, 4 values each (lane l of the 8: elements 4 l .. 4 l + 3).
+// q8_0: the block's amax in all 8 lanes (a maximum does not depend on the order), then the scalar formulas of
+// QuantizeBlock per element; returns this lane's 4 codes packed into a dword.
+__device__ __forceinline__ uint32_t QuantizeLanesQ8(const float4 v, uint16_t* scale) {
+#pragma clang fp contract(off)
+  float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+  amax = fmaxf(amax, Dpp<kQuadSwap1>(amax));
+  amax = fmaxf(amax, Dpp<kQuadSwap2>(amax));
+  amax = fmaxf(amax, Dpp<kHalfMirror>(amax));
+  const float d = amax / 127.0f;
+  const float inv = d > 0.0f ? 1.0f / d : 0.0f;
+  *scale = __builtin_bit_cast(uint16_t, static_cast<_Float16>(d));
+  const uint32_t c0 = static_cast<uint8_t>(static_cast<int8_t>(CodeQ8(v.x * inv)));
+  const uint32_t c1 = static_cast<uint8_t>(static_cast<int8_t>(CodeQ8(v.y * inv)));
+  const uint32_t c2 = static_cast<uint8_t>(static_cast<int8_t>(CodeQ8(v.z * inv)));
+  const uint32_t c3 = static_cast<uint8_t>(static_cast<int8_t>(CodeQ8(v.w * inv)));
+  return c0 | (c1 << 8) | (c2 << 16) | (c3 << 24);
+}
+// q4_0: ggml takes the value of largest magnitude, the first one on ties, so the reduction carries (|x|, index,
+// x) and prefers the lower index; d = that value / -8. Lanes 0-3 of the 8 return 4 bytes: low nibbles their own
+// elements j, high nibbles the elements j + 16 held by the lane four further on.
+__device__ __forceinline__ uint32_t QuantizeLanesQ4(const float4 v, int lane_in_block, uint16_t* scale) {
+#pragma clang fp contract(off)
+  const float e[4] = {v.x, v.y, v.z, v.w};
+  float av = fabsf(e[0]), mx = e[0];
+  int ix = 4 * lane_in_block;
 #pragma unroll
-    for (int j = 0; j < CB / 16; ++j) dst[j] = c4[j];
-  } else {
-    pools.vs[(ph * NB + b) * PT + t] = scale;
-    // q8_0: row (32 b + j) of [D][PT]; q4_0: row (16 b + j) of [NB * 16][PT]
-    uint8_t* dst = pools.vq + (ph * NB + b) * CB * PT + t;
+  for (int j = 1; j < 4; ++j)
+    if (av < fabsf(e[j])) av = fabsf(e[j]), mx = e[j], ix = 4 * lane_in_block + j;
+  auto merge = [&](float oav, float omx, int oix) {
+    if (oav > av || (oav == av && oix < ix)) av = oav, mx = omx, ix = oix;
+  };
+  merge(Dpp<kQuadSwap1>(av), Dpp<kQuadSwap1>(mx), DppI<kQuadSwap1>(ix));
+  merge(Dpp<kQuadSwap2>(av), Dpp<kQuadSwap2>(mx), DppI<kQuadSwap2>(ix));
+  merge(Dpp<kHalfMirror>(av), Dpp<kHalfMirror>(mx), DppI<kHalfMirror>(ix));
+  const float d = mx / -8.0f;
+  const float id = d != 0.0f ? 1.0f / d : 0.0f;
+  *scale = __builtin_bit_cast(uint16_t, static_cast<_Float16>(d));
+  uint32_t nib = 0;
 #pragma unroll
-    for (int j = 0; j < CB; ++j) dst[size_t(j) * PT] = code[j];
+  for (int j = 0; j < 4; ++j) {
+    const int q = min(15, static_cast<int>(static_cast<int8_t>(static_cast<int>(e[j] * id + 8.5f))));
+    nib |= static_cast<uint32_t>(q) << (8 * j);
   }
+  // the nibbles of the lane four further on (row_shr would move the wrong way: take them through a lane shuffle)
+  const uint32_t hi = static_cast<uint32_t>(__shfl_down(static_cast<int>(nib), 4, 64));
+  return nib | (hi << 4);
 }
 
 }  // namespace yahkv
