@@ -214,6 +214,36 @@ int yahkv_pagepool_free(yahkv_pagepool* p, const int32_t* pages, int32_t n);
 /* Hands out the free pages in the order of a seeded Fisher-Yates shuffle from now on (tests and benches use
  * it for a scrambled table, as gen_decode_attn's checker does, dattn_q_check.py:151). */
 void yahkv_pagepool_shuffle(yahkv_pagepool* p, uint64_t seed);
+/* Shared pages: every page has an owner count (1 after alloc). retain adds an owner to allocated pages (a sequence
+ * forked from a shared prefix keeps the prefix's full pages); free removes one, and a page returns to the free
+ * list when its last owner lets go. refcount: owners of a page, 0 = free, -1 = no such page.
+ * (The reference has no allocator; its prefix reuse is the whole-state slot, loom_prefill.hpp:976-1024.) */
+int yahkv_pagepool_retain(yahkv_pagepool* pool, const int32_t* pages, int32_t n);
+int32_t yahkv_pagepool_refcount(const yahkv_pagepool* pool, int32_t page);
+/* yahkv_validate_page_table for tables with shared pages: a page may appear in as many rows as it has owners in
+ * `pool` (never twice in one row, never a free page). */
+int yahkv_validate_shared_page_table(const yahkv_geometry* g, const yahkv_pagepool* pool, const int32_t* table,
+                                     int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs);
+
+/* Copy whole pages inside the pools: page src_pages[i] -> page dst_pages[i] (device int32 arrays), all four
+ * pools. For a fork: the shared prefix's last, partly filled page must be private before the fork appends. */
+int yahkv_copy_pages(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* src_pages,
+                     const int32_t* dst_pages, int32_t n, void* stream);
+
+/* Slots: the sequence state of one sequence, raw, as one buffer: a 64-byte header (u64 magic "YKVSLOT1", format,
+ * kv heads, head_dim, page_tokens, pages, tokens, 4 buffers) followed by the sequence's pages of kq, ks, vq, vs in
+ * logical order. pack gathers them through the sequence's page-table row (device int32 [n_pages]) into `slot`
+ * (device, yahkv_slot_bytes); unpack scatters a slot into the pages named by a row (any free pages of pools with
+ * the same geometry); check validates a header on the host and returns the page and token counts.
+ * Follows the reference's slot, `{magic, T, B, chunks, nbufs}` + raw buffers, which loads only into the same set
+ * (engine/model/loom_prefill.hpp:976-1024). */
+size_t yahkv_slot_bytes(const yahkv_geometry* g, int32_t n_pages);
+int yahkv_slot_pack(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* table_row, int32_t n_pages,
+                    int32_t n_tokens, void* slot, void* stream);
+int yahkv_slot_check(const yahkv_geometry* g, const void* header, size_t slot_bytes, int32_t* n_pages,
+                     int32_t* n_tokens);
+int yahkv_slot_unpack(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* table_row, int32_t n_pages,
+                      const void* slot, void* stream);
 
 #ifdef __cplusplus
 }

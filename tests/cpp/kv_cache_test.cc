@@ -152,6 +152,45 @@ int main() {
     tiny.ResumeAt(0, 16);
     ExpectThrow([&] { tiny.Step(1, dk.get(), dv.get(), YAHKV_BF16, dq.get(), YAHKV_BF16, scale, nullptr, static_cast<float*>(dout.get())); },
                 "Step past the context must throw");
+    // ---- fork (shared prefix pages) and slot files
+    {
+      auto gathered = [&](KvDecoder& d, int seq) {
+        const size_t bytes = size_t(d.length(seq)) * H * (D / 32) * 34;
+        std::vector<uint8_t> k(bytes), v(bytes);
+        DeviceBuffer bk(bytes), bv(bytes);
+        const yahkv_pools pp{d.state().kq.ptr, d.state().ks.ptr, d.state().vq.ptr, d.state().vs.ptr};
+        d.Upload();
+        Check(yahkv_gather_blocks(&g, &pp, static_cast<const int32_t*>(d.state().ptab.ptr) + size_t(seq) * d.page_table_stride(),
+                                  d.length(seq), bk.get(), bv.get(), nullptr), "gather");
+        CheckHip(hipMemcpy(k.data(), bk.get(), bytes, hipMemcpyDeviceToHost), "d2h");
+        CheckHip(hipMemcpy(v.data(), bv.get(), bytes, hipMemcpyDeviceToHost), "d2h");
+        k.insert(k.end(), v.begin(), v.end());
+        return k;
+      };
+      dec.Release(1);
+      const int free0 = dec.free_pages();
+      const int len2 = dec.length(2), full = len2 / 16, partial = len2 % 16 != 0;
+      dec.Fork(2, 1);
+      Expect(dec.length(1) == len2 && dec.free_pages() == free0 - partial, "a fork takes one page at most");
+      for (int i = 0; i < full; ++i) Expect(dec.pages(1)[size_t(i)] == dec.pages(2)[size_t(i)], "full pages are shared");
+      if (partial) Expect(dec.pages(1).back() != dec.pages(2).back(), "the partly filled page is private");
+      Expect(gathered(dec, 1) == gathered(dec, 2), "a fork holds the same blocks");
+      dec.Release(2);  // the parent goes: the shared pages stay with the child
+      Expect(dec.free_pages() == free0 - partial + partial, "the parent's private page comes back");
+      const std::vector<uint8_t> child = gathered(dec, 1);
+      const std::string path = "/tmp/yahkv_kv_cache_test.slot";
+      dec.SaveSlot(1, path);
+      KvDecoder other(g, 2, T);
+      other.Bind(other.OwnState(7));
+      Expect(other.LoadSlot(1, path) == len2, "LoadSlot returns the tokens it covers");
+      Expect(gathered(other, 1) == child, "a loaded slot holds the same blocks");
+      yahkv_geometry g2 = g;
+      g2.page_tokens = 32;
+      KvDecoder wrong(g2, 1, T);
+      wrong.Bind(wrong.OwnState());
+      ExpectThrow([&] { wrong.LoadSlot(0, path); }, "a slot of another geometry must be refused");
+      std::remove(path.c_str());
+    }
     std::printf("kv_cache_test: ok (prefill %.2e, decode %.2e max relative error)\n", e1, e2);
     return 0;
   } catch (const std::exception& e) {

@@ -105,3 +105,25 @@ def test_page_allocator_invariants(yahkv):
             if k <= pool.free_count:
                 held += pool.alloc(k)
         assert len(set(held)) == len(held) and len(held) + pool.free_count == 64 and all(0 <= p < 64 for p in held)
+
+
+def test_page_owner_counts(yahkv):
+    """retain / free: a page returns to the free list only when its last owner lets go."""
+    pool = yahkv.PagePool(8)
+    a = pool.alloc(3)
+    assert [pool.refcount(p) for p in a] == [1, 1, 1] and pool.refcount(7) == 0 and pool.refcount(8) == -1
+    pool.retain(a[:2])                                   # a fork shares the first two pages
+    assert [pool.refcount(p) for p in a] == [2, 2, 1]
+    pool.free(a)                                         # the parent lets go: only the unshared page is free again
+    assert pool.free_count == 6 and [pool.refcount(p) for p in a] == [1, 1, 0]
+    with pytest.raises(yahkv.YahkvError) as e:
+        pool.retain([a[2]])                              # a free page cannot gain an owner
+    assert e.value.status == -3
+    with pytest.raises(yahkv.YahkvError) as e:
+        pool.free([a[0], a[0]])                          # the same page twice in one call
+    assert e.value.status == -3
+    pool.free(a[:2])
+    assert pool.free_count == 8
+    assert pool.alloc(8) == list(range(8))               # lowest id first again
+    assert yahkv.lib.yahkv_slot_bytes(__import__("ctypes").byref(yahkv.geometry(8, 24, 4, 256, 64, 4)), 3) == \
+        64 + 3 * sum(yahkv.pool_bytes(yahkv.geometry(8, 24, 4, 256, 64, 1)).values())

@@ -71,6 +71,14 @@ def _load():
     lib.yahkv_pagepool_alloc.argtypes = [vp, i32, i32p]
     lib.yahkv_pagepool_free.argtypes = [vp, i32p, i32]
     lib.yahkv_pagepool_shuffle.argtypes = [vp, C.c_uint64]
+    lib.yahkv_pagepool_retain.argtypes = [vp, i32p, i32]
+    lib.yahkv_pagepool_refcount.argtypes = [vp, i32]
+    lib.yahkv_copy_pages.argtypes = [G, P, i32p, i32p, i32, vp]
+    lib.yahkv_slot_bytes.restype = C.c_size_t
+    lib.yahkv_slot_bytes.argtypes = [G, i32]
+    lib.yahkv_slot_pack.argtypes = [G, P, i32p, i32, i32, vp, vp]
+    lib.yahkv_slot_check.argtypes = [G, vp, C.c_size_t, C.POINTER(C.c_int32), C.POINTER(C.c_int32)]
+    lib.yahkv_slot_unpack.argtypes = [G, P, i32p, i32, vp, vp]
     return lib
 
 
@@ -137,6 +145,13 @@ class PagePool:
 
     def shuffle(self, seed):
         lib.yahkv_pagepool_shuffle(self._p, seed)
+
+    def retain(self, pages):
+        arr = (C.c_int32 * max(len(pages), 1))(*pages)
+        _check(lib.yahkv_pagepool_retain(self._p, C.cast(arr, C.c_void_p), len(pages)), "pagepool_retain")
+
+    def refcount(self, page):
+        return lib.yahkv_pagepool_refcount(self._p, page)
 
 
 # ---- device side (torch supplies memory and the stream) --------------------------------------------------------------
@@ -305,6 +320,37 @@ def prefill_attend_tiles(pools, table, prefix_len, max_prefix_len, q, scale, out
                                           _dtype_code(out), _dp(workspace), workspace.numel(), _stream()),
            "prefill_attend_tiles")
     return out
+
+
+def copy_pages(pools, src_pages, dst_pages):
+    """Whole pages src_pages[i] -> dst_pages[i] (int32 cuda tensors) in all four pools."""
+    g, st = pools.geom, pools.struct()
+    _check(lib.yahkv_copy_pages(C.byref(g), C.byref(st), _dp(src_pages), _dp(dst_pages), src_pages.numel(), _stream()),
+           "copy_pages")
+
+
+def slot_pack(pools, table_row, n_pages, n_tokens):
+    """The first n_pages pages of a sequence (table_row: int32 cuda tensor) as one uint8 cuda tensor: header + pages."""
+    import torch
+    g, st = pools.geom, pools.struct()
+    slot = torch.empty(lib.yahkv_slot_bytes(C.byref(g), n_pages), dtype=torch.uint8, device=table_row.device)
+    _check(lib.yahkv_slot_pack(C.byref(g), C.byref(st), _dp(table_row), n_pages, n_tokens, _dp(slot), _stream()),
+           "slot_pack")
+    return slot
+
+
+def slot_check(g, slot_host):
+    """slot_host: numpy uint8 array of a whole slot; returns (n_pages, n_tokens) or raises."""
+    n_pages, n_tokens = C.c_int32(), C.c_int32()
+    _check(lib.yahkv_slot_check(C.byref(g), slot_host.ctypes.data, slot_host.nbytes, C.byref(n_pages),
+                                C.byref(n_tokens)), "slot_check")
+    return n_pages.value, n_tokens.value
+
+
+def slot_unpack(pools, table_row, n_pages, slot):
+    """Scatter a slot (uint8 cuda tensor) into the pages named by table_row[:n_pages]."""
+    g, st = pools.geom, pools.struct()
+    _check(lib.yahkv_slot_unpack(C.byref(g), C.byref(st), _dp(table_row), n_pages, _dp(slot), _stream()), "slot_unpack")
 
 
 def gather_blocks(pools, table_row, n_tokens):

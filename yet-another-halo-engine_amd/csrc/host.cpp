@@ -1,6 +1,7 @@
 // Host-only entry points of include/yahkv.h: geometry checks, pool sizes, page-table validation and the page allocator.
 #include <algorithm>
 #include <cstdint>
+#include <functional>
 #include <new>
 #include <vector>
 
@@ -57,29 +58,41 @@ size_t yahkv_bytes_per_token(const yahkv_geometry* g) {
   return size_t(2) * m.n_kv * m.nb() * (m.code_bytes() + 2);
 }
 
-int yahkv_validate_page_table(const yahkv_geometry* g, const int32_t* table, int32_t page_table_stride,
-                              const int32_t* seq_len, int32_t n_seqs) {
-  if (const int st = CheckGeometry(g)) return st;
+namespace {
+// owners == nullptr: a page may appear once in the whole table; else page p may appear at most owners[p] times, and
+// never twice in one row.
+int ValidateTable(const yahkv_geometry* g, const int32_t* table, int32_t page_table_stride, const int32_t* seq_len,
+                  int32_t n_seqs, const std::vector<int32_t>* owners) {
+  if (const int st = yahkv::CheckGeometry(g)) return st;
   if (table == nullptr || seq_len == nullptr || n_seqs <= 0 || page_table_stride <= 0) return YAHKV_ERR_ARG;
-  std::vector<bool> used(static_cast<size_t>(g->n_pages), false);
+  std::vector<int32_t> used(static_cast<size_t>(g->n_pages), 0), row_of(static_cast<size_t>(g->n_pages), -1);
   for (int32_t s = 0; s < n_seqs; ++s) {
     if (seq_len[s] < 0) return YAHKV_ERR_ARG;
     const int64_t np = (int64_t(seq_len[s]) + g->page_tokens - 1) / g->page_tokens;
     if (np > page_table_stride) return YAHKV_ERR_PAGE;
     for (int64_t p = 0; p < np; ++p) {
       const int32_t pg = table[int64_t(s) * page_table_stride + p];
-      if (pg < 0 || pg >= g->n_pages || used[static_cast<size_t>(pg)]) return YAHKV_ERR_PAGE;
-      used[static_cast<size_t>(pg)] = true;
+      if (pg < 0 || pg >= g->n_pages) return YAHKV_ERR_PAGE;
+      const size_t i = static_cast<size_t>(pg);
+      const int32_t limit = owners == nullptr ? 1 : (*owners)[i];
+      if (++used[i] > limit || row_of[i] == s) return YAHKV_ERR_PAGE;
+      row_of[i] = s;
     }
   }
   return YAHKV_OK;
+}
+}  // namespace
+
+int yahkv_validate_page_table(const yahkv_geometry* g, const int32_t* table, int32_t page_table_stride,
+                              const int32_t* seq_len, int32_t n_seqs) {
+  return ValidateTable(g, table, page_table_stride, seq_len, n_seqs, nullptr);
 }
 
 // ---- page allocator -------------------------------------------------------------------------------------------
 
 struct yahkv_pagepool {
   std::vector<int32_t> free_list;  // handed out from the back
-  std::vector<uint8_t> is_free;
+  std::vector<int32_t> refs;       // owners of a page; 0 = free
 };
 
 yahkv_pagepool* yahkv_pagepool_create(int32_t n_pages) {
@@ -88,7 +101,7 @@ yahkv_pagepool* yahkv_pagepool_create(int32_t n_pages) {
   if (p == nullptr) return nullptr;
   p->free_list.resize(static_cast<size_t>(n_pages));
   for (int32_t i = 0; i < n_pages; ++i) p->free_list[static_cast<size_t>(i)] = n_pages - 1 - i;  // lowest id first
-  p->is_free.assign(static_cast<size_t>(n_pages), 1);
+  p->refs.assign(static_cast<size_t>(n_pages), 0);
   return p;
 }
 
@@ -104,26 +117,51 @@ int yahkv_pagepool_alloc(yahkv_pagepool* p, int32_t n, int32_t* out) {
   for (int32_t i = 0; i < n; ++i) {
     out[i] = p->free_list.back();
     p->free_list.pop_back();
-    p->is_free[static_cast<size_t>(out[i])] = 0;
+    p->refs[static_cast<size_t>(out[i])] = 1;
   }
   return YAHKV_OK;
 }
 
+// One owner less for each page; a page goes back to the free list when its last owner lets go.
 int yahkv_pagepool_free(yahkv_pagepool* p, const int32_t* pages, int32_t n) {
   if (p == nullptr || n < 0 || (n > 0 && pages == nullptr)) return YAHKV_ERR_ARG;
-  const int32_t total = static_cast<int32_t>(p->is_free.size());
+  const int32_t total = static_cast<int32_t>(p->refs.size());
   for (int32_t i = 0; i < n; ++i) {  // check everything first: free none on error
-    if (pages[i] < 0 || pages[i] >= total || p->is_free[static_cast<size_t>(pages[i])]) return YAHKV_ERR_PAGE;
+    if (pages[i] < 0 || pages[i] >= total || p->refs[static_cast<size_t>(pages[i])] <= 0) return YAHKV_ERR_PAGE;
     for (int32_t j = 0; j < i; ++j)
       if (pages[j] == pages[i]) return YAHKV_ERR_PAGE;
   }
+  bool any = false;
   for (int32_t i = 0; i < n; ++i) {
-    p->is_free[static_cast<size_t>(pages[i])] = 1;
-    p->free_list.push_back(pages[i]);
+    if (--p->refs[static_cast<size_t>(pages[i])] == 0) {
+      p->free_list.push_back(pages[i]);
+      any = true;
+    }
   }
   // keep "lowest id first": the back of the list is the smallest free id
-  std::sort(p->free_list.begin(), p->free_list.end(), [](int32_t a, int32_t b) { return a > b; });
+  if (any) std::sort(p->free_list.begin(), p->free_list.end(), std::greater<int32_t>());
   return YAHKV_OK;
+}
+
+// One owner more for each page (a sequence forked from a shared prefix keeps the prefix's full pages).
+int yahkv_pagepool_retain(yahkv_pagepool* p, const int32_t* pages, int32_t n) {
+  if (p == nullptr || n < 0 || (n > 0 && pages == nullptr)) return YAHKV_ERR_ARG;
+  const int32_t total = static_cast<int32_t>(p->refs.size());
+  for (int32_t i = 0; i < n; ++i)
+    if (pages[i] < 0 || pages[i] >= total || p->refs[static_cast<size_t>(pages[i])] <= 0) return YAHKV_ERR_PAGE;
+  for (int32_t i = 0; i < n; ++i) ++p->refs[static_cast<size_t>(pages[i])];
+  return YAHKV_OK;
+}
+
+int yahkv_validate_shared_page_table(const yahkv_geometry* g, const yahkv_pagepool* p, const int32_t* table,
+                                     int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs) {
+  if (p == nullptr || g == nullptr || static_cast<int64_t>(p->refs.size()) != g->n_pages) return YAHKV_ERR_ARG;
+  return ValidateTable(g, table, page_table_stride, seq_len, n_seqs, &p->refs);
+}
+
+int32_t yahkv_pagepool_refcount(const yahkv_pagepool* p, int32_t page) {
+  if (p == nullptr || page < 0 || page >= static_cast<int32_t>(p->refs.size())) return -1;
+  return p->refs[static_cast<size_t>(page)];
 }
 
 void yahkv_pagepool_shuffle(yahkv_pagepool* p, uint64_t seed) {

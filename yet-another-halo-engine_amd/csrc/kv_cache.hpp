@@ -17,6 +17,7 @@
 
 #include <algorithm>
 #include <cstdint>
+#include <cstdio>
 #include <cstring>
 #include <memory>
 #include <stdexcept>
@@ -94,6 +95,11 @@ class PagePool {
     Check(yahkv_pagepool_free(p_, pages.data(), static_cast<int32_t>(pages.size())), "page pool");
   }
   void Shuffle(uint64_t seed) { yahkv_pagepool_shuffle(p_, seed); }
+  void Retain(const std::vector<int32_t>& pages) {
+    Check(yahkv_pagepool_retain(p_, pages.data(), static_cast<int32_t>(pages.size())), "page pool");
+  }
+  int32_t owners(int32_t page) const { return yahkv_pagepool_refcount(p_, page); }
+  const yahkv_pagepool* handle() const { return p_; }
 
  private:
   yahkv_pagepool* p_;
@@ -182,6 +188,80 @@ class KvDecoder {
     pg.clear();
     len_[size_t(seq)] = 0;
   }
+  // Sequence `dst` (empty) becomes a copy of `src` that shares its full pages; the last, partly filled page is copied,
+  // so both can go on appending. (The reference reuses a prefix by loading a saved slot, loom_prefill.hpp:976-1024.)
+  void Fork(int32_t src, int32_t dst) {
+    if (!bound_) throw KvError("decoder: no state bound");
+    if (src == dst || !pages_.at(size_t(dst)).empty()) throw KvError("decoder: fork needs an empty target sequence");
+    const auto& from = pages_.at(size_t(src));
+    const int32_t len = len_[size_t(src)], full = len / g_.page_tokens;
+    std::vector<int32_t> shared(from.begin(), from.begin() + full);
+    pool_->Retain(shared);
+    auto& to = pages_[size_t(dst)];
+    to = shared;
+    if (len % g_.page_tokens != 0) {
+      const std::vector<int32_t> own = pool_->Alloc(1);
+      const int32_t pair[2] = {from[size_t(full)], own[0]};
+      DeviceBuffer ids(sizeof pair);
+      CheckHip(hipMemcpyAsync(ids.get(), pair, sizeof pair, hipMemcpyHostToDevice, stream_), "fork");
+      const yahkv_pools pools{st_.kq.ptr, st_.ks.ptr, st_.vq.ptr, st_.vs.ptr};
+      Check(yahkv_copy_pages(&g_, &pools, static_cast<const int32_t*>(ids.get()),
+                             static_cast<const int32_t*>(ids.get()) + 1, 1, stream_), "copy_pages");
+      CheckHip(hipStreamSynchronize(stream_), "fork");  // `ids` and `pair` go out of scope
+      to.push_back(own[0]);
+    }
+    for (size_t i = 0; i < to.size(); ++i) table_[size_t(dst) * stride_ + i] = to[i];
+    len_[size_t(dst)] = len;
+    table_dirty_ = true;
+  }
+
+  // A sequence's state as a slot file: the 64-byte header and the sequence's pages, raw (yahkv_slot_pack); LoadSlot
+  // puts it into free pages of this decoder and returns the tokens it covers, so the caller continues at that
+  // position (SaveState / LoadState, loom_prefill.hpp:979-1019).
+  void SaveSlot(int32_t seq, const std::string& path) {
+    if (!bound_) throw KvError("decoder: no state bound");
+    const auto& pg = pages_.at(size_t(seq));
+    const int32_t len = len_[size_t(seq)], np = (len + g_.page_tokens - 1) / g_.page_tokens;
+    if (np <= 0) throw KvError("decoder: nothing to save");
+    Upload();
+    const size_t bytes = yahkv_slot_bytes(&g_, np);
+    DeviceBuffer slot(bytes);
+    const yahkv_pools pools{st_.kq.ptr, st_.ks.ptr, st_.vq.ptr, st_.vs.ptr};
+    Check(yahkv_slot_pack(&g_, &pools, static_cast<const int32_t*>(st_.ptab.ptr) + size_t(seq) * stride_, np, len,
+                          slot.get(), stream_), "slot_pack");
+    std::vector<uint8_t> host(bytes);
+    CheckHip(hipMemcpyAsync(host.data(), slot.get(), bytes, hipMemcpyDeviceToHost, stream_), "slot");
+    CheckHip(hipStreamSynchronize(stream_), "slot");
+    FILE* f = std::fopen(path.c_str(), "wb");
+    if (f == nullptr) throw KvError("decoder: cannot write the slot " + path);
+    const bool ok = std::fwrite(host.data(), 1, bytes, f) == bytes;
+    if (std::fclose(f) != 0 || !ok) throw KvError("decoder: short write to the slot " + path);
+    (void)pg;
+  }
+  int32_t LoadSlot(int32_t seq, const std::string& path) {
+    if (!bound_) throw KvError("decoder: no state bound");
+    if (!pages_.at(size_t(seq)).empty()) throw KvError("decoder: a slot loads into an empty sequence");
+    FILE* f = std::fopen(path.c_str(), "rb");
+    if (f == nullptr) throw KvError("decoder: cannot open the slot " + path);
+    std::vector<uint8_t> host;
+    uint8_t buf[1 << 16];
+    for (size_t n; (n = std::fread(buf, 1, sizeof buf, f)) > 0;) host.insert(host.end(), buf, buf + n);
+    std::fclose(f);
+    int32_t np = 0, len = 0;
+    if (yahkv_slot_check(&g_, host.data(), host.size(), &np, &len) != YAHKV_OK)
+      throw KvError("decoder: the slot " + path + " does not match this geometry");
+    Reserve(seq, len);
+    Upload();
+    DeviceBuffer slot(host.size());
+    CheckHip(hipMemcpyAsync(slot.get(), host.data(), host.size(), hipMemcpyHostToDevice, stream_), "slot");
+    const yahkv_pools pools{st_.kq.ptr, st_.ks.ptr, st_.vq.ptr, st_.vs.ptr};
+    Check(yahkv_slot_unpack(&g_, &pools, static_cast<const int32_t*>(st_.ptab.ptr) + size_t(seq) * stride_, np,
+                            slot.get(), stream_), "slot_unpack");
+    CheckHip(hipStreamSynchronize(stream_), "slot");
+    len_[size_t(seq)] = len;
+    return len;
+  }
+
   // The next Step of `seq` writes position pos (after a prefill that filled positions 0 .. pos - 1; loom_decoder.hpp:145).
   void ResumeAt(int32_t seq, int32_t pos) {
     Reserve(seq, pos);
@@ -221,7 +301,8 @@ class KvDecoder {
   // Validates and uploads the page table if it changed (loom_prefill.hpp:1306-1319).
   void Upload() {
     if (!table_dirty_) return;
-    Check(yahkv_validate_page_table(&g_, table_.data(), stride_, PagesAsLengths().data(), max_seqs_), "page table");
+    Check(yahkv_validate_shared_page_table(&g_, pool_->handle(), table_.data(), stride_, PagesAsLengths().data(),
+                                           max_seqs_), "page table");
     CheckHip(hipMemcpyAsync(st_.ptab.ptr, table_.data(), sizeof(int32_t) * table_.size(), hipMemcpyHostToDevice, stream_),
              "page table upload");
     // the host table may be edited again only after this copy has run
