@@ -17,6 +17,7 @@
 // global memory or by the dispatcher, to even out the XCDs, which finish up to 10 % apart. Every variant was slower:
 // each change of pair costs a wave a pipeline fill, and the XCDs that finish first leave their bandwidth to the rest.)
 #include <algorithm>
+#include <cstdio>
 #include <cstdlib>
 
 #include "common.hpp"
@@ -51,15 +52,30 @@ struct DecodeArgs {
   float* acc;        // [(n_chunks + n_seqs * H) * wpc][G][D]
   int32_t n_chunks, wpc;  // chunks = workgroups launched; waves per chunk
   int32_t min_chunk_tiles;
+  int32_t share[9];  // cumulative shares of the eight chunks of a group, in 1/8192 of the group (share[8] = 8192)
 };
 
 __device__ __forceinline__ int ClampLen(const DecodeArgs& a, int s) { return min(max(a.seq_len[s], 0), a.max_len); }
+
+// The line of tiles is cut into groups of eight chunks, 8 A tiles a group; chunk j of a group takes the tiles
+// [share[j], share[j + 1]) / 8192 of it. Workgroup k runs on XCD k % 8 and the XCDs do not read memory equally
+// fast, so the shares follow their speeds and the workgroups finish together.
+__device__ __forceinline__ long long ChunkStart(const DecodeArgs& a, long long A, int k) {
+  return (k / 8) * 8 * A + 8 * A * a.share[k % 8] / 8192;
+}
+__device__ __forceinline__ int ChunkOf(const DecodeArgs& a, long long A, long long tile) {
+  const long long r = tile % (8 * A);
+  int j = 0;
+#pragma unroll
+  for (int i = 1; i < 8; ++i) j += 8 * A * a.share[i] / 8192 <= r;
+  return static_cast<int>(tile / (8 * A)) * 8 + j;
+}
 
 // ---- plan -------------------------------------------------------------------------------------------------------------
 
 // Every workgroup recomputes the prefix sums of the sequences' tile counts in LDS (a few hundred integers), then each
 // thread writes one chunk record. Workgroup 0 also publishes the prefix sums and the chunk size. Chunk k covers tiles
-// [k A, (k + 1) A) of the line, clipped to the line's length.
+// [ChunkStart(k), ChunkStart(k + 1)) of the line, clipped to the line's length: A tiles on average.
 __global__ __launch_bounds__(kPlanThreads) void DattnPlan(const DecodeArgs a) {
   extern __shared__ int lpre[];  // [n_seqs + 1]
   __shared__ int part_sum[kPlanThreads / 64];
@@ -98,8 +114,8 @@ __global__ __launch_bounds__(kPlanThreads) void DattnPlan(const DecodeArgs a) {
   }
   const int k = blockIdx.x * kPlanThreads + t;
   if (k >= a.n_chunks) return;
-  const long long start = k * A;
-  if (start >= line) {
+  const long long start = ChunkStart(a, A, k), end = min(ChunkStart(a, A, k + 1), line);
+  if (start >= end) {
     a.chunks[k] = int4{-1, 0, 0, 0};
     return;
   }
@@ -110,7 +126,7 @@ __global__ __launch_bounds__(kPlanThreads) void DattnPlan(const DecodeArgs a) {
   }
   const int ts = lpre[lo + 1] - lpre[lo];
   const int r = static_cast<int>(start - static_cast<long long>(lpre[lo]) * H);
-  a.chunks[k] = int4{lo, r / ts, r % ts, static_cast<int>(min(A, line - start))};
+  a.chunks[k] = int4{lo, r / ts, r % ts, static_cast<int>(end - start)};
 }
 
 // Position of a wave on its chunk: the pair (s, h) it stands on, which of the chunk's tiles belong to that pair
@@ -296,9 +312,14 @@ void DattnPart(const DecodeArgs a) {
 
   PairCursor cur = FirstPair(a, rec);
   const int32_t* row = nullptr;
+  // The page table is read through the constant address space: nothing writes it while the kernel runs, and only
+  // then does the compiler use scalar loads, which the vector memory counter does not see. As ordinary global loads
+  // they would sit behind the K and V loads already in flight and drain that queue once per tile.
+  typedef const int32_t __attribute__((address_space(4))) * ConstRow;
   auto load_pages = [&](int tile, int (&pg)[PPT]) {
+    const ConstRow crow = (ConstRow)(reinterpret_cast<uintptr_t>(row));
 #pragma unroll
-    for (int j = 0; j < PPT; ++j) pg[j] = ClampPage(row[min(tile * PPT + j, a.stride - 1)], g.n_pages);
+    for (int j = 0; j < PPT; ++j) pg[j] = ClampPage(crow[min(tile * PPT + j, a.stride - 1)], g.n_pages);
   };
   auto page_head = [&](const int (&pg)[PPT], int tok_in_tile) -> size_t {  // (page, kv head) index of a key of the tile
     int p = pg[0];
@@ -306,21 +327,26 @@ void DattnPart(const DecodeArgs a) {
     for (int j = 1; j < PPT; ++j) p = tok_in_tile / PT == j ? pg[j] : p;
     return size_t(p) * H + cur.h;
   };
+  // Addresses are a base per (page, kv head), which is the same for the whole wave when a tile is one page, plus a
+  // 32-bit offset per lane: the form the scalar-base addressing mode of the global loads takes.
+  constexpr uint32_t KB = Q8 ? 32 : 16;  // bytes of K codes per key and block
   auto load_k = [&](int tt, const int (&pg)[PPT]) {
     const int tk = 32 * tt + n32;
     const size_t ph = page_head(pg, tk);
-    const int t = tk % PT;
+    const uint32_t t = tk % PT;
+    const uint8_t* kp = a.pools.kq + ph * (NB * PT * KB);
+    const uint32_t off = t * KB + (KB / 2) * half;
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
       if constexpr (Q8) {
-        const uint4 v = *reinterpret_cast<const uint4*>(a.pools.kq + ((ph * NB + b) * PT + t) * 32 + 16 * half);
+        const uint4 v = *reinterpret_cast<const uint4*>(kp + (b * PT * KB + off));
         kb[b][0] = v.x, kb[b][1] = v.y, kb[b][2] = v.z, kb[b][3] = v.w;
       } else {
-        const uint2 v = *reinterpret_cast<const uint2*>(a.pools.kq + ((ph * NB + b) * PT + t) * 16 + 8 * half);
+        const uint2 v = *reinterpret_cast<const uint2*>(kp + (b * PT * KB + off));
         kb[b][0] = v.x, kb[b][1] = v.y;
       }
     }
-    const uint16_t* sp = a.pools.ks + (ph * PT + t) * NB;
+    const uint8_t* sp = reinterpret_cast<const uint8_t*>(a.pools.ks) + ph * (PT * NB * 2) + t * (NB * 2);
     if (NB == 8) {
       ksc = *reinterpret_cast<const uint4*>(sp);
     } else {
@@ -330,19 +356,16 @@ void DattnPart(const DecodeArgs a) {
   };
   auto load_v = [&](int hf, const int (&pg)[PPT]) {
     const size_t ph = page_head(pg, 16 * kg);
-    const int t0 = (16 * kg) % PT;
+    const uint32_t off = n16 * PT + (16 * kg) % PT;
+    const uint8_t* vp = a.pools.vq + ph * (Q8 ? D * PT : NB * 16 * PT);
 #pragma unroll
-    for (int j = 0; j < NVB; ++j) {
-      if constexpr (Q8)
-        vb[j] = *reinterpret_cast<const uint4*>(a.pools.vq + (ph * D + 16 * (hf * NVB + j) + n16) * PT + t0);
-      else
-        vb[j] = *reinterpret_cast<const uint4*>(a.pools.vq + ((ph * NB + hf * NVB + j) * 16 + n16) * PT + t0);
-    }
+    for (int j = 0; j < NVB; ++j) vb[j] = *reinterpret_cast<const uint4*>(vp + (16 * (hf * NVB + j) * PT + off));
     if (hf == 0) {  // with the first half come the tile's V scales: lane = (block, 8 keys)
       const int b = lane / 8, chunk = lane % 8;
       if (b < NB) {
         const size_t ps = page_head(pg, 8 * chunk);
-        vsr = *reinterpret_cast<const uint4*>(a.pools.vs + (ps * NB + b) * PT + (8 * chunk) % PT);
+        const uint32_t soff = (b * PT + (8 * chunk) % PT) * 2;
+        vsr = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint8_t*>(a.pools.vs) + ps * (NB * PT * 2) + soff);
       }
     }
   };
@@ -457,7 +480,8 @@ void DattnPart(const DecodeArgs a) {
     int pgc[PPT], pgn[PPT];
     load_pages(tile, pgc);
     load_k(0, pgc);
-    load_v(0, pgc);
+    load_v(1, pgc);  // not used (the first pass has no previous tile): it keeps the count of loads in flight at the
+                     // head of the loop the same as on the way round, see below
 #pragma unroll
     for (int e = 0; e < QE; ++e) {
       const int i = lane + 64 * e;
@@ -474,16 +498,18 @@ void DattnPart(const DecodeArgs a) {
       const int nidx = take();
       const bool has_next = nidx < cur.base + cur.n;  // the wave's next tile is in the same pair
       const int ntile = cur.first + (nidx - cur.base);
-      if (has_next) load_pages(ntile, pgn);
+      // Every pass issues the same loads whether or not the wave has a next tile in this pair (without one it
+      // reads the first half of this tile's K again and drops it): the compiler counts outstanding loads along
+      // every path into a wait and takes the smallest, so a load issued on one path only turns the waits after the
+      // join into waits for everything.
+      load_pages(has_next ? ntile : tile, pgn);
       scores(0);
       load_k(1, pgc);
-      if (!first) {
-        pv(1);  // second half of the previous tile's P.V: lp and lvs still hold that tile
-        load_v(0, pgc);
-      }
+      if (!first) pv(1);  // second half of the previous tile's P.V: lp and lvs still hold that tile
+      load_v(0, pgc);
       first = false;
       scores(1);
-      if (has_next) load_k(0, pgn);
+      load_k(0, pgn);
       // ---- online softmax (base 2); keys at or past len are masked by select, so stale scales cannot leak
       float alpha[4];
 #pragma unroll
@@ -543,56 +569,92 @@ void DattnPart(const DecodeArgs a) {
 
 // ---- reduce -------------------------------------------------------------------------------------------------------------
 
-// One workgroup per (query head, sequence), thread = dim (gen_decode_attn.py:338-411). The pair's partials are those
-// of the waves of the chunks its stretch of the line overlaps; their weights e^(M_p - M) are computed once per
-// workgroup, by one thread each, so that the sum over partials is a loop of independent loads.
-constexpr int kReduceBatch = 256;  // partial slots weighed at a time
-__global__ void DattnReduce(const DecodeArgs a) {
+// One workgroup per (query head, sequence) (gen_decode_attn.py:338-411). The pair's partials are those of the waves
+// of the chunks its stretch of the line overlaps. Their weights e^(M_p - M) are computed once per workgroup, by one
+// thread each, and the partials that weigh something are listed in order. The threads then form groups of D / 4
+// lanes (four dims a lane); each group sums every n-th listed partial, several 16-byte loads in flight and no
+// branch inside, and the groups' sums meet in LDS. A single long sequence leaves hundreds of partials per pair and
+// only a few workgroups here, which is why the partials are spread over the workgroup as well.
+constexpr int kReduceThreads = 256;  // also the number of partial slots weighed at a time
+constexpr int kReduceDepth = 4;      // partials a group loads together
+__global__ __launch_bounds__(kReduceThreads) void DattnReduce(const DecodeArgs a) {
   const Geom g = a.g;
   const int G = g.group(), H = g.n_kv, D = g.hd;
-  const int hq = blockIdx.x, s = blockIdx.y, d = threadIdx.x;
+  const int hq = blockIdx.x, s = blockIdx.y, t = threadIdx.x;
   const int h = hq / G, gi = hq % G;
-  const size_t o = (size_t(s) * g.n_q + hq) * D + d;
+  const size_t o = (size_t(s) * g.n_q + hq) * D;
   const int ts = a.tprefix[s + 1] - a.tprefix[s];
   if (ts <= 0) {  // length 0
-    a.out[o] = 0.0f;
+    if (t < D) a.out[o + t] = 0.0f;
     return;
   }
   const int A_ = a.header[1], pair = s * H + h;
   const long long first = static_cast<long long>(a.tprefix[s]) * H + static_cast<long long>(h) * ts;
-  const int k0 = static_cast<int>(first / A_), k1 = static_cast<int>((first + ts - 1) / A_);
+  const int k0 = ChunkOf(a, A_, first), k1 = ChunkOf(a, A_, first + ts - 1);
   const size_t p0 = size_t(k0 + pair) * a.wpc, p1 = size_t(k1 + pair + 1) * a.wpc;
-  __shared__ float wgt[kReduceBatch];
-  __shared__ float red[4];
+  constexpr int NW = kReduceThreads / 64;
+  __shared__ float wgt[kReduceThreads], wl[kReduceThreads];
+  __shared__ int slot[kReduceThreads];
+  __shared__ float red[NW];
+  __shared__ int wave_n[NW];
+  __shared__ __align__(16) float sums[kReduceThreads * 4];  // [group][D]
+  __shared__ float lsums[kReduceThreads / 32];
   // waves that got no tile of this pair left l = 0 (and no acc): they weigh nothing
   float M = kNegMax;
-  for (size_t p = p0 + d; p < p1; p += D)
+  for (size_t p = p0 + t; p < p1; p += kReduceThreads)
     if (a.ml[(p * G + gi) * 2 + 1] > 0.0f) M = fmaxf(M, a.ml[(p * G + gi) * 2]);
   M = WaveMax(M);
-  if (d % 64 == 0) red[d / 64] = M;
+  if (t % 64 == 0) red[t / 64] = M;
   __syncthreads();
   M = red[0];
-  for (int w = 1; w < D / 64; ++w) M = fmaxf(M, red[w]);
-  float L = 0.0f, A = 0.0f;
-  for (size_t b0 = p0; b0 < p1; b0 += kReduceBatch) {
-    const int nb = static_cast<int>(min(p1 - b0, size_t(kReduceBatch)));
+  for (int w = 1; w < NW; ++w) M = fmaxf(M, red[w]);
+  const int lanes = D / 4, n_groups = kReduceThreads / lanes, grp = t / lanes, dl = t % lanes;
+  float L = 0.0f;
+  float4 A = {0.0f, 0.0f, 0.0f, 0.0f};
+  for (size_t b0 = p0; b0 < p1; b0 += kReduceThreads) {
+    const int nb = static_cast<int>(min(p1 - b0, size_t(kReduceThreads)));
+    float l = 0.0f, m = 0.0f;
+    if (t < nb) l = a.ml[((b0 + t) * G + gi) * 2 + 1], m = a.ml[((b0 + t) * G + gi) * 2];
+    const unsigned long long mask = __ballot(l > 0.0f);
+    __syncthreads();  // the previous batch's lists have been read
+    if (t % 64 == 0) wave_n[t / 64] = __popcll(mask);
     __syncthreads();
-    for (int i = d; i < nb; i += D) {
-      const float l = a.ml[((b0 + i) * G + gi) * 2 + 1];
-      wgt[i] = l > 0.0f ? __expf(a.ml[((b0 + i) * G + gi) * 2] - M) : 0.0f;
+    int at = __popcll(mask & ((1ull << (t % 64)) - 1)), n = 0;  // n: partials of this batch that weigh something
+    for (int w = 0; w < NW; ++w) {
+      if (w < t / 64) at += wave_n[w];
+      n += wave_n[w];
+    }
+    if (l > 0.0f) {
+      const float w = __expf(m - M);
+      wgt[at] = w, wl[at] = w * l, slot[at] = t;
     }
     __syncthreads();
-    for (int i = 0; i < nb; ++i) {
-      const float w = wgt[i];
-      if (w > 0.0f) {  // uniform over the workgroup
-        L = __builtin_fmaf(w, a.ml[((b0 + i) * G + gi) * 2 + 1], L);
-        A = __builtin_fmaf(w, a.acc[((b0 + i) * G + gi) * D + d], A);
+    for (int j0 = grp * kReduceDepth; j0 < n; j0 += n_groups * kReduceDepth) {
+      float4 v[kReduceDepth];
+#pragma unroll
+      for (int j = 0; j < kReduceDepth; ++j)
+        v[j] = *reinterpret_cast<const float4*>(&a.acc[((b0 + slot[min(j0 + j, n - 1)]) * G + gi) * D + 4 * dl]);
+#pragma unroll
+      for (int j = 0; j < kReduceDepth; ++j) {
+        if (j0 + j < n) {
+          const float w = wgt[j0 + j];
+          A.x = __builtin_fmaf(w, v[j].x, A.x), A.y = __builtin_fmaf(w, v[j].y, A.y);
+          A.z = __builtin_fmaf(w, v[j].z, A.z), A.w = __builtin_fmaf(w, v[j].w, A.w);
+          L += wl[j0 + j];
+        }
       }
     }
   }
-  float v = A / L;
-  if (a.gate != nullptr) v *= 1.0f / (1.0f + __expf(-a.gate[o]));
-  a.out[o] = v;
+  *reinterpret_cast<float4*>(&sums[grp * D + 4 * dl]) = A;
+  if (dl == 0) lsums[grp] = L;
+  __syncthreads();
+  if (t < D) {
+    float v = 0.0f, lt = 0.0f;
+    for (int q = 0; q < n_groups; ++q) v += sums[q * D + t], lt += lsums[q];
+    v /= lt;
+    if (a.gate != nullptr) v *= 1.0f / (1.0f + __expf(-a.gate[o + t]));
+    a.out[o + t] = v;
+  }
 }
 
 // ---- host side ----------------------------------------------------------------------------------------------------------
@@ -600,6 +662,7 @@ __global__ void DattnReduce(const DecodeArgs a) {
 // Workspace layout and chunk count, from the host's bounds alone (the lengths are on the device).
 struct Plan {
   int32_t max_len, n_chunks, wpc, min_chunk_tiles;
+  int32_t share[9];
   size_t off_tprefix, off_chunks, off_ml, off_acc, bytes;
 };
 size_t Align(size_t x) { return (x + 255) & ~size_t(255); }
@@ -629,6 +692,23 @@ Plan MakePlan(const Geom& g, int32_t n_seqs, int32_t max_seq_len) {
   p.n_chunks = EnvInt("YAHKV_DECODE_CHUNKS", ComputeUnits(), 1, 1 << 20);
   p.n_chunks =
       static_cast<int32_t>(std::min<int64_t>(p.n_chunks, (line_max + p.min_chunk_tiles - 1) / p.min_chunk_tiles));
+  // Relative speeds of the eight XCDs of an MI355X on this kernel (tiles per unit of time, measured with all of
+  // them reading at once); YAHKV_DECODE_XCD_WEIGHTS="w0,...,w7" overrides them. Shares are kept above half the mean.
+  int w[8] = {1037, 895, 1084, 999, 1065, 980, 1037, 905};
+  if (const char* e = std::getenv("YAHKV_DECODE_XCD_WEIGHTS")) {
+    int v[8];
+    if (std::sscanf(e, "%d,%d,%d,%d,%d,%d,%d,%d", v, v + 1, v + 2, v + 3, v + 4, v + 5, v + 6, v + 7) == 8)
+      std::copy(v, v + 8, w);
+  }
+  if (p.n_chunks % 8 != 0) std::fill(w, w + 8, 1);  // a last group that is not whole would leave the line's end uncovered
+  int64_t sum = 0;
+  for (int j = 0; j < 8; ++j) w[j] = std::max(w[j], 1), sum += w[j];
+  for (int j = 0; j < 8; ++j) w[j] = static_cast<int>(std::max<int64_t>(w[j] * 8192 / sum, 512));
+  sum = 0;
+  for (int j = 0; j < 8; ++j) sum += w[j];
+  p.share[0] = 0;
+  for (int j = 0; j < 8; ++j) p.share[j + 1] = p.share[j] + static_cast<int32_t>(w[j] * 8192 / sum);
+  p.share[8] = 8192;
   const size_t parts = (size_t(p.n_chunks) + size_t(n_seqs) * g.n_kv) * p.wpc;
   p.off_tprefix = 256;
   p.off_chunks = Align(p.off_tprefix + sizeof(int32_t) * (size_t(n_seqs) + 1));
@@ -660,6 +740,7 @@ int Prepare(const yahkv_geometry* g, int32_t page_table_stride, const int32_t* s
   a->ml = reinterpret_cast<float*>(ws + p.off_ml);
   a->acc = reinterpret_cast<float*>(ws + p.off_acc);
   a->n_chunks = p.n_chunks, a->wpc = p.wpc, a->min_chunk_tiles = p.min_chunk_tiles;
+  std::copy(p.share, p.share + 9, a->share);
   return YAHKV_OK;
 }
 
@@ -730,7 +811,7 @@ extern "C" int yahkv_decode_reduce(const yahkv_geometry* g, int32_t page_table_s
     return st;
   if (out == nullptr) return YAHKV_ERR_ARG;
   a.gate = gate, a.out = out;
-  hipLaunchKernelGGL(DattnReduce, dim3(a.g.n_q, n_seqs), dim3(a.g.hd), 0, static_cast<hipStream_t>(stream), a);
+  hipLaunchKernelGGL(DattnReduce, dim3(a.g.n_q, n_seqs), dim3(kReduceThreads), 0, static_cast<hipStream_t>(stream), a);
   return LaunchStatus();
 }
 
