@@ -24,7 +24,9 @@ HBM_PEAK_GBS = 8000.0
 WORKLOADS = {
     # name: (format, batch, lo, hi, outlier channels)
     "ragged_b64_q8_0": dict(fmt=8, batch=64, lo=1024, hi=65536, seed=4),
-    "b1_ctx32k_q8_0": dict(fmt=8, batch=1, lo=32768, hi=32768, seed=4),
+    # one sequence's KV (71 MB) would stay in the 256 MB last-level cache from step to step: the steps rotate over
+    # eight layers' pools, as the layers of a model do
+    "b1_ctx32k_q8_0": dict(fmt=8, batch=1, lo=32768, hi=32768, seed=4, layers=8),
     "b16_ctx128k_q4_0": dict(fmt=4, batch=16, lo=131072, hi=131072, seed=4, outliers=8),
     # chunked prefill: every sequence holds `lo` tokens and takes a chunk of `chunk` more per step
     "prefill_b8_ctx16k_chunk2k_q8_0": dict(fmt=8, batch=8, lo=16384, hi=16384, seed=4, chunk=2048),
@@ -59,7 +61,7 @@ def build_state(yahkv, torch, wl, total_steps):
         table[s, :n] = alloc.alloc(int(n))
     assert alloc.free_count == 0
     yahkv.validate_page_table(g, table, lens + total_steps)
-    pools = yahkv.DevicePools(g)
+    layers = [yahkv.DevicePools(g) for _ in range(wl.get("layers", 1))]
     t_table = torch.from_numpy(table).cuda()
     gen = torch.Generator(device="cuda").manual_seed(wl["seed"])
     chunk = 8192
@@ -68,17 +70,18 @@ def build_state(yahkv, torch, wl, total_steps):
         outl = torch.ones(NKV, HD, device="cuda")
         for h in range(NKV):
             outl[h, torch.from_numpy(rng.permutation(HD)[:wl["outliers"]]).cuda()] = 20.0
-    for s in range(wl["batch"]):                     # fill the prefix through the library's own append
-        for o in range(0, int(lens[s]), chunk):
-            n = min(chunk, int(lens[s]) - o)
-            k = torch.randn((1, n, NKV, HD), generator=gen, device="cuda", dtype=torch.float32)
-            if outl is not None:
-                k = k * outl
-            v = torch.randn((1, n, NKV, HD), generator=gen, device="cuda", dtype=torch.float32)
-            yahkv.append(pools, t_table[s:s + 1], torch.tensor([o], dtype=torch.int32, device="cuda"),
-                         k.to(torch.bfloat16), v.to(torch.bfloat16))
+    for pools in layers:                             # fill the prefix through the library's own append
+        for s in range(wl["batch"]):
+            for o in range(0, int(lens[s]), chunk):
+                n = min(chunk, int(lens[s]) - o)
+                k = torch.randn((1, n, NKV, HD), generator=gen, device="cuda", dtype=torch.float32)
+                if outl is not None:
+                    k = k * outl
+                v = torch.randn((1, n, NKV, HD), generator=gen, device="cuda", dtype=torch.float32)
+                yahkv.append(pools, t_table[s:s + 1], torch.tensor([o], dtype=torch.int32, device="cuda"),
+                             k.to(torch.bfloat16), v.to(torch.bfloat16))
     torch.cuda.synchronize()
-    return g, pools, lens, table, t_table, gen
+    return g, layers, lens, table, t_table, gen
 
 
 def parity_check(yahkv, torch, g, pools, t_table, lens, q, out, scale, rows):
@@ -172,7 +175,8 @@ def prefill_cpu_baseline(wl, scale, prefix=2048, chunk=64):
 
 def run_prefill(a, wl, torch, yahkv):
     """A step: quantize + scatter one chunk per sequence, decode prefix + chunk to bf16 tiles, causal attention."""
-    g, pools, lens, table, t_table, gen = build_state(yahkv, torch, wl, 0)
+    g, layers, lens, table, t_table, gen = build_state(yahkv, torch, wl, 0)
+    pools = layers[0]
     B, chunk, prefix = wl["batch"], wl["chunk"], int(lens.max())
     scale = 1.0 / float(np.sqrt(HD))
     t_prefix = torch.from_numpy(lens).cuda()
@@ -272,7 +276,8 @@ def main():
     if "chunk" in wl:
         return run_prefill(a, wl, torch, yahkv)
     total = a.warmup + a.steps + 1
-    g, pools, lens, table, t_table, gen = build_state(yahkv, torch, wl, total)
+    g, layers, lens, table, t_table, gen = build_state(yahkv, torch, wl, total)
+    pools = layers[0]
     B = wl["batch"]
     scale = 1.0 / float(np.sqrt(HD))
     max_len = int(lens.max()) + total
@@ -288,6 +293,7 @@ def main():
 
     def step(i, pair=None):
         seq_len = len_rows[i + 1]
+        pools = layers[i % len(layers)]     # (with several layers a layer sees every n-th token; the others stay zero blocks)
         yahkv.append(pools, t_table, len_rows[i], knew[i], vnew[i])    # position = current length (device-resident)
         yahkv.decode_plan(g, t_table.shape[1], seq_len, B, max_len, ws)
         if pair:
@@ -331,7 +337,7 @@ def main():
         "dtype": "u8" if wl["fmt"] == 8 else "u4", "data": "synthetic",
         "config": {"workload": a.workload, "batch": B, "ctx_min": int(lens.min()), "ctx_max": int(lens.max()),
                    "ctx_sum": int(lens.sum()), "n_q_heads": NQ, "n_kv_heads": NKV, "head_dim": HD, "page_tokens": PT,
-                   "n_pages": g.n_pages, "kv_format": "q8_0" if wl["fmt"] == 8 else "q4_0",
+                   "n_pages": g.n_pages, "layers_rotated": len(layers), "kv_format": "q8_0" if wl["fmt"] == 8 else "q4_0",
                    "step": "append 1 token/seq + paged decode attention"},
         "pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2), "tok_per_s": round(B / (ms * 1e-3), 1),
         "kv_bytes_per_step": int(kv_bytes), "parity_max_rel_err": float(f"{err:.3e}"), "out_fnv1a": first_hash,
