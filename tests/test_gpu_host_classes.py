@@ -1,5 +1,6 @@
 """The C++ host classes of csrc/kv_cache.hpp (KvDecoder / KvPrefill / PagePool, the reference's LoomDecoder surface)
-run as a standalone program against the CPU oracle. The program is compiled by __graft_entry__.build()."""
+and the continuous-batching driver of csrc/kv_batcher.hpp run as standalone programs against the CPU oracle. The
+programs are compiled by __graft_entry__.build()."""
 import os
 import subprocess
 
@@ -17,9 +18,21 @@ def test_kv_cache_cpp_program():
     assert "kv_cache_test: ok" in r.stdout
 
 
+@pytest.mark.gpu
+def test_kv_batcher_cpp_program():
+    """Twelve requests through a pool too small for them: waiting, side by side, put back and started again; every
+    attention row against the oracle, every finished request's blocks bit-exact, no page lost."""
+    exe = os.path.join(ROOT, "tests", "cpp", "kv_batcher_test")
+    assert os.path.exists(exe), "tests/cpp/kv_batcher_test is not built: run `python __graft_entry__.py build`"
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=100)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "kv_batcher_test: ok" in r.stdout
+
+
 def test_kv_cache_header_is_host_only_cxx():
-    """The header compiles as plain host C++ against the C ABI (no device code, no torch)."""
-    src = '#include "kv_cache.hpp"\nint main() { return sizeof(yahkv_host::KvDecoder) > 0 ? 0 : 1; }\n'
+    """The headers compile as plain host C++ against the C ABI (no device code, no torch)."""
+    src = ('#include "kv_batcher.hpp"\n'
+           'int main() { return sizeof(yahkv_host::KvDecoder) + sizeof(yahkv_host::KvBatcher) > 0 ? 0 : 1; }\n')
     r = subprocess.run(["/opt/rocm/bin/hipcc", "-std=c++17", "-fsyntax-only", "-x", "c++", "-D__HIP_PLATFORM_AMD__",
                         "-I", os.path.join(ROOT, "include"), "-I", os.path.join(ROOT, "yet-another-halo-engine_amd", "csrc"),
                         "-I", "/opt/rocm/include", "-"], input=src, capture_output=True, text=True, timeout=120)
