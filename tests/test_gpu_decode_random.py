@@ -1,0 +1,52 @@
+"""Randomized sweep of the paged decode attention against the CPU oracle: formats, group sizes, head dims, page sizes,
+batch sizes, ragged lengths with empty sequences, query dtypes, a gate now and then, and the planner's chunk count
+forced to values that are not a multiple of eight, smaller than the work and larger than it. Tolerance 2e-3."""
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+from helpers import rel_err, to_bf16_f32
+from test_gpu_decode import gpu_attend, setup
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-3
+
+
+@pytest.mark.parametrize("seed", range(20))
+def test_random_decode_case(yahkv, torch_gpu, seed, monkeypatch):
+    rng = np.random.default_rng(1000 + seed)
+    fmt = int(rng.choice([8, 4]))
+    n_kv = int(rng.choice([1, 2, 4]))
+    group = int(rng.choice([1, 2, 3, 4, 6, 8]))
+    hd = int(rng.choice([128, 256]))
+    pt = int(rng.choice([16, 32, 64]))
+    n_seqs = int(rng.integers(1, 24))
+    top = int(rng.choice([70, 300, 900]))
+    lens = [int(x) for x in rng.integers(0, top + 1, n_seqs)]
+    if rng.random() < 0.5:
+        lens[int(rng.integers(0, n_seqs))] = 0               # an empty sequence in the batch
+    if max(lens) == 0:
+        lens[0] = 1
+    chunks = int(rng.choice([0, 1, 3, 7, 13, 64, 100, 256, 1000]))
+    if chunks:
+        monkeypatch.setenv("YAHKV_DECODE_CHUNKS", str(chunks))
+    if rng.random() < 0.3:
+        monkeypatch.setenv("YAHKV_DECODE_MIN_CHUNK_TILES", str(int(rng.choice([1, 2, 5]))))
+    g, table, host, dev, _ = setup(yahkv, torch_gpu, fmt, n_kv * group, n_kv, hd, pt, lens, seed=seed, fill=0x7F)
+    q = to_bf16_f32(rng.standard_normal((n_seqs, n_kv * group, hd)))
+    gate = rng.standard_normal(q.shape).astype(np.float32) if rng.random() < 0.3 else None
+    kind = str(rng.choice(["bf16", "f16", "f32"]))
+    if kind == "f16":
+        q = q.astype(np.float16).astype(np.float32)
+    scale = float(1 / np.sqrt(hd))
+    slack = int(rng.integers(0, 100))                          # the host's bound may be loose
+    got = gpu_attend(yahkv, torch_gpu, dev, table, lens, q, scale, gate=gate, kind=kind,
+                     max_len=min(max(lens) + slack, table.shape[1] * pt))
+    want = oracle.decode_attend(host, table, lens, q, scale, gate)
+    assert np.all(np.isfinite(got)), (fmt, n_kv, group, hd, pt, lens, chunks)
+    for s, n in enumerate(lens):
+        if n == 0:
+            assert not got[s].any(), "an empty sequence attends to nothing"
+    assert rel_err(got, want) < TOL, (fmt, n_kv, group, hd, pt, lens, chunks, kind)
