@@ -283,10 +283,12 @@ void DattnPart(const DecodeArgs a) {
   __shared__ __align__(16) _Float16 lq_all[kWavesPerGroup][NB][2][2][8][8];
   __shared__ __align__(16) _Float16 lp_all[kWavesPerGroup][kMaxGroup][kTile];
   __shared__ __align__(16) _Float16 lvs_all[kWavesPerGroup][NB][kTile];
+  __shared__ __align__(16) uint8_t lvq_all[kWavesPerGroup][FMT == 8 ? NVB * 1024 : 16];  // half a tile of V codes on its way in (q8_0)
   __shared__ int next_tile;
   auto& lq = lq_all[wave];
   auto& lp = lp_all[wave];
   auto& lvs = lvs_all[wave];
+  auto& lvq = lvq_all[wave];
 
   const int4 rec = a.chunks[blockIdx.x];
   if (rec.x < 0) return;
@@ -354,12 +356,41 @@ void DattnPart(const DecodeArgs a) {
       ksc = uint4{v.x, v.y, 0u, 0u};
     }
   };
-  auto load_v = [&](int hf, const int (&pg)[PPT]) {
-    const size_t ph = page_head(pg, 16 * kg);
+  // V codes do not go to registers directly: the loads write this wave's LDS slot (16 bytes per lane and load, in
+  // lane order), and the registers are filled from there right before the product that uses them. The slot is free
+  // again as soon as it has been read, so the next half of V is requested before that product starts and stays in
+  // flight through the arithmetic; a register is only free after its last use. (LDS has room for one such slot per
+  // wave, so K stays in registers.) When a tile is one page the loads go through a buffer resource of the (page, kv
+  // head) region: for that form the compiler keeps exact counts of the loads in flight, whereas with the flat form
+  // (pages smaller than a tile: the lanes read different pages) it waits for all of them before any loaded register
+  // is used.
+  // q4_0 keeps the plain register loads: that kernel is bound by instruction issue, and the detour costs it more
+  // instructions than the earlier request saves.
+  constexpr bool kLdsV = Q8;
+  auto fetch_v = [&](int hf, const int (&pg)[PPT]) {
     const uint32_t off = n16 * PT + (16 * kg) % PT;
-    const uint8_t* vp = a.pools.vq + ph * (Q8 ? D * PT : NB * 16 * PT);
+    if constexpr (!kLdsV) {
+      const size_t ph = page_head(pg, 16 * kg);
+      const uint8_t* vp = a.pools.vq + ph * (Q8 ? D * PT : NB * 16 * PT);
 #pragma unroll
-    for (int j = 0; j < NVB; ++j) vb[j] = *reinterpret_cast<const uint4*>(vp + (16 * (hf * NVB + j) * PT + off));
+      for (int j = 0; j < NVB; ++j) vb[j] = *reinterpret_cast<const uint4*>(vp + (16 * (hf * NVB + j) * PT + off));
+    } else if constexpr (PPT == 1) {
+      const size_t ph = size_t(pg[0]) * H + cur.h;
+      const auto rv = __builtin_amdgcn_make_buffer_rsrc(
+          const_cast<uint8_t*>(a.pools.vq) + ph * (Q8 ? D * PT : NB * 16 * PT), 0, 0x7fffffff, 0x00020000);
+#pragma unroll
+      for (int j = 0; j < NVB; ++j)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, (__attribute__((address_space(3))) void*)(&lvq[j * 1024]), 16, off,
+                                                 16 * (hf * NVB + j) * PT, 0, 0);
+    } else {
+      const size_t ph = page_head(pg, 16 * kg);
+      const uint8_t* vp = a.pools.vq + ph * (Q8 ? D * PT : NB * 16 * PT);
+#pragma unroll
+      for (int j = 0; j < NVB; ++j)
+        __builtin_amdgcn_global_load_lds(
+            (const __attribute__((address_space(1))) void*)(vp + (16 * (hf * NVB + j) * PT + off)),
+            (__attribute__((address_space(3))) void*)(&lvq[j * 1024]), 16, 0, 0);
+    }
     if (hf == 0) {  // with the first half come the tile's V scales: lane = (block, 8 keys)
       const int b = lane / 8, chunk = lane % 8;
       if (b < NB) {
@@ -368,6 +399,12 @@ void DattnPart(const DecodeArgs a) {
         vsr = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint8_t*>(a.pools.vs) + ps * (NB * PT * 2) + soff);
       }
     }
+  };
+  auto take_v = [&]() {
+    if constexpr (!kLdsV) return;
+#pragma unroll
+    for (int j = 0; j < NVB; ++j) vb[j] = *reinterpret_cast<const uint4*>(&lvq[j * 1024 + lane * 16]);
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the slot has been read before the next fetch is issued
   };
   // the 8 codes of block b this lane feeds to instruction `sub` of the block's pair
   auto kcodes = [&](int b, int sub) -> h8v {
@@ -480,8 +517,8 @@ void DattnPart(const DecodeArgs a) {
     int pgc[PPT], pgn[PPT];
     load_pages(tile, pgc);
     load_k(0, pgc);
-    load_v(1, pgc);  // not used (the first pass has no previous tile): it keeps the count of loads in flight at the
-                     // head of the loop the same as on the way round, see below
+    fetch_v(1, pgc);  // not used (the first pass has no previous tile): it keeps the count of loads in flight at the
+                      // head of the loop the same as on the way round, see below
 #pragma unroll
     for (int e = 0; e < QE; ++e) {
       const int i = lane + 64 * e;
@@ -505,8 +542,12 @@ void DattnPart(const DecodeArgs a) {
       load_pages(has_next ? ntile : tile, pgn);
       scores(0);
       load_k(1, pgc);
-      if (!first) pv(1);  // second half of the previous tile's P.V: lp and lvs still hold that tile
-      load_v(0, pgc);
+      // second half of the previous tile's P.V (lp and lvs still hold that tile), and the request for this tile's
+      // first half of V: before the product when V comes through LDS, after it when the registers are the buffer
+      take_v();
+      if constexpr (kLdsV) fetch_v(0, pgc);
+      if (!first) pv(1);
+      if constexpr (!kLdsV) fetch_v(0, pgc);
       first = false;
       scores(1);
       load_k(0, pgn);
@@ -548,14 +589,17 @@ void DattnPart(const DecodeArgs a) {
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      take_v();  // this tile's first half of V
+      if constexpr (kLdsV) fetch_v(1, pgc);
       pv(0);
-      load_v(1, pgc);
+      if constexpr (!kLdsV) fetch_v(1, pgc);
       idx = nidx;
       if (!has_next) break;
       tile = ntile;
 #pragma unroll
       for (int j = 0; j < PPT; ++j) pgc[j] = pgn[j];
     }
+    take_v();
     pv(1);
     leave_partial();
     __builtin_amdgcn_wave_barrier();  // lq, lp and lvs are rewritten for the next pair
