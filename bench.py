@@ -295,7 +295,6 @@ def main():
         seq_len = len_rows[i + 1]
         pools = layers[i % len(layers)]     # (with several layers a layer sees every n-th token; the others stay zero blocks)
         yahkv.append(pools, t_table, len_rows[i], knew[i], vnew[i])    # position = current length (device-resident)
-        yahkv.decode_plan(g, t_table.shape[1], seq_len, B, max_len, ws)
         if pair:
             pair[0].record()
         yahkv.decode_part(pools, t_table, seq_len, max_len, q, scale, ws)

@@ -20,6 +20,8 @@ float Widen(uint16_t h) { return orc_bf16_to_f32(h); }
 struct Fail : std::runtime_error {
   using std::runtime_error::runtime_error;
 };
+// stderr is unbuffered: if the program dies, the last stage it names is where
+void Stage(const char* what) { std::fprintf(stderr, "kv_cache_test: %s\n", what); }
 void Expect(bool ok, const char* what) {
   if (!ok) throw Fail(what);
 }
@@ -68,6 +70,7 @@ int main() {
     Expect(dec.free_pages() == 40, "fresh pool");
 
     // ---- prefill chunk
+    Stage("prefill chunk");
     std::vector<uint16_t> kb, vb, qb;
     std::vector<float> kf, vf, qf;
     randn_bf16(size_t(B) * chunk * H * D, &kb, &kf);
@@ -102,6 +105,7 @@ int main() {
     Expect(e1 < 2e-3, "prefill attention differs from the oracle");
 
     // ---- decode steps
+    Stage("decode steps");
     double e2 = 0;
     for (int i = 0; i < steps; ++i) {
       std::vector<uint16_t> k1, v1, q1;
@@ -139,6 +143,7 @@ int main() {
     }
 
     // ---- host checks
+    Stage("host checks");
     Expect(dec.length(2) == chunk + steps, "lengths after the steps");
     ExpectThrow([&] { dec.Reserve(0, T + 1); }, "Reserve past the context must throw");
     const int before = dec.free_pages();
@@ -153,6 +158,7 @@ int main() {
     ExpectThrow([&] { tiny.Step(1, dk.get(), dv.get(), YAHKV_BF16, dq.get(), YAHKV_BF16, scale, nullptr, static_cast<float*>(dout.get())); },
                 "Step past the context must throw");
     // ---- fork (shared prefix pages) and slot files
+    Stage("fork and slots");
     {
       auto gathered = [&](KvDecoder& d, int seq) {
         const size_t bytes = size_t(d.length(seq)) * H * (D / 32) * 34;
@@ -191,7 +197,9 @@ int main() {
       ExpectThrow([&] { wrong.LoadSlot(0, path); }, "a slot of another geometry must be refused");
       std::remove(path.c_str());
     }
+    Stage("done");
     std::printf("kv_cache_test: ok (prefill %.2e, decode %.2e max relative error)\n", e1, e2);
+    std::fflush(stdout);
     return 0;
   } catch (const std::exception& e) {
     std::fprintf(stderr, "kv_cache_test: FAILED: %s\n", e.what());

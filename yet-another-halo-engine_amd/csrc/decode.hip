@@ -11,8 +11,8 @@
 // 64-key tiles and the line is cut into equal chunks, one per workgroup, one workgroup per CU: every CU gets the same
 // number of tiles whatever the mix of lengths, in a single round. Inside a workgroup the waves take the chunk's tiles
 // one by one from an LDS counter, because waves of one CU do not run at one speed (the older wave of a SIMD wins the
-// issue arbitration); each wave keeps its own online softmax and leaves one partial per pair it worked on. A small
-// `plan` kernel computes the cut from the device-resident lengths.
+// issue arbitration); each wave keeps its own online softmax and leaves one partial per pair it worked on. Every
+// workgroup computes its piece of the cut from the device-resident lengths itself.
 // (Measured and dropped: finishing the line with short chunks or single tiles handed out dynamically, by a counter in
 // global memory or by the dispatcher, to even out the XCDs, which finish up to 10 % apart. Every variant was slower:
 // each change of pair costs a wave a pipeline fill, and the XCDs that finish first leave their bandwidth to the rest.)
@@ -28,7 +28,6 @@ namespace {
 constexpr float kNegMax = -3.4028234663852886e+38f;
 constexpr int kTile = 64;     // keys per tile: one wavefront, one key per lane in the score phase
 constexpr int kMaxGroup = 8;  // query heads per kv head
-constexpr int kPlanThreads = 256;
 constexpr int kMaxSeqs = 8191;
 constexpr int kWavesPerGroup = 8;  // one workgroup fills a CU at two waves per SIMD
 
@@ -45,9 +44,6 @@ struct DecodeArgs {
   const float* gate;
   float* out;
   // workspace
-  int32_t* header;   // [0] tiles on the line, [1] tiles per chunk
-  int32_t* tprefix;  // [n_seqs + 1] tiles of all earlier sequences (one kv head's worth)
-  int4* chunks;      // [n_chunks] {sequence or -1, kv head, first tile within the pair, tiles in the chunk}
   float* ml;         // [(n_chunks + n_seqs * H) * wpc][G][2]   partial of (chunk k, wave w, pair p): (k + p) * wpc + w
   float* acc;        // [(n_chunks + n_seqs * H) * wpc][G][D]
   int32_t n_chunks, wpc;  // chunks = workgroups launched; waves per chunk
@@ -73,60 +69,57 @@ __device__ __forceinline__ int ChunkOf(const DecodeArgs& a, long long A, long lo
 
 // ---- plan -------------------------------------------------------------------------------------------------------------
 
-// Every workgroup recomputes the prefix sums of the sequences' tile counts in LDS (a few hundred integers), then each
-// thread writes one chunk record. Workgroup 0 also publishes the prefix sums and the chunk size. Chunk k covers tiles
-// [ChunkStart(k), ChunkStart(k + 1)) of the line, clipped to the line's length: A tiles on average.
-__global__ __launch_bounds__(kPlanThreads) void DattnPlan(const DecodeArgs a) {
-  extern __shared__ int lpre[];  // [n_seqs + 1]
-  __shared__ int part_sum[kPlanThreads / 64];
+// The cut of the line is a function of the lengths alone, and every workgroup that needs it recomputes it from them
+// (a few hundred integers from L2) rather than reading the result of a kernel of its own: a dispatch between the
+// append and the attention costs more than all these recomputations together.
+__device__ __forceinline__ int TilesOf(const DecodeArgs& a, int s) { return (ClampLen(a, s) + kTile - 1) / kTile; }
+__device__ __forceinline__ long long ChunkTiles(const DecodeArgs& a, long long line) {
+  // a short line is not cut finer than min_chunk_tiles: each piece costs a partial (G x (D + 2) floats)
+  return max((line + a.n_chunks - 1) / a.n_chunks, static_cast<long long>(a.min_chunk_tiles));
+}
+
+// Chunk k of the line, for a whole workgroup of NT threads (all call it; one barrier inside): {sequence or -1, kv
+// head, first tile within the pair, tiles in the chunk}. Thread t sums the tiles of a slice of the sequences, a scan
+// over the threads gives every slice its place on the line, and the thread whose slice holds the chunk's first tile
+// walks the slice to find the sequence.
+template <int NT>
+__device__ __forceinline__ int4 ChunkRecord(const DecodeArgs& a, int k, int* wave_sum, int4* found) {
   const int t = threadIdx.x, H = a.g.n_kv;
-  const int per = (a.n_seqs + kPlanThreads - 1) / kPlanThreads;
+  const int per = (a.n_seqs + NT - 1) / NT;
   const int s0 = min(t * per, a.n_seqs), s1 = min(s0 + per, a.n_seqs);
   int sum = 0;
-  for (int s = s0; s < s1; ++s) sum += (ClampLen(a, s) + kTile - 1) / kTile;
-  // exclusive prefix of the threads' sums: inclusive scan inside each wave, then the waves' totals
-  int incl = sum;
+  for (int s = s0; s < s1; ++s) sum += TilesOf(a, s);
+  int incl = sum;  // inclusive scan inside the wave, then the waves' totals
 #pragma unroll
   for (int o = 1; o < 64; o <<= 1) {
     const int v = __shfl_up(incl, o, 64);
     if (t % 64 >= o) incl += v;
   }
-  if (t % 64 == 63) part_sum[t / 64] = incl;
+  if (t % 64 == 63) wave_sum[t / 64] = incl;
   __syncthreads();
   int base = incl - sum, total = 0;
 #pragma unroll
-  for (int w = 0; w < kPlanThreads / 64; ++w) {
-    if (w < t / 64) base += part_sum[w];
-    total += part_sum[w];
+  for (int w = 0; w < NT / 64; ++w) {
+    if (w < t / 64) base += wave_sum[w];
+    total += wave_sum[w];
   }
-  for (int s = s0; s < s1; ++s) {
-    lpre[s] = base;
-    base += (ClampLen(a, s) + kTile - 1) / kTile;
-  }
-  if (t == 0) lpre[a.n_seqs] = total;
-  __syncthreads();
-  const long long line = static_cast<long long>(total) * H;  // tiles on the line
-  // a short line is not cut finer than min_chunk_tiles: each piece costs a partial (G x (D + 2) floats)
-  const long long A = max((line + a.n_chunks - 1) / a.n_chunks, static_cast<long long>(a.min_chunk_tiles));
-  if (blockIdx.x == 0) {
-    for (int s = t; s <= a.n_seqs; s += kPlanThreads) a.tprefix[s] = lpre[s];
-    if (t == 0) a.header[0] = static_cast<int>(min(line, 0x7fffffffLL)), a.header[1] = static_cast<int>(A);
-  }
-  const int k = blockIdx.x * kPlanThreads + t;
-  if (k >= a.n_chunks) return;
+  const long long line = static_cast<long long>(total) * H, A = ChunkTiles(a, line);
   const long long start = ChunkStart(a, A, k), end = min(ChunkStart(a, A, k + 1), line);
-  if (start >= end) {
-    a.chunks[k] = int4{-1, 0, 0, 0};
-    return;
+  if (start >= end) return int4{-1, 0, 0, 0};  // the same for every thread
+  if (static_cast<long long>(base) * H <= start && start < static_cast<long long>(base + sum) * H) {
+    int before = base;
+    for (int s = s0; s < s1; ++s) {
+      const int ts = TilesOf(a, s);
+      if (start < static_cast<long long>(before + ts) * H) {
+        const int r = static_cast<int>(start - static_cast<long long>(before) * H);
+        *found = int4{s, r / ts, r % ts, static_cast<int>(end - start)};
+        break;
+      }
+      before += ts;
+    }
   }
-  int lo = 0, hi = a.n_seqs;  // largest s with H * prefix[s] <= start (then sequence s is not empty)
-  while (hi - lo > 1) {
-    const int mid = (lo + hi) / 2;
-    if (static_cast<long long>(lpre[mid]) * H <= start) lo = mid; else hi = mid;
-  }
-  const int ts = lpre[lo + 1] - lpre[lo];
-  const int r = static_cast<int>(start - static_cast<long long>(lpre[lo]) * H);
-  a.chunks[k] = int4{lo, r / ts, r % ts, static_cast<int>(end - start)};
+  __syncthreads();
+  return *found;
 }
 
 // Position of a wave on its chunk: the pair (s, h) it stands on, which of the chunk's tiles belong to that pair
@@ -135,7 +128,7 @@ struct PairCursor {
   int s, h, first, base, n, len;
 };
 __device__ __forceinline__ PairCursor FirstPair(const DecodeArgs& a, const int4 rec) {
-  const int ts = a.tprefix[rec.x + 1] - a.tprefix[rec.x];
+  const int ts = TilesOf(a, rec.x);
   return PairCursor{rec.x, rec.y, rec.z, 0, min(ts - rec.z, rec.w), ClampLen(a, rec.x)};
 }
 // Next pair of the chunk; false when the chunk (of chunk_n tiles) ends with the current pair.
@@ -146,7 +139,7 @@ __device__ __forceinline__ bool NextPair(const DecodeArgs& a, int chunk_n, PairC
   do {  // empty sequences have no tiles on the line
     if (++c->h == a.g.n_kv) c->h = 0, ++c->s;
     if (c->s >= a.n_seqs) return false;
-    ts = a.tprefix[c->s + 1] - a.tprefix[c->s];
+    ts = TilesOf(a, c->s);
     if (ts == 0) c->h = a.g.n_kv - 1;
   } while (ts == 0);
   c->n = min(ts, chunk_n - c->base), c->len = ClampLen(a, c->s);
@@ -285,12 +278,14 @@ void DattnPart(const DecodeArgs a) {
   __shared__ __align__(16) _Float16 lvs_all[kWavesPerGroup][NB][kTile];
   __shared__ __align__(16) uint8_t lvq_all[kWavesPerGroup][FMT == 8 ? NVB * 1024 : 16];  // half a tile of V codes on its way in (q8_0)
   __shared__ int next_tile;
+  __shared__ int wave_sum[kWavesPerGroup];
+  __shared__ int4 chunk_rec;
   auto& lq = lq_all[wave];
   auto& lp = lp_all[wave];
   auto& lvs = lvs_all[wave];
   auto& lvq = lvq_all[wave];
 
-  const int4 rec = a.chunks[blockIdx.x];
+  const int4 rec = ChunkRecord<64 * kWavesPerGroup>(a, blockIdx.x, wave_sum, &chunk_rec);
   if (rec.x < 0) return;
   const int chunk_n = rec.w;
   if (threadIdx.x == 0) next_tile = 0;
@@ -627,13 +622,28 @@ __global__ __launch_bounds__(kReduceThreads) void DattnReduce(const DecodeArgs a
   const int hq = blockIdx.x, s = blockIdx.y, t = threadIdx.x;
   const int h = hq / G, gi = hq % G;
   const size_t o = (size_t(s) * g.n_q + hq) * D;
-  const int ts = a.tprefix[s + 1] - a.tprefix[s];
+  const int ts = TilesOf(a, s);
   if (ts <= 0) {  // length 0
     if (t < D) a.out[o + t] = 0.0f;
     return;
   }
-  const int A_ = a.header[1], pair = s * H + h;
-  const long long first = static_cast<long long>(a.tprefix[s]) * H + static_cast<long long>(h) * ts;
+  // tiles on the line and tiles of the sequences before this one
+  __shared__ int tile_sums[2][kReduceThreads / 64];
+  int total = 0, before = 0;
+  for (int i = t; i < a.n_seqs; i += kReduceThreads) {
+    const int n = TilesOf(a, i);
+    total += n, before += i < s ? n : 0;
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) total += __shfl_xor(total, off, 64), before += __shfl_xor(before, off, 64);
+  if (t % 64 == 0) tile_sums[0][t / 64] = total, tile_sums[1][t / 64] = before;
+  __syncthreads();
+  total = 0, before = 0;
+#pragma unroll
+  for (int w = 0; w < kReduceThreads / 64; ++w) total += tile_sums[0][w], before += tile_sums[1][w];
+  const long long A_ = ChunkTiles(a, static_cast<long long>(total) * H);
+  const int pair = s * H + h;
+  const long long first = static_cast<long long>(before) * H + static_cast<long long>(h) * ts;
   const int k0 = ChunkOf(a, A_, first), k1 = ChunkOf(a, A_, first + ts - 1);
   const size_t p0 = size_t(k0 + pair) * a.wpc, p1 = size_t(k1 + pair + 1) * a.wpc;
   constexpr int NW = kReduceThreads / 64;
@@ -707,7 +717,7 @@ __global__ __launch_bounds__(kReduceThreads) void DattnReduce(const DecodeArgs a
 struct Plan {
   int32_t max_len, n_chunks, wpc, min_chunk_tiles;
   int32_t share[9];
-  size_t off_tprefix, off_chunks, off_ml, off_acc, bytes;
+  size_t off_ml, off_acc, bytes;
 };
 size_t Align(size_t x) { return (x + 255) & ~size_t(255); }
 int ComputeUnits() {
@@ -754,9 +764,7 @@ Plan MakePlan(const Geom& g, int32_t n_seqs, int32_t max_seq_len) {
   for (int j = 0; j < 8; ++j) p.share[j + 1] = p.share[j] + static_cast<int32_t>(w[j] * 8192 / sum);
   p.share[8] = 8192;
   const size_t parts = (size_t(p.n_chunks) + size_t(n_seqs) * g.n_kv) * p.wpc;
-  p.off_tprefix = 256;
-  p.off_chunks = Align(p.off_tprefix + sizeof(int32_t) * (size_t(n_seqs) + 1));
-  p.off_ml = Align(p.off_chunks + sizeof(int4) * size_t(p.n_chunks));
+  p.off_ml = 0;
   p.off_acc = Align(p.off_ml + sizeof(float) * parts * g.group() * 2);
   p.bytes = Align(p.off_acc + sizeof(float) * parts * g.group() * g.hd);
   return p;
@@ -768,7 +776,7 @@ int Prepare(const yahkv_geometry* g, int32_t page_table_stride, const int32_t* s
   if (const int st = CheckGeometry(g)) return st;
   if (seq_len == nullptr || workspace == nullptr) return YAHKV_ERR_ARG;
   if (n_seqs <= 0 || max_seq_len <= 0 || page_table_stride <= 0) return YAHKV_ERR_ARG;
-  if (n_seqs > kMaxSeqs) return YAHKV_ERR_SHAPE;  // the plan kernel keeps one integer per sequence in LDS
+  if (n_seqs > kMaxSeqs) return YAHKV_ERR_SHAPE;  // every workgroup walks all lengths: keep that a few thousand
   if (reinterpret_cast<uintptr_t>(workspace) & 15) return YAHKV_ERR_ARG;
   const Geom m = MakeGeom(*g);
   const Plan p = MakePlan(m, n_seqs, max_seq_len);
@@ -778,9 +786,6 @@ int Prepare(const yahkv_geometry* g, int32_t page_table_stride, const int32_t* s
   // lengths read on the device are clamped to the host's bound and to the table's extent
   a->max_len = static_cast<int32_t>(std::min<int64_t>(p.max_len, int64_t(page_table_stride) * m.pt));
   char* ws = static_cast<char*>(const_cast<void*>(workspace));
-  a->header = reinterpret_cast<int32_t*>(ws);
-  a->tprefix = reinterpret_cast<int32_t*>(ws + p.off_tprefix);
-  a->chunks = reinterpret_cast<int4*>(ws + p.off_chunks);
   a->ml = reinterpret_cast<float*>(ws + p.off_ml);
   a->acc = reinterpret_cast<float*>(ws + p.off_acc);
   a->n_chunks = p.n_chunks, a->wpc = p.wpc, a->min_chunk_tiles = p.min_chunk_tiles;
@@ -804,9 +809,8 @@ extern "C" int yahkv_decode_plan(const yahkv_geometry* g, int32_t page_table_str
   DecodeArgs a;
   if (const int st = Prepare(g, page_table_stride, seq_len, n_seqs, max_seq_len, workspace, workspace_bytes, &a))
     return st;
-  hipLaunchKernelGGL(DattnPlan, dim3((a.n_chunks + kPlanThreads - 1) / kPlanThreads), dim3(kPlanThreads),
-                     sizeof(int) * (size_t(n_seqs) + 1), static_cast<hipStream_t>(stream), a);
-  return LaunchStatus();
+  (void)stream;  // nothing to launch: part and reduce derive the cut from the lengths themselves
+  return YAHKV_OK;
 }
 
 extern "C" int yahkv_decode_part(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
