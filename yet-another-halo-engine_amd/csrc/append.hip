@@ -196,6 +196,117 @@ __global__ __launch_bounds__(64 * kRopeWaves) void AppendRows(const RopeArgs a) 
   }
 }
 
+// Chunks: one workgroup per (sequence, page touched by the chunk, kv head). A token at a time per wavefront, the rows
+// are quantized exactly as above, but the codes and scales go to an LDS image of the page's (page, head) regions, and
+// the image leaves for HBM in 16-byte pieces once the page's tokens are done. Token by token the V codes would be
+// single bytes 64 bytes apart (V lies transposed, [dim][token], so that decode reads 16 tokens of a dim at once) and
+// every K block a 32-byte piece; page by page they are whole lines.
+// Positions clamp to the table as everywhere (gen_decode_attn.py:59-63); where several tokens of a chunk clamp to
+// the same slot (the first or the last of the table), the last token wins, as in a loop over the tokens.
+constexpr int kPageWaves = 4;
+constexpr int kPageAppendMin = 8;  // tokens per sequence from which a call is treated as a chunk
+template <int FMT>
+__global__ __launch_bounds__(64 * kPageWaves) void AppendPages(const RopeArgs a) {
+#pragma clang fp contract(off)
+  const Geom g = a.g;
+  const int NB = g.nb(), H = g.n_kv, PT = g.pt, D = g.hd;
+  constexpr int KB = FMT == 8 ? 32 : 16;                 // bytes of K codes per token and block
+  const int v_rows = FMT == 8 ? D : NB * 16;             // byte rows of the V image, PT bytes each
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64, h = blockIdx.y, s = blockIdx.z;
+  const int nv = a.n_valid != nullptr ? min(max(a.n_valid[s], 0), a.n_new) : a.n_new;
+  if (nv <= 0) return;
+  const int start = a.start_pos[s], last_pos = a.stride * PT - 1;
+  const int p_first = min(max(start, 0), last_pos), p_last = min(max(start + nv - 1, 0), last_pos);
+  const int pi = p_first / PT + blockIdx.x;
+  if (pi > p_last / PT) return;
+  const int t_lo = max(p_first, pi * PT) - pi * PT, t_hi = min(p_last, pi * PT + PT - 1) - pi * PT + 1;
+  const int page = ClampPage(a.table[int64_t(s) * a.stride + pi], g.n_pages);
+  // the token of the chunk that ends up at position pos (the last one, where several clamp to it)
+  auto token_at = [&](int pos) -> int {
+    if (pos == last_pos && start + nv - 1 >= last_pos) return nv - 1;
+    if (pos == 0 && start <= 0) return min(nv - 1, -start);
+    return pos - start;
+  };
+
+  __shared__ __align__(16) uint8_t lk[8 * 64 * 32], lv[256 * (64 + 4)];  // images of the K and V code regions
+  __shared__ __align__(16) uint16_t lks[64 * 8], lvs[8 * 64];      // and of the scale regions
+  const int d0 = 4 * lane, b = lane / 8, lb = lane % 8;
+  const bool has = d0 < D;
+  // A wavefront takes four consecutive tokens at a time (their rows in flight together): a lane then holds, for each
+  // of its four dims, the codes of four neighbouring tokens, which is one dword of the V image instead of four bytes.
+  // (The image's rows are padded by a dword: with rows of exactly PT bytes the 64 lanes of such a store would all
+  // hit one LDS bank.)
+  for (int q = t_lo / 4 + wave; 4 * q < t_hi; q += kPageWaves) {
+    float4 kx[4], vx[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int t = 4 * q + j;
+      kx[j] = vx[j] = float4{0.0f, 0.0f, 0.0f, 0.0f};
+      if (t >= t_lo && t < t_hi && has) {
+        const size_t row = ((size_t(s) * a.n_new + token_at(pi * PT + t)) * H + h) * D;
+        kx[j] = Load4(a.k_src, row + d0, a.src_dtype), vx[j] = Load4(a.v_src, row + d0, a.src_dtype);
+      }
+    }
+    uint32_t vc[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int t = 4 * q + j;
+      uint16_t ksc, vsc;
+      const uint32_t kc = FMT == 8 ? QuantizeLanesQ8(kx[j], &ksc) : QuantizeLanesQ4(kx[j], lb, &ksc);
+      vc[j] = FMT == 8 ? QuantizeLanesQ8(vx[j], &vsc) : QuantizeLanesQ4(vx[j], lb, &vsc);
+      if (!has || t < t_lo || t >= t_hi) continue;
+      if (lb == 0) lks[t * NB + b] = ksc, lvs[b * PT + t] = vsc;
+      if (FMT == 8 || lb < 4) *reinterpret_cast<uint32_t*>(&lk[(b * PT + t) * KB + 4 * lb]) = kc;
+    }
+    if (has && (FMT == 8 || lb < 4)) {
+      const int r0 = FMT == 8 ? d0 : b * 16 + 4 * lb;  // this lane's four byte rows of the V image
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        *reinterpret_cast<uint32_t*>(&lv[(r0 + e) * (PT + 4) + 4 * q]) =
+            ((vc[0] >> (8 * e)) & 0xFF) | (((vc[1] >> (8 * e)) & 0xFF) << 8) | (((vc[2] >> (8 * e)) & 0xFF) << 16) |
+            (((vc[3] >> (8 * e)) & 0xFF) << 24);
+    }
+  }
+  __syncthreads();
+  // ---- the images' written parts to the pools
+  const size_t ph = size_t(page) * H + h;
+  const int n_t = t_hi - t_lo, tid = threadIdx.x, NT = 64 * kPageWaves;
+  {  // K codes: per block the tokens' pieces are contiguous
+    uint8_t* dst = a.pools.kq + ph * (size_t(NB) * PT * KB);
+    const int per_block = n_t * KB / 16;
+    for (int u = tid; u < NB * per_block; u += NT) {
+      const int off = ((u / per_block) * PT + t_lo) * KB + (u % per_block) * 16;
+      *reinterpret_cast<uint4*>(dst + off) = *reinterpret_cast<const uint4*>(&lk[off]);
+    }
+  }
+  {  // K scales: [token][block], 8 bytes at a time
+    uint8_t* dst = reinterpret_cast<uint8_t*>(a.pools.ks) + ph * (size_t(PT) * NB * 2);
+    for (int u = tid; u < n_t * NB / 4; u += NT) {
+      const int off = t_lo * NB * 2 + u * 8;
+      *reinterpret_cast<uint2*>(dst + off) = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint8_t*>(lks) + off);
+    }
+  }
+  uint8_t* vdst = a.pools.vq + ph * (size_t(v_rows) * PT);
+  uint16_t* sdst = a.pools.vs + ph * (size_t(NB) * PT);
+  if (n_t == PT) {  // a whole page: both V regions are contiguous
+    for (int u = tid; u < v_rows * PT / 16; u += NT) {
+      const uint32_t* src = reinterpret_cast<const uint32_t*>(&lv[(u * 16 / PT) * (PT + 4) + u * 16 % PT]);
+      *reinterpret_cast<uint4*>(vdst + u * 16) = uint4{src[0], src[1], src[2], src[3]};
+    }
+    for (int u = tid; u < NB * PT / 8; u += NT)
+      *reinterpret_cast<uint4*>(sdst + u * 8) = *reinterpret_cast<const uint4*>(&lvs[u * 8]);
+  } else {  // the chunk's first or last page: the tokens' bytes of every row
+    for (int u = tid; u < v_rows * n_t; u += NT) {
+      const int r = u / n_t, t = t_lo + u % n_t;
+      vdst[r * PT + t] = lv[r * (PT + 4) + t];
+    }
+    for (int u = tid; u < NB * n_t; u += NT) {
+      const int off = (u / n_t) * PT + t_lo + u % n_t;
+      sdst[off] = lvs[off];
+    }
+  }
+}
+
 // One thread per (K|V, token, kv head, block): the block back in ggml order (scale, then codes).
 template <int FMT>
 __global__ __launch_bounds__(256) void GatherBlocks(Geom g, Pools pools, const int32_t* table_row, int n_tokens,
@@ -263,8 +374,17 @@ extern "C" int yahkv_append(const yahkv_geometry* g, const yahkv_pools* pools, c
   a.g = MakeGeom(*g), a.pools = MakePools(*pools), a.table = page_table, a.stride = page_table_stride;
   a.start_pos = start_pos, a.n_valid = n_valid, a.n_seqs = n_seqs, a.n_new = n_new, a.k_src = k_src, a.v_src = v_src;
   a.src_dtype = src_dtype, a.rotary_dim = 8, a.theta = 1.0f;
-  const dim3 grid(static_cast<unsigned>(n_seqs) * static_cast<unsigned>(n_new));
   hipStream_t st = static_cast<hipStream_t>(stream);
+  if (n_new >= kPageAppendMin && n_seqs <= 65535) {  // a chunk: page by page (the grid's z extent is the batch)
+    const dim3 grid(static_cast<unsigned>((n_new + a.g.pt - 2) / a.g.pt + 1), static_cast<unsigned>(a.g.n_kv),
+                    static_cast<unsigned>(n_seqs));
+    if (g->format == YAHKV_Q8_0)
+      hipLaunchKernelGGL((AppendPages<8>), grid, dim3(64 * kPageWaves), 0, st, a);
+    else
+      hipLaunchKernelGGL((AppendPages<4>), grid, dim3(64 * kPageWaves), 0, st, a);
+    return LaunchStatus();
+  }
+  const dim3 grid(static_cast<unsigned>(n_seqs) * static_cast<unsigned>(n_new));
   if (g->format == YAHKV_Q8_0)
     hipLaunchKernelGGL((AppendRows<8, false>), grid, dim3(64 * kRopeWaves), 0, st, a);
   else
