@@ -108,3 +108,24 @@ def test_append_rejects_bad_arguments(yahkv, torch_gpu):
     import ctypes as C
     rc = yahkv.lib.yahkv_append(C.byref(g), C.byref(st), None, 1, None, None, 1, 1, None, None, 0, None)
     assert rc == -1
+
+
+@pytest.mark.parametrize("fmt,pt", [(8, 64), (4, 16), (8, 32)])
+def test_chunk_positions_clamp_like_a_loop_over_the_tokens(yahkv, torch_gpu, fmt, pt):
+    """A chunk that runs past the table's last position, and one that starts before position 0: every token goes to
+    its clamped position, and where several clamp to the same slot the last one stays, as in the oracle's loop."""
+    torch = torch_gpu
+    rng = np.random.default_rng(fmt + pt)
+    n_kv, hd, stride, n_new = 2, 128, 3, 40
+    g = oracle.geometry(fmt, n_kv, n_kv, hd, pt, 3 * stride + 1)
+    table = make_tables(rng, [stride] * 3, g.n_pages)
+    host = oracle.HostPools(g, fill=0x3C)
+    dev = yahkv.DevicePools(yahkv.geometry(fmt, n_kv, n_kv, hd, pt, g.n_pages), fill=0x3C)
+    start = np.array([stride * pt - 25, -7, stride * pt + 100], np.int32)    # over the end, before 0, all past the end
+    valid = np.array([n_new, 33, 12], np.int32)
+    K = to_bf16_f32(rng.standard_normal((3, n_new, n_kv, hd)))
+    V = to_bf16_f32(rng.standard_normal((3, n_new, n_kv, hd)))
+    oracle.append(host, table, start, valid, K, V)
+    yahkv.append(dev, torch.from_numpy(table).cuda(), torch.from_numpy(start).cuda(), torch_src(torch, K, "bf16"),
+                 torch_src(torch, V, "bf16"), n_valid=torch.from_numpy(valid).cuda())
+    same_pools(dev, host)
