@@ -1,6 +1,7 @@
 """Shared prefixes and slots on the paged pools: a forked sequence shares the prefix's full pages (owner counts) and
 gets a private copy of the partly filled last page; a slot (the pages of one sequence, packed) loads into other
-physical pages. Checks are byte-for-byte on the gathered blocks; attention outputs agree to the last bits of f32."""
+physical pages. Checks are byte-for-byte on the gathered blocks; attention outputs agree within the decode kernel's
+run-to-run variation."""
 import numpy as np
 import pytest
 
@@ -88,9 +89,9 @@ def test_slot_round_trip_into_other_pages(yahkv, torch_gpu, fmt, n_q, n_kv, hd, 
     lens = torch.tensor([n], dtype=torch.int32, device="cuda")
     a = yahkv.decode_attend(dev, row[None], lens, n, q, 0.1)
     b = yahkv.decode_attend(dev2, row2[None], lens, n, q, 0.1)
-    # same bytes; the waves of a workgroup take tiles in an order that varies from run to run, so the f32 sums may
-    # differ in their last bits
-    assert rel_err(a.cpu().numpy(), b.cpu().numpy()) < 1e-5
+    # same bytes; the waves of a workgroup take tiles in an order that varies from run to run, and with it the running
+    # maxima the f16 numerators are rounded against
+    assert rel_err(a.cpu().numpy(), b.cpu().numpy()) < 5e-4
     # untouched pages of the second pools keep their fill
     got = dev2.numpy()
     untouched = sorted(set(range(16)) - set(pages2))

@@ -258,7 +258,7 @@ def decode_attend(pools, table, seq_len, max_seq_len, q, scale, gate=None, out=N
 
 
 def decode_plan(g, table_stride, seq_len, n_seqs, max_seq_len, workspace):
-    """First dispatch of decode_attend: cut the batch into pieces of work."""
+    """Checks the arguments of a decode attention; launches nothing (part and reduce derive the cut themselves)."""
     _check(lib.yahkv_decode_plan(C.byref(g), table_stride, _dp(seq_len), n_seqs, max_seq_len, _dp(workspace),
                                  workspace.numel(), _stream()), "decode_plan")
 
