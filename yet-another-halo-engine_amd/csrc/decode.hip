@@ -246,14 +246,17 @@ __device__ __forceinline__ h8v LoadQ8(const void* q, size_t i, int dt) {
 // in increasing order, so it meets the chunk's (sequence, kv head) pairs in order; for each pair it worked on it keeps
 // an online softmax over its tiles and leaves one partial, for a pair it got no tile of it leaves l = 0.
 //
-// Registers hold half a tile of K (32 keys) and half a tile of V (half the dims) at a time, which keeps the kernel at
-// 256 registers; the four load phases of a tile are rotated against the four arithmetic phases so that every load has
-// arithmetic between its issue and its first use:
-//   scores(keys 0-31)              | load K keys 32-63
-//   P.V(dims D/2.., previous tile) | load V dims 0..D/2 of this tile
-//   scores(keys 32-63)             | load K keys 0-31 of the wave's next tile
-//   softmax, P.V(dims 0..D/2)      | load V dims D/2.. of this tile
-// Page numbers come through scalar loads (they are the same for the whole wave).
+// Registers hold half a tile of K (32 keys) and half a tile of V (half the dims) at a time, which keeps the kernel
+// within 256 registers; the four requests of a tile are rotated against the four arithmetic phases so that every
+// request has arithmetic between its issue and the first use of its data:
+//   scores(keys 0-31)              | K keys 32-63 requested after it
+//   P.V(dims D/2.., previous tile) | V dims 0..D/2 of this tile requested
+//   scores(keys 32-63)             | K keys 0-31 of the wave's next tile requested after it
+//   softmax, P.V(dims 0..D/2)      | V dims D/2.. of this tile requested
+// K loads into the registers the scores have just freed. For q8_0, V loads into an LDS slot of the wave instead and
+// is copied to registers right before its product, so its request goes out before that product (fetch_v / take_v);
+// for q4_0, V loads into registers after the product. Page numbers come through scalar loads (they are the same
+// for the whole wave).
 template <int FMT, int D, int PT>
 __global__ __launch_bounds__(64 * kWavesPerGroup) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void DattnPart(const DecodeArgs a) {
