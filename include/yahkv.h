@@ -142,10 +142,10 @@ int yahkv_append_rope(const yahkv_geometry* g, const yahkv_pools* pools, const i
  * Replaces yah_dattn_part_q + yah_dattn_reduce (gen_decode_attn.py:576-1040, 338-411). */
 size_t yahkv_decode_workspace_bytes(const yahkv_geometry* g, int32_t n_seqs, int32_t max_seq_len);
 /* The dispatches of a decode attention on their own, as LoomDecoder::Step issues its own (loom_decoder.hpp:259-268):
- * `part` leaves partials (M, l, acc) per piece of work in the workspace, `reduce` merges them into out. Both derive
- * the same cut of the batch into equal pieces from the device-resident lengths (the reference needs none: it has one
- * sequence and launches one workgroup per page in use). `plan` checks the arguments and launches nothing; it is kept
- * for callers written against the three-dispatch form. Part and reduce must be given the same geometry, n_seqs,
+ * `part` cuts the batch into equal pieces of work from the device-resident lengths (the reference needs no cut: it
+ * has one sequence and launches one workgroup per page in use) and leaves partials (M, l, acc) per piece in the
+ * workspace, with the prefix sums of the lengths; `reduce` merges the partials into out. `plan` checks the arguments
+ * and launches nothing; it is kept for callers written against the three-dispatch form. Part and reduce must be given the same geometry, n_seqs,
  * max_seq_len, page_table_stride and workspace, in this order on one stream; the lengths must not change in between. */
 int yahkv_decode_plan(const yahkv_geometry* g, int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs,
                       int32_t max_seq_len, void* workspace, size_t workspace_bytes, void* stream);

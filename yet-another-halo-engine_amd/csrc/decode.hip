@@ -44,6 +44,7 @@ struct DecodeArgs {
   const float* gate;
   float* out;
   // workspace
+  int32_t* tprefix;  // [n_seqs + 1] tiles of all earlier sequences (one kv head's worth); written by part, read by reduce
   float* ml;         // [(n_chunks + n_seqs * H) * wpc][G][2]   partial of (chunk k, wave w, pair p): (k + p) * wpc + w
   float* acc;        // [(n_chunks + n_seqs * H) * wpc][G][D]
   int32_t n_chunks, wpc;  // chunks = workgroups launched; waves per chunk
@@ -69,9 +70,10 @@ __device__ __forceinline__ int ChunkOf(const DecodeArgs& a, long long A, long lo
 
 // ---- plan -------------------------------------------------------------------------------------------------------------
 
-// The cut of the line is a function of the lengths alone, and every workgroup that needs it recomputes it from them
-// (a few hundred integers from L2) rather than reading the result of a kernel of its own: a dispatch between the
-// append and the attention costs more than all these recomputations together.
+// The cut of the line is a function of the lengths alone, and every workgroup of the part kernel recomputes its piece
+// from them (a few hundred integers from L2) rather than reading the result of a kernel of its own: a dispatch
+// between the append and the attention costs more than all these recomputations together. The first workgroup
+// leaves the prefix sums in the workspace for the reduce, which needs two of them per workgroup.
 __device__ __forceinline__ int TilesOf(const DecodeArgs& a, int s) { return (ClampLen(a, s) + kTile - 1) / kTile; }
 __device__ __forceinline__ long long ChunkTiles(const DecodeArgs& a, long long line) {
   // a short line is not cut finer than min_chunk_tiles: each piece costs a partial (G x (D + 2) floats)
@@ -102,6 +104,11 @@ __device__ __forceinline__ int4 ChunkRecord(const DecodeArgs& a, int k, int* wav
   for (int w = 0; w < NT / 64; ++w) {
     if (w < t / 64) base += wave_sum[w];
     total += wave_sum[w];
+  }
+  if (k == 0) {
+    int before = base;
+    for (int s = s0; s < s1; ++s) a.tprefix[s] = before, before += TilesOf(a, s);
+    if (t == 0) a.tprefix[a.n_seqs] = total;
   }
   const long long line = static_cast<long long>(total) * H, A = ChunkTiles(a, line);
   const long long start = ChunkStart(a, A, k), end = min(ChunkStart(a, A, k + 1), line);
@@ -630,21 +637,8 @@ __global__ __launch_bounds__(kReduceThreads) void DattnReduce(const DecodeArgs a
     if (t < D) a.out[o + t] = 0.0f;
     return;
   }
-  // tiles on the line and tiles of the sequences before this one
-  __shared__ int tile_sums[2][kReduceThreads / 64];
-  int total = 0, before = 0;
-  for (int i = t; i < a.n_seqs; i += kReduceThreads) {
-    const int n = TilesOf(a, i);
-    total += n, before += i < s ? n : 0;
-  }
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) total += __shfl_xor(total, off, 64), before += __shfl_xor(before, off, 64);
-  if (t % 64 == 0) tile_sums[0][t / 64] = total, tile_sums[1][t / 64] = before;
-  __syncthreads();
-  total = 0, before = 0;
-#pragma unroll
-  for (int w = 0; w < kReduceThreads / 64; ++w) total += tile_sums[0][w], before += tile_sums[1][w];
-  const long long A_ = ChunkTiles(a, static_cast<long long>(total) * H);
+  const int before = a.tprefix[s];  // tiles of the sequences before this one, and tiles on the line
+  const long long A_ = ChunkTiles(a, static_cast<long long>(a.tprefix[a.n_seqs]) * H);
   const int pair = s * H + h;
   const long long first = static_cast<long long>(before) * H + static_cast<long long>(h) * ts;
   const int k0 = ChunkOf(a, A_, first), k1 = ChunkOf(a, A_, first + ts - 1);
@@ -720,7 +714,7 @@ __global__ __launch_bounds__(kReduceThreads) void DattnReduce(const DecodeArgs a
 struct Plan {
   int32_t max_len, n_chunks, wpc, min_chunk_tiles;
   int32_t share[9];
-  size_t off_ml, off_acc, bytes;
+  size_t off_tprefix, off_ml, off_acc, bytes;
 };
 size_t Align(size_t x) { return (x + 255) & ~size_t(255); }
 int ComputeUnits() {
@@ -767,7 +761,8 @@ Plan MakePlan(const Geom& g, int32_t n_seqs, int32_t max_seq_len) {
   for (int j = 0; j < 8; ++j) p.share[j + 1] = p.share[j] + static_cast<int32_t>(w[j] * 8192 / sum);
   p.share[8] = 8192;
   const size_t parts = (size_t(p.n_chunks) + size_t(n_seqs) * g.n_kv) * p.wpc;
-  p.off_ml = 0;
+  p.off_tprefix = 0;
+  p.off_ml = Align(sizeof(int32_t) * (size_t(n_seqs) + 1));
   p.off_acc = Align(p.off_ml + sizeof(float) * parts * g.group() * 2);
   p.bytes = Align(p.off_acc + sizeof(float) * parts * g.group() * g.hd);
   return p;
@@ -789,6 +784,7 @@ int Prepare(const yahkv_geometry* g, int32_t page_table_stride, const int32_t* s
   // lengths read on the device are clamped to the host's bound and to the table's extent
   a->max_len = static_cast<int32_t>(std::min<int64_t>(p.max_len, int64_t(page_table_stride) * m.pt));
   char* ws = static_cast<char*>(const_cast<void*>(workspace));
+  a->tprefix = reinterpret_cast<int32_t*>(ws + p.off_tprefix);
   a->ml = reinterpret_cast<float*>(ws + p.off_ml);
   a->acc = reinterpret_cast<float*>(ws + p.off_acc);
   a->n_chunks = p.n_chunks, a->wpc = p.wpc, a->min_chunk_tiles = p.min_chunk_tiles;
