@@ -50,3 +50,20 @@ def test_random_decode_case(yahkv, torch_gpu, seed, monkeypatch):
         if n == 0:
             assert not got[s].any(), "an empty sequence attends to nothing"
     assert rel_err(got, want) < TOL, (fmt, n_kv, group, hd, pt, lens, chunks, kind)
+
+
+def test_large_batch_of_short_sequences(yahkv, torch_gpu):
+    """1500 sequences of 0 to 40 tokens: every thread of a workgroup owns several sequences when the chunk records are
+    computed, chunks span dozens of (sequence, kv head) pairs, and most partial slots stay empty."""
+    rng = np.random.default_rng(77)
+    n_seqs, n_kv, group, hd, pt = 1500, 2, 4, 128, 16
+    lens = [int(x) for x in rng.integers(0, 41, n_seqs)]
+    g, table, host, dev, _ = setup(yahkv, torch_gpu, 8, n_kv * group, n_kv, hd, pt, lens, seed=78, fill=0x7F)
+    q = to_bf16_f32(rng.standard_normal((n_seqs, n_kv * group, hd)))
+    scale = float(1 / np.sqrt(hd))
+    got = gpu_attend(yahkv, torch_gpu, dev, table, lens, q, scale)
+    want = oracle.decode_attend(host, table, lens, q, scale)
+    assert np.all(np.isfinite(got))
+    assert rel_err(got, want) < TOL
+    for s in np.flatnonzero(np.array(lens) == 0)[:20]:
+        assert not got[s].any()
