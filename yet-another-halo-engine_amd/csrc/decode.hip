@@ -44,11 +44,12 @@ struct DecodeArgs {
   const float* gate;
   float* out;
   // workspace
-  int32_t* tprefix;  // [n_seqs + 1] tiles of all earlier sequences (one kv head's worth); written by part, read by reduce
+  int32_t* tprefix;  // [n_seqs + 1] line units of all earlier sequences (one kv head's worth); written by part, read by reduce
   float* ml;         // [(n_chunks + n_seqs * H) * wpc][G][2]   partial of (chunk k, wave w, pair p): (k + p) * wpc + w
   float* acc;        // [(n_chunks + n_seqs * H) * wpc][G][D]
   int32_t n_chunks, wpc;  // chunks = workgroups launched; waves per chunk
   int32_t min_chunk_tiles;
+  int32_t pair_cost;  // line units a (sequence, kv head) pair takes besides its tiles
   int32_t share[9];  // cumulative shares of the eight chunks of a group, in 1/8192 of the group (share[8] = 8192)
 };
 
@@ -74,59 +75,79 @@ __device__ __forceinline__ int ChunkOf(const DecodeArgs& a, long long A, long lo
 // from them (a few hundred integers from L2) rather than reading the result of a kernel of its own: a dispatch
 // between the append and the attention costs more than all these recomputations together. The first workgroup
 // leaves the prefix sums in the workspace for the reduce, which needs two of them per workgroup.
+//
+// The line is measured in units of one tile's work. A pair (sequence, kv head) of ts tiles takes pair_cost + ts units:
+// first the units that stand for what a change of pair costs every wave of a workgroup (it drains its pipeline,
+// leaves a partial and fetches new queries: about eight tiles' worth per workgroup, measured), then one unit per
+// tile. Cutting this line evenly gives chunks of equal time rather than of equal tiles: without it the workgroups
+// finish up to 50 us apart, by the number of pairs their chunks hold.
 __device__ __forceinline__ int TilesOf(const DecodeArgs& a, int s) { return (ClampLen(a, s) + kTile - 1) / kTile; }
-__device__ __forceinline__ long long ChunkTiles(const DecodeArgs& a, long long line) {
+__device__ __forceinline__ int UnitsOf(const DecodeArgs& a, int ts) { return ts > 0 ? ts + a.pair_cost : 0; }
+__device__ __forceinline__ long long ChunkUnits(const DecodeArgs& a, long long line) {
   // a short line is not cut finer than min_chunk_tiles: each piece costs a partial (G x (D + 2) floats)
   return max((line + a.n_chunks - 1) / a.n_chunks, static_cast<long long>(a.min_chunk_tiles));
 }
 
-// Chunk k of the line, for a whole workgroup of NT threads (all call it; one barrier inside): {sequence or -1, kv
-// head, first tile within the pair, tiles in the chunk}. Thread t sums the tiles of a slice of the sequences, a scan
-// over the threads gives every slice its place on the line, and the thread whose slice holds the chunk's first tile
-// walks the slice to find the sequence.
+// Chunk k of the line, for a whole workgroup of NT threads (all call it; two barriers inside): {sequence or -1, kv
+// head, first tile within the pair, tiles in the chunk}. Thread t sums a slice of the sequences, a scan over the
+// threads gives every slice its place on the line, and the threads whose slices hold the chunk's two ends walk
+// their slices to find the sequences and count the tiles before each end.
 template <int NT>
-__device__ __forceinline__ int4 ChunkRecord(const DecodeArgs& a, int k, int* wave_sum, int4* found) {
-  const int t = threadIdx.x, H = a.g.n_kv;
+__device__ __forceinline__ int4 ChunkRecord(const DecodeArgs& a, int k, int (*wave_sum)[2], int4* found, long long* tiles_at) {
+  const int t = threadIdx.x, H = a.g.n_kv, c = a.pair_cost;
   const int per = (a.n_seqs + NT - 1) / NT;
   const int s0 = min(t * per, a.n_seqs), s1 = min(s0 + per, a.n_seqs);
-  int sum = 0;
-  for (int s = s0; s < s1; ++s) sum += TilesOf(a, s);
-  int incl = sum;  // inclusive scan inside the wave, then the waves' totals
+  int sum = 0, cnt = 0;  // units of the slice, and sequences in it that are not empty
+  for (int s = s0; s < s1; ++s) {
+    const int ts = TilesOf(a, s);
+    sum += UnitsOf(a, ts), cnt += ts > 0;
+  }
+  int incl = sum, incl_cnt = cnt;  // inclusive scans inside the wave, then the waves' totals
 #pragma unroll
   for (int o = 1; o < 64; o <<= 1) {
-    const int v = __shfl_up(incl, o, 64);
-    if (t % 64 >= o) incl += v;
+    const int v = __shfl_up(incl, o, 64), vc = __shfl_up(incl_cnt, o, 64);
+    if (t % 64 >= o) incl += v, incl_cnt += vc;
   }
-  if (t % 64 == 63) wave_sum[t / 64] = incl;
+  if (t % 64 == 63) wave_sum[t / 64][0] = incl, wave_sum[t / 64][1] = incl_cnt;
   __syncthreads();
-  int base = incl - sum, total = 0;
+  int base = incl - sum, base_cnt = incl_cnt - cnt, total = 0, total_cnt = 0;
 #pragma unroll
   for (int w = 0; w < NT / 64; ++w) {
-    if (w < t / 64) base += wave_sum[w];
-    total += wave_sum[w];
+    if (w < t / 64) base += wave_sum[w][0], base_cnt += wave_sum[w][1];
+    total += wave_sum[w][0], total_cnt += wave_sum[w][1];
   }
   if (k == 0) {
     int before = base;
-    for (int s = s0; s < s1; ++s) a.tprefix[s] = before, before += TilesOf(a, s);
+    for (int s = s0; s < s1; ++s) a.tprefix[s] = before, before += UnitsOf(a, TilesOf(a, s));
     if (t == 0) a.tprefix[a.n_seqs] = total;
   }
-  const long long line = static_cast<long long>(total) * H, A = ChunkTiles(a, line);
+  const long long line = static_cast<long long>(total) * H, A = ChunkUnits(a, line);
   const long long start = ChunkStart(a, A, k), end = min(ChunkStart(a, A, k + 1), line);
   if (start >= end) return int4{-1, 0, 0, 0};  // the same for every thread
-  if (static_cast<long long>(base) * H <= start && start < static_cast<long long>(base + sum) * H) {
-    int before = base;
+  if (t == 0 && end == line) tiles_at[1] = static_cast<long long>(total - c * total_cnt) * H;
+  // tiles before line position x, and where x lies, for the thread whose slice holds x
+  auto locate = [&](long long x, int4* where, long long* tiles) {
+    if (x < static_cast<long long>(base) * H || x >= static_cast<long long>(base + sum) * H) return;
+    int before = base, before_cnt = base_cnt;
     for (int s = s0; s < s1; ++s) {
-      const int ts = TilesOf(a, s);
-      if (start < static_cast<long long>(before + ts) * H) {
-        const int r = static_cast<int>(start - static_cast<long long>(before) * H);
-        *found = int4{s, r / ts, r % ts, static_cast<int>(end - start)};
-        break;
+      const int ts = TilesOf(a, s), units = UnitsOf(a, ts);
+      if (x < static_cast<long long>(before + units) * H) {
+        const int r = static_cast<int>(x - static_cast<long long>(before) * H);
+        const int h = r / units, first = max(r % units - c, 0);
+        *tiles = static_cast<long long>(before - c * before_cnt) * H + static_cast<long long>(h) * ts + first;
+        if (where != nullptr) *where = int4{s, h, first, 0};
+        return;
       }
-      before += ts;
+      before += units, before_cnt += ts > 0;
     }
-  }
+  };
+  locate(start, found, &tiles_at[0]);
+  if (end < line) locate(end, nullptr, &tiles_at[1]);
   __syncthreads();
-  return *found;
+  int4 rec = *found;
+  rec.w = static_cast<int>(tiles_at[1] - tiles_at[0]);
+  if (rec.w <= 0) return int4{-1, 0, 0, 0};  // the chunk lies inside a pair's first units
+  return rec;
 }
 
 // Position of a wave on its chunk: the pair (s, h) it stands on, which of the chunk's tiles belong to that pair
@@ -288,14 +309,15 @@ void DattnPart(const DecodeArgs a) {
   __shared__ __align__(16) _Float16 lvs_all[kWavesPerGroup][NB][kTile];
   __shared__ __align__(16) uint8_t lvq_all[kWavesPerGroup][FMT == 8 ? NVB * 1024 : 16];  // half a tile of V codes on its way in (q8_0)
   __shared__ int next_tile;
-  __shared__ int wave_sum[kWavesPerGroup];
+  __shared__ int wave_sum[kWavesPerGroup][2];
   __shared__ int4 chunk_rec;
+  __shared__ long long chunk_tiles[2];
   auto& lq = lq_all[wave];
   auto& lp = lp_all[wave];
   auto& lvs = lvs_all[wave];
   auto& lvq = lvq_all[wave];
 
-  const int4 rec = ChunkRecord<64 * kWavesPerGroup>(a, blockIdx.x, wave_sum, &chunk_rec);
+  const int4 rec = ChunkRecord<64 * kWavesPerGroup>(a, blockIdx.x, wave_sum, &chunk_rec, chunk_tiles);
   if (rec.x < 0) return;
   const int chunk_n = rec.w;
   if (threadIdx.x == 0) next_tile = 0;
@@ -637,10 +659,10 @@ __global__ __launch_bounds__(kReduceThreads) void DattnReduce(const DecodeArgs a
     if (t < D) a.out[o + t] = 0.0f;
     return;
   }
-  const int before = a.tprefix[s];  // tiles of the sequences before this one, and tiles on the line
-  const long long A_ = ChunkTiles(a, static_cast<long long>(a.tprefix[a.n_seqs]) * H);
+  // line units of the sequences before this one and of the whole line; the pair's tiles follow its first units
+  const long long A_ = ChunkUnits(a, static_cast<long long>(a.tprefix[a.n_seqs]) * H);
   const int pair = s * H + h;
-  const long long first = static_cast<long long>(before) * H + static_cast<long long>(h) * ts;
+  const long long first = static_cast<long long>(a.tprefix[s]) * H + static_cast<long long>(h) * UnitsOf(a, ts) + a.pair_cost;
   const int k0 = ChunkOf(a, A_, first), k1 = ChunkOf(a, A_, first + ts - 1);
   const size_t p0 = size_t(k0 + pair) * a.wpc, p1 = size_t(k1 + pair + 1) * a.wpc;
   constexpr int NW = kReduceThreads / 64;
@@ -712,7 +734,7 @@ __global__ __launch_bounds__(kReduceThreads) void DattnReduce(const DecodeArgs a
 
 // Workspace layout and chunk count, from the host's bounds alone (the lengths are on the device).
 struct Plan {
-  int32_t max_len, n_chunks, wpc, min_chunk_tiles;
+  int32_t max_len, n_chunks, wpc, min_chunk_tiles, pair_cost;
   int32_t share[9];
   size_t off_tprefix, off_ml, off_acc, bytes;
 };
@@ -740,6 +762,7 @@ Plan MakePlan(const Geom& g, int32_t n_seqs, int32_t max_seq_len) {
   // one 8-wave workgroup per CU (two waves per SIMD)
   p.wpc = kWavesPerGroup;
   p.min_chunk_tiles = EnvInt("YAHKV_DECODE_MIN_CHUNK_TILES", 2 * kWavesPerGroup, 1, 1 << 20);
+  p.pair_cost = EnvInt("YAHKV_DECODE_PAIR_COST", 8, 0, 1 << 10);
   p.n_chunks = EnvInt("YAHKV_DECODE_CHUNKS", ComputeUnits(), 1, 1 << 20);
   p.n_chunks =
       static_cast<int32_t>(std::min<int64_t>(p.n_chunks, (line_max + p.min_chunk_tiles - 1) / p.min_chunk_tiles));
@@ -787,7 +810,7 @@ int Prepare(const yahkv_geometry* g, int32_t page_table_stride, const int32_t* s
   a->tprefix = reinterpret_cast<int32_t*>(ws + p.off_tprefix);
   a->ml = reinterpret_cast<float*>(ws + p.off_ml);
   a->acc = reinterpret_cast<float*>(ws + p.off_acc);
-  a->n_chunks = p.n_chunks, a->wpc = p.wpc, a->min_chunk_tiles = p.min_chunk_tiles;
+  a->n_chunks = p.n_chunks, a->wpc = p.wpc, a->min_chunk_tiles = p.min_chunk_tiles, a->pair_cost = p.pair_cost;
   std::copy(p.share, p.share + 9, a->share);
   return YAHKV_OK;
 }
