@@ -768,7 +768,7 @@ Plan MakePlan(const Geom& g, int32_t n_seqs, int32_t max_seq_len) {
       static_cast<int32_t>(std::min<int64_t>(p.n_chunks, (line_max + p.min_chunk_tiles - 1) / p.min_chunk_tiles));
   // Relative speeds of the eight XCDs of an MI355X on this kernel (tiles per unit of time, measured with all of
   // them reading at once); YAHKV_DECODE_XCD_WEIGHTS="w0,...,w7" overrides them. Shares are kept above half the mean.
-  int w[8] = {1052, 929, 1058, 967, 1048, 962, 1056, 927};
+  int w[8] = {1050, 942, 1055, 962, 1046, 958, 1052, 942};
   if (const char* e = std::getenv("YAHKV_DECODE_XCD_WEIGHTS")) {
     int v[8];
     if (std::sscanf(e, "%d,%d,%d,%d,%d,%d,%d,%d", v, v + 1, v + 2, v + 3, v + 4, v + 5, v + 6, v + 7) == 8)
