@@ -67,3 +67,20 @@ def test_large_batch_of_short_sequences(yahkv, torch_gpu):
     assert rel_err(got, want) < TOL
     for s in np.flatnonzero(np.array(lens) == 0)[:20]:
         assert not got[s].any()
+
+
+def test_chunks_of_one_or_two_units(yahkv, torch_gpu, monkeypatch):
+    """The finest cut the planner allows (asked for one tile per chunk; it keeps two line units): the eight chunks of
+    a group then differ by whole units, and none inside a pair's stretch may come out empty, because the reduce reads
+    the partials of every chunk between a pair's first and last."""
+    monkeypatch.setenv("YAHKV_DECODE_CHUNKS", "1000")
+    monkeypatch.setenv("YAHKV_DECODE_MIN_CHUNK_TILES", "1")
+    rng = np.random.default_rng(239)
+    lens = [91, 627, 798, 425, 27, 408, 417, 18, 247, 137, 144, 127, 70, 839, 137, 273]
+    for fmt, pair_cost in ((4, "8"), (8, "0"), (8, "3")):
+        monkeypatch.setenv("YAHKV_DECODE_PAIR_COST", pair_cost)
+        g, table, host, dev, _ = setup(yahkv, torch_gpu, fmt, 8, 2, 256, 64, lens, seed=239, fill=0x7F)
+        q = to_bf16_f32(rng.standard_normal((len(lens), 8, 256)))
+        got = gpu_attend(yahkv, torch_gpu, dev, table, lens, q, 0.0625, max_len=896)
+        assert np.all(np.isfinite(got))
+        assert rel_err(got, oracle.decode_attend(host, table, lens, q, 0.0625)) < TOL

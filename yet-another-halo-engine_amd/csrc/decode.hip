@@ -761,7 +761,9 @@ Plan MakePlan(const Geom& g, int32_t n_seqs, int32_t max_seq_len) {
   // Tuning knobs; the environment overrides are for experiments.
   // one 8-wave workgroup per CU (two waves per SIMD)
   p.wpc = kWavesPerGroup;
-  p.min_chunk_tiles = EnvInt("YAHKV_DECODE_MIN_CHUNK_TILES", 2 * kWavesPerGroup, 1, 1 << 20);
+  // at least 2: with chunks of one unit the smaller shares of a group of eight would round to nothing, and the reduce
+  // counts on every chunk inside a pair's stretch of the line having left partials
+  p.min_chunk_tiles = EnvInt("YAHKV_DECODE_MIN_CHUNK_TILES", 2 * kWavesPerGroup, 2, 1 << 20);
   p.pair_cost = EnvInt("YAHKV_DECODE_PAIR_COST", 8, 0, 1 << 10);
   p.n_chunks = EnvInt("YAHKV_DECODE_CHUNKS", ComputeUnits(), 1, 1 << 20);
   p.n_chunks =
