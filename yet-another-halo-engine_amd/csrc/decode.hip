@@ -645,18 +645,22 @@ void DattnPart(const DecodeArgs a) {
 // thread each, and the partials that weigh something are listed in order. The threads then form groups of D / 4
 // lanes (four dims a lane); each group sums every n-th listed partial, several 16-byte loads in flight and no
 // branch inside, and the groups' sums meet in LDS. A single long sequence leaves hundreds of partials per pair and
-// only a few workgroups here, which is why the partials are spread over the workgroup as well.
+// only a few workgroups here, which is why the partials are spread over the workgroup as well, and why a small batch
+// is launched with several workgroups per pair (gridDim.z), each with its own stretch of the head's dims: what bounds
+// such a launch is the number of partial rows in flight.
 constexpr int kReduceThreads = 256;  // also the number of partial slots weighed at a time
 constexpr int kReduceDepth = 4;      // partials a group loads together
+constexpr int kReduceMinDims = 32;   // fewest dims of a head one workgroup sums
 __global__ __launch_bounds__(kReduceThreads) void DattnReduce(const DecodeArgs a) {
   const Geom g = a.g;
   const int G = g.group(), H = g.n_kv, D = g.hd;
   const int hq = blockIdx.x, s = blockIdx.y, t = threadIdx.x;
   const int h = hq / G, gi = hq % G;
-  const size_t o = (size_t(s) * g.n_q + hq) * D;
+  const int DZ = D / gridDim.z, d0 = blockIdx.z * DZ;  // this workgroup's dims are [d0, d0 + DZ)
+  const size_t o = (size_t(s) * g.n_q + hq) * D + d0;
   const int ts = TilesOf(a, s);
   if (ts <= 0) {  // length 0
-    if (t < D) a.out[o + t] = 0.0f;
+    if (t < DZ) a.out[o + t] = 0.0f;
     return;
   }
   // line units of the sequences before this one and of the whole line; the pair's tiles follow its first units
@@ -670,8 +674,8 @@ __global__ __launch_bounds__(kReduceThreads) void DattnReduce(const DecodeArgs a
   __shared__ int slot[kReduceThreads];
   __shared__ float red[NW];
   __shared__ int wave_n[NW];
-  __shared__ __align__(16) float sums[kReduceThreads * 4];  // [group][D]
-  __shared__ float lsums[kReduceThreads / 32];
+  __shared__ __align__(16) float sums[kReduceThreads * 4];  // [group][DZ]
+  __shared__ float lsums[kReduceThreads / (kReduceMinDims / 4)];
   // waves that got no tile of this pair left l = 0 (and no acc): they weigh nothing
   float M = kNegMax;
   for (size_t p = p0 + t; p < p1; p += kReduceThreads)
@@ -681,7 +685,7 @@ __global__ __launch_bounds__(kReduceThreads) void DattnReduce(const DecodeArgs a
   __syncthreads();
   M = red[0];
   for (int w = 1; w < NW; ++w) M = fmaxf(M, red[w]);
-  const int lanes = D / 4, n_groups = kReduceThreads / lanes, grp = t / lanes, dl = t % lanes;
+  const int lanes = DZ / 4, n_groups = kReduceThreads / lanes, grp = t / lanes, dl = t % lanes;
   float L = 0.0f;
   float4 A = {0.0f, 0.0f, 0.0f, 0.0f};
   for (size_t b0 = p0; b0 < p1; b0 += kReduceThreads) {
@@ -706,7 +710,7 @@ __global__ __launch_bounds__(kReduceThreads) void DattnReduce(const DecodeArgs a
       float4 v[kReduceDepth];
 #pragma unroll
       for (int j = 0; j < kReduceDepth; ++j)
-        v[j] = *reinterpret_cast<const float4*>(&a.acc[((b0 + slot[min(j0 + j, n - 1)]) * G + gi) * D + 4 * dl]);
+        v[j] = *reinterpret_cast<const float4*>(&a.acc[((b0 + slot[min(j0 + j, n - 1)]) * G + gi) * D + d0 + 4 * dl]);
 #pragma unroll
       for (int j = 0; j < kReduceDepth; ++j) {
         if (j0 + j < n) {
@@ -718,12 +722,12 @@ __global__ __launch_bounds__(kReduceThreads) void DattnReduce(const DecodeArgs a
       }
     }
   }
-  *reinterpret_cast<float4*>(&sums[grp * D + 4 * dl]) = A;
+  *reinterpret_cast<float4*>(&sums[grp * DZ + 4 * dl]) = A;
   if (dl == 0) lsums[grp] = L;
   __syncthreads();
-  if (t < D) {
+  if (t < DZ) {
     float v = 0.0f, lt = 0.0f;
-    for (int q = 0; q < n_groups; ++q) v += sums[q * D + t], lt += lsums[q];
+    for (int q = 0; q < n_groups; ++q) v += sums[q * DZ + t], lt += lsums[q];
     v /= lt;
     if (a.gate != nullptr) v *= 1.0f / (1.0f + __expf(-a.gate[o + t]));
     a.out[o + t] = v;
@@ -883,7 +887,13 @@ extern "C" int yahkv_decode_reduce(const yahkv_geometry* g, int32_t page_table_s
     return st;
   if (out == nullptr) return YAHKV_ERR_ARG;
   a.gate = gate, a.out = out;
-  hipLaunchKernelGGL(DattnReduce, dim3(a.g.n_q, n_seqs), dim3(kReduceThreads), 0, static_cast<hipStream_t>(stream), a);
+  // a small batch: more workgroups per (query head, sequence), each with a part of the dims, until the CUs have one
+  int split = 1;
+  while (int64_t(a.g.n_q) * n_seqs * split < ComputeUnits() && a.g.hd / (2 * split) >= kReduceMinDims) split *= 2;
+  split = EnvInt("YAHKV_DECODE_REDUCE_SPLIT", split, 1, a.g.hd / kReduceMinDims);
+  while (a.g.hd % split != 0 || (a.g.hd / split) % 4 != 0) --split;
+  hipLaunchKernelGGL(DattnReduce, dim3(a.g.n_q, n_seqs, split), dim3(kReduceThreads), 0,
+                     static_cast<hipStream_t>(stream), a);
   return LaunchStatus();
 }
 
