@@ -50,6 +50,21 @@ __device__ __forceinline__ float4 Load4(const void* src, size_t i, int dtype) {
   if (dtype == YAHKV_F16) return float4{WidenF16(h[0]), WidenF16(h[1]), WidenF16(h[2]), WidenF16(h[3])};
   return float4{WidenBf16(h[0]), WidenBf16(h[1]), WidenBf16(h[2]), WidenBf16(h[3])};
 }
+// The same in two steps, for loads that stay in flight while other work is done: the raw bytes, widened later.
+__device__ __forceinline__ uint4 LoadRaw4(const void* src, size_t i, int dtype) {
+  if (dtype == YAHKV_F32) return *reinterpret_cast<const uint4*>(static_cast<const float*>(src) + i);
+  const uint2 w = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(src) + i);
+  return uint4{w.x, w.y, 0u, 0u};
+}
+__device__ __forceinline__ float4 Widen4(uint4 w, int dtype) {
+  if (dtype == YAHKV_F32)
+    return float4{__builtin_bit_cast(float, w.x), __builtin_bit_cast(float, w.y), __builtin_bit_cast(float, w.z),
+                  __builtin_bit_cast(float, w.w)};
+  const uint16_t h[4] = {static_cast<uint16_t>(w.x & 0xFFFF), static_cast<uint16_t>(w.x >> 16),
+                         static_cast<uint16_t>(w.y & 0xFFFF), static_cast<uint16_t>(w.y >> 16)};
+  if (dtype == YAHKV_F16) return float4{WidenF16(h[0]), WidenF16(h[1]), WidenF16(h[2]), WidenF16(h[3])};
+  return float4{WidenBf16(h[0]), WidenBf16(h[1]), WidenBf16(h[2]), WidenBf16(h[3])};
+}
 __device__ __forceinline__ void Store4(void* dst, size_t i, int dtype, float4 v) {
   if (dtype == YAHKV_F32) {
     *reinterpret_cast<float4*>(static_cast<float*>(dst) + i) = v;
@@ -236,17 +251,25 @@ __global__ __launch_bounds__(64 * kPageWaves) void AppendPages(const RopeArgs a)
   // of its four dims, the codes of four neighbouring tokens, which is one dword of the V image instead of four bytes.
   // (The image's rows are padded by a dword: with rows of exactly PT bytes the 64 lanes of such a store would all
   // hit one LDS bank.)
-  for (int q = t_lo / 4 + wave; 4 * q < t_hi; q += kPageWaves) {
-    float4 kx[4], vx[4];
+  // The rows of the wave's next four tokens are requested before the current four are quantized.
+  uint4 rk[4], rv[4];
+  auto request = [&](int q) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int t = 4 * q + j;
-      kx[j] = vx[j] = float4{0.0f, 0.0f, 0.0f, 0.0f};
+      rk[j] = rv[j] = uint4{0u, 0u, 0u, 0u};  // reads as 0.0 in every source type
       if (t >= t_lo && t < t_hi && has) {
         const size_t row = ((size_t(s) * a.n_new + token_at(pi * PT + t)) * H + h) * D;
-        kx[j] = Load4(a.k_src, row + d0, a.src_dtype), vx[j] = Load4(a.v_src, row + d0, a.src_dtype);
+        rk[j] = LoadRaw4(a.k_src, row + d0, a.src_dtype), rv[j] = LoadRaw4(a.v_src, row + d0, a.src_dtype);
       }
     }
+  };
+  if (4 * (t_lo / 4 + wave) < t_hi) request(t_lo / 4 + wave);
+  for (int q = t_lo / 4 + wave; 4 * q < t_hi; q += kPageWaves) {
+    float4 kx[4], vx[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) kx[j] = Widen4(rk[j], a.src_dtype), vx[j] = Widen4(rv[j], a.src_dtype);
+    if (4 * (q + kPageWaves) < t_hi) request(q + kPageWaves);
     uint32_t vc[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
