@@ -248,6 +248,23 @@ __device__ __forceinline__ h8v NibblesHi8(uint32_t w0, uint32_t w1) {
   return h8v{a[0], a[1], b[0], b[1], c[0], c[1], d[0], d[1]};
 }
 
+// The same without the subtraction, for the first product: 1024 + 128 + code (q8_0), 1024 + nibble (low nibbles),
+// 1024 + 16 * nibble (high nibbles, in place). What the constants add to a score depends on the queries alone and is
+// taken off the block's sum afterwards (see `lcorr` in the kernel).
+__device__ __forceinline__ h8v RawCodes8(uint32_t w0, uint32_t w1) {
+  const uint32_t x0 = w0 ^ 0x80808080u, x1 = w1 ^ 0x80808080u;
+  const uint4 r = {__builtin_amdgcn_perm(0x64646464u, x0, 0x04010400u), __builtin_amdgcn_perm(0x64646464u, x0, 0x04030402u),
+                   __builtin_amdgcn_perm(0x64646464u, x1, 0x04010400u), __builtin_amdgcn_perm(0x64646464u, x1, 0x04030402u)};
+  return __builtin_bit_cast(h8v, r);
+}
+template <uint32_t MASK>
+__device__ __forceinline__ h8v RawNibbles8(uint32_t w0, uint32_t w1) {
+  const uint32_t x0 = w0 & MASK, x1 = w1 & MASK;
+  const uint4 r = {__builtin_amdgcn_perm(0x64646464u, x0, 0x04010400u), __builtin_amdgcn_perm(0x64646464u, x0, 0x04030402u),
+                   __builtin_amdgcn_perm(0x64646464u, x1, 0x04010400u), __builtin_amdgcn_perm(0x64646464u, x1, 0x04030402u)};
+  return __builtin_bit_cast(h8v, r);
+}
+
 // Eight consecutive query elements as f16 (bf16 and f16 sources convert exactly in the normal f16 range).
 __device__ __forceinline__ h8v LoadQ8(const void* q, size_t i, int dt) {
   h8v r;
@@ -304,7 +321,14 @@ void DattnPart(const DecodeArgs a) {
   // never looked at). Entry (b, sub, hf, row) holds the dims of the 8 codes a key lane of that half feeds to
   // instruction `sub`: 32 b + 16 hf + 8 sub + 0..7 for q8_0 (bytes 8 sub .. of its 16), 32 b + 16 sub + 8 hf + 0..7
   // for q4_0 (low nibbles, then high nibbles, of its 8 bytes).
+  // The first product runs on codes with their f16 constant still on (1152 + code for q8_0; 1024 + n for low
+  // nibbles; 1024 + 16 n for high nibbles, whose queries are stored divided by 16): per block and head that adds
+  // (sum of the queries of the block's dims) x 1152 for q8_0, x 1032 (low) and x 72 (high) for q4_0, the -8 of
+  // the nibbles included. `lcorr` holds that sum per (block, head); it comes off the block's product before the
+  // block scale goes on. The products stay exact in f32 (11 x 11 bits), and the sums of 32 of them carry an error of
+  // 2^-24 of 1152 x sum |q|, which is 1e-5 of a typical score.
   __shared__ __align__(16) _Float16 lq_all[kWavesPerGroup][NB][2][2][8][8];
+  __shared__ __align__(16) float lcorr_all[kWavesPerGroup][NB][8];
   __shared__ __align__(16) _Float16 lp_all[kWavesPerGroup][kMaxGroup][kTile];
   __shared__ __align__(16) _Float16 lvs_all[kWavesPerGroup][NB][kTile];
   __shared__ __align__(16) uint8_t lvq_all[kWavesPerGroup][FMT == 8 ? NVB * 1024 : 16];  // half a tile of V codes on its way in (q8_0)
@@ -313,6 +337,7 @@ void DattnPart(const DecodeArgs a) {
   __shared__ int4 chunk_rec;
   __shared__ long long chunk_tiles[2];
   auto& lq = lq_all[wave];
+  auto& lcorr = lcorr_all[wave];
   auto& lp = lp_all[wave];
   auto& lvs = lvs_all[wave];
   auto& lvq = lvq_all[wave];
@@ -435,8 +460,8 @@ void DattnPart(const DecodeArgs a) {
   };
   // the 8 codes of block b this lane feeds to instruction `sub` of the block's pair
   auto kcodes = [&](int b, int sub) -> h8v {
-    if constexpr (Q8) return Codes8(kb[b][2 * sub], kb[b][2 * sub + 1]);
-    return sub == 0 ? NibblesLo8(kb[b][0], kb[b][1]) : NibblesHi8(kb[b][0], kb[b][1]);
+    if constexpr (Q8) return RawCodes8(kb[b][2 * sub], kb[b][2 * sub + 1]);
+    return sub == 0 ? RawNibbles8<0x0F0F0F0Fu>(kb[b][0], kb[b][1]) : RawNibbles8<0xF0F0F0F0u>(kb[b][0], kb[b][1]);
   };
   // scores of the 32 keys in kb against all heads: two blocks (two accumulator chains) at a time
   auto scores = [&](int tt) {
@@ -448,6 +473,9 @@ void DattnPart(const DecodeArgs a) {
       const h8v qa1 = *reinterpret_cast<const h8v*>(&lq[b][1][half][n32 % 8][0]);
       const h8v qb0 = *reinterpret_cast<const h8v*>(&lq[b + 1][0][half][n32 % 8][0]);
       const h8v qb1 = *reinterpret_cast<const h8v*>(&lq[b + 1][1][half][n32 % 8][0]);
+      const float4 k0 = *reinterpret_cast<const float4*>(&lcorr[b][4 * half]);
+      const float4 k1 = *reinterpret_cast<const float4*>(&lcorr[b + 1][4 * half]);
+      const float kc0[4] = {k0.x, k0.y, k0.z, k0.w}, kc1[4] = {k1.x, k1.y, k1.z, k1.w};
       f16v c0 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}, c1 = c0;
       c0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(qa0, kcodes(b, 0), c0, 0, 0, 0);
       c1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(qb0, kcodes(b + 1, 0), c1, 0, 0, 0);
@@ -457,7 +485,8 @@ void DattnPart(const DecodeArgs a) {
       const float d0 = WidenF16(static_cast<uint16_t>(w & 0xFFFF)) * qk_scale;
       const float d1 = WidenF16(static_cast<uint16_t>(w >> 16)) * qk_scale;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) sc[tt][r] = __builtin_fmaf(c1[r], d1, __builtin_fmaf(c0[r], d0, sc[tt][r]));
+      for (int r = 0; r < 4; ++r)
+        sc[tt][r] = __builtin_fmaf(c1[r] - kc1[r], d1, __builtin_fmaf(c0[r] - kc0[r], d0, sc[tt][r]));
       // The empty asm pins the scaled sums here, so the 32x32 accumulators die before the next pair of blocks starts
       // (otherwise every pair's accumulators stay live to the end and the kernel spills).
       asm volatile("" : "+v"(sc[tt][0]), "+v"(sc[tt][1]), "+v"(sc[tt][2]), "+v"(sc[tt][3]));
@@ -548,8 +577,20 @@ void DattnPart(const DecodeArgs a) {
                       // head of the loop the same as on the way round, see below
 #pragma unroll
     for (int e = 0; e < QE; ++e) {
-      const int i = lane + 64 * e;
-      *reinterpret_cast<h8v*>(&lq[i / 32][(i / 16) % 2][(i / 8) % 2][i % 8][0]) = qreg[e];
+      const int i = lane + 64 * e, sub = (i / 16) % 2;
+      // what the codes' constants add to the block's product for head i % 8: the four entries of a (block, head)
+      // lie in lanes 8 apart
+      float t = 0.0f;
+#pragma unroll
+      for (int k = 0; k < 8; ++k) t += static_cast<float>(qreg[e][k]);
+      t *= Q8 ? 1152.0f : (sub == 0 ? 1032.0f : 72.0f);
+      t += __shfl_xor(t, 8, 64);
+      t += __shfl_xor(t, 16, 64);
+      if (lane % 32 < 8) lcorr[i / 32][i % 8] = t;
+      if constexpr (!Q8) {
+        if (sub == 1) qreg[e] *= static_cast<_Float16>(0.0625f);  // high nibbles come as 16 n
+      }
+      *reinterpret_cast<h8v*>(&lq[i / 32][sub][(i / 8) % 2][i % 8][0]) = qreg[e];
     }
 #pragma unroll
     for (int r = 0; r < 4; ++r) m[r] = kNegMax, lsum[r] = 0.0f;
@@ -609,10 +650,13 @@ void DattnPart(const DecodeArgs a) {
           *reinterpret_cast<uint4*>(&lvs[b][8 * chunk]) = uint4{w[0], w[1], w[2], w[3]};
         }
       }
+      // once a pair's maximum has settled (a few tiles into a long sequence) every factor is exactly 1
+      if (__builtin_amdgcn_ballot_w64(alpha[0] != 1.0f || alpha[1] != 1.0f || alpha[2] != 1.0f || alpha[3] != 1.0f) != 0) {
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt)
+        for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) o[nt][r] *= alpha[r];
+          for (int r = 0; r < 4; ++r) o[nt][r] *= alpha[r];
+      }
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
