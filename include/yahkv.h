@@ -179,7 +179,9 @@ size_t yahkv_prefill_workspace_bytes(const yahkv_geometry* g, int32_t n_seqs, in
 /* The two dispatches of the workspace path, for callers that queue them separately (as the reference does with
  * yah_kdeq8 / yah_vdeq8 and yah_attn_wmma, loom_prefill.hpp:3378-3416): decode keys 0 .. prefix_len[s] + chunk_len
  * of every sequence into bf16 tiles in the workspace; then attention of the chunk's queries over those tiles. The
- * tiles stay valid for further queries of the same chunk (e.g. another slice of heads) until the pools change. */
+ * tiles stay valid for further queries of the same chunk (e.g. another slice of heads) until the pools change.
+ * One sequence's tiles of one kv head must stay under 2 GiB (max_prefix_len + chunk_len up to 2^21 tokens at
+ * head_dim 256, 2^22 at 128): longer ones return YAHKV_ERR_SHAPE. */
 int yahkv_prefill_decode_tiles(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
                                int32_t page_table_stride, const int32_t* prefix_len, int32_t n_seqs,
                                int32_t max_prefix_len, int32_t chunk_len, void* workspace, size_t workspace_bytes,

@@ -516,7 +516,10 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
   const int n_keys = min(prefix + q0 + kQueries, prefix + a.chunk_len);
   const int n_tiles = (n_keys + kKeys - 1) / kKeys;
 
-  __shared__ __align__(1024) char lds[2][TIMG];
+  // two K halves and three V halves of tile images: V(t + 2) is on its way in while V(t) and V(t + 1) are in use,
+  // which gives its copies a whole tile's time to land (160 KB at D = 256: all the LDS of a CU)
+  static_assert(TIMG == 2 * KIMG, "the two halves of an image have the same size");
+  __shared__ __align__(1024) char lds[5][KIMG];  // [0], [1]: K halves; [2] .. [4]: V halves
 
   b8v qb[RB][KS];
   int qpos[RB], head[RB];
@@ -540,19 +543,23 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
     for (int dt = 0; dt < NDT; ++dt) o[i][dt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
   }
   const float sscale = a.scale * 1.4426950408889634f;
-  const char* src = img + size_t(pair) * tiles_per_pair * TIMG + size_t(lane) * 16;
   // Copy j (of kCopies) of this wave's share of a tile image into the LDS buffer tile % 2: pieces j < kCopies / 2 are
-  // the K half, the others the V half. Direct global-to-LDS loads: no registers, no vector instructions. The copies
+  // the K half, the others the V half. Direct global-to-LDS loads: no registers, no vector instructions; through a
+  // buffer resource of the pair's images (scalar base and offset, one 32-bit lane offset), which issues faster
+  // than the flat form with its 64-bit address per lane (2 % of the kernel's time). The copies
   // are spread over the arithmetic, because the CU's vector memory path moves about 39 bytes per cycle (measured:
   // 26 cycles per 1 KB wave-wide load, 1700 cycles per 64 KB image) and a burst of them stalls every wave.
+  const auto img_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<char*>(img) + size_t(pair) * tiles_per_pair * TIMG, 0, 0x7fffffff, 0x00020000);
   auto copy_part = [&](int tile, int j) {
     const int c = wave + 4 * j;
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + size_t(tile) * TIMG + c * 1024),
-                                     (__attribute__((address_space(3))) void*)(lds[tile % 2] + c * 1024), 16, 0, 0);
+    char* dst = j < kCopies / 2 ? lds[tile % 2] + c * 1024 : lds[2 + tile % 3] + (c * 1024 - KIMG);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(img_rsrc, (__attribute__((address_space(3))) void*)dst, 16, lane * 16,
+                                             tile * TIMG + c * 1024, 0, 0);
   };
   // byte offsets of this lane's operand reads within an image; the XOR with qn % 8 undoes the images' swizzle
   const int sw = qn % 8;
-  const int koff = qn * (2 * D), voff = KIMG + qn * 128;
+  const int koff = qn * (2 * D), voff = qn * 128;
   auto read_k = [&](const char* buf, int ks, int kt) -> b8v {
     return *reinterpret_cast<const b8v*>(buf + koff + kt * 16 * (2 * D) + 16 * ((4 * ks + jg) ^ sw));
   };
@@ -656,17 +663,18 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
     }
   };
 
-  // Schedule. Iteration t has the scores S^T(t) in registers, K(t + 1) and V(t) in LDS. It computes S^T(t + 1) on the
-  // matrix cores while the vector units turn S^T(t) into numerators (one wave per SIMD: only instructions of the same
-  // wave can overlap), then V^T P^T(t); meanwhile K(t + 2) and V(t + 1) are copied into the halves of the two LDS
-  // buffers that are free. One barrier per tile. Tiles that need the causal mask (the last one or two) and the last
+  // Schedule. Iteration t has the scores S^T(t) in registers, K(t + 1), V(t) and V(t + 1) in LDS (the last maybe
+  // still landing). It computes S^T(t + 1) on the matrix cores while the vector units turn S^T(t) into numerators
+  // (one wave per SIMD: only instructions of the same wave can overlap), then V^T P^T(t); meanwhile K(t + 2) is
+  // copied where K(t) was, and after it V(t + 2) where V(t - 1) was. One barrier per tile; it waits for the K copies,
+  // issued half a tile earlier, and for the V copies of the iteration before, not for the ones just issued. Tiles that need the causal mask (the last one or two) and the last
   // tile take the plain path below the pipelined loop.
   const int n_full = min(n_tiles, (prefix + q0 + 1) / kKeys);  // tiles every query of the workgroup sees whole
   const int n_pipe = min(n_full, n_tiles - 1);
 #pragma unroll
   for (int j = 0; j < kCopies; ++j) copy_part(0, j);
 #pragma unroll
-  for (int j = 0; j < kCopies / 2; ++j) copy_part(min(1, n_tiles - 1), j);  // K(1) (K(0) again if there is no tile 1)
+  for (int j = 0; j < kCopies; ++j) copy_part(min(1, n_tiles - 1), j);  // tile 1 (tile 0 again if there is none)
   __builtin_amdgcn_s_waitcnt(VmCnt(0));
   __syncthreads();
   f4v st[RB][4];
@@ -723,13 +731,16 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
-    pv_product(lds[tile % 2], pv, tile + 1);
+    pv_product(lds[2 + tile % 3], pv, min(tile + 2, n_tiles - 1));
 #pragma unroll
     for (int i = 0; i < RB; ++i)
 #pragma unroll
       for (int kt = 0; kt < 4; ++kt) st[i][kt] = sn[i][kt];
-    __builtin_amdgcn_s_waitcnt(VmCnt(0));  // this wave's pieces of K(tile + 2) and V(tile + 1) have landed
-    __syncthreads();                       // ... and everybody's; everybody is done with K(tile + 1) and V(tile)
+    // The copies complete in the order of their issue: all but the newest kCopies / 2, the pieces of V(tile + 2),
+    // have landed, this wave's pieces of K(tile + 2) and V(tile + 1) among them.
+    // (A bare barrier: __syncthreads() carries a release fence, which waits for every copy in flight.)
+    __builtin_amdgcn_s_waitcnt(VmCnt(kCopies / 2) & 0xF0FF);  // and lgkmcnt(0): this wave's LDS reads have returned
+    __builtin_amdgcn_s_barrier();  // ... and everybody's; everybody is done with K(tile + 1) and V(tile)
   }
   // ---- the last tiles, one phase after the other: masked softmax, second product, then the next tile's scores
   for (; tile < n_tiles; ++tile) {
@@ -749,7 +760,7 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
       move_reference(i, row_max(st[i]));
       numerators(i, st[i], pv[i]);
     }
-    pv_product(lds[tile % 2], pv, more ? tile + 1 : -1);
+    pv_product(lds[2 + tile % 3], pv, tile + 2 < n_tiles ? tile + 2 : -1);
     if (more) {
       const char* kbuf = lds[(tile + 1) % 2];
       clear(st);
@@ -879,6 +890,8 @@ extern "C" int yahkv_prefill_attend_tiles(const yahkv_geometry* g, const yahkv_p
   if (const int rc = CheckWorkspace(a, workspace, workspace_bytes)) return rc;
   const char* img = static_cast<const char*>(workspace);
   const int tiles = TilesPerPair(max_prefix_len, chunk_len);
+  // the attention kernel addresses a pair's images with 32-bit offsets
+  if (int64_t(tiles) * (2 * kKeys * a.g.hd * 2) > 0x7fffffffLL) return YAHKV_ERR_SHAPE;
   hipStream_t st = static_cast<hipStream_t>(stream);
   // At head_dim 128, three row blocks per wave (three heads per workgroup) when the GQA group is a multiple of
   // three: each tile image copied to LDS and each operand read from it then serves half as much arithmetic again.
