@@ -501,6 +501,9 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
   constexpr int KS = D / 32, NDT = D / 16, kHeadsPerGroup = RB;
   constexpr int KIMG = kKeys * D * 2, TIMG = TileImageBytes<D>();
   constexpr int kCopies = TIMG / 1024 / 4;  // 1 KB wave-wide copies per wave and tile
+  // How far the operand reads run ahead of the products that use them, in steps of the first product (8 matrix
+  // instructions each) and in 16-dim tiles of the second (4 each). Measured: 1 and 6 (2 and 2: 3 % slower).
+  constexpr int KP = 1, VP = 6;
   static_assert(kCopies == KS + NDT / 2, "one copy per step of the first product and per two of the second");
   const Geom g = a.g;
   const int G = g.group(), H = g.n_kv;
@@ -563,17 +566,23 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
   auto read_k = [&](const char* buf, int ks, int kt) -> b8v {
     return *reinterpret_cast<const b8v*>(buf + koff + kt * 16 * (2 * D) + 16 * ((4 * ks + jg) ^ sw));
   };
-  // One 32-dim step of S^T = K Q^T: the A operands of step ks + 1 are read before the products of step ks.
-  auto k_step = [&](const char* buf, int ks, b8v (&ka)[2][4], f4v (&st)[RB][4]) {
-    if (ks + 1 < KS) {
+  // One 32-dim step of S^T = K Q^T: the A operands of step ks + KP are read before the products of step ks.
+  auto k_first = [&](const char* buf, b8v (&ka)[KP + 1][4]) {
 #pragma unroll
-      for (int kt = 0; kt < 4; ++kt) ka[(ks + 1) % 2][kt] = read_k(buf, ks + 1, kt);
+    for (int ks = 0; ks < KP; ++ks)
+#pragma unroll
+      for (int kt = 0; kt < 4; ++kt) ka[ks][kt] = read_k(buf, ks, kt);
+  };
+  auto k_step = [&](const char* buf, int ks, b8v (&ka)[KP + 1][4], f4v (&st)[RB][4]) {
+    if (ks + KP < KS) {
+#pragma unroll
+      for (int kt = 0; kt < 4; ++kt) ka[(ks + KP) % (KP + 1)][kt] = read_k(buf, ks + KP, kt);
     }
 #pragma unroll
     for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
       for (int i = 0; i < RB; ++i)
-        st[i][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[ks % 2][kt], qb[i][ks], st[i][kt], 0, 0, 0);
+        st[i][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[ks % (KP + 1)][kt], qb[i][ks], st[i][kt], 0, 0, 0);
   };
   auto clear = [&](f4v (&st)[RB][4]) {
 #pragma unroll
@@ -637,9 +646,11 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
     auto read_v = [&](int dt, int s2) -> b8v {
       return *reinterpret_cast<const b8v*>(buf + voff + dt * 16 * 128 + 16 * ((4 * s2 + jg) ^ sw));
     };
-    b8v va[3][2];  // read two 16-dim tiles ahead
+    b8v va[VP + 1][2];  // read VP 16-dim tiles ahead
 #pragma unroll
-    for (int s2 = 0; s2 < 2; ++s2) va[0][s2] = read_v(0, s2), va[1][s2] = read_v(1, s2);
+    for (int dt = 0; dt < VP; ++dt)
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) va[dt][s2] = read_v(dt, s2);
 #pragma unroll
     for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
@@ -647,15 +658,15 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
         lacc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(OnesBf16(), pv[i][s2], lacc[i], 0, 0, 0);
 #pragma unroll
     for (int dt = 0; dt < NDT; ++dt) {
-      if (dt + 2 < NDT) {
+      if (dt + VP < NDT) {
 #pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2) va[(dt + 2) % 3][s2] = read_v(dt + 2, s2);
+        for (int s2 = 0; s2 < 2; ++s2) va[(dt + VP) % (VP + 1)][s2] = read_v(dt + VP, s2);
       }
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
         for (int i = 0; i < RB; ++i)
-          o[i][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[dt % 3][s2], pv[i][s2], o[i][dt], 0, 0, 0);
+          o[i][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[dt % (VP + 1)][s2], pv[i][s2], o[i][dt], 0, 0, 0);
       if (dt % 2 == 1) {
         if (v_tile >= 0) copy_part(v_tile, KS + dt / 2);
         __builtin_amdgcn_sched_barrier(0);
@@ -680,9 +691,8 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
   f4v st[RB][4];
   clear(st);
   {
-    b8v ka[2][4];
-#pragma unroll
-    for (int kt = 0; kt < 4; ++kt) ka[0][kt] = read_k(lds[0], 0, kt);
+    b8v ka[KP + 1][4];
+    k_first(lds[0], ka);
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       k_step(lds[0], ks, ka, st);
@@ -696,11 +706,10 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
     const int k_tile = min(tile + 2, n_tiles - 1);  // its K half goes where K(tile) was (again K(last) at the end)
     f4v sn[RB][4];
     clear(sn);
-    b8v ka[2][4];
+    b8v ka[KP + 1][4];
     float mx[RB];
     b8v pv[RB][2];
-#pragma unroll
-    for (int kt = 0; kt < 4; ++kt) ka[0][kt] = read_k(kbuf, 0, kt);
+    k_first(kbuf, ka);
 #pragma unroll
     for (int ks = 0; ks < KA; ++ks) {
       k_step(kbuf, ks, ka, sn);
@@ -764,9 +773,8 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
     if (more) {
       const char* kbuf = lds[(tile + 1) % 2];
       clear(st);
-      b8v ka[2][4];
-#pragma unroll
-      for (int kt = 0; kt < 4; ++kt) ka[0][kt] = read_k(kbuf, 0, kt);
+      b8v ka[KP + 1][4];
+      k_first(kbuf, ka);
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
         k_step(kbuf, ks, ka, st);
