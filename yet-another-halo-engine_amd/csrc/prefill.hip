@@ -491,6 +491,11 @@ __device__ __forceinline__ float MaxOverLaneGroups(float v) {
   return fmaxf(__builtin_bit_cast(float, q0), __builtin_bit_cast(float, q1));
 }
 
+template <bool B>
+struct Constant {
+  static constexpr bool value = B;
+};
+
 // s_waitcnt operand: at most n vector memory operations outstanding, the other counters unconstrained
 constexpr int VmCnt(int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); }
 
@@ -641,8 +646,9 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
 #pragma unroll
     for (int s2 = 0; s2 < 2; ++s2) pv[s2] = __builtin_bit_cast(b8v, uint4{w[s2][0], w[s2][1], w[s2][2], w[s2][3]});
   };
-  // O^T += V^T P^T and the denominators; `v_tile` >= 0: the V half of that image is copied meanwhile
-  auto pv_product = [&](const char* buf, const b8v (&pv)[RB][2], int v_tile) {
+  // O^T += V^T P^T and the denominators; `v_tile` >= 0: the V half of that image is copied meanwhile (`always`:
+  // known when compiling, which keeps the products in one scheduling region)
+  auto pv_product = [&](auto always, const char* buf, const b8v (&pv)[RB][2], int v_tile) {
     auto read_v = [&](int dt, int s2) -> b8v {
       return *reinterpret_cast<const b8v*>(buf + voff + dt * 16 * 128 + 16 * ((4 * s2 + jg) ^ sw));
     };
@@ -668,7 +674,7 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
         for (int i = 0; i < RB; ++i)
           o[i][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[dt % (VP + 1)][s2], pv[i][s2], o[i][dt], 0, 0, 0);
       if (dt % 2 == 1) {
-        if (v_tile >= 0) copy_part(v_tile, KS + dt / 2);
+        if (decltype(always)::value || v_tile >= 0) copy_part(v_tile, KS + dt / 2);
         __builtin_amdgcn_sched_barrier(0);
       }
     }
@@ -740,7 +746,7 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
-    pv_product(lds[2 + tile % 3], pv, min(tile + 2, n_tiles - 1));
+    pv_product(Constant<true>{}, lds[2 + tile % 3], pv, min(tile + 2, n_tiles - 1));
 #pragma unroll
     for (int i = 0; i < RB; ++i)
 #pragma unroll
@@ -769,7 +775,7 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
       move_reference(i, row_max(st[i]));
       numerators(i, st[i], pv[i]);
     }
-    pv_product(lds[2 + tile % 3], pv, tile + 2 < n_tiles ? tile + 2 : -1);
+    pv_product(Constant<false>{}, lds[2 + tile % 3], pv, tile + 2 < n_tiles ? tile + 2 : -1);
     if (more) {
       const char* kbuf = lds[(tile + 1) % 2];
       clear(st);
