@@ -723,12 +723,8 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
     }
 #pragma unroll
     for (int i = 0; i < RB; ++i) mx[i] = row_max(st[i]);
-#pragma unroll
-    for (int n = 0; n < KA * 4 * RB; ++n) {  // spread the vector work between the matrix instructions
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-    }
+    // (the compiler spreads the vector work between the matrix instructions by itself; explicit scheduling groups
+    // were 3 % slower)
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int i = 0; i < RB; ++i) move_reference(i, mx[i]);
@@ -739,12 +735,6 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
     }
 #pragma unroll
     for (int i = 0; i < RB; ++i) numerators(i, st[i], pv[i]);
-#pragma unroll
-    for (int n = 0; n < (KS - KA) * 4 * RB; ++n) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-    }
     __builtin_amdgcn_sched_barrier(0);
     pv_product(Constant<true>{}, lds[2 + tile % 3], pv, min(tile + 2, n_tiles - 1));
 #pragma unroll
