@@ -566,10 +566,13 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
                                              tile * TIMG + c * 1024, 0, 0);
   };
   // byte offsets of this lane's operand reads within an image; the XOR with qn % 8 undoes the images' swizzle
-  const int sw = qn % 8;
-  const int koff = qn * (2 * D), voff = qn * 128;
+  // The chunk index (4 n + jg) ^ (qn % 8) is 4 (n ^ h) + (jg ^ l) with h = qn % 8 / 4 and l = qn % 4: per lane one
+  // offset for even n and one for odd n, and everything else is a constant of the instruction.
+  const int sw_l = 16 * (jg ^ (qn % 4)), sw_h = 64 * (qn % 8 / 4);
+  const int koff[2] = {qn * (2 * D) + sw_l + sw_h, qn * (2 * D) + sw_l - sw_h};
+  const int voff[2] = {qn * 128 + sw_l + sw_h, qn * 128 + sw_l - sw_h};
   auto read_k = [&](const char* buf, int ks, int kt) -> b8v {
-    return *reinterpret_cast<const b8v*>(buf + koff + kt * 16 * (2 * D) + 16 * ((4 * ks + jg) ^ sw));
+    return *reinterpret_cast<const b8v*>(buf + koff[ks % 2] + (kt * 16 * (2 * D) + 64 * ks));
   };
   // One 32-dim step of S^T = K Q^T: the A operands of step ks + KP are read before the products of step ks.
   auto k_first = [&](const char* buf, b8v (&ka)[KP + 1][4]) {
@@ -600,9 +603,10 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
   // accumulators by a power of two, which is exact, so moving it late changes nothing in the result, while bf16
   // numerators and f32 sums have room for the factor 2^16. Rescaling is then rare (the first tile, mostly).
   auto row_max = [&](const f4v (&st)[4]) -> float {  // over the 64 keys of the tile, times the softmax scale
-    float mx = fmaxf(fmaxf(st[0][0], st[0][1]), fmaxf(st[0][2], st[0][3]));
+    float mx = fmaxf(st[0][0], st[0][1]);  // a chain of three-operand maxima
+    mx = fmaxf(fmaxf(mx, st[0][2]), st[0][3]);
 #pragma unroll
-    for (int kt = 1; kt < 4; ++kt) mx = fmaxf(mx, fmaxf(fmaxf(st[kt][0], st[kt][1]), fmaxf(st[kt][2], st[kt][3])));
+    for (int kt = 1; kt < 4; ++kt) mx = fmaxf(fmaxf(mx, st[kt][0]), st[kt][1]), mx = fmaxf(fmaxf(mx, st[kt][2]), st[kt][3]);
     return MaxOverLaneGroups(mx) * sscale;  // sscale > 0 is required by the entry point
   };
   auto move_reference = [&](int i, float mx) {
@@ -649,8 +653,13 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
   // O^T += V^T P^T and the denominators; `v_tile` >= 0: the V half of that image is copied meanwhile (`always`:
   // known when compiling, which keeps the products in one scheduling region)
   auto pv_product = [&](auto always, const char* buf, const b8v (&pv)[RB][2], int v_tile) {
+    // (the empty asm keeps the two lane addresses as they are: left alone, the compiler hoists voff + constant out
+    // of the tile loop for every read and adds the buffer's address to each of them again)
+    typedef __attribute__((address_space(3))) const char* LdsPtr;
+    LdsPtr vb0 = (LdsPtr)buf + voff[0], vb1 = (LdsPtr)buf + voff[1];
+    asm volatile("" : "+v"(vb0), "+v"(vb1));
     auto read_v = [&](int dt, int s2) -> b8v {
-      return *reinterpret_cast<const b8v*>(buf + voff + dt * 16 * 128 + 16 * ((4 * s2 + jg) ^ sw));
+      return *reinterpret_cast<const __attribute__((address_space(3))) b8v*>((s2 ? vb1 : vb0) + (dt * 16 * 128 + 64 * s2));
     };
     b8v va[VP + 1][2];  // read VP 16-dim tiles ahead
 #pragma unroll
