@@ -140,3 +140,11 @@ def test_prefill_rejects_bad_arguments(yahkv, torch_gpu):
     rc = yahkv.lib.yahkv_prefill_attend(C.byref(g8), C.byref(st), None, 4, None, 1, 0, 8, None, 0.0625, None, None, 0,
                                         None, 0, None)
     assert rc == -1
+    # a kv head's tile images beyond 2 GiB (prefix + chunk past 2^21 tokens at head_dim 256): refused before any launch
+    # (the workspace is not touched, so its claimed size need not be real)
+    out = torch.empty(q.shape, dtype=torch.bfloat16, device="cuda")
+    small = torch.empty(4096, dtype=torch.uint8, device="cuda")
+    rc = yahkv.lib.yahkv_prefill_attend_tiles(C.byref(g8), C.byref(st), table.data_ptr(), 4, zero.data_ptr(), 1, 1 << 21, 8,
+                                              q.data_ptr(), 0.0625, None, out.data_ptr(), 2, small.data_ptr(), 1 << 50,
+                                              None)
+    assert rc == -2
