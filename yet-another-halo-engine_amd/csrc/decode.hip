@@ -203,7 +203,8 @@ __device__ __forceinline__ float HalfSum32(float v) {
 // q8_0 byte, 3 per q4_0 byte):
 //   scores  S[head][key] = sum_block ks[key][block] * (Q_block . codes_block)       v_mfma_f32_32x32x16_f16, one
 //           32-dim block per pair of instructions (K = 16 each), so the block scale is applied to the f32 result and
-//           the products themselves are exact (codes and f16 queries are exact in f16)
+//           the products themselves are exact (codes and f16 queries are exact in f16; the codes go in with the
+//           constant of their f16 conversion still on, and what that adds comes off the block's sum: `lcorr`)
 //   output  O[head][dim] += sum_key P[head][key] * (vs[key][block] * codes)          v_mfma_f32_16x16x32_f16; the scale
 //           varies along the contraction here, so V is dequantized to f16 (one rounding, 2^-12 relative)
 // The page layouts are chosen for these operand shapes. q8_0: a lane's 16-byte load is 16 dims of one key (K, [block]
