@@ -753,8 +753,12 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
     // The copies complete in the order of their issue: all but the newest kCopies / 2, the pieces of V(tile + 2),
     // have landed, this wave's pieces of K(tile + 2) and V(tile + 1) among them.
     // (A bare barrier: __syncthreads() carries a release fence, which waits for every copy in flight.)
+    // The wavefront-scope fences emit nothing; they keep the compiler from moving LDS accesses across the barrier,
+    // which by itself is not a memory operation to it.
     __builtin_amdgcn_s_waitcnt(VmCnt(kCopies / 2) & 0xF0FF);  // and lgkmcnt(0): this wave's LDS reads have returned
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_s_barrier();  // ... and everybody's; everybody is done with K(tile + 1) and V(tile)
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   }
   // ---- the last tiles, one phase after the other: masked softmax, second product, then the next tile's scores
   for (; tile < n_tiles; ++tile) {
