@@ -142,12 +142,31 @@ def cpu_baseline(wl, lens, scale, budget_tokens=150000):
         times.append(time.perf_counter() - t0)
     t = float(np.median(times))
     bpt = 2 * NKV * (HD // 32) * ((32 if wl["fmt"] == 8 else 16) + 2)
+    ref_append = None
+    if wl["fmt"] == 8 and oracle.ref() is not None:
+        # the reference's own CPU code on this path: QuantizeQ8_0 (engine/core/gguf_quant.cpp:310-320), compiled from its
+        # sources into oracle/_ref; scalar, one thread, as the reference runs it
+        import ctypes as C
+        n_el = 1 << 22
+        x = rng.standard_normal(n_el).astype(np.float32)
+        dst = np.empty(n_el // 32 * 34, np.uint8)
+        fn = oracle.ref().ref_quantize_q8_0
+        fn.argtypes = [C.c_void_p, C.c_uint64, C.c_void_p]
+        fn(x.ctypes.data, n_el, dst.ctypes.data)
+        reps = []
+        for _ in range(3):
+            t0 = time.perf_counter()
+            fn(x.ctypes.data, n_el, dst.ctypes.data)
+            reps.append(time.perf_counter() - t0)
+        ref_append = {"blocks_per_s": round(n_el / 32 / float(np.median(reps)), 0), "kind": "reference", "cores": 1,
+                      "sample": f"the reference's QuantizeQ8_0 on {n_el // 32} blocks of N(0,1), median of 3"}
     return {"value": round(tot * bpt / t / 1e9, 3), "unit": "GB/s", "cores": oracle.threads(), "kind": "port",
             "sample": f"oracle decode attention on the first {len(take)} sequences of the batch ({tot} tokens, "
                       f"{tot * bpt / 1e6:.0f} MB of KV), median of 3 after a warm-up",
             "tok_per_s": round(len(take) / t, 2),
             "append_blocks_per_s": round(tot * 2 * NKV * (HD // 32) / t_quant, 0),
-            "append_note": "oracle scalar block quantizer + page scatter, 1 thread"}
+            "append_note": "oracle scalar block quantizer + page scatter, 1 thread",
+            "append_reference": ref_append}
 
 
 def prefill_cpu_baseline(wl, scale, prefix=2048, chunk=64):
