@@ -206,9 +206,16 @@ def run_prefill(a, wl, torch, yahkv):
     out = torch.empty(q.shape, dtype=torch.bfloat16, device="cuda")
     ws = torch.empty(yahkv.prefill_workspace_bytes(g, B, prefix, chunk), dtype=torch.uint8, device="cuda")
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(a.steps)]
+    ev_app = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(a.steps)]
+    it = iter(ev_app)
 
     def step(pair=None):
+        app = next(it) if pair else None
+        if app:
+            app[0].record()
         yahkv.append(pools, t_table, t_prefix, knew, vnew)
+        if app:
+            app[1].record()
         yahkv.prefill_decode_tiles(pools, t_table, t_prefix, prefix, B, chunk, ws)
         if pair:
             pair[0].record()
@@ -247,6 +254,8 @@ def run_prefill(a, wl, torch, yahkv):
     dt = time.perf_counter() - t0
     ms = dt / a.steps * 1e3
     kern_ms = float(np.mean([p[0].elapsed_time(p[1]) for p in ev]))
+    app_ms = float(np.median([p[0].elapsed_time(p[1]) for p in ev_app]))
+    app_bytes = B * chunk * (2 * NKV * HD * 2 + 2 * NKV * (HD // 32) * 34)   # bf16 K and V rows in, q8_0 blocks out
     flops = float(B) * NQ * chunk * (prefix + (chunk + 1) / 2) * HD * 4   # both products, causal part counted once
     res = {
         "metric": "chunked-prefill attention over paged q8 KV, TFLOP/s (bf16 MFMA) + tok/s",
@@ -258,6 +267,10 @@ def run_prefill(a, wl, torch, yahkv):
                    "step": "append chunk (quantize + scatter) + decode tiles to bf16 + causal attention"},
         "tok_per_s": round(B * chunk / (ms * 1e-3), 1), "flops_per_step": int(flops),
         "parity_max_rel_err": float(f"{err:.3e}"), "out_fnv1a": first_hash,
+        "append": {"kernel": "AppendPages<8>", "ms": round(app_ms, 4), "bytes": int(app_bytes),
+                   "GB/s": round(app_bytes / (app_ms * 1e-3) / 1e9, 1),
+                   "frac_of_hbm_peak": round(app_bytes / (app_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                   "note": "quantize + scatter of the chunk, HIP events around the call (median)"},
         "roofline": {"bound": "mfma", "achieved": round(flops / (kern_ms * 1e-3) / 1e12, 1),
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(flops / (kern_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),

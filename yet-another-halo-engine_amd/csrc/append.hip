@@ -271,15 +271,45 @@ __global__ __launch_bounds__(64 * kPageWaves) void AppendPages(const RopeArgs a)
     for (int j = 0; j < 4; ++j) kx[j] = Widen4(rk[j], a.src_dtype), vx[j] = Widen4(rv[j], a.src_dtype);
     if (4 * (q + kPageWaves) < t_hi) request(q + kPageWaves);
     uint32_t vc[4];
+    if constexpr (FMT == 8) {
+      // Eight rows are in flight (K and V of four tokens) and a block has eight lanes: lane lb of a block takes row
+      // lb's amax and does the two divisions for it (the same operations on the same values, so the same bits),
+      // instead of every lane doing them for every row; the reciprocals go back through lane shuffles.
+      float am[8];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int t = 4 * q + j;
-      uint16_t ksc, vsc;
-      const uint32_t kc = FMT == 8 ? QuantizeLanesQ8(kx[j], &ksc) : QuantizeLanesQ4(kx[j], lb, &ksc);
-      vc[j] = FMT == 8 ? QuantizeLanesQ8(vx[j], &vsc) : QuantizeLanesQ4(vx[j], lb, &vsc);
-      if (!has || t < t_lo || t >= t_hi) continue;
-      if (lb == 0) lks[t * NB + b] = ksc, lvs[b * PT + t] = vsc;
-      if (FMT == 8 || lb < 4) *reinterpret_cast<uint32_t*>(&lk[(b * PT + t) * KB + 4 * lb]) = kc;
+      for (int j = 0; j < 4; ++j) am[j] = BlockAmaxQ8(kx[j]), am[4 + j] = BlockAmaxQ8(vx[j]);
+      float mine = am[0];
+#pragma unroll
+      for (int r = 1; r < 8; ++r) mine = lb == r ? am[r] : mine;
+      float inv;
+      uint16_t sc;
+      ScaleQ8(mine, &inv, &sc);
+      {
+        const int t = 4 * q + lb % 4;  // row lb is K (lb < 4) or V of this token
+        if (has && t >= t_lo && t < t_hi) {
+          if (lb < 4) lks[t * NB + b] = sc;
+          else lvs[b * PT + t] = sc;
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int t = 4 * q + j;
+        const uint32_t kc = CodesLanesQ8(kx[j], __shfl(inv, (lane & ~7) | j, 64));
+        vc[j] = CodesLanesQ8(vx[j], __shfl(inv, (lane & ~7) | (4 + j), 64));
+        if (!has || t < t_lo || t >= t_hi) continue;
+        *reinterpret_cast<uint32_t*>(&lk[(b * PT + t) * KB + 4 * lb]) = kc;
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int t = 4 * q + j;
+        uint16_t ksc, vsc;
+        const uint32_t kc = QuantizeLanesQ4(kx[j], lb, &ksc);
+        vc[j] = QuantizeLanesQ4(vx[j], lb, &vsc);
+        if (!has || t < t_lo || t >= t_hi) continue;
+        if (lb == 0) lks[t * NB + b] = ksc, lvs[b * PT + t] = vsc;
+        if (lb < 4) *reinterpret_cast<uint32_t*>(&lk[(b * PT + t) * KB + 4 * lb]) = kc;
+      }
     }
     if (has && (FMT == 8 || lb < 4)) {
       const int r0 = FMT == 8 ? d0 : b * 16 + 4 * lb;  // this lane's four byte rows of the V image

@@ -44,20 +44,31 @@ __device__ __forceinline__ float WaveSum(float v) {
 // A block of 32 values lies in 8 consecutive lanes, 4 values each (lane l of the 8: elements 4 l .. 4 l + 3).
 // q8_0: the block's amax in all 8 lanes (a maximum does not depend on the order), then the scalar formulas of
 // QuantizeBlock per element; returns this lane's 4 codes packed into a dword.
-__device__ __forceinline__ uint32_t QuantizeLanesQ8(const float4 v, uint16_t* scale) {
-#pragma clang fp contract(off)
+__device__ __forceinline__ float BlockAmaxQ8(const float4 v) {  // the block's amax, in all 8 lanes of the block
   float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
   amax = fmaxf(amax, Dpp<kQuadSwap1>(amax));
   amax = fmaxf(amax, Dpp<kQuadSwap2>(amax));
-  amax = fmaxf(amax, Dpp<kHalfMirror>(amax));
+  return fmaxf(amax, Dpp<kHalfMirror>(amax));
+}
+// d and 1 / d of a block from its amax, with the reference's operations
+__device__ __forceinline__ void ScaleQ8(float amax, float* inv, uint16_t* scale) {
+#pragma clang fp contract(off)
   const float d = amax / 127.0f;
-  const float inv = d > 0.0f ? 1.0f / d : 0.0f;
+  *inv = d > 0.0f ? 1.0f / d : 0.0f;
   *scale = __builtin_bit_cast(uint16_t, static_cast<_Float16>(d));
+}
+__device__ __forceinline__ uint32_t CodesLanesQ8(const float4 v, float inv) {  // this lane's 4 codes in a dword
+#pragma clang fp contract(off)
   const uint32_t c0 = static_cast<uint8_t>(static_cast<int8_t>(CodeQ8(v.x * inv)));
   const uint32_t c1 = static_cast<uint8_t>(static_cast<int8_t>(CodeQ8(v.y * inv)));
   const uint32_t c2 = static_cast<uint8_t>(static_cast<int8_t>(CodeQ8(v.z * inv)));
   const uint32_t c3 = static_cast<uint8_t>(static_cast<int8_t>(CodeQ8(v.w * inv)));
   return c0 | (c1 << 8) | (c2 << 16) | (c3 << 24);
+}
+__device__ __forceinline__ uint32_t QuantizeLanesQ8(const float4 v, uint16_t* scale) {
+  float inv;
+  ScaleQ8(BlockAmaxQ8(v), &inv, scale);
+  return CodesLanesQ8(v, inv);
 }
 // q4_0: ggml takes the value of largest magnitude, the first one on ties, so the reduction carries (|x|, index,
 // x) and prefers the lower index; d = that value / -8. Lanes 0-3 of the 8 return 4 bytes: low nibbles their own
