@@ -46,6 +46,8 @@ def lib():
             getattr(_lib, n).restype = C.c_size_t
             getattr(_lib, n).argtypes = [C.POINTER(Geometry)]
         _lib.orc_threads.restype = C.c_int32
+        _lib.orc_lround_identity_mismatches.restype = C.c_uint64
+        _lib.orc_lround_identity_mismatches.argtypes = [C.c_uint32, C.c_uint32]
     return _lib
 
 
@@ -223,3 +225,9 @@ def prefill_attend(pools, table, prefix_len, q, scale, gate=None, bf16_operands=
 
 def threads():
     return int(lib().orc_threads())
+
+
+def lround_identity_mismatches(first_bits, last_bits):
+    """Floats (both signs) with magnitude bits in [first_bits, last_bits] for which lroundf(r) differs from the
+    truncation of r + copysignf(0.5 - 2^-25, r), the form the append kernels compute."""
+    return int(lib().orc_lround_identity_mismatches(first_bits, last_bits))

@@ -412,3 +412,19 @@ void orc_prefill_attend(const orc_geometry* g, const orc_pools* pools, const int
       free(kd), free(sc), free(acc);
     }
 }
+
+uint64_t orc_lround_identity_mismatches(uint32_t first_bits, uint32_t last_bits) {
+  const float c = 0x1.fffffep-2f; /* the float below one half */
+  uint64_t bad = 0;
+#pragma omp parallel for reduction(+ : bad) schedule(static)
+  for (int64_t u = first_bits; u <= (int64_t)last_bits; ++u) {
+    for (uint32_t sign = 0; sign < 2; ++sign) {
+      const uint32_t bits = (uint32_t)u | (sign << 31);
+      float r;
+      memcpy(&r, &bits, 4);
+      volatile float shifted = r + copysignf(c, r); /* one rounded addition, then the conversion truncates */
+      bad += lroundf(r) != (long)shifted;
+    }
+  }
+  return bad;
+}

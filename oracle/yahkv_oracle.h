@@ -95,6 +95,10 @@ void orc_prefill_attend(const orc_geometry* g, const orc_pools* pools, const int
                         float softmax_scale, const float* gate, float* out, int32_t bf16_operands);
 /* worker threads the attend functions use */
 int32_t orc_threads(void);
+/* Checks an identity a kernel may use in place of lround (gguf_quant.cpp:316): for every float r with bit pattern
+ * magnitude in [first_bits, last_bits], both signs, lroundf(r) against the truncation of r + copysignf(0.5 - 2^-25, r).
+ * Returns the number of values that differ. */
+uint64_t orc_lround_identity_mismatches(uint32_t first_bits, uint32_t last_bits);
 
 #ifdef __cplusplus
 }

@@ -149,3 +149,15 @@ def test_q4_0_invariants():
     assert np.array_equal(oracle.dequantize_q4_0(b).reshape(-1, 32), d16[:, None] * (codes - 8).astype(np.float32))
     z = oracle.quantize_q4_0(np.zeros(32, np.float32))
     assert np.array_equal(z[0], np.array([0, 0x80] + [0x88] * 16, np.uint8))  # all-zero block: d = 0 / -8 = -0.0, codes 8
+
+
+def test_the_kernels_rounding_is_lround_for_every_float_a_code_can_come_from():
+    """The append kernels round x * inv as trunc(r + copysign(0.5 - 2^-25, r)) where the reference calls lround
+    (gguf_quant.cpp:316); codes come from |r| <= 128 (anything larger becomes 0 on both sides). Every float up to
+    129, both signs, 2.2e9 values."""
+    last = int(np.array([129.0], np.float32).view(np.uint32)[0])
+    assert oracle.lround_identity_mismatches(0, last) == 0
+    # the identity is not a tautology: with 0.5 itself the float below one half goes wrong
+    below_half = np.array([0.5], np.float32).view(np.uint32)[0] - 1
+    r = np.array([below_half], np.uint32).view(np.float32)[0]
+    assert int(np.float32(r) + np.float32(0.5)) == 1 and round(float(r)) == 0

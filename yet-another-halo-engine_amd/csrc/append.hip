@@ -220,7 +220,9 @@ __global__ __launch_bounds__(64 * kRopeWaves) void AppendRows(const RopeArgs a) 
 // the same slot (the first or the last of the table), the last token wins, as in a loop over the tokens.
 constexpr int kPageWaves = 4;
 constexpr int kPageAppendMin = 8;  // tokens per sequence from which a call is treated as a chunk
-template <int FMT>
+// SRC: the source rows' type, known when compiling (as a run-time value it put a three-way branch around every
+// row's conversion).
+template <int FMT, int SRC>
 __global__ __launch_bounds__(64 * kPageWaves) void AppendPages(const RopeArgs a) {
 #pragma clang fp contract(off)
   const Geom g = a.g;
@@ -260,7 +262,7 @@ __global__ __launch_bounds__(64 * kPageWaves) void AppendPages(const RopeArgs a)
       rk[j] = rv[j] = uint4{0u, 0u, 0u, 0u};  // reads as 0.0 in every source type
       if (t >= t_lo && t < t_hi && has) {
         const size_t row = ((size_t(s) * a.n_new + token_at(pi * PT + t)) * H + h) * D;
-        rk[j] = LoadRaw4(a.k_src, row + d0, a.src_dtype), rv[j] = LoadRaw4(a.v_src, row + d0, a.src_dtype);
+        rk[j] = LoadRaw4(a.k_src, row + d0, SRC), rv[j] = LoadRaw4(a.v_src, row + d0, SRC);
       }
     }
   };
@@ -268,7 +270,7 @@ __global__ __launch_bounds__(64 * kPageWaves) void AppendPages(const RopeArgs a)
   for (int q = t_lo / 4 + wave; 4 * q < t_hi; q += kPageWaves) {
     float4 kx[4], vx[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) kx[j] = Widen4(rk[j], a.src_dtype), vx[j] = Widen4(rv[j], a.src_dtype);
+    for (int j = 0; j < 4; ++j) kx[j] = Widen4(rk[j], SRC), vx[j] = Widen4(rv[j], SRC);
     if (4 * (q + kPageWaves) < t_hi) request(q + kPageWaves);
     uint32_t vc[4];
     if constexpr (FMT == 8) {
@@ -431,10 +433,18 @@ extern "C" int yahkv_append(const yahkv_geometry* g, const yahkv_pools* pools, c
   if (n_new >= kPageAppendMin && n_seqs <= 65535) {  // a chunk: page by page (the grid's z extent is the batch)
     const dim3 grid(static_cast<unsigned>((n_new + a.g.pt - 2) / a.g.pt + 1), static_cast<unsigned>(a.g.n_kv),
                     static_cast<unsigned>(n_seqs));
-    if (g->format == YAHKV_Q8_0)
-      hipLaunchKernelGGL((AppendPages<8>), grid, dim3(64 * kPageWaves), 0, st, a);
-    else
-      hipLaunchKernelGGL((AppendPages<4>), grid, dim3(64 * kPageWaves), 0, st, a);
+#define YAHKV_LAUNCH_PAGES(FF, SS) hipLaunchKernelGGL((AppendPages<FF, SS>), grid, dim3(64 * kPageWaves), 0, st, a)
+#define YAHKV_LAUNCH_PAGES_FMT(FF)                                   \
+  if (src_dtype == YAHKV_F32) YAHKV_LAUNCH_PAGES(FF, YAHKV_F32);     \
+  else if (src_dtype == YAHKV_F16) YAHKV_LAUNCH_PAGES(FF, YAHKV_F16); \
+  else YAHKV_LAUNCH_PAGES(FF, YAHKV_BF16)
+    if (g->format == YAHKV_Q8_0) {
+      YAHKV_LAUNCH_PAGES_FMT(8);
+    } else {
+      YAHKV_LAUNCH_PAGES_FMT(4);
+    }
+#undef YAHKV_LAUNCH_PAGES_FMT
+#undef YAHKV_LAUNCH_PAGES
     return LaunchStatus();
   }
   const dim3 grid(static_cast<unsigned>(n_seqs) * static_cast<unsigned>(n_new));

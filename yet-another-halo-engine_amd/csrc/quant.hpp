@@ -14,7 +14,12 @@ namespace yahkv {
 
 // A code from x * inv as the x86-64 reference computes it: lround, whose result for a non-finite or out-of-range
 // argument converts to the int8 0 there (only reachable when 1 / d overflowed, i.e. amax < 2^-119).
-__device__ __forceinline__ int CodeQ8(float r) { return fabsf(r) <= 128.0f ? static_cast<int>(roundf(r)) : 0; }
+// In that range lround(r) is the truncation of r + copysign(0.5 - 2^-25, r): adding the float below one half moves
+// exactly the values with a fraction of one half or more past the next integer (r + 0.5 itself would also carry
+// 0.5 - 2^-25 there, through the tie of the addition's rounding). Checked against lroundf for every float up to 129.
+__device__ __forceinline__ int CodeQ8(float r) {
+  return fabsf(r) <= 128.0f ? static_cast<int>(r + copysignf(0x1.fffffep-2f, r)) : 0;
+}
 
 template <int CTRL>
 __device__ __forceinline__ float Dpp(float x) {  // the value of another lane of the row, chosen by a DPP control
