@@ -1,0 +1,57 @@
+"""bench.py's command line and the one JSON line it prints (the fields a driver reads), on the default workload and on
+the prefill workload; more than one GPU is refused with a message."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+BENCH = os.path.join(ROOT, "bench.py")
+COMMON = ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+          "vs_baseline", "dtype", "data", "config", "roofline")
+ROOFLINE = ("bound", "achieved", "peak", "unit", "frac", "traffic")
+
+
+def test_more_than_one_gpu_is_refused():
+    r = subprocess.run([sys.executable, BENCH, "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0
+    assert "ONE GPU" in r.stderr + r.stdout
+
+
+def run(args):
+    r = subprocess.run([sys.executable, BENCH] + args, capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stderr[-2000:]
+    lines = [l for l in r.stdout.splitlines() if l.strip()]
+    assert len(lines) == 1, "bench.py prints exactly one line"
+    return json.loads(lines[0])
+
+
+@pytest.mark.gpu
+def test_decode_line_has_the_fields_a_driver_reads():
+    d = run(["--steps", "3", "--warmup", "1"])
+    for k in COMMON + ("cpu_baseline",):
+        assert k in d, k
+    assert d["n_gpus"] == 1 and d["steps"] == 3 and d["warmup"] == 1 and d["higher_is_better"] is True
+    assert d["unit"] == "GB/s" and d["dtype"] == "u8" and d["vs_baseline"] is None
+    assert d["config"]["workload"] == "ragged_b64_q8_0" and "model" not in d["config"]
+    for k in ROOFLINE:
+        assert k in d["roofline"], k
+    assert d["roofline"]["bound"] == "hbm" and d["roofline"]["peak"] == 8000.0
+    assert abs(d["roofline"]["frac"] - d["roofline"]["achieved"] / d["roofline"]["peak"]) < 1e-3
+    # whole-step throughput = algorithmic bytes / step time
+    assert abs(d["value"] - d["kv_bytes_per_step"] / (d["ms_per_step"] * 1e-3) / 1e9) < 0.01 * d["value"]
+    for k in ("value", "unit", "cores", "kind", "sample"):
+        assert k in d["cpu_baseline"], k
+    assert d["cpu_baseline"]["kind"] in ("port", "reference") and d["cpu_baseline"]["cores"] >= 1
+    assert d["parity_max_rel_err"] < 2e-3
+
+
+@pytest.mark.gpu
+def test_prefill_line():
+    d = run(["--workload", "prefill_b8_ctx16k_chunk2k_q8_0", "--steps", "2", "--warmup", "1", "--no-cpu-baseline"])
+    for k in COMMON + ("append",):
+        assert k in d, k
+    assert d["unit"] == "TFLOP/s" and d["roofline"]["bound"] == "mfma" and d["roofline"]["peak"] == 2500.0
+    assert 0.0 < d["roofline"]["frac"] < 1.0 and 0.0 < d["append"]["frac_of_hbm_peak"] < 1.0
