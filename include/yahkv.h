@@ -60,7 +60,7 @@ typedef enum yahkv_status {
 } yahkv_status;
 
 /* "kv q KB VB" of the reference's decode.txt (loom_decoder.hpp:76-79): K and V share one format here. */
-typedef enum yahkv_format { YAHKV_Q4_0 = 4, YAHKV_Q8_0 = 8 } yahkv_format;
+typedef enum yahkv_format { YAHKV_Q4_0 = 4, YAHKV_Q8_0 = 8, YAHKV_KV_F16 = 16 /* yahkv_f16_* functions only */ } yahkv_format;
 typedef enum yahkv_dtype { YAHKV_F32 = 0, YAHKV_F16 = 1, YAHKV_BF16 = 2 } yahkv_dtype;
 
 typedef struct yahkv_geometry {
@@ -247,6 +247,30 @@ int yahkv_slot_check(const yahkv_geometry* g, const void* header, size_t slot_by
                      int32_t* n_tokens);
 int yahkv_slot_unpack(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* table_row, int32_t n_pages,
                       const void* slot, void* stream);
+
+/* ---- unquantized f16 pools: the reference's fp16 twins of the decode path ------------------------------------------
+ * yah_dattn_kvappend (engine/gpu/loom/tools/gen_decode_attn.py:30-94), yah_dattn_part (:97-335) and yah_dattn_reduce
+ * (:338-411) on pools of f16 K and f16 V^T, with the page table, positions, clamping and argument meaning of the
+ * quantized functions above. geometry.format must be YAHKV_KV_F16; the other limits are the same.
+ * Pool layouts per page and kv head (f16 elements): K [head_dim / 16][page_tokens][16], V^T [head_dim][page_tokens];
+ * each pool is yahkv_f16_pool_bytes long and 16-byte aligned. 4 * n_kv_heads * head_dim bytes per token. */
+typedef struct yahkv_f16_pools {
+  void* k;
+  void* v;
+} yahkv_f16_pools;
+size_t yahkv_f16_pool_bytes(const yahkv_geometry* g);
+/* K and V rows of n_new tokens per sequence (layout and arguments as yahkv_append), rounded to f16 (nearest even,
+ * the reference's fptrunc, gen_decode_attn.py:79-80) and written at their page rows. */
+int yahkv_f16_append(const yahkv_geometry* g, const yahkv_f16_pools* pools, const int32_t* page_table,
+                     int32_t page_table_stride, const int32_t* start_pos, const int32_t* n_valid, int32_t n_seqs,
+                     int32_t n_new, const void* k_src, const void* v_src, int32_t src_dtype, void* stream);
+/* Decode attention over keys 0 .. seq_len[s] - 1 (arguments as yahkv_decode_attend): two dispatches, partials of
+ * fixed stretches of every sequence, then their merge with the optional sigmoid gate. */
+size_t yahkv_f16_decode_workspace_bytes(const yahkv_geometry* g, int32_t n_seqs, int32_t max_seq_len);
+int yahkv_f16_decode_attend(const yahkv_geometry* g, const yahkv_f16_pools* pools, const int32_t* page_table,
+                            int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs, int32_t max_seq_len,
+                            const void* q, int32_t q_dtype, float softmax_scale, const float* gate, float* out,
+                            void* workspace, size_t workspace_bytes, void* stream);
 
 #ifdef __cplusplus
 }

@@ -9,7 +9,7 @@ import os
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libyahkv.so")
 
-Q8_0, Q4_0 = 8, 4
+Q8_0, Q4_0, KV_F16 = 8, 4, 16
 F32, F16, BF16 = 0, 1, 2
 
 
@@ -25,6 +25,10 @@ class Geometry(C.Structure):
 
 class Pools(C.Structure):
     _fields_ = [("kq", C.c_void_p), ("ks", C.c_void_p), ("vq", C.c_void_p), ("vs", C.c_void_p)]
+
+
+class F16PoolsStruct(C.Structure):
+    _fields_ = [("k", C.c_void_p), ("v", C.c_void_p)]
 
 
 class Rope(C.Structure):
@@ -62,6 +66,14 @@ def _load():
     lib.yahkv_prefill_attend.argtypes = [G, P, i32p, i32, i32p, i32, i32, i32, vp, C.c_float, vp, vp, i32, vp,
                                          C.c_size_t, vp]
     lib.yahkv_prefill_attend_tiles.argtypes = lib.yahkv_prefill_attend.argtypes
+    F = C.POINTER(F16PoolsStruct)
+    lib.yahkv_f16_pool_bytes.restype = C.c_size_t
+    lib.yahkv_f16_pool_bytes.argtypes = [G]
+    lib.yahkv_f16_append.argtypes = [G, F, i32p, i32, i32p, i32p, i32, i32, vp, vp, i32, vp]
+    lib.yahkv_f16_decode_workspace_bytes.restype = C.c_size_t
+    lib.yahkv_f16_decode_workspace_bytes.argtypes = [G, i32, i32]
+    lib.yahkv_f16_decode_attend.argtypes = [G, F, i32p, i32, i32p, i32, i32, vp, i32, C.c_float, vp, vp, vp,
+                                            C.c_size_t, vp]
     lib.yahkv_prefill_decode_tiles.argtypes = [G, P, i32p, i32, i32p, i32, i32, i32, vp, C.c_size_t, vp]
     lib.yahkv_gather_blocks.argtypes = [G, P, i32p, i32, vp, vp, vp]
     lib.yahkv_pagepool_create.restype = C.c_void_p
@@ -168,6 +180,66 @@ def _dp(t):
 def _dtype_code(t):
     import torch
     return {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}[t.dtype]
+
+
+class F16Pools:
+    """One layer's unquantized f16 K and V^T pools on the GPU (the reference's kpool / vtpool of the fp16 kernels)."""
+
+    def __init__(self, g, fill=0, device="cuda:0"):
+        import torch
+        assert g.format == KV_F16
+        self.geom = g
+        n = lib.yahkv_f16_pool_bytes(C.byref(g))
+        if n == 0:
+            raise YahkvError(-2, "f16 pools")
+        self.k = torch.full((n,), fill, dtype=torch.uint8, device=device)
+        self.v = torch.full((n,), fill, dtype=torch.uint8, device=device)
+
+    def struct(self):
+        return F16PoolsStruct(self.k.data_ptr(), self.v.data_ptr())
+
+    def numpy(self):
+        """K as [page][H][D / 16][PT][16] and V^T as [page][H][D][PT], uint16 bit patterns."""
+        import numpy as np
+        g = self.geom
+        k = self.k.cpu().numpy().view(np.uint16).reshape(g.n_pages, g.n_kv_heads, g.head_dim // 16, g.page_tokens, 16)
+        v = self.v.cpu().numpy().view(np.uint16).reshape(g.n_pages, g.n_kv_heads, g.head_dim, g.page_tokens)
+        return k, v
+
+
+def f16_geometry(n_q_heads, n_kv_heads, head_dim, page_tokens, n_pages):
+    g = geometry(Q8_0, n_q_heads, n_kv_heads, head_dim, page_tokens, n_pages)  # the same limits
+    g.format = KV_F16
+    return g
+
+
+def f16_append(pools, table, start_pos, k_src, v_src, n_valid=None):
+    """append() for f16 pools: rows rounded to f16 and written at their page rows."""
+    g = pools.geom
+    assert k_src.is_contiguous() and v_src.is_contiguous() and table.is_contiguous() and k_src.dtype == v_src.dtype
+    n_seqs, n_new = k_src.shape[0], k_src.shape[1]
+    assert tuple(k_src.shape) == (n_seqs, n_new, g.n_kv_heads, g.head_dim) and k_src.shape == v_src.shape
+    st = pools.struct()
+    _check(lib.yahkv_f16_append(C.byref(g), C.byref(st), _dp(table), table.shape[1], _dp(start_pos), _dp(n_valid),
+                                n_seqs, n_new, _dp(k_src), _dp(v_src), _dtype_code(k_src), _stream()), "f16_append")
+
+
+def f16_decode_attend(pools, table, seq_len, max_seq_len, q, scale, gate=None, out=None, workspace=None):
+    """decode_attend() over f16 pools; returns out f32 [n_seqs][n_q_heads][D]."""
+    import torch
+    g = pools.geom
+    n_seqs = q.shape[0]
+    assert q.is_contiguous() and table.is_contiguous() and tuple(q.shape) == (n_seqs, g.n_q_heads, g.head_dim)
+    if out is None:
+        out = torch.empty(q.shape, dtype=torch.float32, device=q.device)
+    if workspace is None:
+        need = lib.yahkv_f16_decode_workspace_bytes(C.byref(g), n_seqs, max_seq_len)
+        workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=q.device)
+    st = pools.struct()
+    _check(lib.yahkv_f16_decode_attend(C.byref(g), C.byref(st), _dp(table), table.shape[1], _dp(seq_len), n_seqs,
+                                       max_seq_len, _dp(q), _dtype_code(q), scale, _dp(gate), _dp(out),
+                                       _dp(workspace), workspace.numel(), _stream()), "f16_decode_attend")
+    return out
 
 
 class DevicePools:
