@@ -244,30 +244,60 @@ __global__ __launch_bounds__(64 * kWaves) void PartF16(const F16Args a) {
   }
 }
 
-// One workgroup per (query head, sequence), one thread per dim: the stretches' partials merged with the weights
-// e^(m_p - M), normalized, and the optional sigmoid gate (gen_decode_attn.py:338-411). A sequence of length 0 gives 0.
+// One workgroup per (query head, sequence): the stretches' partials merged with the weights e^(m_p - M), normalized,
+// and the optional sigmoid gate (gen_decode_attn.py:338-411). The weights are computed once, by one thread per
+// stretch, and kept in LDS; then one thread per dim sums the stretches, eight loads in flight and no branch between
+// them (a stretch without keys has weight 0 and its row, which nobody wrote, is read but not used). A sequence of
+// length 0 gives 0.
+constexpr int kMaxSplits = 1024;
 __global__ __launch_bounds__(256) void ReduceF16(const F16Args a) {
   const Geom g = a.g;
   const int G = g.group(), H = g.n_kv, D = g.hd;
-  const int hq = blockIdx.x, s = blockIdx.y, d = threadIdx.x;
-  if (d >= D) return;
+  const int hq = blockIdx.x, s = blockIdx.y, t = threadIdx.x;
   const int h = hq / G, gi = hq % G;
   const size_t p0 = (size_t(s) * H + h) * a.n_splits;
-  float M = kLowest;
-  for (int p = 0; p < a.n_splits; ++p) {
+  __shared__ float w[kMaxSplits];
+  __shared__ float red[4];
+  float mx = kLowest;
+  for (int p = t; p < a.n_splits; p += 256) {
     const float* e = a.ml + ((p0 + p) * G + gi) * 2;
-    if (e[1] > 0.0f) M = fmaxf(M, e[0]);
+    if (e[1] > 0.0f) mx = fmaxf(mx, e[0]);
   }
-  float L = 0.0f, v = 0.0f;
-  for (int p = 0; p < a.n_splits; ++p) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+  if (t % 64 == 0) red[t / 64] = mx;
+  __syncthreads();
+  const float M = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  float lpart = 0.0f;
+  for (int p = t; p < a.n_splits; p += 256) {
     const float* e = a.ml + ((p0 + p) * G + gi) * 2;
-    if (e[1] > 0.0f) {
-      const float w = __expf(e[0] - M);
-      L = __builtin_fmaf(w, e[1], L);
-      v = __builtin_fmaf(w, a.acc[((p0 + p) * G + gi) * D + d], v);
-    }
+    const float wp = e[1] > 0.0f ? __expf(e[0] - M) : 0.0f;
+    w[p] = wp;
+    lpart = e[1] > 0.0f ? __builtin_fmaf(wp, e[1], lpart) : lpart;
   }
-  const size_t o = (size_t(s) * g.n_q + hq) * D + d;
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) lpart += __shfl_xor(lpart, o, 64);
+  __syncthreads();  // red has been read, w is written
+  if (t % 64 == 0) red[t / 64] = lpart;
+  __syncthreads();
+  const float L = (red[0] + red[1]) + (red[2] + red[3]);
+  if (t >= D) return;
+  float v = 0.0f;
+  const float* rows = a.acc + (p0 * G + gi) * D + t;
+  const size_t step = size_t(G) * D;
+  int p = 0;
+  for (; p + 8 <= a.n_splits; p += 8) {
+    float x[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) x[j] = rows[(p + j) * step];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v = w[p + j] > 0.0f ? __builtin_fmaf(w[p + j], x[j], v) : v;
+  }
+  for (; p < a.n_splits; ++p) {
+    const float x = rows[p * step];
+    v = w[p] > 0.0f ? __builtin_fmaf(w[p], x, v) : v;
+  }
+  const size_t o = (size_t(s) * g.n_q + hq) * D + t;
   v = L > 0.0f ? v / L : 0.0f;
   if (a.gate != nullptr) v *= 1.0f / (1.0f + __expf(-a.gate[o]));
   a.out[o] = v;
@@ -292,8 +322,8 @@ Split MakeSplit(const Geom& g, int32_t n_seqs, int32_t max_len) {
   Split sp;
   const int64_t unit = int64_t(kTileKeys) * kWaves;
   const int64_t pairs = int64_t(n_seqs) * g.n_kv;
-  int64_t want = std::max<int64_t>(1, (1024 + pairs - 1) / pairs);
-  want = std::min<int64_t>(want, (int64_t(max_len) + unit - 1) / unit);
+  int64_t want = std::max<int64_t>(1, (4096 + pairs - 1) / pairs);  // about sixteen workgroups per CU
+  want = std::min<int64_t>(std::min<int64_t>(want, kMaxSplits), (int64_t(max_len) + unit - 1) / unit);
   const int64_t keys = ((int64_t(max_len) + want - 1) / want + unit - 1) / unit * unit;
   sp.keys_per_split = static_cast<int32_t>(keys);
   sp.n_splits = static_cast<int32_t>((int64_t(max_len) + keys - 1) / keys);
