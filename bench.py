@@ -30,6 +30,9 @@ WORKLOADS = {
     "b16_ctx128k_q4_0": dict(fmt=4, batch=16, lo=131072, hi=131072, seed=4, outliers=8),
     # chunked prefill: every sequence holds `lo` tokens and takes a chunk of `chunk` more per step
     "prefill_b8_ctx16k_chunk2k_q8_0": dict(fmt=8, batch=8, lo=16384, hi=16384, seed=4, chunk=2048),
+    # the unquantized f16 twins of the decode path (4096 B per token)
+    "b16_ctx128k_f16": dict(fmt=16, batch=16, lo=131072, hi=131072, seed=4),
+    "ragged_b64_f16": dict(fmt=16, batch=64, lo=1024, hi=65536, seed=4),
 }
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 NQ, NKV, HD, PT = 24, 4, 256, 64
@@ -193,6 +196,95 @@ def prefill_cpu_baseline(wl, scale, prefix=2048, chunk=64):
                       "warm-up", "tok_per_s": round(chunk / t, 1)}
 
 
+def run_f16(a, wl, torch, yahkv):
+    """A step on unquantized f16 pools: append one token per sequence + decode attention (partials, then their merge)."""
+    rng = np.random.default_rng(wl["seed"])
+    B = wl["batch"]
+    lens = rng.integers(wl["lo"], wl["hi"] + 1, B).astype(np.int32)
+    total = a.warmup + a.steps + 1
+    pages = (lens + total + PT - 1) // PT
+    n_pages = int(pages.sum())
+    g = yahkv.f16_geometry(NQ, NKV, HD, PT, n_pages)
+    perm = rng.permutation(n_pages).astype(np.int32)
+    table = np.zeros((B, int(pages.max())), np.int32)
+    o = 0
+    for s, n in enumerate(pages):
+        table[s, :n] = perm[o:o + n]
+        o += n
+    pools = yahkv.F16Pools(g)
+    t_table = torch.from_numpy(table).cuda()
+    gen = torch.Generator(device="cuda").manual_seed(wl["seed"])
+    for s in range(B):                                   # fill the prefix through the library's own append
+        for o in range(0, int(lens[s]), 8192):
+            n = min(8192, int(lens[s]) - o)
+            k = torch.randn((1, n, NKV, HD), generator=gen, device="cuda").to(torch.bfloat16)
+            v = torch.randn((1, n, NKV, HD), generator=gen, device="cuda").to(torch.bfloat16)
+            yahkv.f16_append(pools, t_table[s:s + 1], torch.tensor([o], dtype=torch.int32, device="cuda"), k, v)
+    scale = 1.0 / float(np.sqrt(HD))
+    max_len = int(lens.max()) + total
+    len_rows = torch.from_numpy(lens[None, :] + np.arange(total + 1, dtype=np.int32)[:, None]).cuda()
+    q = torch.randn((B, NQ, HD), generator=gen, device="cuda").to(torch.bfloat16)
+    knew = torch.randn((total, B, 1, NKV, HD), generator=gen, device="cuda").to(torch.bfloat16)
+    vnew = torch.randn((total, B, 1, NKV, HD), generator=gen, device="cuda").to(torch.bfloat16)
+    out = torch.empty((B, NQ, HD), dtype=torch.float32, device="cuda")
+    ws = torch.empty(yahkv.lib.yahkv_f16_decode_workspace_bytes(g, B, max_len), dtype=torch.uint8, device="cuda")
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(a.steps)]
+
+    def step(i, pair=None):
+        yahkv.f16_append(pools, t_table, len_rows[i], knew[i], vnew[i])
+        if pair:
+            pair[0].record()
+        yahkv.f16_decode_attend(pools, t_table, len_rows[i + 1], max_len, q, scale, out=out, workspace=ws)
+        if pair:
+            pair[1].record()
+
+    # parity before timing: the shortest sequence against the float64 closed form over the pools' own f16 values
+    step(0)
+    torch.cuda.synchronize()
+    first_hash = fnv1a(out.cpu().numpy().tobytes())
+    s0 = int(np.argmin(lens))
+    n0 = int(lens[s0]) + 1
+    kp, vp = pools.k.view(torch.float16), pools.v.view(torch.float16)
+    kp = kp.view(n_pages, NKV, HD // 16, PT, 16)
+    vp = vp.view(n_pages, NKV, HD, PT)
+    pg = t_table[s0, :(n0 + PT - 1) // PT].long()
+    Kd = kp[pg].permute(0, 3, 1, 2, 4).reshape(-1, NKV, HD)[:n0].double().cpu().numpy()
+    Vd = vp[pg].permute(0, 3, 1, 2).reshape(-1, NKV, HD)[:n0].double().cpu().numpy()
+    qs = q[s0].double().cpu().numpy()
+    err = 0.0
+    for h in range(NQ):
+        sc = Kd[:, h // (NQ // NKV)] @ qs[h] * scale
+        p = np.exp(sc - sc.max())
+        want = (p / p.sum()) @ Vd[:, h // (NQ // NKV)]
+        err = max(err, float(np.abs(out[s0, h].cpu().numpy() - want).max() / np.abs(want).max()))
+    if not err < 2e-3:
+        raise SystemExit(f"bench.py: parity check failed before timing: max relative error {err:.3e}")
+    for i in range(a.warmup):
+        step(1 + i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(a.steps):
+        step(1 + a.warmup + i, ev[i])
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / a.steps * 1e3
+    kern_ms = float(np.mean([p[0].elapsed_time(p[1]) for p in ev]))
+    kv_bytes = float(np.sum(lens + a.warmup + 1 + (a.steps + 1) / 2)) * 2 * NKV * HD * 2
+    gbs, kgbs = kv_bytes / (ms * 1e-3) / 1e9, kv_bytes / (kern_ms * 1e-3) / 1e9
+    print(json.dumps({
+        "metric": "paged f16 KV decode-attn HBM GB/s (% of peak) + tok/s", "value": round(gbs, 1), "unit": "GB/s",
+        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": a.workload, "batch": B, "ctx_min": int(lens.min()), "ctx_max": int(lens.max()),
+                   "ctx_sum": int(lens.sum()), "n_q_heads": NQ, "n_kv_heads": NKV, "head_dim": HD, "page_tokens": PT,
+                   "n_pages": n_pages, "kv_format": "f16", "step": "append 1 token/seq + paged decode attention"},
+        "pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2), "tok_per_s": round(B / (ms * 1e-3), 1),
+        "kv_bytes_per_step": int(kv_bytes), "parity_max_rel_err": float(f"{err:.3e}"), "out_fnv1a": first_hash,
+        "roofline": {"bound": "hbm", "achieved": round(kgbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(kgbs / HBM_PEAK_GBS, 4), "traffic": None, "traffic_source": None,
+                     "kernel": "PartF16<%d, %d> + ReduceF16" % (HD, PT), "kernel_ms": round(kern_ms, 4)},
+        "cpu_baseline": None}))
+
+
 def run_prefill(a, wl, torch, yahkv):
     """A step: quantize + scatter one chunk per sequence, decode prefix + chunk to bf16 tiles, causal attention."""
     g, layers, lens, table, t_table, gen = build_state(yahkv, torch, wl, 0)
@@ -308,6 +400,8 @@ def main():
     wl = WORKLOADS[a.workload]
     if "chunk" in wl:
         return run_prefill(a, wl, torch, yahkv)
+    if wl["fmt"] == 16:
+        return run_f16(a, wl, torch, yahkv)
     total = a.warmup + a.steps + 1
     g, layers, lens, table, t_table, gen = build_state(yahkv, torch, wl, total)
     pools = layers[0]
