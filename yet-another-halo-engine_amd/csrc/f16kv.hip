@@ -9,6 +9,7 @@
 // S[head][key] with v_mfma_f32_32x32x16_f16 (queries as A rows, 8 of 32 rows used), O[head][dim] += P V with
 // v_mfma_f32_16x16x32_f16 (P rounded to f16 against the running maximum).
 #include <algorithm>
+#include <cstdlib>
 
 #include "common.hpp"
 
@@ -322,7 +323,9 @@ Split MakeSplit(const Geom& g, int32_t n_seqs, int32_t max_len) {
   Split sp;
   const int64_t unit = int64_t(kTileKeys) * kWaves;
   const int64_t pairs = int64_t(n_seqs) * g.n_kv;
-  int64_t want = std::max<int64_t>(1, (4096 + pairs - 1) / pairs);  // about sixteen workgroups per CU
+  int64_t target = 4096;  // workgroups in all, about sixteen per CU; YAHKV_F16_WORKGROUPS overrides it for experiments
+  if (const char* e = std::getenv("YAHKV_F16_WORKGROUPS")) target = std::max(1, std::atoi(e));
+  int64_t want = std::max<int64_t>(1, (target + pairs - 1) / pairs);
   want = std::min<int64_t>(std::min<int64_t>(want, kMaxSplits), (int64_t(max_len) + unit - 1) / unit);
   const int64_t keys = ((int64_t(max_len) + want - 1) / want + unit - 1) / unit * unit;
   sp.keys_per_split = static_cast<int32_t>(keys);
