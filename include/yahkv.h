@@ -271,6 +271,16 @@ int yahkv_f16_decode_attend(const yahkv_geometry* g, const yahkv_f16_pools* pool
                             int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs, int32_t max_seq_len,
                             const void* q, int32_t q_dtype, float softmax_scale, const float* gate, float* out,
                             void* workspace, size_t workspace_bytes, void* stream);
+/* Chunked-prefill attention over f16 pools after the chunk has been appended with yahkv_f16_append (arguments as
+ * yahkv_prefill_attend; the workspace is required): the keys' bf16 tiles are converted from the pools (the reference's
+ * attention reads its 16-bit K / V pool directly, gen_attn_fa.py:1589-1595), then the same attention kernel runs. */
+size_t yahkv_f16_prefill_workspace_bytes(const yahkv_geometry* g, int32_t n_seqs, int32_t max_prefix_len,
+                                         int32_t chunk_len);
+int yahkv_f16_prefill_attend(const yahkv_geometry* g, const yahkv_f16_pools* pools, const int32_t* page_table,
+                             int32_t page_table_stride, const int32_t* prefix_len, int32_t n_seqs,
+                             int32_t max_prefix_len, int32_t chunk_len, const void* q, float softmax_scale,
+                             const float* gate, void* out, int32_t out_dtype, void* workspace,
+                             size_t workspace_bytes, void* stream);
 
 #ifdef __cplusplus
 }

@@ -174,3 +174,42 @@ def test_length_beyond_the_bound_is_clamped_and_arguments_are_checked(yahkv, tor
     rc = yahkv.lib.yahkv_f16_decode_attend(C.byref(g), C.byref(st), table.data_ptr(), 8, table.data_ptr(), 1, 100,
                                            q.data_ptr(), 0, 0.1, None, a.data_ptr(), small.data_ptr(), 16, None)
     assert rc == -4
+
+
+@pytest.mark.parametrize("n_q,n_kv,hd,pt,prefix,chunk", [(24, 4, 256, 64, [700, 64, 0], 130), (8, 2, 128, 16, [33], 64),
+                                                         (12, 4, 128, 32, [500, 1000], 70)])
+def test_prefill_over_f16_pools(yahkv, torch_gpu, n_q, n_kv, hd, pt, prefix, chunk):
+    """Causal attention of a chunk over prefix + chunk in f16 pools, against the float64 closed form over the f16
+    values; the tiles and the numerators are bf16, so the bound is that of the quantized prefill test, 4 x 2^-9."""
+    torch = torch_gpu
+    rng = np.random.default_rng(hd + pt + chunk)
+    B = len(prefix)
+    pages = [(p + chunk + pt - 1) // pt for p in prefix]
+    n_pages = sum(pages)
+    g = yahkv.f16_geometry(n_q, n_kv, hd, pt, n_pages)
+    perm = rng.permutation(n_pages).astype(np.int32)
+    table = np.zeros((B, max(pages)), np.int32)
+    o = 0
+    for s, n in enumerate(pages):
+        table[s, :n] = perm[o:o + n]
+        o += n
+    dev = yahkv.F16Pools(g, fill=0x7E)
+    t_table = torch.from_numpy(table).cuda()
+    src = [(rng.standard_normal((p + chunk, n_kv, hd)).astype(np.float32), rng.standard_normal((p + chunk, n_kv, hd)).astype(np.float32))
+           for p in prefix]
+    for s in range(B):
+        yahkv.f16_append(dev, t_table[s:s + 1], torch.zeros(1, dtype=torch.int32, device="cuda"),
+                         tensor(torch, src[s][0][None], "f32"), tensor(torch, src[s][1][None], "f32"))
+    q = to_bf16_f32(rng.standard_normal((B, chunk, n_q, hd)).astype(np.float32))
+    scale = 1.0 / np.sqrt(hd)
+    out = yahkv.f16_prefill_attend(dev, t_table, torch.tensor(prefix, dtype=torch.int32, device="cuda"), max(prefix),
+                                   tensor(torch, q, "bf16"), scale).float().cpu().numpy()
+    assert np.all(np.isfinite(out))
+    worst = 0.0
+    for s in range(B):
+        K, V = src[s][0].astype(np.float16), src[s][1].astype(np.float16)
+        for t in (0, chunk // 2, chunk - 1):
+            n = prefix[s] + t + 1
+            want = closed_form(K[:n], V[:n], q[s, t], scale, n_q)
+            worst = max(worst, float(np.abs(out[s, t] - want).max() / np.abs(want).max()))
+    assert worst < 4 * 2.0 ** -9, worst

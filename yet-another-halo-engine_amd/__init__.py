@@ -70,6 +70,10 @@ def _load():
     lib.yahkv_f16_pool_bytes.restype = C.c_size_t
     lib.yahkv_f16_pool_bytes.argtypes = [G]
     lib.yahkv_f16_append.argtypes = [G, F, i32p, i32, i32p, i32p, i32, i32, vp, vp, i32, vp]
+    lib.yahkv_f16_prefill_workspace_bytes.restype = C.c_size_t
+    lib.yahkv_f16_prefill_workspace_bytes.argtypes = [G, i32, i32, i32]
+    lib.yahkv_f16_prefill_attend.argtypes = [G, F, i32p, i32, i32p, i32, i32, i32, vp, C.c_float, vp, vp, i32, vp,
+                                             C.c_size_t, vp]
     lib.yahkv_f16_decode_workspace_bytes.restype = C.c_size_t
     lib.yahkv_f16_decode_workspace_bytes.argtypes = [G, i32, i32]
     lib.yahkv_f16_decode_attend.argtypes = [G, F, i32p, i32, i32p, i32, i32, vp, i32, C.c_float, vp, vp, vp,
@@ -239,6 +243,24 @@ def f16_decode_attend(pools, table, seq_len, max_seq_len, q, scale, gate=None, o
     _check(lib.yahkv_f16_decode_attend(C.byref(g), C.byref(st), _dp(table), table.shape[1], _dp(seq_len), n_seqs,
                                        max_seq_len, _dp(q), _dtype_code(q), scale, _dp(gate), _dp(out),
                                        _dp(workspace), workspace.numel(), _stream()), "f16_decode_attend")
+    return out
+
+
+def f16_prefill_attend(pools, table, prefix_len, max_prefix_len, q, scale, gate=None, out=None, workspace=None):
+    """prefill_attend() over f16 pools; q bf16 [n_seqs][chunk][n_q_heads][D]; returns out (bf16 unless given)."""
+    import torch
+    g = pools.geom
+    n_seqs, chunk = q.shape[0], q.shape[1]
+    assert q.is_contiguous() and q.dtype == torch.bfloat16 and tuple(q.shape[2:]) == (g.n_q_heads, g.head_dim)
+    if out is None:
+        out = torch.empty(q.shape, dtype=torch.bfloat16, device=q.device)
+    if workspace is None:
+        need = lib.yahkv_f16_prefill_workspace_bytes(C.byref(g), n_seqs, max_prefix_len, chunk)
+        workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=q.device)
+    st = pools.struct()
+    _check(lib.yahkv_f16_prefill_attend(C.byref(g), C.byref(st), _dp(table), table.shape[1], _dp(prefix_len), n_seqs,
+                                        max_prefix_len, chunk, _dp(q), scale, _dp(gate), _dp(out), _dtype_code(out),
+                                        _dp(workspace), workspace.numel(), _stream()), "f16_prefill_attend")
     return out
 
 

@@ -397,6 +397,8 @@ struct ImageArgs {
   int32_t n_seqs, max_prefix, chunk_len;
   char* img;
   int32_t tiles_per_pair;
+  const uint16_t* fk;  // unquantized f16 pools (PrefillImagesF16 only): K [page][H][D / 16][PT][16], V^T [page][H][D][PT]
+  const uint16_t* fv;
 };
 
 template <int D>
@@ -471,6 +473,52 @@ __global__ __launch_bounds__(256) void PrefillImages(const ImageArgs a) {
                               : static_cast<float>(int((byte >> shift) & 0xF) - 8);
         v[e] = kk + e < n_keys ? d * code : 0.0f;
       }
+      o[2 * hf] = PackBf16(v[0], v[1]), o[2 * hf + 1] = PackBf16(v[2], v[3]);
+    }
+    *reinterpret_cast<uint4*>(vimg + size_t(p) * 16) = uint4{o[0], o[1], o[2], o[3]};
+  }
+}
+
+// The same images from unquantized f16 pools (the pools of yahkv_f16_append): a conversion f16 -> bf16, round to
+// nearest even, instead of a decode.
+template <int D, int PT>
+__global__ __launch_bounds__(256) void PrefillImagesF16(const ImageArgs a) {
+  constexpr int CPR = D / 8;  // 16-byte chunks per K row
+  const Geom g = a.g;
+  const int H = g.n_kv, tile = blockIdx.x, pair = blockIdx.y, s = pair / H, h = pair % H, tid = threadIdx.x;
+  const int n_keys = ClampPrefix(a.prefix_len, s, a.max_prefix, a.stride, g.pt, a.chunk_len) + a.chunk_len;
+  if (tile * kKeys >= n_keys) return;
+  const int32_t* row = a.table + int64_t(s) * a.stride;
+  char* kimg = a.img + (size_t(pair) * a.tiles_per_pair + tile) * TileImageBytes<D>();
+  char* vimg = kimg + kKeys * D * 2;
+  auto page_head = [&](int key) -> size_t {
+    return size_t(ClampPage(row[min(key / PT, a.stride - 1)], g.n_pages)) * H + h;
+  };
+  for (int p = tid; p < kKeys * CPR; p += 256) {  // K: chunk = dims 8 c .. 8 c + 7 of one key
+    const int key = p / CPR, c = (p % CPR) ^ (key % 8), kk = tile * kKeys + key;
+    uint32_t o[4] = {0u, 0u, 0u, 0u};
+    if (kk < n_keys) {
+      const uint4 w = *reinterpret_cast<const uint4*>(a.fk + page_head(kk) * (size_t(D) * PT) +
+                                                      (size_t(c / 2) * PT + kk % PT) * 16 + (c % 2) * 8);
+      const uint32_t u[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        o[e] = PackBf16(WidenF16(static_cast<uint16_t>(u[e] & 0xFFFF)), WidenF16(static_cast<uint16_t>(u[e] >> 16)));
+    }
+    *reinterpret_cast<uint4*>(kimg + size_t(p) * 16) = uint4{o[0], o[1], o[2], o[3]};
+  }
+  for (int p = tid; p < D * 8; p += 256) {  // V: chunk = 4 + 4 keys of one dim
+    const int dim = p / 8, c = (p % 8) ^ (dim % 8), s2 = c / 4, jg = c % 4;
+    uint32_t o[4];
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf) {
+      const int kk = tile * kKeys + 32 * s2 + 16 * hf + 4 * jg;  // four keys, always within one page
+      const uint2 w = *reinterpret_cast<const uint2*>(a.fv + (page_head(kk) * D + dim) * size_t(PT) + kk % PT);
+      const uint32_t u[2] = {w.x, w.y};
+      float v[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        v[e] = kk + e < n_keys ? WidenF16(static_cast<uint16_t>(u[e / 2] >> (16 * (e % 2)))) : 0.0f;
       o[2 * hf] = PackBf16(v[0], v[1]), o[2 * hf + 1] = PackBf16(v[2], v[3]);
     }
     *reinterpret_cast<uint4*>(vimg + size_t(p) * 16) = uint4{o[0], o[1], o[2], o[3]};
@@ -953,5 +1001,68 @@ extern "C" int yahkv_prefill_attend(const yahkv_geometry* g, const yahkv_pools* 
   else if (m.pt == 32) YAHKV_LAUNCH_PF(128, 32);
   else YAHKV_LAUNCH_PF(128, 16);
 #undef YAHKV_LAUNCH_PF
+  return LaunchStatus();
+}
+
+
+extern "C" size_t yahkv_f16_prefill_workspace_bytes(const yahkv_geometry* g, int32_t n_seqs, int32_t max_prefix_len,
+                                                    int32_t chunk_len) {
+  if (g == nullptr || g->format != YAHKV_KV_F16 || n_seqs <= 0 || max_prefix_len < 0 || chunk_len <= 0) return 0;
+  yahkv_geometry gq = *g;
+  gq.format = YAHKV_Q8_0;
+  if (CheckGeometry(&gq)) return 0;
+  return ImageBytes(MakeGeom(gq), n_seqs, max_prefix_len, chunk_len);
+}
+
+// Chunked-prefill attention over unquantized f16 pools (the pools of yahkv_f16_append; the reference's attention
+// reads its 16-bit K / V pool directly, gen_attn_fa.py:1589-1595): the keys' tile images are converted from the
+// pools, then the same attention kernel as for the quantized formats runs on them.
+extern "C" int yahkv_f16_prefill_attend(const yahkv_geometry* g, const yahkv_f16_pools* pools,
+                                        const int32_t* page_table, int32_t page_table_stride,
+                                        const int32_t* prefix_len, int32_t n_seqs, int32_t max_prefix_len,
+                                        int32_t chunk_len, const void* q, float softmax_scale, const float* gate,
+                                        void* out, int32_t out_dtype, void* workspace, size_t workspace_bytes,
+                                        void* stream) {
+  if (g == nullptr) return YAHKV_ERR_ARG;
+  if (g->format != YAHKV_KV_F16) return YAHKV_ERR_SHAPE;
+  yahkv_geometry gq = *g;
+  gq.format = YAHKV_Q8_0;  // the same limits on heads, head_dim, page size and pool
+  if (const int rc = CheckGeometry(&gq)) return rc;
+  if (pools == nullptr || pools->k == nullptr || pools->v == nullptr || page_table == nullptr || prefix_len == nullptr)
+    return YAHKV_ERR_ARG;
+  if (n_seqs <= 0 || chunk_len <= 0 || max_prefix_len < 0 || page_table_stride <= 0) return YAHKV_ERR_ARG;
+  if ((reinterpret_cast<uintptr_t>(pools->k) | reinterpret_cast<uintptr_t>(pools->v)) & 15) return YAHKV_ERR_ARG;
+  PrefillArgs a{};
+  a.g = MakeGeom(gq);
+  if (int64_t(page_table_stride) * a.g.pt < chunk_len) return YAHKV_ERR_ARG;
+  a.table = page_table, a.stride = page_table_stride, a.prefix_len = prefix_len, a.n_seqs = n_seqs;
+  a.max_prefix = max_prefix_len, a.chunk_len = chunk_len;
+  if (const int rc = PrepareQueries(q, softmax_scale, gate, out, out_dtype, &a)) return rc;
+  if (const int rc = CheckWorkspace(a, workspace, workspace_bytes)) return rc;
+  const int tiles = TilesPerPair(max_prefix_len, chunk_len);
+  if (int64_t(tiles) * (2 * kKeys * a.g.hd * 2) > 0x7fffffffLL) return YAHKV_ERR_SHAPE;
+  ImageArgs ia{};
+  ia.g = a.g, ia.table = page_table, ia.stride = page_table_stride, ia.prefix_len = prefix_len, ia.n_seqs = n_seqs;
+  ia.max_prefix = max_prefix_len, ia.chunk_len = chunk_len, ia.img = static_cast<char*>(workspace);
+  ia.tiles_per_pair = tiles;
+  ia.fk = static_cast<const uint16_t*>(pools->k), ia.fv = static_cast<const uint16_t*>(pools->v);
+  const dim3 igrid(static_cast<unsigned>(tiles), static_cast<unsigned>(n_seqs * a.g.n_kv));
+  hipStream_t st = static_cast<hipStream_t>(stream);
+#define YAHKV_LAUNCH_IMG16(DD, PP) hipLaunchKernelGGL((PrefillImagesF16<DD, PP>), igrid, dim3(256), 0, st, ia)
+  if (a.g.hd == 256 && a.g.pt == 64) YAHKV_LAUNCH_IMG16(256, 64);
+  else if (a.g.hd == 256 && a.g.pt == 32) YAHKV_LAUNCH_IMG16(256, 32);
+  else if (a.g.hd == 256) YAHKV_LAUNCH_IMG16(256, 16);
+  else if (a.g.pt == 64) YAHKV_LAUNCH_IMG16(128, 64);
+  else if (a.g.pt == 32) YAHKV_LAUNCH_IMG16(128, 32);
+  else YAHKV_LAUNCH_IMG16(128, 16);
+#undef YAHKV_LAUNCH_IMG16
+  if (const int rc = LaunchStatus()) return rc;
+  const char* img = static_cast<const char*>(workspace);
+#define YAHKV_LAUNCH_ATT(DD, RR) \
+  hipLaunchKernelGGL((PrefillAttendImg<DD, RR>), AttendGrid(a, RR), dim3(256), 0, st, a, img, tiles)
+  if (a.g.hd == 256) YAHKV_LAUNCH_ATT(256, 2);
+  else if (a.g.group() % 3 == 0) YAHKV_LAUNCH_ATT(128, 3);
+  else YAHKV_LAUNCH_ATT(128, 2);
+#undef YAHKV_LAUNCH_ATT
   return LaunchStatus();
 }
