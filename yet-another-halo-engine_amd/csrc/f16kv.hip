@@ -111,7 +111,11 @@ __global__ __launch_bounds__(64 * kWaves) void PartF16(const F16Args a) {
   constexpr int NG = D / 16;
   const Geom g = a.g;
   const int G = g.group(), H = g.n_kv;
-  const int split = blockIdx.x, h = blockIdx.y, s = blockIdx.z, tid = threadIdx.x;
+  const int h = blockIdx.y, s = blockIdx.z, tid = threadIdx.x;
+  // Workgroups go to the eight XCDs in turn and the number of stretches is a multiple of eight for long contexts, so
+  // stretch j of every sequence would run on XCD j % 8 and the short sequences, which have only the first few, would
+  // all load the same XCDs: every (sequence, head) starts its stretches one XCD further on.
+  const int split = static_cast<int>((blockIdx.x + unsigned(s) * gridDim.y + h) % gridDim.x);
   const int wave = __builtin_amdgcn_readfirstlane(tid / 64), lane = tid % 64;
   const int n32 = lane % 32, half = lane / 32, n16 = lane % 16, kg = lane / 16;
   const int len = min(max(a.seq_len[s], 0), a.max_len);
