@@ -40,6 +40,7 @@ NQ, NKV, HD, PT = 24, 4, 256, 64
 # counter reads for a plain 1 GiB copy); a measurement made outside this script, recorded with its summary.
 TRAFFIC = {"ragged_b64_q8_0": (5.336e9, "profiles/decode_part_q8_0_ragged_b64.md"),
            "b1_ctx32k_q8_0": (8.76e7, "profiles/decode_part_q8_0_b1_ctx32k.md"),
+           "b16_ctx128k_f16": (8.622e9, "profiles/decode_part_f16_b16_ctx128k.md"),
            "b16_ctx128k_q4_0": (2.450e9, "profiles/decode_part_q4_0_b16_ctx128k.md"),
            "prefill_b8_ctx16k_chunk2k_q8_0": (2.150e9, "profiles/prefill_attend_q8_0_b8_ctx16k_chunk2k.md")}
 
@@ -246,10 +247,11 @@ def run_f16(a, wl, torch, yahkv):
     n0 = int(lens[s0]) + 1
     kp, vp = pools.k.view(torch.float16), pools.v.view(torch.float16)
     kp = kp.view(n_pages, NKV, HD // 16, PT, 16)
-    vp = vp.view(n_pages, NKV, HD, PT)
+    run = min(PT, 32)                                    # V^T lies in runs of at most 32 keys
+    vp = vp.view(n_pages, NKV, PT // run, HD, run)
     pg = t_table[s0, :(n0 + PT - 1) // PT].long()
     Kd = kp[pg].permute(0, 3, 1, 2, 4).reshape(-1, NKV, HD)[:n0].double().cpu().numpy()
-    Vd = vp[pg].permute(0, 3, 1, 2).reshape(-1, NKV, HD)[:n0].double().cpu().numpy()
+    Vd = vp[pg].permute(0, 2, 4, 1, 3).reshape(-1, NKV, HD)[:n0].double().cpu().numpy()
     qs = q[s0].double().cpu().numpy()
     err = 0.0
     for h in range(NQ):
@@ -280,7 +282,8 @@ def run_f16(a, wl, torch, yahkv):
         "pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2), "tok_per_s": round(B / (ms * 1e-3), 1),
         "kv_bytes_per_step": int(kv_bytes), "parity_max_rel_err": float(f"{err:.3e}"), "out_fnv1a": first_hash,
         "roofline": {"bound": "hbm", "achieved": round(kgbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(kgbs / HBM_PEAK_GBS, 4), "traffic": None, "traffic_source": None,
+                     "frac": round(kgbs / HBM_PEAK_GBS, 4), "traffic": TRAFFIC.get(a.workload, (None, None))[0],
+                     "traffic_source": TRAFFIC.get(a.workload, (None, None))[1],
                      "kernel": "PartF16<%d, %d> + ReduceF16" % (HD, PT), "kernel_ms": round(kern_ms, 4)},
         "cpu_baseline": None}))
 

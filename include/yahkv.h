@@ -252,7 +252,8 @@ int yahkv_slot_unpack(const yahkv_geometry* g, const yahkv_pools* pools, const i
  * yah_dattn_kvappend (engine/gpu/loom/tools/gen_decode_attn.py:30-94), yah_dattn_part (:97-335) and yah_dattn_reduce
  * (:338-411) on pools of f16 K and f16 V^T, with the page table, positions, clamping and argument meaning of the
  * quantized functions above. geometry.format must be YAHKV_KV_F16; the other limits are the same.
- * Pool layouts per page and kv head (f16 elements): K [head_dim / 16][page_tokens][16], V^T [head_dim][page_tokens];
+ * Pool layouts per page and kv head (f16 elements): K [head_dim / 16][page_tokens][16], V^T
+ * [page_tokens / R][head_dim][R] in runs of R = min(page_tokens, 32) keys;
  * each pool is yahkv_f16_pool_bytes long and 16-byte aligned. 4 * n_kv_heads * head_dim bytes per token. */
 typedef struct yahkv_f16_pools {
   void* k;

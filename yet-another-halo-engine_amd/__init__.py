@@ -203,11 +203,14 @@ class F16Pools:
         return F16PoolsStruct(self.k.data_ptr(), self.v.data_ptr())
 
     def numpy(self):
-        """K as [page][H][D / 16][PT][16] and V^T as [page][H][D][PT], uint16 bit patterns."""
+        """K as [page][H][D / 16][PT][16] and V^T as [page][H][D][PT], uint16 bit patterns (V^T is stored in runs of
+        min(PT, 32) keys, [page][H][PT / run][D][run]; the runs are put back side by side here)."""
         import numpy as np
         g = self.geom
         k = self.k.cpu().numpy().view(np.uint16).reshape(g.n_pages, g.n_kv_heads, g.head_dim // 16, g.page_tokens, 16)
-        v = self.v.cpu().numpy().view(np.uint16).reshape(g.n_pages, g.n_kv_heads, g.head_dim, g.page_tokens)
+        run = min(g.page_tokens, 32)
+        v = self.v.cpu().numpy().view(np.uint16).reshape(g.n_pages, g.n_kv_heads, g.page_tokens // run, g.head_dim, run)
+        v = v.transpose(0, 1, 3, 2, 4).reshape(g.n_pages, g.n_kv_heads, g.head_dim, g.page_tokens)
         return k, v
 
 

@@ -4,7 +4,7 @@
 //
 // Pool layouts, per page and kv head (elements are f16):
 //   K    [D / 16][PT][16]   a lane's 16-byte load is 8 dims of one key; the 32 keys of a tile are 1 KB per 16-dim group
-//   V^T  [D][PT]            a lane's 16-byte load is 8 keys of one dim
+//   V^T  [PT / R][D][R]      in runs of R = min(PT, 32) keys; a lane's 16-byte load is 8 keys of one dim
 // Both products run on the matrix cores in f16 with f32 accumulation, as in the quantized kernel: scores
 // S[head][key] with v_mfma_f32_32x32x16_f16 (queries as A rows, 8 of 32 rows used), O[head][dim] += P V with
 // v_mfma_f32_16x16x32_f16 (P rounded to f16 against the running maximum).
@@ -55,8 +55,11 @@ struct F16Args {
 __device__ __forceinline__ size_t KOffset(const Geom& g, size_t page_head, int dim, int t) {
   return (page_head * (g.hd / 16) + dim / 16) * (size_t(g.pt) * 16) + size_t(t) * 16 + dim % 16;
 }
+// V^T in runs of at most 32 keys: the 32 keys that one wave takes at a time are whole 64-byte rows of one 16 KB
+// block then, where rows of 64 keys would leave every 128-byte line to two waves at different times.
 __device__ __forceinline__ size_t VOffset(const Geom& g, size_t page_head, int dim, int t) {
-  return (page_head * g.hd + dim) * size_t(g.pt) + t;
+  const int run = min(g.pt, 32);
+  return page_head * (size_t(g.hd) * g.pt) + (size_t(t / run) * g.hd + dim) * run + t % run;
 }
 
 // One thread per (token, kv head, dim): K and V of that element, rounded to f16 (round to nearest even: the
@@ -159,9 +162,11 @@ __global__ __launch_bounds__(64 * kWaves) void PartF16(const F16Args a) {
     {  // V^T: this lane's dim of every 16-dim tile, 8 keys (they lie in one page: pages hold multiples of 16 tokens)
       const int key = key0 + 8 * kg;
       const int page = ClampPage(row[min(key / PT, a.stride - 1)], g.n_pages);
-      const uint16_t* vp = a.v + (size_t(page) * H + h) * (size_t(D) * PT) + n16 * PT + key % PT;
+      constexpr int RUN = PT < 32 ? PT : 32;
+      const uint16_t* vp =
+          a.v + (size_t(page) * H + h) * (size_t(D) * PT) + (key % PT / RUN * D + n16) * RUN + key % RUN;
 #pragma unroll
-      for (int nt = 0; nt < NG; ++nt) vb[nt] = *reinterpret_cast<const h8v*>(vp + 16 * nt * PT);
+      for (int nt = 0; nt < NG; ++nt) vb[nt] = *reinterpret_cast<const h8v*>(vp + 16 * nt * RUN);
     }
     f16v c = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll

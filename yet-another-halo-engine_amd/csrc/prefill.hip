@@ -397,7 +397,7 @@ struct ImageArgs {
   int32_t n_seqs, max_prefix, chunk_len;
   char* img;
   int32_t tiles_per_pair;
-  const uint16_t* fk;  // unquantized f16 pools (PrefillImagesF16 only): K [page][H][D / 16][PT][16], V^T [page][H][D][PT]
+  const uint16_t* fk;  // unquantized f16 pools (PrefillImagesF16 only): K [page][H][D / 16][PT][16], V^T [page][H][PT / R][D][R], R = min(PT, 32)
   const uint16_t* fv;
 };
 
@@ -513,7 +513,9 @@ __global__ __launch_bounds__(256) void PrefillImagesF16(const ImageArgs a) {
 #pragma unroll
     for (int hf = 0; hf < 2; ++hf) {
       const int kk = tile * kKeys + 32 * s2 + 16 * hf + 4 * jg;  // four keys, always within one page
-      const uint2 w = *reinterpret_cast<const uint2*>(a.fv + (page_head(kk) * D + dim) * size_t(PT) + kk % PT);
+      constexpr int RUN = PT < 32 ? PT : 32;  // V^T lies in runs of at most 32 keys
+      const uint2 w = *reinterpret_cast<const uint2*>(a.fv + page_head(kk) * (size_t(D) * PT) +
+                                                      (size_t(kk % PT / RUN) * D + dim) * RUN + kk % RUN);
       const uint32_t u[2] = {w.x, w.y};
       float v[4];
 #pragma unroll
