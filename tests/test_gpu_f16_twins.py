@@ -213,3 +213,31 @@ def test_prefill_over_f16_pools(yahkv, torch_gpu, n_q, n_kv, hd, pt, prefix, chu
             want = closed_form(K[:n], V[:n], q[s, t], scale, n_q)
             worst = max(worst, float(np.abs(out[s, t] - want).max() / np.abs(want).max()))
     assert worst < 4 * 2.0 ** -9, worst
+
+
+def test_prefill_over_f16_pools_checks_its_arguments(yahkv, torch_gpu):
+    import ctypes as C
+    torch = torch_gpu
+    g = yahkv.f16_geometry(8, 2, 128, 16, 8)
+    dev = yahkv.F16Pools(g)
+    table = torch.arange(8, dtype=torch.int32, device="cuda")[None]
+    prefix = torch.zeros(1, dtype=torch.int32, device="cuda")
+    q = torch.zeros((1, 32, 8, 128), dtype=torch.bfloat16, device="cuda")
+    out = torch.empty_like(q)
+    need = yahkv.lib.yahkv_f16_prefill_workspace_bytes(C.byref(g), 1, 0, 32)
+    assert need > 0
+    g8 = yahkv.geometry(8, 8, 2, 128, 16, 8)
+    assert yahkv.lib.yahkv_f16_prefill_workspace_bytes(C.byref(g8), 1, 0, 32) == 0
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    st = dev.struct()
+
+    def call(geom, workspace, n_bytes, chunk=32):
+        return yahkv.lib.yahkv_f16_prefill_attend(C.byref(geom), C.byref(st), table.data_ptr(), 8, prefix.data_ptr(), 1,
+                                                  0, chunk, q.data_ptr(), 0.1, None, out.data_ptr(), 2,
+                                                  workspace, n_bytes, None)
+    assert call(g8, ws.data_ptr(), need) == -2           # a quantized geometry
+    assert call(g, None, 0) == -1                        # the workspace is required
+    assert call(g, ws.data_ptr(), need - 1) == -4        # and must hold the tile images
+    assert call(g, ws.data_ptr(), need, chunk=16 * 8 + 1) == -1   # more chunk positions than the table has rows for
+    assert call(g, ws.data_ptr(), need) == 0
+    torch.cuda.synchronize()
