@@ -81,6 +81,34 @@ def test_positions_clamp_and_the_last_token_wins(yahkv, torch_gpu):
     assert np.array_equal(V[31, 0], (-x[0, 9, 0]).astype(np.float16))
 
 
+@pytest.mark.parametrize("kind", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("hd,pt", [(128, 16), (256, 32), (256, 64), (128, 64)])
+def test_a_chunk_appended_at_once_equals_its_tokens_one_by_one(yahkv, torch_gpu, kind, hd, pt):
+    """Chunks take the kernel that works run by run, single tokens the one that works element by element: the pools
+    must come out the same, byte for byte, also where positions clamp at either end and where a chunk is padded."""
+    torch = torch_gpu
+    rng = np.random.default_rng(hd + pt)
+    n_kv, stride, n_new = 2, 5, 70
+    starts = [3, -4, stride * pt - 40, 17, pt]      # inside, before the start, past the end, odd, on a page edge
+    valid = [70, 70, 70, 33, 9]
+    B = len(starts)
+    g = yahkv.f16_geometry(4, n_kv, hd, pt, B * stride)
+    table = torch.from_numpy(rng.permutation(B * stride).astype(np.int32).reshape(B, stride)).cuda()
+    k = rng.standard_normal((B, n_new, n_kv, hd)).astype(np.float32) * 3
+    v = rng.standard_normal((B, n_new, n_kv, hd)).astype(np.float32) * 3
+    tk, tv = tensor(torch, k, kind), tensor(torch, v, kind)
+    at_once, one_by_one = yahkv.F16Pools(g, fill=0x5A), yahkv.F16Pools(g, fill=0x5A)
+    yahkv.f16_append(at_once, table, torch.tensor(starts, dtype=torch.int32, device="cuda"), tk, tv,
+                     n_valid=torch.tensor(valid, dtype=torch.int32, device="cuda"))
+    for s in range(B):
+        for i in range(valid[s]):
+            yahkv.f16_append(one_by_one, table[s:s + 1], torch.tensor([starts[s] + i], dtype=torch.int32, device="cuda"),
+                             tk[s:s + 1, i:i + 1].contiguous(), tv[s:s + 1, i:i + 1].contiguous())
+    assert torch.equal(at_once.k, one_by_one.k)
+    assert torch.equal(at_once.v, one_by_one.v)
+    assert int((at_once.k != 0x5A).sum()) > 0
+
+
 def closed_form(K, V, q, scale, n_q):
     """float64 softmax(q K^T scale) V over f16 K, V [n][H][D]; q [n_q][D]."""
     n_kv = K.shape[1]

@@ -23,6 +23,7 @@ typedef float f16v __attribute__((ext_vector_type(16)));
 constexpr int kTileKeys = 32;   // keys per tile (one wave, one pass)
 constexpr int kWaves = 4;       // waves per workgroup; they take the tiles of the workgroup's stretch in turn
 constexpr int kMaxHeads = 8;    // query heads per kv head
+constexpr int kRunAppendMinTokens = 8;  // chunks of at least this many tokens per sequence go run by run
 constexpr float kLowest = -3.4028234663852886e+38f;
 constexpr float kLog2e = 1.4426950408889634f, kLn2 = 0.6931471805599453f;
 
@@ -84,6 +85,91 @@ __global__ __launch_bounds__(256) void AppendF16(const F16Args a) {
   const _Float16 vh = static_cast<_Float16>(LoadSrc(a.v_src, src, a.src_dtype));
   a.k[KOffset(g, ph, d, pos % PT)] = __builtin_bit_cast(uint16_t, kh);
   a.v[VOffset(g, ph, d, pos % PT)] = __builtin_bit_cast(uint16_t, vh);
+}
+
+// Eight consecutive source elements from index i (a multiple of 8, the array 16-byte aligned), rounded to f16.
+__device__ __forceinline__ uint4 Rows8(const void* p, size_t i, int dt) {
+  if (dt == YAHKV_F16) return *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(p) + i);
+  float x[8];
+  if (dt == YAHKV_F32) {
+    const float4 lo = *reinterpret_cast<const float4*>(static_cast<const float*>(p) + i);
+    const float4 hi = *reinterpret_cast<const float4*>(static_cast<const float*>(p) + i + 4);
+    x[0] = lo.x, x[1] = lo.y, x[2] = lo.z, x[3] = lo.w, x[4] = hi.x, x[5] = hi.y, x[6] = hi.z, x[7] = hi.w;
+  } else {
+    const uint4 w = *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(p) + i);
+    const uint32_t u[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = WidenBf16(static_cast<uint16_t>(u[e / 2] >> (16 * (e % 2))));
+  }
+  uint32_t o[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e)
+    o[e] = uint32_t(__builtin_bit_cast(uint16_t, static_cast<_Float16>(x[2 * e]))) |
+           uint32_t(__builtin_bit_cast(uint16_t, static_cast<_Float16>(x[2 * e + 1]))) << 16;
+  return uint4{o[0], o[1], o[2], o[3]};
+}
+
+// The same append for chunks: a workgroup takes one kv head of one aligned run of T = min(PT, 32) positions (one run
+// of the V^T layout), reads the tokens' rows with 16-byte loads, turns them round in LDS and writes K as 1 KB pieces
+// and the V^T run as one 16 KB piece. Which token of the chunk a slot takes (clamped positions: the last one wins)
+// is decided per slot, with the rule of AppendF16.
+template <int T>
+__global__ __launch_bounds__(256) void AppendF16Runs(const F16Args a) {
+  const Geom g = a.g;
+  const int H = g.n_kv, PT = g.pt, D = g.hd, C = D / 8;
+  const int h = blockIdx.y, s = blockIdx.z, tid = threadIdx.x;
+  const int nv = a.n_valid != nullptr ? min(max(a.n_valid[s], 0), a.n_new) : a.n_new;
+  if (nv <= 0) return;
+  const int64_t start = a.start_pos[s], last_pos = int64_t(a.stride) * PT - 1;
+  const int64_t lo = min(max(start, int64_t(0)), last_pos), hi = min(max(start + nv - 1, int64_t(0)), last_pos);
+  const int64_t p0 = (lo / T + blockIdx.x) * T;
+  if (p0 > hi) return;
+  constexpr int kRow = 256 + 8;  // f16 elements per token in LDS (head_dim <= 256), padded against bank conflicts
+  __shared__ __align__(16) uint16_t lk[T][kRow];
+  __shared__ __align__(16) uint16_t lv[T][kRow];
+  __shared__ int lsrc[T];
+  if (tid < T) {
+    const int64_t p = p0 + tid;
+    int64_t src = p - start;
+    if (p == last_pos && start + nv - 1 >= last_pos) src = nv - 1;
+    if (p == 0 && start <= 0) src = min(int64_t(nv - 1), -start);
+    lsrc[tid] = src >= 0 && src < nv ? static_cast<int>(src) : -1;
+  }
+  __syncthreads();
+  for (int e = tid; e < T * C; e += 256) {
+    const int t = e / C, c = e % C, src = lsrc[t];
+    if (src < 0) continue;
+    const size_t at = ((size_t(s) * a.n_new + src) * H + h) * D + 8 * c;
+    *reinterpret_cast<uint4*>(&lk[t][8 * c]) = Rows8(a.k_src, at, a.src_dtype);
+    *reinterpret_cast<uint4*>(&lv[t][8 * c]) = Rows8(a.v_src, at, a.src_dtype);
+  }
+  __syncthreads();
+  const int page = ClampPage(a.table[int64_t(s) * a.stride + p0 / PT], g.n_pages);
+  const size_t ph = size_t(page) * H + h;
+  const int t0 = static_cast<int>(p0 % PT);
+  for (int e = tid; e < T * C; e += 256) {  // K: 16 dims of T tokens are 32 T bytes in a row
+    const int g16 = e / (2 * T), t = e / 2 % T, hf = e % 2;
+    if (lsrc[t] < 0) continue;
+    *reinterpret_cast<uint4*>(a.k + KOffset(g, ph, 16 * g16 + 8 * hf, t0 + t)) =
+        *reinterpret_cast<const uint4*>(&lk[t][16 * g16 + 8 * hf]);
+  }
+  for (int e = tid; e < D * (T / 8); e += 256) {  // V^T: T tokens of a dim in a row, the dims one after the other
+    const int d = e / (T / 8), j = e % (T / 8);
+    uint16_t w[8];
+    bool all = true;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) w[i] = lv[8 * j + i][d], all = all && lsrc[8 * j + i] >= 0;
+    uint16_t* dst = a.v + VOffset(g, ph, d, t0 + 8 * j);
+    if (all) {
+      *reinterpret_cast<uint4*>(dst) =
+          uint4{uint32_t(w[0]) | uint32_t(w[1]) << 16, uint32_t(w[2]) | uint32_t(w[3]) << 16,
+                uint32_t(w[4]) | uint32_t(w[5]) << 16, uint32_t(w[6]) | uint32_t(w[7]) << 16};
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        if (lsrc[8 * j + i] >= 0) dst[i] = w[i];
+    }
+  }
 }
 
 __device__ __forceinline__ float HalfMax(float v) {  // over the 32 lanes of a wave half
@@ -370,8 +456,19 @@ extern "C" int yahkv_f16_append(const yahkv_geometry* g, const yahkv_f16_pools* 
   a.g = MakeGeom(*g), a.k = static_cast<uint16_t*>(pools->k), a.v = static_cast<uint16_t*>(pools->v);
   a.table = page_table, a.stride = page_table_stride, a.start_pos = start_pos, a.n_valid = n_valid;
   a.n_seqs = n_seqs, a.n_new = n_new, a.k_src = k_src, a.v_src = v_src, a.src_dtype = src_dtype;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const bool aligned = ((reinterpret_cast<uintptr_t>(k_src) | reinterpret_cast<uintptr_t>(v_src) |
+                         reinterpret_cast<uintptr_t>(pools->k) | reinterpret_cast<uintptr_t>(pools->v)) & 15) == 0;
+  if (n_new >= kRunAppendMinTokens && aligned) {  // chunks: a workgroup per run of positions
+    const int T = std::min(a.g.pt, 32);
+    const dim3 grid(static_cast<unsigned>((n_new + T - 2) / T + 1), static_cast<unsigned>(a.g.n_kv),
+                    static_cast<unsigned>(n_seqs));
+    if (T == 32) hipLaunchKernelGGL(AppendF16Runs<32>, grid, dim3(256), 0, st, a);
+    else hipLaunchKernelGGL(AppendF16Runs<16>, grid, dim3(256), 0, st, a);
+    return LaunchStatus();
+  }
   const dim3 grid(static_cast<unsigned>(n_new), static_cast<unsigned>(a.g.n_kv), static_cast<unsigned>(n_seqs));
-  hipLaunchKernelGGL(AppendF16, grid, dim3(256), 0, static_cast<hipStream_t>(stream), a);
+  hipLaunchKernelGGL(AppendF16, grid, dim3(256), 0, st, a);
   return LaunchStatus();
 }
 
