@@ -33,6 +33,7 @@ WORKLOADS = {
     # the unquantized f16 twins of the decode path (4096 B per token)
     "b16_ctx128k_f16": dict(fmt=16, batch=16, lo=131072, hi=131072, seed=4),
     "ragged_b64_f16": dict(fmt=16, batch=64, lo=1024, hi=65536, seed=4),
+    "prefill_b8_ctx16k_chunk2k_f16": dict(fmt=16, batch=8, lo=16384, hi=16384, seed=4, chunk=2048),
 }
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 NQ, NKV, HD, PT = 24, 4, 256, 64
@@ -377,6 +378,90 @@ def run_prefill(a, wl, torch, yahkv):
     print(json.dumps(res))
 
 
+def run_prefill_f16(a, wl, torch, yahkv):
+    """The prefill step on unquantized f16 pools: append the chunk, then one call that converts prefix + chunk to
+    bf16 tiles and runs the causal attention."""
+    B, chunk, prefix = wl["batch"], wl["chunk"], wl["lo"]
+    rng = np.random.default_rng(wl["seed"])
+    per_seq = (prefix + chunk + PT - 1) // PT
+    n_pages = B * per_seq
+    g = yahkv.f16_geometry(NQ, NKV, HD, PT, n_pages)
+    t_table = torch.from_numpy(rng.permutation(n_pages).astype(np.int32).reshape(B, per_seq)).cuda()
+    pools = yahkv.F16Pools(g)
+    gen = torch.Generator(device="cuda").manual_seed(wl["seed"])
+    for s in range(B):
+        for o in range(0, prefix, 8192):
+            n = min(8192, prefix - o)
+            k = torch.randn((1, n, NKV, HD), generator=gen, device="cuda").to(torch.bfloat16)
+            v = torch.randn((1, n, NKV, HD), generator=gen, device="cuda").to(torch.bfloat16)
+            yahkv.f16_append(pools, t_table[s:s + 1], torch.tensor([o], dtype=torch.int32, device="cuda"), k, v)
+    scale = 1.0 / float(np.sqrt(HD))
+    t_prefix = torch.full((B,), prefix, dtype=torch.int32, device="cuda")
+    q = torch.randn((B, chunk, NQ, HD), generator=gen, device="cuda").to(torch.bfloat16)
+    knew = torch.randn((B, chunk, NKV, HD), generator=gen, device="cuda").to(torch.bfloat16)
+    vnew = torch.randn((B, chunk, NKV, HD), generator=gen, device="cuda").to(torch.bfloat16)
+    out = torch.empty(q.shape, dtype=torch.bfloat16, device="cuda")
+    ws = torch.empty(yahkv.lib.yahkv_f16_prefill_workspace_bytes(g, B, prefix, chunk), dtype=torch.uint8, device="cuda")
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(a.steps)]
+
+    def step(pair=None):
+        yahkv.f16_append(pools, t_table, t_prefix, knew, vnew)
+        if pair:
+            pair[0].record()
+        yahkv.f16_prefill_attend(pools, t_table, t_prefix, prefix, q, scale, out=out, workspace=ws)
+        if pair:
+            pair[1].record()
+
+    # parity before timing: float64 closed form over the pools' own f16 values, a few (query, head) rows of sequence 0
+    step()
+    torch.cuda.synchronize()
+    first_hash = fnv1a(out.view(torch.int16).cpu().numpy().tobytes())
+    n = prefix + chunk
+    run = min(PT, 32)
+    kp = pools.k.view(torch.float16).view(n_pages, NKV, HD // 16, PT, 16)
+    vp = pools.v.view(torch.float16).view(n_pages, NKV, PT // run, HD, run)
+    pg = t_table[0].long()
+    Kd = kp[pg].permute(0, 3, 1, 2, 4).reshape(-1, NKV, HD)[:n].double().cpu().numpy()
+    Vd = vp[pg].permute(0, 2, 4, 1, 3).reshape(-1, NKV, HD)[:n].double().cpu().numpy()
+    err = 0.0
+    for t in (0, chunk // 2, chunk - 1):
+        for h in (0, NQ - 1):
+            sc = Kd[:prefix + t + 1, h // (NQ // NKV)] @ q[0, t, h].double().cpu().numpy() * scale
+            pr = np.exp(sc - sc.max())
+            want = (pr / pr.sum()) @ Vd[:prefix + t + 1, h // (NQ // NKV)]
+            got = out[0, t, h].float().cpu().numpy()
+            err = max(err, float(np.abs(got - want).max() / np.abs(want).max()))
+    if not err < 4 * 2.0 ** -9:
+        raise SystemExit(f"bench.py: parity check failed before timing: max relative error {err:.3e}")
+    for _ in range(a.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(a.steps):
+        step(ev[i])
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / a.steps * 1e3
+    kern_ms = float(np.mean([p[0].elapsed_time(p[1]) for p in ev]))
+    flops = float(B) * NQ * chunk * (prefix + (chunk + 1) / 2) * HD * 4
+    print(json.dumps({
+        "metric": "chunked-prefill attention over paged f16 KV, TFLOP/s (bf16 MFMA) + tok/s",
+        "value": round(flops / (ms * 1e-3) / 1e12, 1), "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps,
+        "warmup": a.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": a.workload, "batch": B, "prefix": prefix, "chunk": chunk, "n_q_heads": NQ,
+                   "n_kv_heads": NKV, "head_dim": HD, "page_tokens": PT, "n_pages": n_pages, "kv_format": "f16",
+                   "step": "append chunk (f16 rounding + scatter) + f16 pages to bf16 tiles + causal attention"},
+        "tok_per_s": round(B * chunk / (ms * 1e-3), 1), "flops_per_step": int(flops),
+        "parity_max_rel_err": float(f"{err:.3e}"), "out_fnv1a": first_hash,
+        "roofline": {"bound": "mfma", "achieved": round(flops / (kern_ms * 1e-3) / 1e12, 1),
+                     "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(flops / (kern_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+                     "traffic": None, "traffic_source": None,
+                     "kernel": "PrefillImagesF16<%d, %d> + PrefillAttendImg<%d, 2>" % (HD, PT, HD),
+                     "kernel_ms": round(kern_ms, 4)},
+        "cpu_baseline": None}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -401,6 +486,8 @@ def main():
         print(json.dumps({"copy_calibration": {"bytes_read": 1 << 30, "bytes_written": 1 << 30, "copies": 5}}))
         return
     wl = WORKLOADS[a.workload]
+    if "chunk" in wl and wl["fmt"] == 16:
+        return run_prefill_f16(a, wl, torch, yahkv)
     if "chunk" in wl:
         return run_prefill(a, wl, torch, yahkv)
     if wl["fmt"] == 16:
