@@ -136,8 +136,27 @@ CASES = [  # n_q, n_kv, hd, pt, lengths
 @pytest.mark.parametrize("n_q,n_kv,hd,pt,lens", CASES)
 @pytest.mark.parametrize("qkind", ["bf16", "f32"])
 def test_decode_against_the_closed_form(yahkv, torch_gpu, n_q, n_kv, hd, pt, lens, qkind):
-    torch = torch_gpu
-    rng = np.random.default_rng(n_q * 1000 + hd + pt)
+    check_decode(yahkv, torch_gpu, n_q, n_kv, hd, pt, lens, qkind, n_q * 1000 + hd + pt)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_decode_on_random_shapes_and_cuts(yahkv, torch_gpu, seed, monkeypatch):
+    """Random group sizes, head dims, page sizes, ragged and empty sequences, and the number of stretches a sequence
+    is cut into forced from one per sequence to one per 128 keys: every cut gives the closed form."""
+    rng = np.random.default_rng(1000 + seed)
+    n_kv, group = int(rng.choice([1, 2, 4])), int(rng.integers(1, 9))
+    hd, pt = int(rng.choice([128, 256])), int(rng.choice([16, 32, 64]))
+    lens = [int(x) for x in rng.integers(0, 3000, int(rng.integers(1, 6)))]
+    if max(lens) == 0:
+        lens[0] = 1
+    wgs = [None, "1", "64", "1000000"][seed % 4]
+    if wgs is not None:
+        monkeypatch.setenv("YAHKV_F16_WORKGROUPS", wgs)
+    check_decode(yahkv, torch_gpu, n_kv * group, n_kv, hd, pt, lens, ["bf16", "f32", "f16"][seed % 3], seed)
+
+
+def check_decode(yahkv, torch, n_q, n_kv, hd, pt, lens, qkind, seed):
+    rng = np.random.default_rng(seed)
     B, max_len = len(lens), max(lens)
     pages = [(l + pt - 1) // pt for l in lens]
     stride = max(max(pages), 1)
@@ -160,6 +179,8 @@ def test_decode_against_the_closed_form(yahkv, torch_gpu, n_q, n_kv, hd, pt, len
     q = rng.standard_normal((B, n_q, hd)).astype(np.float32)
     if qkind == "bf16":
         q = to_bf16_f32(q)
+    if qkind == "f16":
+        q = q.astype(np.float16).astype(np.float32)
     gate = rng.standard_normal((B, n_q, hd)).astype(np.float32) if qkind == "f32" else None
     scale = 1.0 / np.sqrt(hd)
     out = yahkv.f16_decode_attend(dev, t_table, torch.tensor(lens, dtype=torch.int32, device="cuda"), max_len,
