@@ -547,7 +547,9 @@ def main():
     gbs = kv_bytes / (ms * 1e-3) / 1e9
     kgbs = kv_bytes / (kern_ms * 1e-3) / 1e9
     res = {
-        "metric": "paged q8 KV decode-attn HBM GB/s (% of peak) + tok/s, B=64 ragged ctx",
+        "metric": ("paged q8 KV decode-attn HBM GB/s (% of peak) + tok/s, B=64 ragged ctx"
+                   if a.workload == "ragged_b64_q8_0" else
+                   "paged q%d KV decode-attn HBM GB/s (%% of peak) + tok/s" % wl["fmt"]),
         "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "u8" if wl["fmt"] == 8 else "u4", "data": "synthetic",
