@@ -469,6 +469,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="ragged_b64_q8_0", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--graph-replay", action="store_true",
+                    help="decode workloads: also replay the timed steps as one HIP graph and report its time per step")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run plain device copies of 1 GiB (to scale rocprofv3's FETCH_SIZE / WRITE_SIZE)")
     a = ap.parse_args()
@@ -564,6 +566,29 @@ def main():
                      "traffic_source": TRAFFIC.get(a.workload, (None, None))[1],
                      "kernel": "DattnPart<%d, %d, %d>" % (wl["fmt"], HD, PT), "kernel_ms": round(kern_ms, 4)},
     }
+    if a.graph_replay:
+        # The same timed steps (same tokens at the same positions: the pools end up as they are) recorded once into
+        # a HIP graph, so the launches follow each other without the host in between; an extra figure, not `value`.
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(graph, stream=side):
+                for i in range(a.steps):
+                    step(1 + a.warmup + i)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        times = []
+        for _ in range(5):
+            t0 = time.perf_counter()
+            graph.replay()
+            torch.cuda.synchronize()
+            times.append((time.perf_counter() - t0) / a.steps * 1e3)
+        gms = float(np.median(times))
+        res["graph_replay"] = {"ms_per_step": round(gms, 4), "GB/s": round(kv_bytes / (gms * 1e-3) / 1e9, 1),
+                               "tok_per_s": round(B / (gms * 1e-3), 1),
+                               "note": "the timed steps replayed as one HIP graph, median of 5 replays"}
     if not a.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline(wl, lens, scale)
     print(json.dumps(res))
