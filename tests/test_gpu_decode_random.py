@@ -84,3 +84,23 @@ def test_chunks_of_one_or_two_units(yahkv, torch_gpu, monkeypatch):
         got = gpu_attend(yahkv, torch_gpu, dev, table, lens, q, 0.0625, max_len=896)
         assert np.all(np.isfinite(got))
         assert rel_err(got, oracle.decode_attend(host, table, lens, q, 0.0625)) < TOL
+
+
+def test_the_largest_batch_a_call_takes_and_one_more(yahkv, torch_gpu):
+    """8191 sequences in one call (the limit) against the oracle; 8192 are refused as a shape this build has no
+    kernel for, before anything is launched."""
+    torch = torch_gpu
+    rng = np.random.default_rng(79)
+    n_seqs, n_kv, group, hd, pt = 8191, 1, 2, 128, 16
+    lens = [int(x) for x in rng.integers(0, 21, n_seqs)]
+    g, table, host, dev, _ = setup(yahkv, torch, 8, n_kv * group, n_kv, hd, pt, lens, seed=80, fill=0x7F)
+    q = to_bf16_f32(rng.standard_normal((n_seqs, n_kv * group, hd)))
+    scale = float(1 / np.sqrt(hd))
+    got = gpu_attend(yahkv, torch, dev, table, lens, q, scale)
+    want = oracle.decode_attend(host, table, lens, q, scale)
+    assert np.all(np.isfinite(got))
+    assert rel_err(got, want) < TOL
+    more = np.concatenate([table, table[:1]])
+    with pytest.raises(yahkv.YahkvError) as e:
+        gpu_attend(yahkv, torch, dev, more, lens + [1], np.concatenate([q, q[:1]]), scale)
+    assert e.value.status == -2
