@@ -9,10 +9,13 @@
  *                          source (oracle/_ref) and against committed golden vectors made with it
  *   orc_dequantize_q8_0/4_0  bit-exact against the reference's yah::core::Dequantize (oracle/_ref) + golden vectors
  *   orc_f16 / bf16 conversions  brute force over all 65536 bit patterns and directed f32 cases against numpy
- *   orc_quantize_q4_0      PARITY UNPINNED against the reference: it has no q4_0 quantizer. Restates ggml's
- *                          published quantize_row_q4_0_ref (llama.cpp ggml-quants.c, the file
+ *   orc_quantize_q4_0      the reference has no q4_0 quantizer; this restates ggml's published
+ *                          quantize_row_q4_0_ref (llama.cpp ggml-quants.c, the file
  *                          engine/core/gguf_quant.cpp:1 cites; not vendored, no version pinned by the
- *                          reference); checked by invariants only
+ *                          reference). Pinned by known answers worked out by hand from that rule
+ *                          (tests/q4_known_answers.py: halves round up, the clip at code 15, the first of two
+ *                          equal magnitudes decides the sign of the scale at every pair of positions, a
+ *                          scale that is no power of two, the zero block) and by its invariants on random data
  *   orc_append / orc_gather_blocks  page scatter: gather-through-table == contiguous quantize, poison-fill
  *                          proves untouched bytes, brute force on tiny inputs
  *   orc_decode_attend      float64 closed-form softmax over dequantized K/V (what

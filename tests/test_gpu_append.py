@@ -81,6 +81,35 @@ def test_q8_0_golden_blocks_from_the_reference(yahkv, torch_gpu, golden):
     assert np.array_equal(v.cpu().numpy().reshape(-1, 34)[:len(x)], want)
 
 
+@pytest.mark.parametrize("kind", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("hd,pt,n_new", [(128, 16, 1), (256, 64, 1), (256, 64, 64), (128, 32, 24)])
+def test_q4_0_known_answers_through_the_append(yahkv, torch_gpu, kind, hd, pt, n_new):
+    """The hand-computed q4_0 blocks of tests/q4_known_answers.py (ties, clip, first of two equal magnitudes at every
+    pair of positions) through yahkv_append, token by token and as chunks, K and V, then read back as ggml blocks."""
+    torch = torch_gpu
+    from q4_known_answers import known_answers
+    x, want, names = known_answers()
+    n_kv = 2
+    per_tok = n_kv * hd // 32
+    n_tok = (len(x) + per_tok - 1) // per_tok
+    n_tok = (n_tok + n_new - 1) // n_new * n_new
+    xp = np.zeros((n_tok * per_tok, 32), np.float32)
+    xp[:len(x)] = x
+    src = xp.reshape(1, n_tok, n_kv, hd)
+    pages = (n_tok + pt - 1) // pt
+    g = yahkv.geometry(4, 2 * n_kv, n_kv, hd, pt, pages)
+    dev = yahkv.DevicePools(g, fill=0x5A)
+    table = torch.from_numpy(np.random.default_rng(1).permutation(pages).astype(np.int32)[None]).cuda()
+    t = torch_src(torch, src, kind)
+    for o in range(0, n_tok, n_new):
+        yahkv.append(dev, table, torch.tensor([o], dtype=torch.int32, device="cuda"), t[:, o:o + n_new], t[:, o:o + n_new])
+    k, v = yahkv.gather_blocks(dev, table[0], n_tok)
+    for what, got in (("K", k), ("V", v)):
+        got = got.cpu().numpy().reshape(-1, 18)[:len(x)]
+        for i in np.flatnonzero((got != want).any(1)):
+            raise AssertionError(f"{what} block '{names[i]}': got {got[i].tolist()}, want {want[i].tolist()}")
+
+
 def test_append_clamps_bad_positions_and_pages(yahkv, torch_gpu):
     """Positions past the table and page ids outside the pool are clamped, never written out of bounds."""
     torch = torch_gpu

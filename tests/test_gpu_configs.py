@@ -1,0 +1,159 @@
+"""The benchmark configurations that the other GPU tests do not reach at their own geometry and size, through the
+C ABI, in the manner of the reference's checker (engine/gpu/loom/tools/dattn_q_check.py:140-256: seeded inputs, a
+scrambled page table, pools filled with poison first, appended bytes bit-exact, attention against the float64
+closed form over the dequantized blocks):
+  config 2   one sequence of 32768 tokens, q8_0, 24 Q / 4 KV heads, head_dim 256, 64-token pages, a 1024-page pool
+             of which a seeded permutation hands out 512 (+ 1 for the appended token), bf16 query
+  config 5   q4_0, batch 16, the same heads, K with 8 seeded outlier channels per head scaled x 20; at 2048 tokens per
+             sequence against the oracle, and at the full 131072 tokens per sequence against the closed form on the
+             gathered blocks of two sequences; one token appended per sequence before the attention
+"""
+import numpy as np
+import pytest
+
+import oracle
+from helpers import bf16_bits, closed_form, make_tables, rel_err, to_bf16_f32
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-3
+NQ, NKV, HD, PT = 24, 4, 256, 64
+
+
+def bf16_cuda(torch, x):
+    return torch.from_numpy(bf16_bits(x).view(np.int16)).cuda().view(torch.bfloat16)
+
+
+def closed_from_blocks(yahkv, dev, t_row, n, q, scale, fmt):
+    """Float64 closed form over what the library's own pools hold for one sequence (its blocks in ggml order)."""
+    k, v = yahkv.gather_blocks(dev, t_row, n)
+    bb = 34 if fmt == 8 else 18
+    deq = oracle.dequantize_q8_0 if fmt == 8 else oracle.dequantize_q4_0
+    Kd = deq(k.cpu().numpy().reshape(-1, bb)).reshape(n, NKV, HD)
+    Vd = deq(v.cpu().numpy().reshape(-1, bb)).reshape(n, NKV, HD)
+    return closed_form(Kd, Vd, q, scale)
+
+
+def test_config2_one_sequence_of_32768_tokens(yahkv, torch_gpu):
+    torch = torch_gpu
+    rng = np.random.default_rng(22)
+    n, pool_pages = 32768, 1024
+    g = oracle.geometry(8, NQ, NKV, HD, PT, pool_pages)
+    table = rng.permutation(pool_pages).astype(np.int32)[None, :n // PT + 1]        # 513 of the 1024 pages
+    K = to_bf16_f32(rng.standard_normal((1, n + 1, NKV, HD)))
+    V = to_bf16_f32(rng.standard_normal((1, n + 1, NKV, HD)))
+    q = to_bf16_f32(rng.standard_normal((1, NQ, HD)))
+    host = oracle.HostPools(g, fill=0x7F)                                           # f16 0x7F7F is NaN: poison
+    oracle.append(host, table, [0], None, K, V)
+    dev = yahkv.DevicePools(yahkv.geometry(8, NQ, NKV, HD, PT, pool_pages), fill=0x7F)
+    t_table = torch.from_numpy(table).cuda()
+    for o in range(0, n, 8192):                                                     # the prefix in chunks ...
+        yahkv.append(dev, t_table, torch.tensor([o], dtype=torch.int32, device="cuda"),
+                     bf16_cuda(torch, K[:, o:o + 8192]), bf16_cuda(torch, V[:, o:o + 8192]))
+    yahkv.append(dev, t_table, torch.tensor([n], dtype=torch.int32, device="cuda"),  # ... and the step's token
+                 bf16_cuda(torch, K[:, n:]), bf16_cuda(torch, V[:, n:]))
+    got_pools = dev.numpy()
+    for name, want in host.arrays().items():
+        assert np.array_equal(got_pools[name], want), f"pool {name}: written bytes or untouched poison differ"
+    scale = 1.0 / 16
+    lens = torch.tensor([n + 1], dtype=torch.int32, device="cuda")
+    out = yahkv.decode_attend(dev, t_table, lens, n + 1, bf16_cuda(torch, q), scale)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    assert np.all(np.isfinite(got))
+    want = closed_from_blocks(yahkv, dev, t_table[0], n + 1, q[0], scale, 8)
+    err = rel_err(got[0], want)
+    assert err < TOL, err
+    assert rel_err(got, oracle.decode_attend(host, table, [n + 1], q, scale)) < TOL
+    # the appended token counts from its own step on, not before
+    prev = yahkv.decode_attend(dev, t_table, lens - 1, n + 1, bf16_cuda(torch, q), scale).cpu().numpy()
+    assert rel_err(prev[0], closed_from_blocks(yahkv, dev, t_table[0], n, q[0], scale, 8)) < TOL
+    assert np.abs(prev - got).max() > 0
+
+
+def outlier_scales(rng):
+    s = np.ones((NKV, HD), np.float32)
+    for h in range(NKV):
+        s[h, rng.permutation(HD)[:8]] = 20.0
+    return s
+
+
+def test_config5_q4_0_outlier_channels_against_the_oracle(yahkv, torch_gpu):
+    """16 sequences of 2048 tokens (+ 1 appended): pools bit-exact, attention within tolerance of the oracle."""
+    torch = torch_gpu
+    rng = np.random.default_rng(55)
+    B, n = 16, 2048
+    pages = [(n + 1 + PT - 1) // PT] * B
+    g = oracle.geometry(4, NQ, NKV, HD, PT, sum(pages))
+    table = make_tables(rng, pages, g.n_pages)
+    outl = outlier_scales(rng)
+    K = to_bf16_f32(rng.standard_normal((B, n + 1, NKV, HD)).astype(np.float32) * outl)
+    V = to_bf16_f32(rng.standard_normal((B, n + 1, NKV, HD)))
+    q = to_bf16_f32(rng.standard_normal((B, NQ, HD)))
+    host = oracle.HostPools(g, fill=0x7F)
+    oracle.append(host, table, [0] * B, None, K, V)
+    dev = yahkv.DevicePools(yahkv.geometry(4, NQ, NKV, HD, PT, g.n_pages), fill=0x7F)
+    t_table = torch.from_numpy(table).cuda()
+    zeros = torch.zeros(B, dtype=torch.int32, device="cuda")
+    yahkv.append(dev, t_table, zeros, bf16_cuda(torch, K[:, :n]), bf16_cuda(torch, V[:, :n]))
+    yahkv.append(dev, t_table, zeros + n, bf16_cuda(torch, K[:, n:]), bf16_cuda(torch, V[:, n:]))
+    got_pools = dev.numpy()
+    for name, want in host.arrays().items():
+        assert np.array_equal(got_pools[name], want), f"pool {name} differs"
+    # the outlier channels did what they are there for: their blocks' scales are large, their block-mates coarse
+    kblocks, _ = oracle.gather_blocks(host, table[0], 64)
+    d = np.abs(kblocks[..., :2].copy().view(np.float16).astype(np.float32))[..., 0]      # [tok][H][NB]
+    hot = np.zeros((NKV, HD // 32), bool)
+    for h in range(NKV):
+        hot[h, np.flatnonzero(outl[h] > 1) // 32] = True
+    assert d[:, hot].mean() > 4 * d[:, ~hot].mean()
+    scale = 1.0 / 16
+    out = yahkv.decode_attend(dev, t_table, zeros + n + 1, n + 1, bf16_cuda(torch, q), scale)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    assert np.all(np.isfinite(got))
+    want = oracle.decode_attend(host, table, [n + 1] * B, q, scale)
+    for s in range(B):
+        assert rel_err(got[s], want[s]) < TOL, s
+
+
+def test_config5_q4_0_batch16_of_131072_tokens(yahkv, torch_gpu):
+    """The full size: 16 x 131072 tokens, the pool sized to fit exactly, one global shuffle of the pages; the K / V
+    source is drawn on the GPU (torch supplies the random numbers) and quantized by the library's own append, which the
+    test above and the append tests hold to the oracle bit for bit. Checked: the closed form over the gathered blocks
+    of two sequences, and the blocks of every sequence's appended token against the oracle's quantizer."""
+    torch = torch_gpu
+    rng = np.random.default_rng(56)
+    B, n = 16, 131072
+    per_seq = (n + 1 + PT - 1) // PT
+    n_pages = B * per_seq
+    g = yahkv.geometry(4, NQ, NKV, HD, PT, n_pages)
+    table = make_tables(rng, [per_seq] * B, n_pages)
+    yahkv.validate_page_table(g, table, np.full(B, n + 1, np.int32))
+    dev = yahkv.DevicePools(g, fill=0x7F)
+    t_table = torch.from_numpy(table).cuda()
+    outl = torch.from_numpy(outlier_scales(rng)).cuda()
+    gen = torch.Generator(device="cuda").manual_seed(56)
+    for s in range(B):
+        for o in range(0, n, 16384):
+            k = (torch.randn((1, 16384, NKV, HD), generator=gen, device="cuda") * outl).to(torch.bfloat16)
+            v = torch.randn((1, 16384, NKV, HD), generator=gen, device="cuda").to(torch.bfloat16)
+            yahkv.append(dev, t_table[s:s + 1], torch.tensor([o], dtype=torch.int32, device="cuda"), k, v)
+    knew = to_bf16_f32(rng.standard_normal((B, 1, NKV, HD)).astype(np.float32) * outl.cpu().numpy())
+    vnew = to_bf16_f32(rng.standard_normal((B, 1, NKV, HD)))
+    lens = torch.full((B,), n, dtype=torch.int32, device="cuda")
+    yahkv.append(dev, t_table, lens, bf16_cuda(torch, knew), bf16_cuda(torch, vnew))
+    q = to_bf16_f32(rng.standard_normal((B, NQ, HD)))
+    scale = 1.0 / 16
+    out = yahkv.decode_attend(dev, t_table, lens + 1, n + 1, bf16_cuda(torch, q), scale)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    assert np.all(np.isfinite(got))
+    for s in range(B):                                        # the step's token, bit for bit
+        k, v = yahkv.gather_blocks(dev, t_table[s], n + 1)
+        assert np.array_equal(k[n].cpu().numpy().reshape(-1, 18), oracle.quantize_q4_0(knew[s, 0])), s
+        assert np.array_equal(v[n].cpu().numpy().reshape(-1, 18), oracle.quantize_q4_0(vnew[s, 0])), s
+        del k, v
+    for s in (0, B - 1):
+        want = closed_from_blocks(yahkv, dev, t_table[s], n + 1, q[s], scale, 4)
+        err = rel_err(got[s], want)
+        assert err < TOL, (s, err)

@@ -151,6 +151,21 @@ def test_q4_0_invariants():
     assert np.array_equal(z[0], np.array([0, 0x80] + [0x88] * 16, np.uint8))  # all-zero block: d = 0 / -8 = -0.0, codes 8
 
 
+def test_q4_0_known_answers():
+    """ggml's quantize_row_q4_0_ref on hand-computed blocks (tests/q4_known_answers.py): halves round up, the clip at
+    code 15, the first of two equal magnitudes decides the scale's sign, for every pair of positions in a block."""
+    from q4_known_answers import known_answers
+    x, want, names = known_answers()
+    got = oracle.quantize_q4_0(x)
+    for i in np.flatnonzero((got != want).any(1)):
+        raise AssertionError(f"block '{names[i]}': got {got[i].tolist()}, want {want[i].tolist()}")
+    # and what those blocks decode to, worked out the same way: (code - 8) * d
+    y = oracle.dequantize_q4_0(want[:1]).reshape(32)
+    assert list(y[:8]) == [-8, 1, 0, 2, -1, 7, 7, 7] and not y[8:].any()
+    y = oracle.dequantize_q4_0(want[2:3]).reshape(32)
+    assert list(y[:8]) == [8, -7, 0, -1, 1, -2, -7, -7]
+
+
 def test_the_kernels_rounding_is_lround_for_every_float_a_code_can_come_from():
     """The append kernels round x * inv as trunc(r + copysign(0.5 - 2^-25, r)) where the reference calls lround
     (gguf_quant.cpp:316); codes come from |r| <= 128 (anything larger becomes 0 on both sides). Every float up to
