@@ -162,6 +162,21 @@ int yahkv_decode_attend(const yahkv_geometry* g, const yahkv_pools* pools, const
                         const void* q, int32_t q_dtype, float softmax_scale, const float* gate, float* out,
                         void* workspace, size_t workspace_bytes, void* stream);
 
+/* yahkv_decode_attend without a workspace argument, for callers that cannot allocate device memory (code under HIP
+ * graph capture, serving loops and harnesses that forbid hipMalloc). It has no counterpart in the reference. The
+ * partials go to an array that is part of the library's code object: yahkv_decode_static_scratch_bytes() = 32 MiB,
+ * held on every GPU the library runs on until the process ends. A batch whose yahkv_decode_workspace_bytes() exceeds
+ * that returns YAHKV_ERR_WORKSPACE and launches nothing (24 / 4 heads of 256 dims: 64 sequences fit, whatever their
+ * lengths). The function calls no allocator; the device of `stream` must be the current device. Every call on a GPU uses
+ * that GPU's one array: calls that overlap on one GPU (two streams, two threads) race; calls on one stream do not.
+ * Results are those of yahkv_decode_attend. The first call on a device looks the array's address up
+ * (hipGetSymbolAddress): make it before a graph capture begins. */
+size_t yahkv_decode_static_scratch_bytes(void);
+int yahkv_decode_attend_static(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
+                               int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs, int32_t max_seq_len,
+                               const void* q, int32_t q_dtype, float softmax_scale, const float* gate, float* out,
+                               void* stream);
+
 /* Chunked-prefill attention: query t of sequence s (t < chunk_len) sees keys 0 .. prefix_len[s] + t, which
  * must already be in the pools (append the chunk first).
  *   q    [n_seqs][chunk_len][n_q_heads][D] bf16

@@ -61,6 +61,8 @@ def _load():
     lib.yahkv_decode_part.argtypes = [G, P, i32p, i32, i32p, i32, i32, vp, i32, C.c_float, vp, C.c_size_t, vp]
     lib.yahkv_decode_reduce.argtypes = [G, i32, i32p, i32, i32, vp, vp, vp, C.c_size_t, vp]
     lib.yahkv_decode_attend.argtypes = [G, P, i32p, i32, i32p, i32, i32, vp, i32, C.c_float, vp, vp, vp, C.c_size_t, vp]
+    lib.yahkv_decode_static_scratch_bytes.restype = C.c_size_t
+    lib.yahkv_decode_attend_static.argtypes = [G, P, i32p, i32, i32p, i32, i32, vp, i32, C.c_float, vp, vp, vp]
     lib.yahkv_prefill_workspace_bytes.restype = C.c_size_t
     lib.yahkv_prefill_workspace_bytes.argtypes = [G, i32, i32, i32]
     lib.yahkv_prefill_attend.argtypes = [G, P, i32p, i32, i32p, i32, i32, i32, vp, C.c_float, vp, vp, i32, vp,
@@ -351,6 +353,16 @@ def decode_attend(pools, table, seq_len, max_seq_len, q, scale, gate=None, out=N
     _check(lib.yahkv_decode_attend(C.byref(g), C.byref(st), _dp(table), table.shape[1], _dp(seq_len), n_seqs,
                                    max_seq_len, _dp(q), _dtype_code(q), scale, _dp(gate), _dp(out), _dp(workspace),
                                    workspace.numel(), _stream()), "decode_attend")
+    return out
+
+
+def decode_attend_static(pools, table, seq_len, max_seq_len, q, scale, out, gate=None):
+    """decode_attend() on the library's own scratch array: no workspace, no allocation (out is the caller's)."""
+    g = pools.geom
+    st = pools.struct()
+    _check(lib.yahkv_decode_attend_static(C.byref(g), C.byref(st), _dp(table), table.shape[1], _dp(seq_len), q.shape[0],
+                                          max_seq_len, _dp(q), _dtype_code(q), scale, _dp(gate), _dp(out), _stream()),
+           "decode_attend_static")
     return out
 
 

@@ -19,6 +19,7 @@
 #include <algorithm>
 #include <cstdio>
 #include <cstdlib>
+#include <mutex>
 
 #include "common.hpp"
 
@@ -940,6 +941,50 @@ extern "C" int yahkv_decode_reduce(const yahkv_geometry* g, int32_t page_table_s
   hipLaunchKernelGGL(DattnReduce, dim3(a.g.n_q, n_seqs, split), dim3(kReduceThreads), 0,
                      static_cast<hipStream_t>(stream), a);
   return LaunchStatus();
+}
+
+// ---- decode attention without a workspace argument ------------------------------------------------------------------------
+//
+// For callers that cannot allocate device memory at all (code under HIP graph capture, serving loops or harnesses that
+// forbid it): the partials live in an array that is part of the library's code object, so it exists on every GPU the
+// library runs on from the moment the code object is loaded there until the process ends. In host code the array's name
+// is only a handle for the lookup below; the address the kernels use is the one the runtime reports per device.
+constexpr size_t kStaticScratchBytes = size_t(32) << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex scratch_mutex;
+void* scratch_of_device[kMaxDevices];  // the array's address on each device, looked up on the first call there
+
+int StaticScratch(void** ptr) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return YAHKV_ERR_LAUNCH;
+  std::lock_guard<std::mutex> lock(scratch_mutex);
+  if (scratch_of_device[dev] == nullptr) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || p == nullptr) return YAHKV_ERR_LAUNCH;
+    scratch_of_device[dev] = p;
+  }
+  *ptr = scratch_of_device[dev];
+  return YAHKV_OK;
+}
+}  // namespace
+
+extern "C" size_t yahkv_decode_static_scratch_bytes(void) { return kStaticScratchBytes; }
+
+extern "C" int yahkv_decode_attend_static(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
+                                          int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs,
+                                          int32_t max_seq_len, const void* q, int32_t q_dtype, float softmax_scale,
+                                          const float* gate, float* out, void* stream) {
+  if (const int st = CheckGeometry(g)) return st;
+  if (n_seqs <= 0 || max_seq_len <= 0) return YAHKV_ERR_ARG;
+  // the partials of this batch must fit the array: nothing is launched otherwise
+  if (MakePlan(MakeGeom(*g), n_seqs, max_seq_len).bytes > kStaticScratchBytes) return YAHKV_ERR_WORKSPACE;
+  void* ws = nullptr;
+  if (const int st = StaticScratch(&ws)) return st;
+  return yahkv_decode_attend(g, pools, page_table, page_table_stride, seq_len, n_seqs, max_seq_len, q, q_dtype,
+                             softmax_scale, gate, out, ws, kStaticScratchBytes, stream);
 }
 
 extern "C" int yahkv_decode_attend(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
