@@ -232,7 +232,7 @@ def run_f16(a, wl, torch, yahkv):
     knew = torch.randn((total, B, 1, NKV, HD), generator=gen, device="cuda").to(torch.bfloat16)
     vnew = torch.randn((total, B, 1, NKV, HD), generator=gen, device="cuda").to(torch.bfloat16)
     out = torch.empty((B, NQ, HD), dtype=torch.float32, device="cuda")
-    ws = torch.empty(yahkv.lib.yahkv_f16_decode_workspace_bytes(g, B, max_len), dtype=torch.uint8, device="cuda")
+    ws = torch.empty(yahkv.lib.yahkv_f16_decode_workspace_bytes(g, B, max_len, None), dtype=torch.uint8, device="cuda")
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(a.steps)]
 
     def step(i, pair=None):

@@ -51,7 +51,7 @@ extern "C" {
 
 typedef enum yahkv_status {
   YAHKV_OK = 0,
-  YAHKV_ERR_ARG = -1,        /* null pointer, non-positive count, misaligned pointer */
+  YAHKV_ERR_ARG = -1,        /* null pointer, non-positive count, misaligned pointer, pool shorter than the geometry needs */
   YAHKV_ERR_SHAPE = -2,      /* geometry this build has no kernel for */
   YAHKV_ERR_PAGE = -3,       /* page table entry outside the pool, or a page used twice */
   YAHKV_ERR_WORKSPACE = -4,  /* workspace smaller than yahkv_*_workspace_bytes */
@@ -72,12 +72,19 @@ typedef struct yahkv_geometry {
   int32_t n_pages;      /* pages in each of the four pools */
 } yahkv_geometry;
 
-/* Device addresses of one layer's pools, each at least yahkv_*_bytes long and 256-byte aligned. */
+/* Device addresses of one layer's pools, 16-byte aligned, and the length of each buffer in bytes, as the reference's
+ * bindings carry theirs (hrx_buffer_ref_t{buffer, offset, length}, engine/model/loom_runtime.hpp:467-478). Every entry
+ * point that takes pools refuses a pool shorter than yahkv_*_bytes(g) with YAHKV_ERR_ARG before it launches anything,
+ * as the reference refuses an undersized binding (engine/run/hal_run.cc:110-114, loom_decoder.hpp:186-203). */
 typedef struct yahkv_pools {
   void* kq;
   void* ks;
   void* vq;
   void* vs;
+  size_t kq_bytes;
+  size_t ks_bytes;
+  size_t vq_bytes;
+  size_t vs_bytes;
 } yahkv_pools;
 
 /* Library version string and the gfx target the kernels were compiled for. */
@@ -133,40 +140,65 @@ int yahkv_append_rope(const yahkv_geometry* g, const yahkv_pools* pools, const i
                       int32_t n_new, const void* k_src, const void* v_src, int32_t src_dtype, const yahkv_rope* rope,
                       const void* q_src, void* q_out, int32_t q_out_dtype, float* k_out, void* stream);
 
+/* Tuning values of the decode attention. A NULL pointer or a zero field means the default; nothing is read from
+ * the environment or from any other process-wide state. The same options must be given to every call that shares a
+ * workspace (its layout depends on them). */
+typedef struct yahkv_decode_options {
+  int32_t n_chunks;         /* pieces the batch's keys are cut into = workgroups of the split-K kernel; 0: one per
+                               compute unit (f16 pools: workgroups aimed at in all; 0: sixteen per compute unit) */
+  int32_t min_chunk_tiles;  /* fewest 64-key tiles a piece gets (each piece costs a partial); 0: 16; at least 2 */
+  int32_t pair_cost;        /* what a change of (sequence, kv head) costs a workgroup, in tiles; 0: 8; negative: none */
+  int32_t reduce_split;     /* workgroups per (query head, sequence) of the merge; 0: chosen from the batch size */
+  int32_t deterministic;    /* not 0: the waves of a workgroup take its tiles in a fixed pattern, so two calls on the
+                               same bytes give the same bits (by default tiles go first come, first served, and
+                               results differ by about 1e-4 relative from run to run) */
+  int32_t xcd_weight[8];    /* relative read speeds of the eight XCDs, as yahkv_decode_calibrate measures them; the
+                               chunks of a group of eight are sized by them; all 0: equal shares */
+} yahkv_decode_options;
+
 /* Decode attention: one query token per sequence against keys 0 .. seq_len[s] - 1.
- *   q    [n_seqs][n_q_heads][D] of q_dtype (F16 or BF16)
+ *   q    [n_seqs][n_q_heads][D] of q_dtype: F32 (what the reference's kernels take, gen_decode_attn.py:576-590), F16
+ *        or BF16. The kernels compute with f16 queries: F32 rounds to nearest even, BF16 converts exactly in the
+ *        normal f16 range, finite values beyond +-65504 saturate there, NaN and infinities give NaN
  *   gate [n_seqs][n_q_heads][D] f32 or NULL; with a gate, out = ctx * sigmoid(gate) (gen_decode_attn.py:402-407)
  *   out  [n_seqs][n_q_heads][D] f32
  * max_seq_len is a host-side upper bound of seq_len[] (it sizes the grid and the workspace); seq_len
  * values above it are clamped. A sequence of length 0 yields zeros.
  * Replaces yah_dattn_part_q + yah_dattn_reduce (gen_decode_attn.py:576-1040, 338-411). */
-size_t yahkv_decode_workspace_bytes(const yahkv_geometry* g, int32_t n_seqs, int32_t max_seq_len);
-/* The dispatches of a decode attention on their own, as LoomDecoder::Step issues its own (loom_decoder.hpp:259-268):
+size_t yahkv_decode_workspace_bytes(const yahkv_geometry* g, int32_t n_seqs, int32_t max_seq_len,
+                                    const yahkv_decode_options* opt);
+/* The two dispatches of a decode attention on their own, as LoomDecoder::Step issues its own (loom_decoder.hpp:259-268):
  * `part` cuts the batch into equal pieces of work from the device-resident lengths (the reference needs no cut: it
  * has one sequence and launches one workgroup per page in use) and leaves partials (M, l, acc) per piece in the
- * workspace, with the prefix sums of the lengths; `reduce` merges the partials into out. `plan` checks the arguments
- * and launches nothing; it is kept for callers written against the three-dispatch form. Part and reduce must be given the same geometry, n_seqs,
- * max_seq_len, page_table_stride and workspace, in this order on one stream; the lengths must not change in between. */
-int yahkv_decode_plan(const yahkv_geometry* g, int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs,
-                      int32_t max_seq_len, void* workspace, size_t workspace_bytes, void* stream);
+ * workspace, with the prefix sums of the lengths; `reduce` merges the partials into out. Both must be given the same
+ * geometry, n_seqs, max_seq_len, page_table_stride, options and workspace, in this order on one stream; the lengths
+ * must not change in between. */
 int yahkv_decode_part(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
                       int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs, int32_t max_seq_len,
                       const void* q, int32_t q_dtype, float softmax_scale, void* workspace, size_t workspace_bytes,
-                      void* stream);
+                      const yahkv_decode_options* opt, void* stream);
 int yahkv_decode_reduce(const yahkv_geometry* g, int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs,
                         int32_t max_seq_len, const float* gate, float* out, const void* workspace,
-                        size_t workspace_bytes, void* stream);
-/* plan, part, reduce. */
+                        size_t workspace_bytes, const yahkv_decode_options* opt, void* stream);
+/* part, then reduce. */
 int yahkv_decode_attend(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
                         int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs, int32_t max_seq_len,
                         const void* q, int32_t q_dtype, float softmax_scale, const float* gate, float* out,
-                        void* workspace, size_t workspace_bytes, void* stream);
+                        void* workspace, size_t workspace_bytes, const yahkv_decode_options* opt, void* stream);
+/* Measures the relative read speeds of the GPU's eight XCDs on the caller's own batch and writes them to
+ * opt->xcd_weight (the other fields are read): `rounds` times, the split-K kernel runs twice on the given arguments and
+ * the shares are corrected by when each XCD's workgroups finished. A set-up call: it synchronizes the stream and
+ * overwrites the workspace. No counterpart in the reference (one sequence, one workgroup per page). */
+int yahkv_decode_calibrate(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
+                           int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs, int32_t max_seq_len,
+                           const void* q, int32_t q_dtype, void* workspace, size_t workspace_bytes,
+                           yahkv_decode_options* opt, int32_t rounds, void* stream);
 
 /* yahkv_decode_attend without a workspace argument, for callers that cannot allocate device memory (code under HIP
  * graph capture, serving loops and harnesses that forbid hipMalloc). It has no counterpart in the reference. The
  * partials go to an array that is part of the library's code object: yahkv_decode_static_scratch_bytes() = 32 MiB,
  * held on every GPU the library runs on until the process ends. A batch whose yahkv_decode_workspace_bytes() exceeds
- * that returns YAHKV_ERR_WORKSPACE and launches nothing (24 / 4 heads of 256 dims: 64 sequences fit, whatever their
+ * (default options) returns YAHKV_ERR_WORKSPACE and launches nothing (24 / 4 heads of 256 dims: 64 sequences fit, whatever their
  * lengths). The function calls no allocator; the device of `stream` must be the current device. Every call on a GPU uses
  * that GPU's one array: calls that overlap on one GPU (two streams, two threads) race; calls on one stream do not.
  * Results are those of yahkv_decode_attend. The first call on a device looks the array's address up
@@ -273,6 +305,8 @@ int yahkv_slot_unpack(const yahkv_geometry* g, const yahkv_pools* pools, const i
 typedef struct yahkv_f16_pools {
   void* k;
   void* v;
+  size_t k_bytes; /* lengths of the two buffers; shorter than yahkv_f16_pool_bytes(g): YAHKV_ERR_ARG */
+  size_t v_bytes;
 } yahkv_f16_pools;
 size_t yahkv_f16_pool_bytes(const yahkv_geometry* g);
 /* K and V rows of n_new tokens per sequence (layout and arguments as yahkv_append), rounded to f16 (nearest even,
@@ -281,12 +315,14 @@ int yahkv_f16_append(const yahkv_geometry* g, const yahkv_f16_pools* pools, cons
                      int32_t page_table_stride, const int32_t* start_pos, const int32_t* n_valid, int32_t n_seqs,
                      int32_t n_new, const void* k_src, const void* v_src, int32_t src_dtype, void* stream);
 /* Decode attention over keys 0 .. seq_len[s] - 1 (arguments as yahkv_decode_attend): two dispatches, partials of
- * fixed stretches of every sequence, then their merge with the optional sigmoid gate. */
-size_t yahkv_f16_decode_workspace_bytes(const yahkv_geometry* g, int32_t n_seqs, int32_t max_seq_len);
+ * fixed stretches of every sequence, then their merge with the optional sigmoid gate. Of the options only n_chunks is
+ * used. */
+size_t yahkv_f16_decode_workspace_bytes(const yahkv_geometry* g, int32_t n_seqs, int32_t max_seq_len,
+                                        const yahkv_decode_options* opt);
 int yahkv_f16_decode_attend(const yahkv_geometry* g, const yahkv_f16_pools* pools, const int32_t* page_table,
                             int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs, int32_t max_seq_len,
                             const void* q, int32_t q_dtype, float softmax_scale, const float* gate, float* out,
-                            void* workspace, size_t workspace_bytes, void* stream);
+                            void* workspace, size_t workspace_bytes, const yahkv_decode_options* opt, void* stream);
 /* Chunked-prefill attention over f16 pools after the chunk has been appended with yahkv_f16_append (arguments as
  * yahkv_prefill_attend; the workspace is required): the keys' bf16 tiles are converted from the pools (the reference's
  * attention reads its 16-bit K / V pool directly, gen_attn_fa.py:1589-1595), then the same attention kernel runs. */

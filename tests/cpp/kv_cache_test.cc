@@ -105,32 +105,44 @@ int RunTest() {
     const double e1 = RelErr(got, want);
     Expect(e1 < 2e-3, "prefill attention differs from the oracle");
 
-    // ---- decode steps
+    // ---- decode steps: all of them queued back to back, no host wait in between (the positions of a step travel
+    // through staging memory that the next step must not overwrite before its copy has run), then every step's output
+    // against the oracle
     Stage("decode steps");
     double e2 = 0;
-    for (int i = 0; i < steps; ++i) {
-      std::vector<uint16_t> k1, v1, q1;
-      std::vector<float> k1f, v1f, q1f;
-      randn_bf16(size_t(B) * H * D, &k1, &k1f);
-      randn_bf16(size_t(B) * H * D, &v1, &v1f);
-      randn_bf16(size_t(B) * NQ * D, &q1, &q1f);
-      CheckHip(hipMemcpy(dk.get(), k1.data(), k1.size() * 2, hipMemcpyHostToDevice), "h2d");
-      CheckHip(hipMemcpy(dv.get(), v1.data(), v1.size() * 2, hipMemcpyHostToDevice), "h2d");
-      CheckHip(hipMemcpy(dq.get(), q1.data(), q1.size() * 2, hipMemcpyHostToDevice), "h2d");
-      std::vector<int32_t> pos(B), len(B);
-      for (int s = 0; s < B; ++s) pos[s] = dec.length(s), len[s] = pos[s] + 1;
-      dec.Step(B, dk.get(), dv.get(), YAHKV_BF16, dq.get(), YAHKV_BF16, scale, nullptr, static_cast<float*>(dout.get()));
+    {
+      const size_t kv_n = size_t(B) * H * D, q_n = size_t(B) * NQ * D;
+      std::vector<std::vector<float>> k1f(steps), v1f(steps), q1f(steps);
+      DeviceBuffer sk(kv_n * 2 * steps), sv(kv_n * 2 * steps), sq(q_n * 2 * steps), sout(q_n * 4 * steps);
+      for (int i = 0; i < steps; ++i) {
+        std::vector<uint16_t> k1, v1, q1;
+        randn_bf16(kv_n, &k1, &k1f[i]);
+        randn_bf16(kv_n, &v1, &v1f[i]);
+        randn_bf16(q_n, &q1, &q1f[i]);
+        CheckHip(hipMemcpy(static_cast<char*>(sk.get()) + kv_n * 2 * i, k1.data(), kv_n * 2, hipMemcpyHostToDevice), "h2d");
+        CheckHip(hipMemcpy(static_cast<char*>(sv.get()) + kv_n * 2 * i, v1.data(), kv_n * 2, hipMemcpyHostToDevice), "h2d");
+        CheckHip(hipMemcpy(static_cast<char*>(sq.get()) + q_n * 2 * i, q1.data(), q_n * 2, hipMemcpyHostToDevice), "h2d");
+      }
+      std::vector<std::vector<int32_t>> pos(steps, std::vector<int32_t>(B)), len(steps, std::vector<int32_t>(B));
+      for (int i = 0; i < steps; ++i) {
+        for (int s = 0; s < B; ++s) pos[i][s] = dec.length(s), len[i][s] = pos[i][s] + 1;
+        dec.Step(B, static_cast<char*>(sk.get()) + kv_n * 2 * i, static_cast<char*>(sv.get()) + kv_n * 2 * i, YAHKV_BF16,
+                 static_cast<char*>(sq.get()) + q_n * 2 * i, YAHKV_BF16, scale, nullptr,
+                 reinterpret_cast<float*>(static_cast<char*>(sout.get()) + q_n * 4 * i));
+      }
       CheckHip(hipDeviceSynchronize(), "sync");
       refresh_table();
-      orc_append(&og, &op, table.data(), stride, pos.data(), nullptr, B, 1, k1f.data(), v1f.data());
-      std::vector<float> w(q1f.size()), o(q1f.size());
-      orc_decode_attend(&og, &op, table.data(), stride, len.data(), B, q1f.data(), scale, nullptr, w.data());
-      CheckHip(hipMemcpy(o.data(), dout.get(), o.size() * 4, hipMemcpyDeviceToHost), "d2h");
-      e2 = std::max(e2, RelErr(o, w));
+      for (int i = 0; i < steps; ++i) {
+        orc_append(&og, &op, table.data(), stride, pos[i].data(), nullptr, B, 1, k1f[i].data(), v1f[i].data());
+        std::vector<float> w(q_n), o(q_n);
+        orc_decode_attend(&og, &op, table.data(), stride, len[i].data(), B, q1f[i].data(), scale, nullptr, w.data());
+        CheckHip(hipMemcpy(o.data(), static_cast<char*>(sout.get()) + q_n * 4 * i, q_n * 4, hipMemcpyDeviceToHost), "d2h");
+        e2 = std::max(e2, RelErr(o, w));
+      }
     }
     Expect(e2 < 2e-3, "decode attention differs from the oracle");
     // pool contents bit-exact: every sequence's blocks, gathered through the page table, against the oracle's
-    const yahkv_pools dp{st.kq.ptr, st.ks.ptr, st.vq.ptr, st.vs.ptr};
+    const yahkv_pools dp = yahkv_host::PoolsOf(st);
     for (int s = 0; s < B; ++s) {
       const size_t bytes = size_t(dec.length(s)) * H * (D / 32) * 34;
       std::vector<uint8_t> gk(bytes), gv(bytes), wk(bytes), wv(bytes);
@@ -165,7 +177,7 @@ int RunTest() {
         const size_t bytes = size_t(d.length(seq)) * H * (D / 32) * 34;
         std::vector<uint8_t> k(bytes), v(bytes);
         DeviceBuffer bk(bytes), bv(bytes);
-        const yahkv_pools pp{d.state().kq.ptr, d.state().ks.ptr, d.state().vq.ptr, d.state().vs.ptr};
+        const yahkv_pools pp = yahkv_host::PoolsOf(d.state());
         d.Upload();
         Check(yahkv_gather_blocks(&g, &pp, static_cast<const int32_t*>(d.state().ptab.ptr) + size_t(seq) * d.page_table_stride(),
                                   d.length(seq), bk.get(), bv.get(), nullptr), "gather");

@@ -1,0 +1,82 @@
+"""The decode attention's boundary behaviour through the C ABI: the deterministic mode gives the same bits on every
+call, queries beyond the f16 range saturate instead of poisoning the row, f32 queries are taken as the reference's
+kernels take them, and the XCD calibration returns shares that leave the results unchanged."""
+import numpy as np
+import pytest
+
+import oracle
+from helpers import rel_err, to_bf16_f32
+from test_gpu_decode import closed, gpu_attend, setup
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-3
+
+
+@pytest.mark.parametrize("fmt", [8, 4])
+def test_deterministic_mode_repeats_bit_for_bit(yahkv, torch_gpu, fmt):
+    """With opt.deterministic the waves take a workgroup's tiles in a fixed pattern: the same bytes in give the same
+    bits out, call after call, which makes a hash of the output a regression check as the reference's attn_bench uses
+    its FNV hash (engine/run/attn_bench.cc:174-176). Long sequences, so that every wave has several tiles."""
+    torch = torch_gpu
+    lens = [40000, 9000, 64, 20001, 1, 0, 5000, 12345]
+    g, table, host, dev, rng = setup(yahkv, torch, fmt, 24, 4, 256, 64, lens, seed=fmt + 31)
+    q = to_bf16_f32(rng.standard_normal((len(lens), 24, 256)))
+    opt = yahkv.decode_options(deterministic=True)
+    runs = [gpu_attend(yahkv, torch, dev, table, lens, q, 0.0625, opt=opt) for _ in range(4)]
+    for r in runs[1:]:
+        assert np.array_equal(r.view(np.uint32), runs[0].view(np.uint32))
+    assert rel_err(runs[0], oracle.decode_attend(host, table, lens, q, 0.0625)) < TOL
+    # the default mode agrees within the tolerance, not necessarily in every bit
+    free = gpu_attend(yahkv, torch, dev, table, lens, q, 0.0625)
+    assert rel_err(free, runs[0]) < 5e-4
+
+
+@pytest.mark.parametrize("kind", ["bf16", "f32"])
+def test_queries_beyond_the_f16_range_saturate(yahkv, torch_gpu, kind):
+    """The kernels compute with f16 queries. A bf16 or f32 query element of 1e6 is taken as 65504 (not as infinity,
+    which would turn its whole row into NaN); the result is the closed form of the saturated query."""
+    torch = torch_gpu
+    lens = [300, 70]
+    g, table, host, dev, rng = setup(yahkv, torch, 8, 8, 2, 128, 16, lens, seed=77)
+    q = to_bf16_f32(rng.standard_normal((2, 8, 128)))
+    q[0, 3, 5], q[1, 0, 100] = 1e6, -3e38
+    q = to_bf16_f32(q)
+    got = gpu_attend(yahkv, torch, dev, table, lens, q, 1e-6, kind=kind)
+    assert np.all(np.isfinite(got))
+    sat = np.clip(q, -65504, 65504)
+    assert rel_err(got, closed(g, table, host, lens, sat, 1e-6)) < TOL
+
+
+def test_f32_queries_round_to_f16(yahkv, torch_gpu):
+    """f32 queries (the reference's kernels take f32, gen_decode_attn.py:576-590) are rounded to f16, nearest even:
+    the result is the closed form of the rounded query to well within the tolerance, and within it of the unrounded."""
+    torch = torch_gpu
+    lens = [513, 64]
+    g, table, host, dev, rng = setup(yahkv, torch, 8, 24, 4, 256, 64, lens, seed=78)
+    q = rng.standard_normal((2, 24, 256)).astype(np.float32)
+    got = gpu_attend(yahkv, torch, dev, table, lens, q, 0.0625, kind="f32")
+    q16 = q.astype(np.float16).astype(np.float32)
+    assert rel_err(got, closed(g, table, host, lens, q16, 0.0625)) < 5e-4
+    assert rel_err(got, closed(g, table, host, lens, q, 0.0625)) < TOL
+
+
+def test_xcd_calibration_returns_usable_shares(yahkv, torch_gpu):
+    torch = torch_gpu
+    rng0 = np.random.default_rng(5)
+    lens = [int(x) for x in rng0.integers(2000, 30000, 48)]
+    g, table, host, dev, rng = setup(yahkv, torch, 8, 24, 4, 256, 64, lens, seed=79)
+    q = to_bf16_f32(rng.standard_normal((len(lens), 24, 256)))
+    tq = torch.from_numpy(q).cuda().to(torch.bfloat16)
+    t_table = torch.from_numpy(table).cuda()
+    t_lens = torch.tensor(lens, dtype=torch.int32, device="cuda")
+    opt = yahkv.decode_options()
+    ws = torch.empty(yahkv.decode_workspace_bytes(g_dev(yahkv, g), len(lens), max(lens), opt), dtype=torch.uint8, device="cuda")
+    w = yahkv.decode_calibrate(dev, t_table, t_lens, max(lens), tq, ws, opt, rounds=2)
+    assert len(w) == 8 and max(w) == 10000 and min(w) >= 5000, w        # XCDs of one GPU lie within a few percent
+    out = yahkv.decode_attend(dev, t_table, t_lens, max(lens), tq, 0.0625, workspace=ws, opt=opt)
+    torch.cuda.synchronize()
+    assert rel_err(out.cpu().numpy(), oracle.decode_attend(host, table, lens, q, 0.0625)) < TOL
+
+
+def g_dev(yahkv, g):
+    return yahkv.geometry(g.format, g.n_q_heads, g.n_kv_heads, g.head_dim, g.page_tokens, g.n_pages)

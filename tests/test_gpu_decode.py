@@ -26,7 +26,7 @@ def setup(yahkv, torch, fmt, n_q, n_kv, hd, pt, lens, seed, extra_pages=2, fill=
     return g, table, host, dev, rng
 
 
-def gpu_attend(yahkv, torch, dev, table, lens, q, scale, gate=None, kind="bf16", max_len=None):
+def gpu_attend(yahkv, torch, dev, table, lens, q, scale, gate=None, kind="bf16", max_len=None, opt=None):
     if kind == "bf16":
         tq = torch.from_numpy(bf16_bits(q).view(np.int16)).cuda().view(torch.bfloat16)
     elif kind == "f16":
@@ -35,7 +35,7 @@ def gpu_attend(yahkv, torch, dev, table, lens, q, scale, gate=None, kind="bf16",
         tq = torch.from_numpy(q.astype(np.float32)).cuda()
     tg = None if gate is None else torch.from_numpy(gate.astype(np.float32)).cuda()
     out = yahkv.decode_attend(dev, torch.from_numpy(table).cuda(), torch.tensor(lens, dtype=torch.int32, device="cuda"),
-                              max_len or max(max(lens), 1), tq, scale, gate=tg)
+                              max_len or max(max(lens), 1), tq, scale, gate=tg, opt=opt)
     torch.cuda.synchronize()
     return out.cpu().numpy()
 
@@ -151,6 +151,8 @@ def test_workspace_and_argument_checks(yahkv, torch_gpu):
     dev = yahkv.DevicePools(g)
     need = yahkv.decode_workspace_bytes(g, 2, 300)
     assert need > 0
+    # the workspace's size follows the options: both calls must be given the same ones
+    assert yahkv.decode_workspace_bytes(g, 2, 300, yahkv.decode_options(n_chunks=8, min_chunk_tiles=2)) != need
     table = torch.zeros((2, 5), dtype=torch.int32, device="cuda")
     lens = torch.tensor([5, 6], dtype=torch.int32, device="cuda")
     q = torch.zeros((2, 24, 256), dtype=torch.bfloat16, device="cuda")
@@ -158,5 +160,6 @@ def test_workspace_and_argument_checks(yahkv, torch_gpu):
         yahkv.decode_attend(dev, table, lens, 300, q, 0.0625, workspace=torch.empty(need - 16, dtype=torch.uint8, device="cuda"))
     assert e.value.status == -4
     st = dev.struct()
-    rc = yahkv.lib.yahkv_decode_attend(C.byref(g), C.byref(st), None, 5, None, 2, 300, None, 2, 0.0625, None, None, None, 0, None)
+    rc = yahkv.lib.yahkv_decode_attend(C.byref(g), C.byref(st), None, 5, None, 2, 300, None, 2, 0.0625, None, None, None, 0,
+                                       None, None)
     assert rc == -1

@@ -1,8 +1,6 @@
 """Randomized sweep of the paged decode attention against the CPU oracle: formats, group sizes, head dims, page sizes,
 batch sizes, ragged lengths with empty sequences, query dtypes, a gate now and then, and the planner's chunk count
 forced to values that are not a multiple of eight, smaller than the work and larger than it. Tolerance 2e-3."""
-import os
-
 import numpy as np
 import pytest
 
@@ -15,7 +13,7 @@ TOL = 2e-3
 
 
 @pytest.mark.parametrize("seed", range(20))
-def test_random_decode_case(yahkv, torch_gpu, seed, monkeypatch):
+def test_random_decode_case(yahkv, torch_gpu, seed):
     rng = np.random.default_rng(1000 + seed)
     fmt = int(rng.choice([8, 4]))
     n_kv = int(rng.choice([1, 2, 4]))
@@ -30,10 +28,14 @@ def test_random_decode_case(yahkv, torch_gpu, seed, monkeypatch):
     if max(lens) == 0:
         lens[0] = 1
     chunks = int(rng.choice([0, 1, 3, 7, 13, 64, 100, 256, 1000]))
-    if chunks:
-        monkeypatch.setenv("YAHKV_DECODE_CHUNKS", str(chunks))
+    opt = yahkv.decode_options(n_chunks=chunks)
     if rng.random() < 0.3:
-        monkeypatch.setenv("YAHKV_DECODE_MIN_CHUNK_TILES", str(int(rng.choice([1, 2, 5]))))
+        opt.min_chunk_tiles = int(rng.choice([1, 2, 5]))
+    if rng.random() < 0.3:
+        opt.deterministic = 1
+    if rng.random() < 0.3:
+        for j in range(8):
+            opt.xcd_weight[j] = int(rng.choice([0, 1, 900, 1000, 1100, 100000]))
     g, table, host, dev, _ = setup(yahkv, torch_gpu, fmt, n_kv * group, n_kv, hd, pt, lens, seed=seed, fill=0x7F)
     q = to_bf16_f32(rng.standard_normal((n_seqs, n_kv * group, hd)))
     gate = rng.standard_normal(q.shape).astype(np.float32) if rng.random() < 0.3 else None
@@ -43,7 +45,7 @@ def test_random_decode_case(yahkv, torch_gpu, seed, monkeypatch):
     scale = float(1 / np.sqrt(hd))
     slack = int(rng.integers(0, 100))                          # the host's bound may be loose
     got = gpu_attend(yahkv, torch_gpu, dev, table, lens, q, scale, gate=gate, kind=kind,
-                     max_len=min(max(lens) + slack, table.shape[1] * pt))
+                     max_len=min(max(lens) + slack, table.shape[1] * pt), opt=opt)
     want = oracle.decode_attend(host, table, lens, q, scale, gate)
     assert np.all(np.isfinite(got)), (fmt, n_kv, group, hd, pt, lens, chunks)
     for s, n in enumerate(lens):
@@ -69,19 +71,17 @@ def test_large_batch_of_short_sequences(yahkv, torch_gpu):
         assert not got[s].any()
 
 
-def test_chunks_of_one_or_two_units(yahkv, torch_gpu, monkeypatch):
+def test_chunks_of_one_or_two_units(yahkv, torch_gpu):
     """The finest cut the planner allows (asked for one tile per chunk; it keeps two line units): the eight chunks of
     a group then differ by whole units, and none inside a pair's stretch may come out empty, because the reduce reads
     the partials of every chunk between a pair's first and last."""
-    monkeypatch.setenv("YAHKV_DECODE_CHUNKS", "1000")
-    monkeypatch.setenv("YAHKV_DECODE_MIN_CHUNK_TILES", "1")
     rng = np.random.default_rng(239)
     lens = [91, 627, 798, 425, 27, 408, 417, 18, 247, 137, 144, 127, 70, 839, 137, 273]
-    for fmt, pair_cost in ((4, "8"), (8, "0"), (8, "3")):
-        monkeypatch.setenv("YAHKV_DECODE_PAIR_COST", pair_cost)
+    for fmt, pair_cost, weights in ((4, 8, None), (8, -1, None), (8, 3, None), (8, 8, [1, 100000, 1, 1, 50000, 1, 1, 1])):
+        opt = yahkv.decode_options(n_chunks=1000, min_chunk_tiles=1, pair_cost=pair_cost, xcd_weight=weights)
         g, table, host, dev, _ = setup(yahkv, torch_gpu, fmt, 8, 2, 256, 64, lens, seed=239, fill=0x7F)
         q = to_bf16_f32(rng.standard_normal((len(lens), 8, 256)))
-        got = gpu_attend(yahkv, torch_gpu, dev, table, lens, q, 0.0625, max_len=896)
+        got = gpu_attend(yahkv, torch_gpu, dev, table, lens, q, 0.0625, max_len=896, opt=opt)
         assert np.all(np.isfinite(got))
         assert rel_err(got, oracle.decode_attend(host, table, lens, q, 0.0625)) < TOL
 

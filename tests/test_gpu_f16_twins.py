@@ -140,7 +140,7 @@ def test_decode_against_the_closed_form(yahkv, torch_gpu, n_q, n_kv, hd, pt, len
 
 
 @pytest.mark.parametrize("seed", range(12))
-def test_decode_on_random_shapes_and_cuts(yahkv, torch_gpu, seed, monkeypatch):
+def test_decode_on_random_shapes_and_cuts(yahkv, torch_gpu, seed):
     """Random group sizes, head dims, page sizes, ragged and empty sequences, and the number of stretches a sequence
     is cut into forced from one per sequence to one per 128 keys: every cut gives the closed form."""
     rng = np.random.default_rng(1000 + seed)
@@ -149,13 +149,12 @@ def test_decode_on_random_shapes_and_cuts(yahkv, torch_gpu, seed, monkeypatch):
     lens = [int(x) for x in rng.integers(0, 3000, int(rng.integers(1, 6)))]
     if max(lens) == 0:
         lens[0] = 1
-    wgs = [None, "1", "64", "1000000"][seed % 4]
-    if wgs is not None:
-        monkeypatch.setenv("YAHKV_F16_WORKGROUPS", wgs)
-    check_decode(yahkv, torch_gpu, n_kv * group, n_kv, hd, pt, lens, ["bf16", "f32", "f16"][seed % 3], seed)
+    wgs = [0, 1, 64, 1000000][seed % 4]
+    check_decode(yahkv, torch_gpu, n_kv * group, n_kv, hd, pt, lens, ["bf16", "f32", "f16"][seed % 3], seed,
+                 opt=yahkv.decode_options(n_chunks=wgs) if wgs else None)
 
 
-def check_decode(yahkv, torch, n_q, n_kv, hd, pt, lens, qkind, seed):
+def check_decode(yahkv, torch, n_q, n_kv, hd, pt, lens, qkind, seed, opt=None):
     rng = np.random.default_rng(seed)
     B, max_len = len(lens), max(lens)
     pages = [(l + pt - 1) // pt for l in lens]
@@ -184,7 +183,7 @@ def check_decode(yahkv, torch, n_q, n_kv, hd, pt, lens, qkind, seed):
     gate = rng.standard_normal((B, n_q, hd)).astype(np.float32) if qkind == "f32" else None
     scale = 1.0 / np.sqrt(hd)
     out = yahkv.f16_decode_attend(dev, t_table, torch.tensor(lens, dtype=torch.int32, device="cuda"), max_len,
-                                  tensor(torch, q, qkind), scale,
+                                  tensor(torch, q, qkind), scale, opt=opt,
                                   gate=None if gate is None else torch.from_numpy(gate).cuda()).cpu().numpy()
     assert np.all(np.isfinite(out))
     for s, l in enumerate(lens):
@@ -214,14 +213,14 @@ def test_length_beyond_the_bound_is_clamped_and_arguments_are_checked(yahkv, tor
     assert torch.equal(a, b)
     g8 = yahkv.geometry(8, 8, 2, 128, 16, 8)  # a quantized geometry is not an f16 one
     assert yahkv.lib.yahkv_f16_pool_bytes(C.byref(g8)) == 0
-    assert yahkv.lib.yahkv_f16_decode_workspace_bytes(C.byref(g8), 1, 100) == 0
+    assert yahkv.lib.yahkv_f16_decode_workspace_bytes(C.byref(g8), 1, 100, None) == 0
     st = dev.struct()
     rc = yahkv.lib.yahkv_f16_decode_attend(C.byref(g), C.byref(st), table.data_ptr(), 8, None, 1, 100, q.data_ptr(), 0,
-                                           0.1, None, a.data_ptr(), None, 0, None)
+                                           0.1, None, a.data_ptr(), None, 0, None, None)
     assert rc == -1
     small = torch.empty(16, dtype=torch.uint8, device="cuda")
     rc = yahkv.lib.yahkv_f16_decode_attend(C.byref(g), C.byref(st), table.data_ptr(), 8, table.data_ptr(), 1, 100,
-                                           q.data_ptr(), 0, 0.1, None, a.data_ptr(), small.data_ptr(), 16, None)
+                                           q.data_ptr(), 0, 0.1, None, a.data_ptr(), small.data_ptr(), 16, None, None)
     assert rc == -4
 
 

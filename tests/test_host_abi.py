@@ -127,3 +127,75 @@ def test_page_owner_counts(yahkv):
     assert pool.alloc(8) == list(range(8))               # lowest id first again
     assert yahkv.lib.yahkv_slot_bytes(__import__("ctypes").byref(yahkv.geometry(8, 24, 4, 256, 64, 4)), 3) == \
         64 + 3 * sum(yahkv.pool_bytes(yahkv.geometry(8, 24, 4, 256, 64, 1)).values())
+
+
+def test_undersized_pools_are_refused_before_any_launch(yahkv):
+    """Every entry point that takes pools refuses a buffer shorter than the geometry needs (the reference refuses an
+    undersized binding: engine/run/hal_run.cc:110-114, loom_decoder.hpp:186-203). The refusal comes before anything
+    is launched, so the addresses here need not exist (and no GPU is needed)."""
+    lib = yahkv.lib
+    g = yahkv.geometry(yahkv.Q8_0, 24, 4, 256, 64, 8)
+    need = yahkv.pool_bytes(g)
+    fake = 0x10000                                        # a 16-byte aligned address nothing dereferences
+    ok = dict(kq=need["kq"], ks=need["ks"], vq=need["vq"], vs=need["vs"])
+    for short in ("kq", "ks", "vq", "vs"):
+        n = dict(ok)
+        n[short] -= 1
+        p = yahkv.Pools(fake, fake, fake, fake, n["kq"], n["ks"], n["vq"], n["vs"])
+        r, pr = C.byref(g), C.byref(p)
+        ws = 1 << 30
+        assert lib.yahkv_append(r, pr, fake, 4, fake, None, 1, 1, fake, fake, 0, None) == -1, short
+        rope = yahkv.Rope(1e6, 1e-6, 64, None, None)
+        assert lib.yahkv_append_rope(r, pr, fake, 4, fake, None, 1, 1, fake, fake, 0, C.byref(rope), None, None, 0, None,
+                                     None) == -1
+        assert lib.yahkv_decode_part(r, pr, fake, 4, fake, 1, 100, fake, 2, 0.1, fake, ws, None, None) == -1
+        assert lib.yahkv_decode_attend(r, pr, fake, 4, fake, 1, 100, fake, 2, 0.1, None, fake, fake, ws, None, None) == -1
+        assert lib.yahkv_decode_attend_static(r, pr, fake, 4, fake, 1, 100, fake, 2, 0.1, None, fake, None) == -1
+        assert lib.yahkv_prefill_attend(r, pr, fake, 4, fake, 1, 64, 64, fake, 0.1, None, fake, 0, fake, ws, None) == -1
+        assert lib.yahkv_prefill_decode_tiles(r, pr, fake, 4, fake, 1, 64, 64, fake, ws, None) == -1
+        assert lib.yahkv_gather_blocks(r, pr, fake, 10, fake, fake, None) == -1
+        assert lib.yahkv_copy_pages(r, pr, fake, fake, 1, None) == -1
+        assert lib.yahkv_slot_pack(r, pr, fake, 1, 10, fake, None) == -1
+        assert lib.yahkv_slot_unpack(r, pr, fake, 1, fake, None) == -1
+    # a misaligned or missing pool is refused the same way
+    for kq in (fake + 8, 0):
+        p = yahkv.Pools(kq, fake, fake, fake, ok["kq"], ok["ks"], ok["vq"], ok["vs"])
+        assert lib.yahkv_append(C.byref(g), C.byref(p), fake, 4, fake, None, 1, 1, fake, fake, 0, None) == -1
+    # the f16 twins
+    g16 = yahkv.f16_geometry(24, 4, 256, 64, 8)
+    n16 = lib.yahkv_f16_pool_bytes(C.byref(g16))
+    for kb, vb in ((n16 - 1, n16), (n16, n16 - 1)):
+        p = yahkv.F16PoolsStruct(fake, fake, kb, vb)
+        assert lib.yahkv_f16_append(C.byref(g16), C.byref(p), fake, 4, fake, None, 1, 1, fake, fake, 0, None) == -1
+        assert lib.yahkv_f16_decode_attend(C.byref(g16), C.byref(p), fake, 4, fake, 1, 100, fake, 2, 0.1, None, fake, fake,
+                                           1 << 30, None, None) == -1
+        assert lib.yahkv_f16_prefill_attend(C.byref(g16), C.byref(p), fake, 4, fake, 1, 64, 64, fake, 0.1, None, fake, 0,
+                                            fake, 1 << 30, None) == -1
+
+
+def test_slot_header_must_name_exactly_the_pages_its_tokens_fill(yahkv):
+    """A loader scatters as many pages as the header names: a header with more pages than ceil(tokens / page_tokens),
+    or with no tokens, is refused (the reference's LoadState checks its sizes exactly, loom_prefill.hpp:976-1024)."""
+    g = yahkv.geometry(yahkv.Q8_0, 8, 2, 128, 16, 16)
+
+    def header(pages, tokens):
+        n = yahkv.lib.yahkv_slot_bytes(C.byref(g), pages)
+        buf = np.zeros(n, np.uint8)
+        buf[:64].view(np.uint64)[:] = [int.from_bytes(b"YKVSLOT1", "little"), 8, 2, 128, 16, pages, tokens, 4]
+        return buf
+
+    assert yahkv.slot_check(g, header(3, 33)) == (3, 33)
+    assert yahkv.slot_check(g, header(3, 48)) == (3, 48)
+    for pages, tokens in ((3, 32), (3, 0), (2, 33), (5, 17)):
+        with pytest.raises(yahkv.YahkvError) as e:
+            yahkv.slot_check(g, header(pages, tokens))
+        assert e.value.status == -1, (pages, tokens)
+
+
+def test_decode_options_change_only_what_they_name(yahkv):
+    g = yahkv.geometry(yahkv.Q8_0, 24, 4, 256, 64, 1024)
+    base = yahkv.decode_workspace_bytes(g, 64, 65536)
+    assert yahkv.decode_workspace_bytes(g, 64, 65536, yahkv.decode_options()) == base          # zero fields: defaults
+    assert yahkv.decode_workspace_bytes(g, 64, 65536, yahkv.decode_options(deterministic=True, pair_cost=-1,
+                                                                           xcd_weight=[3, 1, 4, 1, 5, 9, 2, 6])) == base
+    assert yahkv.decode_workspace_bytes(g, 64, 65536, yahkv.decode_options(n_chunks=512)) > base

@@ -24,11 +24,18 @@ class Geometry(C.Structure):
 
 
 class Pools(C.Structure):
-    _fields_ = [("kq", C.c_void_p), ("ks", C.c_void_p), ("vq", C.c_void_p), ("vs", C.c_void_p)]
+    _fields_ = [("kq", C.c_void_p), ("ks", C.c_void_p), ("vq", C.c_void_p), ("vs", C.c_void_p),
+                ("kq_bytes", C.c_size_t), ("ks_bytes", C.c_size_t), ("vq_bytes", C.c_size_t), ("vs_bytes", C.c_size_t)]
 
 
 class F16PoolsStruct(C.Structure):
-    _fields_ = [("k", C.c_void_p), ("v", C.c_void_p)]
+    _fields_ = [("k", C.c_void_p), ("v", C.c_void_p), ("k_bytes", C.c_size_t), ("v_bytes", C.c_size_t)]
+
+
+class DecodeOptions(C.Structure):
+    """yahkv_decode_options: zero fields are the defaults."""
+    _fields_ = [("n_chunks", C.c_int32), ("min_chunk_tiles", C.c_int32), ("pair_cost", C.c_int32),
+                ("reduce_split", C.c_int32), ("deterministic", C.c_int32), ("xcd_weight", C.c_int32 * 8)]
 
 
 class Rope(C.Structure):
@@ -56,11 +63,13 @@ def _load():
     lib.yahkv_append_rope.argtypes = [G, P, i32p, i32, i32p, i32p, i32, i32, vp, vp, i32, C.POINTER(Rope), vp, vp, i32,
                                       vp, vp]
     lib.yahkv_decode_workspace_bytes.restype = C.c_size_t
-    lib.yahkv_decode_workspace_bytes.argtypes = [G, i32, i32]
-    lib.yahkv_decode_plan.argtypes = [G, i32, i32p, i32, i32, vp, C.c_size_t, vp]
-    lib.yahkv_decode_part.argtypes = [G, P, i32p, i32, i32p, i32, i32, vp, i32, C.c_float, vp, C.c_size_t, vp]
-    lib.yahkv_decode_reduce.argtypes = [G, i32, i32p, i32, i32, vp, vp, vp, C.c_size_t, vp]
-    lib.yahkv_decode_attend.argtypes = [G, P, i32p, i32, i32p, i32, i32, vp, i32, C.c_float, vp, vp, vp, C.c_size_t, vp]
+    O = C.POINTER(DecodeOptions)
+    lib.yahkv_decode_workspace_bytes.argtypes = [G, i32, i32, O]
+    lib.yahkv_decode_part.argtypes = [G, P, i32p, i32, i32p, i32, i32, vp, i32, C.c_float, vp, C.c_size_t, O, vp]
+    lib.yahkv_decode_reduce.argtypes = [G, i32, i32p, i32, i32, vp, vp, vp, C.c_size_t, O, vp]
+    lib.yahkv_decode_attend.argtypes = [G, P, i32p, i32, i32p, i32, i32, vp, i32, C.c_float, vp, vp, vp, C.c_size_t, O,
+                                        vp]
+    lib.yahkv_decode_calibrate.argtypes = [G, P, i32p, i32, i32p, i32, i32, vp, i32, vp, C.c_size_t, O, i32, vp]
     lib.yahkv_decode_static_scratch_bytes.restype = C.c_size_t
     lib.yahkv_decode_attend_static.argtypes = [G, P, i32p, i32, i32p, i32, i32, vp, i32, C.c_float, vp, vp, vp]
     lib.yahkv_prefill_workspace_bytes.restype = C.c_size_t
@@ -77,9 +86,9 @@ def _load():
     lib.yahkv_f16_prefill_attend.argtypes = [G, F, i32p, i32, i32p, i32, i32, i32, vp, C.c_float, vp, vp, i32, vp,
                                              C.c_size_t, vp]
     lib.yahkv_f16_decode_workspace_bytes.restype = C.c_size_t
-    lib.yahkv_f16_decode_workspace_bytes.argtypes = [G, i32, i32]
+    lib.yahkv_f16_decode_workspace_bytes.argtypes = [G, i32, i32, O]
     lib.yahkv_f16_decode_attend.argtypes = [G, F, i32p, i32, i32p, i32, i32, vp, i32, C.c_float, vp, vp, vp,
-                                            C.c_size_t, vp]
+                                            C.c_size_t, O, vp]
     lib.yahkv_prefill_decode_tiles.argtypes = [G, P, i32p, i32, i32p, i32, i32, i32, vp, C.c_size_t, vp]
     lib.yahkv_gather_blocks.argtypes = [G, P, i32p, i32, vp, vp, vp]
     lib.yahkv_pagepool_create.restype = C.c_void_p
@@ -202,7 +211,7 @@ class F16Pools:
         self.v = torch.full((n,), fill, dtype=torch.uint8, device=device)
 
     def struct(self):
-        return F16PoolsStruct(self.k.data_ptr(), self.v.data_ptr())
+        return F16PoolsStruct(self.k.data_ptr(), self.v.data_ptr(), self.k.numel(), self.v.numel())
 
     def numpy(self):
         """K as [page][H][D / 16][PT][16] and V^T as [page][H][D][PT], uint16 bit patterns (V^T is stored in runs of
@@ -233,7 +242,7 @@ def f16_append(pools, table, start_pos, k_src, v_src, n_valid=None):
                                 n_seqs, n_new, _dp(k_src), _dp(v_src), _dtype_code(k_src), _stream()), "f16_append")
 
 
-def f16_decode_attend(pools, table, seq_len, max_seq_len, q, scale, gate=None, out=None, workspace=None):
+def f16_decode_attend(pools, table, seq_len, max_seq_len, q, scale, gate=None, out=None, workspace=None, opt=None):
     """decode_attend() over f16 pools; returns out f32 [n_seqs][n_q_heads][D]."""
     import torch
     g = pools.geom
@@ -242,12 +251,12 @@ def f16_decode_attend(pools, table, seq_len, max_seq_len, q, scale, gate=None, o
     if out is None:
         out = torch.empty(q.shape, dtype=torch.float32, device=q.device)
     if workspace is None:
-        need = lib.yahkv_f16_decode_workspace_bytes(C.byref(g), n_seqs, max_seq_len)
+        need = lib.yahkv_f16_decode_workspace_bytes(C.byref(g), n_seqs, max_seq_len, _op(opt))
         workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=q.device)
     st = pools.struct()
     _check(lib.yahkv_f16_decode_attend(C.byref(g), C.byref(st), _dp(table), table.shape[1], _dp(seq_len), n_seqs,
                                        max_seq_len, _dp(q), _dtype_code(q), scale, _dp(gate), _dp(out),
-                                       _dp(workspace), workspace.numel(), _stream()), "f16_decode_attend")
+                                       _dp(workspace), workspace.numel(), _op(opt), _stream()), "f16_decode_attend")
     return out
 
 
@@ -282,7 +291,8 @@ class DevicePools:
         self.vs = torch.full((b["vs"],), fill, dtype=torch.uint8, device=device)
 
     def struct(self):
-        return Pools(self.kq.data_ptr(), self.ks.data_ptr(), self.vq.data_ptr(), self.vs.data_ptr())
+        return Pools(self.kq.data_ptr(), self.ks.data_ptr(), self.vq.data_ptr(), self.vs.data_ptr(),
+                     self.kq.numel(), self.ks.numel(), self.vq.numel(), self.vs.numel())
 
     def numpy(self):
         import numpy as np
@@ -334,11 +344,23 @@ def append_rope(pools, table, start_pos, k_src, v_src, theta, eps, rotary_dim, k
     return q_out, k_out
 
 
-def decode_workspace_bytes(g, n_seqs, max_seq_len):
-    return lib.yahkv_decode_workspace_bytes(C.byref(g), n_seqs, max_seq_len)
+def decode_options(n_chunks=0, min_chunk_tiles=0, pair_cost=0, reduce_split=0, deterministic=False, xcd_weight=None):
+    """yahkv_decode_options; zero / None fields are the defaults."""
+    o = DecodeOptions(n_chunks, min_chunk_tiles, pair_cost, reduce_split, 1 if deterministic else 0)
+    for j, w in enumerate(xcd_weight or ()):
+        o.xcd_weight[j] = int(w)
+    return o
 
 
-def decode_attend(pools, table, seq_len, max_seq_len, q, scale, gate=None, out=None, workspace=None):
+def _op(opt):
+    return None if opt is None else C.byref(opt)
+
+
+def decode_workspace_bytes(g, n_seqs, max_seq_len, opt=None):
+    return lib.yahkv_decode_workspace_bytes(C.byref(g), n_seqs, max_seq_len, _op(opt))
+
+
+def decode_attend(pools, table, seq_len, max_seq_len, q, scale, gate=None, out=None, workspace=None, opt=None):
     """q: [n_seqs][n_q_heads][D] f16 / bf16 / f32; returns out f32 of the same shape."""
     import torch
     g = pools.geom
@@ -346,13 +368,13 @@ def decode_attend(pools, table, seq_len, max_seq_len, q, scale, gate=None, out=N
     assert q.is_contiguous() and table.is_contiguous() and tuple(q.shape) == (n_seqs, g.n_q_heads, g.head_dim)
     if out is None:
         out = torch.empty(q.shape, dtype=torch.float32, device=q.device)
-    need = decode_workspace_bytes(g, n_seqs, max_seq_len)
+    need = decode_workspace_bytes(g, n_seqs, max_seq_len, opt)
     if workspace is None:
         workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
     st = pools.struct()
     _check(lib.yahkv_decode_attend(C.byref(g), C.byref(st), _dp(table), table.shape[1], _dp(seq_len), n_seqs,
                                    max_seq_len, _dp(q), _dtype_code(q), scale, _dp(gate), _dp(out), _dp(workspace),
-                                   workspace.numel(), _stream()), "decode_attend")
+                                   workspace.numel(), _op(opt), _stream()), "decode_attend")
     return out
 
 
@@ -366,25 +388,29 @@ def decode_attend_static(pools, table, seq_len, max_seq_len, q, scale, out, gate
     return out
 
 
-def decode_plan(g, table_stride, seq_len, n_seqs, max_seq_len, workspace):
-    """Checks the arguments of a decode attention; launches nothing (part and reduce derive the cut themselves)."""
-    _check(lib.yahkv_decode_plan(C.byref(g), table_stride, _dp(seq_len), n_seqs, max_seq_len, _dp(workspace),
-                                 workspace.numel(), _stream()), "decode_plan")
-
-
-def decode_part(pools, table, seq_len, max_seq_len, q, scale, workspace):
-    """Second dispatch of decode_attend: partials into the workspace."""
+def decode_part(pools, table, seq_len, max_seq_len, q, scale, workspace, opt=None):
+    """First dispatch of decode_attend: partials into the workspace."""
     g = pools.geom
     st = pools.struct()
     _check(lib.yahkv_decode_part(C.byref(g), C.byref(st), _dp(table), table.shape[1], _dp(seq_len), q.shape[0],
                                  max_seq_len, _dp(q), _dtype_code(q), scale, _dp(workspace), workspace.numel(),
-                                 _stream()), "decode_part")
+                                 _op(opt), _stream()), "decode_part")
 
 
-def decode_reduce(g, table_stride, seq_len, n_seqs, max_seq_len, out, workspace, gate=None):
-    """Third dispatch of decode_attend: merge the partials into out."""
+def decode_reduce(g, table_stride, seq_len, n_seqs, max_seq_len, out, workspace, gate=None, opt=None):
+    """Second dispatch of decode_attend: merge the partials into out."""
     _check(lib.yahkv_decode_reduce(C.byref(g), table_stride, _dp(seq_len), n_seqs, max_seq_len, _dp(gate), _dp(out),
-                                   _dp(workspace), workspace.numel(), _stream()), "decode_reduce")
+                                   _dp(workspace), workspace.numel(), _op(opt), _stream()), "decode_reduce")
+
+
+def decode_calibrate(pools, table, seq_len, max_seq_len, q, workspace, opt, rounds=2):
+    """Measures the XCDs' relative speeds on this batch into opt.xcd_weight (synchronizes; overwrites the workspace)."""
+    g = pools.geom
+    st = pools.struct()
+    _check(lib.yahkv_decode_calibrate(C.byref(g), C.byref(st), _dp(table), table.shape[1], _dp(seq_len), q.shape[0],
+                                      max_seq_len, _dp(q), _dtype_code(q), _dp(workspace), workspace.numel(),
+                                      C.byref(opt), rounds, _stream()), "decode_calibrate")
+    return list(opt.xcd_weight)
 
 
 def prefill_workspace_bytes(g, n_seqs, max_prefix_len, chunk_len):

@@ -404,15 +404,11 @@ namespace {
 int CheckAppend(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
                 int32_t page_table_stride, const int32_t* start_pos, int32_t n_seqs, int32_t n_new, const void* k_src,
                 const void* v_src, int32_t src_dtype) {
-  if (const int st = CheckGeometry(g)) return st;
-  if (pools == nullptr || pools->kq == nullptr || pools->ks == nullptr || pools->vq == nullptr ||
-      pools->vs == nullptr || page_table == nullptr || start_pos == nullptr || k_src == nullptr || v_src == nullptr)
-    return YAHKV_ERR_ARG;
+  if (const int st = CheckPools(g, pools)) return st;
+  if (page_table == nullptr || start_pos == nullptr || k_src == nullptr || v_src == nullptr) return YAHKV_ERR_ARG;
   if (n_seqs <= 0 || n_new <= 0 || page_table_stride <= 0) return YAHKV_ERR_ARG;
   if (src_dtype != YAHKV_F32 && src_dtype != YAHKV_F16 && src_dtype != YAHKV_BF16) return YAHKV_ERR_ARG;
-  if ((reinterpret_cast<uintptr_t>(pools->kq) | reinterpret_cast<uintptr_t>(pools->vq) |
-       reinterpret_cast<uintptr_t>(k_src) | reinterpret_cast<uintptr_t>(v_src)) & 15)
-    return YAHKV_ERR_ARG;
+  if ((reinterpret_cast<uintptr_t>(k_src) | reinterpret_cast<uintptr_t>(v_src)) & 15) return YAHKV_ERR_ARG;
   if (int64_t(n_seqs) * n_new > 0x7FFFFFFF) return YAHKV_ERR_SHAPE;
   return YAHKV_OK;
 }
@@ -467,7 +463,6 @@ extern "C" int yahkv_append_rope(const yahkv_geometry* g, const yahkv_pools* poo
   if ((q_src == nullptr) != (q_out == nullptr)) return YAHKV_ERR_ARG;
   if (q_src != nullptr && q_out_dtype != YAHKV_F32 && q_out_dtype != YAHKV_F16 && q_out_dtype != YAHKV_BF16)
     return YAHKV_ERR_ARG;
-  if ((reinterpret_cast<uintptr_t>(pools->kq) | reinterpret_cast<uintptr_t>(pools->vq)) & 15) return YAHKV_ERR_ARG;
   const Geom m = MakeGeom(*g);
   if (rope->rotary_dim < 8 || rope->rotary_dim > m.hd || rope->rotary_dim % 8 != 0) return YAHKV_ERR_ARG;
   if (!(rope->theta > 0.0f) || !(rope->eps >= 0.0f)) return YAHKV_ERR_ARG;
@@ -488,9 +483,8 @@ extern "C" int yahkv_append_rope(const yahkv_geometry* g, const yahkv_pools* poo
 
 extern "C" int yahkv_gather_blocks(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* table_row,
                                    int32_t n_tokens, void* dst_k, void* dst_v, void* stream) {
-  if (const int st = CheckGeometry(g)) return st;
-  if (pools == nullptr || table_row == nullptr || dst_k == nullptr || dst_v == nullptr || n_tokens <= 0)
-    return YAHKV_ERR_ARG;
+  if (const int st = CheckPools(g, pools)) return st;
+  if (table_row == nullptr || dst_k == nullptr || dst_v == nullptr || n_tokens <= 0) return YAHKV_ERR_ARG;
   const Geom m = MakeGeom(*g);
   const int64_t items = int64_t(2) * n_tokens * m.n_kv * m.nb();
   const unsigned blocks = static_cast<unsigned>((items + 255) / 256);

@@ -53,6 +53,8 @@ __device__ __forceinline__ float LoadSrc(const void* p, size_t i, int dt) {
 }
 
 int CheckGeometry(const yahkv_geometry* g);
+// Geometry, then the four pools: not null, 16-byte aligned, each at least as long as the geometry needs.
+int CheckPools(const yahkv_geometry* g, const yahkv_pools* pools);
 inline int LaunchStatus() { return hipGetLastError() == hipSuccess ? YAHKV_OK : YAHKV_ERR_LAUNCH; }
 
 }  // namespace yahkv

@@ -20,6 +20,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <mutex>
+#include <vector>
 
 #include "common.hpp"
 
@@ -52,6 +53,8 @@ struct DecodeArgs {
   int32_t min_chunk_tiles;
   int32_t pair_cost;  // line units a (sequence, kv head) pair takes besides its tiles
   int32_t share[9];  // cumulative shares of the eight chunks of a group, in 1/8192 of the group (share[8] = 8192)
+  int32_t deterministic;  // waves take the chunk's tiles in a fixed pattern instead of first come, first served
+  unsigned long long* stamps;  // calibration only: [n_chunks] the time each workgroup's last wave finished
 };
 
 __device__ __forceinline__ int ClampLen(const DecodeArgs& a, int s) { return min(max(a.seq_len[s], 0), a.max_len); }
@@ -267,7 +270,13 @@ __device__ __forceinline__ h8v RawNibbles8(uint32_t w0, uint32_t w1) {
   return __builtin_bit_cast(h8v, r);
 }
 
-// Eight consecutive query elements as f16 (bf16 and f16 sources convert exactly in the normal f16 range).
+// Eight consecutive query elements as f16. f16 sources are taken as they are; bf16 sources convert exactly in the
+// normal f16 range, f32 sources (what the reference's kernels take, gen_decode_attn.py:576) round to nearest even;
+// finite values beyond the f16 range saturate at +-65504 instead of becoming infinite (an infinite score would turn the
+// whole row into NaN); NaN and infinite inputs give NaN.
+__device__ __forceinline__ _Float16 SaturateToF16(float x) {
+  return static_cast<_Float16>(__builtin_fminf(__builtin_fmaxf(x, -65504.0f), 65504.0f) + (x - x));  // x - x: 0, or NaN
+}
 __device__ __forceinline__ h8v LoadQ8(const void* q, size_t i, int dt) {
   h8v r;
   if (dt == YAHKV_F32) {
@@ -275,14 +284,14 @@ __device__ __forceinline__ h8v LoadQ8(const void* q, size_t i, int dt) {
     const float4 b = *reinterpret_cast<const float4*>(static_cast<const float*>(q) + i + 4);
     const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
 #pragma unroll
-    for (int j = 0; j < 8; ++j) r[j] = static_cast<_Float16>(v[j]);
+    for (int j = 0; j < 8; ++j) r[j] = SaturateToF16(v[j]);
   } else {
     const uint4 a = *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(q) + i);
     const uint32_t w[4] = {a.x, a.y, a.z, a.w};
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const uint16_t hbits = static_cast<uint16_t>(w[j / 2] >> (16 * (j % 2)));
-      r[j] = dt == YAHKV_F16 ? __builtin_bit_cast(_Float16, hbits) : static_cast<_Float16>(WidenBf16(hbits));
+      r[j] = dt == YAHKV_F16 ? __builtin_bit_cast(_Float16, hbits) : SaturateToF16(WidenBf16(hbits));
     }
   }
   return r;
@@ -344,12 +353,19 @@ void DattnPart(const DecodeArgs a) {
   auto& lvs = lvs_all[wave];
   auto& lvq = lvq_all[wave];
 
+  if (a.stamps != nullptr && threadIdx.x == 0) a.stamps[blockIdx.x] = wall_clock64();
   const int4 rec = ChunkRecord<64 * kWavesPerGroup>(a, blockIdx.x, wave_sum, &chunk_rec, chunk_tiles);
   if (rec.x < 0) return;
   const int chunk_n = rec.w;
   if (threadIdx.x == 0) next_tile = 0;
   __syncthreads();
+  int my_next = wave;
   auto take = [&]() -> int {  // the next tile of the chunk nobody has taken yet (>= chunk_n: none left)
+    if (a.deterministic) {    // wave w takes tiles w, w + 8, ...: the same sums in the same order on every run
+      const int v = my_next;
+      my_next += kWavesPerGroup;
+      return v;
+    }
     int v = 0;
     if (lane == 0) v = __hip_atomic_fetch_add(&next_tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     return __builtin_amdgcn_readfirstlane(v);
@@ -682,6 +698,7 @@ void DattnPart(const DecodeArgs a) {
     if (!worked) leave_empty();
     worked = false;
   } while (NextPair(a, chunk_n, &cur));
+  if (a.stamps != nullptr && lane == 0) atomicMax(&a.stamps[a.n_chunks + blockIdx.x], wall_clock64());
 }
 
 // ---- reduce -------------------------------------------------------------------------------------------------------------
@@ -786,7 +803,7 @@ __global__ __launch_bounds__(kReduceThreads) void DattnReduce(const DecodeArgs a
 struct Plan {
   int32_t max_len, n_chunks, wpc, min_chunk_tiles, pair_cost;
   int32_t share[9];
-  size_t off_tprefix, off_ml, off_acc, bytes;
+  size_t off_tprefix, off_ml, off_acc, off_stamps, bytes;
 };
 size_t Align(size_t x) { return (x + 255) & ~size_t(255); }
 int ComputeUnits() {
@@ -799,60 +816,65 @@ int ComputeUnits() {
   }();
   return cus;
 }
-int EnvInt(const char* name, int fallback, int lo, int hi) {
-  const char* e = std::getenv(name);
-  return e == nullptr ? fallback : std::min(hi, std::max(lo, std::atoi(e)));
+// Tuning values of a call: the caller's options where given, else the defaults.
+struct Tuning {
+  int32_t n_chunks, min_chunk_tiles, pair_cost, reduce_split, deterministic;
+  int32_t xcd_weight[8];
+};
+Tuning MakeTuning(const yahkv_decode_options* o) {
+  Tuning t{};
+  // one 8-wave workgroup per CU (two waves per SIMD)
+  t.n_chunks = o != nullptr && o->n_chunks > 0 ? std::min(o->n_chunks, 1 << 20) : ComputeUnits();
+  // at least 2: with chunks of one unit the smaller shares of a group of eight would round to nothing, and the merge
+  // counts on every chunk inside a pair's stretch of the line having left partials
+  t.min_chunk_tiles = o != nullptr && o->min_chunk_tiles > 0 ? std::min(std::max(o->min_chunk_tiles, 2), 1 << 20)
+                                                             : 2 * kWavesPerGroup;
+  t.pair_cost = o == nullptr || o->pair_cost == 0 ? 8 : std::min(std::max(o->pair_cost, 0), 1 << 10);
+  t.reduce_split = o != nullptr ? std::max(o->reduce_split, 0) : 0;
+  t.deterministic = o != nullptr && o->deterministic != 0;
+  for (int j = 0; j < 8; ++j) t.xcd_weight[j] = o != nullptr ? std::max(o->xcd_weight[j], 0) : 0;
+  return t;
 }
-Plan MakePlan(const Geom& g, int32_t n_seqs, int32_t max_seq_len) {
+Plan MakePlan(const Geom& g, int32_t n_seqs, int32_t max_seq_len, const Tuning& t) {
   Plan p;
   p.max_len = std::max(max_seq_len, 1);
   const int64_t max_tiles = (int64_t(p.max_len) + kTile - 1) / kTile;
   const int64_t line_max = max_tiles * n_seqs * g.n_kv;
-  // Tuning knobs; the environment overrides are for experiments.
-  // one 8-wave workgroup per CU (two waves per SIMD)
   p.wpc = kWavesPerGroup;
-  // at least 2: with chunks of one unit the smaller shares of a group of eight would round to nothing, and the reduce
-  // counts on every chunk inside a pair's stretch of the line having left partials
-  p.min_chunk_tiles = EnvInt("YAHKV_DECODE_MIN_CHUNK_TILES", 2 * kWavesPerGroup, 2, 1 << 20);
-  p.pair_cost = EnvInt("YAHKV_DECODE_PAIR_COST", 8, 0, 1 << 10);
-  p.n_chunks = EnvInt("YAHKV_DECODE_CHUNKS", ComputeUnits(), 1, 1 << 20);
+  p.min_chunk_tiles = t.min_chunk_tiles, p.pair_cost = t.pair_cost;
   p.n_chunks =
-      static_cast<int32_t>(std::min<int64_t>(p.n_chunks, (line_max + p.min_chunk_tiles - 1) / p.min_chunk_tiles));
-  // Relative speeds of the eight XCDs of an MI355X on this kernel (tiles per unit of time, measured with all of
-  // them reading at once); YAHKV_DECODE_XCD_WEIGHTS="w0,...,w7" overrides them. Shares are kept above half the mean.
-  int w[8] = {1050, 942, 1055, 962, 1046, 958, 1052, 942};
-  if (const char* e = std::getenv("YAHKV_DECODE_XCD_WEIGHTS")) {
-    int v[8];
-    if (std::sscanf(e, "%d,%d,%d,%d,%d,%d,%d,%d", v, v + 1, v + 2, v + 3, v + 4, v + 5, v + 6, v + 7) == 8)
-      std::copy(v, v + 8, w);
-  }
-  if (p.n_chunks % 8 != 0) std::fill(w, w + 8, 1);  // a last group that is not whole would leave the line's end uncovered
-  int64_t sum = 0;
-  for (int j = 0; j < 8; ++j) w[j] = std::max(w[j], 1), sum += w[j];
-  for (int j = 0; j < 8; ++j) w[j] = static_cast<int>(std::max<int64_t>(w[j] * 8192 / sum, 512));
-  sum = 0;
-  for (int j = 0; j < 8; ++j) sum += w[j];
+      static_cast<int32_t>(std::min<int64_t>(t.n_chunks, (line_max + p.min_chunk_tiles - 1) / p.min_chunk_tiles));
+  // Shares of the eight chunks of a group: by the caller's relative XCD speeds (yahkv_decode_calibrate measures them),
+  // equal without them. Every share keeps at least 1 / 16 of the group, which at two line units per chunk is one unit:
+  // no chunk inside a pair's stretch comes out empty.
+  int64_t w[8], sum = 0;
+  for (int j = 0; j < 8; ++j) w[j] = t.xcd_weight[j], sum += w[j];
+  // (a last group that is not whole would leave the line's end uncovered: equal shares then)
+  if (sum == 0 || p.n_chunks % 8 != 0) std::fill(w, w + 8, int64_t(1)), sum = 8;
   p.share[0] = 0;
-  for (int j = 0; j < 8; ++j) p.share[j + 1] = p.share[j] + static_cast<int32_t>(w[j] * 8192 / sum);
+  for (int j = 0; j < 8; ++j) p.share[j + 1] = p.share[j] + 512 + static_cast<int32_t>(w[j] * (8192 - 8 * 512) / sum);
   p.share[8] = 8192;
   const size_t parts = (size_t(p.n_chunks) + size_t(n_seqs) * g.n_kv) * p.wpc;
   p.off_tprefix = 0;
   p.off_ml = Align(sizeof(int32_t) * (size_t(n_seqs) + 1));
   p.off_acc = Align(p.off_ml + sizeof(float) * parts * g.group() * 2);
-  p.bytes = Align(p.off_acc + sizeof(float) * parts * g.group() * g.hd);
+  p.off_stamps = Align(p.off_acc + sizeof(float) * parts * g.group() * g.hd);  // for yahkv_decode_calibrate
+  p.bytes = Align(p.off_stamps + 2 * sizeof(unsigned long long) * size_t(p.n_chunks));
   return p;
 }
 
 // Fills the launch arguments all dispatches share; returns a status.
 int Prepare(const yahkv_geometry* g, int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs,
-            int32_t max_seq_len, const void* workspace, size_t workspace_bytes, DecodeArgs* a) {
+            int32_t max_seq_len, const void* workspace, size_t workspace_bytes, const yahkv_decode_options* opt,
+            DecodeArgs* a) {
   if (const int st = CheckGeometry(g)) return st;
   if (seq_len == nullptr || workspace == nullptr) return YAHKV_ERR_ARG;
   if (n_seqs <= 0 || max_seq_len <= 0 || page_table_stride <= 0) return YAHKV_ERR_ARG;
   if (n_seqs > kMaxSeqs) return YAHKV_ERR_SHAPE;  // every workgroup walks all lengths: keep that a few thousand
   if (reinterpret_cast<uintptr_t>(workspace) & 15) return YAHKV_ERR_ARG;
   const Geom m = MakeGeom(*g);
-  const Plan p = MakePlan(m, n_seqs, max_seq_len);
+  const Tuning t = MakeTuning(opt);
+  const Plan p = MakePlan(m, n_seqs, max_seq_len, t);
   if (workspace_bytes < p.bytes) return YAHKV_ERR_WORKSPACE;
   *a = DecodeArgs{};
   a->g = m, a->stride = page_table_stride, a->seq_len = seq_len, a->n_seqs = n_seqs;
@@ -863,48 +885,13 @@ int Prepare(const yahkv_geometry* g, int32_t page_table_stride, const int32_t* s
   a->ml = reinterpret_cast<float*>(ws + p.off_ml);
   a->acc = reinterpret_cast<float*>(ws + p.off_acc);
   a->n_chunks = p.n_chunks, a->wpc = p.wpc, a->min_chunk_tiles = p.min_chunk_tiles, a->pair_cost = p.pair_cost;
+  a->deterministic = t.deterministic;
   std::copy(p.share, p.share + 9, a->share);
   return YAHKV_OK;
 }
 
-}  // namespace
-}  // namespace yahkv
-
-using namespace yahkv;
-
-extern "C" size_t yahkv_decode_workspace_bytes(const yahkv_geometry* g, int32_t n_seqs, int32_t max_seq_len) {
-  if (CheckGeometry(g) || n_seqs <= 0 || max_seq_len <= 0) return 0;
-  return MakePlan(MakeGeom(*g), n_seqs, max_seq_len).bytes;
-}
-
-extern "C" int yahkv_decode_plan(const yahkv_geometry* g, int32_t page_table_stride, const int32_t* seq_len,
-                                 int32_t n_seqs, int32_t max_seq_len, void* workspace, size_t workspace_bytes,
-                                 void* stream) {
-  DecodeArgs a;
-  if (const int st = Prepare(g, page_table_stride, seq_len, n_seqs, max_seq_len, workspace, workspace_bytes, &a))
-    return st;
-  (void)stream;  // nothing to launch: part and reduce derive the cut from the lengths themselves
-  return YAHKV_OK;
-}
-
-extern "C" int yahkv_decode_part(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
-                                 int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs,
-                                 int32_t max_seq_len, const void* q, int32_t q_dtype, float softmax_scale,
-                                 void* workspace, size_t workspace_bytes, void* stream) {
-  DecodeArgs a;
-  if (const int st = Prepare(g, page_table_stride, seq_len, n_seqs, max_seq_len, workspace, workspace_bytes, &a))
-    return st;
-  if (pools == nullptr || pools->kq == nullptr || pools->ks == nullptr || pools->vq == nullptr ||
-      pools->vs == nullptr || page_table == nullptr || q == nullptr)
-    return YAHKV_ERR_ARG;
-  if (q_dtype != YAHKV_F32 && q_dtype != YAHKV_F16 && q_dtype != YAHKV_BF16) return YAHKV_ERR_ARG;
-  if ((reinterpret_cast<uintptr_t>(pools->kq) | reinterpret_cast<uintptr_t>(pools->vq) |
-       reinterpret_cast<uintptr_t>(pools->ks) | reinterpret_cast<uintptr_t>(pools->vs) |
-       reinterpret_cast<uintptr_t>(q)) & 15)
-    return YAHKV_ERR_ARG;
-  a.pools = MakePools(*pools), a.table = page_table, a.q = q, a.q_dtype = q_dtype, a.scale = softmax_scale;
+int LaunchPart(const DecodeArgs& a, hipStream_t st) {
   const Geom& m = a.g;
-  hipStream_t st = static_cast<hipStream_t>(stream);
   const dim3 grid(static_cast<unsigned>(a.n_chunks));
 #define YAHKV_LAUNCH_PART(FF, DD, PP) \
   hipLaunchKernelGGL((DattnPart<FF, DD, PP>), grid, dim3(64 * kWavesPerGroup), 0, st, a)
@@ -925,22 +912,119 @@ extern "C" int yahkv_decode_part(const yahkv_geometry* g, const yahkv_pools* poo
   return LaunchStatus();
 }
 
+int CheckPartArgs(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table, const void* q,
+                  int32_t q_dtype) {
+  if (const int st = CheckPools(g, pools)) return st;
+  if (page_table == nullptr || q == nullptr || (reinterpret_cast<uintptr_t>(q) & 15)) return YAHKV_ERR_ARG;
+  if (q_dtype != YAHKV_F32 && q_dtype != YAHKV_F16 && q_dtype != YAHKV_BF16) return YAHKV_ERR_ARG;
+  return YAHKV_OK;
+}
+
+}  // namespace
+}  // namespace yahkv
+
+using namespace yahkv;
+
+extern "C" size_t yahkv_decode_workspace_bytes(const yahkv_geometry* g, int32_t n_seqs, int32_t max_seq_len,
+                                               const yahkv_decode_options* opt) {
+  if (CheckGeometry(g) || n_seqs <= 0 || max_seq_len <= 0) return 0;
+  return MakePlan(MakeGeom(*g), n_seqs, max_seq_len, MakeTuning(opt)).bytes;
+}
+
+extern "C" int yahkv_decode_part(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
+                                 int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs,
+                                 int32_t max_seq_len, const void* q, int32_t q_dtype, float softmax_scale,
+                                 void* workspace, size_t workspace_bytes, const yahkv_decode_options* opt,
+                                 void* stream) {
+  DecodeArgs a;
+  if (const int st = Prepare(g, page_table_stride, seq_len, n_seqs, max_seq_len, workspace, workspace_bytes, opt, &a))
+    return st;
+  if (const int st = CheckPartArgs(g, pools, page_table, q, q_dtype)) return st;
+  a.pools = MakePools(*pools), a.table = page_table, a.q = q, a.q_dtype = q_dtype, a.scale = softmax_scale;
+  return LaunchPart(a, static_cast<hipStream_t>(stream));
+}
+
 extern "C" int yahkv_decode_reduce(const yahkv_geometry* g, int32_t page_table_stride, const int32_t* seq_len,
                                    int32_t n_seqs, int32_t max_seq_len, const float* gate, float* out,
-                                   const void* workspace, size_t workspace_bytes, void* stream) {
+                                   const void* workspace, size_t workspace_bytes, const yahkv_decode_options* opt,
+                                   void* stream) {
   DecodeArgs a;
-  if (const int st = Prepare(g, page_table_stride, seq_len, n_seqs, max_seq_len, workspace, workspace_bytes, &a))
+  if (const int st = Prepare(g, page_table_stride, seq_len, n_seqs, max_seq_len, workspace, workspace_bytes, opt, &a))
     return st;
   if (out == nullptr) return YAHKV_ERR_ARG;
   a.gate = gate, a.out = out;
   // a small batch: more workgroups per (query head, sequence), each with a part of the dims, until the CUs have one
   int split = 1;
   while (int64_t(a.g.n_q) * n_seqs * split < ComputeUnits() && a.g.hd / (2 * split) >= kReduceMinDims) split *= 2;
-  split = EnvInt("YAHKV_DECODE_REDUCE_SPLIT", split, 1, a.g.hd / kReduceMinDims);
+  const int asked = MakeTuning(opt).reduce_split;
+  if (asked > 0) split = std::min(asked, a.g.hd / kReduceMinDims);
   while (a.g.hd % split != 0 || (a.g.hd / split) % 4 != 0) --split;
   hipLaunchKernelGGL(DattnReduce, dim3(a.g.n_q, n_seqs, split), dim3(kReduceThreads), 0,
                      static_cast<hipStream_t>(stream), a);
   return LaunchStatus();
+}
+
+extern "C" int yahkv_decode_attend(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
+                                   int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs,
+                                   int32_t max_seq_len, const void* q, int32_t q_dtype, float softmax_scale,
+                                   const float* gate, float* out, void* workspace, size_t workspace_bytes,
+                                   const yahkv_decode_options* opt, void* stream) {
+  if (out == nullptr) return YAHKV_ERR_ARG;
+  if (const int st = yahkv_decode_part(g, pools, page_table, page_table_stride, seq_len, n_seqs, max_seq_len, q,
+                                       q_dtype, softmax_scale, workspace, workspace_bytes, opt, stream))
+    return st;
+  return yahkv_decode_reduce(g, page_table_stride, seq_len, n_seqs, max_seq_len, gate, out, workspace,
+                             workspace_bytes, opt, stream);
+}
+
+// Relative read speeds of the eight XCDs on the caller's own batch. Workgroup k of a dispatch runs on XCD k % 8, and the
+// XCDs of one GPU do not read memory equally fast (up to 10 % apart, measured); chunk shares that follow their speeds
+// let all workgroups finish together. Each round runs the part kernel twice with the current shares (the first launch
+// warms caches and clocks), reads when each workgroup's last wave finished, and sets every XCD's weight to its share
+// divided by its mean time. Synchronizes the stream: a set-up call, not part of a step.
+extern "C" int yahkv_decode_calibrate(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
+                                      int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs,
+                                      int32_t max_seq_len, const void* q, int32_t q_dtype, void* workspace,
+                                      size_t workspace_bytes, yahkv_decode_options* opt, int32_t rounds,
+                                      void* stream) {
+  if (opt == nullptr || rounds <= 0) return YAHKV_ERR_ARG;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  for (int32_t r = 0; r < rounds; ++r) {
+    DecodeArgs a;
+    if (const int rc = Prepare(g, page_table_stride, seq_len, n_seqs, max_seq_len, workspace, workspace_bytes, opt, &a))
+      return rc;
+    if (const int rc = CheckPartArgs(g, pools, page_table, q, q_dtype)) return rc;
+    if (a.n_chunks % 8 != 0) return YAHKV_OK;  // a batch too small for whole groups is cut into equal shares anyway
+    a.pools = MakePools(*pools), a.table = page_table, a.q = q, a.q_dtype = q_dtype, a.scale = 1.0f;
+    const Plan p = MakePlan(a.g, n_seqs, max_seq_len, MakeTuning(opt));
+    a.stamps = reinterpret_cast<unsigned long long*>(static_cast<char*>(workspace) + p.off_stamps);
+    const size_t n = 2 * size_t(a.n_chunks);  // [0, n_chunks): start of each workgroup, [n_chunks, ..): its end
+    std::vector<unsigned long long> stamps(n);
+    for (int pass = 0; pass < 2; ++pass) {
+      if (hipMemsetAsync(a.stamps, 0, n * sizeof(unsigned long long), st) != hipSuccess) return YAHKV_ERR_LAUNCH;
+      if (const int rc = LaunchPart(a, st)) return rc;
+    }
+    if (hipMemcpyAsync(stamps.data(), a.stamps, n * sizeof(unsigned long long), hipMemcpyDeviceToHost, st) != hipSuccess ||
+        hipStreamSynchronize(st) != hipSuccess)
+      return YAHKV_ERR_LAUNCH;
+    unsigned long long start = ~0ull;
+    for (int k = 0; k < a.n_chunks; ++k)
+      if (stamps[size_t(k)] != 0) start = std::min(start, stamps[size_t(k)]);
+    double t[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    int cnt[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int k = 0; k < a.n_chunks; ++k) {
+      const unsigned long long end = stamps[size_t(a.n_chunks) + size_t(k)];
+      if (end > start) t[k % 8] += double(end - start), ++cnt[k % 8];
+    }
+    double speed[8], top = 0;
+    for (int j = 0; j < 8; ++j) {
+      if (cnt[j] == 0 || t[j] <= 0) return YAHKV_OK;  // an XCD without work: nothing to learn from this batch
+      speed[j] = double(a.share[j + 1] - a.share[j]) / (t[j] / cnt[j]);
+      top = std::max(top, speed[j]);
+    }
+    for (int j = 0; j < 8; ++j) opt->xcd_weight[j] = std::max(1, static_cast<int32_t>(speed[j] / top * 10000.0 + 0.5));
+  }
+  return YAHKV_OK;
 }
 
 // ---- decode attention without a workspace argument ------------------------------------------------------------------------
@@ -977,28 +1061,13 @@ extern "C" int yahkv_decode_attend_static(const yahkv_geometry* g, const yahkv_p
                                           int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs,
                                           int32_t max_seq_len, const void* q, int32_t q_dtype, float softmax_scale,
                                           const float* gate, float* out, void* stream) {
-  if (const int st = CheckGeometry(g)) return st;
+  if (const int st = CheckPools(g, pools)) return st;
   if (n_seqs <= 0 || max_seq_len <= 0) return YAHKV_ERR_ARG;
   // the partials of this batch must fit the array: nothing is launched otherwise
-  if (MakePlan(MakeGeom(*g), n_seqs, max_seq_len).bytes > kStaticScratchBytes) return YAHKV_ERR_WORKSPACE;
+  if (MakePlan(MakeGeom(*g), n_seqs, max_seq_len, MakeTuning(nullptr)).bytes > kStaticScratchBytes)
+    return YAHKV_ERR_WORKSPACE;
   void* ws = nullptr;
   if (const int st = StaticScratch(&ws)) return st;
   return yahkv_decode_attend(g, pools, page_table, page_table_stride, seq_len, n_seqs, max_seq_len, q, q_dtype,
-                             softmax_scale, gate, out, ws, kStaticScratchBytes, stream);
-}
-
-extern "C" int yahkv_decode_attend(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
-                                   int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs,
-                                   int32_t max_seq_len, const void* q, int32_t q_dtype, float softmax_scale,
-                                   const float* gate, float* out, void* workspace, size_t workspace_bytes,
-                                   void* stream) {
-  if (out == nullptr) return YAHKV_ERR_ARG;
-  if (const int st = yahkv_decode_plan(g, page_table_stride, seq_len, n_seqs, max_seq_len, workspace, workspace_bytes,
-                                       stream))
-    return st;
-  if (const int st = yahkv_decode_part(g, pools, page_table, page_table_stride, seq_len, n_seqs, max_seq_len, q,
-                                       q_dtype, softmax_scale, workspace, workspace_bytes, stream))
-    return st;
-  return yahkv_decode_reduce(g, page_table_stride, seq_len, n_seqs, max_seq_len, gate, out, workspace,
-                             workspace_bytes, stream);
+                             softmax_scale, gate, out, ws, kStaticScratchBytes, nullptr, stream);
 }

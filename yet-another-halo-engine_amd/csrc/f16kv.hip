@@ -409,17 +409,27 @@ int CheckF16Geometry(const yahkv_geometry* g) {
   return CheckGeometry(&q);
 }
 
+// Geometry, then the two pools: not null, 16-byte aligned, each at least as long as the geometry needs.
+int CheckF16Pools(const yahkv_geometry* g, const yahkv_f16_pools* pools) {
+  if (const int st = CheckF16Geometry(g)) return st;
+  if (pools == nullptr || pools->k == nullptr || pools->v == nullptr) return YAHKV_ERR_ARG;
+  if ((reinterpret_cast<uintptr_t>(pools->k) | reinterpret_cast<uintptr_t>(pools->v)) & 15) return YAHKV_ERR_ARG;
+  const size_t need = size_t(g->n_pages) * g->n_kv_heads * g->head_dim * g->page_tokens * 2;
+  if (pools->k_bytes < need || pools->v_bytes < need) return YAHKV_ERR_ARG;
+  return YAHKV_OK;
+}
+
 struct Split {
   int32_t n_splits, keys_per_split;
   size_t off_acc, bytes;
 };
 // Stretches of every sequence: enough workgroups for a few per CU, a stretch a multiple of the four waves' tiles.
-Split MakeSplit(const Geom& g, int32_t n_seqs, int32_t max_len) {
+Split MakeSplit(const Geom& g, int32_t n_seqs, int32_t max_len, const yahkv_decode_options* opt) {
   Split sp;
   const int64_t unit = int64_t(kTileKeys) * kWaves;
   const int64_t pairs = int64_t(n_seqs) * g.n_kv;
-  int64_t target = 4096;  // workgroups in all, about sixteen per CU; YAHKV_F16_WORKGROUPS overrides it for experiments
-  if (const char* e = std::getenv("YAHKV_F16_WORKGROUPS")) target = std::max(1, std::atoi(e));
+  // workgroups in all: about sixteen per CU unless the caller's options say otherwise
+  const int64_t target = opt != nullptr && opt->n_chunks > 0 ? opt->n_chunks : 4096;
   int64_t want = std::max<int64_t>(1, (target + pairs - 1) / pairs);
   want = std::min<int64_t>(std::min<int64_t>(want, kMaxSplits), (int64_t(max_len) + unit - 1) / unit);
   const int64_t keys = ((int64_t(max_len) + want - 1) / want + unit - 1) / unit * unit;
@@ -445,10 +455,8 @@ extern "C" int yahkv_f16_append(const yahkv_geometry* g, const yahkv_f16_pools* 
                                 int32_t page_table_stride, const int32_t* start_pos, const int32_t* n_valid,
                                 int32_t n_seqs, int32_t n_new, const void* k_src, const void* v_src,
                                 int32_t src_dtype, void* stream) {
-  if (const int st = CheckF16Geometry(g)) return st;
-  if (pools == nullptr || pools->k == nullptr || pools->v == nullptr || page_table == nullptr ||
-      start_pos == nullptr || k_src == nullptr || v_src == nullptr)
-    return YAHKV_ERR_ARG;
+  if (const int st = CheckF16Pools(g, pools)) return st;
+  if (page_table == nullptr || start_pos == nullptr || k_src == nullptr || v_src == nullptr) return YAHKV_ERR_ARG;
   if (n_seqs <= 0 || n_new <= 0 || page_table_stride <= 0) return YAHKV_ERR_ARG;
   if (src_dtype != YAHKV_F32 && src_dtype != YAHKV_F16 && src_dtype != YAHKV_BF16) return YAHKV_ERR_ARG;
   if (n_seqs > 65535) return YAHKV_ERR_SHAPE;  // the grid's z extent
@@ -457,8 +465,7 @@ extern "C" int yahkv_f16_append(const yahkv_geometry* g, const yahkv_f16_pools* 
   a.table = page_table, a.stride = page_table_stride, a.start_pos = start_pos, a.n_valid = n_valid;
   a.n_seqs = n_seqs, a.n_new = n_new, a.k_src = k_src, a.v_src = v_src, a.src_dtype = src_dtype;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  const bool aligned = ((reinterpret_cast<uintptr_t>(k_src) | reinterpret_cast<uintptr_t>(v_src) |
-                         reinterpret_cast<uintptr_t>(pools->k) | reinterpret_cast<uintptr_t>(pools->v)) & 15) == 0;
+  const bool aligned = ((reinterpret_cast<uintptr_t>(k_src) | reinterpret_cast<uintptr_t>(v_src)) & 15) == 0;
   if (n_new >= kRunAppendMinTokens && aligned) {  // chunks: a workgroup per run of positions
     const int T = std::min(a.g.pt, 32);
     const dim3 grid(static_cast<unsigned>((n_new + T - 2) / T + 1), static_cast<unsigned>(a.g.n_kv),
@@ -472,29 +479,27 @@ extern "C" int yahkv_f16_append(const yahkv_geometry* g, const yahkv_f16_pools* 
   return LaunchStatus();
 }
 
-extern "C" size_t yahkv_f16_decode_workspace_bytes(const yahkv_geometry* g, int32_t n_seqs, int32_t max_seq_len) {
+extern "C" size_t yahkv_f16_decode_workspace_bytes(const yahkv_geometry* g, int32_t n_seqs, int32_t max_seq_len,
+                                                   const yahkv_decode_options* opt) {
   if (CheckF16Geometry(g) || n_seqs <= 0 || max_seq_len <= 0) return 0;
-  return MakeSplit(MakeGeom(*g), n_seqs, max_seq_len).bytes;
+  return MakeSplit(MakeGeom(*g), n_seqs, max_seq_len, opt).bytes;
 }
 
 extern "C" int yahkv_f16_decode_attend(const yahkv_geometry* g, const yahkv_f16_pools* pools,
                                        const int32_t* page_table, int32_t page_table_stride, const int32_t* seq_len,
                                        int32_t n_seqs, int32_t max_seq_len, const void* q, int32_t q_dtype,
                                        float softmax_scale, const float* gate, float* out, void* workspace,
-                                       size_t workspace_bytes, void* stream) {
-  if (const int st = CheckF16Geometry(g)) return st;
-  if (pools == nullptr || pools->k == nullptr || pools->v == nullptr || page_table == nullptr || seq_len == nullptr ||
-      q == nullptr || out == nullptr || workspace == nullptr)
+                                       size_t workspace_bytes, const yahkv_decode_options* opt, void* stream) {
+  if (const int st = CheckF16Pools(g, pools)) return st;
+  if (page_table == nullptr || seq_len == nullptr || q == nullptr || out == nullptr || workspace == nullptr)
     return YAHKV_ERR_ARG;
   if (n_seqs <= 0 || max_seq_len <= 0 || page_table_stride <= 0) return YAHKV_ERR_ARG;
   if (q_dtype != YAHKV_F32 && q_dtype != YAHKV_F16 && q_dtype != YAHKV_BF16) return YAHKV_ERR_ARG;
-  if ((reinterpret_cast<uintptr_t>(pools->k) | reinterpret_cast<uintptr_t>(pools->v) |
-       reinterpret_cast<uintptr_t>(workspace)) & 15)
-    return YAHKV_ERR_ARG;
+  if (reinterpret_cast<uintptr_t>(workspace) & 15) return YAHKV_ERR_ARG;
   if (n_seqs > 65535) return YAHKV_ERR_SHAPE;
   F16Args a{};
   a.g = MakeGeom(*g);
-  const Split sp = MakeSplit(a.g, n_seqs, max_seq_len);
+  const Split sp = MakeSplit(a.g, n_seqs, max_seq_len, opt);
   if (workspace_bytes < sp.bytes) return YAHKV_ERR_WORKSPACE;
   a.k = static_cast<uint16_t*>(pools->k), a.v = static_cast<uint16_t*>(pools->v);
   a.table = page_table, a.stride = page_table_stride, a.seq_len = seq_len, a.n_seqs = n_seqs;

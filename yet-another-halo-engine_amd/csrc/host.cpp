@@ -19,6 +19,20 @@ int CheckGeometry(const yahkv_geometry* g) {
   return YAHKV_OK;
 }
 
+int CheckPools(const yahkv_geometry* g, const yahkv_pools* pools) {
+  if (const int st = CheckGeometry(g)) return st;
+  if (pools == nullptr || pools->kq == nullptr || pools->ks == nullptr || pools->vq == nullptr || pools->vs == nullptr)
+    return YAHKV_ERR_ARG;
+  if ((reinterpret_cast<uintptr_t>(pools->kq) | reinterpret_cast<uintptr_t>(pools->ks) |
+       reinterpret_cast<uintptr_t>(pools->vq) | reinterpret_cast<uintptr_t>(pools->vs)) & 15)
+    return YAHKV_ERR_ARG;
+  // the kernels address pages 0 .. n_pages - 1 of every pool: a shorter buffer is refused here, before any launch
+  if (pools->kq_bytes < yahkv_kq_bytes(g) || pools->ks_bytes < yahkv_ks_bytes(g) ||
+      pools->vq_bytes < yahkv_vq_bytes(g) || pools->vs_bytes < yahkv_vs_bytes(g))
+    return YAHKV_ERR_ARG;
+  return YAHKV_OK;
+}
+
 }  // namespace yahkv
 
 using yahkv::CheckGeometry;
@@ -31,7 +45,7 @@ const char* yahkv_version(void) { return "yahkv 0.1 (gfx950)"; }
 const char* yahkv_strerror(int status) {
   switch (status) {
     case YAHKV_OK: return "ok";
-    case YAHKV_ERR_ARG: return "bad argument (null or misaligned pointer, non-positive count)";
+    case YAHKV_ERR_ARG: return "bad argument (null or misaligned pointer, non-positive count, pool shorter than the geometry needs)";
     case YAHKV_ERR_SHAPE: return "no kernel for this geometry";
     case YAHKV_ERR_PAGE: return "page table entry out of range or page used twice";
     case YAHKV_ERR_WORKSPACE: return "workspace too small";

@@ -255,7 +255,7 @@ class KvBatcher {
       L.kq = DeviceBuffer(yahkv_kq_bytes(&g_)), L.ks = DeviceBuffer(yahkv_ks_bytes(&g_));
       L.vq = DeviceBuffer(yahkv_vq_bytes(&g_)), L.vs = DeviceBuffer(yahkv_vs_bytes(&g_));
     }
-    workspace_ = DeviceBuffer(yahkv_decode_workspace_bytes(&g_, max_running, context));
+    workspace_ = DeviceBuffer(yahkv_decode_workspace_bytes(&g_, max_running, context, nullptr));
     // per step: table rows of the planned requests, then prefix, valid, position and length columns
     rows_ = size_t(max_running) + size_t(max_prefill);
     stage_ints_ = rows_ * size_t(stride_) + 4 * rows_;
@@ -338,7 +338,7 @@ class KvBatcher {
       const int32_t* dt = d + size_t(np) * stride_;
       Check(yahkv_append(&g_, &pools, dt, stride_, d_pos, nullptr, nd, 1, dk, dv, kv_dtype, stream_), "append");
       Check(yahkv_decode_attend(&g_, &pools, dt, stride_, d_len, nd, T, dq, dq_dtype, softmax_scale, nullptr, dout,
-                                workspace_.get(), workspace_.size(), stream_), "decode_attend");
+                                workspace_.get(), workspace_.size(), nullptr, stream_), "decode_attend");
     }
   }
   void Commit() { sched_.Commit(); }
@@ -354,7 +354,7 @@ class KvBatcher {
   const yahkv_geometry& geometry() const { return g_; }
   yahkv_pools pools(int32_t layer) const {
     const Layer& L = layers_.at(size_t(layer));
-    return yahkv_pools{L.kq.get(), L.ks.get(), L.vq.get(), L.vs.get()};
+    return yahkv_pools{L.kq.get(), L.ks.get(), L.vq.get(), L.vs.get(), L.kq.size(), L.ks.size(), L.vq.size(), L.vs.size()};
   }
   const std::vector<int32_t>& pages(int64_t id) const { return sched_.pages(id); }
   int32_t length(int64_t id) const { return sched_.length(id); }

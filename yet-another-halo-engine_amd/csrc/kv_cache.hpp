@@ -76,6 +76,11 @@ struct KvDecoderState {
   BufferRef ptab;            // int32 [max_seqs][pages_per_seq]
 };
 
+// The ABI's view of a state's pools: addresses and lengths (the entry points refuse pools shorter than the geometry needs).
+inline yahkv_pools PoolsOf(const KvDecoderState& st) {
+  return yahkv_pools{st.kq.ptr, st.ks.ptr, st.vq.ptr, st.vs.ptr, st.kq.length, st.ks.length, st.vq.length, st.vs.length};
+}
+
 // Host page allocator with a free list (yahkv_pagepool_*).
 class PagePool {
  public:
@@ -118,13 +123,19 @@ class KvDecoder {
     len_.assign(size_t(max_seqs_), 0);
     pages_.resize(size_t(max_seqs_));
     pos_dev_ = DeviceBuffer(sizeof(int32_t) * size_t(max_seqs_) * 2);  // [0]: positions to write, [1]: lengths to attend
-    workspace_ = DeviceBuffer(yahkv_decode_workspace_bytes(&g_, max_seqs_, T_));
-    CheckHip(hipHostMalloc(reinterpret_cast<void**>(&pos_host_), sizeof(int32_t) * size_t(max_seqs_) * 2), "hipHostMalloc");
+    workspace_ = DeviceBuffer(yahkv_decode_workspace_bytes(&g_, max_seqs_, T_, nullptr));
+    // Positions travel through pinned host memory; a step's copy may still be waiting in the stream when the next
+    // step is queued, so there is a ring of staging rows, each with an event that tells when its copy has run.
+    CheckHip(hipHostMalloc(reinterpret_cast<void**>(&pos_host_), sizeof(int32_t) * size_t(max_seqs_) * 2 * kStaging),
+             "hipHostMalloc");
+    for (auto& e : staged_) CheckHip(hipEventCreateWithFlags(&e, hipEventDisableTiming), "hipEventCreate");
   }
   KvDecoder(const KvDecoder&) = delete;
   KvDecoder& operator=(const KvDecoder&) = delete;
   ~KvDecoder() {
     if (pos_host_ != nullptr) (void)hipHostFree(pos_host_);
+    for (auto& e : staged_)
+      if (e != nullptr) (void)hipEventDestroy(e);
   }
 
   int32_t context() const { return T_; }
@@ -204,7 +215,7 @@ class KvDecoder {
       const int32_t pair[2] = {from[size_t(full)], own[0]};
       DeviceBuffer ids(sizeof pair);
       CheckHip(hipMemcpyAsync(ids.get(), pair, sizeof pair, hipMemcpyHostToDevice, stream_), "fork");
-      const yahkv_pools pools{st_.kq.ptr, st_.ks.ptr, st_.vq.ptr, st_.vs.ptr};
+      const yahkv_pools pools = PoolsOf(st_);
       Check(yahkv_copy_pages(&g_, &pools, static_cast<const int32_t*>(ids.get()),
                              static_cast<const int32_t*>(ids.get()) + 1, 1, stream_), "copy_pages");
       CheckHip(hipStreamSynchronize(stream_), "fork");  // `ids` and `pair` go out of scope
@@ -226,7 +237,7 @@ class KvDecoder {
     Upload();
     const size_t bytes = yahkv_slot_bytes(&g_, np);
     DeviceBuffer slot(bytes);
-    const yahkv_pools pools{st_.kq.ptr, st_.ks.ptr, st_.vq.ptr, st_.vs.ptr};
+    const yahkv_pools pools = PoolsOf(st_);
     Check(yahkv_slot_pack(&g_, &pools, static_cast<const int32_t*>(st_.ptab.ptr) + size_t(seq) * stride_, np, len,
                           slot.get(), stream_), "slot_pack");
     std::vector<uint8_t> host(bytes);
@@ -250,11 +261,16 @@ class KvDecoder {
     int32_t np = 0, len = 0;
     if (yahkv_slot_check(&g_, host.data(), host.size(), &np, &len) != YAHKV_OK)
       throw KvError("decoder: the slot " + path + " does not match this geometry");
+    // the header's page count is the one the tokens need, and the sequence's row holds exactly those pages: a slot
+    // never reaches pages the sequence does not own
+    if (np != (len + g_.page_tokens - 1) / g_.page_tokens || np > stride_)
+      throw KvError("decoder: the slot " + path + " names more pages than its tokens fill");
     Reserve(seq, len);
+    if (int32_t(pages_[size_t(seq)].size()) != np) throw KvError("decoder: the slot " + path + " does not fit the sequence");
     Upload();
     DeviceBuffer slot(host.size());
     CheckHip(hipMemcpyAsync(slot.get(), host.data(), host.size(), hipMemcpyHostToDevice, stream_), "slot");
-    const yahkv_pools pools{st_.kq.ptr, st_.ks.ptr, st_.vq.ptr, st_.vs.ptr};
+    const yahkv_pools pools = PoolsOf(st_);
     Check(yahkv_slot_unpack(&g_, &pools, static_cast<const int32_t*>(st_.ptab.ptr) + size_t(seq) * stride_, np,
                             slot.get(), stream_), "slot_unpack");
     CheckHip(hipStreamSynchronize(stream_), "slot");
@@ -275,24 +291,28 @@ class KvDecoder {
             float softmax_scale, const float* gate, float* out) {
     if (!bound_) throw KvError("decoder: no state bound");
     if (n_seqs <= 0 || n_seqs > max_seqs_) throw KvError("decoder: bad batch");
-    int32_t max_len = 0;
-    for (int32_t s = 0; s < n_seqs; ++s) {
+    for (int32_t s = 0; s < n_seqs; ++s)
       if (len_[size_t(s)] >= T_) throw KvError("decoder: position past the set's context");
+    // the staging row of this step: free once the copy queued from it kStaging steps ago has run
+    const size_t slot = step_ % kStaging;
+    if (step_ >= kStaging) CheckHip(hipEventSynchronize(staged_[slot]), "positions");
+    int32_t* row = pos_host_ + slot * size_t(max_seqs_) * 2;
+    for (int32_t s = 0; s < n_seqs; ++s) {
       Reserve(s, len_[size_t(s)] + 1);
-      pos_host_[s] = len_[size_t(s)];
-      pos_host_[max_seqs_ + s] = ++len_[size_t(s)];
-      max_len = std::max(max_len, len_[size_t(s)]);
+      row[s] = len_[size_t(s)];
+      row[max_seqs_ + s] = ++len_[size_t(s)];
     }
     Upload();
-    CheckHip(hipMemcpyAsync(pos_dev_.get(), pos_host_, sizeof(int32_t) * size_t(max_seqs_) * 2, hipMemcpyHostToDevice,
+    CheckHip(hipMemcpyAsync(pos_dev_.get(), row, sizeof(int32_t) * size_t(max_seqs_) * 2, hipMemcpyHostToDevice,
                             stream_), "positions");
-    const yahkv_pools pools{st_.kq.ptr, st_.ks.ptr, st_.vq.ptr, st_.vs.ptr};
+    CheckHip(hipEventRecord(staged_[slot], stream_), "positions");
+    ++step_;
+    const yahkv_pools pools = PoolsOf(st_);
     const int32_t* pos = static_cast<const int32_t*>(pos_dev_.get());
     const int32_t* ptab = static_cast<const int32_t*>(st_.ptab.ptr);
     Check(yahkv_append(&g_, &pools, ptab, stride_, pos, nullptr, n_seqs, 1, k, v, kv_dtype, stream_), "append");
     Check(yahkv_decode_attend(&g_, &pools, ptab, stride_, pos + max_seqs_, n_seqs, T_, q, q_dtype, softmax_scale,
-                              gate, out, workspace_.get(), workspace_.size(), stream_), "decode_attend");
-    (void)max_len;
+                              gate, out, workspace_.get(), workspace_.size(), nullptr, stream_), "decode_attend");
   }
 
   const yahkv_geometry& geometry() const { return g_; }
@@ -326,7 +346,10 @@ class KvDecoder {
   std::vector<DeviceBuffer> own_;
   std::unique_ptr<PagePool> pool_;
   DeviceBuffer pos_dev_, workspace_;
-  int32_t* pos_host_ = nullptr;
+  static constexpr size_t kStaging = 4;
+  int32_t* pos_host_ = nullptr;  // [kStaging][2][max_seqs]
+  hipEvent_t staged_[kStaging] = {nullptr, nullptr, nullptr, nullptr};
+  size_t step_ = 0;
   KvDecoderState st_;
   bool bound_ = false, table_dirty_ = true;
 };
@@ -355,7 +378,7 @@ class KvPrefill {
                             dec_.stream()), "prefix lengths");
     CheckHip(hipStreamSynchronize(dec_.stream()), "prefix lengths");  // `prefix` is a local
     const KvDecoderState& st = dec_.state();
-    const yahkv_pools pools{st.kq.ptr, st.ks.ptr, st.vq.ptr, st.vs.ptr};
+    const yahkv_pools pools = PoolsOf(st);
     const int32_t* ptab = static_cast<const int32_t*>(st.ptab.ptr);
     const int32_t* pre = static_cast<const int32_t*>(prefix_dev_.get());
     Check(yahkv_append(&dec_.geometry(), &pools, ptab, dec_.page_table_stride(), pre, nullptr, n_seqs, chunk_len, k, v,

@@ -872,14 +872,9 @@ namespace {
 int PreparePrefill(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
                    int32_t page_table_stride, const int32_t* prefix_len, int32_t n_seqs, int32_t max_prefix_len,
                    int32_t chunk_len, PrefillArgs* a) {
-  if (const int st = CheckGeometry(g)) return st;
-  if (pools == nullptr || pools->kq == nullptr || pools->ks == nullptr || pools->vq == nullptr ||
-      pools->vs == nullptr || page_table == nullptr || prefix_len == nullptr)
-    return YAHKV_ERR_ARG;
+  if (const int st = CheckPools(g, pools)) return st;
+  if (page_table == nullptr || prefix_len == nullptr) return YAHKV_ERR_ARG;
   if (n_seqs <= 0 || chunk_len <= 0 || max_prefix_len < 0 || page_table_stride <= 0) return YAHKV_ERR_ARG;
-  if ((reinterpret_cast<uintptr_t>(pools->kq) | reinterpret_cast<uintptr_t>(pools->vq) |
-       reinterpret_cast<uintptr_t>(pools->ks) | reinterpret_cast<uintptr_t>(pools->vs)) & 15)
-    return YAHKV_ERR_ARG;
   const Geom m = MakeGeom(*g);
   if (int64_t(page_table_stride) * m.pt < chunk_len) return YAHKV_ERR_ARG;
   *a = PrefillArgs{};
@@ -1034,6 +1029,7 @@ extern "C" int yahkv_f16_prefill_attend(const yahkv_geometry* g, const yahkv_f16
     return YAHKV_ERR_ARG;
   if (n_seqs <= 0 || chunk_len <= 0 || max_prefix_len < 0 || page_table_stride <= 0) return YAHKV_ERR_ARG;
   if ((reinterpret_cast<uintptr_t>(pools->k) | reinterpret_cast<uintptr_t>(pools->v)) & 15) return YAHKV_ERR_ARG;
+  if (pools->k_bytes < yahkv_f16_pool_bytes(g) || pools->v_bytes < yahkv_f16_pool_bytes(g)) return YAHKV_ERR_ARG;
   PrefillArgs a{};
   a.g = MakeGeom(gq);
   if (int64_t(page_table_stride) * a.g.pt < chunk_len) return YAHKV_ERR_ARG;

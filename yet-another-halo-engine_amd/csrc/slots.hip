@@ -54,16 +54,6 @@ __global__ __launch_bounds__(256) void MovePages(Geom g, Pools pools, const int3
   }
 }
 
-int CheckPools(const yahkv_geometry* g, const yahkv_pools* pools) {
-  if (const int st = CheckGeometry(g)) return st;
-  if (pools == nullptr || pools->kq == nullptr || pools->ks == nullptr || pools->vq == nullptr || pools->vs == nullptr)
-    return YAHKV_ERR_ARG;
-  if ((reinterpret_cast<uintptr_t>(pools->kq) | reinterpret_cast<uintptr_t>(pools->ks) |
-       reinterpret_cast<uintptr_t>(pools->vq) | reinterpret_cast<uintptr_t>(pools->vs)) & 15)
-    return YAHKV_ERR_ARG;
-  return YAHKV_OK;
-}
-
 }  // namespace
 }  // namespace yahkv
 
@@ -106,7 +96,8 @@ extern "C" int yahkv_slot_check(const yahkv_geometry* g, const void* header, siz
   if (h[1] != uint64_t(g->format) || h[2] != uint64_t(g->n_kv_heads) || h[3] != uint64_t(g->head_dim) ||
       h[4] != uint64_t(g->page_tokens))
     return YAHKV_ERR_SHAPE;  // a slot loads only into pools of the same format and geometry
-  if (h[5] == 0 || h[5] > 0x7FFFFFFFu || h[6] > h[5] * h[4]) return YAHKV_ERR_ARG;
+  // at least one token, and exactly the pages those tokens fill (a loader trusts the page count for its scatter)
+  if (h[5] == 0 || h[5] > 0x7FFFFFFFu || h[6] == 0 || h[5] != (h[6] + h[4] - 1) / h[4]) return YAHKV_ERR_ARG;
   if (yahkv_slot_bytes(g, static_cast<int32_t>(h[5])) != slot_bytes) return YAHKV_ERR_ARG;
   if (n_pages != nullptr) *n_pages = static_cast<int32_t>(h[5]);
   if (n_tokens != nullptr) *n_tokens = static_cast<int32_t>(h[6]);
