@@ -186,7 +186,7 @@ int yahkv_decode_attend(const yahkv_geometry* g, const yahkv_pools* pools, const
                         const void* q, int32_t q_dtype, float softmax_scale, const float* gate, float* out,
                         void* workspace, size_t workspace_bytes, const yahkv_decode_options* opt, void* stream);
 /* Measures the relative read speeds of the GPU's eight XCDs on the caller's own batch and writes them to
- * opt->xcd_weight (the other fields are read): `rounds` times, the split-K kernel runs twice on the given arguments and
+ * opt->xcd_weight (the other fields are read): `rounds` times, the split-K kernel runs five times on the given arguments and
  * the shares are corrected by when each XCD's workgroups finished. A set-up call: it synchronizes the stream and
  * overwrites the workspace. No counterpart in the reference (one sequence, one workgroup per page). */
 int yahkv_decode_calibrate(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,

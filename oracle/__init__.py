@@ -36,12 +36,12 @@ _lib = None
 _ref = None
 
 
-def lib():
+def lib(path=None):
     global _lib
     if _lib is None:
-        if not os.path.exists(LIB):
+        if path is None and not os.path.exists(LIB):
             build()
-        _lib = C.CDLL(LIB)
+        _lib = C.CDLL(path or LIB)
         for n in ("orc_kq_bytes", "orc_ks_bytes", "orc_vq_bytes", "orc_vs_bytes"):
             getattr(_lib, n).restype = C.c_size_t
             getattr(_lib, n).argtypes = [C.POINTER(Geometry)]
@@ -49,6 +49,27 @@ def lib():
         _lib.orc_lround_identity_mismatches.restype = C.c_uint64
         _lib.orc_lround_identity_mismatches.argtypes = [C.c_uint32, C.c_uint32]
     return _lib
+
+
+def use_native_build():
+    """For the benchmark's CPU-baseline leg: compile the oracle again for this machine's own host cores with the
+    reference's host flags (-O3 -march=native -ffp-contract=off, engine/build_hrx.sh:26) and use that library from now
+    on. The committed build recipe leaves -march out so that the library runs on whatever box it is carried to; a
+    native build cannot travel. Falls back to the portable library if no compiler is here. Returns the flags in use."""
+    global _lib
+    import tempfile
+    out = os.path.join(tempfile.gettempdir(), f"liboracle_native_{os.getpid()}.so")
+    flags = ["-std=c11", "-O3", "-march=native", "-ffp-contract=off", "-fopenmp", "-fPIC", "-shared"]
+    try:
+        subprocess.run(["gcc"] + flags + ["-o", out, os.path.join(HERE, "yahkv_oracle.c"), "-lm"], check=True,
+                       capture_output=True, timeout=120)
+    except (OSError, subprocess.SubprocessError):
+        lib()
+        return "gcc -O3 -ffp-contract=off -fopenmp (portable build: no compiler on this box for -march=native)"
+    _lib = None
+    lib(out)
+    os.unlink(out)                                            # the mapping stays; the file need not
+    return "gcc " + " ".join(flags[1:5])
 
 
 def ref():
@@ -209,7 +230,7 @@ def decode_attend(pools, table, seq_len, q, scale, gate=None):
     return out
 
 
-def prefill_attend(pools, table, prefix_len, q, scale, gate=None, bf16_operands=False):
+def prefill_attend(pools, table, prefix_len, q, scale, gate=None):
     """q f32 [n_seqs][chunk_len][n_q_heads][D]."""
     g = pools.geom
     table, prefix_len = _i32(table), _i32(prefix_len)
@@ -219,7 +240,7 @@ def prefill_attend(pools, table, prefix_len, q, scale, gate=None, bf16_operands=
     st = pools.struct()
     lib().orc_prefill_attend(C.byref(g), C.byref(st), _ptr(table), C.c_int32(table.shape[1]), _ptr(prefix_len),
                              C.c_int32(q.shape[0]), C.c_int32(q.shape[1]), _ptr(q), C.c_float(scale), _ptr(gate),
-                             _ptr(out), C.c_int32(1 if bf16_operands else 0))
+                             _ptr(out))
     return out
 
 

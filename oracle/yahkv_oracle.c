@@ -8,7 +8,7 @@
  *   decode attention   engine/gpu/loom/tools/gen_decode_attn.py:97-335 (one partial (M, l, acc) per page),
  *                      338-411 (merge of the pages, gate), masking key < pos + 1 (:145,167)
  *   prefill attention  engine/gpu/loom/tools/gen_attn_fa.py:1-21 (query start_pos + t sees keys 0..start_pos + t)
- * Build: gcc -O2 -ffp-contract=off -fopenmp (no -ffast-math: the rounding below is the contract).
+ * Build: gcc -O3 -ffp-contract=off -fopenmp (no -ffast-math: the rounding below is the contract).
  */
 #include "yahkv_oracle.h"
 
@@ -356,11 +356,9 @@ void orc_norm_rope(const float* x, const float* weight, int32_t n_rows, int32_t 
   }
 }
 
-static float round_bf16(float x) { return orc_bf16_to_f32(orc_f32_to_bf16(x)); }
-
 void orc_prefill_attend(const orc_geometry* g, const orc_pools* pools, const int32_t* table, int32_t stride,
                         const int32_t* prefix_len, int32_t n_seqs, int32_t chunk_len, const float* q,
-                        float softmax_scale, const float* gate, float* out, int32_t bf16_operands) {
+                        float softmax_scale, const float* gate, float* out) {
   const int H = g->n_kv_heads, NQ = g->n_q_heads, G = NQ / H, D = g->head_dim, PT = g->page_tokens;
 #pragma omp parallel for collapse(2) schedule(dynamic, 1)
   for (int s = 0; s < n_seqs; ++s)
@@ -379,8 +377,6 @@ void orc_prefill_attend(const orc_geometry* g, const orc_pools* pools, const int
         deq_page(g, pools, 0, page, h, nt, kd + (size_t)p * PT * D);
         deq_page(g, pools, 1, page, h, nt, vd + (size_t)p * PT * D);
       }
-      if (bf16_operands)
-        for (size_t i = 0; i < (size_t)np * PT * D * 2; ++i) kd[i] = round_bf16(kd[i]);
       for (int t = 0; t < chunk_len; ++t)
         for (int gi = 0; gi < G; ++gi) {
           const size_t row = (((size_t)s * chunk_len + t) * NQ + (size_t)h * G + gi) * D;
@@ -392,16 +388,12 @@ void orc_prefill_attend(const orc_geometry* g, const orc_pools* pools, const int
             sc[k] = dot * softmax_scale;
             if (sc[k] > M) M = sc[k];
           }
-          /* bf16 model: numerators are taken against the maximum rounded up to a whole power of two, so that
-           * where they are rounded does not depend on the order in which a running maximum met the keys */
-          if (bf16_operands) M = ceil(M * 1.4426950408889634) / 1.4426950408889634;
           double l = 0;
           for (int d = 0; d < D; ++d) acc[d] = 0;
           for (int k = 0; k < keys; ++k) {
             const double e = exp(sc[k] - M);
-            const double pe = bf16_operands ? (double)round_bf16((float)e) : e;
-            l += pe; /* the denominator sums what the numerator multiplies */
-            for (int d = 0; d < D; ++d) acc[d] += pe * vd[(size_t)k * D + d];
+            l += e;
+            for (int d = 0; d < D; ++d) acc[d] += e * vd[(size_t)k * D + d];
           }
           for (int d = 0; d < D; ++d) {
             double v = acc[d] / l;

@@ -88,14 +88,11 @@ void orc_gather_blocks(const orc_geometry* g, const orc_pools* pools, const int3
 void orc_decode_attend(const orc_geometry* g, const orc_pools* pools, const int32_t* table, int32_t stride,
                        const int32_t* seq_len, int32_t n_seqs, const float* q, float softmax_scale,
                        const float* gate, float* out);
-/* q f32 [n_seqs][chunk_len][n_q_heads][D]; out f32 same shape. bf16_operands != 0 rounds the dequantized K and V
- * and the softmax numerators to bf16 before they are multiplied, which is what a bf16 matrix unit sees; the
- * numerators are then 2^(score * log2 e - ceil(max score * log2 e)): with the maximum a whole power of two, an
- * online softmax that rescales by powers of two rounds every numerator exactly as this global form does. The
- * denominator is the sum of the rounded numerators. */
+/* q f32 [n_seqs][chunk_len][n_q_heads][D]; out f32 same shape. Exact arithmetic on the dequantized values: f64 sums,
+ * one global maximum (nothing of a matrix unit's operand rounding is modelled). */
 void orc_prefill_attend(const orc_geometry* g, const orc_pools* pools, const int32_t* table, int32_t stride,
                         const int32_t* prefix_len, int32_t n_seqs, int32_t chunk_len, const float* q,
-                        float softmax_scale, const float* gate, float* out, int32_t bf16_operands);
+                        float softmax_scale, const float* gate, float* out);
 /* worker threads the attend functions use */
 int32_t orc_threads(void);
 /* Checks an identity a kernel may use in place of lround (gguf_quant.cpp:316): for every float r with bit pattern

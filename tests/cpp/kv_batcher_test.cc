@@ -179,7 +179,7 @@ int RunTest() {
           const int32_t pos = w.pos, len = w.pos + w.n;
           orc_append(&m.og, &op, m.table.data(), T / PT, &pos, nullptr, 1, w.n, kf.data(), vf.data());
           if (pre)
-            orc_prefill_attend(&m.og, &op, m.table.data(), T / PT, &pos, 1, w.n, qf.data(), scale, nullptr, want.data(), 1);
+            orc_prefill_attend(&m.og, &op, m.table.data(), T / PT, &pos, 1, w.n, qf.data(), scale, nullptr, want.data());
           else
             orc_decode_attend(&m.og, &op, m.table.data(), T / PT, &len, 1, qf.data(), scale, nullptr, want.data());
           const float* got = pre ? &got_p[size_t(i) * CHUNK * q_row] : &got_d[size_t(i - np) * q_row];

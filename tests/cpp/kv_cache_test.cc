@@ -100,7 +100,7 @@ int RunTest() {
     const orc_pools op{hkq.data(), hks.data(), hvq.data(), hvs.data()};
     orc_append(&og, &op, table.data(), stride, zero.data(), nullptr, B, chunk, kf.data(), vf.data());
     std::vector<float> want(qf.size()), got(qf.size());
-    orc_prefill_attend(&og, &op, table.data(), stride, pre_len.data(), B, chunk, qf.data(), scale, nullptr, want.data(), 1);
+    orc_prefill_attend(&og, &op, table.data(), stride, pre_len.data(), B, chunk, qf.data(), scale, nullptr, want.data());
     CheckHip(hipMemcpy(got.data(), dout.get(), got.size() * 4, hipMemcpyDeviceToHost), "d2h");
     const double e1 = RelErr(got, want);
     Expect(e1 < 2e-3, "prefill attention differs from the oracle");

@@ -228,7 +228,7 @@ def test_length_beyond_the_bound_is_clamped_and_arguments_are_checked(yahkv, tor
                                                          (12, 4, 128, 32, [500, 1000], 70)])
 def test_prefill_over_f16_pools(yahkv, torch_gpu, n_q, n_kv, hd, pt, prefix, chunk):
     """Causal attention of a chunk over prefix + chunk in f16 pools, against the float64 closed form over the f16
-    values; the tiles and the numerators are bf16, so the bound is that of the quantized prefill test, 4 x 2^-9."""
+    values: the pools' values reach the matrix unit as they are, the numerators are f16; bound 2e-3."""
     torch = torch_gpu
     rng = np.random.default_rng(hd + pt + chunk)
     B = len(prefix)
@@ -260,7 +260,7 @@ def test_prefill_over_f16_pools(yahkv, torch_gpu, n_q, n_kv, hd, pt, prefix, chu
             n = prefix[s] + t + 1
             want = closed_form(K[:n], V[:n], q[s, t], scale, n_q)
             worst = max(worst, float(np.abs(out[s, t] - want).max() / np.abs(want).max()))
-    assert worst < 4 * 2.0 ** -9, worst
+    assert worst < 2e-3, worst
 
 
 def test_prefill_over_f16_pools_checks_its_arguments(yahkv, torch_gpu):

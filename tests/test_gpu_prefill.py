@@ -1,7 +1,6 @@
-"""GPU chunked-prefill attention against the CPU oracle that models the bf16 operands of the matrix unit (K, V and the
-softmax numerators rounded to bf16, f32 sums): tolerance 2e-3 max relative error, max |got - want| / max |want|. The
-error against the exact closed form on the dequantized K / V is reported and bounded more loosely: bf16 operands
-alone carry 2^-9 relative error each, which short contexts do not average out."""
+"""GPU chunked-prefill attention against the CPU oracle's exact arithmetic on the dequantized K / V (f64 sums, nothing
+of the matrix unit's operand rounding modelled): tolerance 2e-3 max relative error, max |got - want| / max |want|. The
+kernels feed the matrix unit f16 keys, values and numerators (2^-12 relative each); measured 2e-4 .. 5e-4."""
 import numpy as np
 import pytest
 
@@ -36,7 +35,7 @@ def build(yahkv, torch, fmt, n_q, n_kv, hd, pt, prefix, chunk, seed, fill=0):
     return g, table, host, dev, t_table, rng, to_t
 
 
-# path "images": decode to bf16 tile images in a workspace, then attention; "fused": one kernel, no workspace (q8_0)
+# path "images": decode to f16 tile images in a workspace, then attention; "fused": one kernel, no workspace (q8_0)
 @pytest.mark.parametrize("path,fmt,n_q,n_kv,hd,pt,prefix,chunk", [
     ("images", 8, 24, 4, 256, 64, [100, 0, 64 * 3 + 5], 70),
     ("images", 8, 24, 4, 256, 64, [1000], 256),
@@ -69,14 +68,17 @@ def test_prefill_against_oracle(yahkv, torch_gpu, path, fmt, n_q, n_kv, hd, pt, 
         torch.cuda.synchronize()
         got = out.cpu().numpy()
         assert np.all(np.isfinite(got))
-        want = oracle.prefill_attend(host, table, prefix, q, scale, gt, bf16_operands=True)
-        assert rel_err(got, want) < TOL
         exact = oracle.prefill_attend(host, table, prefix, q, scale, gt)
-        assert rel_err(got, exact) < 3 * 2.0 ** -9
-    # bf16 output: the same numbers rounded once more
+        assert rel_err(got, exact) < 1e-3                        # half the tolerance: measured 2e-4 .. 5e-4
+    exact = oracle.prefill_attend(host, table, prefix, q, scale, None)
+    # f16 output (what the reference's kernel writes, gen_attn_fa.py:1589-1595): the same numbers rounded once more
+    out16 = yahkv.prefill_attend(dev, t_table, t_prefix, max(prefix), to_t(q), scale, out_dtype=torch.float16,
+                                 workspace=ws)
+    assert rel_err(out16.float().cpu().numpy(), exact) < TOL
+    # bf16 output: its own rounding, 2^-9 of the largest element, comes on top
     out16 = yahkv.prefill_attend(dev, t_table, t_prefix, max(prefix), to_t(q), scale, out_dtype=torch.bfloat16,
                                  workspace=ws)
-    assert rel_err(out16.float().cpu().numpy(), oracle.prefill_attend(host, table, prefix, q, scale, None, True)) < 2 * 2.0 ** -9
+    assert rel_err(out16.float().cpu().numpy(), exact) < 1e-3 + 2.0 ** -9
 
 
 @pytest.mark.parametrize("ws", [None, False], ids=["images", "fused"])
@@ -91,20 +93,21 @@ def test_prefill_special_cases(yahkv, torch_gpu, ws):
     got = yahkv.prefill_attend(dev, t_table, t_prefix, 77, to_t(q), 0.0625, workspace=ws).cpu().numpy()
     (ks, kc), (vs, vc) = logical_blocks(host.arrays(), g, table[0], chunk)
     Kd, Vd = dequant(ks, kc), dequant(vs, vc)
-    assert rel_err(got[0, 0], np.repeat(to_bf16_f32(Vd[0]), 6, 0)) < 1e-6       # one visible key: out = bf16(V row)
+    v16 = Vd[0].astype(np.float16).astype(np.float32)
+    assert rel_err(got[0, 0], np.repeat(v16, 6, 0)) < 1e-6                       # one visible key: out = f16(V row)
     for t in (1, 17, chunk - 1):
-        assert rel_err(got[0, t], closed_form(Kd[:t + 1], Vd[:t + 1], q[0, t], 0.0625)) < 3 * 2.0 ** -9
+        assert rel_err(got[0, t], closed_form(Kd[:t + 1], Vd[:t + 1], q[0, t], 0.0625)) < TOL
     lens = [p + chunk for p in prefix]
     one = yahkv.prefill_attend(dev, t_table, torch.tensor([l - 1 for l in lens], dtype=torch.int32, device="cuda"),
                                max(lens), to_t(q[:, -1:]), 0.0625, workspace=ws).cpu().numpy()
     dec = yahkv.decode_attend(dev, t_table, torch.tensor(lens, dtype=torch.int32, device="cuda"), max(lens),
                               to_t(q[:, -1]), 0.0625).cpu().numpy()
-    assert rel_err(one[:, 0], dec) < 3 * 2.0 ** -9
+    assert rel_err(one[:, 0], dec) < TOL
     assert rel_err(one[:, 0], got[:, -1]) < 1e-6                                 # same query, same keys, same kernel
 
 
 def test_both_paths_agree(yahkv, torch_gpu):
-    """The two paths feed the matrix unit the same bf16 values; only the order of the f32 sums differs."""
+    """The two paths feed the matrix unit the same f16 values; only the order of the f32 sums differs."""
     torch = torch_gpu
     prefix, chunk = [300, 5], 100
     g, table, host, dev, t_table, rng, to_t = build(yahkv, torch, 8, 24, 4, 256, 64, prefix, chunk, seed=6)
@@ -112,7 +115,7 @@ def test_both_paths_agree(yahkv, torch_gpu):
     t_prefix = torch.tensor(prefix, dtype=torch.int32, device="cuda")
     a = yahkv.prefill_attend(dev, t_table, t_prefix, 300, q, 0.0625).cpu().numpy()
     b = yahkv.prefill_attend(dev, t_table, t_prefix, 300, q, 0.0625, workspace=False).cpu().numpy()
-    assert rel_err(a, b) < 1e-3
+    assert rel_err(a, b) < 2e-4
     ws = torch.empty(yahkv.prefill_workspace_bytes(dev.geom, 2, 400, chunk), dtype=torch.uint8, device="cuda")
     c = yahkv.prefill_attend(dev, t_table, t_prefix, 400, q, 0.0625, workspace=ws).cpu().numpy()   # a looser bound
     assert np.array_equal(a, c)
@@ -140,11 +143,12 @@ def test_prefill_rejects_bad_arguments(yahkv, torch_gpu):
     rc = yahkv.lib.yahkv_prefill_attend(C.byref(g8), C.byref(st), None, 4, None, 1, 0, 8, None, 0.0625, None, None, 0,
                                         None, 0, None)
     assert rc == -1
-    # a kv head's tile images beyond 2 GiB (prefix + chunk past 2^21 tokens at head_dim 256): refused before any launch
-    # (the workspace is not touched, so its claimed size need not be real)
+    # a kv head's tile images beyond 2 GiB (prefix + chunk past 2^21 tokens at head_dim 256): refused as a shape, before
+    # the workspace's size is even looked at (the size given is the buffer's real one: were the refusal missing, the
+    # answer would be "workspace too small", never a launch)
     out = torch.empty(q.shape, dtype=torch.bfloat16, device="cuda")
     small = torch.empty(4096, dtype=torch.uint8, device="cuda")
     rc = yahkv.lib.yahkv_prefill_attend_tiles(C.byref(g8), C.byref(st), table.data_ptr(), 4, zero.data_ptr(), 1, 1 << 21, 8,
-                                              q.data_ptr(), 0.0625, None, out.data_ptr(), 2, small.data_ptr(), 1 << 50,
+                                              q.data_ptr(), 0.0625, None, out.data_ptr(), 2, small.data_ptr(), 4096,
                                               None)
     assert rc == -2

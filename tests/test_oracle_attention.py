@@ -188,6 +188,3 @@ def test_prefill_against_closed_form_and_decode(fmt):
     one = oracle.prefill_attend(pools, table, [l - 1 for l in lens], q[:, -1:], scale, gate[:, -1:])
     dec = oracle.decode_attend(pools, table, lens, q[:, -1], scale, gate[:, -1])
     assert rel_err(one[:, 0], dec) < 3e-6
-    # bf16 operand rounding: each of K, V and P carries 2^-9 relative error, which short contexts do not average out
-    b16 = oracle.prefill_attend(pools, table, prefix, q, scale, gate, bf16_operands=True)
-    assert 0 < rel_err(b16, got) < 3 * 2.0 ** -9

@@ -261,13 +261,13 @@ def f16_decode_attend(pools, table, seq_len, max_seq_len, q, scale, gate=None, o
 
 
 def f16_prefill_attend(pools, table, prefix_len, max_prefix_len, q, scale, gate=None, out=None, workspace=None):
-    """prefill_attend() over f16 pools; q bf16 [n_seqs][chunk][n_q_heads][D]; returns out (bf16 unless given)."""
+    """prefill_attend() over f16 pools; q bf16 [n_seqs][chunk][n_q_heads][D]; returns out (f16 unless given)."""
     import torch
     g = pools.geom
     n_seqs, chunk = q.shape[0], q.shape[1]
     assert q.is_contiguous() and q.dtype == torch.bfloat16 and tuple(q.shape[2:]) == (g.n_q_heads, g.head_dim)
     if out is None:
-        out = torch.empty(q.shape, dtype=torch.bfloat16, device=q.device)
+        out = torch.empty(q.shape, dtype=torch.float16, device=q.device)
     if workspace is None:
         need = lib.yahkv_f16_prefill_workspace_bytes(C.byref(g), n_seqs, max_prefix_len, chunk)
         workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=q.device)

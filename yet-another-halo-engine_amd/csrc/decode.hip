@@ -844,15 +844,30 @@ Plan MakePlan(const Geom& g, int32_t n_seqs, int32_t max_seq_len, const Tuning& 
   p.min_chunk_tiles = t.min_chunk_tiles, p.pair_cost = t.pair_cost;
   p.n_chunks =
       static_cast<int32_t>(std::min<int64_t>(t.n_chunks, (line_max + p.min_chunk_tiles - 1) / p.min_chunk_tiles));
-  // Shares of the eight chunks of a group: by the caller's relative XCD speeds (yahkv_decode_calibrate measures them),
-  // equal without them. Every share keeps at least 1 / 16 of the group, which at two line units per chunk is one unit:
-  // no chunk inside a pair's stretch comes out empty.
-  int64_t w[8], sum = 0;
+  // Shares of the eight chunks of a group: proportional to the caller's relative XCD speeds (yahkv_decode_calibrate
+  // measures them), equal without them. No share falls below 1 / 16 of the group, which at two line units per chunk is
+  // one unit: no chunk inside a pair's stretch comes out empty. (Shares below that bound are raised to it and the rest
+  // is dealt out again among the others.)
+  double w[8], share[8];
+  double sum = 0;
   for (int j = 0; j < 8; ++j) w[j] = t.xcd_weight[j], sum += w[j];
   // (a last group that is not whole would leave the line's end uncovered: equal shares then)
-  if (sum == 0 || p.n_chunks % 8 != 0) std::fill(w, w + 8, int64_t(1)), sum = 8;
+  if (sum <= 0 || p.n_chunks % 8 != 0) std::fill(w, w + 8, 1.0);
+  bool low[8] = {false, false, false, false, false, false, false, false};
+  for (int round = 0; round < 8; ++round) {
+    double free_sum = 0, left = 8192;
+    for (int j = 0; j < 8; ++j) low[j] ? left -= 512 : free_sum += w[j];
+    bool again = false;
+    for (int j = 0; j < 8; ++j) {
+      share[j] = low[j] || free_sum <= 0 ? 512 : w[j] * left / free_sum;
+      if (share[j] < 512) low[j] = again = true;
+    }
+    if (!again) break;
+  }
   p.share[0] = 0;
-  for (int j = 0; j < 8; ++j) p.share[j + 1] = p.share[j] + 512 + static_cast<int32_t>(w[j] * (8192 - 8 * 512) / sum);
+  for (int j = 0; j < 8; ++j) p.share[j + 1] = p.share[j] + std::max(512, static_cast<int32_t>(share[j]));
+  // rounding leaves a few 8192ths over or short: the last chunks take them, none going below its bound
+  for (int j = 8, over = p.share[8] - 8192; j >= 1; --j) p.share[j] = std::min(p.share[j] - over, 8192 - 512 * (8 - j));
   p.share[8] = 8192;
   const size_t parts = (size_t(p.n_chunks) + size_t(n_seqs) * g.n_kv) * p.wpc;
   p.off_tprefix = 0;
@@ -977,11 +992,13 @@ extern "C" int yahkv_decode_attend(const yahkv_geometry* g, const yahkv_pools* p
                              workspace_bytes, opt, stream);
 }
 
+constexpr int kCalibrationLaunches = 4;  // measured launches per round of yahkv_decode_calibrate
+
 // Relative read speeds of the eight XCDs on the caller's own batch. Workgroup k of a dispatch runs on XCD k % 8, and the
 // XCDs of one GPU do not read memory equally fast (up to 10 % apart, measured); chunk shares that follow their speeds
-// let all workgroups finish together. Each round runs the part kernel twice with the current shares (the first launch
-// warms caches and clocks), reads when each workgroup's last wave finished, and sets every XCD's weight to its share
-// divided by its mean time. Synchronizes the stream: a set-up call, not part of a step.
+// let all workgroups finish together. Each round runs the part kernel five times with the current shares (the first
+// launch warms caches and clocks), reads when each workgroup's last wave finished, and sets every XCD's weight to its
+// share divided by its mean time over the four measured launches. Synchronizes the stream: a set-up call, not part of a step.
 extern "C" int yahkv_decode_calibrate(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
                                       int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs,
                                       int32_t max_seq_len, const void* q, int32_t q_dtype, void* workspace,
@@ -1000,21 +1017,22 @@ extern "C" int yahkv_decode_calibrate(const yahkv_geometry* g, const yahkv_pools
     a.stamps = reinterpret_cast<unsigned long long*>(static_cast<char*>(workspace) + p.off_stamps);
     const size_t n = 2 * size_t(a.n_chunks);  // [0, n_chunks): start of each workgroup, [n_chunks, ..): its end
     std::vector<unsigned long long> stamps(n);
-    for (int pass = 0; pass < 2; ++pass) {
-      if (hipMemsetAsync(a.stamps, 0, n * sizeof(unsigned long long), st) != hipSuccess) return YAHKV_ERR_LAUNCH;
-      if (const int rc = LaunchPart(a, st)) return rc;
-    }
-    if (hipMemcpyAsync(stamps.data(), a.stamps, n * sizeof(unsigned long long), hipMemcpyDeviceToHost, st) != hipSuccess ||
-        hipStreamSynchronize(st) != hipSuccess)
-      return YAHKV_ERR_LAUNCH;
-    unsigned long long start = ~0ull;
-    for (int k = 0; k < a.n_chunks; ++k)
-      if (stamps[size_t(k)] != 0) start = std::min(start, stamps[size_t(k)]);
     double t[8] = {0, 0, 0, 0, 0, 0, 0, 0};
     int cnt[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    for (int k = 0; k < a.n_chunks; ++k) {
-      const unsigned long long end = stamps[size_t(a.n_chunks) + size_t(k)];
-      if (end > start) t[k % 8] += double(end - start), ++cnt[k % 8];
+    for (int pass = 0; pass < 1 + kCalibrationLaunches; ++pass) {  // the first launch warms caches and clocks
+      if (hipMemsetAsync(a.stamps, 0, n * sizeof(unsigned long long), st) != hipSuccess) return YAHKV_ERR_LAUNCH;
+      if (const int rc = LaunchPart(a, st)) return rc;
+      if (pass == 0) continue;
+      if (hipMemcpyAsync(stamps.data(), a.stamps, n * sizeof(unsigned long long), hipMemcpyDeviceToHost, st) != hipSuccess ||
+          hipStreamSynchronize(st) != hipSuccess)
+        return YAHKV_ERR_LAUNCH;
+      unsigned long long start = ~0ull;
+      for (int k = 0; k < a.n_chunks; ++k)
+        if (stamps[size_t(k)] != 0) start = std::min(start, stamps[size_t(k)]);
+      for (int k = 0; k < a.n_chunks; ++k) {
+        const unsigned long long end = stamps[size_t(a.n_chunks) + size_t(k)];
+        if (end > start) t[k % 8] += double(end - start), ++cnt[k % 8];
+      }
     }
     double speed[8], top = 0;
     for (int j = 0; j < 8; ++j) {

@@ -1,14 +1,18 @@
-// Chunked-prefill attention over the paged, block-quantized prefix: a FlashAttention-style kernel on bf16 MFMA.
+// Chunked-prefill attention over the paged, block-quantized prefix: a FlashAttention-style kernel on 16-bit MFMA.
 //
 // Semantics follow the reference's prefill attention (engine/gpu/loom/tools/gen_attn_fa.py:1-21, launch signature
 // :1589-1595): query t of the chunk sees keys 0 .. prefix + t, which the caller has already appended to the pools;
 // online softmax in base 2 (:1614), output o / l, times sigmoid(gate) if a gate is given (:4230). Quantized K / V are
-// decoded while they are staged into LDS (:2664-2779), here to bf16: value = bf16(d * code), round to nearest even.
+// decoded while they are staged into LDS (:2664-2779) to f16, as the reference's kernel computes in f16 (:1252-1595):
+// value = f16(d * code), round to nearest even, saturated at the largest finite f16 (d * code can reach 65504 * 127).
+// The chunk's bf16 queries become f16 the same way (exact in the normal f16 range), and so do the softmax numerators.
+// f16 and bf16 run at the same MFMA rate; f16's three more mantissa bits are what brings the result within 2e-3 of
+// exact arithmetic on 18K keys (bf16 keys alone cost 1.5e-3 there).
 //
 // Shape of the computation (everything is transposed so that keys run along MFMA rows and queries along lanes):
 //   S^T[key][q] = sum_dim K[key][dim] Q[q][dim]     A = K tile from LDS (16 keys x 32 dims), B = Q^T (registers)
 //   O^T[dim][q] += sum_key V^T[dim][key] P^T[key][q]  A = V^T tile from LDS (16 dims x 32 keys), B = P^T (registers)
-// v_mfma_f32_16x16x32_bf16 leaves S^T with one query per lane and keys down the registers, which is exactly the
+// v_mfma_f32_16x16x32_f16 leaves S^T with one query per lane and keys down the registers, which is exactly the
 // B-operand shape of the second product: P never leaves the registers, the row maximum needs two cross-lane steps, and
 // the rescaling factor of a lane's accumulators is the lane's own.
 // A workgroup (4 waves) owns 64 consecutive chunk positions of one sequence for two query heads of one kv head: eight
@@ -26,7 +30,12 @@ constexpr int kQueries = 64; // chunk positions per workgroup
 constexpr int kFusedRowBlocks = 2;  // row blocks (16 queries of one head) per wave of the one-pass kernel
 constexpr float kNegBig = -3.4028234663852886e+38f;
 
-typedef __bf16 b8v __attribute__((ext_vector_type(8)));
+typedef _Float16 h8v __attribute__((ext_vector_type(8)));
+// The softmax numerators are 2^(score - m) with a reference point m that sits kBias below the (rounded-up) largest
+// score seen when it was set and is moved when a score exceeds it by more than kBias + kSlack: the numerators then
+// stay below 2^(kBias + kSlack), well inside f16's range, while a numerator 2^-24 of the largest is still a normal
+// f16. Numerators and denominators carry the same factor, so it cancels.
+constexpr float kBias = 10.0f, kSlack = 4.0f;
 typedef float f4v __attribute__((ext_vector_type(4)));
 
 struct PrefillArgs {
@@ -43,8 +52,25 @@ struct PrefillArgs {
   int32_t out_dtype;
 };
 
-__device__ __forceinline__ b8v OnesBf16() {  // 1.0 in all eight slots
-  return __builtin_bit_cast(b8v, uint4{0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u});
+__device__ __forceinline__ h8v OnesF16() {  // 1.0 in all eight slots
+  return __builtin_bit_cast(h8v, uint4{0x3C003C00u, 0x3C003C00u, 0x3C003C00u, 0x3C003C00u});
+}
+typedef _Float16 h2v __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t PackF16(float a, float b) {  // round to nearest even (one v_cvt_pk_f16_f32)
+  const h2v v = {static_cast<_Float16>(a), static_cast<_Float16>(b)};
+  return __builtin_bit_cast(uint32_t, v);
+}
+// For K and V values: finite values beyond the f16 range saturate at +-65504 (NaN stays NaN).
+__device__ __forceinline__ float ClampF16(float x) { return __builtin_fminf(__builtin_fmaxf(x, -65504.0f), 65504.0f) + (x - x); }
+__device__ __forceinline__ uint32_t PackF16Sat(float a, float b) { return PackF16(ClampF16(a), ClampF16(b)); }
+// Eight bf16 query elements as f16.
+__device__ __forceinline__ h8v QueryF16(const uint16_t* p) {
+  const uint4 w = *reinterpret_cast<const uint4*>(p);
+  const uint32_t u[4] = {w.x, w.y, w.z, w.w};
+  uint32_t o[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) o[e] = PackF16Sat(WidenBf16(static_cast<uint16_t>(u[e] & 0xFFFF)), WidenBf16(static_cast<uint16_t>(u[e] >> 16)));
+  return __builtin_bit_cast(h8v, uint4{o[0], o[1], o[2], o[3]});
 }
 __device__ __forceinline__ uint32_t PackBf16(float a, float b) {  // round to nearest even
   typedef __bf16 b2v __attribute__((ext_vector_type(2)));
@@ -52,7 +78,7 @@ __device__ __forceinline__ uint32_t PackBf16(float a, float b) {  // round to ne
   return __builtin_bit_cast(uint32_t, v);
 }
 
-// Sixteen int8 codes times one scale, as sixteen bf16 (two 16-byte halves).
+// Sixteen int8 codes times one scale, as sixteen f16 (two 16-byte halves).
 __device__ __forceinline__ void Decode16(const uint4 c, float d, uint4* lo, uint4* hi) {
   const uint32_t w[4] = {c.x ^ 0x80808080u, c.y ^ 0x80808080u, c.z ^ 0x80808080u, c.w ^ 0x80808080u};
   const float off = -128.0f * d;
@@ -63,7 +89,7 @@ __device__ __forceinline__ void Decode16(const uint4 c, float d, uint4* lo, uint
     const float f1 = __builtin_fmaf(static_cast<float>((w[i] >> 8) & 0xFF), d, off);
     const float f2 = __builtin_fmaf(static_cast<float>((w[i] >> 16) & 0xFF), d, off);
     const float f3 = __builtin_fmaf(static_cast<float>(w[i] >> 24), d, off);
-    o[2 * i] = PackBf16(f0, f1), o[2 * i + 1] = PackBf16(f2, f3);
+    o[2 * i] = PackF16Sat(f0, f1), o[2 * i + 1] = PackF16Sat(f2, f3);
   }
   *lo = uint4{o[0], o[1], o[2], o[3]}, *hi = uint4{o[4], o[5], o[6], o[7]};
 }
@@ -76,14 +102,14 @@ __device__ __forceinline__ void Decode16V(const uint4 c, const uint4 s0, const u
   for (int i = 0; i < 8; ++i) {
     const float d0 = WidenF16(static_cast<uint16_t>(sw[i] & 0xFFFF)), d1 = WidenF16(static_cast<uint16_t>(sw[i] >> 16));
     const uint32_t b0 = (w[i / 2] >> (16 * (i % 2))) & 0xFF, b1 = (w[i / 2] >> (16 * (i % 2) + 8)) & 0xFF;
-    o[i] = PackBf16(__builtin_fmaf(static_cast<float>(b0), d0, -128.0f * d0),
-                    __builtin_fmaf(static_cast<float>(b1), d1, -128.0f * d1));
+    o[i] = PackF16Sat(__builtin_fmaf(static_cast<float>(b0), d0, -128.0f * d0),
+                      __builtin_fmaf(static_cast<float>(b1), d1, -128.0f * d1));
   }
   *lo = uint4{o[0], o[1], o[2], o[3]}, *hi = uint4{o[4], o[5], o[6], o[7]};
 }
 
 // out = o / l (* sigmoid(gate)); lane (query, lane group jg) holds dims 16 dt + 4 jg + r of its query in each row block.
-// The denominators l are the sums of the bf16 numerators, accumulated by the matrix unit against an all-ones operand
+// The denominators l are the sums of the f16 numerators, accumulated by the matrix unit against an all-ones operand
 // next to V^T: numerators and denominator then carry the same rounding, and a lone key returns its V row exactly.
 template <int D, int RB>
 __device__ __forceinline__ void StoreRows(const PrefillArgs& a, int s, int h, int G, int jg, const f4v (&o)[RB][D / 16],
@@ -123,7 +149,7 @@ template <int D, int PT>
 __global__ __launch_bounds__(256) void PrefillAttendQ8(const PrefillArgs a) {
   constexpr int NB = D / 32, NDT = D / 16, KS = D / 32;  // blocks, 16-dim tiles, 32-dim steps of the first product
   constexpr int RB = kFusedRowBlocks, kHeadsPerGroup = RB;  // 4 waves x RB row blocks = 64 positions x RB heads
-  constexpr int KSTR = D + 8, VSTR = kKeys + 8;          // LDS row strides (bf16), padded against bank conflicts
+  constexpr int KSTR = D + 8, VSTR = kKeys + 8;          // LDS row strides (f16), padded against bank conflicts
   constexpr int KCH = kKeys * D / 16 / 256;              // 16-code chunks of a tile per thread
   const Geom g = a.g;
   const int G = g.group(), H = g.n_kv;
@@ -141,12 +167,12 @@ __global__ __launch_bounds__(256) void PrefillAttendQ8(const PrefillArgs a) {
   const int n_keys = min(prefix + q0 + kQueries, prefix + a.chunk_len);
   const int n_tiles = (n_keys + kKeys - 1) / kKeys;
 
-  __shared__ __align__(16) __bf16 lk[kKeys][KSTR];  // K tile, [key][dim]
-  __shared__ __align__(16) __bf16 lv[D][VSTR];      // V^T tile, [dim][key]
+  __shared__ __align__(16) _Float16 lk[kKeys][KSTR];  // K tile, [key][dim]
+  __shared__ __align__(16) _Float16 lv[D][VSTR];      // V^T tile, [dim][key]
   __shared__ __align__(16) uint16_t lvs[NB][kKeys]; // V scales of the tile (f16 bits), [block][key]
 
   // ---- this wave's row blocks: rb = RB * wave + i -> head 2 hp + rb / 4, queries q0 + 16 (rb % 4) + 0..15
-  b8v qb[RB][KS];
+  h8v qb[RB][KS];
   int qpos[RB];   // chunk position of this lane's query in block i (may be >= chunk_len: then it is never stored)
   int head[RB];   // head within the group (may be >= G: then the block is never stored)
 #pragma unroll
@@ -157,7 +183,7 @@ __global__ __launch_bounds__(256) void PrefillAttendQ8(const PrefillArgs a) {
     const int t = min(qpos[i], a.chunk_len - 1), hd = min(head[i], G - 1);
     const uint16_t* qp = a.q + ((size_t(s) * a.chunk_len + t) * g.n_q + size_t(h) * G + hd) * D;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) qb[i][ks] = *reinterpret_cast<const b8v*>(qp + 32 * ks + 8 * jg);
+    for (int ks = 0; ks < KS; ++ks) qb[i][ks] = QueryF16(qp + 32 * ks + 8 * jg);
   }
   f4v o[RB][NDT];
   float m[RB];
@@ -251,21 +277,21 @@ __global__ __launch_bounds__(256) void PrefillAttendQ8(const PrefillArgs a) {
     {
       // A operands are read one 32-dim step ahead of the products that use them; the scheduling groups spread the
       // vector work of the V decode between the matrix instructions (one wave per SIMD: nothing else hides latency).
-      b8v ka[2][4];
+      h8v ka[2][4];
 #pragma unroll
-      for (int kt = 0; kt < 4; ++kt) ka[0][kt] = *reinterpret_cast<const b8v*>(&lk[16 * kt + qn][8 * jg]);
+      for (int kt = 0; kt < 4; ++kt) ka[0][kt] = *reinterpret_cast<const h8v*>(&lk[16 * kt + qn][8 * jg]);
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
         if (ks + 1 < KS) {
 #pragma unroll
           for (int kt = 0; kt < 4; ++kt)
-            ka[(ks + 1) % 2][kt] = *reinterpret_cast<const b8v*>(&lk[16 * kt + qn][32 * (ks + 1) + 8 * jg]);
+            ka[(ks + 1) % 2][kt] = *reinterpret_cast<const h8v*>(&lk[16 * kt + qn][32 * (ks + 1) + 8 * jg]);
         }
 #pragma unroll
         for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
           for (int i = 0; i < RB; ++i)
-            st[i][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[ks % 2][kt], qb[i][ks], st[i][kt], 0, 0, 0);
+            st[i][kt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[ks % 2][kt], qb[i][ks], st[i][kt], 0, 0, 0);
         if (ks % (KS / KCH) == KS / KCH - 1) {
           stage_v(ks / (KS / KCH));
 #pragma unroll
@@ -298,7 +324,7 @@ __global__ __launch_bounds__(256) void PrefillAttendQ8(const PrefillArgs a) {
       mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
       // The running maximum moves in whole powers of two: rescaling is then exact, so the result does not depend on
       // the order in which the maximum was met (and it moves less often).
-      const float mn = fmaxf(m[i], __builtin_ceilf(mx));
+      const float mn = fmaxf(m[i], __builtin_ceilf(mx) - kBias);
       const float alpha = __builtin_amdgcn_exp2f(m[i] - mn);
       m[i] = mn;
 #pragma unroll
@@ -307,8 +333,8 @@ __global__ __launch_bounds__(256) void PrefillAttendQ8(const PrefillArgs a) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) p[r] = __builtin_amdgcn_exp2f(st[i][kt][r] - mn);
         // step kt / 2 takes keys 32 (kt / 2) + {4 jg + r} from its even tile and + 16 + {4 jg + r} from its odd one
-        pb[i][kt / 2][2 * (kt % 2)] = PackBf16(p[0], p[1]);
-        pb[i][kt / 2][2 * (kt % 2) + 1] = PackBf16(p[2], p[3]);
+        pb[i][kt / 2][2 * (kt % 2)] = PackF16(p[0], p[1]);
+        pb[i][kt / 2][2 * (kt % 2) + 1] = PackF16(p[2], p[3]);
       }
       if (alpha != 1.0f) {
 #pragma unroll
@@ -322,25 +348,25 @@ __global__ __launch_bounds__(256) void PrefillAttendQ8(const PrefillArgs a) {
     __syncthreads();  // every wave is done with lk, and V(tile) is complete in lv
     // ---- O^T += V^T P^T; the A operand's key slots follow pb: 4 keys at 32 s2 + 4 jg, 4 at 32 s2 + 16 + 4 jg
     {
-      auto read_v = [&](int dt, int s2) -> b8v {
+      auto read_v = [&](int dt, int s2) -> h8v {
         const uint2 v0 = *reinterpret_cast<const uint2*>(&lv[16 * dt + qn][32 * s2 + 4 * jg]);
         const uint2 v1 = *reinterpret_cast<const uint2*>(&lv[16 * dt + qn][32 * s2 + 16 + 4 * jg]);
-        return __builtin_bit_cast(b8v, uint4{v0.x, v0.y, v1.x, v1.y});
+        return __builtin_bit_cast(h8v, uint4{v0.x, v0.y, v1.x, v1.y});
       };
-      b8v pv[RB][2];
+      h8v pv[RB][2];
 #pragma unroll
       for (int i = 0; i < RB; ++i)
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2)
-          pv[i][s2] = __builtin_bit_cast(b8v, uint4{pb[i][s2][0], pb[i][s2][1], pb[i][s2][2], pb[i][s2][3]});
-      b8v va[3][2];  // read two 16-dim tiles ahead
+          pv[i][s2] = __builtin_bit_cast(h8v, uint4{pb[i][s2][0], pb[i][s2][1], pb[i][s2][2], pb[i][s2][3]});
+      h8v va[3][2];  // read two 16-dim tiles ahead
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2) va[0][s2] = read_v(0, s2), va[1][s2] = read_v(1, s2);
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
         for (int i = 0; i < RB; ++i)
-          lacc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(OnesBf16(), pv[i][s2], lacc[i], 0, 0, 0);
+          lacc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(OnesF16(), pv[i][s2], lacc[i], 0, 0, 0);
 #pragma unroll
       for (int dt = 0; dt < NDT; ++dt) {
         if (dt + 2 < NDT) {
@@ -351,7 +377,7 @@ __global__ __launch_bounds__(256) void PrefillAttendQ8(const PrefillArgs a) {
         for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
           for (int i = 0; i < RB; ++i)
-            o[i][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[dt % 3][s2], pv[i][s2], o[i][dt], 0, 0, 0);
+            o[i][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va[dt % 3][s2], pv[i][s2], o[i][dt], 0, 0, 0);
         if (dt % (NDT / KCH) == NDT / KCH - 1) {
           stage_k(dt / (NDT / KCH));  // K(tile + 1), or stale bytes after the last tile
 #pragma unroll
@@ -380,11 +406,11 @@ __global__ __launch_bounds__(256) void PrefillAttendQ8(const PrefillArgs a) {
 // vector instructions and the matrix instructions compete for the wave's issue slots. When the caller provides a
 // workspace, the prefix is decoded once per call instead (the reference does the same: yah_kdeq8 / yah_vdeq8 into an
 // f16 pool before yah_attn_wmma, gen_attn_fa.py:4648-4861): `PrefillImages` writes, per (sequence, kv head, tile of
-// 64 keys), the bf16 K tile and V^T tile exactly as the attention kernel wants them in LDS, and `PrefillAttendImg`
+// 64 keys), the f16 K tile and V^T tile exactly as the attention kernel wants them in LDS, and `PrefillAttendImg`
 // copies images to LDS with direct global-to-LDS loads (no registers, no vector instructions) one tile ahead.
 //
-// K image: 64 rows (keys) of D bf16; the 16-byte chunk c of row r sits at chunk position c ^ (r % 8).
-// V image: D rows (dims) of 64 bf16; chunk c = 4 s2 + jg of row r holds keys 32 s2 + 4 jg + 0..3 and 32 s2 + 16 +
+// K image: 64 rows (keys) of D f16; the 16-byte chunk c of row r sits at chunk position c ^ (r % 8).
+// V image: D rows (dims) of 64 f16; chunk c = 4 s2 + jg of row r holds keys 32 s2 + 4 jg + 0..3 and 32 s2 + 16 +
 // 4 jg + 0..3 (the eight k-slots of lane group jg in step s2 of the second product) and sits at position c ^ (r % 8).
 // With the XOR, the sixteen rows a wave reads at once fall into different banks. Keys at or past the end of the
 // sequence are zero in both images.
@@ -443,7 +469,7 @@ __global__ __launch_bounds__(256) void PrefillImages(const ImageArgs a) {
           v[e] = d * static_cast<float>(int((((e < 4 ? w.x : w.y) >> (8 * (e % 4))) >> (off / 16 * 4)) & 0xF) - 8);
       }
 #pragma unroll
-      for (int e = 0; e < 4; ++e) o[e] = PackBf16(v[2 * e], v[2 * e + 1]);
+      for (int e = 0; e < 4; ++e) o[e] = PackF16Sat(v[2 * e], v[2 * e + 1]);
     }
     *reinterpret_cast<uint4*>(kimg + size_t(p) * 16) = uint4{o[0], o[1], o[2], o[3]};
   }
@@ -473,14 +499,14 @@ __global__ __launch_bounds__(256) void PrefillImages(const ImageArgs a) {
                               : static_cast<float>(int((byte >> shift) & 0xF) - 8);
         v[e] = kk + e < n_keys ? d * code : 0.0f;
       }
-      o[2 * hf] = PackBf16(v[0], v[1]), o[2 * hf + 1] = PackBf16(v[2], v[3]);
+      o[2 * hf] = PackF16Sat(v[0], v[1]), o[2 * hf + 1] = PackF16Sat(v[2], v[3]);
     }
     *reinterpret_cast<uint4*>(vimg + size_t(p) * 16) = uint4{o[0], o[1], o[2], o[3]};
   }
 }
 
-// The same images from unquantized f16 pools (the pools of yahkv_f16_append): a conversion f16 -> bf16, round to
-// nearest even, instead of a decode.
+// The same images from unquantized f16 pools (the pools of yahkv_f16_append): the pools' own f16 values, moved into
+// the images' order.
 template <int D, int PT>
 __global__ __launch_bounds__(256) void PrefillImagesF16(const ImageArgs a) {
   constexpr int CPR = D / 8;  // 16-byte chunks per K row
@@ -500,10 +526,7 @@ __global__ __launch_bounds__(256) void PrefillImagesF16(const ImageArgs a) {
     if (kk < n_keys) {
       const uint4 w = *reinterpret_cast<const uint4*>(a.fk + page_head(kk) * (size_t(D) * PT) +
                                                       (size_t(c / 2) * PT + kk % PT) * 16 + (c % 2) * 8);
-      const uint32_t u[4] = {w.x, w.y, w.z, w.w};
-#pragma unroll
-      for (int e = 0; e < 4; ++e)
-        o[e] = PackBf16(WidenF16(static_cast<uint16_t>(u[e] & 0xFFFF)), WidenF16(static_cast<uint16_t>(u[e] >> 16)));
+      o[0] = w.x, o[1] = w.y, o[2] = w.z, o[3] = w.w;
     }
     *reinterpret_cast<uint4*>(kimg + size_t(p) * 16) = uint4{o[0], o[1], o[2], o[3]};
   }
@@ -516,12 +539,11 @@ __global__ __launch_bounds__(256) void PrefillImagesF16(const ImageArgs a) {
       constexpr int RUN = PT < 32 ? PT : 32;  // V^T lies in runs of at most 32 keys
       const uint2 w = *reinterpret_cast<const uint2*>(a.fv + page_head(kk) * (size_t(D) * PT) +
                                                       (size_t(kk % PT / RUN) * D + dim) * RUN + kk % RUN);
-      const uint32_t u[2] = {w.x, w.y};
-      float v[4];
+      uint32_t u[2] = {w.x, w.y};
 #pragma unroll
-      for (int e = 0; e < 4; ++e)
-        v[e] = kk + e < n_keys ? WidenF16(static_cast<uint16_t>(u[e / 2] >> (16 * (e % 2)))) : 0.0f;
-      o[2 * hf] = PackBf16(v[0], v[1]), o[2 * hf + 1] = PackBf16(v[2], v[3]);
+      for (int e = 0; e < 4; ++e)  // keys at or past the end are zero in the image
+        if (kk + e >= n_keys) u[e / 2] &= e % 2 ? 0x0000FFFFu : 0xFFFF0000u;
+      o[2 * hf] = u[0], o[2 * hf + 1] = u[1];
     }
     *reinterpret_cast<uint4*>(vimg + size_t(p) * 16) = uint4{o[0], o[1], o[2], o[3]};
   }
@@ -579,7 +601,7 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
   static_assert(TIMG == 2 * KIMG, "the two halves of an image have the same size");
   __shared__ __align__(1024) char lds[5][KIMG];  // [0], [1]: K halves; [2] .. [4]: V halves
 
-  b8v qb[RB][KS];
+  h8v qb[RB][KS];
   int qpos[RB], head[RB];
 #pragma unroll
   for (int i = 0; i < RB; ++i) {
@@ -589,7 +611,7 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
     const int t = min(qpos[i], a.chunk_len - 1), hd = min(head[i], G - 1);
     const uint16_t* qp = a.q + ((size_t(s) * a.chunk_len + t) * g.n_q + size_t(h) * G + hd) * D;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) qb[i][ks] = *reinterpret_cast<const b8v*>(qp + 32 * ks + 8 * jg);
+    for (int ks = 0; ks < KS; ++ks) qb[i][ks] = QueryF16(qp + 32 * ks + 8 * jg);
   }
   f4v o[RB][NDT];
   float m[RB];
@@ -621,17 +643,17 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
   const int sw_l = 16 * (jg ^ (qn % 4)), sw_h = 64 * (qn % 8 / 4);
   const int koff[2] = {qn * (2 * D) + sw_l + sw_h, qn * (2 * D) + sw_l - sw_h};
   const int voff[2] = {qn * 128 + sw_l + sw_h, qn * 128 + sw_l - sw_h};
-  auto read_k = [&](const char* buf, int ks, int kt) -> b8v {
-    return *reinterpret_cast<const b8v*>(buf + koff[ks % 2] + (kt * 16 * (2 * D) + 64 * ks));
+  auto read_k = [&](const char* buf, int ks, int kt) -> h8v {
+    return *reinterpret_cast<const h8v*>(buf + koff[ks % 2] + (kt * 16 * (2 * D) + 64 * ks));
   };
   // One 32-dim step of S^T = K Q^T: the A operands of step ks + KP are read before the products of step ks.
-  auto k_first = [&](const char* buf, b8v (&ka)[KP + 1][4]) {
+  auto k_first = [&](const char* buf, h8v (&ka)[KP + 1][4]) {
 #pragma unroll
     for (int ks = 0; ks < KP; ++ks)
 #pragma unroll
       for (int kt = 0; kt < 4; ++kt) ka[ks][kt] = read_k(buf, ks, kt);
   };
-  auto k_step = [&](const char* buf, int ks, b8v (&ka)[KP + 1][4], f4v (&st)[RB][4]) {
+  auto k_step = [&](const char* buf, int ks, h8v (&ka)[KP + 1][4], f4v (&st)[RB][4]) {
     if (ks + KP < KS) {
 #pragma unroll
       for (int kt = 0; kt < 4; ++kt) ka[(ks + KP) % (KP + 1)][kt] = read_k(buf, ks + KP, kt);
@@ -640,7 +662,7 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
     for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
       for (int i = 0; i < RB; ++i)
-        st[i][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[ks % (KP + 1)][kt], qb[i][ks], st[i][kt], 0, 0, 0);
+        st[i][kt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[ks % (KP + 1)][kt], qb[i][ks], st[i][kt], 0, 0, 0);
   };
   auto clear = [&](f4v (&st)[RB][4]) {
 #pragma unroll
@@ -649,9 +671,9 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
       for (int kt = 0; kt < 4; ++kt) st[i][kt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
   };
   // Online softmax per query (= per lane). The reference point m of the numerators 2^(score - m) is a whole power
-  // of two and is only moved when a score exceeds it by more than 2^16: moving it rescales numerators, sums and
-  // accumulators by a power of two, which is exact, so moving it late changes nothing in the result, while bf16
-  // numerators and f32 sums have room for the factor 2^16. Rescaling is then rare (the first tile, mostly).
+  // of two and is only moved when a score exceeds it by more than 2^(kBias + kSlack): moving it rescales numerators,
+  // sums and accumulators by a power of two, which is exact, so moving it late changes nothing in the result, while f16
+  // numerators and f32 sums have room for that factor. Rescaling is then rare (the first tile, mostly).
   auto row_max = [&](const f4v (&st)[4]) -> float {  // over the 64 keys of the tile, times the softmax scale
     float mx = fmaxf(st[0][0], st[0][1]);  // a chain of three-operand maxima
     mx = fmaxf(fmaxf(mx, st[0][2]), st[0][3]);
@@ -660,9 +682,9 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
     return MaxOverLaneGroups(mx) * sscale;  // sscale > 0 is required by the entry point
   };
   auto move_reference = [&](int i, float mx) {
-    if (__builtin_expect(__builtin_amdgcn_ballot_w64(mx > m[i] + 16.0f) != 0, 0)) {
-      const b8v zero = {0, 0, 0, 0, 0, 0, 0, 0};
-      const float mn = mx > m[i] + 16.0f ? __builtin_ceilf(mx) : m[i];
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(mx > m[i] + (kBias + kSlack)) != 0, 0)) {
+      const h8v zero = {0, 0, 0, 0, 0, 0, 0, 0};
+      const float mn = mx > m[i] + (kBias + kSlack) ? __builtin_ceilf(mx) - kBias : m[i];
       const float alpha = __builtin_amdgcn_exp2f(m[i] - mn);
       m[i] = mn;
       // The rescaled accumulators go back through a matrix instruction with zero factors: that keeps them in the
@@ -674,7 +696,7 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
         asm volatile("" : "+a"(t));
 #pragma unroll
         for (int r = 0; r < 4; ++r) t[r] *= alpha;
-        lacc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(zero, zero, t, 0, 0, 0);
+        lacc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(zero, zero, t, 0, 0, 0);
       }
 #pragma unroll
       for (int dt = 0; dt < NDT; ++dt) {
@@ -682,36 +704,36 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
         asm volatile("" : "+a"(t));
 #pragma unroll
         for (int r = 0; r < 4; ++r) t[r] *= alpha;
-        o[i][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(zero, zero, t, 0, 0, 0);
+        o[i][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(zero, zero, t, 0, 0, 0);
       }
     }
   };
-  // bf16 numerators of row block i as B operands of the second product: [32-key step] 4 + 4 keys per lane
-  auto numerators = [&](int i, const f4v (&st)[4], b8v (&pv)[2]) {
+  // f16 numerators of row block i as B operands of the second product: [32-key step] 4 + 4 keys per lane
+  auto numerators = [&](int i, const f4v (&st)[4], h8v (&pv)[2]) {
     uint32_t w[2][4];
 #pragma unroll
     for (int kt = 0; kt < 4; ++kt) {
       float p[4];
 #pragma unroll
       for (int r = 0; r < 4; ++r) p[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(st[kt][r], sscale, -m[i]));
-      w[kt / 2][2 * (kt % 2)] = PackBf16(p[0], p[1]);
-      w[kt / 2][2 * (kt % 2) + 1] = PackBf16(p[2], p[3]);
+      w[kt / 2][2 * (kt % 2)] = PackF16(p[0], p[1]);
+      w[kt / 2][2 * (kt % 2) + 1] = PackF16(p[2], p[3]);
     }
 #pragma unroll
-    for (int s2 = 0; s2 < 2; ++s2) pv[s2] = __builtin_bit_cast(b8v, uint4{w[s2][0], w[s2][1], w[s2][2], w[s2][3]});
+    for (int s2 = 0; s2 < 2; ++s2) pv[s2] = __builtin_bit_cast(h8v, uint4{w[s2][0], w[s2][1], w[s2][2], w[s2][3]});
   };
   // O^T += V^T P^T and the denominators; `v_tile` >= 0: the V half of that image is copied meanwhile (`always`:
   // known when compiling, which keeps the products in one scheduling region)
-  auto pv_product = [&](auto always, const char* buf, const b8v (&pv)[RB][2], int v_tile) {
+  auto pv_product = [&](auto always, const char* buf, const h8v (&pv)[RB][2], int v_tile) {
     // (the empty asm keeps the two lane addresses as they are: left alone, the compiler hoists voff + constant out
     // of the tile loop for every read and adds the buffer's address to each of them again)
     typedef __attribute__((address_space(3))) const char* LdsPtr;
     LdsPtr vb0 = (LdsPtr)buf + voff[0], vb1 = (LdsPtr)buf + voff[1];
     asm volatile("" : "+v"(vb0), "+v"(vb1));
-    auto read_v = [&](int dt, int s2) -> b8v {
-      return *reinterpret_cast<const __attribute__((address_space(3))) b8v*>((s2 ? vb1 : vb0) + (dt * 16 * 128 + 64 * s2));
+    auto read_v = [&](int dt, int s2) -> h8v {
+      return *reinterpret_cast<const __attribute__((address_space(3))) h8v*>((s2 ? vb1 : vb0) + (dt * 16 * 128 + 64 * s2));
     };
-    b8v va[VP + 1][2];  // read VP 16-dim tiles ahead
+    h8v va[VP + 1][2];  // read VP 16-dim tiles ahead
 #pragma unroll
     for (int dt = 0; dt < VP; ++dt)
 #pragma unroll
@@ -720,7 +742,7 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
     for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
       for (int i = 0; i < RB; ++i)
-        lacc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(OnesBf16(), pv[i][s2], lacc[i], 0, 0, 0);
+        lacc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(OnesF16(), pv[i][s2], lacc[i], 0, 0, 0);
 #pragma unroll
     for (int dt = 0; dt < NDT; ++dt) {
       if (dt + VP < NDT) {
@@ -731,7 +753,7 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
       for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
         for (int i = 0; i < RB; ++i)
-          o[i][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[dt % (VP + 1)][s2], pv[i][s2], o[i][dt], 0, 0, 0);
+          o[i][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va[dt % (VP + 1)][s2], pv[i][s2], o[i][dt], 0, 0, 0);
       if (dt % 2 == 1) {
         if (decltype(always)::value || v_tile >= 0) copy_part(v_tile, KS + dt / 2);
         __builtin_amdgcn_sched_barrier(0);
@@ -756,7 +778,7 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
   f4v st[RB][4];
   clear(st);
   {
-    b8v ka[KP + 1][4];
+    h8v ka[KP + 1][4];
     k_first(lds[0], ka);
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
@@ -771,9 +793,9 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
     const int k_tile = min(tile + 2, n_tiles - 1);  // its K half goes where K(tile) was (again K(last) at the end)
     f4v sn[RB][4];
     clear(sn);
-    b8v ka[KP + 1][4];
+    h8v ka[KP + 1][4];
     float mx[RB];
-    b8v pv[RB][2];
+    h8v pv[RB][2];
     k_first(kbuf, ka);
 #pragma unroll
     for (int ks = 0; ks < KA; ++ks) {
@@ -822,7 +844,7 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
           for (int r = 0; r < 4; ++r)
             if (tile * kKeys + 16 * kt + 4 * jg + r > prefix + qpos[i]) st[i][kt][r] = kNegBig;
     }
-    b8v pv[RB][2];
+    h8v pv[RB][2];
 #pragma unroll
     for (int i = 0; i < RB; ++i) {
       move_reference(i, row_max(st[i]));
@@ -832,7 +854,7 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
     if (more) {
       const char* kbuf = lds[(tile + 1) % 2];
       clear(st);
-      b8v ka[KP + 1][4];
+      h8v ka[KP + 1][4];
       k_first(kbuf, ka);
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
@@ -949,11 +971,12 @@ extern "C" int yahkv_prefill_attend_tiles(const yahkv_geometry* g, const yahkv_p
                                     chunk_len, &a))
     return rc;
   if (const int rc = PrepareQueries(q, softmax_scale, gate, out, out_dtype, &a)) return rc;
+  const int tiles = TilesPerPair(max_prefix_len, chunk_len);
+  // the attention kernel addresses a pair's images with 32-bit offsets (checked before the workspace's size, so that
+  // no size a caller claims can get such a launch through)
+  if (int64_t(tiles) * (2 * kKeys * a.g.hd * 2) > 0x7fffffffLL) return YAHKV_ERR_SHAPE;
   if (const int rc = CheckWorkspace(a, workspace, workspace_bytes)) return rc;
   const char* img = static_cast<const char*>(workspace);
-  const int tiles = TilesPerPair(max_prefix_len, chunk_len);
-  // the attention kernel addresses a pair's images with 32-bit offsets
-  if (int64_t(tiles) * (2 * kKeys * a.g.hd * 2) > 0x7fffffffLL) return YAHKV_ERR_SHAPE;
   hipStream_t st = static_cast<hipStream_t>(stream);
   // At head_dim 128, three row blocks per wave (three heads per workgroup) when the GQA group is a multiple of
   // three: each tile image copied to LDS and each operand read from it then serves half as much arithmetic again.
@@ -1036,9 +1059,9 @@ extern "C" int yahkv_f16_prefill_attend(const yahkv_geometry* g, const yahkv_f16
   a.table = page_table, a.stride = page_table_stride, a.prefix_len = prefix_len, a.n_seqs = n_seqs;
   a.max_prefix = max_prefix_len, a.chunk_len = chunk_len;
   if (const int rc = PrepareQueries(q, softmax_scale, gate, out, out_dtype, &a)) return rc;
-  if (const int rc = CheckWorkspace(a, workspace, workspace_bytes)) return rc;
   const int tiles = TilesPerPair(max_prefix_len, chunk_len);
   if (int64_t(tiles) * (2 * kKeys * a.g.hd * 2) > 0x7fffffffLL) return YAHKV_ERR_SHAPE;
+  if (const int rc = CheckWorkspace(a, workspace, workspace_bytes)) return rc;
   ImageArgs ia{};
   ia.g = a.g, ia.table = page_table, ia.stride = page_table_stride, ia.prefix_len = prefix_len, ia.n_seqs = n_seqs;
   ia.max_prefix = max_prefix_len, ia.chunk_len = chunk_len, ia.img = static_cast<char*>(workspace);
