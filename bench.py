@@ -501,7 +501,7 @@ def run_decode(a, wl, torch, yahkv):
     knew = torch.randn((total, B, 1, NKV, HD), generator=gen, device="cuda").to(torch.bfloat16)
     vnew = torch.randn((total, B, 1, NKV, HD), generator=gen, device="cuda").to(torch.bfloat16)
     out = torch.empty((B, NQ, HD), dtype=torch.float32, device="cuda")
-    opt = yahkv.decode_options()
+    opt = yahkv.decode_options(one_launch=a.one_launch)
     ws = torch.empty(yahkv.decode_workspace_bytes(g, B, max_len, opt), dtype=torch.uint8, device="cuda")
     # set-up, as a server does once: the XCDs' relative read speeds on this batch (equal shares without it)
     xcd = yahkv.decode_calibrate(pools, t_table, len_rows[0], max_len, q, ws, opt, rounds=3) if not a.no_calibrate else None
@@ -513,10 +513,15 @@ def run_decode(a, wl, torch, yahkv):
         yahkv.append(pools, t_table, len_rows[i], knew[i], vnew[i])    # position = current length (device-resident)
         if pair:
             pair[0].record()
-        yahkv.decode_part(pools, t_table, seq_len, max_len, q, scale, ws, opt=opt)
-        if pair:
-            pair[1].record()
-        yahkv.decode_reduce(g, t_table.shape[1], seq_len, B, max_len, out, ws, opt=opt)
+        if not a.one_launch:                # the reference's form: partials, then their merge in a dispatch of its own
+            yahkv.decode_part(pools, t_table, seq_len, max_len, q, scale, ws, opt=opt)
+            if pair:
+                pair[1].record()
+            yahkv.decode_reduce(g, t_table.shape[1], seq_len, B, max_len, out, ws, opt=opt)
+        else:                               # one launch: the split-K kernel's workgroups merge what they finish last
+            yahkv.decode_attend(pools, t_table, seq_len, max_len, q, scale, out=out, workspace=ws, opt=opt)
+            if pair:
+                pair[1].record()
 
     # parity before timing: first step, a few sequences against the float64 closed form
     step(0)
@@ -555,7 +560,8 @@ def run_decode(a, wl, torch, yahkv):
         "config": {"workload": a.workload, "batch": B, "ctx_min": int(lens.min()), "ctx_max": int(lens.max()),
                    "ctx_sum": int(lens.sum()), "n_q_heads": NQ, "n_kv_heads": NKV, "head_dim": HD, "page_tokens": PT,
                    "n_pages": g.n_pages, "layers_rotated": len(layers), "kv_format": "q8_0" if wl["fmt"] == 8 else "q4_0",
-                   "step": "append 1 token/seq + paged decode attention", "xcd_weight": xcd},
+                   "step": "append 1 token/seq + paged decode attention (%s)" %
+                           ("one launch" if a.one_launch else "part + reduce"), "xcd_weight": xcd},
         "pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2), "tok_per_s": round(B / (ms * 1e-3), 1),
         "kv_bytes_per_step": int(kv_bytes), "parity_max_rel_err": float(f"{err:.3e}"), "out_fnv1a": first_hash,
         "roofline": {"bound": "hbm", "achieved": round(kgbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
@@ -617,6 +623,8 @@ def main():
     ap.add_argument("--no-also", action="store_true",
                     help="default workload only: do not time the other configurations for the line's `also` object")
     ap.add_argument("--no-calibrate", action="store_true", help="decode workloads: equal chunk shares for all XCDs")
+    ap.add_argument("--one-launch", action="store_true",
+                    help="decode workloads: yahkv_decode_attend with opt.one_launch instead of part + reduce")
     ap.add_argument("--graph-replay", action="store_true",
                     help="decode workloads: also replay the timed steps as one HIP graph and report its time per step")
     ap.add_argument("--copy-calibration", action="store_true",

@@ -154,6 +154,10 @@ typedef struct yahkv_decode_options {
                                results differ by about 1e-4 relative from run to run) */
   int32_t xcd_weight[8];    /* relative read speeds of the eight XCDs, as yahkv_decode_calibrate measures them; the
                                chunks of a group of eight are sized by them; all 0: equal shares */
+  int32_t one_launch;       /* not 0: yahkv_decode_attend issues one dispatch instead of two: the workgroup that is last
+                               to finish a pair's keys merges the pair's partials itself. Same results; measured slower
+                               than the two dispatches on an MI355X (partials cross between XCDs through memory), so it
+                               is for callers to whom the number of dispatches matters more than the time */
 } yahkv_decode_options;
 
 /* Decode attention: one query token per sequence against keys 0 .. seq_len[s] - 1.
@@ -180,7 +184,7 @@ int yahkv_decode_part(const yahkv_geometry* g, const yahkv_pools* pools, const i
 int yahkv_decode_reduce(const yahkv_geometry* g, int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs,
                         int32_t max_seq_len, const float* gate, float* out, const void* workspace,
                         size_t workspace_bytes, const yahkv_decode_options* opt, void* stream);
-/* part, then reduce. */
+/* part, then reduce (one dispatch that does both with opt->one_launch). out must be 16-byte aligned. */
 int yahkv_decode_attend(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
                         int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs, int32_t max_seq_len,
                         const void* q, int32_t q_dtype, float softmax_scale, const float* gate, float* out,

@@ -80,3 +80,38 @@ def test_xcd_calibration_returns_usable_shares(yahkv, torch_gpu):
 
 def g_dev(yahkv, g):
     return yahkv.geometry(g.format, g.n_q_heads, g.n_kv_heads, g.head_dim, g.page_tokens, g.n_pages)
+
+
+@pytest.mark.parametrize("fmt,n_q,n_kv,hd,pt", [(8, 24, 4, 256, 64), (4, 24, 4, 256, 64), (8, 8, 2, 128, 16), (4, 16, 2, 256, 32)])
+def test_one_launch_form_gives_the_two_dispatches_results(yahkv, torch_gpu, fmt, n_q, n_kv, hd, pt):
+    """opt.one_launch: the workgroup that is last to finish a pair's keys merges the pair itself. Sequences that lie in
+    one chunk, that span many, that are empty; twice on one workspace (the tickets of the first call are left clean),
+    then with the chunk count forced up so that every pair spans several chunks; with the deterministic pattern the
+    one dispatch repeats bit for bit as well."""
+    torch = torch_gpu
+    lens = [1, 0, 63, 64, 65, 700, 5000, 31, 12000, 129, 2500, 0, 64 * 40]
+    g, table, host, dev, rng = setup(yahkv, torch, fmt, n_q, n_kv, hd, pt, lens, seed=fmt + hd + pt, fill=0x7F)
+    q = to_bf16_f32(rng.standard_normal((len(lens), n_q, hd)))
+    gate = rng.standard_normal(q.shape).astype(np.float32)
+    scale = float(1 / np.sqrt(hd))
+    want = oracle.decode_attend(host, table, lens, q, scale, gate)
+    for opt in (yahkv.decode_options(one_launch=True), yahkv.decode_options(one_launch=True, n_chunks=1000, min_chunk_tiles=2),
+                yahkv.decode_options(one_launch=True, n_chunks=7)):
+        ws = torch.empty(yahkv.decode_workspace_bytes(g_dev(yahkv, g), len(lens), max(lens), opt), dtype=torch.uint8, device="cuda")
+        ws.random_(0, 256)                                     # nothing in the workspace has to start at zero
+        tq = torch.from_numpy(q).cuda().to(torch.bfloat16)
+        tg = torch.from_numpy(gate).cuda()
+        t_table = torch.from_numpy(table).cuda()
+        t_lens = torch.tensor(lens, dtype=torch.int32, device="cuda")
+        for _ in range(2):
+            out = torch.full(q.shape, float("nan"), device="cuda")
+            yahkv.decode_attend(dev, t_table, t_lens, max(lens), tq, scale, gate=tg, out=out, workspace=ws, opt=opt)
+            torch.cuda.synchronize()
+            got = out.cpu().numpy()
+            assert np.all(np.isfinite(got))
+            assert not got[1].any() and not got[11].any()
+            assert rel_err(got, want) < TOL
+    det = yahkv.decode_options(one_launch=True, deterministic=True)
+    runs = [gpu_attend(yahkv, torch, dev, table, lens, q, scale, opt=det) for _ in range(3)]
+    assert np.array_equal(runs[0].view(np.uint32), runs[1].view(np.uint32))
+    assert np.array_equal(runs[0].view(np.uint32), runs[2].view(np.uint32))

@@ -33,6 +33,8 @@ def test_random_decode_case(yahkv, torch_gpu, seed):
         opt.min_chunk_tiles = int(rng.choice([1, 2, 5]))
     if rng.random() < 0.3:
         opt.deterministic = 1
+    if rng.random() < 0.5:
+        opt.one_launch = 1
     if rng.random() < 0.3:
         for j in range(8):
             opt.xcd_weight[j] = int(rng.choice([0, 1, 900, 1000, 1100, 100000]))

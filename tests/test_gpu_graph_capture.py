@@ -14,8 +14,10 @@ from test_gpu_decode import setup
 pytestmark = pytest.mark.gpu
 
 
-def test_decode_step_replays_from_a_graph(yahkv, torch_gpu):
+@pytest.mark.parametrize("one_launch", [False, True], ids=["part_reduce", "one_launch"])
+def test_decode_step_replays_from_a_graph(yahkv, torch_gpu, one_launch):
     torch = torch_gpu
+    opt = yahkv.decode_options(one_launch=one_launch, n_chunks=24, min_chunk_tiles=2)   # pairs that span several chunks
     lens = [700, 64, 1, 333]
     g, table, host, dev, rng = setup(yahkv, torch, 8, 24, 4, 256, 64, [n + 1 for n in lens], seed=21)
     t_table = torch.from_numpy(table).cuda()
@@ -25,11 +27,11 @@ def test_decode_step_replays_from_a_graph(yahkv, torch_gpu):
     k = torch.randn((4, 1, 4, 256), device="cuda").to(torch.bfloat16)
     v = torch.randn((4, 1, 4, 256), device="cuda").to(torch.bfloat16)
     out = torch.empty((4, 24, 256), dtype=torch.float32, device="cuda")
-    ws = torch.empty(yahkv.decode_workspace_bytes(dev.geom, 4, 701), dtype=torch.uint8, device="cuda")
+    ws = torch.empty(yahkv.decode_workspace_bytes(dev.geom, 4, 701, opt), dtype=torch.uint8, device="cuda")
 
     def step():
         yahkv.append(dev, t_table, pos, k, v)
-        yahkv.decode_attend(dev, t_table, seq_len, 701, q, 0.0625, out=out, workspace=ws)
+        yahkv.decode_attend(dev, t_table, seq_len, 701, q, 0.0625, out=out, workspace=ws, opt=opt)
 
     step()                                            # eager: also the one-time host set-up of the library
     torch.cuda.synchronize()

@@ -75,10 +75,11 @@ def test_prefill_against_oracle(yahkv, torch_gpu, path, fmt, n_q, n_kv, hd, pt, 
     out16 = yahkv.prefill_attend(dev, t_table, t_prefix, max(prefix), to_t(q), scale, out_dtype=torch.float16,
                                  workspace=ws)
     assert rel_err(out16.float().cpu().numpy(), exact) < TOL
-    # bf16 output: its own rounding, 2^-9 of the largest element, comes on top
+    # bf16 output: its own rounding comes on top, up to 2^-8 of an element (8 significant bits), which is more than
+    # the whole tolerance: callers that need 2e-3 take f16 or f32 output
     out16 = yahkv.prefill_attend(dev, t_table, t_prefix, max(prefix), to_t(q), scale, out_dtype=torch.bfloat16,
                                  workspace=ws)
-    assert rel_err(out16.float().cpu().numpy(), exact) < 1e-3 + 2.0 ** -9
+    assert rel_err(out16.float().cpu().numpy(), exact) < 1e-3 + 2.0 ** -8
 
 
 @pytest.mark.parametrize("ws", [None, False], ids=["images", "fused"])

@@ -35,7 +35,8 @@ class F16PoolsStruct(C.Structure):
 class DecodeOptions(C.Structure):
     """yahkv_decode_options: zero fields are the defaults."""
     _fields_ = [("n_chunks", C.c_int32), ("min_chunk_tiles", C.c_int32), ("pair_cost", C.c_int32),
-                ("reduce_split", C.c_int32), ("deterministic", C.c_int32), ("xcd_weight", C.c_int32 * 8)]
+                ("reduce_split", C.c_int32), ("deterministic", C.c_int32), ("xcd_weight", C.c_int32 * 8),
+                ("one_launch", C.c_int32)]
 
 
 class Rope(C.Structure):
@@ -344,9 +345,11 @@ def append_rope(pools, table, start_pos, k_src, v_src, theta, eps, rotary_dim, k
     return q_out, k_out
 
 
-def decode_options(n_chunks=0, min_chunk_tiles=0, pair_cost=0, reduce_split=0, deterministic=False, xcd_weight=None):
+def decode_options(n_chunks=0, min_chunk_tiles=0, pair_cost=0, reduce_split=0, deterministic=False, xcd_weight=None,
+                   one_launch=False):
     """yahkv_decode_options; zero / None fields are the defaults."""
     o = DecodeOptions(n_chunks, min_chunk_tiles, pair_cost, reduce_split, 1 if deterministic else 0)
+    o.one_launch = 1 if one_launch else 0
     for j, w in enumerate(xcd_weight or ()):
         o.xcd_weight[j] = int(w)
     return o

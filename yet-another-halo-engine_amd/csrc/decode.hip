@@ -17,6 +17,7 @@
 // global memory or by the dispatcher, to even out the XCDs, which finish up to 10 % apart. Every variant was slower:
 // each change of pair costs a wave a pipeline fill, and the XCDs that finish first leave their bandwidth to the rest.)
 #include <algorithm>
+#include <atomic>
 #include <cstdio>
 #include <cstdlib>
 #include <mutex>
@@ -32,6 +33,7 @@ constexpr int kTile = 64;     // keys per tile: one wavefront, one key per lane 
 constexpr int kMaxGroup = 8;  // query heads per kv head
 constexpr int kMaxSeqs = 8191;
 constexpr int kWavesPerGroup = 8;  // one workgroup fills a CU at two waves per SIMD
+constexpr int kMergeSlots = 512;   // partial slots the in-kernel merge weighs at a time
 
 struct DecodeArgs {
   Geom g;
@@ -55,6 +57,10 @@ struct DecodeArgs {
   int32_t share[9];  // cumulative shares of the eight chunks of a group, in 1/8192 of the group (share[8] = 8192)
   int32_t deterministic;  // waves take the chunk's tiles in a fixed pattern instead of first come, first served
   unsigned long long* stamps;  // calibration only: [n_chunks] the time each workgroup's last wave finished
+  // one launch for part and merge: the workgroup that is last to finish a pair's tiles merges the pair's partials
+  int32_t fused;
+  uint32_t epoch;               // never 0, different in every launch (graph replays aside: see Arrive)
+  unsigned long long* tickets;  // [n_seqs * H] arrivals per pair: (epoch << 32) | workgroups that have arrived
 };
 
 __device__ __forceinline__ int ClampLen(const DecodeArgs& a, int s) { return min(max(a.seq_len[s], 0), a.max_len); }
@@ -96,8 +102,11 @@ __device__ __forceinline__ long long ChunkUnits(const DecodeArgs& a, long long l
 // head, first tile within the pair, tiles in the chunk}. Thread t sums a slice of the sequences, a scan over the
 // threads gives every slice its place on the line, and the threads whose slices hold the chunk's two ends walk
 // their slices to find the sequences and count the tiles before each end.
+// Also leaves, for the merge: tiles_at[2], the line coordinate of the first tile of the chunk's first pair, and
+// tiles_at[3], the line units per chunk (the A of ChunkStart / ChunkOf).
 template <int NT>
-__device__ __forceinline__ int4 ChunkRecord(const DecodeArgs& a, int k, int (*wave_sum)[2], int4* found, long long* tiles_at) {
+__device__ __forceinline__ int4 ChunkRecord(const DecodeArgs& a, int k, int (*wave_sum)[2], int4* found, long long* tiles_at,
+                                            bool* any_empty) {
   const int t = threadIdx.x, H = a.g.n_kv, c = a.pair_cost;
   const int per = (a.n_seqs + NT - 1) / NT;
   const int s0 = min(t * per, a.n_seqs), s1 = min(s0 + per, a.n_seqs);
@@ -106,6 +115,7 @@ __device__ __forceinline__ int4 ChunkRecord(const DecodeArgs& a, int k, int (*wa
     const int ts = TilesOf(a, s);
     sum += UnitsOf(a, ts), cnt += ts > 0;
   }
+  *any_empty = cnt < s1 - s0;
   int incl = sum, incl_cnt = cnt;  // inclusive scans inside the wave, then the waves' totals
 #pragma unroll
   for (int o = 1; o < 64; o <<= 1) {
@@ -126,6 +136,7 @@ __device__ __forceinline__ int4 ChunkRecord(const DecodeArgs& a, int k, int (*wa
     if (t == 0) a.tprefix[a.n_seqs] = total;
   }
   const long long line = static_cast<long long>(total) * H, A = ChunkUnits(a, line);
+  if (t == 0) tiles_at[3] = A;
   const long long start = ChunkStart(a, A, k), end = min(ChunkStart(a, A, k + 1), line);
   if (start >= end) return int4{-1, 0, 0, 0};  // the same for every thread
   if (t == 0 && end == line) tiles_at[1] = static_cast<long long>(total - c * total_cnt) * H;
@@ -139,7 +150,10 @@ __device__ __forceinline__ int4 ChunkRecord(const DecodeArgs& a, int k, int (*wa
         const int r = static_cast<int>(x - static_cast<long long>(before) * H);
         const int h = r / units, first = max(r % units - c, 0);
         *tiles = static_cast<long long>(before - c * before_cnt) * H + static_cast<long long>(h) * ts + first;
-        if (where != nullptr) *where = int4{s, h, first, 0};
+        if (where != nullptr) {
+          *where = int4{s, h, first, 0};
+          tiles_at[2] = static_cast<long long>(before) * H + static_cast<long long>(h) * units + c;
+        }
         return;
       }
       before += units, before_cnt += ts > 0;
@@ -175,6 +189,22 @@ __device__ __forceinline__ bool NextPair(const DecodeArgs& a, int chunk_n, PairC
     if (ts == 0) c->h = a.g.n_kv - 1;
   } while (ts == 0);
   c->n = min(ts, chunk_n - c->base), c->len = ClampLen(a, c->s);
+  return true;
+}
+// The same walk for the merge at the kernel's end, which also needs to know where on the line a pair lies: its tiles
+// in all and the line coordinate of its first tile.
+struct MergeCursor {
+  PairCursor c;
+  int ts;
+  long long line0;
+};
+__device__ __forceinline__ MergeCursor FirstMergePair(const DecodeArgs& a, const int4 rec, long long line0) {
+  return MergeCursor{FirstPair(a, rec), TilesOf(a, rec.x), line0};
+}
+__device__ __forceinline__ bool NextMergePair(const DecodeArgs& a, int chunk_n, MergeCursor* m) {
+  const long long next = m->line0 + m->ts + a.pair_cost;  // the next pair's first units follow this pair's tiles
+  if (!NextPair(a, chunk_n, &m->c)) return false;         // (sequences without keys take none)
+  m->line0 = next, m->ts = TilesOf(a, m->c.s);
   return true;
 }
 __device__ __forceinline__ size_t PartialIndex(const DecodeArgs& a, int chunk, int wave, const PairCursor& c) {
@@ -297,6 +327,61 @@ __device__ __forceinline__ h8v LoadQ8(const void* q, size_t i, int dt) {
   return r;
 }
 
+// Partials travel between workgroups on different XCDs, whose L2 caches do not see each other's lines: they are
+// written through to memory and read past the L2 (cache policy sc1, device scope) by these buffer accesses. Fences of
+// device scope would do it too, but they write back and invalidate a whole L2, and with it the K / V lines the XCD's
+// other workgroups have in flight (measured: 12 % of the kernel's time).
+constexpr int kDeviceScope = 16;  // the sc1 bit of a buffer instruction's cache policy
+typedef unsigned int u4v __attribute__((__vector_size__(4 * sizeof(unsigned int))));
+typedef unsigned int u2v __attribute__((__vector_size__(2 * sizeof(unsigned int))));
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t DeviceBuffer(const void* base) {  // base: the same in every lane
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, 0x7fffffff, 0x00020000);
+}
+__device__ __forceinline__ void StoreDevice(__amdgpu_buffer_rsrc_t r, uint32_t byte_offset, float v) {
+  __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned int, v), r, byte_offset, 0, kDeviceScope);
+}
+__device__ __forceinline__ void StoreDevice2(__amdgpu_buffer_rsrc_t r, uint32_t byte_offset, float x, float y) {
+  const u2v w = {__builtin_bit_cast(unsigned int, x), __builtin_bit_cast(unsigned int, y)};
+  __builtin_amdgcn_raw_buffer_store_b64(w, r, byte_offset, 0, kDeviceScope);
+}
+__device__ __forceinline__ float2 LoadDevice2(__amdgpu_buffer_rsrc_t r, uint32_t byte_offset) {
+  const u2v w = __builtin_amdgcn_raw_buffer_load_b64(r, byte_offset, 0, kDeviceScope);
+  const unsigned int w0 = w[0], w1 = w[1];  // (a bit cast applied to w[1] directly reads w[0] with this compiler)
+  return float2{__builtin_bit_cast(float, w0), __builtin_bit_cast(float, w1)};
+}
+template <int N>
+struct LoadDeviceN;
+template <>
+struct LoadDeviceN<4> {
+  typedef float type __attribute__((ext_vector_type(4)));
+  static __device__ __forceinline__ type load(__amdgpu_buffer_rsrc_t r, uint32_t byte_offset) {
+    return __builtin_bit_cast(type, __builtin_amdgcn_raw_buffer_load_b128(r, byte_offset, 0, kDeviceScope));
+  }
+};
+template <>
+struct LoadDeviceN<2> {
+  typedef float type __attribute__((ext_vector_type(2)));
+  static __device__ __forceinline__ type load(__amdgpu_buffer_rsrc_t r, uint32_t byte_offset) {
+    return __builtin_bit_cast(type, __builtin_amdgcn_raw_buffer_load_b64(r, byte_offset, 0, kDeviceScope));
+  }
+};
+
+// A workgroup announces that its partials of a pair are written; true for the one that is last of `n`, which then owns
+// the merge. The ticket word carries the launch's epoch above the count: a word with another epoch in it (memory that
+// was never used, or the zero the last arrival of an earlier launch left) counts as empty, so the workspace needs no
+// clearing, and the last arrival puts the zero back, so a graph replay, which repeats its epoch, starts clean too.
+__device__ __forceinline__ int Arrive(unsigned long long* ticket, uint32_t epoch, uint32_t n) {
+  unsigned long long old = __hip_atomic_load(ticket, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  while (true) {
+    const uint32_t count = static_cast<uint32_t>(old >> 32) == epoch ? static_cast<uint32_t>(old) : 0u;
+    const bool last = count + 1 == n;
+    const unsigned long long next = last ? 0ull : (static_cast<unsigned long long>(epoch) << 32) | (count + 1);
+    if (__hip_atomic_compare_exchange_strong(ticket, &old, next, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                             __HIP_MEMORY_SCOPE_AGENT))
+      return last ? 1 : 0;
+  }
+}
+
 // One workgroup of eight waves per chunk, one workgroup per CU (two waves per SIMD). The waves share nothing but the
 // LDS counter that hands out the chunk's tiles; after the first barrier no wave waits for another. A wave takes tiles
 // in increasing order, so it meets the chunk's (sequence, kv head) pairs in order; for each pair it worked on it keeps
@@ -342,11 +427,14 @@ void DattnPart(const DecodeArgs a) {
   __shared__ __align__(16) float lcorr_all[kWavesPerGroup][NB][8];
   __shared__ __align__(16) _Float16 lp_all[kWavesPerGroup][kMaxGroup][kTile];
   __shared__ __align__(16) _Float16 lvs_all[kWavesPerGroup][NB][kTile];
-  __shared__ __align__(16) uint8_t lvq_all[kWavesPerGroup][FMT == 8 ? NVB * 1024 : 16];  // half a tile of V codes on its way in (q8_0)
+  // half a tile of V codes on its way in (q8_0); at the kernel's end, either format: the waves' sums of a merge
+  __shared__ __align__(16) uint8_t lvq_all[kWavesPerGroup][FMT == 8 ? NVB * 1024 : sizeof(float) * kMaxGroup * D];
   __shared__ int next_tile;
   __shared__ int wave_sum[kWavesPerGroup][2];
   __shared__ int4 chunk_rec;
-  __shared__ long long chunk_tiles[2];
+  __shared__ long long chunk_tiles[4];  // [2], [3]: for the merge, see ChunkRecord
+  __shared__ int merge_flag;
+  __shared__ float merge_m[kMaxGroup], merge_l[kWavesPerGroup][kMaxGroup], merge_w[kWavesPerGroup][kMaxGroup];
   auto& lq = lq_all[wave];
   auto& lcorr = lcorr_all[wave];
   auto& lp = lp_all[wave];
@@ -354,7 +442,20 @@ void DattnPart(const DecodeArgs a) {
   auto& lvq = lvq_all[wave];
 
   if (a.stamps != nullptr && threadIdx.x == 0) a.stamps[blockIdx.x] = wall_clock64();
-  const int4 rec = ChunkRecord<64 * kWavesPerGroup>(a, blockIdx.x, wave_sum, &chunk_rec, chunk_tiles);
+  bool any_empty = false;
+  const int4 rec = ChunkRecord<64 * kWavesPerGroup>(a, blockIdx.x, wave_sum, &chunk_rec, chunk_tiles, &any_empty);
+  // One launch for part and merge: sequences without keys have no pair on the line and nobody merges them, so the
+  // first workgroup writes their rows of zeros (its threads have just looked at a slice of the lengths each).
+  if (a.fused && blockIdx.x == 0 && any_empty) {
+    constexpr int NTH = 64 * kWavesPerGroup;
+    const int per = (a.n_seqs + NTH - 1) / NTH;
+    const int s0 = min(static_cast<int>(threadIdx.x) * per, a.n_seqs), s1 = min(s0 + per, a.n_seqs);
+    for (int s = s0; s < s1; ++s)
+      if (TilesOf(a, s) == 0) {
+        float4* row = reinterpret_cast<float4*>(a.out + size_t(s) * g.n_q * D);
+        for (int i = 0; i < g.n_q * D / 4; ++i) row[i] = float4{0.0f, 0.0f, 0.0f, 0.0f};
+      }
+  }
   if (rec.x < 0) return;
   const int chunk_n = rec.w;
   if (threadIdx.x == 0) next_tile = 0;
@@ -541,16 +642,17 @@ void DattnPart(const DecodeArgs a) {
   // l = 0 for a pair this wave got no tile of (the reduce then skips it)
   auto leave_empty = [&]() {
     const size_t part = PartialIndex(a, blockIdx.x, wave, cur) * G;
-    if (lane < G) a.ml[(part + lane) * 2] = kNegMax, a.ml[(part + lane) * 2 + 1] = 0.0f;
+    if (lane < G) StoreDevice2(DeviceBuffer(a.ml + part * 2), lane * 8, kNegMax, 0.0f);
   };
   // the pair's partial, straight from registers (natural-log units, as the reduce expects)
   auto leave_partial = [&]() {
     const size_t part = PartialIndex(a, blockIdx.x, wave, cur) * G;
+    const auto rml = DeviceBuffer(a.ml + part * 2), racc = DeviceBuffer(a.acc + part * D);
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const float l = HalfSum32(lsum[r]);
       const int head = 4 * half + r;
-      if (n32 == 0 && head < G) a.ml[(part + head) * 2] = m[r] * kLn2, a.ml[(part + head) * 2 + 1] = l;
+      if (n32 == 0 && head < G) StoreDevice2(rml, head * 8, m[r] * kLn2, l);
     }
     if (kg == 0 || kg == 2) {
 #pragma unroll
@@ -558,7 +660,7 @@ void DattnPart(const DecodeArgs a) {
         const int head = 2 * kg + r;
         if (head < G) {
 #pragma unroll
-          for (int nt = 0; nt < NT; ++nt) a.acc[(part + head) * D + 16 * nt + n16] = o[nt][r];
+          for (int nt = 0; nt < NT; ++nt) StoreDevice(racc, (head * D + 16 * nt + n16) * 4, o[nt][r]);
         }
       }
     }
@@ -566,6 +668,7 @@ void DattnPart(const DecodeArgs a) {
 
   int idx = take();
   bool worked = false;  // this wave has worked on the pair `cur`
+  bool held = false;    // ... and still holds its partial of it in registers: the chunk's last pair, one-launch form
   while (true) {
     // ---- move to the pair of tile idx; pairs passed without a tile get an empty partial
     bool more = idx < chunk_n;
@@ -690,15 +793,228 @@ void DattnPart(const DecodeArgs a) {
     }
     take_v();
     pv(1);
+    // One launch for part and merge: what a wave has of the chunk's last pair stays in its registers, and the waves'
+    // shares of that pair meet in LDS below instead of travelling through memory one by one.
+    if (a.fused && cur.base + cur.n >= chunk_n) {
+      held = true;
+      break;
+    }
     leave_partial();
     __builtin_amdgcn_wave_barrier();  // lq, lp and lvs are rewritten for the next pair
   }
-  // pairs of the chunk after this wave's last tile
-  do {
-    if (!worked) leave_empty();
-    worked = false;
-  } while (NextPair(a, chunk_n, &cur));
+  // pairs of the chunk after this wave's last tile (of the last pair, a wave that holds nothing says so in LDS below)
+  if (!held) {
+    do {
+      if (!worked && !(a.fused && cur.base + cur.n >= chunk_n)) leave_empty();
+      worked = false;
+    } while (NextPair(a, chunk_n, &cur));
+  }
   if (a.stamps != nullptr && lane == 0) atomicMax(&a.stamps[a.n_chunks + blockIdx.x], wall_clock64());
+  if (!a.fused) return;
+
+  // ---- the merge, in the same launch (gen_decode_attn.py:338-411 is the reference's separate dispatch). A pair's
+  // partials come from the workgroups of every chunk its tiles lie in; each of them, when all its waves are done,
+  // announces itself on the pair's ticket, and the one that finds all the others already there merges the pair. Nobody
+  // waits for anybody. LDS: the V slots, which nobody needs any more, hold the waves' sums.
+  static_assert(sizeof(lvq_all) >= sizeof(float) * kWavesPerGroup * kMaxGroup * D, "merge sums fit the V slots");
+  float* const sums = reinterpret_cast<float*>(&lvq_all[0][0]);  // [wave][head][D]
+  constexpr int NTH = 64 * kWavesPerGroup;
+  constexpr int VPL = D / 64;  // dims per lane
+  typedef typename LoadDeviceN<VPL>::type fvv;
+
+  // -- the chunk's last pair: the waves' shares, still in registers, are merged through LDS into one partial
+  if (n32 == 0) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) merge_w[wave][4 * half + r] = held ? m[r] : kNegMax;
+  }
+  __syncthreads();  // (every wave is past its last tile: the V slots are free)
+  {
+    float f[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      float M = kNegMax;
+#pragma unroll
+      for (int w = 0; w < kWavesPerGroup; ++w) M = fmaxf(M, merge_w[w][4 * half + r]);
+      f[r] = held ? __builtin_amdgcn_exp2f(m[r] - M) : 0.0f;
+      const float l = held ? HalfSum32(lsum[r]) * f[r] : 0.0f;
+      if (n32 == 0) merge_l[wave][4 * half + r] = l;
+      if (n32 == 0 && wave == 0) merge_m[4 * half + r] = M;  // (log2 units)
+    }
+    if (kg == 0 || kg == 2) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+          sums[(wave * kMaxGroup + 2 * kg + r) * D + 16 * nt + n16] = held ? o[nt][r] * f[r] : 0.0f;
+    }
+  }
+  __syncthreads();
+
+  int4 mrec = chunk_rec;  // (read again rather than kept in registers through the tile loop)
+  mrec.w = static_cast<int>(chunk_tiles[1] - chunk_tiles[0]);
+  const int merge_n = mrec.w;
+  const long long units_per_chunk = chunk_tiles[3];
+  // writes one row of the output from the waves' sums in LDS
+  auto finish = [&](int s_, int h_) {
+    for (int i = threadIdx.x; i < G * D; i += NTH) {
+      const int gi = i / D, d = i % D;
+      float v = 0.0f, l = 0.0f;
+#pragma unroll
+      for (int w = 0; w < kWavesPerGroup; ++w) v += sums[(w * kMaxGroup + gi) * D + d], l += merge_l[w][gi];
+      v /= l;
+      const size_t o_ = (size_t(s_) * g.n_q + size_t(h_) * G + gi) * D + d;
+      if (a.gate != nullptr) v *= 1.0f / (1.0f + __expf(-a.gate[o_]));
+      a.out[o_] = v;
+    }
+  };
+  // merges the partials of a pair that lie in memory: chunks k0 .. k1, eight slots each, most of them empty (a chunk
+  // that held the pair as its last leaves one slot, a wave without a tile of the pair none). Memory is a few
+  // microseconds away here, so everything is asked for in as few rounds as possible: all (maximum, sum) entries at
+  // once for the heads' maxima; again, 512 slots at a time, for a table of weights in LDS; then every wave asks for
+  // the rows of its non-empty slots, a few slots' rows together.
+  static_assert(sizeof(lq_all) >= sizeof(float) * kMergeSlots * kMaxGroup, "the weights fit the query operands' LDS");
+  float* const wgt = reinterpret_cast<float*>(&lq_all[0][0][0][0][0][0]);  // [slot][head], 0 for an empty slot
+  auto merge = [&](int s_, int h_, int k0, int k1) {
+    const int pair = s_ * H + h_;
+    const size_t slot0 = size_t(k0 + pair) * a.wpc;
+    const int n_slots = (k1 - k0 + 1) * a.wpc;
+    const int gi = threadIdx.x % kMaxGroup, sl = threadIdx.x / kMaxGroup;  // thread = (slot mod 64, head)
+    constexpr int SPT = kMergeSlots / (NTH / kMaxGroup);                   // slots per thread and sweep: 8
+    float M = kNegMax;
+    for (int b0 = 0; b0 < n_slots; b0 += kMergeSlots) {
+      const auto rml = DeviceBuffer(a.ml + (slot0 + b0) * G * 2);
+      float2 v[SPT];
+#pragma unroll
+      for (int u = 0; u < SPT; ++u) {
+        const int j = sl + (NTH / kMaxGroup) * u;
+        v[u] = gi < G && b0 + j < n_slots ? LoadDevice2(rml, (j * G + gi) * 8) : float2{kNegMax, 0.0f};
+      }
+#pragma unroll
+      for (int u = 0; u < SPT; ++u)
+        if (v[u].y > 0.0f) M = fmaxf(M, v[u].x);
+    }
+    // (lanes of one head are 8 apart: three steps across the wave, then the waves through LDS)
+    M = fmaxf(M, __shfl_xor(M, 8, 64)), M = fmaxf(M, __shfl_xor(M, 16, 64)), M = fmaxf(M, __shfl_xor(M, 32, 64));
+    if (lane < kMaxGroup) merge_w[wave][lane] = M;
+    __syncthreads();
+    M = kNegMax;
+#pragma unroll
+    for (int w = 0; w < kWavesPerGroup; ++w) M = fmaxf(M, merge_w[w][gi]);
+    fvv acc[kMaxGroup];
+    float L = 0.0f;  // of head gi, this thread's slots
+#pragma unroll
+    for (int q_ = 0; q_ < kMaxGroup; ++q_) {
+#pragma unroll
+      for (int e = 0; e < VPL; ++e) acc[q_][e] = 0.0f;
+    }
+    for (int b0 = 0; b0 < n_slots; b0 += kMergeSlots) {
+      const int nb = min(n_slots - b0, kMergeSlots);
+      const auto rml = DeviceBuffer(a.ml + (slot0 + b0) * G * 2);
+      float2 v[SPT];
+#pragma unroll
+      for (int u = 0; u < SPT; ++u) {
+        const int j = sl + (NTH / kMaxGroup) * u;
+        v[u] = gi < G && j < nb ? LoadDevice2(rml, (j * G + gi) * 8) : float2{kNegMax, 0.0f};
+      }
+#pragma unroll
+      for (int u = 0; u < SPT; ++u) {
+        const float w = v[u].y > 0.0f ? __expf(v[u].x - M) : 0.0f;
+        L = __builtin_fmaf(w, v[u].y, L);
+        wgt[(sl + (NTH / kMaxGroup) * u) * kMaxGroup + gi] = w;
+      }
+      __syncthreads();
+      // Wave w takes slot (c, r) of chunk c when (c + r) % 8 == w: a chunk's single slot (r = 0) goes to wave c % 8,
+      // and the eight slots of a chunk that left all of them go to the eight waves. One r at a time, four chunks'
+      // slots together.
+      for (int r = 0; r < kWavesPerGroup; ++r) {
+        for (int c0 = (wave - r + kWavesPerGroup) % kWavesPerGroup; c0 * kWavesPerGroup < nb; c0 += 4 * kWavesPerGroup) {
+          fvv row[4][kMaxGroup];
+          float wv[4][kMaxGroup];
+#pragma unroll
+          for (int t = 0; t < 4; ++t) {
+            const int j = (c0 + kWavesPerGroup * t) * kWavesPerGroup + r;
+            const bool in = j < nb;
+            const auto racc = DeviceBuffer(a.acc + (slot0 + b0 + (in ? j : 0)) * G * D);
+#pragma unroll
+            for (int q_ = 0; q_ < kMaxGroup; ++q_) {
+              wv[t][q_] = in && q_ < G ? wgt[j * kMaxGroup + q_] : 0.0f;  // the same in every lane
+              if (wv[t][q_] > 0.0f) row[t][q_] = LoadDeviceN<VPL>::load(racc, (q_ * D + VPL * lane) * 4);
+            }
+          }
+#pragma unroll
+          for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int q_ = 0; q_ < kMaxGroup; ++q_)
+              if (wv[t][q_] > 0.0f) {
+#pragma unroll
+                for (int e = 0; e < VPL; ++e) acc[q_][e] = __builtin_fmaf(wv[t][q_], row[t][q_][e], acc[q_][e]);
+              }
+        }
+      }
+      __syncthreads();  // the table is free for the next 512 slots
+    }
+    // the sums of the threads of one head (lanes 8 apart), then of the waves
+    L += __shfl_xor(L, 8, 64), L += __shfl_xor(L, 16, 64), L += __shfl_xor(L, 32, 64);
+    if (lane < kMaxGroup) merge_l[wave][lane] = L;
+#pragma unroll
+    for (int q_ = 0; q_ < kMaxGroup; ++q_)
+      if (q_ < G) *reinterpret_cast<fvv*>(&sums[(wave * kMaxGroup + q_) * D + VPL * lane]) = acc[q_];
+    __syncthreads();
+    finish(s_, h_);
+    __syncthreads();  // the sums are free for the next pair
+  };
+
+  // announces this workgroup's partials of a pair and merges the pair if all the others are in
+  auto arrive_and_merge = [&](int s_, int h_, int k0, int k1) {
+    // every partial of this workgroup for the pair has reached memory before the workgroup says so
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (threadIdx.x == 0)
+      merge_flag = k0 == k1 ? 1 : Arrive(&a.tickets[s_ * H + h_], a.epoch, static_cast<uint32_t>(k1 - k0 + 1));
+    __syncthreads();
+    const bool mine = merge_flag != 0;
+    __syncthreads();  // (the flag is free again)
+    if (mine) merge(s_, h_, k0, k1);
+  };
+  // The last pair first, while its sum is in LDS: finished here if all of it was this workgroup's, else written out
+  // as this chunk's one partial of it (slot 0; the other seven slots stay empty).
+  {
+    MergeCursor mc = FirstMergePair(a, mrec, chunk_tiles[2]);
+    while (NextMergePair(a, merge_n, &mc)) {
+    }
+    const int s_ = mc.c.s, h_ = mc.c.h;
+    const int k0 = ChunkOf(a, units_per_chunk, mc.line0), k1 = ChunkOf(a, units_per_chunk, mc.line0 + mc.ts - 1);
+    if (k0 == k1) {
+      finish(s_, h_);
+      __syncthreads();
+    } else {
+      const size_t part = (size_t(blockIdx.x) + size_t(s_) * H + h_) * a.wpc * G;
+      const auto rml = DeviceBuffer(a.ml + part * 2), racc = DeviceBuffer(a.acc + part * D);
+      for (int i = threadIdx.x; i < G * D; i += NTH) {
+        const int gi = i / D, d = i % D;
+        float v = 0.0f;
+#pragma unroll
+        for (int w = 0; w < kWavesPerGroup; ++w) v += sums[(w * kMaxGroup + gi) * D + d];
+        StoreDevice(racc, i * 4, v);
+        if (d < a.wpc) {
+          float l = 0.0f;
+#pragma unroll
+          for (int w = 0; w < kWavesPerGroup; ++w) l += merge_l[w][gi];
+          StoreDevice2(rml, (d * G + gi) * 8, merge_m[gi] * kLn2, d == 0 ? l : 0.0f);
+        }
+      }
+      arrive_and_merge(s_, h_, k0, k1);
+    }
+  }
+  // the pairs before it ended in this chunk; their partials went to memory wave by wave
+  MergeCursor mc = FirstMergePair(a, mrec, chunk_tiles[2]);
+  while (mc.c.base + mc.c.n < merge_n) {
+    const int s_ = mc.c.s, h_ = mc.c.h;
+    const int k0 = ChunkOf(a, units_per_chunk, mc.line0), k1 = ChunkOf(a, units_per_chunk, mc.line0 + mc.ts - 1);
+    arrive_and_merge(s_, h_, k0, k1);
+    if (!NextMergePair(a, merge_n, &mc)) break;
+  }
 }
 
 // ---- reduce -------------------------------------------------------------------------------------------------------------
@@ -803,7 +1119,7 @@ __global__ __launch_bounds__(kReduceThreads) void DattnReduce(const DecodeArgs a
 struct Plan {
   int32_t max_len, n_chunks, wpc, min_chunk_tiles, pair_cost;
   int32_t share[9];
-  size_t off_tprefix, off_ml, off_acc, off_stamps, bytes;
+  size_t off_tprefix, off_tickets, off_ml, off_acc, off_stamps, bytes;
 };
 size_t Align(size_t x) { return (x + 255) & ~size_t(255); }
 int ComputeUnits() {
@@ -818,7 +1134,7 @@ int ComputeUnits() {
 }
 // Tuning values of a call: the caller's options where given, else the defaults.
 struct Tuning {
-  int32_t n_chunks, min_chunk_tiles, pair_cost, reduce_split, deterministic;
+  int32_t n_chunks, min_chunk_tiles, pair_cost, reduce_split, deterministic, one_launch;
   int32_t xcd_weight[8];
 };
 Tuning MakeTuning(const yahkv_decode_options* o) {
@@ -832,6 +1148,7 @@ Tuning MakeTuning(const yahkv_decode_options* o) {
   t.pair_cost = o == nullptr || o->pair_cost == 0 ? 8 : std::min(std::max(o->pair_cost, 0), 1 << 10);
   t.reduce_split = o != nullptr ? std::max(o->reduce_split, 0) : 0;
   t.deterministic = o != nullptr && o->deterministic != 0;
+  t.one_launch = o != nullptr && o->one_launch != 0;
   for (int j = 0; j < 8; ++j) t.xcd_weight[j] = o != nullptr ? std::max(o->xcd_weight[j], 0) : 0;
   return t;
 }
@@ -871,7 +1188,8 @@ Plan MakePlan(const Geom& g, int32_t n_seqs, int32_t max_seq_len, const Tuning& 
   p.share[8] = 8192;
   const size_t parts = (size_t(p.n_chunks) + size_t(n_seqs) * g.n_kv) * p.wpc;
   p.off_tprefix = 0;
-  p.off_ml = Align(sizeof(int32_t) * (size_t(n_seqs) + 1));
+  p.off_tickets = Align(sizeof(int32_t) * (size_t(n_seqs) + 1));
+  p.off_ml = Align(p.off_tickets + sizeof(unsigned long long) * size_t(n_seqs) * g.n_kv);
   p.off_acc = Align(p.off_ml + sizeof(float) * parts * g.group() * 2);
   p.off_stamps = Align(p.off_acc + sizeof(float) * parts * g.group() * g.hd);  // for yahkv_decode_calibrate
   p.bytes = Align(p.off_stamps + 2 * sizeof(unsigned long long) * size_t(p.n_chunks));
@@ -897,6 +1215,7 @@ int Prepare(const yahkv_geometry* g, int32_t page_table_stride, const int32_t* s
   a->max_len = static_cast<int32_t>(std::min<int64_t>(p.max_len, int64_t(page_table_stride) * m.pt));
   char* ws = static_cast<char*>(const_cast<void*>(workspace));
   a->tprefix = reinterpret_cast<int32_t*>(ws + p.off_tprefix);
+  a->tickets = reinterpret_cast<unsigned long long*>(ws + p.off_tickets);
   a->ml = reinterpret_cast<float*>(ws + p.off_ml);
   a->acc = reinterpret_cast<float*>(ws + p.off_acc);
   a->n_chunks = p.n_chunks, a->wpc = p.wpc, a->min_chunk_tiles = p.min_chunk_tiles, a->pair_cost = p.pair_cost;
@@ -979,17 +1298,38 @@ extern "C" int yahkv_decode_reduce(const yahkv_geometry* g, int32_t page_table_s
   return LaunchStatus();
 }
 
+namespace {
+// A number no two launches of this process share (0 is what a ticket holds between launches).
+uint32_t NextEpoch() {
+  static std::atomic<uint32_t> counter{0};
+  uint32_t e = 0;
+  while (e == 0) e = counter.fetch_add(1, std::memory_order_relaxed) + 1;
+  return e;
+}
+}  // namespace
+
+// Two dispatches, partials and their merge; or, if the caller's options ask for it, one: the split-K kernel, whose
+// workgroups then also merge the pairs they are last to finish.
 extern "C" int yahkv_decode_attend(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
                                    int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs,
                                    int32_t max_seq_len, const void* q, int32_t q_dtype, float softmax_scale,
                                    const float* gate, float* out, void* workspace, size_t workspace_bytes,
                                    const yahkv_decode_options* opt, void* stream) {
-  if (out == nullptr) return YAHKV_ERR_ARG;
-  if (const int st = yahkv_decode_part(g, pools, page_table, page_table_stride, seq_len, n_seqs, max_seq_len, q,
-                                       q_dtype, softmax_scale, workspace, workspace_bytes, opt, stream))
+  if (out == nullptr || (reinterpret_cast<uintptr_t>(out) & 15)) return YAHKV_ERR_ARG;
+  if (!MakeTuning(opt).one_launch) {
+    if (const int st = yahkv_decode_part(g, pools, page_table, page_table_stride, seq_len, n_seqs, max_seq_len, q,
+                                         q_dtype, softmax_scale, workspace, workspace_bytes, opt, stream))
+      return st;
+    return yahkv_decode_reduce(g, page_table_stride, seq_len, n_seqs, max_seq_len, gate, out, workspace,
+                               workspace_bytes, opt, stream);
+  }
+  DecodeArgs a;
+  if (const int st = Prepare(g, page_table_stride, seq_len, n_seqs, max_seq_len, workspace, workspace_bytes, opt, &a))
     return st;
-  return yahkv_decode_reduce(g, page_table_stride, seq_len, n_seqs, max_seq_len, gate, out, workspace,
-                             workspace_bytes, opt, stream);
+  if (const int st = CheckPartArgs(g, pools, page_table, q, q_dtype)) return st;
+  a.pools = MakePools(*pools), a.table = page_table, a.q = q, a.q_dtype = q_dtype, a.scale = softmax_scale;
+  a.gate = gate, a.out = out, a.fused = 1, a.epoch = NextEpoch();
+  return LaunchPart(a, static_cast<hipStream_t>(stream));
 }
 
 constexpr int kCalibrationLaunches = 4;  // measured launches per round of yahkv_decode_calibrate
