@@ -23,6 +23,9 @@ def _run(cmd):
     return err
 
 
+EXTRA = os.environ.get("YAHKV_EXTRA_FLAGS", "").split()   # e.g. -DYAHKV_PREFILL_WIDE=1 for the alternative prefill kernel
+
+
 def build(verbose=False, only=None):
     """Every source is compiled (one hipcc per file, side by side) and the objects are linked. `only`: names of the
     sources to compile again, the other objects are taken as they are (for work on one kernel file)."""
@@ -32,7 +35,7 @@ def build(verbose=False, only=None):
     objs = {s: os.path.join(obj_dir, os.path.splitext(s)[0] + ".o") for s in SOURCES}
     todo = [s for s in SOURCES if only is None or s in only or not os.path.exists(objs[s])]
     with ThreadPoolExecutor(max_workers=min(8, len(todo) or 1)) as ex:
-        errs = list(ex.map(lambda s: _run([HIPCC] + FLAGS + inc + ["-c", os.path.join(HERE, "csrc", s), "-o", objs[s]]),
+        errs = list(ex.map(lambda s: _run([HIPCC] + FLAGS + EXTRA + inc + ["-c", os.path.join(HERE, "csrc", s), "-o", objs[s]]),
                            todo))
     errs.append(_run([HIPCC, "--offload-arch=gfx950", "-fPIC", "-shared"] + [objs[s] for s in SOURCES] + ["-o", LIB]))
     if verbose and any(e.strip() for e in errs):

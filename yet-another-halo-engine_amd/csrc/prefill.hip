@@ -423,6 +423,7 @@ struct ImageArgs {
   int32_t n_seqs, max_prefix, chunk_len;
   char* img;
   int32_t tiles_per_pair;
+  int32_t wide;        // V images for the kernel on 32x32x16 matrix instructions (see PrefillAttendWide)
   const uint16_t* fk;  // unquantized f16 pools (PrefillImagesF16 only): K [page][H][D / 16][PT][16], V^T [page][H][PT / R][D][R], R = min(PT, 32)
   const uint16_t* fv;
 };
@@ -478,7 +479,8 @@ __global__ __launch_bounds__(256) void PrefillImages(const ImageArgs a) {
     uint32_t o[4];
 #pragma unroll
     for (int hf = 0; hf < 2; ++hf) {
-      const int kk = tile * kKeys + 32 * s2 + 16 * hf + 4 * jg;  // four keys, always within one page
+      // four keys, always within one page
+      const int kk = tile * kKeys + (a.wide ? 16 * (c / 2) + 8 * hf + 4 * (c % 2) : 32 * s2 + 16 * hf + 4 * jg);
       const size_t ph = page_head(kk);
       const int t = kk % PT;
       const uint2 sw = *reinterpret_cast<const uint2*>(a.pools.vs + (ph * NB + b) * PT + t);
@@ -535,7 +537,8 @@ __global__ __launch_bounds__(256) void PrefillImagesF16(const ImageArgs a) {
     uint32_t o[4];
 #pragma unroll
     for (int hf = 0; hf < 2; ++hf) {
-      const int kk = tile * kKeys + 32 * s2 + 16 * hf + 4 * jg;  // four keys, always within one page
+      // four keys, always within one page
+      const int kk = tile * kKeys + (a.wide ? 16 * (c / 2) + 8 * hf + 4 * (c % 2) : 32 * s2 + 16 * hf + 4 * jg);
       constexpr int RUN = PT < 32 ? PT : 32;  // V^T lies in runs of at most 32 keys
       const uint2 w = *reinterpret_cast<const uint2*>(a.fv + page_head(kk) * (size_t(D) * PT) +
                                                       (size_t(kk % PT / RUN) * D + dim) * RUN + kk % RUN);
@@ -869,12 +872,307 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
   StoreRows<D, RB>(a, s, h, G, jg, o, lacc, qpos, head);
 }
 
+
+// ---- the same attention on 32x32x16 matrix instructions ------------------------------------------------------------------
+//
+// v_mfma_f32_32x32x16_f16 does the work of two 16x16x32 instructions in one issue slot and runs 32 cycles in the matrix
+// pipe, which leaves the wave's other instructions (exponentials, conversions, LDS reads, copies) twice the room between
+// two matrix instructions. A wave owns 32 consecutive chunk positions of one head: the queries are the 32 columns of
+// every product.
+//   S^T[key][q]: A = 32 keys x 16 dims from the K image (lane = key, lane half = which 8 dims), B = Q^T in registers;
+//   the result leaves lane (q, half) with keys 8 i + 4 half + j (i, j < 4) of the 32-key tile in register 4 i + j.
+//   O^T[dim][q] += V^T[dim][key] P^T[key][q]: a step takes 16 keys; the lane half's eight k-slots are the keys of two
+//   consecutive i of the scores it already holds, 16 s + 4 half + j and 16 s + 8 + 4 half + j: P never leaves the
+//   registers, and the V image is written in that order (ImageArgs::wide).
+// The K image is the one of the 16x16x32 kernel. Work split, LDS buffers, copies and the schedule are the same.
+// Measured slower than that kernel (see UseWide): both move the same bytes through LDS per tile (every wave reads the
+// whole K and V tile for its 32 queries, 256 KB per tile and workgroup) and spend the same time in the matrix pipe;
+// this one has half as many independent accumulator chains to put between a read and its use.
+typedef float f16v __attribute__((ext_vector_type(16)));
+
+template <int D>
+__global__ __launch_bounds__(256) void PrefillAttendWide(const PrefillArgs a, const char* img, int tiles_per_pair) {
+  constexpr int KS = D / 16, NDT = D / 32, kHeadsPerGroup = 2;
+  constexpr int KIMG = kKeys * D * 2, TIMG = TileImageBytes<D>();
+  constexpr int kCopies = TIMG / 1024 / 4;  // 1 KB wave-wide copies per wave and tile
+  static_assert(kCopies == KS / 2 + NDT, "one copy per two steps of the first product and per dim tile of the second");
+  const Geom g = a.g;
+  const int G = g.group(), H = g.n_kv;
+  const int n_qt = (a.chunk_len + kQueries - 1) / kQueries, n_hp = (G + kHeadsPerGroup - 1) / kHeadsPerGroup;
+  const int bid = blockIdx.x, xcd = bid % 8, local = bid / 8, per_pair = n_qt * n_hp;
+  const int pair = xcd + 8 * (local / per_pair), qt = n_qt - 1 - (local % per_pair) / n_hp, hp = local % n_hp;
+  if (pair >= a.n_seqs * H) return;
+  const int s = pair / H, h = pair % H;
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / 64), lane = tid % 64;
+  const int qn = lane % 32, h2 = lane / 32;
+  const int prefix = ClampPrefix(a.prefix_len, s, a.max_prefix, a.stride, g.pt, a.chunk_len);
+  const int q0 = qt * kQueries;
+  const int n_keys = min(prefix + q0 + kQueries, prefix + a.chunk_len);
+  const int n_tiles = (n_keys + kKeys - 1) / kKeys;
+  __shared__ __align__(1024) char lds[5][KIMG];  // [0], [1]: K halves; [2] .. [4]: V halves
+
+  const int head = kHeadsPerGroup * hp + wave / 2;
+  const int qpos = q0 + 32 * (wave % 2) + qn;
+  h8v qb[KS];
+  {
+    const int t = min(qpos, a.chunk_len - 1), hd = min(head, G - 1);
+    const uint16_t* qp = a.q + ((size_t(s) * a.chunk_len + t) * g.n_q + size_t(h) * G + hd) * D;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qb[ks] = QueryF16(qp + 16 * ks + 8 * h2);
+  }
+  f16v o[NDT], lacc;
+  float m = kNegBig;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) lacc[r] = 0.0f;
+#pragma unroll
+  for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[dt][r] = 0.0f;
+  const float sscale = a.scale * 1.4426950408889634f;
+  const auto img_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<char*>(img) + size_t(pair) * tiles_per_pair * TIMG, 0, 0x7fffffff, 0x00020000);
+  auto copy_part = [&](int tile, int j) {
+    const int c = wave + 4 * j;
+    char* dst = j < kCopies / 2 ? lds[tile % 2] + c * 1024 : lds[2 + tile % 3] + (c * 1024 - KIMG);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(img_rsrc, (__attribute__((address_space(3))) void*)dst, 16, lane * 16,
+                                             tile * TIMG + c * 1024, 0, 0);
+  };
+  // Operand reads: row = lane % 32 (+ 32 per tile of keys or dims), 16-byte chunk 2 step + half, at the swizzled
+  // position chunk ^ (row % 8). The XOR splits into a per-lane part for each step % 4 and a constant of the instruction.
+  const int x = qn % 8;
+  int koff[4], voff[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int c = 16 * ((h2 ^ (x & 1)) + 2 * (e ^ (x >> 1)));
+    koff[e] = qn * (2 * D) + c, voff[e] = qn * 128 + c;
+  }
+  typedef __attribute__((address_space(3))) const char* LdsPtr;
+  auto read_k = [&](const char* buf, int ks, int kt) -> h8v {
+    return *reinterpret_cast<const h8v*>(buf + koff[ks % 4] + (kt * 32 * (2 * D) + 128 * (ks / 4)));
+  };
+  // The A operands of step ks + KP are read before the products of step ks: a step is two matrix instructions, 64
+  // cycles, and an LDS read takes longer than that to return.
+  constexpr int KP = 3;
+  auto k_step = [&](const char* buf, int ks, h8v (&ka)[KP + 1][2], f16v (&st)[2]) {
+    if (ks + KP < KS) {
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt) ka[(ks + KP) % (KP + 1)][kt] = read_k(buf, ks + KP, kt);
+    }
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+      st[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka[ks % (KP + 1)][kt], qb[ks], st[kt], 0, 0, 0);
+  };
+  auto k_first = [&](const char* buf, h8v (&ka)[KP + 1][2]) {
+#pragma unroll
+    for (int ks = 0; ks < KP; ++ks)
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt) ka[ks][kt] = read_k(buf, ks, kt);
+  };
+  auto clear = [&](f16v (&st)[2]) {
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) st[kt][r] = 0.0f;
+  };
+  auto row_max = [&](const f16v (&st)[2]) -> float {  // over the 64 keys of the tile, times the softmax scale
+    float mx = fmaxf(st[0][0], st[0][1]);
+#pragma unroll
+    for (int r = 2; r < 16; r += 2) mx = fmaxf(fmaxf(mx, st[0][r]), st[0][r + 1]);
+#pragma unroll
+    for (int r = 0; r < 16; r += 2) mx = fmaxf(fmaxf(mx, st[1][r]), st[1][r + 1]);
+    const uint32_t u = __builtin_bit_cast(uint32_t, mx);
+    const auto sw = __builtin_amdgcn_permlane32_swap(u, u, false, false);  // the other half's keys
+    const uint32_t s0 = sw[0], s1 = sw[1];
+    return fmaxf(__builtin_bit_cast(float, s0), __builtin_bit_cast(float, s1)) * sscale;
+  };
+  auto move_reference = [&](float mx) {
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(mx > m + (kBias + kSlack)) != 0, 0)) {
+      const h8v zero = {0, 0, 0, 0, 0, 0, 0, 0};
+      const float mn = mx > m + (kBias + kSlack) ? __builtin_ceilf(mx) - kBias : m;
+      const float alpha = __builtin_amdgcn_exp2f(m - mn);
+      m = mn;
+      {  // (through a matrix instruction with zero factors, so that the accumulators stay where they are: see above)
+        f16v t = lacc;
+        asm volatile("" : "+a"(t));
+#pragma unroll
+        for (int r = 0; r < 16; ++r) t[r] *= alpha;
+        lacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(zero, zero, t, 0, 0, 0);
+      }
+#pragma unroll
+      for (int dt = 0; dt < NDT; ++dt) {
+        f16v t = o[dt];
+        asm volatile("" : "+a"(t));
+#pragma unroll
+        for (int r = 0; r < 16; ++r) t[r] *= alpha;
+        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(zero, zero, t, 0, 0, 0);
+      }
+    }
+  };
+  // f16 numerators as B operands of the second product: step s = 2 kt + u takes registers 8 u .. 8 u + 7 of tile kt
+  auto numerators = [&](const f16v (&st)[2], h8v (&pv)[4]) {
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        uint32_t w[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(st[kt][8 * u + 2 * e], sscale, -m));
+          const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(st[kt][8 * u + 2 * e + 1], sscale, -m));
+          w[e] = PackF16(p0, p1);
+        }
+        pv[2 * kt + u] = __builtin_bit_cast(h8v, uint4{w[0], w[1], w[2], w[3]});
+      }
+  };
+  auto pv_product = [&](auto always, const char* buf, const h8v (&pv)[4], int v_tile) {
+    LdsPtr vb[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) vb[e] = (LdsPtr)buf + voff[e];
+    asm volatile("" : "+v"(vb[0]), "+v"(vb[1]), "+v"(vb[2]), "+v"(vb[3]));
+    auto read_v = [&](int dt, int s_) -> h8v {
+      return *reinterpret_cast<const __attribute__((address_space(3))) h8v*>(vb[s_] + dt * 32 * 128);
+    };
+    constexpr int VA = 2;  // dim tiles the operand reads run ahead
+    h8v va[VA + 1][4];
+#pragma unroll
+    for (int dt = 0; dt < VA; ++dt)
+#pragma unroll
+      for (int s_ = 0; s_ < 4; ++s_) va[dt][s_] = read_v(dt, s_);
+#pragma unroll
+    for (int s_ = 0; s_ < 4; ++s_) lacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(OnesF16(), pv[s_], lacc, 0, 0, 0);
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt) {
+      if (dt + VA < NDT) {
+#pragma unroll
+        for (int s_ = 0; s_ < 4; ++s_) va[(dt + VA) % (VA + 1)][s_] = read_v(dt + VA, s_);
+      }
+#pragma unroll
+      for (int s_ = 0; s_ < 4; ++s_)
+        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va[dt % (VA + 1)][s_], pv[s_], o[dt], 0, 0, 0);
+      if (decltype(always)::value || v_tile >= 0) copy_part(v_tile, KS / 2 + dt);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  const int n_full = min(n_tiles, (prefix + q0 + 1) / kKeys);  // tiles every query of the workgroup sees whole
+  const int n_pipe = min(n_full, n_tiles - 1);
+#pragma unroll
+  for (int j = 0; j < kCopies; ++j) copy_part(0, j);
+#pragma unroll
+  for (int j = 0; j < kCopies; ++j) copy_part(min(1, n_tiles - 1), j);
+  __builtin_amdgcn_s_waitcnt(VmCnt(0));
+  __syncthreads();
+  f16v st[2];
+  clear(st);
+  {
+    h8v ka[KP + 1][2];
+    k_first(lds[0], ka);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      k_step(lds[0], ks, ka, st);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  int tile = 0;
+  constexpr int KA = KS / 4;  // steps of the next tile's first product that run beside the row maximum
+  for (; tile < n_pipe; ++tile) {
+    const char* kbuf = lds[(tile + 1) % 2];
+    const int k_tile = min(tile + 2, n_tiles - 1);
+    f16v sn[2];
+    clear(sn);
+    h8v ka[KP + 1][2];
+    h8v pv[4];
+    k_first(kbuf, ka);
+#pragma unroll
+    for (int ks = 0; ks < KA; ++ks) {
+      k_step(kbuf, ks, ka, sn);
+      if (ks % 2 == 1) copy_part(k_tile, ks / 2);
+    }
+    const float mx = row_max(st);
+    __builtin_amdgcn_sched_barrier(0);
+    move_reference(mx);
+#pragma unroll
+    for (int ks = KA; ks < KS; ++ks) {
+      k_step(kbuf, ks, ka, sn);
+      if (ks % 2 == 1) copy_part(k_tile, ks / 2);
+    }
+    numerators(st, pv);
+    __builtin_amdgcn_sched_barrier(0);
+    pv_product(Constant<true>{}, lds[2 + tile % 3], pv, min(tile + 2, n_tiles - 1));
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) st[kt] = sn[kt];
+    __builtin_amdgcn_s_waitcnt(VmCnt(kCopies / 2) & 0xF0FF);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  }
+  for (; tile < n_tiles; ++tile) {
+    const bool more = tile + 1 < n_tiles;
+    if ((tile + 1) * kKeys > prefix + q0 + 1) {
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          if (tile * kKeys + 32 * kt + 8 * (r / 4) + 4 * h2 + r % 4 > prefix + qpos) st[kt][r] = kNegBig;
+    }
+    h8v pv[4];
+    move_reference(row_max(st));
+    numerators(st, pv);
+    pv_product(Constant<false>{}, lds[2 + tile % 3], pv, tile + 2 < n_tiles ? tile + 2 : -1);
+    if (more) {
+      const char* kbuf = lds[(tile + 1) % 2];
+      clear(st);
+      h8v ka[KP + 1][2];
+      k_first(kbuf, ka);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        k_step(kbuf, ks, ka, st);
+        if (tile + 2 < n_tiles && ks % 2 == 1) copy_part(tile + 2, ks / 2);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    __builtin_amdgcn_s_waitcnt(VmCnt(0));
+    __syncthreads();
+  }
+  // out = o / l (* sigmoid(gate)): lane (q, half) holds dims 32 dt + 8 i + 4 half + j of its query in register 4 i + j
+  if (head < G && qpos < a.chunk_len) {
+    const float inv = 1.0f / lacc[0];
+    const size_t base = ((size_t(s) * a.chunk_len + qpos) * g.n_q + size_t(h) * G + head) * D;
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const size_t e = base + 32 * dt + 8 * i + 4 * h2;
+        float v[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          v[j] = o[dt][4 * i + j] * inv;
+          if (a.gate != nullptr) v[j] *= 1.0f / (1.0f + __expf(-a.gate[e + j]));
+        }
+        if (a.out_dtype == YAHKV_F32) {
+          *reinterpret_cast<float4*>(static_cast<float*>(a.out) + e) = float4{v[0], v[1], v[2], v[3]};
+        } else if (a.out_dtype == YAHKV_BF16) {
+          *reinterpret_cast<uint2*>(static_cast<uint16_t*>(a.out) + e) = uint2{PackBf16(v[0], v[1]), PackBf16(v[2], v[3])};
+        } else {
+          *reinterpret_cast<uint2*>(static_cast<uint16_t*>(a.out) + e) = uint2{PackF16(v[0], v[1]), PackF16(v[2], v[3])};
+        }
+      }
+  }
+}
+
 }  // namespace
 }  // namespace yahkv
 
 using namespace yahkv;
 
 namespace {
+#ifndef YAHKV_PREFILL_WIDE
+#define YAHKV_PREFILL_WIDE 0
+#endif
+// Which attention kernel serves a geometry, and with it the order of the keys in the V images. The kernel on 32x32x16
+// matrix instructions (head_dim 256 only) is built in with -DYAHKV_PREFILL_WIDE=1; it gives the same results and is
+// measured slower than the one on 16x16x32 (8 x (16384 + 2048) tokens: 6.66 ms against 5.87 ms), so it is off.
+bool UseWide(const Geom& m) { return YAHKV_PREFILL_WIDE && m.hd == 256; }
 int32_t TilesPerPair(int32_t max_prefix_len, int32_t chunk_len) {
   return static_cast<int32_t>((int64_t(max_prefix_len) + chunk_len + kKeys - 1) / kKeys);
 }
@@ -940,6 +1238,7 @@ extern "C" int yahkv_prefill_decode_tiles(const yahkv_geometry* g, const yahkv_p
   ia.g = m, ia.pools = a.pools, ia.table = page_table, ia.stride = page_table_stride, ia.prefix_len = prefix_len;
   ia.n_seqs = n_seqs, ia.max_prefix = max_prefix_len, ia.chunk_len = chunk_len;
   ia.img = static_cast<char*>(workspace), ia.tiles_per_pair = TilesPerPair(max_prefix_len, chunk_len);
+  ia.wide = UseWide(m);
   const dim3 igrid(static_cast<unsigned>(ia.tiles_per_pair), static_cast<unsigned>(n_seqs * m.n_kv));
   hipStream_t st = static_cast<hipStream_t>(stream);
 #define YAHKV_LAUNCH_IMG(FF, DD, PP) hipLaunchKernelGGL((PrefillImages<FF, DD, PP>), igrid, dim3(256), 0, st, ia)
@@ -983,7 +1282,8 @@ extern "C" int yahkv_prefill_attend_tiles(const yahkv_geometry* g, const yahkv_p
   // (At head_dim 256 three blocks' accumulators and query operands do not fit the register file: 140 spills.)
 #define YAHKV_LAUNCH_ATT(DD, RR) \
   hipLaunchKernelGGL((PrefillAttendImg<DD, RR>), AttendGrid(a, RR), dim3(256), 0, st, a, img, tiles)
-  if (a.g.hd == 256) YAHKV_LAUNCH_ATT(256, 2);
+  if (UseWide(a.g)) hipLaunchKernelGGL((PrefillAttendWide<256>), AttendGrid(a, 2), dim3(256), 0, st, a, img, tiles);
+  else if (a.g.hd == 256) YAHKV_LAUNCH_ATT(256, 2);
   else if (a.g.group() % 3 == 0) YAHKV_LAUNCH_ATT(128, 3);
   else YAHKV_LAUNCH_ATT(128, 2);
 #undef YAHKV_LAUNCH_ATT
@@ -1065,7 +1365,7 @@ extern "C" int yahkv_f16_prefill_attend(const yahkv_geometry* g, const yahkv_f16
   ImageArgs ia{};
   ia.g = a.g, ia.table = page_table, ia.stride = page_table_stride, ia.prefix_len = prefix_len, ia.n_seqs = n_seqs;
   ia.max_prefix = max_prefix_len, ia.chunk_len = chunk_len, ia.img = static_cast<char*>(workspace);
-  ia.tiles_per_pair = tiles;
+  ia.tiles_per_pair = tiles, ia.wide = UseWide(a.g);
   ia.fk = static_cast<const uint16_t*>(pools->k), ia.fv = static_cast<const uint16_t*>(pools->v);
   const dim3 igrid(static_cast<unsigned>(tiles), static_cast<unsigned>(n_seqs * a.g.n_kv));
   hipStream_t st = static_cast<hipStream_t>(stream);
@@ -1081,7 +1381,8 @@ extern "C" int yahkv_f16_prefill_attend(const yahkv_geometry* g, const yahkv_f16
   const char* img = static_cast<const char*>(workspace);
 #define YAHKV_LAUNCH_ATT(DD, RR) \
   hipLaunchKernelGGL((PrefillAttendImg<DD, RR>), AttendGrid(a, RR), dim3(256), 0, st, a, img, tiles)
-  if (a.g.hd == 256) YAHKV_LAUNCH_ATT(256, 2);
+  if (UseWide(a.g)) hipLaunchKernelGGL((PrefillAttendWide<256>), AttendGrid(a, 2), dim3(256), 0, st, a, img, tiles);
+  else if (a.g.hd == 256) YAHKV_LAUNCH_ATT(256, 2);
   else if (a.g.group() % 3 == 0) YAHKV_LAUNCH_ATT(128, 3);
   else YAHKV_LAUNCH_ATT(128, 2);
 #undef YAHKV_LAUNCH_ATT
