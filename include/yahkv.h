@@ -190,7 +190,7 @@ int yahkv_decode_attend(const yahkv_geometry* g, const yahkv_pools* pools, const
                         const void* q, int32_t q_dtype, float softmax_scale, const float* gate, float* out,
                         void* workspace, size_t workspace_bytes, const yahkv_decode_options* opt, void* stream);
 /* Measures the relative read speeds of the GPU's eight XCDs on the caller's own batch and writes them to
- * opt->xcd_weight (the other fields are read): `rounds` times, the split-K kernel runs five times on the given arguments and
+ * opt->xcd_weight (the other fields are read): `rounds` times, the split-K kernel runs nine times on the given arguments and
  * the shares are corrected by when each XCD's workgroups finished. A set-up call: it synchronizes the stream and
  * overwrites the workspace. No counterpart in the reference (one sequence, one workgroup per page). */
 int yahkv_decode_calibrate(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
@@ -218,18 +218,21 @@ int yahkv_decode_attend_static(const yahkv_geometry* g, const yahkv_pools* pools
  *   q    [n_seqs][chunk_len][n_q_heads][D] bf16
  *   gate [n_seqs][chunk_len][n_q_heads][D] f32 or NULL
  *   out  [n_seqs][chunk_len][n_q_heads][D] of out_dtype (F32, F16 or BF16)
- * prefix_len is device int32 [n_seqs]; max_prefix_len is its host-side upper bound; softmax_scale > 0. K, V and
- * the softmax numerators enter the matrix unit as bf16 (round to nearest even), sums are f32.
- * With a workspace of yahkv_prefill_workspace_bytes() the prefix is decoded to bf16 once per call and the attention
+ * prefix_len is device int32 [n_seqs]; max_prefix_len is its host-side upper bound; softmax_scale > 0. K, V, the
+ * queries and the softmax numerators enter the matrix unit as f16 (round to nearest even; finite values beyond
+ * +-65504 saturate there), as in the reference's kernel (gen_attn_fa.py:1252-1595); sums are f32. The result lies
+ * within 2e-3 (max |error| / max |value|) of exact arithmetic on the dequantized K / V for F32 and F16 output; BF16
+ * output adds its own rounding, up to 2^-8 of an element.
+ * With a workspace of yahkv_prefill_workspace_bytes() the prefix is decoded to f16 once per call and the attention
  * kernel reads the decoded tiles (the reference's yah_kdeq8 / yah_vdeq8 into a 16-bit pool followed by yah_attn_wmma,
  * gen_attn_fa.py:4648-4861, 1589-1595); q8_0 and q4_0. With workspace NULL the tiles are decoded inside the attention
- * kernel while they are staged (gen_attn_fa.py:2664-2779): no extra memory, slower, q8_0 only
- * (q4_0: YAHKV_ERR_WORKSPACE). Both give the same results up to the order of f32 sums. */
+ * kernel while they are staged (gen_attn_fa.py:2664-2779, vq4_unpack for the 4-bit codes): no extra memory, slower.
+ * Both give the same results up to the order of f32 sums. */
 size_t yahkv_prefill_workspace_bytes(const yahkv_geometry* g, int32_t n_seqs, int32_t max_prefix_len,
                                      int32_t chunk_len);
 /* The two dispatches of the workspace path, for callers that queue them separately (as the reference does with
  * yah_kdeq8 / yah_vdeq8 and yah_attn_wmma, loom_prefill.hpp:3378-3416): decode keys 0 .. prefix_len[s] + chunk_len
- * of every sequence into bf16 tiles in the workspace; then attention of the chunk's queries over those tiles. The
+ * of every sequence into f16 tiles in the workspace; then attention of the chunk's queries over those tiles. The
  * tiles stay valid for further queries of the same chunk (e.g. another slice of heads) until the pools change.
  * One sequence's tiles of one kv head must stay under 2 GiB (max_prefix_len + chunk_len up to 2^21 tokens at
  * head_dim 256, 2^22 at 128): longer ones return YAHKV_ERR_SHAPE. */
@@ -328,7 +331,7 @@ int yahkv_f16_decode_attend(const yahkv_geometry* g, const yahkv_f16_pools* pool
                             const void* q, int32_t q_dtype, float softmax_scale, const float* gate, float* out,
                             void* workspace, size_t workspace_bytes, const yahkv_decode_options* opt, void* stream);
 /* Chunked-prefill attention over f16 pools after the chunk has been appended with yahkv_f16_append (arguments as
- * yahkv_prefill_attend; the workspace is required): the keys' bf16 tiles are converted from the pools (the reference's
+ * yahkv_prefill_attend; the workspace is required): the keys' f16 tiles are put together from the pools (the reference's
  * attention reads its 16-bit K / V pool directly, gen_attn_fa.py:1589-1595), then the same attention kernel runs. */
 size_t yahkv_f16_prefill_workspace_bytes(const yahkv_geometry* g, int32_t n_seqs, int32_t max_prefix_len,
                                          int32_t chunk_len);

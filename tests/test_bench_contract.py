@@ -46,6 +46,12 @@ def test_decode_line_has_the_fields_a_driver_reads():
         assert k in d["cpu_baseline"], k
     assert d["cpu_baseline"]["kind"] in ("port", "reference") and d["cpu_baseline"]["cores"] >= 1
     assert d["parity_max_rel_err"] < 2e-3
+    # the other configurations that fill a GPU are timed by the same run, into one object of the same line
+    assert sorted(d["also"]) == ["b16_ctx128k_q4_0", "b1_ctx32k_q8_0", "prefill_b8_ctx16k_chunk2k_q8_0"]
+    for name, r in d["also"].items():
+        assert r["value"] > 0 and r["ms_per_step"] > 0 and r["parity_max_rel_err"] < 2e-3, name
+        assert 0.0 < r["roofline"]["frac"] < 1.0 and r["roofline"]["bound"] == ("mfma" if "prefill" in name else "hbm")
+    assert "config1_tiny" in d["cpu_baseline"]["configs"] and "config2_b1_ctx32k" in d["cpu_baseline"]["configs"]
 
 
 @pytest.mark.gpu
@@ -54,4 +60,5 @@ def test_prefill_line():
     for k in COMMON + ("append",):
         assert k in d, k
     assert d["unit"] == "TFLOP/s" and d["roofline"]["bound"] == "mfma" and d["roofline"]["peak"] == 2500.0
+    assert d["dtype"] == "f16" and d["parity_max_rel_err"] < 2e-3
     assert 0.0 < d["roofline"]["frac"] < 1.0 and 0.0 < d["append"]["frac_of_hbm_peak"] < 1.0

@@ -35,7 +35,7 @@ def build(yahkv, torch, fmt, n_q, n_kv, hd, pt, prefix, chunk, seed, fill=0):
     return g, table, host, dev, t_table, rng, to_t
 
 
-# path "images": decode to f16 tile images in a workspace, then attention; "fused": one kernel, no workspace (q8_0)
+# path "images": decode to f16 tile images in a workspace, then attention; "fused": one kernel, no workspace
 @pytest.mark.parametrize("path,fmt,n_q,n_kv,hd,pt,prefix,chunk", [
     ("images", 8, 24, 4, 256, 64, [100, 0, 64 * 3 + 5], 70),
     ("images", 8, 24, 4, 256, 64, [1000], 256),
@@ -52,6 +52,9 @@ def build(yahkv, torch, fmt, n_q, n_kv, hd, pt, prefix, chunk, seed, fill=0):
     ("fused", 8, 8, 2, 128, 16, [37, 0, 64], 21),
     ("fused", 8, 6, 2, 256, 32, [31, 500], 64),
     ("fused", 8, 10, 2, 128, 64, [129], 130),
+    ("fused", 4, 24, 4, 256, 64, [100, 0, 64 * 3 + 5], 70),
+    ("fused", 4, 8, 2, 128, 16, [37, 0, 64], 21),
+    ("fused", 4, 6, 2, 256, 32, [31, 500], 64),
 ])
 def test_prefill_against_oracle(yahkv, torch_gpu, path, fmt, n_q, n_kv, hd, pt, prefix, chunk):
     torch = torch_gpu
@@ -130,9 +133,6 @@ def test_prefill_rejects_bad_arguments(yahkv, torch_gpu):
     table = torch.zeros((1, 4), dtype=torch.int32, device="cuda")
     q = torch.zeros((1, 8, 24, 256), dtype=torch.bfloat16, device="cuda")
     zero = torch.zeros(1, dtype=torch.int32, device="cuda")
-    with pytest.raises(yahkv.YahkvError) as e:                                    # q4_0 needs the workspace
-        yahkv.prefill_attend(dev, table, zero, 0, q, 0.0625, workspace=False)
-    assert e.value.status == -4
     with pytest.raises(yahkv.YahkvError) as e:                                    # workspace too small
         yahkv.prefill_attend(dev, table, zero, 0, q, 0.0625, workspace=torch.empty(256, dtype=torch.uint8, device="cuda"))
     assert e.value.status == -4

@@ -425,7 +425,7 @@ def prefill_attend(pools, table, prefix_len, max_prefix_len, q, scale, gate=None
     """q: [n_seqs][chunk][n_q_heads][D] bf16; returns out (f32 unless out / out_dtype say otherwise), same shape.
 
     workspace: a uint8 device tensor of prefill_workspace_bytes() (None: one is allocated for the call) selects the
-    two-pass path, decode to bf16 tile images and then attention; False selects the one-pass kernel (q8_0 only)."""
+    two-pass path, decode to f16 tile images and then attention; False selects the one-pass kernel."""
     import torch
     g = pools.geom
     assert q.is_contiguous() and q.dtype == torch.bfloat16 and table.is_contiguous()

@@ -1332,13 +1332,13 @@ extern "C" int yahkv_decode_attend(const yahkv_geometry* g, const yahkv_pools* p
   return LaunchPart(a, static_cast<hipStream_t>(stream));
 }
 
-constexpr int kCalibrationLaunches = 4;  // measured launches per round of yahkv_decode_calibrate
+constexpr int kCalibrationLaunches = 8;  // measured launches per round of yahkv_decode_calibrate
 
 // Relative read speeds of the eight XCDs on the caller's own batch. Workgroup k of a dispatch runs on XCD k % 8, and the
 // XCDs of one GPU do not read memory equally fast (up to 10 % apart, measured); chunk shares that follow their speeds
-// let all workgroups finish together. Each round runs the part kernel five times with the current shares (the first
+// let all workgroups finish together. Each round runs the part kernel nine times with the current shares (the first
 // launch warms caches and clocks), reads when each workgroup's last wave finished, and sets every XCD's weight to its
-// share divided by its mean time over the four measured launches. Synchronizes the stream: a set-up call, not part of a step.
+// share divided by its mean time over the eight measured launches. Synchronizes the stream: a set-up call, not part of a step.
 extern "C" int yahkv_decode_calibrate(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
                                       int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs,
                                       int32_t max_seq_len, const void* q, int32_t q_dtype, void* workspace,

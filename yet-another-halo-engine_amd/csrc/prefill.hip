@@ -78,10 +78,14 @@ __device__ __forceinline__ uint32_t PackBf16(float a, float b) {  // round to ne
   return __builtin_bit_cast(uint32_t, v);
 }
 
-// Sixteen int8 codes times one scale, as sixteen f16 (two 16-byte halves).
-__device__ __forceinline__ void Decode16(const uint4 c, float d, uint4* lo, uint4* hi) {
-  const uint32_t w[4] = {c.x ^ 0x80808080u, c.y ^ 0x80808080u, c.z ^ 0x80808080u, c.w ^ 0x80808080u};
-  const float off = -128.0f * d;
+// Sixteen codes times one scale, as sixteen f16 (two 16-byte halves). q8_0: sixteen int8 codes. q4_0: the low
+// (SHIFT 0) or high (SHIFT 4) nibbles of a block's sixteen bytes, value (n - 8) * d.
+template <int FMT>
+__device__ __forceinline__ void Decode16(const uint4 c, float d, int shift, uint4* lo, uint4* hi) {
+  uint32_t w[4] = {c.x, c.y, c.z, c.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) w[i] = FMT == 8 ? w[i] ^ 0x80808080u : (w[i] >> shift) & 0x0F0F0F0Fu;
+  const float off = (FMT == 8 ? -128.0f : -8.0f) * d;
   uint32_t o[8];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {  // v_cvt_f32_ubyteN on code + 128, then one fma brings it back and scales it
@@ -93,17 +97,21 @@ __device__ __forceinline__ void Decode16(const uint4 c, float d, uint4* lo, uint
   }
   *lo = uint4{o[0], o[1], o[2], o[3]}, *hi = uint4{o[4], o[5], o[6], o[7]};
 }
-// Sixteen int8 codes of one dim, sixteen keys, each with its own scale.
-__device__ __forceinline__ void Decode16V(const uint4 c, const uint4 s0, const uint4 s1, uint4* lo, uint4* hi) {
-  const uint32_t w[4] = {c.x ^ 0x80808080u, c.y ^ 0x80808080u, c.z ^ 0x80808080u, c.w ^ 0x80808080u};
+// Sixteen codes of one dim, sixteen keys, each with its own scale (q4_0: one nibble of the sixteen bytes of a byte row).
+template <int FMT>
+__device__ __forceinline__ void Decode16V(const uint4 c, const uint4 s0, const uint4 s1, int shift, uint4* lo, uint4* hi) {
+  uint32_t w[4] = {c.x, c.y, c.z, c.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) w[i] = FMT == 8 ? w[i] ^ 0x80808080u : (w[i] >> shift) & 0x0F0F0F0Fu;
+  constexpr float kZero = FMT == 8 ? -128.0f : -8.0f;
   const uint32_t sw[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
   uint32_t o[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     const float d0 = WidenF16(static_cast<uint16_t>(sw[i] & 0xFFFF)), d1 = WidenF16(static_cast<uint16_t>(sw[i] >> 16));
     const uint32_t b0 = (w[i / 2] >> (16 * (i % 2))) & 0xFF, b1 = (w[i / 2] >> (16 * (i % 2) + 8)) & 0xFF;
-    o[i] = PackF16Sat(__builtin_fmaf(static_cast<float>(b0), d0, -128.0f * d0),
-                      __builtin_fmaf(static_cast<float>(b1), d1, -128.0f * d1));
+    o[i] = PackF16Sat(__builtin_fmaf(static_cast<float>(b0), d0, kZero * d0),
+                      __builtin_fmaf(static_cast<float>(b1), d1, kZero * d1));
   }
   *lo = uint4{o[0], o[1], o[2], o[3]}, *hi = uint4{o[4], o[5], o[6], o[7]};
 }
@@ -145,8 +153,8 @@ __device__ __forceinline__ void StoreRows(const PrefillArgs& a, int s, int h, in
   }
 }
 
-template <int D, int PT>
-__global__ __launch_bounds__(256) void PrefillAttendQ8(const PrefillArgs a) {
+template <int FMT, int D, int PT>
+__global__ __launch_bounds__(256) void PrefillAttendFused(const PrefillArgs a) {
   constexpr int NB = D / 32, NDT = D / 16, KS = D / 32;  // blocks, 16-dim tiles, 32-dim steps of the first product
   constexpr int RB = kFusedRowBlocks, kHeadsPerGroup = RB;  // 4 waves x RB row blocks = 64 positions x RB heads
   constexpr int KSTR = D + 8, VSTR = kKeys + 8;          // LDS row strides (f16), padded against bank conflicts
@@ -210,14 +218,16 @@ __global__ __launch_bounds__(256) void PrefillAttendQ8(const PrefillArgs a) {
       const int c = tid + 256 * j, b = c / 128, key = (c % 128) / 2, hf = c % 2;
       const int kk = min(tile * kKeys + key, a.stride * PT - 1);
       const size_t ph = page_head(kk);
-      kraw[j] = *reinterpret_cast<const uint4*>(a.pools.kq + ((ph * NB + b) * PT + kk % PT) * 32 + 16 * hf);
+      // q8_0: this half's sixteen codes; q4_0: the block's sixteen bytes (this half is one nibble of each)
+      kraw[j] = FMT == 8 ? *reinterpret_cast<const uint4*>(a.pools.kq + ((ph * NB + b) * PT + kk % PT) * 32 + 16 * hf)
+                         : *reinterpret_cast<const uint4*>(a.pools.kq + ((ph * NB + b) * PT + kk % PT) * 16);
       ksr[j] = a.pools.ks[(ph * PT + kk % PT) * NB + b];
     }
   };
   auto stage_k = [&](int j) {
     const int c = tid + 256 * j, b = c / 128, key = (c % 128) / 2, hf = c % 2;
     uint4 lo, hi;
-    Decode16(kraw[j], WidenF16(ksr[j]), &lo, &hi);
+    Decode16<FMT>(kraw[j], WidenF16(ksr[j]), 4 * hf, &lo, &hi);
     uint4* dst = reinterpret_cast<uint4*>(&lk[key][32 * b + 16 * hf]);
     dst[0] = lo, dst[1] = hi;
   };
@@ -226,7 +236,10 @@ __global__ __launch_bounds__(256) void PrefillAttendQ8(const PrefillArgs a) {
     for (int j = 0; j < KCH; ++j) {
       const int c = tid + 256 * j, d = c / 4, k0 = 16 * (c % 4);
       const int kk = min(tile * kKeys + k0, a.stride * PT - 16);
-      vraw[j] = *reinterpret_cast<const uint4*>(a.pools.vq + (page_head(kk) * D + d) * PT + kk % PT);
+      // q4_0: byte row d % 16 of block d / 32 holds dims d % 16 (low nibbles) and 16 + d % 16 (high) of the block
+      vraw[j] = FMT == 8 ? *reinterpret_cast<const uint4*>(a.pools.vq + (page_head(kk) * D + d) * PT + kk % PT)
+                         : *reinterpret_cast<const uint4*>(a.pools.vq + ((page_head(kk) * NB + d / 32) * 16 + d % 16) * PT +
+                                                           kk % PT);
     }
   };
   auto fetch_vs = [&](int tile) {  // the tile's V scales: thread = (block, 8 keys)
@@ -252,7 +265,7 @@ __global__ __launch_bounds__(256) void PrefillAttendQ8(const PrefillArgs a) {
     const int c = tid + 256 * j, d = c / 4, k0 = 16 * (c % 4);
     const uint4* sp = reinterpret_cast<const uint4*>(&lvs[d / 32][k0]);
     uint4 lo, hi;
-    Decode16V(vraw[j], sp[0], sp[1], &lo, &hi);
+    Decode16V<FMT>(vraw[j], sp[0], sp[1], d % 32 / 16 * 4, &lo, &hi);
     uint4* dst = reinterpret_cast<uint4*>(&lv[d][k0]);
     dst[0] = lo, dst[1] = hi;
   };
@@ -1310,16 +1323,22 @@ extern "C" int yahkv_prefill_attend(const yahkv_geometry* g, const yahkv_pools* 
     return rc;
   if (const int rc = PrepareQueries(q, softmax_scale, gate, out, out_dtype, &a)) return rc;
   const Geom& m = a.g;
-  if (m.format != 8) return YAHKV_ERR_WORKSPACE;  // q4_0 pools are only served through the tile images
   const dim3 grid = AttendGrid(a, kFusedRowBlocks);
   hipStream_t st = static_cast<hipStream_t>(stream);
-#define YAHKV_LAUNCH_PF(DD, PP) hipLaunchKernelGGL((PrefillAttendQ8<DD, PP>), grid, dim3(256), 0, st, a)
-  if (m.hd == 256 && m.pt == 64) YAHKV_LAUNCH_PF(256, 64);
-  else if (m.hd == 256 && m.pt == 32) YAHKV_LAUNCH_PF(256, 32);
-  else if (m.hd == 256) YAHKV_LAUNCH_PF(256, 16);
-  else if (m.pt == 64) YAHKV_LAUNCH_PF(128, 64);
-  else if (m.pt == 32) YAHKV_LAUNCH_PF(128, 32);
-  else YAHKV_LAUNCH_PF(128, 16);
+#define YAHKV_LAUNCH_PF(FF, DD, PP) hipLaunchKernelGGL((PrefillAttendFused<FF, DD, PP>), grid, dim3(256), 0, st, a)
+#define YAHKV_LAUNCH_PF_FMT(FF)                                      \
+  if (m.hd == 256 && m.pt == 64) YAHKV_LAUNCH_PF(FF, 256, 64);          \
+  else if (m.hd == 256 && m.pt == 32) YAHKV_LAUNCH_PF(FF, 256, 32);     \
+  else if (m.hd == 256) YAHKV_LAUNCH_PF(FF, 256, 16);                   \
+  else if (m.pt == 64) YAHKV_LAUNCH_PF(FF, 128, 64);                    \
+  else if (m.pt == 32) YAHKV_LAUNCH_PF(FF, 128, 32);                    \
+  else YAHKV_LAUNCH_PF(FF, 128, 16)
+  if (m.format == 8) {
+    YAHKV_LAUNCH_PF_FMT(8);
+  } else {
+    YAHKV_LAUNCH_PF_FMT(4);
+  }
+#undef YAHKV_LAUNCH_PF_FMT
 #undef YAHKV_LAUNCH_PF
   return LaunchStatus();
 }
