@@ -314,7 +314,7 @@ def run_f16(a, wl, torch, yahkv):
 
 
 def run_prefill(a, wl, torch, yahkv):
-    """A step: quantize + scatter one chunk per sequence, decode prefix + chunk to bf16 tiles, causal attention."""
+    """A step: quantize + scatter one chunk per sequence, decode prefix + chunk to f16 tiles, causal attention."""
     g, layers, lens, table, t_table, gen = build_state(yahkv, torch, wl, 0)
     pools = layers[0]
     B, chunk, prefix = wl["batch"], wl["chunk"], int(lens.max())
@@ -405,7 +405,7 @@ def run_prefill(a, wl, torch, yahkv):
 
 def run_prefill_f16(a, wl, torch, yahkv):
     """The prefill step on unquantized f16 pools: append the chunk, then one call that converts prefix + chunk to
-    bf16 tiles and runs the causal attention."""
+    f16 tiles and runs the causal attention."""
     B, chunk, prefix = wl["batch"], wl["chunk"], wl["lo"]
     rng = np.random.default_rng(wl["seed"])
     per_seq = (prefix + chunk + PT - 1) // PT
