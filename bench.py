@@ -488,7 +488,10 @@ def run_prefill_f16(a, wl, torch, yahkv):
 
 
 def run_decode(a, wl, torch, yahkv):
-    """A step on quantized pools: append one token per sequence, split-K partials, their merge."""
+    """A step on quantized pools: one new token per sequence and the attention over the sequence with it. Two dispatches
+    (yahkv_decode_step's): split-K partials over the tokens already in the pools, then the merge, which also quantizes
+    the new token, writes it to its page and adds its term. --separate-append: three dispatches, the reference's order
+    (append, partials, merge)."""
     total = a.warmup + a.steps + 1
     g, layers, lens, table, t_table, gen = build_state(yahkv, torch, wl, total)
     pools = layers[0]
@@ -507,10 +510,20 @@ def run_decode(a, wl, torch, yahkv):
     # set-up, as a server does once: the XCDs' relative read speeds on this batch (equal shares without it)
     xcd = yahkv.decode_calibrate(pools, t_table, len_rows[0], max_len, q, ws, opt, rounds=3) if not a.no_calibrate else None
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(a.steps)]
+    separate = a.separate_append or a.one_launch
 
     def step(i, pair=None):
         seq_len = len_rows[i + 1]
         pools = layers[i % len(layers)]     # (with several layers a layer sees every n-th token; the others stay zero blocks)
+        if not separate:
+            if pair:
+                pair[0].record()
+            yahkv.decode_part(pools, t_table, len_rows[i], max_len, q, scale, ws, opt=opt)   # the tokens before the step
+            if pair:
+                pair[1].record()
+            yahkv.decode_step_reduce(pools, t_table, seq_len, max_len, knew[i][:, 0], vnew[i][:, 0], q, scale, out, ws,
+                                     opt=opt)
+            return
         yahkv.append(pools, t_table, len_rows[i], knew[i], vnew[i])    # position = current length (device-resident)
         if pair:
             pair[0].record()
@@ -552,7 +565,8 @@ def run_decode(a, wl, torch, yahkv):
     ms = dt / a.steps * 1e3
     kern_ms = float(np.mean([p[0].elapsed_time(p[1]) for p in ev[::EVENT_EVERY]]))
     gbs = kv_bytes / (ms * 1e-3) / 1e9
-    kgbs = kv_bytes / (kern_ms * 1e-3) / 1e9
+    # (in the two-dispatch step the split-K kernel runs over the tokens before the step's own: one fewer per sequence)
+    kgbs = (kv_bytes - (0 if separate else B * bpt)) / (kern_ms * 1e-3) / 1e9
     res = {
         "metric": ("paged q8 KV decode-attn HBM GB/s (% of peak) + tok/s, B=64 ragged ctx"
                    if a.workload == "ragged_b64_q8_0" else
@@ -564,7 +578,9 @@ def run_decode(a, wl, torch, yahkv):
                    "ctx_sum": int(lens.sum()), "n_q_heads": NQ, "n_kv_heads": NKV, "head_dim": HD, "page_tokens": PT,
                    "n_pages": g.n_pages, "layers_rotated": len(layers), "kv_format": "q8_0" if wl["fmt"] == 8 else "q4_0",
                    "step": "append 1 token/seq + paged decode attention (%s)" %
-                           ("one launch" if a.one_launch else "part + reduce"), "xcd_weight": xcd},
+                           ("append, one launch for part and merge" if a.one_launch else
+                            "append, part, reduce" if separate else "part, reduce with the append in it"),
+                   "xcd_weight": xcd},
         "pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2), "tok_per_s": round(B / (ms * 1e-3), 1),
         "kv_bytes_per_step": int(kv_bytes), "parity_max_rel_err": float(f"{err:.3e}"), "out_fnv1a": first_hash,
         "roofline": {"bound": "hbm", "achieved": round(kgbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
@@ -630,6 +646,8 @@ def main():
                     help="decode workloads: opt.deterministic (fixed tile pattern per wave: same bytes in, same bits out)")
     ap.add_argument("--one-launch", action="store_true",
                     help="decode workloads: yahkv_decode_attend with opt.one_launch instead of part + reduce")
+    ap.add_argument("--separate-append", action="store_true",
+                    help="decode workloads: the step's token is appended by a dispatch of its own (three per step)")
     ap.add_argument("--graph-replay", action="store_true",
                     help="decode workloads: also replay the timed steps as one HIP graph and report its time per step")
     ap.add_argument("--copy-calibration", action="store_true",

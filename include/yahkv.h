@@ -189,6 +189,27 @@ int yahkv_decode_attend(const yahkv_geometry* g, const yahkv_pools* pools, const
                         int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs, int32_t max_seq_len,
                         const void* q, int32_t q_dtype, float softmax_scale, const float* gate, float* out,
                         void* workspace, size_t workspace_bytes, const yahkv_decode_options* opt, void* stream);
+/* One decode step of a layer, LoomDecoder::Step's sequence kappend, vappend, part_q, reduce
+ * (loom_decoder.hpp:253-268), in two dispatches: the result is that of yahkv_append(n_new = 1, start_pos =
+ * seq_len - 1) followed by yahkv_decode_attend, pools and output. seq_len[s] counts the step's own token, which goes
+ * to position seq_len[s] - 1 (clamped to the table like every position); a sequence with seq_len[s] <= 0 gets no
+ * token and rows of zeros. k_new, v_new: [n_seqs][H][D] of new_dtype (F32, F16 or BF16), 16-byte aligned. The split-K
+ * dispatch runs over the tokens the pools already hold; the merge quantizes the new token (the append kernels'
+ * arithmetic, bit for bit), writes it to its slot and adds its term. opt->one_launch is refused (YAHKV_ERR_ARG). */
+int yahkv_decode_step(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
+                      int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs, int32_t max_seq_len,
+                      const void* k_new, const void* v_new, int32_t new_dtype, const void* q, int32_t q_dtype,
+                      float softmax_scale, const float* gate, float* out, void* workspace, size_t workspace_bytes,
+                      const yahkv_decode_options* opt, void* stream);
+/* The second dispatch of yahkv_decode_step on its own, for callers that issue the two themselves (a timer or other
+ * work between them). The first is yahkv_decode_part with the lengths BEFORE the step (every seq_len one less; a
+ * device array of its own, since lengths are read on the device) and otherwise the same arguments; this call takes
+ * the lengths after the step, as yahkv_decode_step does. */
+int yahkv_decode_step_reduce(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
+                             int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs, int32_t max_seq_len,
+                             const void* k_new, const void* v_new, int32_t new_dtype, const void* q, int32_t q_dtype,
+                             float softmax_scale, const float* gate, float* out, void* workspace,
+                             size_t workspace_bytes, const yahkv_decode_options* opt, void* stream);
 /* Measures the relative read speeds of the GPU's eight XCDs on the caller's own batch and writes them to
  * opt->xcd_weight (the other fields are read): `rounds` times, the split-K kernel runs nine times on the given arguments and
  * the shares are corrected by when each XCD's workgroups finished. A set-up call: it synchronizes the stream and

@@ -14,10 +14,10 @@ from test_gpu_decode import setup
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("one_launch", [False, True], ids=["part_reduce", "one_launch"])
-def test_decode_step_replays_from_a_graph(yahkv, torch_gpu, one_launch):
+@pytest.mark.parametrize("form", ["part_reduce", "one_launch", "step"])
+def test_decode_step_replays_from_a_graph(yahkv, torch_gpu, form):
     torch = torch_gpu
-    opt = yahkv.decode_options(one_launch=one_launch, n_chunks=24, min_chunk_tiles=2)   # pairs that span several chunks
+    opt = yahkv.decode_options(one_launch=form == "one_launch", n_chunks=24, min_chunk_tiles=2)   # pairs that span several chunks
     lens = [700, 64, 1, 333]
     g, table, host, dev, rng = setup(yahkv, torch, 8, 24, 4, 256, 64, [n + 1 for n in lens], seed=21)
     t_table = torch.from_numpy(table).cuda()
@@ -30,6 +30,9 @@ def test_decode_step_replays_from_a_graph(yahkv, torch_gpu, one_launch):
     ws = torch.empty(yahkv.decode_workspace_bytes(dev.geom, 4, 701, opt), dtype=torch.uint8, device="cuda")
 
     def step():
+        if form == "step":                            # append and attention in the step call's two dispatches
+            yahkv.decode_step(dev, t_table, seq_len, 701, k[:, 0], v[:, 0], q, 0.0625, out=out, workspace=ws, opt=opt)
+            return
         yahkv.append(dev, t_table, pos, k, v)
         yahkv.decode_attend(dev, t_table, seq_len, 701, q, 0.0625, out=out, workspace=ws, opt=opt)
 

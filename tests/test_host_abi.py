@@ -151,6 +151,8 @@ def test_undersized_pools_are_refused_before_any_launch(yahkv):
         assert lib.yahkv_decode_part(r, pr, fake, 4, fake, 1, 100, fake, 2, 0.1, fake, ws, None, None) == -1
         assert lib.yahkv_decode_attend(r, pr, fake, 4, fake, 1, 100, fake, 2, 0.1, None, fake, fake, ws, None, None) == -1
         assert lib.yahkv_decode_attend_static(r, pr, fake, 4, fake, 1, 100, fake, 2, 0.1, None, fake, None) == -1
+        assert lib.yahkv_decode_step(r, pr, fake, 4, fake, 1, 100, fake, fake, 2, fake, 2, 0.1, None, fake, fake, ws, None,
+                                     None) == -1
         assert lib.yahkv_prefill_attend(r, pr, fake, 4, fake, 1, 64, 64, fake, 0.1, None, fake, 0, fake, ws, None) == -1
         assert lib.yahkv_prefill_decode_tiles(r, pr, fake, 4, fake, 1, 64, 64, fake, ws, None) == -1
         assert lib.yahkv_gather_blocks(r, pr, fake, 10, fake, fake, None) == -1

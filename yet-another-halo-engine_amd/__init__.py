@@ -70,6 +70,9 @@ def _load():
     lib.yahkv_decode_reduce.argtypes = [G, i32, i32p, i32, i32, vp, vp, vp, C.c_size_t, O, vp]
     lib.yahkv_decode_attend.argtypes = [G, P, i32p, i32, i32p, i32, i32, vp, i32, C.c_float, vp, vp, vp, C.c_size_t, O,
                                         vp]
+    lib.yahkv_decode_step.argtypes = [G, P, i32p, i32, i32p, i32, i32, vp, vp, i32, vp, i32, C.c_float, vp, vp, vp,
+                                      C.c_size_t, O, vp]
+    lib.yahkv_decode_step_reduce.argtypes = lib.yahkv_decode_step.argtypes
     lib.yahkv_decode_calibrate.argtypes = [G, P, i32p, i32, i32p, i32, i32, vp, i32, vp, C.c_size_t, O, i32, vp]
     lib.yahkv_decode_static_scratch_bytes.restype = C.c_size_t
     lib.yahkv_decode_attend_static.argtypes = [G, P, i32p, i32, i32p, i32, i32, vp, i32, C.c_float, vp, vp, vp]
@@ -378,6 +381,38 @@ def decode_attend(pools, table, seq_len, max_seq_len, q, scale, gate=None, out=N
     _check(lib.yahkv_decode_attend(C.byref(g), C.byref(st), _dp(table), table.shape[1], _dp(seq_len), n_seqs,
                                    max_seq_len, _dp(q), _dtype_code(q), scale, _dp(gate), _dp(out), _dp(workspace),
                                    workspace.numel(), _op(opt), _stream()), "decode_attend")
+    return out
+
+
+def decode_step(pools, table, seq_len, max_seq_len, k_new, v_new, q, scale, gate=None, out=None, workspace=None,
+                opt=None):
+    """Append + attention of one decode step in two dispatches. seq_len counts the step's own token, whose K / V rows
+    are k_new, v_new [n_seqs][n_kv_heads][D] (f32 / f16 / bf16); q as for decode_attend. Returns out f32."""
+    import torch
+    g = pools.geom
+    n_seqs = q.shape[0]
+    assert q.is_contiguous() and table.is_contiguous() and tuple(q.shape) == (n_seqs, g.n_q_heads, g.head_dim)
+    assert k_new.is_contiguous() and v_new.is_contiguous() and k_new.dtype == v_new.dtype
+    assert tuple(k_new.shape) == tuple(v_new.shape) == (n_seqs, g.n_kv_heads, g.head_dim)
+    if out is None:
+        out = torch.empty(q.shape, dtype=torch.float32, device=q.device)
+    if workspace is None:
+        workspace = torch.empty(decode_workspace_bytes(g, n_seqs, max_seq_len, opt), dtype=torch.uint8, device=q.device)
+    st = pools.struct()
+    _check(lib.yahkv_decode_step(C.byref(g), C.byref(st), _dp(table), table.shape[1], _dp(seq_len), n_seqs, max_seq_len,
+                                 _dp(k_new), _dp(v_new), _dtype_code(k_new), _dp(q), _dtype_code(q), scale, _dp(gate),
+                                 _dp(out), _dp(workspace), workspace.numel(), _op(opt), _stream()), "decode_step")
+    return out
+
+
+def decode_step_reduce(pools, table, seq_len, max_seq_len, k_new, v_new, q, scale, out, workspace, gate=None, opt=None):
+    """Second dispatch of decode_step (the first: decode_part on the lengths before the step)."""
+    g = pools.geom
+    st = pools.struct()
+    _check(lib.yahkv_decode_step_reduce(C.byref(g), C.byref(st), _dp(table), table.shape[1], _dp(seq_len), q.shape[0],
+                                        max_seq_len, _dp(k_new), _dp(v_new), _dtype_code(k_new), _dp(q), _dtype_code(q),
+                                        scale, _dp(gate), _dp(out), _dp(workspace), workspace.numel(), _op(opt),
+                                        _stream()), "decode_step_reduce")
     return out
 
 

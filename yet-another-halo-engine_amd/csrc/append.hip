@@ -41,15 +41,6 @@ struct RopeArgs {
   float* k_out;       // [n_seqs][n_new][H][D] f32 or null: the rotated K rows, for callers that want them
 };
 
-// Four consecutive elements of a source / destination row (element index a multiple of 4).
-__device__ __forceinline__ float4 Load4(const void* src, size_t i, int dtype) {
-  if (dtype == YAHKV_F32) return *reinterpret_cast<const float4*>(static_cast<const float*>(src) + i);
-  const uint2 w = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(src) + i);
-  const uint16_t h[4] = {static_cast<uint16_t>(w.x & 0xFFFF), static_cast<uint16_t>(w.x >> 16),
-                         static_cast<uint16_t>(w.y & 0xFFFF), static_cast<uint16_t>(w.y >> 16)};
-  if (dtype == YAHKV_F16) return float4{WidenF16(h[0]), WidenF16(h[1]), WidenF16(h[2]), WidenF16(h[3])};
-  return float4{WidenBf16(h[0]), WidenBf16(h[1]), WidenBf16(h[2]), WidenBf16(h[3])};
-}
 // The same in two steps, for loads that stay in flight while other work is done: the raw bytes, widened later.
 __device__ __forceinline__ uint4 LoadRaw4(const void* src, size_t i, int dtype) {
   if (dtype == YAHKV_F32) return *reinterpret_cast<const uint4*>(static_cast<const float*>(src) + i);
@@ -95,7 +86,7 @@ template <int FMT, bool ROPE>
 __global__ __launch_bounds__(64 * kRopeWaves) void AppendRows(const RopeArgs a) {
 #pragma clang fp contract(off)
   const Geom g = a.g;
-  const int NB = g.nb(), H = g.n_kv, PT = g.pt, D = g.hd, NQ = a.q_src != nullptr ? g.n_q : 0;
+  const int H = g.n_kv, PT = g.pt, D = g.hd, NQ = a.q_src != nullptr ? g.n_q : 0;
   const int rows_per_token = 2 * H + NQ;
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   const int i = int(blockIdx.x % a.n_new), s = int(blockIdx.x / a.n_new);
@@ -184,29 +175,14 @@ __global__ __launch_bounds__(64 * kRopeWaves) void AppendRows(const RopeArgs a) 
       }
       if (!is_v && a.k_out != nullptr && has) *reinterpret_cast<float4*>(a.k_out + off + d0) = v;
       // quantize: block b = lanes 8 b .. 8 b + 7
-      const int h = is_v ? row - H : row, b = lane / 8, lb = lane % 8;
+      const int h = is_v ? row - H : row, lb = lane % 8;
       uint16_t scale;
       const uint32_t codes = FMT == 8 ? QuantizeLanesQ8(v, &scale) : QuantizeLanesQ4(v, lb, &scale);
       if (!has) continue;
-      const size_t ph = size_t(page) * H + h;
-      if (!is_v) {
-        if (lb == 0) a.pools.ks[(ph * PT + t) * NB + b] = scale;
-        if (FMT == 8)
-          *reinterpret_cast<uint32_t*>(a.pools.kq + ((ph * NB + b) * PT + t) * 32 + 4 * lb) = codes;
-        else if (lb < 4)
-          *reinterpret_cast<uint32_t*>(a.pools.kq + ((ph * NB + b) * PT + t) * 16 + 4 * lb) = codes;
-      } else {
-        if (lb == 0) a.pools.vs[(ph * NB + b) * PT + t] = scale;
-        if (FMT == 8) {  // row (32 b + 4 lb + e) of [D][PT]
-          uint8_t* dst = a.pools.vq + (ph * D + d0) * PT + t;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) dst[size_t(e) * PT] = static_cast<uint8_t>(codes >> (8 * e));
-        } else if (lb < 4) {  // row (16 b + 4 lb + e) of [NB * 16][PT]
-          uint8_t* dst = a.pools.vq + ((ph * NB + b) * 16 + 4 * lb) * PT + t;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) dst[size_t(e) * PT] = static_cast<uint8_t>(codes >> (8 * e));
-        }
-      }
+      if (!is_v)
+        StoreRowK<FMT>(a.pools, g, page, h, t, lane, codes, scale);
+      else
+        StoreRowV<FMT>(a.pools, g, page, h, t, lane, codes, scale);
     }
   }
 }

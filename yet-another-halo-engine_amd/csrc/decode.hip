@@ -24,6 +24,7 @@
 #include <vector>
 
 #include "common.hpp"
+#include "quant.hpp"
 
 namespace yahkv {
 namespace {
@@ -61,9 +62,21 @@ struct DecodeArgs {
   int32_t fused;
   uint32_t epoch;               // never 0, different in every launch (graph replays aside: see Arrive)
   unsigned long long* tickets;  // [n_seqs * H] arrivals per pair: (epoch << 32) | workgroups that have arrived
+  // The step form (append + attention in two launches): seq_len counts the step's own token, which is not in the
+  // pools yet. The part kernel then covers the len_bias = -1 shorter sequences already there, and the reduce
+  // quantizes the token's rows, writes them to the pools and adds the token's term to the sums (StepRows).
+  int32_t len_bias;
+};
+// The step's own token for the reduce kernel: K / V rows [n_seqs][H][D] of `dtype`, or null pointers.
+struct StepRows {
+  const void* k;
+  const void* v;
+  int32_t dtype;
 };
 
-__device__ __forceinline__ int ClampLen(const DecodeArgs& a, int s) { return min(max(a.seq_len[s], 0), a.max_len); }
+__device__ __forceinline__ int ClampLen(const DecodeArgs& a, int s) {
+  return min(max(a.seq_len[s] + a.len_bias, 0), a.max_len);
+}
 
 // The line of tiles is cut into groups of eight chunks, 8 A tiles a group; chunk j of a group takes the tiles
 // [share[j], share[j + 1]) / 8192 of it. Workgroup k runs on XCD k % 8 and the XCDs do not read memory equally
@@ -398,7 +411,9 @@ __device__ __forceinline__ int Arrive(unsigned long long* ticket, uint32_t epoch
 // is copied to registers right before its product, so its request goes out before that product (fetch_v / take_v);
 // for q4_0, V loads into registers after the product. Page numbers come through scalar loads (they are the same
 // for the whole wave).
-template <int FMT, int D, int PT>
+// FUSED: the one-launch form, whose merge follows the split-K work in the same kernel. It is a template argument and
+// not a field of the arguments because the merge's registers would otherwise be the plain kernel's too (spills).
+template <int FMT, int D, int PT, bool FUSED>
 __global__ __launch_bounds__(64 * kWavesPerGroup) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void DattnPart(const DecodeArgs a) {
   constexpr int NB = D / 32, NT = D / 16, PPT = kTile / PT;
@@ -446,7 +461,7 @@ void DattnPart(const DecodeArgs a) {
   const int4 rec = ChunkRecord<64 * kWavesPerGroup>(a, blockIdx.x, wave_sum, &chunk_rec, chunk_tiles, &any_empty);
   // One launch for part and merge: sequences without keys have no pair on the line and nobody merges them, so the
   // first workgroup writes their rows of zeros (its threads have just looked at a slice of the lengths each).
-  if (a.fused && blockIdx.x == 0 && any_empty) {
+  if (FUSED && blockIdx.x == 0 && any_empty) {
     constexpr int NTH = 64 * kWavesPerGroup;
     const int per = (a.n_seqs + NTH - 1) / NTH;
     const int s0 = min(static_cast<int>(threadIdx.x) * per, a.n_seqs), s1 = min(s0 + per, a.n_seqs);
@@ -795,7 +810,7 @@ void DattnPart(const DecodeArgs a) {
     pv(1);
     // One launch for part and merge: what a wave has of the chunk's last pair stays in its registers, and the waves'
     // shares of that pair meet in LDS below instead of travelling through memory one by one.
-    if (a.fused && cur.base + cur.n >= chunk_n) {
+    if (FUSED && cur.base + cur.n >= chunk_n) {
       held = true;
       break;
     }
@@ -805,12 +820,12 @@ void DattnPart(const DecodeArgs a) {
   // pairs of the chunk after this wave's last tile (of the last pair, a wave that holds nothing says so in LDS below)
   if (!held) {
     do {
-      if (!worked && !(a.fused && cur.base + cur.n >= chunk_n)) leave_empty();
+      if (!worked && !(FUSED && cur.base + cur.n >= chunk_n)) leave_empty();
       worked = false;
     } while (NextPair(a, chunk_n, &cur));
   }
   if (a.stamps != nullptr && lane == 0) atomicMax(&a.stamps[a.n_chunks + blockIdx.x], wall_clock64());
-  if (!a.fused) return;
+  if (!FUSED) return;
 
   // ---- the merge, in the same launch (gen_decode_attn.py:338-411 is the reference's separate dispatch). A pair's
   // partials come from the workgroups of every chunk its tiles lie in; each of them, when all its waves are done,
@@ -1027,10 +1042,61 @@ void DattnPart(const DecodeArgs a) {
 // only a few workgroups here, which is why the partials are spread over the workgroup as well, and why a small batch
 // is launched with several workgroups per pair (gridDim.z), each with its own stretch of the head's dims: what bounds
 // such a launch is the number of partial rows in flight.
+//
+// The step form (rows given): the sequence's newest token is not in the pools yet. The first wave quantizes its K
+// row of this kv head exactly as the append kernel does (quant.hpp), takes the score of the dequantized row against
+// this workgroup's query head, and the second wave does the same for the V row and leaves the dequantized values in
+// LDS; the token then enters the sums like one more partial (maximum = its score, sum = 1, accumulator = its V row).
+// The workgroup of the group's first query head (and first stretch of dims) also writes the codes and scales to the
+// token's slot, so after the launch the pools hold what yahkv_append would have written.
+__device__ __forceinline__ void StepToken(const DecodeArgs& a, const StepRows& rows, int s, int h, int hq, int wave, int lane, bool writes,
+                                          float* score, float* vrow) {
+  const Geom& g = a.g;
+  const int D = g.hd, d0 = 4 * lane;
+  const bool has = d0 < D, is_v = wave == 1;
+  float4 x = {0.0f, 0.0f, 0.0f, 0.0f};
+  if (has) x = Load4(is_v ? rows.v : rows.k, (size_t(s) * g.n_kv + h) * D + d0, rows.dtype);
+  uint16_t scale;
+  uint32_t own, codes;
+  if (g.format == 8) {
+    codes = QuantizeLanesQ8(x, &scale), own = codes;
+  } else {
+    codes = QuantizeLanesQ4(x, lane % 8, &scale, &own);
+  }
+  const float d = WidenF16(scale);
+  float v[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int byte = static_cast<int>((own >> (8 * j)) & 0xFFu);
+    v[j] = static_cast<float>(g.format == 8 ? static_cast<int>(static_cast<int8_t>(byte)) : byte - 8) * d;
+  }
+  if (writes && has) {  // the token's place: as in the append kernels, position clamped to the table
+    const int pos = min(max(a.seq_len[s] - 1, 0), a.stride * g.pt - 1);
+    const int page = ClampPage(a.table[int64_t(s) * a.stride + pos / g.pt], g.n_pages), slot = pos % g.pt;
+    if (g.format == 8) {
+      if (is_v) StoreRowV<8>(a.pools, g, page, h, slot, lane, codes, scale);
+      else StoreRowK<8>(a.pools, g, page, h, slot, lane, codes, scale);
+    } else {
+      if (is_v) StoreRowV<4>(a.pools, g, page, h, slot, lane, codes, scale);
+      else StoreRowK<4>(a.pools, g, page, h, slot, lane, codes, scale);
+    }
+  }
+  if (is_v) {
+    if (has) *reinterpret_cast<float4*>(&vrow[d0]) = float4{v[0], v[1], v[2], v[3]};
+    return;
+  }
+  float4 qv = {0.0f, 0.0f, 0.0f, 0.0f};  // the query as the part kernel sees it: f16, saturated
+  if (has) qv = Load4(a.q, (size_t(s) * g.n_q + hq) * D + d0, a.q_dtype);
+  float dot = static_cast<float>(SaturateToF16(qv.x)) * v[0] + static_cast<float>(SaturateToF16(qv.y)) * v[1] +
+              static_cast<float>(SaturateToF16(qv.z)) * v[2] + static_cast<float>(SaturateToF16(qv.w)) * v[3];
+  dot = WaveSum(dot);
+  if (lane == 0) *score = dot * a.scale;
+}
+
 constexpr int kReduceThreads = 256;  // also the number of partial slots weighed at a time
 constexpr int kReduceDepth = 4;      // partials a group loads together
 constexpr int kReduceMinDims = 32;   // fewest dims of a head one workgroup sums
-__global__ __launch_bounds__(kReduceThreads) void DattnReduce(const DecodeArgs a) {
+__global__ __launch_bounds__(kReduceThreads) void DattnReduce(const DecodeArgs a, const StepRows rows) {
   const Geom g = a.g;
   const int G = g.group(), H = g.n_kv, D = g.hd;
   const int hq = blockIdx.x, s = blockIdx.y, t = threadIdx.x;
@@ -1038,16 +1104,24 @@ __global__ __launch_bounds__(kReduceThreads) void DattnReduce(const DecodeArgs a
   const int DZ = D / gridDim.z, d0 = blockIdx.z * DZ;  // this workgroup's dims are [d0, d0 + DZ)
   const size_t o = (size_t(s) * g.n_q + hq) * D + d0;
   const int ts = TilesOf(a, s);
-  if (ts <= 0) {  // length 0
+  const bool has_new = rows.k != nullptr && a.seq_len[s] >= 1;  // the step form, and the sequence has a new token
+  if (ts <= 0 && !has_new) {  // length 0
     if (t < DZ) a.out[o + t] = 0.0f;
     return;
   }
+  __shared__ float new_score;
+  __shared__ __align__(16) float new_v[256];
+  if (has_new && t < 128) StepToken(a, rows, s, h, hq, t / 64, t % 64, gi == 0 && blockIdx.z == 0, &new_score, new_v);
   // line units of the sequences before this one and of the whole line; the pair's tiles follow its first units
-  const long long A_ = ChunkUnits(a, static_cast<long long>(a.tprefix[a.n_seqs]) * H);
-  const int pair = s * H + h;
-  const long long first = static_cast<long long>(a.tprefix[s]) * H + static_cast<long long>(h) * UnitsOf(a, ts) + a.pair_cost;
-  const int k0 = ChunkOf(a, A_, first), k1 = ChunkOf(a, A_, first + ts - 1);
-  const size_t p0 = size_t(k0 + pair) * a.wpc, p1 = size_t(k1 + pair + 1) * a.wpc;
+  size_t p0 = 0, p1 = 0;  // (a sequence that has nothing but its new token has no partials)
+  if (ts > 0) {
+    const long long A_ = ChunkUnits(a, static_cast<long long>(a.tprefix[a.n_seqs]) * H);
+    const int pair = s * H + h;
+    const long long first =
+        static_cast<long long>(a.tprefix[s]) * H + static_cast<long long>(h) * UnitsOf(a, ts) + a.pair_cost;
+    const int k0 = ChunkOf(a, A_, first), k1 = ChunkOf(a, A_, first + ts - 1);
+    p0 = size_t(k0 + pair) * a.wpc, p1 = size_t(k1 + pair + 1) * a.wpc;
+  }
   constexpr int NW = kReduceThreads / 64;
   __shared__ float wgt[kReduceThreads], wl[kReduceThreads];
   __shared__ int slot[kReduceThreads];
@@ -1064,6 +1138,7 @@ __global__ __launch_bounds__(kReduceThreads) void DattnReduce(const DecodeArgs a
   __syncthreads();
   M = red[0];
   for (int w = 1; w < NW; ++w) M = fmaxf(M, red[w]);
+  if (has_new) M = fmaxf(M, new_score);
   const int lanes = DZ / 4, n_groups = kReduceThreads / lanes, grp = t / lanes, dl = t % lanes;
   float L = 0.0f;
   float4 A = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -1107,6 +1182,10 @@ __global__ __launch_bounds__(kReduceThreads) void DattnReduce(const DecodeArgs a
   if (t < DZ) {
     float v = 0.0f, lt = 0.0f;
     for (int q = 0; q < n_groups; ++q) v += sums[q * DZ + t], lt += lsums[q];
+    if (has_new) {
+      const float w = __expf(new_score - M);
+      v = __builtin_fmaf(w, new_v[d0 + t], v), lt += w;
+    }
     v /= lt;
     if (a.gate != nullptr) v *= 1.0f / (1.0f + __expf(-a.gate[o + t]));
     a.out[o + t] = v;
@@ -1227,8 +1306,11 @@ int Prepare(const yahkv_geometry* g, int32_t page_table_stride, const int32_t* s
 int LaunchPart(const DecodeArgs& a, hipStream_t st) {
   const Geom& m = a.g;
   const dim3 grid(static_cast<unsigned>(a.n_chunks));
-#define YAHKV_LAUNCH_PART(FF, DD, PP) \
-  hipLaunchKernelGGL((DattnPart<FF, DD, PP>), grid, dim3(64 * kWavesPerGroup), 0, st, a)
+#define YAHKV_LAUNCH_PART(FF, DD, PP)                                                                          \
+  do {                                                                                                         \
+    if (a.fused) hipLaunchKernelGGL((DattnPart<FF, DD, PP, true>), grid, dim3(64 * kWavesPerGroup), 0, st, a); \
+    else hipLaunchKernelGGL((DattnPart<FF, DD, PP, false>), grid, dim3(64 * kWavesPerGroup), 0, st, a);        \
+  } while (0)
 #define YAHKV_LAUNCH_FMT(FF)                                       \
   if (m.hd == 256 && m.pt == 64) YAHKV_LAUNCH_PART(FF, 256, 64);      \
   else if (m.hd == 256 && m.pt == 32) YAHKV_LAUNCH_PART(FF, 256, 32); \
@@ -1243,6 +1325,17 @@ int LaunchPart(const DecodeArgs& a, hipStream_t st) {
   }
 #undef YAHKV_LAUNCH_FMT
 #undef YAHKV_LAUNCH_PART
+  return LaunchStatus();
+}
+
+int LaunchReduce(const DecodeArgs& a, const StepRows& rows, const yahkv_decode_options* opt, hipStream_t st) {
+  // a small batch: more workgroups per (query head, sequence), each with a part of the dims, until the CUs have one
+  int split = 1;
+  while (int64_t(a.g.n_q) * a.n_seqs * split < ComputeUnits() && a.g.hd / (2 * split) >= kReduceMinDims) split *= 2;
+  const int asked = MakeTuning(opt).reduce_split;
+  if (asked > 0) split = std::min(asked, a.g.hd / kReduceMinDims);
+  while (a.g.hd % split != 0 || (a.g.hd / split) % 4 != 0) --split;
+  hipLaunchKernelGGL(DattnReduce, dim3(a.g.n_q, a.n_seqs, split), dim3(kReduceThreads), 0, st, a, rows);
   return LaunchStatus();
 }
 
@@ -1287,15 +1380,54 @@ extern "C" int yahkv_decode_reduce(const yahkv_geometry* g, int32_t page_table_s
     return st;
   if (out == nullptr) return YAHKV_ERR_ARG;
   a.gate = gate, a.out = out;
-  // a small batch: more workgroups per (query head, sequence), each with a part of the dims, until the CUs have one
-  int split = 1;
-  while (int64_t(a.g.n_q) * n_seqs * split < ComputeUnits() && a.g.hd / (2 * split) >= kReduceMinDims) split *= 2;
-  const int asked = MakeTuning(opt).reduce_split;
-  if (asked > 0) split = std::min(asked, a.g.hd / kReduceMinDims);
-  while (a.g.hd % split != 0 || (a.g.hd / split) % 4 != 0) --split;
-  hipLaunchKernelGGL(DattnReduce, dim3(a.g.n_q, n_seqs, split), dim3(kReduceThreads), 0,
-                     static_cast<hipStream_t>(stream), a);
-  return LaunchStatus();
+  return LaunchReduce(a, StepRows{nullptr, nullptr, 0}, opt, static_cast<hipStream_t>(stream));
+}
+
+// Append and attention of one decode step in two launches instead of three: the part kernel runs over the tokens the
+// pools already hold (lengths one shorter than given), and the reduce quantizes the step's own token, writes it to its
+// slot and adds its term to the sums (see StepToken). seq_len[s] counts the new token, which lies at position
+// seq_len[s] - 1; a sequence with seq_len[s] <= 0 is left alone (nothing appended, its output rows zero).
+extern "C" int yahkv_decode_step_reduce(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
+                                        int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs,
+                                        int32_t max_seq_len, const void* k_new, const void* v_new, int32_t new_dtype,
+                                        const void* q, int32_t q_dtype, float softmax_scale, const float* gate,
+                                        float* out, void* workspace, size_t workspace_bytes,
+                                        const yahkv_decode_options* opt, void* stream) {
+  if (out == nullptr || (reinterpret_cast<uintptr_t>(out) & 15)) return YAHKV_ERR_ARG;
+  if (k_new == nullptr || v_new == nullptr) return YAHKV_ERR_ARG;
+  if ((reinterpret_cast<uintptr_t>(k_new) | reinterpret_cast<uintptr_t>(v_new)) & 15) return YAHKV_ERR_ARG;
+  if (new_dtype != YAHKV_F32 && new_dtype != YAHKV_F16 && new_dtype != YAHKV_BF16) return YAHKV_ERR_ARG;
+  if (MakeTuning(opt).one_launch) return YAHKV_ERR_ARG;  // the token enters in the merge's own launch
+  DecodeArgs a;
+  if (const int st = Prepare(g, page_table_stride, seq_len, n_seqs, max_seq_len, workspace, workspace_bytes, opt, &a))
+    return st;
+  if (const int st = CheckPartArgs(g, pools, page_table, q, q_dtype)) return st;
+  a.pools = MakePools(*pools), a.table = page_table, a.q = q, a.q_dtype = q_dtype, a.scale = softmax_scale;
+  a.len_bias = -1, a.gate = gate, a.out = out;
+  return LaunchReduce(a, StepRows{k_new, v_new, new_dtype}, opt, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int yahkv_decode_step(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
+                                 int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs,
+                                 int32_t max_seq_len, const void* k_new, const void* v_new, int32_t new_dtype,
+                                 const void* q, int32_t q_dtype, float softmax_scale, const float* gate, float* out,
+                                 void* workspace, size_t workspace_bytes, const yahkv_decode_options* opt,
+                                 void* stream) {
+  if (out == nullptr || k_new == nullptr || v_new == nullptr) return YAHKV_ERR_ARG;  // before anything is launched
+  if ((reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(k_new) | reinterpret_cast<uintptr_t>(v_new)) & 15)
+    return YAHKV_ERR_ARG;
+  if (new_dtype != YAHKV_F32 && new_dtype != YAHKV_F16 && new_dtype != YAHKV_BF16) return YAHKV_ERR_ARG;
+  if (MakeTuning(opt).one_launch) return YAHKV_ERR_ARG;
+  DecodeArgs a;
+  if (const int st = Prepare(g, page_table_stride, seq_len, n_seqs, max_seq_len, workspace, workspace_bytes, opt, &a))
+    return st;
+  if (const int st = CheckPartArgs(g, pools, page_table, q, q_dtype)) return st;
+  a.pools = MakePools(*pools), a.table = page_table, a.q = q, a.q_dtype = q_dtype, a.scale = softmax_scale;
+  a.len_bias = -1;
+  if (const int st = LaunchPart(a, static_cast<hipStream_t>(stream))) return st;
+  return yahkv_decode_step_reduce(g, pools, page_table, page_table_stride, seq_len, n_seqs, max_seq_len, k_new, v_new,
+                                  new_dtype, q, q_dtype, softmax_scale, gate, out, workspace, workspace_bytes, opt,
+                                  stream);
 }
 
 namespace {

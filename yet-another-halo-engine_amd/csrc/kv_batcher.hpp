@@ -319,7 +319,7 @@ class KvBatcher {
     if (np + nd == 0) return;
     const int32_t* d = static_cast<const int32_t*>(stage_dev_.get());
     const int32_t* d_prefix = d + rows_ * size_t(stride_);
-    const int32_t *d_valid = d_prefix + rows_, *d_pos = d_valid + rows_, *d_len = d_pos + rows_;
+    const int32_t *d_valid = d_prefix + rows_, *d_len = d_valid + 2 * size_t(rows_);  // (between them: the decode rows' positions)
     const yahkv_pools pools = this->pools(layer);
     const int32_t chunk = sched_.chunk(), T = sched_.context();
     if (np > 0) {
@@ -336,9 +336,9 @@ class KvBatcher {
     if (nd > 0) {
       if (dk == nullptr || dv == nullptr || dq == nullptr || dout == nullptr) throw KvError("batcher: decode rows missing");
       const int32_t* dt = d + size_t(np) * stride_;
-      Check(yahkv_append(&g_, &pools, dt, stride_, d_pos, nullptr, nd, 1, dk, dv, kv_dtype, stream_), "append");
-      Check(yahkv_decode_attend(&g_, &pools, dt, stride_, d_len, nd, T, dq, dq_dtype, softmax_scale, nullptr, dout,
-                                workspace_.get(), workspace_.size(), nullptr, stream_), "decode_attend");
+      // append + attention of the decode rows in two dispatches (the merge stores the new tokens)
+      Check(yahkv_decode_step(&g_, &pools, dt, stride_, d_len, nd, T, dk, dv, kv_dtype, dq, dq_dtype, softmax_scale,
+                              nullptr, dout, workspace_.get(), workspace_.size(), nullptr, stream_), "decode_step");
     }
   }
   void Commit() { sched_.Commit(); }

@@ -286,7 +286,9 @@ class KvDecoder {
 
   // Queues one decode step for sequences 0 .. n_seqs - 1: K / V rows [n_seqs][1][H][D] of kv_dtype are appended at each
   // sequence's current length, then q [n_seqs][n_q][D] attends over the lengthened sequences into out f32.
-  // Order as LoomDecoder::Step: append, then part, then reduce (loom_decoder.hpp:253-268).
+  // What LoomDecoder::Step does in four dispatches (kappend, vappend, part, reduce: loom_decoder.hpp:253-268) takes two
+  // here: the split-K pass over the tokens already in the pools, and the merge, which quantizes and stores the new
+  // token and adds its term (yahkv_decode_step).
   void Step(int32_t n_seqs, const void* k, const void* v, int32_t kv_dtype, const void* q, int32_t q_dtype,
             float softmax_scale, const float* gate, float* out) {
     if (!bound_) throw KvError("decoder: no state bound");
@@ -310,9 +312,9 @@ class KvDecoder {
     const yahkv_pools pools = PoolsOf(st_);
     const int32_t* pos = static_cast<const int32_t*>(pos_dev_.get());
     const int32_t* ptab = static_cast<const int32_t*>(st_.ptab.ptr);
-    Check(yahkv_append(&g_, &pools, ptab, stride_, pos, nullptr, n_seqs, 1, k, v, kv_dtype, stream_), "append");
-    Check(yahkv_decode_attend(&g_, &pools, ptab, stride_, pos + max_seqs_, n_seqs, T_, q, q_dtype, softmax_scale,
-                              gate, out, workspace_.get(), workspace_.size(), nullptr, stream_), "decode_attend");
+    Check(yahkv_decode_step(&g_, &pools, ptab, stride_, pos + max_seqs_, n_seqs, T_, k, v, kv_dtype, q, q_dtype,
+                            softmax_scale, gate, out, workspace_.get(), workspace_.size(), nullptr, stream_),
+          "decode_step");
   }
 
   const yahkv_geometry& geometry() const { return g_; }

@@ -78,7 +78,9 @@ __device__ __forceinline__ uint32_t QuantizeLanesQ8(const float4 v, uint16_t* sc
 // q4_0: ggml takes the value of largest magnitude, the first one on ties, so the reduction carries (|x|, index,
 // x) and prefers the lower index; d = that value / -8. Lanes 0-3 of the 8 return 4 bytes: low nibbles their own
 // elements j, high nibbles the elements j + 16 held by the lane four further on.
-__device__ __forceinline__ uint32_t QuantizeLanesQ4(const float4 v, int lane_in_block, uint16_t* scale) {
+// `own`, if given, receives this lane's own four nibbles, one per byte.
+__device__ __forceinline__ uint32_t QuantizeLanesQ4(const float4 v, int lane_in_block, uint16_t* scale,
+                                                    uint32_t* own = nullptr) {
 #pragma clang fp contract(off)
   const float e[4] = {v.x, v.y, v.z, v.w};
   float av = fabsf(e[0]), mx = e[0];
@@ -101,9 +103,53 @@ __device__ __forceinline__ uint32_t QuantizeLanesQ4(const float4 v, int lane_in_
     const int q = min(15, static_cast<int>(static_cast<int8_t>(static_cast<int>(e[j] * id + 8.5f))));
     nib |= static_cast<uint32_t>(q) << (8 * j);
   }
+  if (own != nullptr) *own = nib;
   // the nibbles of the lane four further on (row_shr would move the wrong way: take them through a lane shuffle)
   const uint32_t hi = static_cast<uint32_t>(__shfl_down(static_cast<int>(nib), 4, 64));
   return nib | (hi << 4);
+}
+
+// Four consecutive elements of a source row of f32, f16 or bf16 values (element index a multiple of 4).
+__device__ __forceinline__ float4 Load4(const void* src, size_t i, int dtype) {
+  if (dtype == YAHKV_F32) return *reinterpret_cast<const float4*>(static_cast<const float*>(src) + i);
+  const uint2 w = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(src) + i);
+  const uint16_t h[4] = {static_cast<uint16_t>(w.x & 0xFFFF), static_cast<uint16_t>(w.x >> 16),
+                         static_cast<uint16_t>(w.y & 0xFFFF), static_cast<uint16_t>(w.y >> 16)};
+  if (dtype == YAHKV_F16) return float4{WidenF16(h[0]), WidenF16(h[1]), WidenF16(h[2]), WidenF16(h[3])};
+  return float4{WidenBf16(h[0]), WidenBf16(h[1]), WidenBf16(h[2]), WidenBf16(h[3])};
+}
+
+// Where a quantized row goes. A row of head_dim values lies across a wavefront, four consecutive dims per lane (lanes
+// at or past head_dim / 4 hold nothing and must not call these); block b is lanes 8 b .. 8 b + 7 and `codes` is what
+// the quantizers above return for the lane. K: codes [page][H][block][slot][32 | 16], scales [page][H][slot][block];
+// V: codes transposed, [page][H][dim][slot] (q8_0) or [page][H][block][16][slot] (q4_0, a byte per pair of dims),
+// scales [page][H][block][slot].
+template <int FMT>
+__device__ __forceinline__ void StoreRowK(const Pools& pools, const Geom& g, int page, int h, int slot, int lane,
+                                          uint32_t codes, uint16_t scale) {
+  const int NB = g.nb(), PT = g.pt, b = lane / 8, lb = lane % 8;
+  const size_t ph = size_t(page) * g.n_kv + h;
+  if (lb == 0) pools.ks[(ph * PT + slot) * NB + b] = scale;
+  if (FMT == 8)
+    *reinterpret_cast<uint32_t*>(pools.kq + ((ph * NB + b) * PT + slot) * 32 + 4 * lb) = codes;
+  else if (lb < 4)
+    *reinterpret_cast<uint32_t*>(pools.kq + ((ph * NB + b) * PT + slot) * 16 + 4 * lb) = codes;
+}
+template <int FMT>
+__device__ __forceinline__ void StoreRowV(const Pools& pools, const Geom& g, int page, int h, int slot, int lane,
+                                          uint32_t codes, uint16_t scale) {
+  const int NB = g.nb(), PT = g.pt, b = lane / 8, lb = lane % 8;
+  const size_t ph = size_t(page) * g.n_kv + h;
+  if (lb == 0) pools.vs[(ph * NB + b) * PT + slot] = scale;
+  if (FMT == 8) {  // row (32 b + 4 lb + e) of [D][PT]
+    uint8_t* dst = pools.vq + (ph * g.hd + 4 * lane) * PT + slot;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) dst[size_t(e) * PT] = static_cast<uint8_t>(codes >> (8 * e));
+  } else if (lb < 4) {  // row (16 b + 4 lb + e) of [NB * 16][PT]
+    uint8_t* dst = pools.vq + ((ph * NB + b) * 16 + 4 * lb) * PT + slot;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) dst[size_t(e) * PT] = static_cast<uint8_t>(codes >> (8 * e));
+  }
 }
 
 }  // namespace yahkv
