@@ -27,9 +27,10 @@ WORKLOADS = {
     # one sequence's KV (71 MB) would stay in the 256 MB last-level cache from step to step: the steps rotate over
     # eight layers' pools, as the layers of a model do
     "b1_ctx32k_q8_0": dict(fmt=8, batch=1, lo=32768, hi=32768, seed=4, layers=8),
-    # (after an idle GPU this kernel's launches run 0.41 ms, then up to 0.57 ms from about the seventh on, and settle
-    # at 0.43 ms after twenty: the default warm-up waits for that)
-    "b16_ctx128k_q4_0": dict(fmt=4, batch=16, lo=131072, hi=131072, seed=4, outliers=8, warmup=25),
+    # (this kernel runs as fast as the shader clock up to about 2.1 GHz, and after an idle GPU the clock falls from 2.4 to
+    # 1.3 GHz within 3 ms and is back at the 2.1 GHz it holds under this kernel some 30 ms later: the default warm-up
+    # waits for that, and the line's after_idle object holds the steps timed right after an idle period)
+    "b16_ctx128k_q4_0": dict(fmt=4, batch=16, lo=131072, hi=131072, seed=4, outliers=8, warmup=80),
     # chunked prefill: every sequence holds `lo` tokens and takes a chunk of `chunk` more per step (the first six
     # launches of the attention kernel after an idle GPU run up to 25 % longer than the later ones)
     "prefill_b8_ctx16k_chunk2k_q8_0": dict(fmt=8, batch=8, lo=16384, hi=16384, seed=4, chunk=2048, warmup=10),
@@ -92,6 +93,26 @@ def build_state(yahkv, torch, wl, total_steps):
                              k.to(torch.bfloat16), v.to(torch.bfloat16))
     torch.cuda.synchronize()
     return g, layers, lens, table, t_table, gen
+
+
+def clock_trace(yahkv, torch, launch, n=60, idle_s=3.0):
+    """After `idle_s` seconds without GPU work: n launches of `launch` (a callable that queues the workload's dominant
+    kernel), each followed by the library's clock probe. Returns per launch its duration (HIP events) and the shader
+    clock right after it. An extra figure for instruction-bound kernels, whose speed follows the clock."""
+    res = torch.zeros((n, 2), dtype=torch.int64, device="cuda")
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
+    torch.cuda.synchronize()
+    time.sleep(idle_s)
+    for i in range(n):
+        ev[i][0].record()
+        launch()
+        ev[i][1].record()
+        yahkv.shader_clock_probe(res[i], 2000)       # 20 us
+    torch.cuda.synchronize()
+    r = res.cpu().numpy().astype(np.float64)
+    return {"idle_s": idle_s, "kernel_ms": [round(a.elapsed_time(b), 4) for a, b in ev],
+            "shader_mhz": [int(round(x)) for x in r[:, 0] / np.maximum(r[:, 1], 1) * 100.0],
+            "note": "launches of the dominant kernel back to back after an idle GPU, the shader clock after each"}
 
 
 def parity_check(yahkv, torch, g, pools, t_table, lens, q, out, scale, rows):
@@ -398,6 +419,9 @@ def run_prefill(a, wl, torch, yahkv):
                      "traffic": TRAFFIC[a.workload][0], "traffic_source": TRAFFIC[a.workload][1],
                      "kernel": "PrefillAttendImg<%d, 2>" % HD, "kernel_ms": round(kern_ms, 4)},
     }
+    if a.clock_trace:
+        res["clock_trace"] = clock_trace(
+            yahkv, torch, lambda: yahkv.prefill_attend_tiles(pools, t_table, t_prefix, prefix, q, scale, out, ws), n=24)
     if not a.no_cpu_baseline:
         res["cpu_baseline"] = prefill_cpu_baseline(wl, scale)
     return res
@@ -492,7 +516,7 @@ def run_decode(a, wl, torch, yahkv):
     (yahkv_decode_step's): split-K partials over the tokens already in the pools, then the merge, which also quantizes
     the new token, writes it to its page and adds its term. --separate-append: three dispatches, the reference's order
     (append, partials, merge)."""
-    total = a.warmup + a.steps + 1
+    total = a.warmup + 2 * a.steps + 1                # (the second set of steps: the ones timed after an idle period)
     g, layers, lens, table, t_table, gen = build_state(yahkv, torch, wl, total)
     pools = layers[0]
     B = wl["batch"]
@@ -588,6 +612,21 @@ def run_decode(a, wl, torch, yahkv):
                      "traffic_source": TRAFFIC.get(a.workload, (None, None))[1],
                      "kernel": "DattnPart<%d, %d, %d>" % (wl["fmt"], HD, PT), "kernel_ms": round(kern_ms, 4)},
     }
+    # The same number of steps again, right after three idle seconds and without warm-up: what a server's first steps
+    # after a pause cost (the shader clock dips for some tens of milliseconds then; kernels bound by HBM hardly notice,
+    # the q4_0 kernel does). An extra figure, not `value`.
+    time.sleep(3.0)
+    t0 = time.perf_counter()
+    for i in range(a.steps):
+        step(1 + a.warmup + a.steps + i)
+    torch.cuda.synchronize()
+    cold_ms = (time.perf_counter() - t0) / a.steps * 1e3
+    res["after_idle"] = {"ms_per_step": round(cold_ms, 4), "GB/s": round(kv_bytes / (cold_ms * 1e-3) / 1e9, 1),
+                         "note": "%d steps right after 3 idle seconds, no warm-up" % a.steps}
+    if a.clock_trace:
+        last = a.warmup + a.steps + 1
+        res["clock_trace"] = clock_trace(
+            yahkv, torch, lambda: yahkv.decode_part(pools, t_table, len_rows[last], max_len, q, scale, ws, opt=opt))
     if a.graph_replay:
         # The same timed steps (same tokens at the same positions: the pools end up as they are) recorded once into
         # a HIP graph, so the launches follow each other without the host in between; an extra figure, not `value`.
@@ -648,6 +687,9 @@ def main():
                     help="decode workloads: yahkv_decode_attend with opt.one_launch instead of part + reduce")
     ap.add_argument("--separate-append", action="store_true",
                     help="decode workloads: the step's token is appended by a dispatch of its own (three per step)")
+    ap.add_argument("--clock-trace", action="store_true",
+                    help="also: after the timing and three idle seconds, launches of the dominant kernel back to back with "
+                         "the shader clock after each (quantized decode and prefill workloads)")
     ap.add_argument("--graph-replay", action="store_true",
                     help="decode workloads: also replay the timed steps as one HIP graph and report its time per step")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -677,10 +719,10 @@ def main():
             torch.cuda.empty_cache()
             sub = argparse.Namespace(**vars(a))
             sub.workload, sub.graph_replay, sub.no_cpu_baseline = name, "chunk" not in WORKLOADS[name], True
-            sub.warmup = WORKLOADS[name].get("warmup", 3)
+            sub.warmup, sub.clock_trace = WORKLOADS[name].get("warmup", 3), False
             r = run_workload(sub, torch, yahkv)
             keep = ("metric", "value", "unit", "ms_per_step", "steps", "warmup", "tok_per_s", "parity_max_rel_err", "roofline",
-                    "graph_replay", "append", "pct_of_hbm_peak", "out_fnv1a")
+                    "graph_replay", "after_idle", "append", "pct_of_hbm_peak", "out_fnv1a")
             res["also"][name] = {k: r[k] for k in keep if k in r}
     print(json.dumps(res))
 

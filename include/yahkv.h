@@ -219,6 +219,13 @@ int yahkv_decode_calibrate(const yahkv_geometry* g, const yahkv_pools* pools, co
                            const void* q, int32_t q_dtype, void* workspace, size_t workspace_bytes,
                            yahkv_decode_options* opt, int32_t rounds, void* stream);
 
+/* Diagnostics, no counterpart in the reference: a one-wave kernel on `stream` that counts shader-clock cycles over
+ * `ticks` (1 .. 100000) ticks of the GPU's constant 100 MHz counter and writes {cycles, ticks} as two uint64 to
+ * device memory; 100 * cycles / ticks is the shader clock in MHz at that point of the stream. The instruction-bound
+ * kernels (q4_0 decode, prefill) run as fast as that clock, which is unsteady for some tens of milliseconds after an
+ * idle period. */
+int yahkv_shader_clock_probe(void* cycles_and_ticks, int32_t ticks, void* stream);
+
 /* yahkv_decode_attend without a workspace argument, for callers that cannot allocate device memory (code under HIP
  * graph capture, serving loops and harnesses that forbid hipMalloc). It has no counterpart in the reference. The
  * partials go to an array that is part of the library's code object: yahkv_decode_static_scratch_bytes() = 32 MiB,

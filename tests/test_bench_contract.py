@@ -51,6 +51,8 @@ def test_decode_line_has_the_fields_a_driver_reads():
     for name, r in d["also"].items():
         assert r["value"] > 0 and r["ms_per_step"] > 0 and r["parity_max_rel_err"] < 2e-3, name
         assert 0.0 < r["roofline"]["frac"] < 1.0 and r["roofline"]["bound"] == ("mfma" if "prefill" in name else "hbm")
+    # the decode workloads also say what their steps cost right after an idle period (an extra figure)
+    assert d["after_idle"]["ms_per_step"] > 0 and d["also"]["b16_ctx128k_q4_0"]["after_idle"]["ms_per_step"] > 0
     assert "config1_tiny" in d["cpu_baseline"]["configs"] and "config2_b1_ctx32k" in d["cpu_baseline"]["configs"]
 
 

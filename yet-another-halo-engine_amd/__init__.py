@@ -74,6 +74,7 @@ def _load():
                                       C.c_size_t, O, vp]
     lib.yahkv_decode_step_reduce.argtypes = lib.yahkv_decode_step.argtypes
     lib.yahkv_decode_calibrate.argtypes = [G, P, i32p, i32, i32p, i32, i32, vp, i32, vp, C.c_size_t, O, i32, vp]
+    lib.yahkv_shader_clock_probe.argtypes = [vp, i32, vp]
     lib.yahkv_decode_static_scratch_bytes.restype = C.c_size_t
     lib.yahkv_decode_attend_static.argtypes = [G, P, i32p, i32, i32p, i32, i32, vp, i32, C.c_float, vp, vp, vp]
     lib.yahkv_prefill_workspace_bytes.restype = C.c_size_t
@@ -414,6 +415,11 @@ def decode_step_reduce(pools, table, seq_len, max_seq_len, k_new, v_new, q, scal
                                         scale, _dp(gate), _dp(out), _dp(workspace), workspace.numel(), _op(opt),
                                         _stream()), "decode_step_reduce")
     return out
+
+
+def shader_clock_probe(out, ticks=2000):
+    """Queues the clock probe; out: an int64 cuda tensor of two elements, {shader cycles, 100 MHz ticks} once it ran."""
+    _check(lib.yahkv_shader_clock_probe(_dp(out), ticks, _stream()), "shader_clock_probe")
 
 
 def decode_attend_static(pools, table, seq_len, max_seq_len, q, scale, out, gate=None):

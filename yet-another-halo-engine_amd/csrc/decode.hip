@@ -1517,6 +1517,32 @@ extern "C" int yahkv_decode_calibrate(const yahkv_geometry* g, const yahkv_pools
   return YAHKV_OK;
 }
 
+// ---- the shader clock, as a kernel sees it -----------------------------------------------------------------------------------
+//
+// One wave counts shader cycles over `ticks` ticks of the constant 100 MHz counter (both counters are the hardware's
+// own). What it is for: the instruction-bound kernels here (q4_0 decode, prefill) run as fast as the shader clock, and
+// after an idle period the clock is not steady for some tens of milliseconds; a caller that times them can record the
+// clock beside each launch (bench.py --clock-trace does).
+namespace yahkv {
+namespace {
+__global__ void ShaderClockProbe(unsigned long long* out, int ticks) {
+  if (threadIdx.x != 0) return;
+  const unsigned long long w0 = wall_clock64(), c0 = clock64();
+  unsigned long long w = w0;
+  while (w - w0 < static_cast<unsigned long long>(ticks)) w = wall_clock64();  // the counter always advances
+  out[0] = clock64() - c0, out[1] = w - w0;
+}
+}  // namespace
+}  // namespace yahkv
+
+extern "C" int yahkv_shader_clock_probe(void* cycles_and_ticks, int32_t ticks, void* stream) {
+  if (cycles_and_ticks == nullptr || (reinterpret_cast<uintptr_t>(cycles_and_ticks) & 7)) return YAHKV_ERR_ARG;
+  if (ticks <= 0 || ticks > 100000) return YAHKV_ERR_ARG;  // at most a millisecond
+  hipLaunchKernelGGL(ShaderClockProbe, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream),
+                     static_cast<unsigned long long*>(cycles_and_ticks), ticks);
+  return LaunchStatus();
+}
+
 // ---- decode attention without a workspace argument ------------------------------------------------------------------------
 //
 // For callers that cannot allocate device memory at all (code under HIP graph capture, serving loops or harnesses that
