@@ -110,9 +110,37 @@ def clock_trace(yahkv, torch, launch, n=60, idle_s=3.0):
         yahkv.shader_clock_probe(res[i], 2000)       # 20 us
     torch.cuda.synchronize()
     r = res.cpu().numpy().astype(np.float64)
-    return {"idle_s": idle_s, "kernel_ms": [round(a.elapsed_time(b), 4) for a, b in ev],
-            "shader_mhz": [int(round(x)) for x in r[:, 0] / np.maximum(r[:, 1], 1) * 100.0],
-            "note": "launches of the dominant kernel back to back after an idle GPU, the shader clock after each"}
+    trace = {"idle_s": idle_s, "kernel_ms": [round(a.elapsed_time(b), 4) for a, b in ev],
+             "shader_mhz": [int(round(x)) for x in r[:, 0] / np.maximum(r[:, 1], 1) * 100.0],
+             "note": "launches of the dominant kernel back to back after an idle GPU, the shader clock after each"}
+    # The clock WHILE the kernel runs: the same launches back to back (the GPU is warm now), and probes of 0.5 ms each on
+    # a second stream beside them. The probe's wave shares a CU with the kernel's workgroups, so the launches run a
+    # little slower than alone (much slower where one workgroup per CU holds a fixed share of the work).
+    per = float(np.median(trace["kernel_ms"][n // 2:]))
+    n_load = max(int(120.0 / per), 8)                  # about 120 ms of load
+    n_probe = int(n_load * per / 0.5) + 20
+    side = torch.cuda.Stream()
+    res = torch.zeros((n_probe, 2), dtype=torch.int64, device="cuda")
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(n_load):
+        launch()
+    e1.record()
+    side.wait_event(e0)
+    with torch.cuda.stream(side):
+        for i in range(n_probe):
+            yahkv.shader_clock_probe(res[i], 50000)
+    torch.cuda.synchronize()
+    total = e0.elapsed_time(e1)
+    r = res.cpu().numpy().astype(np.float64)
+    mhz = (r[:, 0] / np.maximum(r[:, 1], 1) * 100.0)[:max(min(int(total / 0.5) - 2, n_probe), 1)]
+    trace["under_load"] = {"shader_mhz_median": int(np.median(mhz[len(mhz) // 2:])),
+                           "shader_mhz_p10_p90": [int(np.percentile(mhz[len(mhz) // 2:], 10)),
+                                                  int(np.percentile(mhz[len(mhz) // 2:], 90))],
+                           "kernel_ms_beside_the_probe": round(total / n_load, 4), "launches": n_load,
+                           "note": "probes of 0.5 ms on a second stream while the launches run; second half of them"}
+    return trace
 
 
 def parity_check(yahkv, torch, g, pools, t_table, lens, q, out, scale, rows):
