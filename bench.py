@@ -638,7 +638,8 @@ def run_decode(a, wl, torch, yahkv):
         "roofline": {"bound": "hbm", "achieved": round(kgbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(kgbs / HBM_PEAK_GBS, 4), "traffic": TRAFFIC.get(a.workload, (None, None))[0],
                      "traffic_source": TRAFFIC.get(a.workload, (None, None))[1],
-                     "kernel": "DattnPart<%d, %d, %d>" % (wl["fmt"], HD, PT), "kernel_ms": round(kern_ms, 4)},
+                     "kernel": "DattnPart<%d, %d, %d, %s>" % (wl["fmt"], HD, PT, "true" if a.one_launch else "false"),
+                     "kernel_ms": round(kern_ms, 4)},
     }
     # The same number of steps again, right after three idle seconds and without warm-up: what a server's first steps
     # after a pause cost (the shader clock dips for some tens of milliseconds then; kernels bound by HBM hardly notice,
