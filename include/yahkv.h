@@ -192,8 +192,9 @@ int yahkv_decode_attend(const yahkv_geometry* g, const yahkv_pools* pools, const
 /* One decode step of a layer, LoomDecoder::Step's sequence kappend, vappend, part_q, reduce
  * (loom_decoder.hpp:253-268), in two dispatches: the result is that of yahkv_append(n_new = 1, start_pos =
  * seq_len - 1) followed by yahkv_decode_attend, pools and output. seq_len[s] counts the step's own token, which goes
- * to position seq_len[s] - 1 (clamped to the table like every position); a sequence with seq_len[s] <= 0 gets no
- * token and rows of zeros. k_new, v_new: [n_seqs][H][D] of new_dtype (F32, F16 or BF16), 16-byte aligned. The split-K
+ * to position seq_len[s] - 1 (clamped to the table like every position, and attended to exactly when the attention
+ * of the two separate calls would reach it; lengths the host's validation accepts always are); a sequence with
+ * seq_len[s] <= 0 gets no token and rows of zeros. k_new, v_new: [n_seqs][H][D] of new_dtype (F32, F16 or BF16), 16-byte aligned. The split-K
  * dispatch runs over the tokens the pools already hold; the merge quantizes the new token (the append kernels'
  * arithmetic, bit for bit), writes it to its slot and adds its term. opt->one_launch is refused (YAHKV_ERR_ARG). */
 int yahkv_decode_step(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,

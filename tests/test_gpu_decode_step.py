@@ -167,3 +167,37 @@ def test_step_refuses_bad_arguments(yahkv, torch_gpu):
     assert yahkv.lib.yahkv_decode_step(C.byref(g), C.byref(st), table.data_ptr(), 2, lens.data_ptr(), 1, 32,
                                        kv.data_ptr(), kv.data_ptr(), 0, q.data_ptr(), 0, 0.1, None, out.data_ptr(),
                                        ws.data_ptr(), 16, None, None) == -4
+
+
+def test_large_batch_of_short_sequences_through_the_step(yahkv, torch_gpu):
+    """1200 sequences of 0 to 40 tokens: most chunks span dozens of (sequence, kv head) pairs, many sequences have
+    nothing but their new token (no partial at all), some have none."""
+    rng = np.random.default_rng(91)
+    lens = [int(x) for x in rng.integers(0, 41, 1200)]
+    run_case(yahkv, torch_gpu, 8, 8, 2, 128, 16, lens, seed=92)
+
+
+def test_positions_past_the_table_clamp_as_in_the_append(yahkv, torch_gpu):
+    """Lengths that the host's validation would refuse still behave as the two separate calls do. A length beyond what
+    the page table covers: the token goes to the table's last slot, as yahkv_append puts it (positions clamp to the
+    table, gen_decode_attn.py:59-63), and the attention runs over the table's extent. A length beyond the host's bound
+    where the table reaches further: the token is stored at its position and the attention stops short of it."""
+    torch = torch_gpu
+    rng = np.random.default_rng(93)
+    n_q, n_kv, hd, pt = 8, 2, 128, 16
+    g, table, host, (dev, dev2), _ = build(yahkv, 8, n_q, n_kv, hd, pt, [49, 49, 49], seed=94)   # 48 tokens held each
+    table = table[:, :3].copy()                           # ... and a table that ends there
+    extent = table.shape[1] * pt
+    t_table = torch.from_numpy(table).cuda()
+    k = to_dev(torch, to_bf16_f32(rng.standard_normal((3, n_kv, hd))), "bf16")
+    v = to_dev(torch, to_bf16_f32(rng.standard_normal((3, n_kv, hd))), "bf16")
+    q = to_dev(torch, to_bf16_f32(rng.standard_normal((3, n_q, hd))), "bf16")
+    for lens, bound in (([extent + 7, extent, 20], extent + 7), ([40, 31, 30], 30)):
+        t_lens = torch.tensor(lens, dtype=torch.int32, device="cuda")
+        got = yahkv.decode_step(dev, t_table, t_lens, bound, k, v, q, 0.1).cpu().numpy()
+        yahkv.append(dev2, t_table, t_lens - 1, k[:, None], v[:, None])
+        two = yahkv.decode_attend(dev2, t_table, t_lens, bound, q, 0.1).cpu().numpy()
+        a, b = dev.numpy(), dev2.numpy()
+        for name in a:
+            assert np.array_equal(a[name], b[name]), (name, lens)
+        assert np.all(np.isfinite(got)) and rel_err(got, two) < 6e-4, lens

@@ -74,8 +74,18 @@ struct StepRows {
   int32_t dtype;
 };
 
+// Keys of sequence s the part kernel covers. In the step form (len_bias = -1) the length counts a token that is not in
+// the pools yet and will go to position len - 1, clamped to the table like every position; the kernel covers what an
+// attention after the append would cover, less that token's slot: the slot is the last covered position in every
+// case but one (a length beyond the host's bound while the table reaches further: the attention then stops short of
+// the new token, as it would after an append of its own).
+__device__ __forceinline__ bool StepSeesNewToken(const DecodeArgs& a, int len) {
+  const int covered = min(max(len, 0), a.max_len), slot = min(max(len - 1, 0), a.stride * a.g.pt - 1);
+  return len >= 1 && slot == covered - 1;
+}
 __device__ __forceinline__ int ClampLen(const DecodeArgs& a, int s) {
-  return min(max(a.seq_len[s] + a.len_bias, 0), a.max_len);
+  const int len = a.seq_len[s], covered = min(max(len, 0), a.max_len);
+  return a.len_bias != 0 && StepSeesNewToken(a, len) ? covered - 1 : covered;
 }
 
 // The line of tiles is cut into groups of eight chunks, 8 A tiles a group; chunk j of a group takes the tiles
@@ -1104,14 +1114,16 @@ __global__ __launch_bounds__(kReduceThreads) void DattnReduce(const DecodeArgs a
   const int DZ = D / gridDim.z, d0 = blockIdx.z * DZ;  // this workgroup's dims are [d0, d0 + DZ)
   const size_t o = (size_t(s) * g.n_q + hq) * D + d0;
   const int ts = TilesOf(a, s);
-  const bool has_new = rows.k != nullptr && a.seq_len[s] >= 1;  // the step form, and the sequence has a new token
-  if (ts <= 0 && !has_new) {  // length 0
+  // the step form: a sequence with a new token has it stored, and (but for the case StepSeesNewToken describes) attended to
+  const bool stores_new = rows.k != nullptr && a.seq_len[s] >= 1;
+  const bool has_new = stores_new && StepSeesNewToken(a, a.seq_len[s]);
+  __shared__ float new_score;
+  __shared__ __align__(16) float new_v[256];
+  if (stores_new && t < 128) StepToken(a, rows, s, h, hq, t / 64, t % 64, gi == 0 && blockIdx.z == 0, &new_score, new_v);
+  if (ts <= 0 && !has_new) {  // nothing to attend to
     if (t < DZ) a.out[o + t] = 0.0f;
     return;
   }
-  __shared__ float new_score;
-  __shared__ __align__(16) float new_v[256];
-  if (has_new && t < 128) StepToken(a, rows, s, h, hq, t / 64, t % 64, gi == 0 && blockIdx.z == 0, &new_score, new_v);
   // line units of the sequences before this one and of the whole line; the pair's tiles follow its first units
   size_t p0 = 0, p1 = 0;  // (a sequence that has nothing but its new token has no partials)
   if (ts > 0) {
