@@ -34,6 +34,7 @@ WORKLOADS = {
     # chunked prefill: every sequence holds `lo` tokens and takes a chunk of `chunk` more per step (the first six
     # launches of the attention kernel after an idle GPU run up to 25 % longer than the later ones)
     "prefill_b8_ctx16k_chunk2k_q8_0": dict(fmt=8, batch=8, lo=16384, hi=16384, seed=4, chunk=2048, warmup=10),
+    "prefill_b8_ctx16k_chunk2k_q4_0": dict(fmt=4, batch=8, lo=16384, hi=16384, seed=4, chunk=2048, warmup=10),
     # the unquantized f16 twins of the decode path (4096 B per token)
     "b16_ctx128k_f16": dict(fmt=16, batch=16, lo=131072, hi=131072, seed=4),
     "ragged_b64_f16": dict(fmt=16, batch=64, lo=1024, hi=65536, seed=4),
@@ -385,6 +386,13 @@ def run_prefill(a, wl, torch, yahkv):
         yahkv.append(pools, t_table, t_prefix, knew, vnew)
         if app:
             app[1].record()
+        if a.one_pass:                      # no workspace: the kernel that decodes each tile while staging it
+            if pair:
+                pair[0].record()
+            yahkv.prefill_attend(pools, t_table, t_prefix, prefix, q, scale, out=out, workspace=False)
+            if pair:
+                pair[1].record()
+            return
         yahkv.prefill_decode_tiles(pools, t_table, t_prefix, prefix, B, chunk, ws)
         if pair:
             pair[0].record()
@@ -402,8 +410,9 @@ def run_prefill(a, wl, torch, yahkv):
     err = 0.0
     for s_ in (0, B - 1):
         k, v = yahkv.gather_blocks(pools, t_table[s_], n)
-        Kd = oracle.dequantize_q8_0(k.cpu().numpy().reshape(-1, 34)).reshape(n, NKV, HD).astype(np.float64)
-        Vd = oracle.dequantize_q8_0(v.cpu().numpy().reshape(-1, 34)).reshape(n, NKV, HD).astype(np.float64)
+        deq, bb = (oracle.dequantize_q8_0, 34) if wl["fmt"] == 8 else (oracle.dequantize_q4_0, 18)
+        Kd = deq(k.cpu().numpy().reshape(-1, bb)).reshape(n, NKV, HD).astype(np.float64)
+        Vd = deq(v.cpu().numpy().reshape(-1, bb)).reshape(n, NKV, HD).astype(np.float64)
         for t in (0, 1, chunk // 3, chunk // 2, chunk - 65, chunk - 1):
             for h in (0, 7, 13, NQ - 1):
                 sc = Kd[:prefix + t + 1, h // (NQ // NKV)] @ q[s_, t, h].float().cpu().numpy().astype(np.float64) * scale
@@ -425,27 +434,31 @@ def run_prefill(a, wl, torch, yahkv):
     ms = dt / a.steps * 1e3
     kern_ms = float(np.mean([p[0].elapsed_time(p[1]) for p in ev]))
     app_ms = float(np.median([p[0].elapsed_time(p[1]) for p in ev_app]))
-    app_bytes = B * chunk * (2 * NKV * HD * 2 + 2 * NKV * (HD // 32) * 34)   # bf16 K and V rows in, q8_0 blocks out
+    app_bytes = B * chunk * (2 * NKV * HD * 2 + 2 * NKV * (HD // 32) * (34 if wl["fmt"] == 8 else 18))   # bf16 rows in, blocks out
     flops = float(B) * NQ * chunk * (prefix + (chunk + 1) / 2) * HD * 4   # both products, causal part counted once
     res = {
-        "metric": "chunked-prefill attention over paged q8 KV, TFLOP/s (f16 MFMA) + tok/s",
+        "metric": "chunked-prefill attention over paged q%d KV, TFLOP/s (f16 MFMA) + tok/s" % wl["fmt"],
         "value": round(flops / (ms * 1e-3) / 1e12, 1), "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps,
         "warmup": a.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f16", "data": "synthetic",
         "config": {"workload": a.workload, "batch": B, "prefix": prefix, "chunk": chunk, "n_q_heads": NQ,
-                   "n_kv_heads": NKV, "head_dim": HD, "page_tokens": PT, "n_pages": g.n_pages, "kv_format": "q8_0",
-                   "step": "append chunk (quantize + scatter) + decode tiles to f16 + causal attention"},
+                   "n_kv_heads": NKV, "head_dim": HD, "page_tokens": PT, "n_pages": g.n_pages,
+                   "kv_format": "q%d_0" % wl["fmt"],
+                   "step": ("append chunk (quantize + scatter) + causal attention that decodes its tiles itself" if a.one_pass
+                            else "append chunk (quantize + scatter) + decode tiles to f16 + causal attention")},
         "tok_per_s": round(B * chunk / (ms * 1e-3), 1), "flops_per_step": int(flops),
         "parity_max_rel_err": float(f"{err:.3e}"), "out_fnv1a": first_hash,
-        "append": {"kernel": "AppendPages<8>", "ms": round(app_ms, 4), "bytes": int(app_bytes),
+        "append": {"kernel": "AppendPages<%d, 2>" % wl["fmt"], "ms": round(app_ms, 4), "bytes": int(app_bytes),
                    "GB/s": round(app_bytes / (app_ms * 1e-3) / 1e9, 1),
                    "frac_of_hbm_peak": round(app_bytes / (app_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                    "note": "quantize + scatter of the chunk, HIP events around the call (median)"},
         "roofline": {"bound": "mfma", "achieved": round(flops / (kern_ms * 1e-3) / 1e12, 1),
                      "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(flops / (kern_ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
-                     "traffic": TRAFFIC[a.workload][0], "traffic_source": TRAFFIC[a.workload][1],
-                     "kernel": "PrefillAttendImg<%d, 2>" % HD, "kernel_ms": round(kern_ms, 4)},
+                     "traffic": None if a.one_pass else TRAFFIC.get(a.workload, (None, None))[0],
+                     "traffic_source": None if a.one_pass else TRAFFIC.get(a.workload, (None, None))[1],
+                     "kernel": ("PrefillAttendFused<%d, %d, %d>" % (wl["fmt"], HD, PT) if a.one_pass
+                                else "PrefillAttendImg<%d, 2>" % HD), "kernel_ms": round(kern_ms, 4)},
     }
     if a.clock_trace:
         res["clock_trace"] = clock_trace(
@@ -714,6 +727,8 @@ def main():
                     help="decode workloads: opt.deterministic (fixed tile pattern per wave: same bytes in, same bits out)")
     ap.add_argument("--one-launch", action="store_true",
                     help="decode workloads: yahkv_decode_attend with opt.one_launch instead of part + reduce")
+    ap.add_argument("--one-pass", action="store_true",
+                    help="quantized prefill workloads: no workspace, the attention kernel decodes its tiles itself")
     ap.add_argument("--separate-append", action="store_true",
                     help="decode workloads: the step's token is appended by a dispatch of its own (three per step)")
     ap.add_argument("--clock-trace", action="store_true",
