@@ -1064,8 +1064,15 @@ __device__ __forceinline__ void StepToken(const DecodeArgs& a, const StepRows& r
   const Geom& g = a.g;
   const int D = g.hd, d0 = 4 * lane;
   const bool has = d0 < D, is_v = wave == 1;
-  float4 x = {0.0f, 0.0f, 0.0f, 0.0f};
+  // everything this wave reads is asked for before anything is stored (a load behind a store waits for it)
+  float4 x = {0.0f, 0.0f, 0.0f, 0.0f}, qv = x;
   if (has) x = Load4(is_v ? rows.v : rows.k, (size_t(s) * g.n_kv + h) * D + d0, rows.dtype);
+  if (has && !is_v) qv = Load4(a.q, (size_t(s) * g.n_q + hq) * D + d0, a.q_dtype);  // as the part kernel sees it: f16
+  int page = 0, slot = 0;
+  if (writes) {  // the token's place: as in the append kernels, position clamped to the table
+    const int pos = min(max(a.seq_len[s] - 1, 0), a.stride * g.pt - 1);
+    page = ClampPage(a.table[int64_t(s) * a.stride + pos / g.pt], g.n_pages), slot = pos % g.pt;
+  }
   uint16_t scale;
   uint32_t own, codes;
   if (g.format == 8) {
@@ -1080,9 +1087,7 @@ __device__ __forceinline__ void StepToken(const DecodeArgs& a, const StepRows& r
     const int byte = static_cast<int>((own >> (8 * j)) & 0xFFu);
     v[j] = static_cast<float>(g.format == 8 ? static_cast<int>(static_cast<int8_t>(byte)) : byte - 8) * d;
   }
-  if (writes && has) {  // the token's place: as in the append kernels, position clamped to the table
-    const int pos = min(max(a.seq_len[s] - 1, 0), a.stride * g.pt - 1);
-    const int page = ClampPage(a.table[int64_t(s) * a.stride + pos / g.pt], g.n_pages), slot = pos % g.pt;
+  if (writes && has) {
     if (g.format == 8) {
       if (is_v) StoreRowV<8>(a.pools, g, page, h, slot, lane, codes, scale);
       else StoreRowK<8>(a.pools, g, page, h, slot, lane, codes, scale);
@@ -1095,8 +1100,6 @@ __device__ __forceinline__ void StepToken(const DecodeArgs& a, const StepRows& r
     if (has) *reinterpret_cast<float4*>(&vrow[d0]) = float4{v[0], v[1], v[2], v[3]};
     return;
   }
-  float4 qv = {0.0f, 0.0f, 0.0f, 0.0f};  // the query as the part kernel sees it: f16, saturated
-  if (has) qv = Load4(a.q, (size_t(s) * g.n_q + hq) * D + d0, a.q_dtype);
   float dot = static_cast<float>(SaturateToF16(qv.x)) * v[0] + static_cast<float>(SaturateToF16(qv.y)) * v[1] +
               static_cast<float>(SaturateToF16(qv.z)) * v[2] + static_cast<float>(SaturateToF16(qv.w)) * v[3];
   dot = WaveSum(dot);
