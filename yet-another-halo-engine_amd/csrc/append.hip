@@ -302,12 +302,18 @@ __global__ __launch_bounds__(64 * kPageWaves) void AppendPages(const RopeArgs a)
   // ---- the images' written parts to the pools
   const size_t ph = size_t(page) * H + h;
   const int n_t = t_hi - t_lo, tid = threadIdx.x, NT = 64 * kPageWaves;
+  const int lg_pt = __builtin_ctz(static_cast<unsigned>(PT));  // pages are 16, 32 or 64 tokens
   {  // K codes: per block the tokens' pieces are contiguous
     uint8_t* dst = a.pools.kq + ph * (size_t(NB) * PT * KB);
-    const int per_block = n_t * KB / 16;
-    for (int u = tid; u < NB * per_block; u += NT) {
-      const int off = ((u / per_block) * PT + t_lo) * KB + (u % per_block) * 16;
-      *reinterpret_cast<uint4*>(dst + off) = *reinterpret_cast<const uint4*>(&lk[off]);
+    if (n_t == PT) {  // a whole page (most of a chunk's): the region as it lies, no division by a run-time value
+      for (int u = tid; u < (NB * KB / 16) << lg_pt; u += NT)
+        *reinterpret_cast<uint4*>(dst + u * 16) = *reinterpret_cast<const uint4*>(&lk[u * 16]);
+    } else {
+      const int per_block = n_t * KB / 16;
+      for (int u = tid; u < NB * per_block; u += NT) {
+        const int off = ((u / per_block) * PT + t_lo) * KB + (u % per_block) * 16;
+        *reinterpret_cast<uint4*>(dst + off) = *reinterpret_cast<const uint4*>(&lk[off]);
+      }
     }
   }
   {  // K scales: [token][block], 8 bytes at a time
@@ -320,8 +326,8 @@ __global__ __launch_bounds__(64 * kPageWaves) void AppendPages(const RopeArgs a)
   uint8_t* vdst = a.pools.vq + ph * (size_t(v_rows) * PT);
   uint16_t* sdst = a.pools.vs + ph * (size_t(NB) * PT);
   if (n_t == PT) {  // a whole page: both V regions are contiguous
-    for (int u = tid; u < v_rows * PT / 16; u += NT) {
-      const uint32_t* src = reinterpret_cast<const uint32_t*>(&lv[(u * 16 / PT) * (PT + 4) + u * 16 % PT]);
+    for (int u = tid; u < (v_rows << lg_pt) / 16; u += NT) {
+      const uint32_t* src = reinterpret_cast<const uint32_t*>(&lv[((u * 16) >> lg_pt) * (PT + 4) + ((u * 16) & (PT - 1))]);
       *reinterpret_cast<uint4*>(vdst + u * 16) = uint4{src[0], src[1], src[2], src[3]};
     }
     for (int u = tid; u < NB * PT / 8; u += NT)

@@ -12,13 +12,15 @@
 
 namespace yahkv {
 
-// A code from x * inv as the x86-64 reference computes it: lround, whose result for a non-finite or out-of-range
-// argument converts to the int8 0 there (only reachable when 1 / d overflowed, i.e. amax < 2^-119).
-// In that range lround(r) is the truncation of r + copysign(0.5 - 2^-25, r): adding the float below one half moves
-// exactly the values with a fraction of one half or more past the next integer (r + 0.5 itself would also carry
-// 0.5 - 2^-25 there, through the tie of the addition's rounding). Checked against lroundf for every float up to 129.
-__device__ __forceinline__ int CodeQ8(float r) {
-  return fabsf(r) <= 128.0f ? static_cast<int>(r + copysignf(0x1.fffffep-2f, r)) : 0;
+// A code from r = x * inv as the x86-64 reference computes it: lround. For |r| <= 128, lround(r) is the truncation of
+// r + copysign(0.5 - 2^-25, r): adding the float below one half moves exactly the values with a fraction of one half
+// or more past the next integer (r + 0.5 itself would also carry 0.5 - 2^-25 there, through the tie of the addition's
+// rounding). Checked against lroundf for every float up to 129. Beyond that range (only reachable when 1 / d
+// overflowed, i.e. amax < 2^-119: the products are then infinite or NaN) lround's result converts to the int8 0 on the
+// reference's machine; CodesLanesQ8 sees to that case once per block.
+__device__ __forceinline__ int RoundQ8(float r) {
+#pragma clang fp contract(off)
+  return static_cast<int>(r + copysignf(0x1.fffffep-2f, r));
 }
 
 template <int CTRL>
@@ -62,13 +64,13 @@ __device__ __forceinline__ void ScaleQ8(float amax, float* inv, uint16_t* scale)
   *inv = d > 0.0f ? 1.0f / d : 0.0f;
   *scale = __builtin_bit_cast(uint16_t, static_cast<_Float16>(d));
 }
-__device__ __forceinline__ uint32_t CodesLanesQ8(const float4 v, float inv) {  // this lane's 4 codes in a dword
+// This lane's 4 codes in a dword. |x * inv| is at most 127 (and a bit of rounding) whenever inv is finite, so whether
+// the products are in RoundQ8's range is one question per block, asked of inv.
+__device__ __forceinline__ uint32_t CodesLanesQ8(const float4 v, float inv) {
 #pragma clang fp contract(off)
-  const uint32_t c0 = static_cast<uint8_t>(static_cast<int8_t>(CodeQ8(v.x * inv)));
-  const uint32_t c1 = static_cast<uint8_t>(static_cast<int8_t>(CodeQ8(v.y * inv)));
-  const uint32_t c2 = static_cast<uint8_t>(static_cast<int8_t>(CodeQ8(v.z * inv)));
-  const uint32_t c3 = static_cast<uint8_t>(static_cast<int8_t>(CodeQ8(v.w * inv)));
-  return c0 | (c1 << 8) | (c2 << 16) | (c3 << 24);
+  const uint32_t c0 = static_cast<uint32_t>(RoundQ8(v.x * inv)) & 0xFFu, c1 = static_cast<uint32_t>(RoundQ8(v.y * inv)) & 0xFFu;
+  const uint32_t c2 = static_cast<uint32_t>(RoundQ8(v.z * inv)) & 0xFFu, c3 = static_cast<uint32_t>(RoundQ8(v.w * inv)) & 0xFFu;
+  return inv < __builtin_inff() ? c0 | (c1 << 8) | (c2 << 16) | (c3 << 24) : 0u;
 }
 __device__ __forceinline__ uint32_t QuantizeLanesQ8(const float4 v, uint16_t* scale) {
   float inv;
