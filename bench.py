@@ -570,7 +570,8 @@ def run_decode(a, wl, torch, yahkv):
     knew = torch.randn((total, B, 1, NKV, HD), generator=gen, device="cuda").to(torch.bfloat16)
     vnew = torch.randn((total, B, 1, NKV, HD), generator=gen, device="cuda").to(torch.bfloat16)
     out = torch.empty((B, NQ, HD), dtype=torch.float32, device="cuda")
-    opt = yahkv.decode_options(one_launch=a.one_launch, deterministic=a.deterministic)
+    opt = yahkv.decode_options(one_launch=a.one_launch, deterministic=a.deterministic,
+                               min_chunk_tiles=a.min_chunk_tiles)
     ws = torch.empty(yahkv.decode_workspace_bytes(g, B, max_len, opt), dtype=torch.uint8, device="cuda")
     # set-up, as a server does once: the XCDs' relative read speeds on this batch (equal shares without it)
     xcd = yahkv.decode_calibrate(pools, t_table, len_rows[0], max_len, q, ws, opt, rounds=3) if not a.no_calibrate else None
@@ -729,6 +730,8 @@ def main():
                     help="decode workloads: yahkv_decode_attend with opt.one_launch instead of part + reduce")
     ap.add_argument("--one-pass", action="store_true",
                     help="quantized prefill workloads: no workspace, the attention kernel decodes its tiles itself")
+    ap.add_argument("--min-chunk-tiles", type=int, default=0,
+                    help="decode workloads: yahkv_decode_options::min_chunk_tiles (0: the library's default)")
     ap.add_argument("--separate-append", action="store_true",
                     help="decode workloads: the step's token is appended by a dispatch of its own (three per step)")
     ap.add_argument("--clock-trace", action="store_true",
