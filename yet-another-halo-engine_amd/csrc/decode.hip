@@ -95,11 +95,18 @@ __device__ __forceinline__ long long ChunkStart(const DecodeArgs& a, long long A
   return (k / 8) * 8 * A + 8 * A * a.share[k % 8] / 8192;
 }
 __device__ __forceinline__ int ChunkOf(const DecodeArgs& a, long long A, long long tile) {
-  const long long r = tile % (8 * A);
+  const long long span = 8 * A;
+  long long group, r;
+  if (tile >= 0 && tile < (1ll << 31) && span < (1ll << 31)) {  // one 32-bit division (see ChunkUnits)
+    const uint32_t q = static_cast<uint32_t>(tile) / static_cast<uint32_t>(span);
+    group = q, r = tile - static_cast<long long>(q) * span;
+  } else {
+    group = tile / span, r = tile % span;
+  }
   int j = 0;
 #pragma unroll
-  for (int i = 1; i < 8; ++i) j += 8 * A * a.share[i] / 8192 <= r;
-  return static_cast<int>(tile / (8 * A)) * 8 + j;
+  for (int i = 1; i < 8; ++i) j += span * a.share[i] / 8192 <= r;
+  return static_cast<int>(group) * 8 + j;
 }
 
 // ---- plan -------------------------------------------------------------------------------------------------------------
@@ -116,9 +123,15 @@ __device__ __forceinline__ int ChunkOf(const DecodeArgs& a, long long A, long lo
 // finish up to 50 us apart, by the number of pairs their chunks hold.
 __device__ __forceinline__ int TilesOf(const DecodeArgs& a, int s) { return (ClampLen(a, s) + kTile - 1) / kTile; }
 __device__ __forceinline__ int UnitsOf(const DecodeArgs& a, int ts) { return ts > 0 ? ts + a.pair_cost : 0; }
+// (Divisions of line coordinates: 64-bit divisions by run-time values are long sequences of scalar instructions, which
+// every wave of the merge kernel would repeat; a line below 2^31 units, any real one, takes the 32-bit form.)
 __device__ __forceinline__ long long ChunkUnits(const DecodeArgs& a, long long line) {
   // a short line is not cut finer than min_chunk_tiles: each piece costs a partial (G x (D + 2) floats)
-  return max((line + a.n_chunks - 1) / a.n_chunks, static_cast<long long>(a.min_chunk_tiles));
+  const long long per = line < (1ll << 31) - (1 << 21)
+                            ? static_cast<long long>((static_cast<uint32_t>(line) + static_cast<uint32_t>(a.n_chunks) - 1u) /
+                                                     static_cast<uint32_t>(a.n_chunks))
+                            : (line + a.n_chunks - 1) / a.n_chunks;
+  return max(per, static_cast<long long>(a.min_chunk_tiles));
 }
 
 // Chunk k of the line, for a whole workgroup of NT threads (all call it; two barriers inside): {sequence or -1, kv
@@ -1114,7 +1127,8 @@ __global__ __launch_bounds__(kReduceThreads) void DattnReduce(const DecodeArgs a
   const int G = g.group(), H = g.n_kv, D = g.hd;
   const int hq = blockIdx.x, s = blockIdx.y, t = threadIdx.x;
   const int h = hq / G, gi = hq % G;
-  const int DZ = D / gridDim.z, d0 = blockIdx.z * DZ;  // this workgroup's dims are [d0, d0 + DZ)
+  // this workgroup's dims are [d0, d0 + DZ); the launch's z extent divides a head_dim of 128 or 256: a power of two
+  const int DZ = D >> __builtin_ctz(gridDim.z), d0 = blockIdx.z * DZ;
   const size_t o = (size_t(s) * g.n_q + hq) * D + d0;
   const int ts = TilesOf(a, s);
   // the step form: a sequence with a new token has it stored, and (but for the case StepSeesNewToken describes) attended to
@@ -1154,7 +1168,8 @@ __global__ __launch_bounds__(kReduceThreads) void DattnReduce(const DecodeArgs a
   M = red[0];
   for (int w = 1; w < NW; ++w) M = fmaxf(M, red[w]);
   if (has_new) M = fmaxf(M, new_score);
-  const int lanes = DZ / 4, n_groups = kReduceThreads / lanes, grp = t / lanes, dl = t % lanes;
+  const int lg_lanes = __builtin_ctz(static_cast<unsigned>(DZ)) - 2;  // four dims a lane
+  const int lanes = 1 << lg_lanes, n_groups = kReduceThreads >> lg_lanes, grp = t >> lg_lanes, dl = t & (lanes - 1);
   float L = 0.0f;
   float4 A = {0.0f, 0.0f, 0.0f, 0.0f};
   for (size_t b0 = p0; b0 < p1; b0 += kReduceThreads) {
