@@ -57,9 +57,9 @@ struct DecodeArgs {
   int32_t pair_cost;  // line units a (sequence, kv head) pair takes besides its tiles
   int32_t share[9];  // cumulative shares of the eight chunks of a group, in 1/8192 of the group (share[8] = 8192)
   int32_t deterministic;  // waves take the chunk's tiles in a fixed pattern instead of first come, first served
-  unsigned long long* stamps;  // calibration only: [n_chunks] the time each workgroup's last wave finished
+  unsigned long long* stamps;  // calibration only: [2 * n_chunks] when each workgroup started, and when its last wave finished
   // one launch for part and merge: the workgroup that is last to finish a pair's tiles merges the pair's partials
-  int32_t fused;
+  int32_t fused;                // (read by the host, which launches the kernel's one-launch instance)
   uint32_t epoch;               // never 0, different in every launch (graph replays aside: see Arrive)
   unsigned long long* tickets;  // [n_seqs * H] arrivals per pair: (epoch << 32) | workgroups that have arrived
   // The step form (append + attention in two launches): seq_len counts the step's own token, which is not in the
@@ -1138,7 +1138,7 @@ __global__ __launch_bounds__(kReduceThreads) void DattnReduce(const DecodeArgs a
   __shared__ __align__(16) float new_v[256];
   if (stores_new && t < 128) StepToken(a, rows, s, h, hq, t / 64, t % 64, gi == 0 && blockIdx.z == 0, &new_score, new_v);
   if (ts <= 0 && !has_new) {  // nothing to attend to
-    if (t < DZ) a.out[o + t] = 0.0f;
+    for (int d = t; d < DZ; d += kReduceThreads) a.out[o + d] = 0.0f;
     return;
   }
   // line units of the sequences before this one and of the whole line; the pair's tiles follow its first units
@@ -1209,16 +1209,16 @@ __global__ __launch_bounds__(kReduceThreads) void DattnReduce(const DecodeArgs a
   *reinterpret_cast<float4*>(&sums[grp * DZ + 4 * dl]) = A;
   if (dl == 0) lsums[grp] = L;
   __syncthreads();
-  if (t < DZ) {
+  for (int d = t; d < DZ; d += kReduceThreads) {
     float v = 0.0f, lt = 0.0f;
-    for (int q = 0; q < n_groups; ++q) v += sums[q * DZ + t], lt += lsums[q];
+    for (int q = 0; q < n_groups; ++q) v += sums[q * DZ + d], lt += lsums[q];
     if (has_new) {
       const float w = __expf(new_score - M);
-      v = __builtin_fmaf(w, new_v[d0 + t], v), lt += w;
+      v = __builtin_fmaf(w, new_v[d0 + d], v), lt += w;
     }
     v /= lt;
-    if (a.gate != nullptr) v *= 1.0f / (1.0f + __expf(-a.gate[o + t]));
-    a.out[o + t] = v;
+    if (a.gate != nullptr) v *= 1.0f / (1.0f + __expf(-a.gate[o + d]));
+    a.out[o + d] = v;
   }
 }
 
