@@ -406,12 +406,19 @@ struct LoadDeviceN<2> {
 // the merge. The ticket word carries the launch's epoch above the count: a word with another epoch in it (memory that
 // was never used, or the zero the last arrival of an earlier launch left) counts as empty, so the workspace needs no
 // clearing, and the last arrival puts the zero back, so a graph replay, which repeats its epoch, starts clean too.
+// Only the first arrival of a launch has to replace the word (compare and swap); the others, who find the launch's
+// epoch in it, add one, which no number of simultaneous arrivals turns into retries.
 __device__ __forceinline__ int Arrive(unsigned long long* ticket, uint32_t epoch, uint32_t n) {
   unsigned long long old = __hip_atomic_load(ticket, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   while (true) {
-    const uint32_t count = static_cast<uint32_t>(old >> 32) == epoch ? static_cast<uint32_t>(old) : 0u;
-    const bool last = count + 1 == n;
-    const unsigned long long next = last ? 0ull : (static_cast<unsigned long long>(epoch) << 32) | (count + 1);
+    if (static_cast<uint32_t>(old >> 32) == epoch) {
+      old = __hip_atomic_fetch_add(ticket, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (static_cast<uint32_t>(old) + 1 != n) return 0;
+      __hip_atomic_store(ticket, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // everybody has arrived
+      return 1;
+    }
+    const bool last = n == 1;
+    const unsigned long long next = last ? 0ull : (static_cast<unsigned long long>(epoch) << 32) | 1ull;
     if (__hip_atomic_compare_exchange_strong(ticket, &old, next, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
                                              __HIP_MEMORY_SCOPE_AGENT))
       return last ? 1 : 0;
