@@ -64,3 +64,16 @@ def test_prefill_line():
     assert d["unit"] == "TFLOP/s" and d["roofline"]["bound"] == "mfma" and d["roofline"]["peak"] == 2500.0
     assert d["dtype"] == "f16" and d["parity_max_rel_err"] < 2e-3
     assert 0.0 < d["roofline"]["frac"] < 1.0 and 0.0 < d["append"]["frac_of_hbm_peak"] < 1.0
+
+
+@pytest.mark.gpu
+def test_clock_trace_and_step_options():
+    """--clock-trace adds the launch-by-launch durations with the shader clock after each and the clock under load; the
+    step's other forms (--separate-append, --graph-replay) give a line of the same shape."""
+    d = run(["--workload", "b1_ctx32k_q8_0", "--steps", "4", "--warmup", "1", "--no-cpu-baseline", "--clock-trace",
+             "--graph-replay", "--separate-append"])
+    ct = d["clock_trace"]
+    assert len(ct["kernel_ms"]) == len(ct["shader_mhz"]) == 60
+    assert all(300 < m < 3500 for m in ct["shader_mhz"]) and 300 < ct["under_load"]["shader_mhz_median"] < 3500
+    assert d["graph_replay"]["ms_per_step"] > 0 and "append, part, reduce" in d["config"]["step"]
+    assert d["roofline"]["kernel"] == "DattnPart<8, 256, 64, false>"
