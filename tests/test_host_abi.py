@@ -201,3 +201,33 @@ def test_decode_options_change_only_what_they_name(yahkv):
     assert yahkv.decode_workspace_bytes(g, 64, 65536, yahkv.decode_options(deterministic=True, pair_cost=-1,
                                                                            xcd_weight=[3, 1, 4, 1, 5, 9, 2, 6])) == base
     assert yahkv.decode_workspace_bytes(g, 64, 65536, yahkv.decode_options(n_chunks=512)) > base
+
+
+def test_header_is_plain_c(tmp_path):
+    """include/yahkv.h is the boundary a C, cgo or JNI binding includes: it must compile as C99 without warnings, and a C
+    program must link against the library with nothing but the header."""
+    import shutil
+    import subprocess
+    if shutil.which("gcc") is None:
+        pytest.skip("no gcc")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    src = tmp_path / "t.c"
+    src.write_text('#include <stdio.h>\n#include "yahkv.h"\n'
+                   "int main(void) {\n"
+                   "  yahkv_geometry g = {YAHKV_Q8_0, 24, 4, 256, 64, 8};\n"
+                   "  yahkv_decode_options o = {0};\n"
+                   '  printf("%zu %zu %d\\n", yahkv_kq_bytes(&g), yahkv_decode_workspace_bytes(&g, 2, 1000, &o),\n'
+                   "         yahkv_check_geometry(&g));\n"
+                   "  return 0;\n}\n")
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", "-I", os.path.join(root, "include"),
+                    "-fsyntax-only", str(src)], check=True)
+    pkg = os.path.join(root, "yet-another-halo-engine_amd")
+    exe = tmp_path / "t"
+    r = subprocess.run(["gcc", "-std=c99", "-I", os.path.join(root, "include"), str(src), "-L", pkg, "-lyahkv",
+                        "-Wl,-rpath," + pkg, "-Wl,-rpath,/opt/rocm/lib", "-L/opt/rocm/lib", "-o", str(exe)],
+                       capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-2000:]
+    out = subprocess.run([str(exe)], capture_output=True, text=True, timeout=60)
+    assert out.returncode == 0, out.stderr[-2000:]
+    kq, ws, ok = out.stdout.split()
+    assert int(kq) == 8 * 4 * 8 * 64 * 32 and int(ws) > 0 and int(ok) == 0
