@@ -2,8 +2,9 @@
  *
  * C ABI of the shared library libyahkv.so. Every entry point takes plain pointers and sizes; device
  * pointers are raw HIP device addresses, `stream` is a hipStream_t passed as void*. Entry points return
- * 0 on success or a negative yahkv_status; they never throw, never synchronize the device and, except
- * for yahkv_pagepool_*, never allocate.
+ * 0 on success or a negative yahkv_status; they never throw, never synchronize the device (the set-up call
+ * yahkv_decode_calibrate aside, which waits for its own measurements) and, except for yahkv_pagepool_*, never
+ * allocate.
  *
  * The entry points replace, for this path, the reference engine's kernel dispatches
  * (LoomDevice::Dispatch, engine/model/loom_runtime.hpp:372-376) issued by LoomDecoder::Step
