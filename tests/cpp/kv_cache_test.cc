@@ -123,6 +123,11 @@ int RunTest() {
         CheckHip(hipMemcpy(static_cast<char*>(sv.get()) + kv_n * 2 * i, v1.data(), kv_n * 2, hipMemcpyHostToDevice), "h2d");
         CheckHip(hipMemcpy(static_cast<char*>(sq.get()) + q_n * 2 * i, q1.data(), q_n * 2, hipMemcpyHostToDevice), "h2d");
       }
+      // the set-up call a server makes once: the XCDs' shares for this batch (a batch too small for whole groups of
+      // chunks keeps equal shares); the steps below must come out the same either way
+      dec.Calibrate(B, sq.get(), YAHKV_BF16, 2);
+      for (int j = 0; j < 8; ++j)
+        if (dec.options().xcd_weight[j] < 0) throw std::runtime_error("calibration left a negative weight");
       std::vector<std::vector<int32_t>> pos(steps, std::vector<int32_t>(B)), len(steps, std::vector<int32_t>(B));
       for (int i = 0; i < steps; ++i) {
         for (int s = 0; s < B; ++s) pos[i][s] = dec.length(s), len[i][s] = pos[i][s] + 1;

@@ -313,9 +313,28 @@ class KvDecoder {
     const int32_t* pos = static_cast<const int32_t*>(pos_dev_.get());
     const int32_t* ptab = static_cast<const int32_t*>(st_.ptab.ptr);
     Check(yahkv_decode_step(&g_, &pools, ptab, stride_, pos + max_seqs_, n_seqs, T_, k, v, kv_dtype, q, q_dtype,
-                            softmax_scale, gate, out, workspace_.get(), workspace_.size(), nullptr, stream_),
+                            softmax_scale, gate, out, workspace_.get(), workspace_.size(), &opt_, stream_),
           "decode_step");
   }
+
+  // Set-up, once a batch is in place (and again when its shape changes much): measures the XCDs' relative read speeds
+  // on sequences 0 .. n_seqs - 1 as they stand and keeps them for the steps to come (yahkv_decode_calibrate; worth
+  // about a percent of a large batch's step). Waits for the stream; the pools and lengths are left as they are.
+  void Calibrate(int32_t n_seqs, const void* q, int32_t q_dtype, int32_t rounds = 3) {
+    if (!bound_) throw KvError("decoder: no state bound");
+    if (n_seqs <= 0 || n_seqs > max_seqs_) throw KvError("decoder: bad batch");
+    Upload();
+    std::vector<int32_t> len(size_t(max_seqs_), 0);
+    for (int32_t s = 0; s < n_seqs; ++s) len[size_t(s)] = len_[size_t(s)];
+    DeviceBuffer dlen(sizeof(int32_t) * size_t(max_seqs_));
+    CheckHip(hipMemcpyAsync(dlen.get(), len.data(), sizeof(int32_t) * len.size(), hipMemcpyHostToDevice, stream_), "lengths");
+    CheckHip(hipStreamSynchronize(stream_), "lengths");
+    const yahkv_pools pools = PoolsOf(st_);
+    Check(yahkv_decode_calibrate(&g_, &pools, static_cast<const int32_t*>(st_.ptab.ptr), stride_,
+                                 static_cast<const int32_t*>(dlen.get()), n_seqs, T_, q, q_dtype, workspace_.get(),
+                                 workspace_.size(), &opt_, rounds, stream_), "decode_calibrate");
+  }
+  const yahkv_decode_options& options() const { return opt_; }
 
   const yahkv_geometry& geometry() const { return g_; }
   const KvDecoderState& state() const { return st_; }
@@ -348,6 +367,7 @@ class KvDecoder {
   std::vector<DeviceBuffer> own_;
   std::unique_ptr<PagePool> pool_;
   DeviceBuffer pos_dev_, workspace_;
+  yahkv_decode_options opt_{};  // defaults, and the XCD shares once Calibrate has run
   static constexpr size_t kStaging = 4;
   int32_t* pos_host_ = nullptr;  // [kStaging][2][max_seqs]
   hipEvent_t staged_[kStaging] = {nullptr, nullptr, nullptr, nullptr};
