@@ -119,16 +119,17 @@ __device__ __forceinline__ void Decode16V(const uint4 c, const uint4 s0, const u
 // out = o / l (* sigmoid(gate)); lane (query, lane group jg) holds dims 16 dt + 4 jg + r of its query in each row block.
 // The denominators l are the sums of the f16 numerators, accumulated by the matrix unit against an all-ones operand
 // next to V^T: numerators and denominator then carry the same rounding, and a lone key returns its V row exactly.
-template <int D, int RB>
-__device__ __forceinline__ void StoreRows(const PrefillArgs& a, int s, int h, int G, int jg, const f4v (&o)[RB][D / 16],
-                                          const f4v (&lacc)[RB], const int (&qpos)[RB], const int (&head)[RB]) {
-  constexpr int NDT = D / 16;
+// (NDT of the head's 16-dim tiles, starting with dim `dim0`: a wave that holds only part of its rows' dims)
+template <int D, int RB, int NDT = D / 16>
+__device__ __forceinline__ void StoreRows(const PrefillArgs& a, int s, int h, int G, int jg, const f4v (&o)[RB][NDT],
+                                          const f4v (&lacc)[RB], const int (&qpos)[RB], const int (&head)[RB],
+                                          int dim0 = 0) {
   const Geom& g = a.g;
 #pragma unroll
   for (int i = 0; i < RB; ++i) {
     if (head[i] >= G || qpos[i] >= a.chunk_len) continue;
     const float inv = 1.0f / lacc[i][0];  // every row of the all-ones product holds the query's denominator
-    const size_t base = ((size_t(s) * a.chunk_len + qpos[i]) * g.n_q + size_t(h) * G + head[i]) * D;
+    const size_t base = ((size_t(s) * a.chunk_len + qpos[i]) * g.n_q + size_t(h) * G + head[i]) * D + dim0;
 #pragma unroll
     for (int dt = 0; dt < NDT; ++dt) {
       float v[4];
@@ -886,6 +887,371 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
 }
 
 
+// ---- the same attention with the four waves working as two pairs ---------------------------------------------------
+//
+// In PrefillAttendImg every wave reads the whole K and V tile from LDS for its 32 queries: 1 KB of operand reads per two
+// matrix instructions, 256 KB per tile and workgroup, and with half of those reads left out (wrong results, timing
+// only) that kernel runs 24 % faster. Here a wave holds 64 queries (one head's 64 chunk positions) and a pair of waves
+// shares them: in S^T = K Q^T wave b of the pair takes the tile's keys 32 b .. 32 b + 31 against all 64 queries, in
+// O^T += V^T P^T it takes dims (D / 2) b .. of all 64 keys. Every operand read then feeds four matrix instructions
+// (144 KB of reads per tile and workgroup), and a wave's registers hold 64 queries' B operands (D / 2 registers) and
+// half of their accumulators (D / 2) where the other kernel holds 32 queries' (D / 4) and all of theirs (D / 2).
+// The price: a wave makes the numerators of its own 32 keys only and needs the pair's other 32 for the second
+// product. They go through LDS (4 KB per wave and tile) at the tile's one barrier, which therefore sits between the
+// softmax and the second product; the second product starts with the wave's own half while the other half arrives.
+// Each wave of a pair keeps its own reference point m of the numerators (it sees only its keys' scores); the waves
+// exchange m with the numerators, and where the two differ (the first tile or two of a row) both move to the larger
+// one, which rescales by powers of two as moving m always does.
+// LDS: two K halves, two V halves (a third V half as in the other kernel does not fit beside the numerators), one
+// 16 KB buffer of numerators, and a counter per wave that says which tiles the wave is through with. Before a wave
+// copies V(t + 1) where V(t - 1) was or replaces its numerators of tile t - 1, it looks at the four counters (all
+// waves are through with tile t - 1 as a rule by then; otherwise it waits). Copies: V(t + 1) beside the first
+// product of tile t + 1 (after that look), K(t + 3) beside the second product of tile t, where K(t + 1) was; the wait
+// before the barrier leaves the newest eight (V(t + 1)) in flight.
+// Measured on 8 x (16384 + 2048) tokens, D = 256: 6.9 - 7.0 ms against 6.0 - 6.25 ms of PrefillAttendImg<256, 2> on
+// the same box, so this kernel is built in only with -DYAHKV_PREFILL_PAIRS=1. Its LDS operand reads no longer bound
+// it (half of them left out: no change), but what it adds costs more than they did: the exchange of numerators at the
+// barrier (0.5 ms; matrix pipe idle from the last exponential to the first product after the barrier), the barrier
+// itself in the middle of a tile's work (0.4 ms), 4 more matrix instructions per tile for the denominators that
+// both waves of a pair sum, and the copies, squeezed by the two-buffer schedule (1.1 ms against 0.8 ms there).
+template <int D>
+__global__ __launch_bounds__(256) void PrefillAttendPair(const PrefillArgs a, const char* img, int tiles_per_pair) {
+  constexpr int KS = D / 32, NDH = D / 32, RB = 4, kHeadsPerGroup = 2;  // NDH: 16-dim tiles of a wave's half of the dims
+  constexpr int KIMG = kKeys * D * 2, TIMG = TileImageBytes<D>();
+  constexpr int kCopies = TIMG / 1024 / 4;  // 1 KB wave-wide copies per wave and tile
+  constexpr int VP = 3;                     // the V operand reads run this many 16-dim tiles ahead
+  static_assert(kCopies == 2 * NDH, "one copy per 16-dim tile of each half of the second product");
+  const Geom g = a.g;
+  const int G = g.group(), H = g.n_kv;
+  const int n_qt = (a.chunk_len + kQueries - 1) / kQueries, n_hp = (G + kHeadsPerGroup - 1) / kHeadsPerGroup;
+  const int bid = blockIdx.x, xcd = bid % 8, local = bid / 8, per_pair = n_qt * n_hp;
+  const int pair = xcd + 8 * (local / per_pair), qt = n_qt - 1 - (local % per_pair) / n_hp, hp = local % n_hp;
+  if (pair >= a.n_seqs * H) return;
+  const int s = pair / H, h = pair % H;
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / 64), lane = tid % 64;
+  const int b = wave & 1, partner = wave ^ 1;  // the wave's half of the keys / dims; the wave with the other half
+  const int qn = lane % 16, jg = lane / 16;
+  const int prefix = ClampPrefix(a.prefix_len, s, a.max_prefix, a.stride, g.pt, a.chunk_len);
+  const int q0 = qt * kQueries;
+  const int n_keys = min(prefix + q0 + kQueries, prefix + a.chunk_len);
+  const int n_tiles = (n_keys + kKeys - 1) / kKeys;
+
+  // One LDS object on purpose: with several, the compiler tells them apart by alias scopes, and with scopes on the
+  // copies' LDS side it makes every LDS read that follows a copy wait for the copy (vmcnt(0)), which serializes the
+  // kernel; without them it leaves the ordering of copies and reads to the waits written here.
+  constexpr int kPBuf = 4 * KIMG, kMBuf = kPBuf + 4 * RB * 64 * 16, kTaken = kMBuf + 4 * 16 * 16;
+  __shared__ __align__(1024) char lds_all[kTaken + 16];
+  typedef char (*Halves)[KIMG];
+  const Halves lds = reinterpret_cast<Halves>(lds_all);  // [0], [1]: K halves of tile images; [2], [3]: V halves
+  // per wave: its numerators as the second product's B operands
+  typedef uint4 (*PBuf)[RB][64];
+  const PBuf pbuf = reinterpret_cast<PBuf>(lds_all + kPBuf);
+  // per wave and query column: the reference points of its 4 row blocks
+  typedef f4v (*MBuf)[16];
+  const MBuf mbuf = reinterpret_cast<MBuf>(lds_all + kMBuf);
+  // per wave: the tiles it is through with (second product included). Plain accesses: the compiler makes an atomic or
+  // volatile LDS access wait for every copy in flight; the empty asm has the counters read again wherever the read
+  // is written.
+  typedef int i4v __attribute__((ext_vector_type(4)));
+  typedef __attribute__((address_space(3))) i4v* LdsCounters;
+  const LdsCounters through = (LdsCounters)(lds_all + kTaken);
+  auto slowest = [&]() -> int {  // tiles every wave of the workgroup is through with
+    LdsCounters p = through;
+    asm volatile("" : "+v"(p) : : "memory");
+    const i4v t = *p;
+    return min(min(t[0], t[1]), min(t[2], t[3]));
+  };
+
+  h8v qb[RB][KS];
+  int qpos[RB], head[RB];
+#pragma unroll
+  for (int i = 0; i < RB; ++i) {
+    head[i] = kHeadsPerGroup * hp + wave / 2;
+    qpos[i] = q0 + 16 * i + qn;
+    const int t = min(qpos[i], a.chunk_len - 1), hd = min(head[i], G - 1);
+    const uint16_t* qp = a.q + ((size_t(s) * a.chunk_len + t) * g.n_q + size_t(h) * G + hd) * D;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qb[i][ks] = QueryF16(qp + 32 * ks + 8 * jg);
+  }
+  f4v o[RB][NDH];
+  float m[RB];
+  f4v lacc[RB];
+#pragma unroll
+  for (int i = 0; i < RB; ++i) {
+    m[i] = kNegBig, lacc[i] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int dt = 0; dt < NDH; ++dt) o[i][dt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
+  }
+  const float sscale = a.scale * 1.4426950408889634f;
+  const auto img_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<char*>(img) + size_t(pair) * tiles_per_pair * TIMG, 0, 0x7fffffff, 0x00020000);
+  // copy j (of kCopies) of this wave's share of the image of `tile` (the last tile's when there is no such tile) into
+  // the buffers of that parity: pieces j < kCopies / 2 are the K half, the others V
+  auto copy_part = [&](int tile, int j) {
+    const int c = wave + 4 * j;
+    char* dst = j < kCopies / 2 ? lds[tile % 2] + c * 1024 : lds[2 + tile % 2] + (c * 1024 - KIMG);
+    tile = min(tile, n_tiles - 1);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(img_rsrc, (__attribute__((address_space(3))) void*)dst, 16, lane * 16,
+                                             tile * TIMG + c * 1024, 0, 0);
+  };
+  // byte offsets of this lane's operand reads within an image (see PrefillAttendImg); K rows are the wave's 32 keys,
+  // V^T rows the wave's D / 2 dims, `own` the 32-key step of the wave's own keys and `other` its partner's
+  const int sw_l = 16 * (jg ^ (qn % 4)), sw_h = 64 * (qn % 8 / 4);
+  const int krow = (32 * b + qn) * (2 * D) + sw_l;
+  const int koff[2] = {krow + sw_h, krow - sw_h};
+  const int vrow = (16 * NDH * b + qn) * 128 + sw_l;
+  const int v_own = vrow + 64 * b + (b ? -sw_h : sw_h), v_other = vrow + 64 * (1 - b) + (b ? sw_h : -sw_h);
+  auto read_k = [&](const char* buf, int ks, int kt) -> h8v {
+    return *reinterpret_cast<const h8v*>(buf + koff[ks % 2] + (kt * 16 * (2 * D) + 64 * ks));
+  };
+  // One 32-dim step of S^T = K Q^T for the wave's 32 keys: the A operands of the next step are read before the
+  // products of this one.
+  auto k_first = [&](const char* buf, h8v (&ka)[2][2]) {
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) ka[0][kt] = read_k(buf, 0, kt);
+  };
+  auto k_step = [&](const char* buf, int ks, h8v (&ka)[2][2], f4v (&st)[RB][2]) {
+    if (ks + 1 < KS) {
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt) ka[(ks + 1) % 2][kt] = read_k(buf, ks + 1, kt);
+    }
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int i = 0; i < RB; ++i)
+        st[i][kt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[ks % 2][kt], qb[i][ks], st[i][kt], 0, 0, 0);
+  };
+  auto clear = [&](f4v (&st)[RB][2]) {
+#pragma unroll
+    for (int i = 0; i < RB; ++i)
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt) st[i][kt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
+  };
+  // Largest score of a query over the wave's 32 keys, times the softmax scale; a row whose 32 keys are all masked
+  // gives kNegBig itself, which moves no reference point.
+  auto row_max = [&](auto masked, const f4v (&st)[2]) -> float {
+    float mx = fmaxf(st[0][0], st[0][1]);
+    mx = fmaxf(fmaxf(mx, st[0][2]), st[0][3]);
+    mx = fmaxf(fmaxf(mx, st[1][0]), st[1][1]), mx = fmaxf(fmaxf(mx, st[1][2]), st[1][3]);
+    const float r = MaxOverLaneGroups(mx);
+    return decltype(masked)::value && r == kNegBig ? kNegBig : r * sscale;  // sscale > 0 is required by the entry point
+  };
+  // sums, accumulators of row block i times alpha (a power of two); through a matrix instruction with zero factors,
+  // which keeps them in the accumulation registers (see PrefillAttendImg)
+  auto rescale = [&](int i, float alpha) {
+    const h8v zero = {0, 0, 0, 0, 0, 0, 0, 0};
+    {
+      f4v t = lacc[i];
+      asm volatile("" : "+a"(t));
+#pragma unroll
+      for (int r = 0; r < 4; ++r) t[r] *= alpha;
+      lacc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(zero, zero, t, 0, 0, 0);
+    }
+#pragma unroll
+    for (int dt = 0; dt < NDH; ++dt) {
+      f4v t = o[i][dt];
+      asm volatile("" : "+a"(t));
+#pragma unroll
+      for (int r = 0; r < 4; ++r) t[r] *= alpha;
+      o[i][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(zero, zero, t, 0, 0, 0);
+    }
+  };
+  auto move_reference = [&](int i, float mx) {
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(mx > m[i] + (kBias + kSlack)) != 0, 0)) {
+      const float mn = mx > m[i] + (kBias + kSlack) ? __builtin_ceilf(mx) - kBias : m[i];
+      const float alpha = __builtin_amdgcn_exp2f(m[i] - mn);
+      m[i] = mn;
+      rescale(i, alpha);
+    }
+  };
+  // f16 numerators of row block i over the wave's 32 keys: the B operand of the 32-key step `b` of the second product
+  auto numerators = [&](auto masked, int i, const f4v (&st)[2]) -> h8v {
+    uint32_t w[4];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) {
+      float p[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        p[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(st[kt][r], sscale, -m[i]));
+        if (decltype(masked)::value && m[i] == kNegBig) p[r] = 0.0f;  // no key of the row seen yet: nothing to weigh
+      }
+      w[2 * kt] = PackF16(p[0], p[1]), w[2 * kt + 1] = PackF16(p[2], p[3]);
+    }
+    return __builtin_bit_cast(h8v, uint4{w[0], w[1], w[2], w[3]});
+  };
+  typedef __attribute__((address_space(3))) const char* LdsPtr;
+  // One 32-key step of O^T += V^T P^T over the wave's dims, and of the denominators; `copy(dt)` issues a tile copy
+  // beside the products of dim tile dt.
+  auto pv_half = [&](LdsPtr vb, const h8v (&p)[RB], auto copy) {
+    asm volatile("" : "+v"(vb));  // (keeps the compiler from folding the lane address into every read's own register)
+    auto read_v = [&](int dt) -> h8v {
+      return *reinterpret_cast<const __attribute__((address_space(3))) h8v*>(vb + dt * 16 * 128);
+    };
+    h8v va[VP + 1];
+#pragma unroll
+    for (int dt = 0; dt < VP; ++dt) va[dt] = read_v(dt);
+#pragma unroll
+    for (int i = 0; i < RB; ++i) lacc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(OnesF16(), p[i], lacc[i], 0, 0, 0);
+#pragma unroll
+    for (int dt = 0; dt < NDH; ++dt) {
+      if (dt + VP < NDH) va[(dt + VP) % (VP + 1)] = read_v(dt + VP);
+#pragma unroll
+      for (int i = 0; i < RB; ++i)
+        o[i][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va[dt % (VP + 1)], p[i], o[i][dt], 0, 0, 0);
+      copy(dt);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  // One tile: the first product of the next tile beside the softmax of this one, the exchange of numerators at the
+  // barrier, the second product of this tile. `masked`: the tile may hold keys some query must not see, and may be
+  // the last one.
+  f4v st[RB][2];
+  auto tile_step = [&](auto masked, int tile) {
+    constexpr bool MASKED = decltype(masked)::value;
+    constexpr int KA = KS / 4;  // steps of the next tile's first product that run beside the row maxima
+    const bool more = !MASKED || tile + 1 < n_tiles;
+    const char* kbuf = lds[(tile + 1) % 2];
+    f4v sn[RB][2];
+    h8v ka[2][2];
+    float mx[RB];
+    h8v pvo[RB];
+    clear(sn);
+    // Before V(tile + 1) may go where V(tile - 1) was, and before this wave's numerators replace those of the tile
+    // before, every wave must be through with that tile's second product: the waves say so in LDS, and the wait is a
+    // look at the four counters, which as a rule are there by the time the row maxima are done.
+    auto wait_for_all = [&]() {
+      int t = slowest();
+      while (t < tile) {
+        __builtin_amdgcn_s_sleep(1);
+        t = slowest();
+      }
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    };
+    if (MASKED) {
+      if (more) {
+        k_first(kbuf, ka);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) k_step(kbuf, ks, ka, sn);
+      }
+#pragma unroll
+      for (int i = 0; i < RB; ++i)
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            if (tile * kKeys + 32 * b + 16 * kt + 4 * jg + r > prefix + qpos[i]) st[i][kt][r] = kNegBig;
+#pragma unroll
+      for (int i = 0; i < RB; ++i) move_reference(i, row_max(masked, st[i]));
+      wait_for_all();
+      if (more) {
+#pragma unroll
+        for (int j = kCopies / 2; j < kCopies; ++j) copy_part(tile + 1, j);
+      }
+#pragma unroll
+      for (int i = 0; i < RB; ++i) pvo[i] = numerators(masked, i, st[i]);
+    } else {
+      k_first(kbuf, ka);
+#pragma unroll
+      for (int ks = 0; ks < KA; ++ks) k_step(kbuf, ks, ka, sn);
+#pragma unroll
+      for (int i = 0; i < RB; ++i) mx[i] = row_max(masked, st[i]);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < RB; ++i) move_reference(i, mx[i]);
+      wait_for_all();
+      // the rest of the first product with the numerators beside it (the vector units' work between the matrix
+      // instructions) and the copies of V(tile + 1)
+#pragma unroll
+      for (int ks = KA; ks < KS; ++ks) {
+        k_step(kbuf, ks, ka, sn);
+        copy_part(tile + 1, kCopies / 2 + (ks - KA));
+      }
+#pragma unroll
+      for (int i = 0; i < RB; ++i) pvo[i] = numerators(masked, i, st[i]);
+#pragma unroll
+      for (int j = kCopies / 2 + (KS - KA); j < kCopies; ++j) copy_part(tile + 1, j);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < RB; ++i) pbuf[wave][i][lane] = __builtin_bit_cast(uint4, pvo[i]);
+    mbuf[wave][qn] = f4v{m[0], m[1], m[2], m[3]};  // (the four lane groups of a column write the same values)
+    // The copies complete in the order of their issue: all but the newest kCopies / 2, the pieces of V(tile + 1)
+    // just issued, have landed, this wave's pieces of K(tile + 2) and V(tile) among them; its numerators are written
+    // and its operand reads have returned (lgkmcnt(0)): then the barrier says the same of every wave.
+    // (A bare barrier: __syncthreads() carries a release fence, which waits for every copy in flight. The
+    // wavefront-scope fences emit nothing; they keep the compiler from moving LDS accesses across the barrier.)
+    __builtin_amdgcn_s_waitcnt((MASKED ? VmCnt(0) : VmCnt(kCopies / 2)) & 0xF0FF);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const f4v mp = mbuf[partner][qn];
+    h8v pvp[RB];
+#pragma unroll
+    for (int i = 0; i < RB; ++i) pvp[i] = __builtin_bit_cast(h8v, pbuf[partner][i][lane]);
+    LdsPtr vbuf = (LdsPtr)lds[2 + tile % 2];
+    const bool k_copy = !MASKED || tile + 3 < n_tiles;  // K(tile + 3) goes where K(tile + 1) was
+    pv_half(vbuf + v_own, pvo, [&](int dt) {
+      if (dt % 2 == 1 && k_copy) copy_part(tile + 3, dt / 2);
+    });
+    // the pair's two reference points: where they differ, both waves go to the larger one
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(mp[0] != m[0] || mp[1] != m[1] || mp[2] != m[2] || mp[3] != m[3]) != 0, 0)) {
+#pragma unroll
+      for (int i = 0; i < RB; ++i) {
+        const float mn = fmaxf(m[i], mp[i]);
+        const float alpha = __builtin_amdgcn_exp2f(m[i] - mn), beta = __builtin_amdgcn_exp2f(mp[i] - mn);
+        m[i] = mn;
+        rescale(i, alpha);
+        const _Float16 bh = static_cast<_Float16>(beta);  // a power of two, or zero when it is below f16's range
+#pragma unroll
+        for (int e = 0; e < 8; ++e) pvp[i][e] *= bh;
+      }
+    }
+    pv_half(vbuf + v_other, pvp, [&](int dt) {
+      if (dt % 2 == 1 && k_copy) copy_part(tile + 3, NDH / 2 + dt / 2);
+    });
+    // LDS serves a wave's accesses in order: once the counter is written, this wave's reads of V(tile) and of its
+    // partner's numerators have been served
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    reinterpret_cast<__attribute__((address_space(3))) int*>(through)[wave] = tile + 1;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    if (more) {
+#pragma unroll
+      for (int i = 0; i < RB; ++i)
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt) st[i][kt] = sn[i][kt];
+    }
+  };
+
+  // ---- prologue: K(0), K(1), V(0); S^T(0); then K(2) where K(0) was
+  if (tid < 4) reinterpret_cast<__attribute__((address_space(3))) int*>(through)[tid] = 0;
+#pragma unroll
+  for (int j = 0; j < kCopies; ++j) copy_part(0, j);
+#pragma unroll
+  for (int j = 0; j < kCopies / 2; ++j) copy_part(1, j);
+  __builtin_amdgcn_s_waitcnt(VmCnt(0));
+  __syncthreads();
+  clear(st);
+  {
+    h8v ka[2][2];
+    k_first(lds[0], ka);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      k_step(lds[0], ks, ka, st);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < kCopies / 2; ++j) copy_part(2, j);
+  const int n_full = min(n_tiles, (prefix + q0 + 1) / kKeys);  // tiles every query of the workgroup sees whole
+  const int n_pipe = min(n_full, n_tiles - 1);
+  int tile = 0;
+  for (; tile < n_pipe; ++tile) tile_step(Constant<false>{}, tile);
+  for (; tile < n_tiles; ++tile) tile_step(Constant<true>{}, tile);
+  StoreRows<D, RB, NDH>(a, s, h, G, jg, o, lacc, qpos, head, 16 * NDH * b);
+}
+
 // ---- the same attention on 32x32x16 matrix instructions ------------------------------------------------------------------
 //
 // v_mfma_f32_32x32x16_f16 does the work of two 16x16x32 instructions in one issue slot and runs 32 cycles in the matrix
@@ -1182,6 +1548,9 @@ namespace {
 #ifndef YAHKV_PREFILL_WIDE
 #define YAHKV_PREFILL_WIDE 0
 #endif
+#ifndef YAHKV_PREFILL_PAIRS
+#define YAHKV_PREFILL_PAIRS 0
+#endif
 // Which attention kernel serves a geometry, and with it the order of the keys in the V images. The kernel on 32x32x16
 // matrix instructions (head_dim 256 only) is built in with -DYAHKV_PREFILL_WIDE=1; it gives the same results and is
 // measured slower than the one on 16x16x32 (8 x (16384 + 2048) tokens: 6.66 ms against 5.87 ms), so it is off.
@@ -1296,6 +1665,7 @@ extern "C" int yahkv_prefill_attend_tiles(const yahkv_geometry* g, const yahkv_p
 #define YAHKV_LAUNCH_ATT(DD, RR) \
   hipLaunchKernelGGL((PrefillAttendImg<DD, RR>), AttendGrid(a, RR), dim3(256), 0, st, a, img, tiles)
   if (UseWide(a.g)) hipLaunchKernelGGL((PrefillAttendWide<256>), AttendGrid(a, 2), dim3(256), 0, st, a, img, tiles);
+  else if (a.g.hd == 256 && YAHKV_PREFILL_PAIRS) hipLaunchKernelGGL((PrefillAttendPair<256>), AttendGrid(a, 2), dim3(256), 0, st, a, img, tiles);
   else if (a.g.hd == 256) YAHKV_LAUNCH_ATT(256, 2);
   else if (a.g.group() % 3 == 0) YAHKV_LAUNCH_ATT(128, 3);
   else YAHKV_LAUNCH_ATT(128, 2);
@@ -1401,6 +1771,7 @@ extern "C" int yahkv_f16_prefill_attend(const yahkv_geometry* g, const yahkv_f16
 #define YAHKV_LAUNCH_ATT(DD, RR) \
   hipLaunchKernelGGL((PrefillAttendImg<DD, RR>), AttendGrid(a, RR), dim3(256), 0, st, a, img, tiles)
   if (UseWide(a.g)) hipLaunchKernelGGL((PrefillAttendWide<256>), AttendGrid(a, 2), dim3(256), 0, st, a, img, tiles);
+  else if (a.g.hd == 256 && YAHKV_PREFILL_PAIRS) hipLaunchKernelGGL((PrefillAttendPair<256>), AttendGrid(a, 2), dim3(256), 0, st, a, img, tiles);
   else if (a.g.hd == 256) YAHKV_LAUNCH_ATT(256, 2);
   else if (a.g.group() % 3 == 0) YAHKV_LAUNCH_ATT(128, 3);
   else YAHKV_LAUNCH_ATT(128, 2);
