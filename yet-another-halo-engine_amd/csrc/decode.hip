@@ -557,18 +557,18 @@ void DattnPart(const DecodeArgs a) {
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
       if constexpr (Q8) {
-        const uint4 v = *reinterpret_cast<const uint4*>(kp + (b * PT * KB + off));
+        const uint4 v = StreamLoad(reinterpret_cast<const uint4*>(kp + (b * PT * KB + off)));
         kb[b][0] = v.x, kb[b][1] = v.y, kb[b][2] = v.z, kb[b][3] = v.w;
       } else {
-        const uint2 v = *reinterpret_cast<const uint2*>(kp + (b * PT * KB + off));
+        const uint2 v = StreamLoad(reinterpret_cast<const uint2*>(kp + (b * PT * KB + off)));
         kb[b][0] = v.x, kb[b][1] = v.y;
       }
     }
     const uint8_t* sp = reinterpret_cast<const uint8_t*>(a.pools.ks) + ph * (PT * NB * 2) + t * (NB * 2);
     if (NB == 8) {
-      ksc = *reinterpret_cast<const uint4*>(sp);
+      ksc = StreamLoad(reinterpret_cast<const uint4*>(sp));
     } else {
-      const uint2 v = *reinterpret_cast<const uint2*>(sp);
+      const uint2 v = StreamLoad(reinterpret_cast<const uint2*>(sp));
       ksc = uint4{v.x, v.y, 0u, 0u};
     }
   };
@@ -589,7 +589,7 @@ void DattnPart(const DecodeArgs a) {
       const size_t ph = page_head(pg, 16 * kg);
       const uint8_t* vp = a.pools.vq + ph * (Q8 ? D * PT : NB * 16 * PT);
 #pragma unroll
-      for (int j = 0; j < NVB; ++j) vb[j] = *reinterpret_cast<const uint4*>(vp + (16 * (hf * NVB + j) * PT + off));
+      for (int j = 0; j < NVB; ++j) vb[j] = StreamLoad(reinterpret_cast<const uint4*>(vp + (16 * (hf * NVB + j) * PT + off)));
     } else if constexpr (PPT == 1) {
       const size_t ph = size_t(pg[0]) * H + cur.h;
       const auto rv = __builtin_amdgcn_make_buffer_rsrc(
@@ -597,7 +597,7 @@ void DattnPart(const DecodeArgs a) {
 #pragma unroll
       for (int j = 0; j < NVB; ++j)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, (__attribute__((address_space(3))) void*)(&lvq[j * 1024]), 16, off,
-                                                 16 * (hf * NVB + j) * PT, 0, 0);
+                                                 16 * (hf * NVB + j) * PT, 0, kStreamed);
     } else {
       const size_t ph = page_head(pg, 16 * kg);
       const uint8_t* vp = a.pools.vq + ph * (Q8 ? D * PT : NB * 16 * PT);
@@ -605,14 +605,14 @@ void DattnPart(const DecodeArgs a) {
       for (int j = 0; j < NVB; ++j)
         __builtin_amdgcn_global_load_lds(
             (const __attribute__((address_space(1))) void*)(vp + (16 * (hf * NVB + j) * PT + off)),
-            (__attribute__((address_space(3))) void*)(&lvq[j * 1024]), 16, 0, 0);
+            (__attribute__((address_space(3))) void*)(&lvq[j * 1024]), 16, 0, kStreamed);
     }
     if (hf == 0) {  // with the first half come the tile's V scales: lane = (block, 8 keys)
       const int b = lane / 8, chunk = lane % 8;
       if (b < NB) {
         const size_t ps = page_head(pg, 8 * chunk);
         const uint32_t soff = (b * PT + (8 * chunk) % PT) * 2;
-        vsr = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint8_t*>(a.pools.vs) + ps * (NB * PT * 2) + soff);
+        vsr = StreamLoad(reinterpret_cast<const uint4*>(reinterpret_cast<const uint8_t*>(a.pools.vs) + ps * (NB * PT * 2) + soff));
       }
     }
   };

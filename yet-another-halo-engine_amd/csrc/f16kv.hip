@@ -243,7 +243,7 @@ __global__ __launch_bounds__(64 * kWaves) void PartF16(const F16Args a) {
       const int page = ClampPage(row[min(key / PT, a.stride - 1)], g.n_pages);
       const uint16_t* kp = a.k + (size_t(page) * H + h) * (size_t(D) * PT) + (key % PT) * 16 + 8 * half;
 #pragma unroll
-      for (int g16 = 0; g16 < NG; ++g16) kb[g16] = *reinterpret_cast<const h8v*>(kp + g16 * PT * 16);
+      for (int g16 = 0; g16 < NG; ++g16) kb[g16] = StreamLoad(reinterpret_cast<const h8v*>(kp + g16 * PT * 16));
     }
     {  // V^T: this lane's dim of every 16-dim tile, 8 keys (they lie in one page: pages hold multiples of 16 tokens)
       const int key = key0 + 8 * kg;
@@ -252,7 +252,7 @@ __global__ __launch_bounds__(64 * kWaves) void PartF16(const F16Args a) {
       const uint16_t* vp =
           a.v + (size_t(page) * H + h) * (size_t(D) * PT) + (key % PT / RUN * D + n16) * RUN + key % RUN;
 #pragma unroll
-      for (int nt = 0; nt < NG; ++nt) vb[nt] = *reinterpret_cast<const h8v*>(vp + 16 * nt * RUN);
+      for (int nt = 0; nt < NG; ++nt) vb[nt] = StreamLoad(reinterpret_cast<const h8v*>(vp + 16 * nt * RUN));
     }
     f16v c = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll

@@ -473,12 +473,12 @@ __global__ __launch_bounds__(256) void PrefillImages(const ImageArgs a) {
       const float d = WidenF16(a.pools.ks[(ph * PT + t) * NB + b]);
       float v[8];
       if constexpr (Q8) {
-        const uint2 w = *reinterpret_cast<const uint2*>(a.pools.kq + ((ph * NB + b) * PT + t) * 32 + off);
+        const uint2 w = StreamLoad(reinterpret_cast<const uint2*>(a.pools.kq + ((ph * NB + b) * PT + t) * 32 + off));
 #pragma unroll
         for (int e = 0; e < 8; ++e)
           v[e] = d * static_cast<float>(static_cast<int8_t>(((e < 4 ? w.x : w.y) >> (8 * (e % 4))) & 0xFF));
       } else {  // byte j of a block: low nibble dim j, high nibble dim 16 + j
-        const uint2 w = *reinterpret_cast<const uint2*>(a.pools.kq + ((ph * NB + b) * PT + t) * 16 + off % 16);
+        const uint2 w = StreamLoad(reinterpret_cast<const uint2*>(a.pools.kq + ((ph * NB + b) * PT + t) * 16 + off % 16));
 #pragma unroll
         for (int e = 0; e < 8; ++e)
           v[e] = d * static_cast<float>(int((((e < 4 ? w.x : w.y) >> (8 * (e % 4))) >> (off / 16 * 4)) & 0xF) - 8);
@@ -501,9 +501,9 @@ __global__ __launch_bounds__(256) void PrefillImages(const ImageArgs a) {
       uint32_t w;
       int shift = 0;
       if constexpr (Q8) {
-        w = *reinterpret_cast<const uint32_t*>(a.pools.vq + (ph * D + dim) * PT + t);
+        w = StreamLoad(reinterpret_cast<const uint32_t*>(a.pools.vq + (ph * D + dim) * PT + t));
       } else {  // byte row j of a block: low nibble dim j, high nibble dim 16 + j
-        w = *reinterpret_cast<const uint32_t*>(a.pools.vq + ((ph * NB + b) * 16 + dim % 16) * PT + t);
+        w = StreamLoad(reinterpret_cast<const uint32_t*>(a.pools.vq + ((ph * NB + b) * 16 + dim % 16) * PT + t));
         shift = dim % 32 / 16 * 4;
       }
       float v[4];
@@ -540,8 +540,8 @@ __global__ __launch_bounds__(256) void PrefillImagesF16(const ImageArgs a) {
     const int key = p / CPR, c = (p % CPR) ^ (key % 8), kk = tile * kKeys + key;
     uint32_t o[4] = {0u, 0u, 0u, 0u};
     if (kk < n_keys) {
-      const uint4 w = *reinterpret_cast<const uint4*>(a.fk + page_head(kk) * (size_t(D) * PT) +
-                                                      (size_t(c / 2) * PT + kk % PT) * 16 + (c % 2) * 8);
+      const uint4 w = StreamLoad(reinterpret_cast<const uint4*>(a.fk + page_head(kk) * (size_t(D) * PT) +
+                                                                (size_t(c / 2) * PT + kk % PT) * 16 + (c % 2) * 8));
       o[0] = w.x, o[1] = w.y, o[2] = w.z, o[3] = w.w;
     }
     *reinterpret_cast<uint4*>(kimg + size_t(p) * 16) = uint4{o[0], o[1], o[2], o[3]};
@@ -554,8 +554,8 @@ __global__ __launch_bounds__(256) void PrefillImagesF16(const ImageArgs a) {
       // four keys, always within one page
       const int kk = tile * kKeys + (a.wide ? 16 * (c / 2) + 8 * hf + 4 * (c % 2) : 32 * s2 + 16 * hf + 4 * jg);
       constexpr int RUN = PT < 32 ? PT : 32;  // V^T lies in runs of at most 32 keys
-      const uint2 w = *reinterpret_cast<const uint2*>(a.fv + page_head(kk) * (size_t(D) * PT) +
-                                                      (size_t(kk % PT / RUN) * D + dim) * RUN + kk % RUN);
+      const uint2 w = StreamLoad(reinterpret_cast<const uint2*>(a.fv + page_head(kk) * (size_t(D) * PT) +
+                                                                (size_t(kk % PT / RUN) * D + dim) * RUN + kk % RUN));
       uint32_t u[2] = {w.x, w.y};
 #pragma unroll
       for (int e = 0; e < 4; ++e)  // keys at or past the end are zero in the image
