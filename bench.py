@@ -45,10 +45,10 @@ EVENT_EVERY = 4      # decode workloads: HIP events around the split-K kernel on
 NQ, NKV, HD, PT = 24, 4, 256, 64
 # HBM bytes per launch of the split-K kernel from rocprofv3 counters (FETCH_SIZE + WRITE_SIZE, each scaled by what the
 # counter reads for a plain 1 GiB copy); a measurement made outside this script, recorded with its summary.
-TRAFFIC = {"ragged_b64_q8_0": (5.336e9, "profiles/decode_part_q8_0_ragged_b64.md"),
-           "b1_ctx32k_q8_0": (8.72e7, "profiles/decode_part_q8_0_b1_ctx32k.md"),
-           "b16_ctx128k_f16": (8.622e9, "profiles/decode_part_f16_b16_ctx128k.md"),
-           "b16_ctx128k_q4_0": (2.444e9, "profiles/decode_part_q4_0_b16_ctx128k.md"),
+TRAFFIC = {"ragged_b64_q8_0": (5.327e9, "profiles/decode_part_q8_0_ragged_b64.md"),
+           "b1_ctx32k_q8_0": (8.60e7, "profiles/decode_part_q8_0_b1_ctx32k.md"),
+           "b16_ctx128k_f16": (8.619e9, "profiles/decode_part_f16_b16_ctx128k.md"),
+           "b16_ctx128k_q4_0": (2.445e9, "profiles/decode_part_q4_0_b16_ctx128k.md"),
            "prefill_b8_ctx16k_chunk2k_q8_0": (2.150e9, "profiles/prefill_attend_q8_0_b8_ctx16k_chunk2k.md")}
 
 
