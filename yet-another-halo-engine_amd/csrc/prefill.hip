@@ -423,11 +423,14 @@ __global__ __launch_bounds__(256) void PrefillAttendFused(const PrefillArgs a) {
 // 64 keys), the f16 K tile and V^T tile exactly as the attention kernel wants them in LDS, and `PrefillAttendImg`
 // copies images to LDS with direct global-to-LDS loads (no registers, no vector instructions) one tile ahead.
 //
-// K image: 64 rows (keys) of D f16; the 16-byte chunk c of row r sits at chunk position c ^ (r % 8).
+// K image: 64 rows (keys) of D f16; the 16-byte chunk c of row r sits at chunk position c ^ (r % 16).
 // V image: D rows (dims) of 64 f16; chunk c = 4 s2 + jg of row r holds keys 32 s2 + 4 jg + 0..3 and 32 s2 + 16 +
 // 4 jg + 0..3 (the eight k-slots of lane group jg in step s2 of the second product) and sits at position c ^ (r % 8).
-// With the XOR, the sixteen rows a wave reads at once fall into different banks. Keys at or past the end of the
-// sequence are zero in both images.
+// With the XOR, the sixteen rows a wave reads at once (four 16-byte chunks of each) fall into different banks: a K
+// row is a multiple of 256 bytes, the width of the LDS banks, so sixteen rows need sixteen different chunk positions
+// (with c ^ (r % 8), rows r and r + 8 met in the same banks and a wave-wide read took twice as long: 33 against 17
+// cycles, measured with the reads alone); V^T rows are 128 bytes, where eight positions and the rows' own alternation
+// between the two halves of the banks do. Keys at or past the end of the sequence are zero in both images.
 struct ImageArgs {
   Geom g;
   Pools pools;
@@ -465,7 +468,7 @@ __global__ __launch_bounds__(256) void PrefillImages(const ImageArgs a) {
     return size_t(ClampPage(row[min(key / PT, a.stride - 1)], g.n_pages)) * H + h;
   };
   for (int p = tid; p < kKeys * CPR; p += 256) {  // K: chunk = dims 8 c .. 8 c + 7 of one key
-    const int key = p / CPR, c = (p % CPR) ^ (key % 8), kk = tile * kKeys + key;
+    const int key = p / CPR, c = (p % CPR) ^ (key % 16), kk = tile * kKeys + key;
     uint32_t o[4] = {0u, 0u, 0u, 0u};
     if (kk < n_keys) {
       const size_t ph = page_head(kk);
@@ -537,7 +540,7 @@ __global__ __launch_bounds__(256) void PrefillImagesF16(const ImageArgs a) {
     return size_t(ClampPage(row[min(key / PT, a.stride - 1)], g.n_pages)) * H + h;
   };
   for (int p = tid; p < kKeys * CPR; p += 256) {  // K: chunk = dims 8 c .. 8 c + 7 of one key
-    const int key = p / CPR, c = (p % CPR) ^ (key % 8), kk = tile * kKeys + key;
+    const int key = p / CPR, c = (p % CPR) ^ (key % 16), kk = tile * kKeys + key;
     uint32_t o[4] = {0u, 0u, 0u, 0u};
     if (kk < n_keys) {
       const uint4 w = StreamLoad(reinterpret_cast<const uint4*>(a.fk + page_head(kk) * (size_t(D) * PT) +
@@ -654,14 +657,18 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
     __builtin_amdgcn_raw_ptr_buffer_load_lds(img_rsrc, (__attribute__((address_space(3))) void*)dst, 16, lane * 16,
                                              tile * TIMG + c * 1024, 0, 0);
   };
-  // byte offsets of this lane's operand reads within an image; the XOR with qn % 8 undoes the images' swizzle
+  // byte offsets of this lane's operand reads within an image; the XOR undoes the images' swizzle (K rows: chunk ^
+  // (key % 16); V^T rows: chunk ^ (dim % 8)).
   // The chunk index (4 n + jg) ^ (qn % 8) is 4 (n ^ h) + (jg ^ l) with h = qn % 8 / 4 and l = qn % 4: per lane one
   // offset for even n and one for odd n, and everything else is a constant of the instruction.
   const int sw_l = 16 * (jg ^ (qn % 4)), sw_h = 64 * (qn % 8 / 4);
-  const int koff[2] = {qn * (2 * D) + sw_l + sw_h, qn * (2 * D) + sw_l - sw_h};
+  // (K: (4 n + jg) ^ qn is 4 (n ^ qn / 4) + (jg ^ l): one offset per lane for each n % 4)
+  int koff[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) koff[e] = qn * (2 * D) + sw_l + 64 * (e ^ (qn / 4));
   const int voff[2] = {qn * 128 + sw_l + sw_h, qn * 128 + sw_l - sw_h};
   auto read_k = [&](const char* buf, int ks, int kt) -> h8v {
-    return *reinterpret_cast<const h8v*>(buf + koff[ks % 2] + (kt * 16 * (2 * D) + 64 * ks));
+    return *reinterpret_cast<const h8v*>(buf + koff[ks % 4] + (kt * 16 * (2 * D) + 64 * (ks & ~3)));
   };
   // One 32-dim step of S^T = K Q^T: the A operands of step ks + KP are read before the products of step ks.
   auto k_first = [&](const char* buf, h8v (&ka)[KP + 1][4]) {
@@ -998,11 +1005,13 @@ __global__ __launch_bounds__(256) void PrefillAttendPair(const PrefillArgs a, co
   // V^T rows the wave's D / 2 dims, `own` the 32-key step of the wave's own keys and `other` its partner's
   const int sw_l = 16 * (jg ^ (qn % 4)), sw_h = 64 * (qn % 8 / 4);
   const int krow = (32 * b + qn) * (2 * D) + sw_l;
-  const int koff[2] = {krow + sw_h, krow - sw_h};
+  int koff[4];  // K rows are swizzled by key % 16: one offset per lane for each step % 4
+#pragma unroll
+  for (int e = 0; e < 4; ++e) koff[e] = krow + 64 * (e ^ (qn / 4));
   const int vrow = (16 * NDH * b + qn) * 128 + sw_l;
   const int v_own = vrow + 64 * b + (b ? -sw_h : sw_h), v_other = vrow + 64 * (1 - b) + (b ? sw_h : -sw_h);
   auto read_k = [&](const char* buf, int ks, int kt) -> h8v {
-    return *reinterpret_cast<const h8v*>(buf + koff[ks % 2] + (kt * 16 * (2 * D) + 64 * ks));
+    return *reinterpret_cast<const h8v*>(buf + koff[ks % 4] + (kt * 16 * (2 * D) + 64 * (ks & ~3)));
   };
   // One 32-dim step of S^T = K Q^T for the wave's 32 keys: the A operands of the next step are read before the
   // products of this one.
@@ -1317,17 +1326,17 @@ __global__ __launch_bounds__(256) void PrefillAttendWide(const PrefillArgs a, co
                                              tile * TIMG + c * 1024, 0, 0);
   };
   // Operand reads: row = lane % 32 (+ 32 per tile of keys or dims), 16-byte chunk 2 step + half, at the swizzled
-  // position chunk ^ (row % 8). The XOR splits into a per-lane part for each step % 4 and a constant of the instruction.
-  const int x = qn % 8;
-  int koff[4], voff[4];
+  // position chunk ^ (row % 16) in the K image and chunk ^ (row % 8) in the V image. The XOR splits into a per-lane
+  // part for each step % 8 (K) or step % 4 (V) and a constant of the instruction.
+  const int x = qn % 8, xk = qn % 16;
+  int koff[8], voff[4];
 #pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    const int c = 16 * ((h2 ^ (x & 1)) + 2 * (e ^ (x >> 1)));
-    koff[e] = qn * (2 * D) + c, voff[e] = qn * 128 + c;
-  }
+  for (int e = 0; e < 8; ++e) koff[e] = qn * (2 * D) + 16 * ((h2 ^ (xk & 1)) + 2 * (e ^ (xk >> 1)));
+#pragma unroll
+  for (int e = 0; e < 4; ++e) voff[e] = qn * 128 + 16 * ((h2 ^ (x & 1)) + 2 * (e ^ (x >> 1)));
   typedef __attribute__((address_space(3))) const char* LdsPtr;
   auto read_k = [&](const char* buf, int ks, int kt) -> h8v {
-    return *reinterpret_cast<const h8v*>(buf + koff[ks % 4] + (kt * 32 * (2 * D) + 128 * (ks / 4)));
+    return *reinterpret_cast<const h8v*>(buf + koff[ks % 8] + (kt * 32 * (2 * D) + 256 * (ks / 8)));
   };
   // The A operands of step ks + KP are read before the products of step ks: a step is two matrix instructions, 64
   // cycles, and an LDS read takes longer than that to return.
