@@ -46,7 +46,7 @@ __global__ __launch_bounds__(256) void MovePages(Geom g, Pools pools, const int3
     from = in_slot, to = base + bytes * size_t(ClampPage(dst[i], g.n_pages));
   }
   for (size_t o = size_t(threadIdx.x) * 16; o < bytes; o += 256 * 16)
-    *reinterpret_cast<uint4*>(to + o) = *reinterpret_cast<const uint4*>(from + o);
+    *reinterpret_cast<uint4*>(to + o) = StreamLoad(reinterpret_cast<const uint4*>(from + o));  // read once
   if (mode == 1 && i == 0 && which == 0 && threadIdx.x == 0) {
     uint64_t* h = reinterpret_cast<uint64_t*>(slot);
     h[0] = kSlotMagic, h[1] = uint64_t(g.format), h[2] = uint64_t(g.n_kv), h[3] = uint64_t(g.hd);
