@@ -61,7 +61,8 @@ def use_native_build():
     out = os.path.join(tempfile.gettempdir(), f"liboracle_native_{os.getpid()}.so")
     flags = ["-std=c11", "-O3", "-march=native", "-ffp-contract=off", "-fopenmp", "-fPIC", "-shared"]
     try:
-        subprocess.run(["gcc"] + flags + ["-o", out, os.path.join(HERE, "yahkv_oracle.c"), "-lm"], check=True,
+        subprocess.run(["gcc"] + flags + ["-o", out, os.path.join(HERE, "yahkv_oracle.c"),
+                        os.path.join(HERE, "kv8_oracle.c"), "-lm"], check=True,
                        capture_output=True, timeout=120)
     except (OSError, subprocess.SubprocessError):
         lib()
