@@ -61,7 +61,12 @@ typedef enum yahkv_status {
 } yahkv_status;
 
 /* "kv q KB VB" of the reference's decode.txt (loom_decoder.hpp:76-79): K and V share one format here. */
-typedef enum yahkv_format { YAHKV_Q4_0 = 4, YAHKV_Q8_0 = 8, YAHKV_KV_F16 = 16 /* yahkv_f16_* functions only */ } yahkv_format;
+typedef enum yahkv_format {
+  YAHKV_Q4_0 = 4,
+  YAHKV_Q8_0 = 8,
+  YAHKV_KV_F16 = 16,   /* yahkv_f16_* functions only */
+  YAHKV_KV8A16 = 816   /* the reference's own format, "kv q 8 8": yahkv_kv8_* functions only */
+} yahkv_format;
 typedef enum yahkv_dtype { YAHKV_F32 = 0, YAHKV_F16 = 1, YAHKV_BF16 = 2 } yahkv_dtype;
 
 typedef struct yahkv_geometry {
@@ -366,6 +371,101 @@ int yahkv_f16_decode_attend(const yahkv_geometry* g, const yahkv_f16_pools* pool
 size_t yahkv_f16_prefill_workspace_bytes(const yahkv_geometry* g, int32_t n_seqs, int32_t max_prefix_len,
                                          int32_t chunk_len);
 int yahkv_f16_prefill_attend(const yahkv_geometry* g, const yahkv_f16_pools* pools, const int32_t* page_table,
+                             int32_t page_table_stride, const int32_t* prefix_len, int32_t n_seqs,
+                             int32_t max_prefix_len, int32_t chunk_len, const void* q, float softmax_scale,
+                             const float* gate, void* out, int32_t out_dtype, void* workspace,
+                             size_t workspace_bytes, void* stream);
+
+/* ---- kv8a16: the reference's own KV format, byte for byte ------------------------------------------------------------
+ * What the reference runs when decode.txt says "kv q 8 8" (docs/architecture.md:214-230, loom_decoder.hpp:64-87).
+ * geometry.format must be YAHKV_KV8A16, head_dim 256 and page_tokens 256 (gen_decode_attn.py:21-27); W = n_kv_heads *
+ * 256. Buffers, in the reference's own layouts (loom_decoder.hpp:43-51,151-154), rows and tiles of a pool of n_pages pages:
+ *   kq     u32 [n_pages * 256][W / 4]         K codes u = rne((f16(k) - mean) / s) + 128, s = amax / 127 per (token, kv head,
+ *                                             128-dim half); bytes of a dword hold dims (d0, d2, d1, d3) (gen_kvq.py:166-285);
+ *                                             row of position p: table[p / 256] * 256 + p % 256 (gen_kvq.py:48-71)
+ *   ks     u32 [n_pages * 256][W / 128]       f16 pairs (256 s, -384 s), index kv head * 2 + half
+ *   vq     u32 [H][n_pages * 16][256][4]      V codes per channel per 16-key tile around the tile's midrange c with step
+ *                                             s = range / 254, both rounded to f16 first: u = clamp(rne((v - c) / s) + 128,
+ *                                             0, 255); dword w of a (tile, dim) holds keys 4 w + (0, 2, 1, 3)
+ *                                             (gen_kvq.py:474-660); tile of position p: table[p / 256] * 16 + (p / 16) % 16
+ *   vs     u32 [H][n_pages * 16][256]         f16 pairs (256 s, c - 384 s)
+ * and, where the reference's decoder holds one of each for its single sequence (loom_decoder.hpp:43-51: km, vopen), one
+ * per page:
+ *   km     f32 [n_pages][W]                   the channel means of the sequence whose FIRST page this is (yah_kmean,
+ *                                             gen_kvq.py:99-163); zero them for a sequence that starts with decode steps
+ *   vopen  f16 [n_pages][W][16]               the open tile of the sequence whose NEWEST page this is: the keys of the
+ *                                             sequence's last 16-key tile, unquantized (gen_decode_attn.py:436-573)
+ * 2336 bytes per token (kq + ks + vq + vs; architecture.md:219). All buffers 16-byte aligned. */
+typedef struct yahkv_kv8_pools {
+  void* kq;
+  void* ks;
+  void* km;
+  void* vq;
+  void* vs;
+  void* vopen;
+  size_t kq_bytes; /* lengths of the six buffers; shorter than yahkv_kv8_*_bytes(g): YAHKV_ERR_ARG */
+  size_t ks_bytes;
+  size_t km_bytes;
+  size_t vq_bytes;
+  size_t vs_bytes;
+  size_t vopen_bytes;
+} yahkv_kv8_pools;
+/* Replace LoomDecoder::KqBytes/KsBytes/VqBytes/VsBytes at "kv q 8 8" (loom_decoder.hpp:151-154). */
+size_t yahkv_kv8_kq_bytes(const yahkv_geometry* g);
+size_t yahkv_kv8_ks_bytes(const yahkv_geometry* g);
+size_t yahkv_kv8_km_bytes(const yahkv_geometry* g);
+size_t yahkv_kv8_vq_bytes(const yahkv_geometry* g);
+size_t yahkv_kv8_vs_bytes(const yahkv_geometry* g);
+size_t yahkv_kv8_vopen_bytes(const yahkv_geometry* g);
+/* Channel means of each sequence's first chunk: mean over rows 0 .. min(n_rows, max(n_valid[s], 1)) - 1 of k_src
+ * ([n_seqs][n_rows][W] of src_dtype, truncated to f16 first), in yah_kmean's fixed order of f32 sums
+ * (gen_kvq.py:99-163), written to km[table[s][0]]. Call it before the append of a sequence's first chunk, as the
+ * reference does on chunk 0 only (loom_prefill.hpp:3343-3345). n_valid: device int32 [n_seqs] or NULL. */
+int yahkv_kv8_kmean(const yahkv_geometry* g, const yahkv_kv8_pools* pools, const int32_t* page_table,
+                    int32_t page_table_stride, const int32_t* n_valid, int32_t n_seqs, int32_t n_rows,
+                    const void* k_src, int32_t src_dtype, void* stream);
+/* Append n_new tokens per sequence at positions start_pos[s] + i (arguments as yahkv_append; k_src / v_src
+ * [n_seqs][n_new][W]). Positions at or past page_table_stride * 256 are not written; rows at or past n_valid[s] are
+ * not written either (the reference zero-fills its single sequence's padding rows, gen_kvq.py:20; here they may
+ * belong to somebody else).
+ * n_new == 1 replaces yah_dattn_kappend + yah_dattn_vappend (gen_decode_attn.py:1043-1107, 436-573): the K row is
+ *   quantized, V goes to its key of the open tile, and the tile is quantized when that key is its 16th.
+ * n_new >= 2 replaces yah_kq8 + yah_vq8 + yah_vseed (gen_kvq.py:166-285, 474-730): every 16-key tile the chunk
+ *   touches is quantized (keys before the chunk come from the open tile, keys past the last real token repeat it,
+ *   gen_kvq.py:484-486), and the tile of the last real token is left in the open tile, keys past it zero. The
+ *   reference's chunks start on a page boundary; here any start works. */
+int yahkv_kv8_append(const yahkv_geometry* g, const yahkv_kv8_pools* pools, const int32_t* page_table,
+                     int32_t page_table_stride, const int32_t* start_pos, const int32_t* n_valid, int32_t n_seqs,
+                     int32_t n_new, const void* k_src, const void* v_src, int32_t src_dtype, void* stream);
+/* Decode attention (arguments as yahkv_decode_attend): keys 0 .. seq_len[s] - 1, the closed V tiles from codes, the
+ * tile of key seq_len[s] - 1 from the open tile, K - mean from codes (the mean shifts every score of a row alike and
+ * cancels in the softmax, architecture.md:206). Two dispatches: split-K over the closed tiles, then the merge, which
+ * also takes the open tile's keys. Replaces yah_dattn_part_q + yah_dattn_reduce (gen_decode_attn.py:576-1040,
+ * 338-411). Of the options, one_launch is refused. */
+size_t yahkv_kv8_decode_workspace_bytes(const yahkv_geometry* g, int32_t n_seqs, int32_t max_seq_len,
+                                        const yahkv_decode_options* opt);
+int yahkv_kv8_decode_attend(const yahkv_geometry* g, const yahkv_kv8_pools* pools, const int32_t* page_table,
+                            int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs, int32_t max_seq_len,
+                            const void* q, int32_t q_dtype, float softmax_scale, const float* gate, float* out,
+                            void* workspace, size_t workspace_bytes, const yahkv_decode_options* opt, void* stream);
+/* One decode step, LoomDecoder::Step's kappend, vappend, part_q, reduce (loom_decoder.hpp:253-268), in two dispatches
+ * (arguments as yahkv_decode_step): seq_len[s] counts the step's own token, which goes to position seq_len[s] - 1.
+ * The result is that of yahkv_kv8_append(n_new = 1) followed by yahkv_kv8_decode_attend, pools and output. Steps of a
+ * sequence must be contiguous, as the reference demands of its quantized V (loom_decoder.hpp:233-235): the open
+ * tile must hold the keys since the last 16-key boundary. seq_len[s] must not exceed max_seq_len. */
+int yahkv_kv8_decode_step(const yahkv_geometry* g, const yahkv_kv8_pools* pools, const int32_t* page_table,
+                          int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs, int32_t max_seq_len,
+                          const void* k_new, const void* v_new, int32_t new_dtype, const void* q, int32_t q_dtype,
+                          float softmax_scale, const float* gate, float* out, void* workspace, size_t workspace_bytes,
+                          const yahkv_decode_options* opt, void* stream);
+/* Chunked-prefill attention over kv8a16 pools after the chunk has been appended (arguments as yahkv_prefill_attend;
+ * the workspace is required): keys 0 .. prefix_len[s] + chunk_len are decoded once into f16 tiles with the
+ * reference's own decode, one f16 fma f16(1 + u / 256) * S + C' per element, every V tile from codes (yah_kdeq8 /
+ * yah_vdeq8, gen_attn_fa.py:4648-4861), then the attention kernel of yahkv_prefill_attend_tiles runs
+ * (yah_attn_wmma, gen_attn_fa.py:1589-1595). */
+size_t yahkv_kv8_prefill_workspace_bytes(const yahkv_geometry* g, int32_t n_seqs, int32_t max_prefix_len,
+                                         int32_t chunk_len);
+int yahkv_kv8_prefill_attend(const yahkv_geometry* g, const yahkv_kv8_pools* pools, const int32_t* page_table,
                              int32_t page_table_stride, const int32_t* prefix_len, int32_t n_seqs,
                              int32_t max_prefix_len, int32_t chunk_len, const void* q, float softmax_scale,
                              const float* gate, void* out, int32_t out_dtype, void* workspace,

@@ -79,7 +79,7 @@ class HostPools:
         f = np.uint32(fill * 0x01010101)
         self.kq = np.full((P * PT, W // 4), f, np.uint32)
         self.ks = np.full((P * PT, W // 128), f, np.uint32)
-        self.km = np.zeros((P, W), np.float32)
+        self.km = np.full((P, W), f, np.uint32).view(np.float32)
         self.vq = np.full((H, P * 16, HD, 4), f, np.uint32)
         self.vs = np.full((H, P * 16, HD), f, np.uint32)
         self.vo = np.full((P, W, 16), np.uint16(fill * 257), np.uint16)

@@ -9,7 +9,7 @@ import os
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libyahkv.so")
 
-Q8_0, Q4_0, KV_F16 = 8, 4, 16
+Q8_0, Q4_0, KV_F16, KV8A16 = 8, 4, 16, 816
 F32, F16, BF16 = 0, 1, 2
 
 
@@ -30,6 +30,11 @@ class Pools(C.Structure):
 
 class F16PoolsStruct(C.Structure):
     _fields_ = [("k", C.c_void_p), ("v", C.c_void_p), ("k_bytes", C.c_size_t), ("v_bytes", C.c_size_t)]
+
+
+class Kv8PoolsStruct(C.Structure):
+    _NAMES = ("kq", "ks", "km", "vq", "vs", "vopen")
+    _fields_ = [(n, C.c_void_p) for n in _NAMES] + [(n + "_bytes", C.c_size_t) for n in _NAMES]
 
 
 class DecodeOptions(C.Structure):
@@ -95,6 +100,22 @@ def _load():
     lib.yahkv_f16_decode_attend.argtypes = [G, F, i32p, i32, i32p, i32, i32, vp, i32, C.c_float, vp, vp, vp,
                                             C.c_size_t, O, vp]
     lib.yahkv_prefill_decode_tiles.argtypes = [G, P, i32p, i32, i32p, i32, i32, i32, vp, C.c_size_t, vp]
+    K8 = C.POINTER(Kv8PoolsStruct)
+    for n in Kv8PoolsStruct._NAMES:
+        getattr(lib, f"yahkv_kv8_{n}_bytes").restype = C.c_size_t
+        getattr(lib, f"yahkv_kv8_{n}_bytes").argtypes = [G]
+    lib.yahkv_kv8_kmean.argtypes = [G, K8, i32p, i32, i32p, i32, i32, vp, i32, vp]
+    lib.yahkv_kv8_append.argtypes = [G, K8, i32p, i32, i32p, i32p, i32, i32, vp, vp, i32, vp]
+    lib.yahkv_kv8_decode_workspace_bytes.restype = C.c_size_t
+    lib.yahkv_kv8_decode_workspace_bytes.argtypes = [G, i32, i32, O]
+    lib.yahkv_kv8_decode_attend.argtypes = [G, K8, i32p, i32, i32p, i32, i32, vp, i32, C.c_float, vp, vp, vp, C.c_size_t,
+                                            O, vp]
+    lib.yahkv_kv8_prefill_workspace_bytes.restype = C.c_size_t
+    lib.yahkv_kv8_prefill_workspace_bytes.argtypes = [G, i32, i32, i32]
+    lib.yahkv_kv8_prefill_attend.argtypes = [G, K8, i32p, i32, i32p, i32, i32, i32, vp, C.c_float, vp, vp, i32, vp,
+                                             C.c_size_t, vp]
+    lib.yahkv_kv8_decode_step.argtypes = [G, K8, i32p, i32, i32p, i32, i32, vp, vp, i32, vp, i32, C.c_float, vp, vp, vp,
+                                          C.c_size_t, O, vp]
     lib.yahkv_gather_blocks.argtypes = [G, P, i32p, i32, vp, vp, vp]
     lib.yahkv_pagepool_create.restype = C.c_void_p
     lib.yahkv_pagepool_create.argtypes = [i32]
@@ -544,3 +565,121 @@ def gather_blocks(pools, table_row, n_tokens):
     _check(lib.yahkv_gather_blocks(C.byref(g), C.byref(st), _dp(table_row), n_tokens, _dp(k), _dp(v), _stream()),
            "gather_blocks")
     return k, v
+
+
+# ---- kv8a16: the reference's own KV format (yahkv_kv8_*) --------------------------------------------------------------
+
+def kv8_geometry(n_q_heads, n_kv_heads, n_pages):
+    g = Geometry(KV8A16, n_q_heads, n_kv_heads, 256, 256, n_pages)
+    if lib.yahkv_kv8_kq_bytes(C.byref(g)) == 0:
+        raise YahkvError(-2, "kv8a16 geometry")
+    return g
+
+
+class Kv8Pools:
+    """One layer's kv8a16 buffers on the GPU, in the reference's layouts: kq, ks, vq, vs (LoomDecoderState), and per page
+    the channel means (km) and the open V tile (vopen)."""
+
+    NAMES = Kv8PoolsStruct._NAMES
+
+    def __init__(self, g, fill=0, device="cuda:0"):
+        import torch
+        assert g.format == KV8A16
+        self.geom = g
+        for n in self.NAMES:
+            nbytes = getattr(lib, f"yahkv_kv8_{n}_bytes")(C.byref(g))
+            setattr(self, n, torch.full((nbytes,), fill, dtype=torch.uint8, device=device))
+
+    def struct(self):
+        return Kv8PoolsStruct(*[getattr(self, n).data_ptr() for n in self.NAMES],
+                              *[getattr(self, n).numel() for n in self.NAMES])
+
+    def numpy(self):
+        """The buffers as the arrays documented in include/yahkv.h (vopen under the oracle's name `vo`)."""
+        import numpy as np
+        g = self.geom
+        H, P, W = g.n_kv_heads, g.n_pages, g.n_kv_heads * 256
+        raw = {n: getattr(self, n).cpu().numpy() for n in self.NAMES}
+        return {"kq": raw["kq"].view(np.uint32).reshape(P * 256, W // 4), "ks": raw["ks"].view(np.uint32).reshape(P * 256, W // 128),
+                "km": raw["km"].view(np.float32).reshape(P, W), "vq": raw["vq"].view(np.uint32).reshape(H, P * 16, 256, 4),
+                "vs": raw["vs"].view(np.uint32).reshape(H, P * 16, 256), "vo": raw["vopen"].view(np.uint16).reshape(P, W, 16)}
+
+    def load(self, arrays):
+        import numpy as np
+        import torch
+        for n in self.NAMES:
+            a = arrays["vo" if n == "vopen" else n]
+            getattr(self, n).copy_(torch.from_numpy(np.ascontiguousarray(a).view(np.uint8).reshape(-1)))
+
+
+def kv8_kmean(pools, table, k_src, n_valid=None):
+    """Channel means of each sequence's first chunk k_src [n_seqs][n_rows][H][256], written to km of its first page."""
+    g = pools.geom
+    assert k_src.is_contiguous() and table.is_contiguous() and tuple(k_src.shape[2:]) == (g.n_kv_heads, 256)
+    st = pools.struct()
+    _check(lib.yahkv_kv8_kmean(C.byref(g), C.byref(st), _dp(table), table.shape[1], _dp(n_valid), k_src.shape[0],
+                               k_src.shape[1], _dp(k_src), _dtype_code(k_src), _stream()), "kv8_kmean")
+
+
+def kv8_append(pools, table, start_pos, k_src, v_src, n_valid=None):
+    """k_src / v_src: [n_seqs][n_new][H][256]; n_new == 1 is the decoder's append, more the prefill's chunk."""
+    g = pools.geom
+    assert k_src.is_contiguous() and v_src.is_contiguous() and table.is_contiguous() and k_src.dtype == v_src.dtype
+    assert tuple(k_src.shape[2:]) == (g.n_kv_heads, 256) and k_src.shape == v_src.shape
+    st = pools.struct()
+    _check(lib.yahkv_kv8_append(C.byref(g), C.byref(st), _dp(table), table.shape[1], _dp(start_pos), _dp(n_valid),
+                                k_src.shape[0], k_src.shape[1], _dp(k_src), _dp(v_src), _dtype_code(k_src), _stream()),
+           "kv8_append")
+
+
+def _kv8_out_ws(g, q, n_seqs, max_seq_len, out, workspace, opt):
+    import torch
+    assert q.is_contiguous() and tuple(q.shape) == (n_seqs, g.n_q_heads, 256)
+    if out is None:
+        out = torch.empty(q.shape, dtype=torch.float32, device=q.device)
+    if workspace is None:
+        need = lib.yahkv_kv8_decode_workspace_bytes(C.byref(g), n_seqs, max_seq_len, _op(opt))
+        workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=q.device)
+    return out, workspace
+
+
+def kv8_decode_attend(pools, table, seq_len, max_seq_len, q, scale, gate=None, out=None, workspace=None, opt=None):
+    g = pools.geom
+    out, workspace = _kv8_out_ws(g, q, q.shape[0], max_seq_len, out, workspace, opt)
+    st = pools.struct()
+    _check(lib.yahkv_kv8_decode_attend(C.byref(g), C.byref(st), _dp(table), table.shape[1], _dp(seq_len), q.shape[0],
+                                       max_seq_len, _dp(q), _dtype_code(q), scale, _dp(gate), _dp(out), _dp(workspace),
+                                       workspace.numel(), _op(opt), _stream()), "kv8_decode_attend")
+    return out
+
+
+def kv8_decode_step(pools, table, seq_len, max_seq_len, k_new, v_new, q, scale, gate=None, out=None, workspace=None,
+                    opt=None):
+    """seq_len counts the step's token; k_new / v_new [n_seqs][H][256]."""
+    g = pools.geom
+    assert k_new.is_contiguous() and v_new.is_contiguous() and k_new.dtype == v_new.dtype
+    out, workspace = _kv8_out_ws(g, q, q.shape[0], max_seq_len, out, workspace, opt)
+    st = pools.struct()
+    _check(lib.yahkv_kv8_decode_step(C.byref(g), C.byref(st), _dp(table), table.shape[1], _dp(seq_len), q.shape[0],
+                                     max_seq_len, _dp(k_new), _dp(v_new), _dtype_code(k_new), _dp(q), _dtype_code(q),
+                                     scale, _dp(gate), _dp(out), _dp(workspace), workspace.numel(), _op(opt), _stream()),
+           "kv8_decode_step")
+    return out
+
+
+def kv8_prefill_attend(pools, table, prefix_len, max_prefix_len, q, scale, gate=None, out=None, workspace=None):
+    """prefill_attend() over kv8a16 pools; q bf16 [n_seqs][chunk][n_q_heads][256]; returns out (f16 unless given)."""
+    import torch
+    g = pools.geom
+    n_seqs, chunk = q.shape[0], q.shape[1]
+    assert q.is_contiguous() and q.dtype == torch.bfloat16 and tuple(q.shape[2:]) == (g.n_q_heads, 256)
+    if out is None:
+        out = torch.empty(q.shape, dtype=torch.float16, device=q.device)
+    if workspace is None:
+        need = lib.yahkv_kv8_prefill_workspace_bytes(C.byref(g), n_seqs, max_prefix_len, chunk)
+        workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=q.device)
+    st = pools.struct()
+    _check(lib.yahkv_kv8_prefill_attend(C.byref(g), C.byref(st), _dp(table), table.shape[1], _dp(prefix_len), n_seqs,
+                                        max_prefix_len, chunk, _dp(q), scale, _dp(gate), _dp(out), _dtype_code(out),
+                                        _dp(workspace), workspace.numel(), _stream()), "kv8_prefill_attend")
+    return out

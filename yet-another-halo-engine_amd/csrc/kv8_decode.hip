@@ -1,0 +1,587 @@
+// Paged GQA decode attention over kv8a16 pools (the reference's own KV format, see kv8.hpp): split-K over the closed
+// 16-key V tiles, then a merge that also takes the keys of the open tile and, in the step form, appends the step's token.
+//
+// Follows yah_dattn_part_q + yah_dattn_reduce (engine/gpu/loom/tools/gen_decode_attn.py:576-1040, 338-411): K of every
+// key from codes, `(u - 128) * S / 256` per 128-dim half; V of every tile before the newest from codes,
+// `u * (S / 256) + (S + C')`; the newest tile from the open f16 tile; keys at or past the length masked. The cut of the
+// work (stream-K over a line of 64-key tiles, one 8-wave workgroup per CU) is the one of decode.hip, shared through
+// decode_cut.hpp; what differs is what a wave does with a tile:
+//   K rows lie [token][kv head][256 bytes], so the 32 keys a score instruction wants (one key per lane) are 256-byte
+//      pieces 1 KB apart. They are copied to the wave's LDS slot by `buffer_load ... lds` with each row's 256 bytes
+//      across 16 lanes (whole cache lines per wave instruction), 16-byte chunks XOR-swizzled by row so that the
+//      operand reads (lane = key) meet no bank conflicts. Scores run on v_mfma_f32_32x32x16_f16 over the codes with
+//      their f16 constant still on (0x6400 | u = 1024 + u); per 128-dim half and head the constant's share,
+//      1152 * sum(q), comes off the f32 sum before the half's scale goes on, so the products are exact.
+//   V tiles lie [kv head][tile][dim][16 keys]: a lane's 16-byte load is one dim's 16 keys of one tile, which with four
+//      tiles across the four lane groups is the operand shape of v_mfma_f32_16x16x32_f16. Codes become f16
+//      1 + u / 256 by a shift and a mask (what the byte order (k0, k2, k1, k3) is for, gen_kvq.py:480-483) and one
+//      packed f16 fma with the (tile, dim) stats gives the value (the reference's prefill-side decode; its decode side
+//      does the same in f32). P is rounded to f16 as in decode.hip.
+#include <algorithm>
+#include <cstdint>
+
+#include "decode_cut.hpp"
+#include "kv8.hpp"
+#include "quant.hpp"
+
+namespace yahkv {
+namespace {
+
+// ---- the split-K kernel ---------------------------------------------------------------------------------------------
+template <int DUMMY>
+__global__ __launch_bounds__(64 * kWavesPerGroup) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void Kv8Part(const DecodeArgs a, const Kv8Pools pools) {
+  constexpr int D = kKv8Dim, NT = D / 16;
+  constexpr float kLog2e = 1.4426950408889634f, kLn2 = 0.6931471805599453f;
+  const Geom g = a.g;
+  const int G = g.group(), H = g.n_kv;
+  const size_t tiles16 = size_t(g.n_pages) * 16;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64), lane = threadIdx.x % 64;
+  const int n32 = lane % 32, half = lane / 32;
+  const int n16 = lane % 16, kg = lane / 16;
+
+  // Query A-operands [step m of 16][lane half][head row][8 dims]: step m = 2 j + sub covers, in lane half hf, the 8
+  // bytes `sub` of the 16-byte chunk 2 j + hf of a key's row: dims 16 (2 j + hf) + 8 sub + (0, 2, 1, 3, 4, 6, 5, 7).
+  __shared__ __align__(16) _Float16 lq_all[kWavesPerGroup][16][2][8][8];
+  __shared__ __align__(16) float lcorr_all[kWavesPerGroup][2][8];
+  __shared__ __align__(16) _Float16 lp_all[kWavesPerGroup][kMaxGroup][kTile];
+  __shared__ __align__(16) uint8_t lk_all[kWavesPerGroup][32 * 256];  // 32 key rows, chunks swizzled by row
+  __shared__ int next_tile;
+  __shared__ int wave_sum[kWavesPerGroup][2];
+  __shared__ int4 chunk_rec;
+  __shared__ long long chunk_tiles[4];
+  auto& lq = lq_all[wave];
+  auto& lcorr = lcorr_all[wave];
+  auto& lp = lp_all[wave];
+  auto& lk = lk_all[wave];
+
+  if (a.stamps != nullptr && threadIdx.x == 0) a.stamps[blockIdx.x] = wall_clock64();
+  bool any_empty = false;
+  const int4 rec = ChunkRecord<64 * kWavesPerGroup>(a, blockIdx.x, wave_sum, &chunk_rec, chunk_tiles, &any_empty);
+  if (rec.x < 0) return;
+  const int chunk_n = rec.w;
+  if (threadIdx.x == 0) next_tile = 0;
+  __syncthreads();
+  int my_next = wave;
+  auto take = [&]() -> int {
+    if (a.deterministic) {
+      const int v = my_next;
+      my_next += kWavesPerGroup;
+      return v;
+    }
+    int v = 0;
+    if (lane == 0) v = __hip_atomic_fetch_add(&next_tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    return __builtin_amdgcn_readfirstlane(v);
+  };
+
+  uint2 ksc;       // this lane's key: the two halves' scale pairs
+  uint4 vb[NT / 2];  // 16 keys of this lane's dim in this lane group's tile (one half of the dims at a time)
+  uint32_t vst[NT / 2];
+  float m[4], lsum[4], sc[2][4];
+  f4v o[NT];
+  const float qk_scale = a.scale * kLog2e;
+  const int prow = n16 < 4 ? n16 : (n16 >= 8 && n16 < 12 ? n16 - 4 : 0);
+
+  PairCursor cur = FirstPair(a, rec);
+  const int32_t* row = nullptr;
+  typedef const int32_t __attribute__((address_space(4))) * ConstRow;
+  // a 64-key tile lies inside one 256-token page
+  auto load_page = [&](int tile) -> int {
+    const ConstRow crow = (ConstRow)(reinterpret_cast<uintptr_t>(row));
+    return ClampPage(crow[min(tile / 4, a.stride - 1)], g.n_pages);
+  };
+  // K: the 32 rows of half tile tt to the LDS slot, four rows per instruction; lane l of instruction i carries chunk
+  // (l % 16) ^ (row % 16) of row 4 i + l / 16 to LDS position 1024 i + 16 l
+  auto load_k = [&](int tile, int tt, int page) {
+    const size_t row0 = size_t(page) * kKv8Page + (tile % 4) * kTile + 32 * tt;
+    const auto rk = __builtin_amdgcn_make_buffer_rsrc(
+        reinterpret_cast<uint8_t*>(pools.kq) + (row0 * H + cur.h) * 256, 0, 0x7fffffff, 0x00020000);
+    const uint32_t r = lane / 16, c = lane % 16;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const uint32_t rr = 4 * i + r;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, (__attribute__((address_space(3))) void*)(&lk[i * 1024]), 16,
+                                               rr * (H * 256) + ((c ^ (rr & 15)) << 4), 0, 0, kStreamed);
+    }
+    const uint32_t* sp = pools.ks + ((row0 + n32) * H + cur.h) * 2;
+    ksc = StreamLoad(reinterpret_cast<const uint2*>(sp));
+  };
+  auto fetch_v = [&](int tile, int hf, int page) {
+    const size_t pt = size_t(page) * 16 + (tile % 4) * 4 + kg;
+    const uint32_t* vp = pools.vq + ((size_t(cur.h) * tiles16 + pt) * 256 + 128 * hf + n16) * 4;
+    const uint32_t* sp = pools.vs + (size_t(cur.h) * tiles16 + pt) * 256 + 128 * hf + n16;
+#pragma unroll
+    for (int j = 0; j < NT / 2; ++j) vb[j] = StreamLoad(reinterpret_cast<const uint4*>(vp + 64 * j));
+#pragma unroll
+    for (int j = 0; j < NT / 2; ++j) vst[j] = StreamLoad(sp + 16 * j);
+  };
+  // scores of the 32 keys in the LDS slot against all heads: the two 128-dim halves are two accumulator chains
+  auto scores = [&](int tt) {
+    f16v c0 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}, c1 = c0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint4 w0 = *reinterpret_cast<const uint4*>(&lk[n32 * 256 + (((2 * j + half) ^ (n32 & 15)) << 4)]);
+      const uint4 w1 = *reinterpret_cast<const uint4*>(&lk[n32 * 256 + (((2 * (j + 4) + half) ^ (n32 & 15)) << 4)]);
+      const h8v qa0 = *reinterpret_cast<const h8v*>(&lq[2 * j][half][n32 % 8][0]);
+      const h8v qa1 = *reinterpret_cast<const h8v*>(&lq[2 * j + 1][half][n32 % 8][0]);
+      const h8v qb0 = *reinterpret_cast<const h8v*>(&lq[2 * (j + 4)][half][n32 % 8][0]);
+      const h8v qb1 = *reinterpret_cast<const h8v*>(&lq[2 * (j + 4) + 1][half][n32 % 8][0]);
+      const uint4 ka = {__builtin_amdgcn_perm(0x64646464u, w0.x, 0x04010400u), __builtin_amdgcn_perm(0x64646464u, w0.x, 0x04030402u),
+                        __builtin_amdgcn_perm(0x64646464u, w0.y, 0x04010400u), __builtin_amdgcn_perm(0x64646464u, w0.y, 0x04030402u)};
+      const uint4 kb = {__builtin_amdgcn_perm(0x64646464u, w0.z, 0x04010400u), __builtin_amdgcn_perm(0x64646464u, w0.z, 0x04030402u),
+                        __builtin_amdgcn_perm(0x64646464u, w0.w, 0x04010400u), __builtin_amdgcn_perm(0x64646464u, w0.w, 0x04030402u)};
+      const uint4 kc = {__builtin_amdgcn_perm(0x64646464u, w1.x, 0x04010400u), __builtin_amdgcn_perm(0x64646464u, w1.x, 0x04030402u),
+                        __builtin_amdgcn_perm(0x64646464u, w1.y, 0x04010400u), __builtin_amdgcn_perm(0x64646464u, w1.y, 0x04030402u)};
+      const uint4 kd = {__builtin_amdgcn_perm(0x64646464u, w1.z, 0x04010400u), __builtin_amdgcn_perm(0x64646464u, w1.z, 0x04030402u),
+                        __builtin_amdgcn_perm(0x64646464u, w1.w, 0x04010400u), __builtin_amdgcn_perm(0x64646464u, w1.w, 0x04030402u)};
+      c0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(qa0, __builtin_bit_cast(h8v, ka), c0, 0, 0, 0);
+      c1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(qb0, __builtin_bit_cast(h8v, kc), c1, 0, 0, 0);
+      c0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(qa1, __builtin_bit_cast(h8v, kb), c0, 0, 0, 0);
+      c1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(qb1, __builtin_bit_cast(h8v, kd), c1, 0, 0, 0);
+    }
+    const float4 k0 = *reinterpret_cast<const float4*>(&lcorr[0][4 * half]);
+    const float4 k1 = *reinterpret_cast<const float4*>(&lcorr[1][4 * half]);
+    const float kc0[4] = {k0.x, k0.y, k0.z, k0.w}, kc1[4] = {k1.x, k1.y, k1.z, k1.w};
+    const float d0 = WidenF16(static_cast<uint16_t>(ksc.x & 0xFFFF)) * (qk_scale * 0.00390625f);
+    const float d1 = WidenF16(static_cast<uint16_t>(ksc.y & 0xFFFF)) * (qk_scale * 0.00390625f);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) sc[tt][r] = __builtin_fmaf(c1[r] - kc1[r], d1, (c0[r] - kc0[r]) * d0);
+  };
+  // P.V for one half of the dims, from vb, vst and lp; tiles at or past `live16` (the pair's closed tiles) count zero
+  auto pv = [&](int tile, int hf, int live16) {
+    const h8v pa0 = *reinterpret_cast<const h8v*>(&lp[prow][16 * kg]);
+    const h8v pa1 = *reinterpret_cast<const h8v*>(&lp[prow][16 * kg + 8]);
+    const bool dead = tile * 4 + kg >= live16;
+#pragma unroll
+    for (int j = 0; j < NT / 2; ++j) {
+      const uint32_t st = dead ? 0u : vst[j];
+      const h2v sp = __builtin_bit_cast(h2v, st);
+      const h2v S2 = {sp[0], sp[0]}, C2 = {sp[1], sp[1]};
+      const uint32_t w[4] = {vb[j].x, vb[j].y, vb[j].z, vb[j].w};
+      h2v f[8];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        f[2 * i] = __builtin_bit_cast(h2v, ((w[i] << 2) & 0x03fc03fcu) | 0x3c003c00u);      // keys 4 i, 4 i + 1
+        f[2 * i + 1] = __builtin_bit_cast(h2v, ((w[i] >> 6) & 0x03fc03fcu) | 0x3c003c00u);  // keys 4 i + 2, 4 i + 3
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) f[i] = __builtin_elementwise_fma(f[i], S2, C2);
+      const h8v v0 = {f[0][0], f[0][1], f[1][0], f[1][1], f[2][0], f[2][1], f[3][0], f[3][1]};
+      const h8v v1 = {f[4][0], f[4][1], f[5][0], f[5][1], f[6][0], f[6][1], f[7][0], f[7][1]};
+      const int nt = hf * (NT / 2) + j;
+      o[nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa0, v0, o[nt], 0, 0, 0);
+      o[nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa1, v1, o[nt], 0, 0, 0);
+    }
+  };
+  auto leave_empty = [&]() {
+    const size_t part = PartialIndex(a, blockIdx.x, wave, cur) * G;
+    if (lane < G) StoreDevice2(DeviceBuffer(a.ml + part * 2), lane * 8, kNegMax, 0.0f);
+  };
+  auto leave_partial = [&]() {
+    const size_t part = PartialIndex(a, blockIdx.x, wave, cur) * G;
+    const auto rml = DeviceBuffer(a.ml + part * 2), racc = DeviceBuffer(a.acc + part * D);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const float l = HalfSum32(lsum[r]);
+      const int head = 4 * half + r;
+      if (n32 == 0 && head < G) StoreDevice2(rml, head * 8, m[r] * kLn2, l);
+    }
+    if (kg == 0 || kg == 2) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int head = 2 * kg + r;
+        if (head < G) {
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt) StoreDevice(racc, (head * D + 16 * nt + n16) * 4, o[nt][r]);
+        }
+      }
+    }
+  };
+
+  int idx = take();
+  bool worked = false;
+  while (true) {
+    bool more = idx < chunk_n;
+    while (more && idx >= cur.base + cur.n) {
+      if (!worked) leave_empty();
+      worked = false;
+      more = NextPair(a, chunk_n, &cur);
+    }
+    if (!more) break;
+    // ---- first tile of this wave in the pair: query operands, the constants' shares, empty state, first loads
+    row = a.table + int64_t(cur.s) * a.stride;
+    const int live16 = cur.len / 16;  // closed 16-key tiles of the pair (cur.len is a multiple of 16)
+    int tile = cur.first + (idx - cur.base);
+    int pgc = load_page(tile), pgn;
+    load_k(tile, 0, pgc);
+    fetch_v(tile, 1, pgc);  // not used: keeps the count of loads in flight at the loop's head the same on every pass
+    {
+      float hsum[2] = {0.0f, 0.0f};  // per (128-dim half, head row lane % 8): this lane's share
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        // entry i = lane + 64 e: step m = i / 16, lane half hf = (i / 8) % 2, head row rw = i % 8
+        const int i = lane + 64 * e, mm = i / 16, hf = (i / 8) % 2, rw = i % 8;
+        const int d0 = 16 * (2 * (mm / 2) + hf) + 8 * (mm % 2);
+        h8v qv = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (rw < G) qv = LoadQ8(a.q, (size_t(cur.s) * g.n_q + size_t(cur.h) * G + rw) * D + d0, a.q_dtype);
+        float t = 0.0f;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) t += static_cast<float>(qv[k]);
+        hsum[mm / 8] += t;  // e = 0, 1: steps 0-7 (dims 0-127); e = 2, 3: steps 8-15
+        const h8v qs = {qv[0], qv[2], qv[1], qv[3], qv[4], qv[6], qv[5], qv[7]};  // the codes' byte order
+        *reinterpret_cast<h8v*>(&lq[mm][hf][rw][0]) = qs;
+      }
+#pragma unroll
+      for (int hh = 0; hh < 2; ++hh) {
+        float t = hsum[hh] * 1152.0f;
+        t += __shfl_xor(t, 8, 64), t += __shfl_xor(t, 16, 64), t += __shfl_xor(t, 32, 64);
+        if (lane < 8) lcorr[hh][lane] = t;
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) m[r] = kNegMax, lsum[r] = 0.0f;
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) o[nt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
+    worked = true;
+    bool first = true;
+    int ptile = tile;
+    while (true) {
+      const int nidx = take();
+      const bool has_next = nidx < cur.base + cur.n;
+      const int ntile = cur.first + (nidx - cur.base);
+      pgn = load_page(has_next ? ntile : tile);
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      scores(0);
+      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the slot has been read before it is filled again
+      __builtin_amdgcn_sched_barrier(0);
+      load_k(tile, 1, pgc);
+      if (!first) pv(ptile, 1, live16);
+      fetch_v(tile, 0, pgc);
+      first = false;
+      scores(1);
+      __builtin_amdgcn_s_waitcnt(0xC07F);
+      __builtin_amdgcn_sched_barrier(0);
+      load_k(has_next ? ntile : tile, 0, pgn);
+      float alpha[4];
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt) {
+        const bool valid = tile * kTile + 32 * tt + n32 < cur.len;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) sc[tt][r] = valid ? sc[tt][r] : kNegMax;
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float mn = fmaxf(m[r], HalfMax32(fmaxf(sc[0][r], sc[1][r])));
+        alpha[r] = __builtin_amdgcn_exp2f(m[r] - mn);
+        m[r] = mn;
+        const float p0 = __builtin_amdgcn_exp2f(sc[0][r] - mn), p1 = __builtin_amdgcn_exp2f(sc[1][r] - mn);
+        lsum[r] = __builtin_fmaf(lsum[r], alpha[r], p0 + p1);
+        lp[4 * half + r][n32] = static_cast<_Float16>(p0);
+        lp[4 * half + r][32 + n32] = static_cast<_Float16>(p1);
+      }
+      if (__builtin_amdgcn_ballot_w64(alpha[0] != 1.0f || alpha[1] != 1.0f || alpha[2] != 1.0f || alpha[3] != 1.0f) != 0) {
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) o[nt][r] *= alpha[r];
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      pv(tile, 0, live16);
+      fetch_v(tile, 1, pgc);
+      idx = nidx;
+      ptile = tile;
+      if (!has_next) break;
+      tile = ntile;
+      pgc = pgn;
+    }
+    pv(ptile, 1, live16);
+    leave_partial();
+    __builtin_amdgcn_s_waitcnt(0);  // the slot's last copy (issued for a tile that is not coming) has landed
+    __builtin_amdgcn_wave_barrier();
+  }
+  do {
+    if (!worked) leave_empty();
+    worked = false;
+  } while (NextPair(a, chunk_n, &cur));
+  if (a.stamps != nullptr && lane == 0) atomicMax(&a.stamps[a.n_chunks + blockIdx.x], wall_clock64());
+}
+
+// ---- the merge, with the open tile and the step's token -----------------------------------------------------------------
+
+constexpr int kReduceThreads = 256;
+constexpr int kReduceDepth = 4;
+constexpr int kReduceMinDims = 32;
+constexpr int kTail = 17;  // keys the merge adds itself: up to 16 of the open tile, one of them the step's new token
+
+// One workgroup per (query head, sequence, stretch of dims), as DattnReduce of decode.hip, plus the keys the split-K
+// kernel leaves out: those of the sequence's newest 16-key tile, whose K is in the pools as codes and whose V is in the
+// open f16 tile; in the step form the newest of them is the step's own token, which is quantized here with the append
+// kernels' functions, scored from its codes as the reference's part_q would (the K append runs first there,
+// loom_decoder.hpp:254-261), and written to the pools by the workgroup of the group's first query head.
+__global__ __launch_bounds__(kReduceThreads) void Kv8Reduce(const DecodeArgs a, const Kv8Pools pools, const StepRows rows) {
+  const Geom g = a.g;
+  const Kv8Geom kg8{g.n_q, g.n_kv, g.n_pages};
+  constexpr int D = kKv8Dim;
+  const int G = g.group(), H = g.n_kv;
+  const int hq = blockIdx.x, s = blockIdx.y, t = threadIdx.x;
+  const int h = hq / G, gi = hq % G;
+  const int DZ = D >> __builtin_ctz(gridDim.z), d0 = blockIdx.z * DZ;
+  const size_t o = (size_t(s) * g.n_q + hq) * D + d0;
+  const bool step = rows.k != nullptr;
+  const int len = min(max(a.seq_len[s], 0), a.max_len);
+  const int ts = TilesOf(a, s);
+  __shared__ float tail_score[kTail];
+  __shared__ __align__(16) float new_v[D];
+  if (len <= 0) {
+    for (int d = t; d < DZ; d += kReduceThreads) a.out[o + d] = 0.0f;
+    return;
+  }
+  const int closed = (len - 1) & ~15;           // keys the split-K kernel covered
+  const int n_pool = step ? len - 1 : len;      // keys whose rows are in the pools
+  const int n_tail = n_pool - closed;           // of them in the newest tile: 0 .. 16
+  const int32_t* trow = a.table + int64_t(s) * a.stride;
+  const int page = ClampPage(trow[min(closed / kKv8Page, a.stride - 1)], g.n_pages);
+  const int page0 = ClampPage(trow[0], g.n_pages);
+  // ---- scores of the open tile's keys: thread = (key t / 16, 16 dims of the head)
+  {
+    const int j = t / 16, c = t % 16;
+    float part = 0.0f;
+    if (j < n_tail) {
+      const size_t r = size_t(page) * kKv8Page + closed % kKv8Page + j;
+      const uint4 w = *reinterpret_cast<const uint4*>(pools.kq + kg8.kq_row(r, h) + 4 * c);
+      const uint32_t pair = pools.ks[kg8.ks_row(r, h) + c / 8];
+      const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+      const size_t qi = (size_t(s) * g.n_q + hq) * D + 16 * c;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float4 q4 = Load4(a.q, qi + 4 * i, a.q_dtype);
+        const float qe[4] = {static_cast<float>(SaturateToF16(q4.x)), static_cast<float>(SaturateToF16(q4.y)),
+                             static_cast<float>(SaturateToF16(q4.z)), static_cast<float>(SaturateToF16(q4.w))};
+        // byte slots (d0, d2, d1, d3)
+        part += (static_cast<float>(ww[i] & 255u) - 128.0f) * qe[0] + (static_cast<float>((ww[i] >> 16) & 255u) - 128.0f) * qe[1] +
+                (static_cast<float>((ww[i] >> 8) & 255u) - 128.0f) * qe[2] + (static_cast<float>(ww[i] >> 24) - 128.0f) * qe[3];
+      }
+      part *= WidenF16(static_cast<uint16_t>(pair & 0xFFFF)) * 0.00390625f;
+    }
+    part += Dpp<kQuadSwap1>(part);
+    part += Dpp<kQuadSwap2>(part);
+    part += Dpp<kHalfMirror>(part);
+    part += Dpp<kRowMirror>(part);
+    if (c == 0 && j < n_tail) tail_score[j] = part * a.scale;
+  }
+  // ---- the step's token: wave 0 takes its K row, wave 1 its V row (64 lanes x 4 dims = the head)
+  if (step) {
+    const int wave = t / 64, lane = t % 64;
+    const bool writes = gi == 0 && blockIdx.z == 0;
+    const int pos = len - 1;
+    const int wpage = ClampPage(trow[min(pos / kKv8Page, a.stride - 1)], g.n_pages);
+    const size_t src = (size_t(s) * H + h) * D + 4 * lane;
+    if (wave == 0) {
+#pragma clang fp contract(off)
+      const float4 x = Load4(rows.k, src, rows.dtype);
+      const float4 mean = *reinterpret_cast<const float4*>(pools.km + kg8.km_head(page0, h) + 4 * lane);
+      const float4 c = {TruncF16(x.x) - mean.x, TruncF16(x.y) - mean.y, TruncF16(x.z) - mean.z, TruncF16(x.w) - mean.w};
+      float amax = fmaxf(fmaxf(fabsf(c.x), fabsf(c.y)), fmaxf(fabsf(c.z), fabsf(c.w)));
+#pragma unroll
+      for (int off = 16; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+      float inv;
+      uint32_t pair;
+      Kv8ScaleK(amax, &inv, &pair);
+      const uint32_t codes = Kv8CodesK(c, inv);
+      if (writes) {
+        const size_t r = size_t(wpage) * kKv8Page + pos % kKv8Page;
+        pools.kq[kg8.kq_row(r, h) + lane] = codes;
+        if (lane % 32 == 0) pools.ks[kg8.ks_row(r, h) + lane / 32] = pair;
+      }
+      const float4 q4 = Load4(a.q, (size_t(s) * g.n_q + hq) * D + 4 * lane, a.q_dtype);
+      float dot = (static_cast<float>(codes & 255u) - 128.0f) * static_cast<float>(SaturateToF16(q4.x)) +
+                  (static_cast<float>((codes >> 16) & 255u) - 128.0f) * static_cast<float>(SaturateToF16(q4.y)) +
+                  (static_cast<float>((codes >> 8) & 255u) - 128.0f) * static_cast<float>(SaturateToF16(q4.z)) +
+                  (static_cast<float>(codes >> 24) - 128.0f) * static_cast<float>(SaturateToF16(q4.w));
+      dot *= WidenF16(static_cast<uint16_t>(pair & 0xFFFF)) * 0.00390625f;
+      dot = WaveSum(dot);
+      if (lane == 0) tail_score[n_tail] = dot * a.scale;
+    } else if (wave == 1) {
+      const float4 v = Load4(rows.v, src, rows.dtype);
+      const float ve[4] = {v.x, v.y, v.z, v.w};
+      const int key = pos % 16;
+      *reinterpret_cast<float4*>(&new_v[4 * lane]) = float4{TruncF16(v.x), TruncF16(v.y), TruncF16(v.z), TruncF16(v.w)};
+      if (writes) {
+        uint16_t* vo = pools.vo + kg8.vo_head(wpage, h) + size_t(4 * lane) * 16;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) vo[e * 16 + key] = F16Bits(ve[e]);
+        if (key == 15) {  // the tile's 16th key: quantize it into its place (yah_dattn_vappend)
+          const size_t pt = size_t(wpage) * 16 + (pos / 16) % 16;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const uint4 lo = *reinterpret_cast<const uint4*>(vo + e * 16), hi = *reinterpret_cast<const uint4*>(vo + e * 16 + 8);
+            const uint32_t w[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+            float x[16];
+#pragma unroll
+            for (int j = 0; j < 16; ++j) x[j] = WidenF16(static_cast<uint16_t>(w[j / 2] >> (16 * (j % 2))));
+            x[15] = TruncF16(ve[e]);
+            uint4 codes;
+            uint32_t stats;
+            Kv8QuantTile(x, &codes, &stats);
+            *reinterpret_cast<uint4*>(pools.vq + kg8.vq_tile(h, pt) + size_t(4 * lane + e) * 4) = codes;
+            pools.vs[kg8.vs_tile(h, pt) + 4 * lane + e] = stats;
+          }
+        }
+      }
+    }
+  }
+  const int n_extra = n_tail + (step ? 1 : 0);  // 1 .. 17
+  size_t p0 = 0, p1 = 0;
+  if (ts > 0) {
+    const long long A_ = ChunkUnits(a, static_cast<long long>(a.tprefix[a.n_seqs]) * H);
+    const int pair = s * H + h;
+    const long long first =
+        static_cast<long long>(a.tprefix[s]) * H + static_cast<long long>(h) * UnitsOf(a, ts) + a.pair_cost;
+    const int k0 = ChunkOf(a, A_, first), k1 = ChunkOf(a, A_, first + ts - 1);
+    p0 = size_t(k0 + pair) * a.wpc, p1 = size_t(k1 + pair + 1) * a.wpc;
+  }
+  constexpr int NW = kReduceThreads / 64;
+  __shared__ float wgt[kReduceThreads], wl[kReduceThreads];
+  __shared__ int slot[kReduceThreads];
+  __shared__ float red[NW];
+  __shared__ int wave_n[NW];
+  __shared__ __align__(16) float sums[kReduceThreads * 4];
+  __shared__ float lsums[kReduceThreads / (kReduceMinDims / 4)];
+  float M = kNegMax;
+  for (size_t p = p0 + t; p < p1; p += kReduceThreads)
+    if (a.ml[(p * G + gi) * 2 + 1] > 0.0f) M = fmaxf(M, a.ml[(p * G + gi) * 2]);
+  M = WaveMax(M);
+  if (t % 64 == 0) red[t / 64] = M;
+  __syncthreads();  // (also: the tail's scores and the new token's V row are in LDS)
+  M = red[0];
+  for (int w = 1; w < NW; ++w) M = fmaxf(M, red[w]);
+  for (int j = 0; j < n_extra; ++j) M = fmaxf(M, tail_score[j]);
+  const int lg_lanes = __builtin_ctz(static_cast<unsigned>(DZ)) - 2;
+  const int lanes = 1 << lg_lanes, n_groups = kReduceThreads >> lg_lanes, grp = t >> lg_lanes, dl = t & (lanes - 1);
+  float L = 0.0f;
+  float4 A = {0.0f, 0.0f, 0.0f, 0.0f};
+  for (size_t b0 = p0; b0 < p1; b0 += kReduceThreads) {
+    const int nb = static_cast<int>(min(p1 - b0, size_t(kReduceThreads)));
+    float l = 0.0f, mm = 0.0f;
+    if (t < nb) l = a.ml[((b0 + t) * G + gi) * 2 + 1], mm = a.ml[((b0 + t) * G + gi) * 2];
+    const unsigned long long mask = __ballot(l > 0.0f);
+    __syncthreads();
+    if (t % 64 == 0) wave_n[t / 64] = __popcll(mask);
+    __syncthreads();
+    int at = __popcll(mask & ((1ull << (t % 64)) - 1)), n = 0;
+    for (int w = 0; w < NW; ++w) {
+      if (w < t / 64) at += wave_n[w];
+      n += wave_n[w];
+    }
+    if (l > 0.0f) {
+      const float w = __expf(mm - M);
+      wgt[at] = w, wl[at] = w * l, slot[at] = t;
+    }
+    __syncthreads();
+    for (int j0 = grp * kReduceDepth; j0 < n; j0 += n_groups * kReduceDepth) {
+      float4 v[kReduceDepth];
+#pragma unroll
+      for (int j = 0; j < kReduceDepth; ++j)
+        v[j] = *reinterpret_cast<const float4*>(&a.acc[((b0 + slot[min(j0 + j, n - 1)]) * G + gi) * D + d0 + 4 * dl]);
+#pragma unroll
+      for (int j = 0; j < kReduceDepth; ++j) {
+        if (j0 + j < n) {
+          const float w = wgt[j0 + j];
+          A.x = __builtin_fmaf(w, v[j].x, A.x), A.y = __builtin_fmaf(w, v[j].y, A.y);
+          A.z = __builtin_fmaf(w, v[j].z, A.z), A.w = __builtin_fmaf(w, v[j].w, A.w);
+          L += wl[j0 + j];
+        }
+      }
+    }
+  }
+  *reinterpret_cast<float4*>(&sums[grp * DZ + 4 * dl]) = A;
+  if (dl == 0) lsums[grp] = L;
+  __syncthreads();
+  for (int d = t; d < DZ; d += kReduceThreads) {
+    float v = 0.0f, lt = 0.0f;
+    for (int q = 0; q < n_groups; ++q) v += sums[q * DZ + d], lt += lsums[q];
+    // the open tile's keys, as partials of one key each: V from the open f16 tile, the step's token from its source row
+    const uint16_t* vo = pools.vo + kg8.vo_head(page, h) + size_t(d0 + d) * 16;
+    uint32_t w[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (n_tail > 0) {
+      const uint4 lo = *reinterpret_cast<const uint4*>(vo), hi = *reinterpret_cast<const uint4*>(vo + 8);
+      w[0] = lo.x, w[1] = lo.y, w[2] = lo.z, w[3] = lo.w, w[4] = hi.x, w[5] = hi.y, w[6] = hi.z, w[7] = hi.w;
+    }
+    for (int j = 0; j < n_extra; ++j) {
+      const float wj = __expf(tail_score[j] - M);
+      const float x = j < n_tail ? WidenF16(static_cast<uint16_t>(w[j / 2] >> (16 * (j % 2)))) : new_v[d0 + d];
+      v = __builtin_fmaf(wj, x, v), lt += wj;
+    }
+    v /= lt;
+    if (a.gate != nullptr) v *= 1.0f / (1.0f + __expf(-a.gate[o + d]));
+    a.out[o + d] = v;
+  }
+}
+
+int CheckArgs(const yahkv_geometry* g, const yahkv_kv8_pools* pools, const int32_t* page_table, const void* q, int32_t q_dtype,
+              const float* out) {
+  if (const int st = CheckKv8Pools(g, pools)) return st;
+  if (page_table == nullptr || q == nullptr || (reinterpret_cast<uintptr_t>(q) & 15)) return YAHKV_ERR_ARG;
+  if (q_dtype != YAHKV_F32 && q_dtype != YAHKV_F16 && q_dtype != YAHKV_BF16) return YAHKV_ERR_ARG;
+  if (out == nullptr || (reinterpret_cast<uintptr_t>(out) & 15)) return YAHKV_ERR_ARG;
+  return YAHKV_OK;
+}
+
+int Launch(const yahkv_geometry* g, const yahkv_kv8_pools* pools, const int32_t* page_table, int32_t stride,
+           const int32_t* seq_len, int32_t n_seqs, int32_t max_seq_len, const StepRows& rows, const void* q, int32_t q_dtype,
+           float softmax_scale, const float* gate, float* out, void* workspace, size_t workspace_bytes,
+           const yahkv_decode_options* opt, hipStream_t st) {
+  if (const int rc = CheckArgs(g, pools, page_table, q, q_dtype, out)) return rc;
+  if (MakeTuning(opt).one_launch) return YAHKV_ERR_ARG;
+  DecodeArgs a;
+  if (const int rc = Prepare(MakeGeom(*g), stride, seq_len, n_seqs, max_seq_len, workspace, workspace_bytes, opt, &a)) return rc;
+  a.table = page_table, a.q = q, a.q_dtype = q_dtype, a.scale = softmax_scale, a.gate = gate, a.out = out;
+  a.open_tile = 1;
+  const Kv8Pools p = MakeKv8Pools(*pools);
+  hipLaunchKernelGGL(Kv8Part<0>, dim3(static_cast<unsigned>(a.n_chunks)), dim3(64 * kWavesPerGroup), 0, st, a, p);
+  if (const int rc = LaunchStatus()) return rc;
+  int split = 1;
+  while (int64_t(a.g.n_q) * a.n_seqs * split < ComputeUnits() && a.g.hd / (2 * split) >= kReduceMinDims) split *= 2;
+  const int asked = MakeTuning(opt).reduce_split;
+  if (asked > 0) split = std::min(asked, a.g.hd / kReduceMinDims);
+  while (a.g.hd % split != 0 || (a.g.hd / split) % 4 != 0) --split;
+  hipLaunchKernelGGL(Kv8Reduce, dim3(a.g.n_q, a.n_seqs, split), dim3(kReduceThreads), 0, st, a, p, rows);
+  return LaunchStatus();
+}
+
+}  // namespace
+}  // namespace yahkv
+
+using namespace yahkv;
+
+extern "C" size_t yahkv_kv8_decode_workspace_bytes(const yahkv_geometry* g, int32_t n_seqs, int32_t max_seq_len,
+                                                   const yahkv_decode_options* opt) {
+  if (CheckKv8Geometry(g) || n_seqs <= 0 || max_seq_len <= 0) return 0;
+  return MakePlan(MakeGeom(*g), n_seqs, max_seq_len, MakeTuning(opt)).bytes;
+}
+
+extern "C" int yahkv_kv8_decode_attend(const yahkv_geometry* g, const yahkv_kv8_pools* pools, const int32_t* page_table,
+                                       int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs,
+                                       int32_t max_seq_len, const void* q, int32_t q_dtype, float softmax_scale,
+                                       const float* gate, float* out, void* workspace, size_t workspace_bytes,
+                                       const yahkv_decode_options* opt, void* stream) {
+  return Launch(g, pools, page_table, page_table_stride, seq_len, n_seqs, max_seq_len, StepRows{nullptr, nullptr, 0}, q,
+                q_dtype, softmax_scale, gate, out, workspace, workspace_bytes, opt, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int yahkv_kv8_decode_step(const yahkv_geometry* g, const yahkv_kv8_pools* pools, const int32_t* page_table,
+                                     int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs,
+                                     int32_t max_seq_len, const void* k_new, const void* v_new, int32_t new_dtype,
+                                     const void* q, int32_t q_dtype, float softmax_scale, const float* gate, float* out,
+                                     void* workspace, size_t workspace_bytes, const yahkv_decode_options* opt,
+                                     void* stream) {
+  if (k_new == nullptr || v_new == nullptr) return YAHKV_ERR_ARG;
+  if ((reinterpret_cast<uintptr_t>(k_new) | reinterpret_cast<uintptr_t>(v_new)) & 15) return YAHKV_ERR_ARG;
+  if (new_dtype != YAHKV_F32 && new_dtype != YAHKV_F16 && new_dtype != YAHKV_BF16) return YAHKV_ERR_ARG;
+  return Launch(g, pools, page_table, page_table_stride, seq_len, n_seqs, max_seq_len, StepRows{k_new, v_new, new_dtype},
+                q, q_dtype, softmax_scale, gate, out, workspace, workspace_bytes, opt, static_cast<hipStream_t>(stream));
+}

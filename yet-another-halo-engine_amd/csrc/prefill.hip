@@ -21,6 +21,7 @@
 // K / V tile is fetched and decoded once per workgroup and used by all eight blocks (the reference decodes once per
 // layer into an f16 pool for the same reason, :4648-4861).
 #include "common.hpp"
+#include "kv8.hpp"
 
 namespace yahkv {
 namespace {
@@ -440,9 +441,9 @@ struct ImageArgs {
   int32_t n_seqs, max_prefix, chunk_len;
   char* img;
   int32_t tiles_per_pair;
-  int32_t wide;        // V images for the kernel on 32x32x16 matrix instructions (see PrefillAttendWide)
   const uint16_t* fk;  // unquantized f16 pools (PrefillImagesF16 only): K [page][H][D / 16][PT][16], V^T [page][H][PT / R][D][R], R = min(PT, 32)
   const uint16_t* fv;
+  Kv8Pools kv8;        // kv8a16 pools (PrefillImagesKv8 only)
 };
 
 template <int D>
@@ -497,7 +498,7 @@ __global__ __launch_bounds__(256) void PrefillImages(const ImageArgs a) {
 #pragma unroll
     for (int hf = 0; hf < 2; ++hf) {
       // four keys, always within one page
-      const int kk = tile * kKeys + (a.wide ? 16 * (c / 2) + 8 * hf + 4 * (c % 2) : 32 * s2 + 16 * hf + 4 * jg);
+      const int kk = tile * kKeys + 32 * s2 + 16 * hf + 4 * jg;
       const size_t ph = page_head(kk);
       const int t = kk % PT;
       const uint2 sw = *reinterpret_cast<const uint2*>(a.pools.vs + (ph * NB + b) * PT + t);
@@ -555,11 +556,68 @@ __global__ __launch_bounds__(256) void PrefillImagesF16(const ImageArgs a) {
 #pragma unroll
     for (int hf = 0; hf < 2; ++hf) {
       // four keys, always within one page
-      const int kk = tile * kKeys + (a.wide ? 16 * (c / 2) + 8 * hf + 4 * (c % 2) : 32 * s2 + 16 * hf + 4 * jg);
+      const int kk = tile * kKeys + 32 * s2 + 16 * hf + 4 * jg;
       constexpr int RUN = PT < 32 ? PT : 32;  // V^T lies in runs of at most 32 keys
       const uint2 w = StreamLoad(reinterpret_cast<const uint2*>(a.fv + page_head(kk) * (size_t(D) * PT) +
                                                                 (size_t(kk % PT / RUN) * D + dim) * RUN + kk % RUN));
       uint32_t u[2] = {w.x, w.y};
+#pragma unroll
+      for (int e = 0; e < 4; ++e)  // keys at or past the end are zero in the image
+        if (kk + e >= n_keys) u[e / 2] &= e % 2 ? 0x0000FFFFu : 0xFFFF0000u;
+      o[2 * hf] = u[0], o[2 * hf + 1] = u[1];
+    }
+    *reinterpret_cast<uint4*>(vimg + size_t(p) * 16) = uint4{o[0], o[1], o[2], o[3]};
+  }
+}
+
+// The same images from kv8a16 pools (kv8.hpp), decoded as the reference's prefill does it (yah_kdeq8 / yah_vdeq8,
+// gen_attn_fa.py:4648-4861): a code u becomes the f16 1 + u / 256 by a shift and a mask (the byte order (d0, d2, d1, d3)
+// makes the two masks of a dword give the pairs in order), and one f16 fma with the pair (S, C') gives the value:
+// K - mean from (256 s, -384 s) of the row's 128-dim half, V from the (tile, dim) stats; every V tile from its codes.
+__device__ __forceinline__ void Kv8DecodeDword(uint32_t w, uint32_t pair, uint32_t* lo, uint32_t* hi) {
+  typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+  const h2 sp = __builtin_bit_cast(h2, pair);
+  const h2 S = {sp[0], sp[0]}, C = {sp[1], sp[1]};
+  const h2 a = __builtin_bit_cast(h2, ((w << 2) & 0x03fc03fcu) | 0x3c003c00u);  // elements 0, 1 of the dword's four
+  const h2 b = __builtin_bit_cast(h2, ((w >> 6) & 0x03fc03fcu) | 0x3c003c00u);  // elements 2, 3
+  *lo = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(a, S, C));
+  *hi = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(b, S, C));
+}
+template <int DUMMY>
+__global__ __launch_bounds__(256) void PrefillImagesKv8(const ImageArgs a) {
+  constexpr int D = kKv8Dim, PT = kKv8Page, CPR = D / 8;
+  const Geom g = a.g;
+  const Kv8Geom kg{g.n_q, g.n_kv, g.n_pages};
+  const int H = g.n_kv, tile = blockIdx.x, pair = blockIdx.y, s = pair / H, h = pair % H, tid = threadIdx.x;
+  const int n_keys = ClampPrefix(a.prefix_len, s, a.max_prefix, a.stride, PT, a.chunk_len) + a.chunk_len;
+  if (tile * kKeys >= n_keys) return;
+  const int32_t* row = a.table + int64_t(s) * a.stride;
+  char* kimg = a.img + (size_t(pair) * a.tiles_per_pair + tile) * TileImageBytes<D>();
+  char* vimg = kimg + kKeys * D * 2;
+  const int page = ClampPage(row[min(tile * kKeys / PT, a.stride - 1)], g.n_pages);  // a 64-key tile lies in one page
+  for (int p = tid; p < kKeys * CPR; p += 256) {  // K: chunk = dims 8 c .. 8 c + 7 of one key
+    const int key = p / CPR, c = (p % CPR) ^ (key % 16), kk = tile * kKeys + key;
+    uint32_t o[4] = {0u, 0u, 0u, 0u};
+    if (kk < n_keys) {
+      const size_t r = size_t(page) * PT + kk % PT;
+      const uint2 w = StreamLoad(reinterpret_cast<const uint2*>(a.kv8.kq + kg.kq_row(r, h) + 2 * c));
+      const uint32_t sc = a.kv8.ks[kg.ks_row(r, h) + c / 16];
+      Kv8DecodeDword(w.x, sc, &o[0], &o[1]);
+      Kv8DecodeDword(w.y, sc, &o[2], &o[3]);
+    }
+    *reinterpret_cast<uint4*>(kimg + size_t(p) * 16) = uint4{o[0], o[1], o[2], o[3]};
+  }
+  for (int p = tid; p < D * 8; p += 256) {  // V: chunk = 4 + 4 keys of one dim
+    const int dim = p / 8, c = (p % 8) ^ (dim % 8), s2 = c / 4, jg = c % 4;
+    uint32_t o[4];
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf) {
+      const int kk = tile * kKeys + 32 * s2 + 16 * hf + 4 * jg;  // four keys: dword (kk % 16) / 4 of their 16-key tile
+      const size_t pt = size_t(page) * 16 + (kk / 16) % 16;
+      const uint32_t w = StreamLoad(a.kv8.vq + kg.vq_tile(h, pt) + size_t(dim) * 4 + (kk % 16) / 4);
+      const uint32_t st = a.kv8.vs[kg.vs_tile(h, pt) + dim];
+      uint32_t u[2];
+      Kv8DecodeDword(w, st, &u[0], &u[1]);
 #pragma unroll
       for (int e = 0; e < 4; ++e)  // keys at or past the end are zero in the image
         if (kk + e >= n_keys) u[e / 2] &= e % 2 ? 0x0000FFFFu : 0xFFFF0000u;
@@ -894,676 +952,12 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
 }
 
 
-// ---- the same attention with the four waves working as two pairs ---------------------------------------------------
-//
-// In PrefillAttendImg every wave reads the whole K and V tile from LDS for its 32 queries: 1 KB of operand reads per two
-// matrix instructions, 256 KB per tile and workgroup, and with half of those reads left out (wrong results, timing
-// only) that kernel runs 24 % faster. Here a wave holds 64 queries (one head's 64 chunk positions) and a pair of waves
-// shares them: in S^T = K Q^T wave b of the pair takes the tile's keys 32 b .. 32 b + 31 against all 64 queries, in
-// O^T += V^T P^T it takes dims (D / 2) b .. of all 64 keys. Every operand read then feeds four matrix instructions
-// (144 KB of reads per tile and workgroup), and a wave's registers hold 64 queries' B operands (D / 2 registers) and
-// half of their accumulators (D / 2) where the other kernel holds 32 queries' (D / 4) and all of theirs (D / 2).
-// The price: a wave makes the numerators of its own 32 keys only and needs the pair's other 32 for the second
-// product. They go through LDS (4 KB per wave and tile) at the tile's one barrier, which therefore sits between the
-// softmax and the second product; the second product starts with the wave's own half while the other half arrives.
-// Each wave of a pair keeps its own reference point m of the numerators (it sees only its keys' scores); the waves
-// exchange m with the numerators, and where the two differ (the first tile or two of a row) both move to the larger
-// one, which rescales by powers of two as moving m always does.
-// LDS: two K halves, two V halves (a third V half as in the other kernel does not fit beside the numerators), one
-// 16 KB buffer of numerators, and a counter per wave that says which tiles the wave is through with. Before a wave
-// copies V(t + 1) where V(t - 1) was or replaces its numerators of tile t - 1, it looks at the four counters (all
-// waves are through with tile t - 1 as a rule by then; otherwise it waits). Copies: V(t + 1) beside the first
-// product of tile t + 1 (after that look), K(t + 3) beside the second product of tile t, where K(t + 1) was; the wait
-// before the barrier leaves the newest eight (V(t + 1)) in flight.
-// Measured on 8 x (16384 + 2048) tokens, D = 256: 6.9 - 7.0 ms against 6.0 - 6.25 ms of PrefillAttendImg<256, 2> on
-// the same box, so this kernel is built in only with -DYAHKV_PREFILL_PAIRS=1. Its LDS operand reads no longer bound
-// it (half of them left out: no change), but what it adds costs more than they did: the exchange of numerators at the
-// barrier (0.5 ms; matrix pipe idle from the last exponential to the first product after the barrier), the barrier
-// itself in the middle of a tile's work (0.4 ms), 4 more matrix instructions per tile for the denominators that
-// both waves of a pair sum, and the copies, squeezed by the two-buffer schedule (1.1 ms against 0.8 ms there).
-template <int D>
-__global__ __launch_bounds__(256) void PrefillAttendPair(const PrefillArgs a, const char* img, int tiles_per_pair) {
-  constexpr int KS = D / 32, NDH = D / 32, RB = 4, kHeadsPerGroup = 2;  // NDH: 16-dim tiles of a wave's half of the dims
-  constexpr int KIMG = kKeys * D * 2, TIMG = TileImageBytes<D>();
-  constexpr int kCopies = TIMG / 1024 / 4;  // 1 KB wave-wide copies per wave and tile
-  constexpr int VP = 3;                     // the V operand reads run this many 16-dim tiles ahead
-  static_assert(kCopies == 2 * NDH, "one copy per 16-dim tile of each half of the second product");
-  const Geom g = a.g;
-  const int G = g.group(), H = g.n_kv;
-  const int n_qt = (a.chunk_len + kQueries - 1) / kQueries, n_hp = (G + kHeadsPerGroup - 1) / kHeadsPerGroup;
-  const int bid = blockIdx.x, xcd = bid % 8, local = bid / 8, per_pair = n_qt * n_hp;
-  const int pair = xcd + 8 * (local / per_pair), qt = n_qt - 1 - (local % per_pair) / n_hp, hp = local % n_hp;
-  if (pair >= a.n_seqs * H) return;
-  const int s = pair / H, h = pair % H;
-  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / 64), lane = tid % 64;
-  const int b = wave & 1, partner = wave ^ 1;  // the wave's half of the keys / dims; the wave with the other half
-  const int qn = lane % 16, jg = lane / 16;
-  const int prefix = ClampPrefix(a.prefix_len, s, a.max_prefix, a.stride, g.pt, a.chunk_len);
-  const int q0 = qt * kQueries;
-  const int n_keys = min(prefix + q0 + kQueries, prefix + a.chunk_len);
-  const int n_tiles = (n_keys + kKeys - 1) / kKeys;
-
-  // One LDS object on purpose: with several, the compiler tells them apart by alias scopes, and with scopes on the
-  // copies' LDS side it makes every LDS read that follows a copy wait for the copy (vmcnt(0)), which serializes the
-  // kernel; without them it leaves the ordering of copies and reads to the waits written here.
-  constexpr int kPBuf = 4 * KIMG, kMBuf = kPBuf + 4 * RB * 64 * 16, kTaken = kMBuf + 4 * 16 * 16;
-  __shared__ __align__(1024) char lds_all[kTaken + 16];
-  typedef char (*Halves)[KIMG];
-  const Halves lds = reinterpret_cast<Halves>(lds_all);  // [0], [1]: K halves of tile images; [2], [3]: V halves
-  // per wave: its numerators as the second product's B operands
-  typedef uint4 (*PBuf)[RB][64];
-  const PBuf pbuf = reinterpret_cast<PBuf>(lds_all + kPBuf);
-  // per wave and query column: the reference points of its 4 row blocks
-  typedef f4v (*MBuf)[16];
-  const MBuf mbuf = reinterpret_cast<MBuf>(lds_all + kMBuf);
-  // per wave: the tiles it is through with (second product included). Plain accesses: the compiler makes an atomic or
-  // volatile LDS access wait for every copy in flight; the empty asm has the counters read again wherever the read
-  // is written.
-  typedef int i4v __attribute__((ext_vector_type(4)));
-  typedef __attribute__((address_space(3))) i4v* LdsCounters;
-  const LdsCounters through = (LdsCounters)(lds_all + kTaken);
-  auto slowest = [&]() -> int {  // tiles every wave of the workgroup is through with
-    LdsCounters p = through;
-    asm volatile("" : "+v"(p) : : "memory");
-    const i4v t = *p;
-    return min(min(t[0], t[1]), min(t[2], t[3]));
-  };
-
-  h8v qb[RB][KS];
-  int qpos[RB], head[RB];
-#pragma unroll
-  for (int i = 0; i < RB; ++i) {
-    head[i] = kHeadsPerGroup * hp + wave / 2;
-    qpos[i] = q0 + 16 * i + qn;
-    const int t = min(qpos[i], a.chunk_len - 1), hd = min(head[i], G - 1);
-    const uint16_t* qp = a.q + ((size_t(s) * a.chunk_len + t) * g.n_q + size_t(h) * G + hd) * D;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) qb[i][ks] = QueryF16(qp + 32 * ks + 8 * jg);
-  }
-  f4v o[RB][NDH];
-  float m[RB];
-  f4v lacc[RB];
-#pragma unroll
-  for (int i = 0; i < RB; ++i) {
-    m[i] = kNegBig, lacc[i] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-    for (int dt = 0; dt < NDH; ++dt) o[i][dt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
-  }
-  const float sscale = a.scale * 1.4426950408889634f;
-  const auto img_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<char*>(img) + size_t(pair) * tiles_per_pair * TIMG, 0, 0x7fffffff, 0x00020000);
-  // copy j (of kCopies) of this wave's share of the image of `tile` (the last tile's when there is no such tile) into
-  // the buffers of that parity: pieces j < kCopies / 2 are the K half, the others V
-  auto copy_part = [&](int tile, int j) {
-    const int c = wave + 4 * j;
-    char* dst = j < kCopies / 2 ? lds[tile % 2] + c * 1024 : lds[2 + tile % 2] + (c * 1024 - KIMG);
-    tile = min(tile, n_tiles - 1);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(img_rsrc, (__attribute__((address_space(3))) void*)dst, 16, lane * 16,
-                                             tile * TIMG + c * 1024, 0, 0);
-  };
-  // byte offsets of this lane's operand reads within an image (see PrefillAttendImg); K rows are the wave's 32 keys,
-  // V^T rows the wave's D / 2 dims, `own` the 32-key step of the wave's own keys and `other` its partner's
-  const int sw_l = 16 * (jg ^ (qn % 4)), sw_h = 64 * (qn % 8 / 4);
-  const int krow = (32 * b + qn) * (2 * D) + sw_l;
-  int koff[4];  // K rows are swizzled by key % 16: one offset per lane for each step % 4
-#pragma unroll
-  for (int e = 0; e < 4; ++e) koff[e] = krow + 64 * (e ^ (qn / 4));
-  const int vrow = (16 * NDH * b + qn) * 128 + sw_l;
-  const int v_own = vrow + 64 * b + (b ? -sw_h : sw_h), v_other = vrow + 64 * (1 - b) + (b ? sw_h : -sw_h);
-  auto read_k = [&](const char* buf, int ks, int kt) -> h8v {
-    return *reinterpret_cast<const h8v*>(buf + koff[ks % 4] + (kt * 16 * (2 * D) + 64 * (ks & ~3)));
-  };
-  // One 32-dim step of S^T = K Q^T for the wave's 32 keys: the A operands of the next step are read before the
-  // products of this one.
-  auto k_first = [&](const char* buf, h8v (&ka)[2][2]) {
-#pragma unroll
-    for (int kt = 0; kt < 2; ++kt) ka[0][kt] = read_k(buf, 0, kt);
-  };
-  auto k_step = [&](const char* buf, int ks, h8v (&ka)[2][2], f4v (&st)[RB][2]) {
-    if (ks + 1 < KS) {
-#pragma unroll
-      for (int kt = 0; kt < 2; ++kt) ka[(ks + 1) % 2][kt] = read_k(buf, ks + 1, kt);
-    }
-#pragma unroll
-    for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-      for (int i = 0; i < RB; ++i)
-        st[i][kt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[ks % 2][kt], qb[i][ks], st[i][kt], 0, 0, 0);
-  };
-  auto clear = [&](f4v (&st)[RB][2]) {
-#pragma unroll
-    for (int i = 0; i < RB; ++i)
-#pragma unroll
-      for (int kt = 0; kt < 2; ++kt) st[i][kt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
-  };
-  // Largest score of a query over the wave's 32 keys, times the softmax scale; a row whose 32 keys are all masked
-  // gives kNegBig itself, which moves no reference point.
-  auto row_max = [&](auto masked, const f4v (&st)[2]) -> float {
-    float mx = fmaxf(st[0][0], st[0][1]);
-    mx = fmaxf(fmaxf(mx, st[0][2]), st[0][3]);
-    mx = fmaxf(fmaxf(mx, st[1][0]), st[1][1]), mx = fmaxf(fmaxf(mx, st[1][2]), st[1][3]);
-    const float r = MaxOverLaneGroups(mx);
-    return decltype(masked)::value && r == kNegBig ? kNegBig : r * sscale;  // sscale > 0 is required by the entry point
-  };
-  // sums, accumulators of row block i times alpha (a power of two); through a matrix instruction with zero factors,
-  // which keeps them in the accumulation registers (see PrefillAttendImg)
-  auto rescale = [&](int i, float alpha) {
-    const h8v zero = {0, 0, 0, 0, 0, 0, 0, 0};
-    {
-      f4v t = lacc[i];
-      asm volatile("" : "+a"(t));
-#pragma unroll
-      for (int r = 0; r < 4; ++r) t[r] *= alpha;
-      lacc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(zero, zero, t, 0, 0, 0);
-    }
-#pragma unroll
-    for (int dt = 0; dt < NDH; ++dt) {
-      f4v t = o[i][dt];
-      asm volatile("" : "+a"(t));
-#pragma unroll
-      for (int r = 0; r < 4; ++r) t[r] *= alpha;
-      o[i][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(zero, zero, t, 0, 0, 0);
-    }
-  };
-  auto move_reference = [&](int i, float mx) {
-    if (__builtin_expect(__builtin_amdgcn_ballot_w64(mx > m[i] + (kBias + kSlack)) != 0, 0)) {
-      const float mn = mx > m[i] + (kBias + kSlack) ? __builtin_ceilf(mx) - kBias : m[i];
-      const float alpha = __builtin_amdgcn_exp2f(m[i] - mn);
-      m[i] = mn;
-      rescale(i, alpha);
-    }
-  };
-  // f16 numerators of row block i over the wave's 32 keys: the B operand of the 32-key step `b` of the second product
-  auto numerators = [&](auto masked, int i, const f4v (&st)[2]) -> h8v {
-    uint32_t w[4];
-#pragma unroll
-    for (int kt = 0; kt < 2; ++kt) {
-      float p[4];
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        p[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(st[kt][r], sscale, -m[i]));
-        if (decltype(masked)::value && m[i] == kNegBig) p[r] = 0.0f;  // no key of the row seen yet: nothing to weigh
-      }
-      w[2 * kt] = PackF16(p[0], p[1]), w[2 * kt + 1] = PackF16(p[2], p[3]);
-    }
-    return __builtin_bit_cast(h8v, uint4{w[0], w[1], w[2], w[3]});
-  };
-  typedef __attribute__((address_space(3))) const char* LdsPtr;
-  // One 32-key step of O^T += V^T P^T over the wave's dims, and of the denominators; `copy(dt)` issues a tile copy
-  // beside the products of dim tile dt.
-  auto pv_half = [&](LdsPtr vb, const h8v (&p)[RB], auto copy) {
-    asm volatile("" : "+v"(vb));  // (keeps the compiler from folding the lane address into every read's own register)
-    auto read_v = [&](int dt) -> h8v {
-      return *reinterpret_cast<const __attribute__((address_space(3))) h8v*>(vb + dt * 16 * 128);
-    };
-    h8v va[VP + 1];
-#pragma unroll
-    for (int dt = 0; dt < VP; ++dt) va[dt] = read_v(dt);
-#pragma unroll
-    for (int i = 0; i < RB; ++i) lacc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(OnesF16(), p[i], lacc[i], 0, 0, 0);
-#pragma unroll
-    for (int dt = 0; dt < NDH; ++dt) {
-      if (dt + VP < NDH) va[(dt + VP) % (VP + 1)] = read_v(dt + VP);
-#pragma unroll
-      for (int i = 0; i < RB; ++i)
-        o[i][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va[dt % (VP + 1)], p[i], o[i][dt], 0, 0, 0);
-      copy(dt);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-  };
-
-  // One tile: the first product of the next tile beside the softmax of this one, the exchange of numerators at the
-  // barrier, the second product of this tile. `masked`: the tile may hold keys some query must not see, and may be
-  // the last one.
-  f4v st[RB][2];
-  auto tile_step = [&](auto masked, int tile) {
-    constexpr bool MASKED = decltype(masked)::value;
-    constexpr int KA = KS / 4;  // steps of the next tile's first product that run beside the row maxima
-    const bool more = !MASKED || tile + 1 < n_tiles;
-    const char* kbuf = lds[(tile + 1) % 2];
-    f4v sn[RB][2];
-    h8v ka[2][2];
-    float mx[RB];
-    h8v pvo[RB];
-    clear(sn);
-    // Before V(tile + 1) may go where V(tile - 1) was, and before this wave's numerators replace those of the tile
-    // before, every wave must be through with that tile's second product: the waves say so in LDS, and the wait is a
-    // look at the four counters, which as a rule are there by the time the row maxima are done.
-    auto wait_for_all = [&]() {
-      int t = slowest();
-      while (t < tile) {
-        __builtin_amdgcn_s_sleep(1);
-        t = slowest();
-      }
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    };
-    if (MASKED) {
-      if (more) {
-        k_first(kbuf, ka);
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) k_step(kbuf, ks, ka, sn);
-      }
-#pragma unroll
-      for (int i = 0; i < RB; ++i)
-#pragma unroll
-        for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-          for (int r = 0; r < 4; ++r)
-            if (tile * kKeys + 32 * b + 16 * kt + 4 * jg + r > prefix + qpos[i]) st[i][kt][r] = kNegBig;
-#pragma unroll
-      for (int i = 0; i < RB; ++i) move_reference(i, row_max(masked, st[i]));
-      wait_for_all();
-      if (more) {
-#pragma unroll
-        for (int j = kCopies / 2; j < kCopies; ++j) copy_part(tile + 1, j);
-      }
-#pragma unroll
-      for (int i = 0; i < RB; ++i) pvo[i] = numerators(masked, i, st[i]);
-    } else {
-      k_first(kbuf, ka);
-#pragma unroll
-      for (int ks = 0; ks < KA; ++ks) k_step(kbuf, ks, ka, sn);
-#pragma unroll
-      for (int i = 0; i < RB; ++i) mx[i] = row_max(masked, st[i]);
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int i = 0; i < RB; ++i) move_reference(i, mx[i]);
-      wait_for_all();
-      // the rest of the first product with the numerators beside it (the vector units' work between the matrix
-      // instructions) and the copies of V(tile + 1)
-#pragma unroll
-      for (int ks = KA; ks < KS; ++ks) {
-        k_step(kbuf, ks, ka, sn);
-        copy_part(tile + 1, kCopies / 2 + (ks - KA));
-      }
-#pragma unroll
-      for (int i = 0; i < RB; ++i) pvo[i] = numerators(masked, i, st[i]);
-#pragma unroll
-      for (int j = kCopies / 2 + (KS - KA); j < kCopies; ++j) copy_part(tile + 1, j);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int i = 0; i < RB; ++i) pbuf[wave][i][lane] = __builtin_bit_cast(uint4, pvo[i]);
-    mbuf[wave][qn] = f4v{m[0], m[1], m[2], m[3]};  // (the four lane groups of a column write the same values)
-    // The copies complete in the order of their issue: all but the newest kCopies / 2, the pieces of V(tile + 1)
-    // just issued, have landed, this wave's pieces of K(tile + 2) and V(tile) among them; its numerators are written
-    // and its operand reads have returned (lgkmcnt(0)): then the barrier says the same of every wave.
-    // (A bare barrier: __syncthreads() carries a release fence, which waits for every copy in flight. The
-    // wavefront-scope fences emit nothing; they keep the compiler from moving LDS accesses across the barrier.)
-    __builtin_amdgcn_s_waitcnt((MASKED ? VmCnt(0) : VmCnt(kCopies / 2)) & 0xF0FF);
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    const f4v mp = mbuf[partner][qn];
-    h8v pvp[RB];
-#pragma unroll
-    for (int i = 0; i < RB; ++i) pvp[i] = __builtin_bit_cast(h8v, pbuf[partner][i][lane]);
-    LdsPtr vbuf = (LdsPtr)lds[2 + tile % 2];
-    const bool k_copy = !MASKED || tile + 3 < n_tiles;  // K(tile + 3) goes where K(tile + 1) was
-    pv_half(vbuf + v_own, pvo, [&](int dt) {
-      if (dt % 2 == 1 && k_copy) copy_part(tile + 3, dt / 2);
-    });
-    // the pair's two reference points: where they differ, both waves go to the larger one
-    if (__builtin_expect(__builtin_amdgcn_ballot_w64(mp[0] != m[0] || mp[1] != m[1] || mp[2] != m[2] || mp[3] != m[3]) != 0, 0)) {
-#pragma unroll
-      for (int i = 0; i < RB; ++i) {
-        const float mn = fmaxf(m[i], mp[i]);
-        const float alpha = __builtin_amdgcn_exp2f(m[i] - mn), beta = __builtin_amdgcn_exp2f(mp[i] - mn);
-        m[i] = mn;
-        rescale(i, alpha);
-        const _Float16 bh = static_cast<_Float16>(beta);  // a power of two, or zero when it is below f16's range
-#pragma unroll
-        for (int e = 0; e < 8; ++e) pvp[i][e] *= bh;
-      }
-    }
-    pv_half(vbuf + v_other, pvp, [&](int dt) {
-      if (dt % 2 == 1 && k_copy) copy_part(tile + 3, NDH / 2 + dt / 2);
-    });
-    // LDS serves a wave's accesses in order: once the counter is written, this wave's reads of V(tile) and of its
-    // partner's numerators have been served
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    reinterpret_cast<__attribute__((address_space(3))) int*>(through)[wave] = tile + 1;
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    if (more) {
-#pragma unroll
-      for (int i = 0; i < RB; ++i)
-#pragma unroll
-        for (int kt = 0; kt < 2; ++kt) st[i][kt] = sn[i][kt];
-    }
-  };
-
-  // ---- prologue: K(0), K(1), V(0); S^T(0); then K(2) where K(0) was
-  if (tid < 4) reinterpret_cast<__attribute__((address_space(3))) int*>(through)[tid] = 0;
-#pragma unroll
-  for (int j = 0; j < kCopies; ++j) copy_part(0, j);
-#pragma unroll
-  for (int j = 0; j < kCopies / 2; ++j) copy_part(1, j);
-  __builtin_amdgcn_s_waitcnt(VmCnt(0));
-  __syncthreads();
-  clear(st);
-  {
-    h8v ka[2][2];
-    k_first(lds[0], ka);
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      k_step(lds[0], ks, ka, st);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-  }
-  __syncthreads();
-#pragma unroll
-  for (int j = 0; j < kCopies / 2; ++j) copy_part(2, j);
-  const int n_full = min(n_tiles, (prefix + q0 + 1) / kKeys);  // tiles every query of the workgroup sees whole
-  const int n_pipe = min(n_full, n_tiles - 1);
-  int tile = 0;
-  for (; tile < n_pipe; ++tile) tile_step(Constant<false>{}, tile);
-  for (; tile < n_tiles; ++tile) tile_step(Constant<true>{}, tile);
-  StoreRows<D, RB, NDH>(a, s, h, G, jg, o, lacc, qpos, head, 16 * NDH * b);
-}
-
-// ---- the same attention on 32x32x16 matrix instructions ------------------------------------------------------------------
-//
-// v_mfma_f32_32x32x16_f16 does the work of two 16x16x32 instructions in one issue slot and runs 32 cycles in the matrix
-// pipe, which leaves the wave's other instructions (exponentials, conversions, LDS reads, copies) twice the room between
-// two matrix instructions. A wave owns 32 consecutive chunk positions of one head: the queries are the 32 columns of
-// every product.
-//   S^T[key][q]: A = 32 keys x 16 dims from the K image (lane = key, lane half = which 8 dims), B = Q^T in registers;
-//   the result leaves lane (q, half) with keys 8 i + 4 half + j (i, j < 4) of the 32-key tile in register 4 i + j.
-//   O^T[dim][q] += V^T[dim][key] P^T[key][q]: a step takes 16 keys; the lane half's eight k-slots are the keys of two
-//   consecutive i of the scores it already holds, 16 s + 4 half + j and 16 s + 8 + 4 half + j: P never leaves the
-//   registers, and the V image is written in that order (ImageArgs::wide).
-// The K image is the one of the 16x16x32 kernel. Work split, LDS buffers, copies and the schedule are the same.
-// Measured slower than that kernel (see UseWide): both move the same bytes through LDS per tile (every wave reads the
-// whole K and V tile for its 32 queries, 256 KB per tile and workgroup) and spend the same time in the matrix pipe;
-// this one has half as many independent accumulator chains to put between a read and its use.
-typedef float f16v __attribute__((ext_vector_type(16)));
-
-template <int D>
-__global__ __launch_bounds__(256) void PrefillAttendWide(const PrefillArgs a, const char* img, int tiles_per_pair) {
-  constexpr int KS = D / 16, NDT = D / 32, kHeadsPerGroup = 2;
-  constexpr int KIMG = kKeys * D * 2, TIMG = TileImageBytes<D>();
-  constexpr int kCopies = TIMG / 1024 / 4;  // 1 KB wave-wide copies per wave and tile
-  static_assert(kCopies == KS / 2 + NDT, "one copy per two steps of the first product and per dim tile of the second");
-  const Geom g = a.g;
-  const int G = g.group(), H = g.n_kv;
-  const int n_qt = (a.chunk_len + kQueries - 1) / kQueries, n_hp = (G + kHeadsPerGroup - 1) / kHeadsPerGroup;
-  const int bid = blockIdx.x, xcd = bid % 8, local = bid / 8, per_pair = n_qt * n_hp;
-  const int pair = xcd + 8 * (local / per_pair), qt = n_qt - 1 - (local % per_pair) / n_hp, hp = local % n_hp;
-  if (pair >= a.n_seqs * H) return;
-  const int s = pair / H, h = pair % H;
-  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / 64), lane = tid % 64;
-  const int qn = lane % 32, h2 = lane / 32;
-  const int prefix = ClampPrefix(a.prefix_len, s, a.max_prefix, a.stride, g.pt, a.chunk_len);
-  const int q0 = qt * kQueries;
-  const int n_keys = min(prefix + q0 + kQueries, prefix + a.chunk_len);
-  const int n_tiles = (n_keys + kKeys - 1) / kKeys;
-  __shared__ __align__(1024) char lds[5][KIMG];  // [0], [1]: K halves; [2] .. [4]: V halves
-
-  const int head = kHeadsPerGroup * hp + wave / 2;
-  const int qpos = q0 + 32 * (wave % 2) + qn;
-  h8v qb[KS];
-  {
-    const int t = min(qpos, a.chunk_len - 1), hd = min(head, G - 1);
-    const uint16_t* qp = a.q + ((size_t(s) * a.chunk_len + t) * g.n_q + size_t(h) * G + hd) * D;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) qb[ks] = QueryF16(qp + 16 * ks + 8 * h2);
-  }
-  f16v o[NDT], lacc;
-  float m = kNegBig;
-#pragma unroll
-  for (int r = 0; r < 16; ++r) lacc[r] = 0.0f;
-#pragma unroll
-  for (int dt = 0; dt < NDT; ++dt)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) o[dt][r] = 0.0f;
-  const float sscale = a.scale * 1.4426950408889634f;
-  const auto img_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<char*>(img) + size_t(pair) * tiles_per_pair * TIMG, 0, 0x7fffffff, 0x00020000);
-  auto copy_part = [&](int tile, int j) {
-    const int c = wave + 4 * j;
-    char* dst = j < kCopies / 2 ? lds[tile % 2] + c * 1024 : lds[2 + tile % 3] + (c * 1024 - KIMG);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(img_rsrc, (__attribute__((address_space(3))) void*)dst, 16, lane * 16,
-                                             tile * TIMG + c * 1024, 0, 0);
-  };
-  // Operand reads: row = lane % 32 (+ 32 per tile of keys or dims), 16-byte chunk 2 step + half, at the swizzled
-  // position chunk ^ (row % 16) in the K image and chunk ^ (row % 8) in the V image. The XOR splits into a per-lane
-  // part for each step % 8 (K) or step % 4 (V) and a constant of the instruction.
-  const int x = qn % 8, xk = qn % 16;
-  int koff[8], voff[4];
-#pragma unroll
-  for (int e = 0; e < 8; ++e) koff[e] = qn * (2 * D) + 16 * ((h2 ^ (xk & 1)) + 2 * (e ^ (xk >> 1)));
-#pragma unroll
-  for (int e = 0; e < 4; ++e) voff[e] = qn * 128 + 16 * ((h2 ^ (x & 1)) + 2 * (e ^ (x >> 1)));
-  typedef __attribute__((address_space(3))) const char* LdsPtr;
-  auto read_k = [&](const char* buf, int ks, int kt) -> h8v {
-    return *reinterpret_cast<const h8v*>(buf + koff[ks % 8] + (kt * 32 * (2 * D) + 256 * (ks / 8)));
-  };
-  // The A operands of step ks + KP are read before the products of step ks: a step is two matrix instructions, 64
-  // cycles, and an LDS read takes longer than that to return.
-  constexpr int KP = 3;
-  auto k_step = [&](const char* buf, int ks, h8v (&ka)[KP + 1][2], f16v (&st)[2]) {
-    if (ks + KP < KS) {
-#pragma unroll
-      for (int kt = 0; kt < 2; ++kt) ka[(ks + KP) % (KP + 1)][kt] = read_k(buf, ks + KP, kt);
-    }
-#pragma unroll
-    for (int kt = 0; kt < 2; ++kt)
-      st[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka[ks % (KP + 1)][kt], qb[ks], st[kt], 0, 0, 0);
-  };
-  auto k_first = [&](const char* buf, h8v (&ka)[KP + 1][2]) {
-#pragma unroll
-    for (int ks = 0; ks < KP; ++ks)
-#pragma unroll
-      for (int kt = 0; kt < 2; ++kt) ka[ks][kt] = read_k(buf, ks, kt);
-  };
-  auto clear = [&](f16v (&st)[2]) {
-#pragma unroll
-    for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) st[kt][r] = 0.0f;
-  };
-  auto row_max = [&](const f16v (&st)[2]) -> float {  // over the 64 keys of the tile, times the softmax scale
-    float mx = fmaxf(st[0][0], st[0][1]);
-#pragma unroll
-    for (int r = 2; r < 16; r += 2) mx = fmaxf(fmaxf(mx, st[0][r]), st[0][r + 1]);
-#pragma unroll
-    for (int r = 0; r < 16; r += 2) mx = fmaxf(fmaxf(mx, st[1][r]), st[1][r + 1]);
-    const uint32_t u = __builtin_bit_cast(uint32_t, mx);
-    const auto sw = __builtin_amdgcn_permlane32_swap(u, u, false, false);  // the other half's keys
-    const uint32_t s0 = sw[0], s1 = sw[1];
-    return fmaxf(__builtin_bit_cast(float, s0), __builtin_bit_cast(float, s1)) * sscale;
-  };
-  auto move_reference = [&](float mx) {
-    if (__builtin_expect(__builtin_amdgcn_ballot_w64(mx > m + (kBias + kSlack)) != 0, 0)) {
-      const h8v zero = {0, 0, 0, 0, 0, 0, 0, 0};
-      const float mn = mx > m + (kBias + kSlack) ? __builtin_ceilf(mx) - kBias : m;
-      const float alpha = __builtin_amdgcn_exp2f(m - mn);
-      m = mn;
-      {  // (through a matrix instruction with zero factors, so that the accumulators stay where they are: see above)
-        f16v t = lacc;
-        asm volatile("" : "+a"(t));
-#pragma unroll
-        for (int r = 0; r < 16; ++r) t[r] *= alpha;
-        lacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(zero, zero, t, 0, 0, 0);
-      }
-#pragma unroll
-      for (int dt = 0; dt < NDT; ++dt) {
-        f16v t = o[dt];
-        asm volatile("" : "+a"(t));
-#pragma unroll
-        for (int r = 0; r < 16; ++r) t[r] *= alpha;
-        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(zero, zero, t, 0, 0, 0);
-      }
-    }
-  };
-  // f16 numerators as B operands of the second product: step s = 2 kt + u takes registers 8 u .. 8 u + 7 of tile kt
-  auto numerators = [&](const f16v (&st)[2], h8v (&pv)[4]) {
-#pragma unroll
-    for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-      for (int u = 0; u < 2; ++u) {
-        uint32_t w[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(st[kt][8 * u + 2 * e], sscale, -m));
-          const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(st[kt][8 * u + 2 * e + 1], sscale, -m));
-          w[e] = PackF16(p0, p1);
-        }
-        pv[2 * kt + u] = __builtin_bit_cast(h8v, uint4{w[0], w[1], w[2], w[3]});
-      }
-  };
-  auto pv_product = [&](auto always, const char* buf, const h8v (&pv)[4], int v_tile) {
-    LdsPtr vb[4];
-#pragma unroll
-    for (int e = 0; e < 4; ++e) vb[e] = (LdsPtr)buf + voff[e];
-    asm volatile("" : "+v"(vb[0]), "+v"(vb[1]), "+v"(vb[2]), "+v"(vb[3]));
-    auto read_v = [&](int dt, int s_) -> h8v {
-      return *reinterpret_cast<const __attribute__((address_space(3))) h8v*>(vb[s_] + dt * 32 * 128);
-    };
-    constexpr int VA = 2;  // dim tiles the operand reads run ahead
-    h8v va[VA + 1][4];
-#pragma unroll
-    for (int dt = 0; dt < VA; ++dt)
-#pragma unroll
-      for (int s_ = 0; s_ < 4; ++s_) va[dt][s_] = read_v(dt, s_);
-#pragma unroll
-    for (int s_ = 0; s_ < 4; ++s_) lacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(OnesF16(), pv[s_], lacc, 0, 0, 0);
-#pragma unroll
-    for (int dt = 0; dt < NDT; ++dt) {
-      if (dt + VA < NDT) {
-#pragma unroll
-        for (int s_ = 0; s_ < 4; ++s_) va[(dt + VA) % (VA + 1)][s_] = read_v(dt + VA, s_);
-      }
-#pragma unroll
-      for (int s_ = 0; s_ < 4; ++s_)
-        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va[dt % (VA + 1)][s_], pv[s_], o[dt], 0, 0, 0);
-      if (decltype(always)::value || v_tile >= 0) copy_part(v_tile, KS / 2 + dt);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-  };
-
-  const int n_full = min(n_tiles, (prefix + q0 + 1) / kKeys);  // tiles every query of the workgroup sees whole
-  const int n_pipe = min(n_full, n_tiles - 1);
-#pragma unroll
-  for (int j = 0; j < kCopies; ++j) copy_part(0, j);
-#pragma unroll
-  for (int j = 0; j < kCopies; ++j) copy_part(min(1, n_tiles - 1), j);
-  __builtin_amdgcn_s_waitcnt(VmCnt(0));
-  __syncthreads();
-  f16v st[2];
-  clear(st);
-  {
-    h8v ka[KP + 1][2];
-    k_first(lds[0], ka);
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      k_step(lds[0], ks, ka, st);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-  }
-  int tile = 0;
-  constexpr int KA = KS / 4;  // steps of the next tile's first product that run beside the row maximum
-  for (; tile < n_pipe; ++tile) {
-    const char* kbuf = lds[(tile + 1) % 2];
-    const int k_tile = min(tile + 2, n_tiles - 1);
-    f16v sn[2];
-    clear(sn);
-    h8v ka[KP + 1][2];
-    h8v pv[4];
-    k_first(kbuf, ka);
-#pragma unroll
-    for (int ks = 0; ks < KA; ++ks) {
-      k_step(kbuf, ks, ka, sn);
-      if (ks % 2 == 1) copy_part(k_tile, ks / 2);
-    }
-    const float mx = row_max(st);
-    __builtin_amdgcn_sched_barrier(0);
-    move_reference(mx);
-#pragma unroll
-    for (int ks = KA; ks < KS; ++ks) {
-      k_step(kbuf, ks, ka, sn);
-      if (ks % 2 == 1) copy_part(k_tile, ks / 2);
-    }
-    numerators(st, pv);
-    __builtin_amdgcn_sched_barrier(0);
-    pv_product(Constant<true>{}, lds[2 + tile % 3], pv, min(tile + 2, n_tiles - 1));
-#pragma unroll
-    for (int kt = 0; kt < 2; ++kt) st[kt] = sn[kt];
-    __builtin_amdgcn_s_waitcnt(VmCnt(kCopies / 2) & 0xF0FF);
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-  }
-  for (; tile < n_tiles; ++tile) {
-    const bool more = tile + 1 < n_tiles;
-    if ((tile + 1) * kKeys > prefix + q0 + 1) {
-#pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-        for (int r = 0; r < 16; ++r)
-          if (tile * kKeys + 32 * kt + 8 * (r / 4) + 4 * h2 + r % 4 > prefix + qpos) st[kt][r] = kNegBig;
-    }
-    h8v pv[4];
-    move_reference(row_max(st));
-    numerators(st, pv);
-    pv_product(Constant<false>{}, lds[2 + tile % 3], pv, tile + 2 < n_tiles ? tile + 2 : -1);
-    if (more) {
-      const char* kbuf = lds[(tile + 1) % 2];
-      clear(st);
-      h8v ka[KP + 1][2];
-      k_first(kbuf, ka);
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        k_step(kbuf, ks, ka, st);
-        if (tile + 2 < n_tiles && ks % 2 == 1) copy_part(tile + 2, ks / 2);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-    }
-    __builtin_amdgcn_s_waitcnt(VmCnt(0));
-    __syncthreads();
-  }
-  // out = o / l (* sigmoid(gate)): lane (q, half) holds dims 32 dt + 8 i + 4 half + j of its query in register 4 i + j
-  if (head < G && qpos < a.chunk_len) {
-    const float inv = 1.0f / lacc[0];
-    const size_t base = ((size_t(s) * a.chunk_len + qpos) * g.n_q + size_t(h) * G + head) * D;
-#pragma unroll
-    for (int dt = 0; dt < NDT; ++dt)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const size_t e = base + 32 * dt + 8 * i + 4 * h2;
-        float v[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          v[j] = o[dt][4 * i + j] * inv;
-          if (a.gate != nullptr) v[j] *= 1.0f / (1.0f + __expf(-a.gate[e + j]));
-        }
-        if (a.out_dtype == YAHKV_F32) {
-          *reinterpret_cast<float4*>(static_cast<float*>(a.out) + e) = float4{v[0], v[1], v[2], v[3]};
-        } else if (a.out_dtype == YAHKV_BF16) {
-          *reinterpret_cast<uint2*>(static_cast<uint16_t*>(a.out) + e) = uint2{PackBf16(v[0], v[1]), PackBf16(v[2], v[3])};
-        } else {
-          *reinterpret_cast<uint2*>(static_cast<uint16_t*>(a.out) + e) = uint2{PackF16(v[0], v[1]), PackF16(v[2], v[3])};
-        }
-      }
-  }
-}
-
 }  // namespace
 }  // namespace yahkv
 
 using namespace yahkv;
 
 namespace {
-#ifndef YAHKV_PREFILL_WIDE
-#define YAHKV_PREFILL_WIDE 0
-#endif
-#ifndef YAHKV_PREFILL_PAIRS
-#define YAHKV_PREFILL_PAIRS 0
-#endif
-// Which attention kernel serves a geometry, and with it the order of the keys in the V images. The kernel on 32x32x16
-// matrix instructions (head_dim 256 only) is built in with -DYAHKV_PREFILL_WIDE=1; it gives the same results and is
-// measured slower than the one on 16x16x32 (8 x (16384 + 2048) tokens: 6.66 ms against 5.87 ms), so it is off.
-bool UseWide(const Geom& m) { return YAHKV_PREFILL_WIDE && m.hd == 256; }
 int32_t TilesPerPair(int32_t max_prefix_len, int32_t chunk_len) {
   return static_cast<int32_t>((int64_t(max_prefix_len) + chunk_len + kKeys - 1) / kKeys);
 }
@@ -1629,7 +1023,6 @@ extern "C" int yahkv_prefill_decode_tiles(const yahkv_geometry* g, const yahkv_p
   ia.g = m, ia.pools = a.pools, ia.table = page_table, ia.stride = page_table_stride, ia.prefix_len = prefix_len;
   ia.n_seqs = n_seqs, ia.max_prefix = max_prefix_len, ia.chunk_len = chunk_len;
   ia.img = static_cast<char*>(workspace), ia.tiles_per_pair = TilesPerPair(max_prefix_len, chunk_len);
-  ia.wide = UseWide(m);
   const dim3 igrid(static_cast<unsigned>(ia.tiles_per_pair), static_cast<unsigned>(n_seqs * m.n_kv));
   hipStream_t st = static_cast<hipStream_t>(stream);
 #define YAHKV_LAUNCH_IMG(FF, DD, PP) hipLaunchKernelGGL((PrefillImages<FF, DD, PP>), igrid, dim3(256), 0, st, ia)
@@ -1673,9 +1066,7 @@ extern "C" int yahkv_prefill_attend_tiles(const yahkv_geometry* g, const yahkv_p
   // (At head_dim 256 three blocks' accumulators and query operands do not fit the register file: 140 spills.)
 #define YAHKV_LAUNCH_ATT(DD, RR) \
   hipLaunchKernelGGL((PrefillAttendImg<DD, RR>), AttendGrid(a, RR), dim3(256), 0, st, a, img, tiles)
-  if (UseWide(a.g)) hipLaunchKernelGGL((PrefillAttendWide<256>), AttendGrid(a, 2), dim3(256), 0, st, a, img, tiles);
-  else if (a.g.hd == 256 && YAHKV_PREFILL_PAIRS) hipLaunchKernelGGL((PrefillAttendPair<256>), AttendGrid(a, 2), dim3(256), 0, st, a, img, tiles);
-  else if (a.g.hd == 256) YAHKV_LAUNCH_ATT(256, 2);
+  if (a.g.hd == 256) YAHKV_LAUNCH_ATT(256, 2);
   else if (a.g.group() % 3 == 0) YAHKV_LAUNCH_ATT(128, 3);
   else YAHKV_LAUNCH_ATT(128, 2);
 #undef YAHKV_LAUNCH_ATT
@@ -1763,7 +1154,7 @@ extern "C" int yahkv_f16_prefill_attend(const yahkv_geometry* g, const yahkv_f16
   ImageArgs ia{};
   ia.g = a.g, ia.table = page_table, ia.stride = page_table_stride, ia.prefix_len = prefix_len, ia.n_seqs = n_seqs;
   ia.max_prefix = max_prefix_len, ia.chunk_len = chunk_len, ia.img = static_cast<char*>(workspace);
-  ia.tiles_per_pair = tiles, ia.wide = UseWide(a.g);
+  ia.tiles_per_pair = tiles;
   ia.fk = static_cast<const uint16_t*>(pools->k), ia.fv = static_cast<const uint16_t*>(pools->v);
   const dim3 igrid(static_cast<unsigned>(tiles), static_cast<unsigned>(n_seqs * a.g.n_kv));
   hipStream_t st = static_cast<hipStream_t>(stream);
@@ -1779,11 +1170,48 @@ extern "C" int yahkv_f16_prefill_attend(const yahkv_geometry* g, const yahkv_f16
   const char* img = static_cast<const char*>(workspace);
 #define YAHKV_LAUNCH_ATT(DD, RR) \
   hipLaunchKernelGGL((PrefillAttendImg<DD, RR>), AttendGrid(a, RR), dim3(256), 0, st, a, img, tiles)
-  if (UseWide(a.g)) hipLaunchKernelGGL((PrefillAttendWide<256>), AttendGrid(a, 2), dim3(256), 0, st, a, img, tiles);
-  else if (a.g.hd == 256 && YAHKV_PREFILL_PAIRS) hipLaunchKernelGGL((PrefillAttendPair<256>), AttendGrid(a, 2), dim3(256), 0, st, a, img, tiles);
-  else if (a.g.hd == 256) YAHKV_LAUNCH_ATT(256, 2);
+  if (a.g.hd == 256) YAHKV_LAUNCH_ATT(256, 2);
   else if (a.g.group() % 3 == 0) YAHKV_LAUNCH_ATT(128, 3);
   else YAHKV_LAUNCH_ATT(128, 2);
 #undef YAHKV_LAUNCH_ATT
+  return LaunchStatus();
+}
+
+extern "C" size_t yahkv_kv8_prefill_workspace_bytes(const yahkv_geometry* g, int32_t n_seqs, int32_t max_prefix_len,
+                                                    int32_t chunk_len) {
+  if (CheckKv8Geometry(g) || n_seqs <= 0 || max_prefix_len < 0 || chunk_len <= 0) return 0;
+  return ImageBytes(MakeGeom(*g), n_seqs, max_prefix_len, chunk_len);
+}
+
+// Chunked-prefill attention over kv8a16 pools: the keys' f16 tile images are decoded from the pools with the reference's
+// own prefill-side decode, then the same attention kernel as for the other formats runs on them.
+extern "C" int yahkv_kv8_prefill_attend(const yahkv_geometry* g, const yahkv_kv8_pools* pools,
+                                        const int32_t* page_table, int32_t page_table_stride,
+                                        const int32_t* prefix_len, int32_t n_seqs, int32_t max_prefix_len,
+                                        int32_t chunk_len, const void* q, float softmax_scale, const float* gate,
+                                        void* out, int32_t out_dtype, void* workspace, size_t workspace_bytes,
+                                        void* stream) {
+  if (const int rc = CheckKv8Pools(g, pools)) return rc;
+  if (page_table == nullptr || prefix_len == nullptr) return YAHKV_ERR_ARG;
+  if (n_seqs <= 0 || chunk_len <= 0 || max_prefix_len < 0 || page_table_stride <= 0) return YAHKV_ERR_ARG;
+  PrefillArgs a{};
+  a.g = MakeGeom(*g);
+  if (int64_t(page_table_stride) * a.g.pt < chunk_len) return YAHKV_ERR_ARG;
+  a.table = page_table, a.stride = page_table_stride, a.prefix_len = prefix_len, a.n_seqs = n_seqs;
+  a.max_prefix = max_prefix_len, a.chunk_len = chunk_len;
+  if (const int rc = PrepareQueries(q, softmax_scale, gate, out, out_dtype, &a)) return rc;
+  const int tiles = TilesPerPair(max_prefix_len, chunk_len);
+  if (int64_t(tiles) * (2 * kKeys * a.g.hd * 2) > 0x7fffffffLL) return YAHKV_ERR_SHAPE;
+  if (const int rc = CheckWorkspace(a, workspace, workspace_bytes)) return rc;
+  ImageArgs ia{};
+  ia.g = a.g, ia.table = page_table, ia.stride = page_table_stride, ia.prefix_len = prefix_len, ia.n_seqs = n_seqs;
+  ia.max_prefix = max_prefix_len, ia.chunk_len = chunk_len, ia.img = static_cast<char*>(workspace);
+  ia.tiles_per_pair = tiles, ia.kv8 = MakeKv8Pools(*pools);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  hipLaunchKernelGGL(PrefillImagesKv8<0>, dim3(static_cast<unsigned>(tiles), static_cast<unsigned>(n_seqs * a.g.n_kv)),
+                     dim3(256), 0, st, ia);
+  if (const int rc = LaunchStatus()) return rc;
+  hipLaunchKernelGGL((PrefillAttendImg<256, 2>), AttendGrid(a, 2), dim3(256), 0, st, a,
+                     static_cast<const char*>(workspace), tiles);
   return LaunchStatus();
 }
