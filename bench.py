@@ -39,6 +39,9 @@ WORKLOADS = {
     "b16_ctx128k_f16": dict(fmt=16, batch=16, lo=131072, hi=131072, seed=4),
     "ragged_b64_f16": dict(fmt=16, batch=64, lo=1024, hi=65536, seed=4),
     "prefill_b8_ctx16k_chunk2k_f16": dict(fmt=16, batch=8, lo=16384, hi=16384, seed=4, chunk=2048, warmup=10),
+    # the reference's own KV format (kv8a16: 2336 B per token, 256-token pages), the same ragged batch
+    "ragged_b64_kv8a16": dict(fmt=816, batch=64, lo=1024, hi=65536, seed=4),
+    "b1_ctx32k_kv8a16": dict(fmt=816, batch=1, lo=32768, hi=32768, seed=4, layers=8),
 }
 MFMA_F16_PEAK_TFLOPS = 2500.0
 EVENT_EVERY = 4      # decode workloads: HIP events around the split-K kernel on every fourth timed step
@@ -142,6 +145,17 @@ def clock_trace(yahkv, torch, launch, n=60, idle_s=3.0):
                            "kernel_ms_beside_the_probe": round(total / n_load, 4), "launches": n_load,
                            "note": "probes of 0.5 ms on a second stream while the launches run; second half of them"}
     return trace
+
+
+def closed_form_err(Kd, Vd, qs, scale, got):
+    """max |got - want| / max |want| of one sequence against softmax(q K^T scale) V in float64 (Kd, Vd [n][H][D])."""
+    Kd, Vd, qs = Kd.astype(np.float64), Vd.astype(np.float64), qs.astype(np.float64)
+    want = np.zeros((NQ, HD))
+    for h in range(NQ):
+        sc = Kd[:, h // (NQ // NKV)] @ qs[h] * scale
+        p = np.exp(sc - sc.max())
+        want[h] = (p / p.sum()) @ Vd[:, h // (NQ // NKV)]
+    return float(np.abs(got - want).max() / np.abs(want).max())
 
 
 def parity_check(yahkv, torch, g, pools, t_table, lens, q, out, scale, rows):
@@ -360,6 +374,105 @@ def run_f16(a, wl, torch, yahkv):
                      "frac": round(kgbs / HBM_PEAK_GBS, 4), "traffic": TRAFFIC.get(a.workload, (None, None))[0],
                      "traffic_source": TRAFFIC.get(a.workload, (None, None))[1],
                      "kernel": "PartF16<%d, %d> + ReduceF16" % (HD, PT), "kernel_ms": round(kern_ms, 4)},
+        "cpu_baseline": None}
+
+
+def run_kv8(a, wl, torch, yahkv):
+    """A step on kv8a16 pools (the reference's own format): one new token per sequence and the attention over the
+    sequence with it, LoomDecoder::Step's kappend, vappend, part_q, reduce (loom_decoder.hpp:253-268) in two dispatches:
+    split-K partials over the closed 16-key tiles, then the merge, which takes the open tile's keys, quantizes the new
+    token's K row, puts its V row into the open tile and closes the tile on its 16th key."""
+    rng = np.random.default_rng(wl["seed"])
+    B, PG = wl["batch"], 256
+    lens = rng.integers(wl["lo"], wl["hi"] + 1, B).astype(np.int32)
+    total = a.warmup + a.steps + 1
+    pages = (lens + total + PG - 1) // PG
+    n_layers = wl.get("layers", 1)
+    n_pages = int(pages.sum())                       # the pool fits the job exactly
+    g = yahkv.kv8_geometry(NQ, NKV, n_pages)
+    alloc = yahkv.PagePool(n_pages)
+    alloc.shuffle(12345)
+    table = np.zeros((B, int(pages.max())), np.int32)
+    for s, n in enumerate(pages):
+        table[s, :n] = alloc.alloc(int(n))
+    assert alloc.free_count == 0
+    layers = [yahkv.Kv8Pools(g) for _ in range(n_layers)]
+    t_table = torch.from_numpy(table).cuda()
+    gen = torch.Generator(device="cuda").manual_seed(wl["seed"])
+    for pools in layers:                             # the prefix through the library's own kmean + chunk append
+        for s in range(B):
+            for o in range(0, int(lens[s]), 8192):
+                n = min(8192, int(lens[s]) - o)
+                k = (torch.randn((1, n, NKV, HD), generator=gen, device="cuda") + 0.5).to(torch.bfloat16)
+                v = torch.randn((1, n, NKV, HD), generator=gen, device="cuda").to(torch.bfloat16)
+                if o == 0:
+                    yahkv.kv8_kmean(pools, t_table[s:s + 1], k)
+                yahkv.kv8_append(pools, t_table[s:s + 1], torch.tensor([o], dtype=torch.int32, device="cuda"), k, v)
+    scale = 1.0 / float(np.sqrt(HD))
+    max_len = int(lens.max()) + total
+    len_rows = torch.from_numpy(lens[None, :] + np.arange(total + 1, dtype=np.int32)[:, None]).cuda()
+    q = torch.randn((B, NQ, HD), generator=gen, device="cuda").to(torch.bfloat16)
+    knew = torch.randn((total, B, NKV, HD), generator=gen, device="cuda").to(torch.bfloat16)
+    vnew = torch.randn((total, B, NKV, HD), generator=gen, device="cuda").to(torch.bfloat16)
+    out = torch.empty((B, NQ, HD), dtype=torch.float32, device="cuda")
+    opt = yahkv.decode_options(deterministic=a.deterministic, min_chunk_tiles=a.min_chunk_tiles)
+    ws = torch.empty(yahkv.lib.yahkv_kv8_decode_workspace_bytes(g, B, max_len, opt), dtype=torch.uint8, device="cuda")
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(a.steps)]
+
+    def step(i, pair=None):
+        pools = layers[i % n_layers]
+        seq_len = len_rows[i + 1]
+        if pair:
+            pair[0].record()
+        yahkv.kv8_decode_part(pools, t_table, seq_len, max_len, q, scale, ws, opt=opt)
+        if pair:
+            pair[1].record()
+        yahkv.kv8_decode_reduce(pools, t_table, seq_len, max_len, q, scale, out, ws, knew[i], vnew[i], opt=opt)
+
+    # parity before timing: the first step's output of the shortest, the median and the longest sequence against the
+    # float64 closed form over the oracle's dequantized model of those sequences' pages
+    step(0)
+    torch.cuda.synchronize()
+    first_hash = fnv1a(out.cpu().numpy().tobytes())
+    from oracle import kv8 as okv8
+    order = np.argsort(lens)
+    rows = sorted({int(order[0]), int(order[len(order) // 2]), int(order[-1])})
+    err = 0.0
+    for s in rows:
+        n = int(lens[s]) + 1
+        hp, row = okv8.pools_of_sequence(layers[0], table[s], n)
+        Kd, Vd = okv8.dense(hp, row, n)
+        err = max(err, closed_form_err(Kd, Vd, q[s].float().cpu().numpy(), scale, out[s].cpu().numpy()))
+    if not err < 2e-3:
+        raise SystemExit(f"bench.py: parity check failed before timing: max relative error {err:.3e}")
+    for i in range(a.warmup):
+        step(1 + i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(a.steps):
+        step(1 + a.warmup + i, ev[i] if i % EVENT_EVERY == 0 else None)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / a.steps * 1e3
+    kern_ms = float(np.mean([p[0].elapsed_time(p[1]) for p in ev[::EVENT_EVERY]]))
+    bpt = 2336                                           # kq 1024 + ks 32 + vq 1024 + vs 256 (architecture.md:219)
+    tokens = [int(lens.sum()) + B * (2 + a.warmup + i) for i in range(a.steps)]
+    kv_bytes = float(np.mean(tokens)) * bpt
+    gbs, kgbs = kv_bytes / (ms * 1e-3) / 1e9, kv_bytes / (kern_ms * 1e-3) / 1e9
+    return {
+        "metric": "paged kv8a16 KV decode-attn HBM GB/s (% of peak) + tok/s", "value": round(gbs, 1), "unit": "GB/s",
+        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+        "config": {"workload": a.workload, "batch": B, "ctx_min": int(lens.min()), "ctx_max": int(lens.max()),
+                   "ctx_sum": int(lens.sum()), "n_q_heads": NQ, "n_kv_heads": NKV, "head_dim": HD, "page_tokens": PG,
+                   "n_pages": n_pages, "layers_rotated": n_layers, "kv_format": "kv8a16",
+                   "step": "append 1 token/seq + paged decode attention (part, reduce with the open tile and the append in it)"},
+        "pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2), "tok_per_s": round(B / (ms * 1e-3), 1),
+        "kv_bytes_per_step": int(kv_bytes), "parity_max_rel_err": float(f"{err:.3e}"), "parity_rows": rows,
+        "out_fnv1a": first_hash,
+        "roofline": {"bound": "hbm", "achieved": round(kgbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(kgbs / HBM_PEAK_GBS, 4), "traffic": TRAFFIC.get(a.workload, (None, None))[0],
+                     "traffic_source": TRAFFIC.get(a.workload, (None, None))[1],
+                     "kernel": "Kv8Part", "kernel_ms": round(kern_ms, 4)},
         "cpu_baseline": None}
 
 
@@ -706,6 +819,8 @@ def run_workload(a, torch, yahkv):
         return run_prefill(a, wl, torch, yahkv)
     if wl["fmt"] == 16:
         return run_f16(a, wl, torch, yahkv)
+    if wl["fmt"] == 816:
+        return run_kv8(a, wl, torch, yahkv)
     return run_decode(a, wl, torch, yahkv)
 
 

@@ -448,6 +448,19 @@ int yahkv_kv8_decode_attend(const yahkv_geometry* g, const yahkv_kv8_pools* pool
                             int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs, int32_t max_seq_len,
                             const void* q, int32_t q_dtype, float softmax_scale, const float* gate, float* out,
                             void* workspace, size_t workspace_bytes, const yahkv_decode_options* opt, void* stream);
+/* The two dispatches of yahkv_kv8_decode_attend and yahkv_kv8_decode_step on their own, as LoomDecoder::Step issues
+ * its own (loom_decoder.hpp:259-268); both take the same lengths (whether or not they count a token still to be
+ * appended, the split-K dispatch covers the 16-key tiles that are closed once it is). With k_new / v_new the merge is
+ * the step's (it appends that token and attends to it), with both NULL the plain one. */
+int yahkv_kv8_decode_part(const yahkv_geometry* g, const yahkv_kv8_pools* pools, const int32_t* page_table,
+                          int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs, int32_t max_seq_len,
+                          const void* q, int32_t q_dtype, float softmax_scale, void* workspace, size_t workspace_bytes,
+                          const yahkv_decode_options* opt, void* stream);
+int yahkv_kv8_decode_reduce(const yahkv_geometry* g, const yahkv_kv8_pools* pools, const int32_t* page_table,
+                            int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs, int32_t max_seq_len,
+                            const void* k_new, const void* v_new, int32_t new_dtype, const void* q, int32_t q_dtype,
+                            float softmax_scale, const float* gate, float* out, void* workspace,
+                            size_t workspace_bytes, const yahkv_decode_options* opt, void* stream);
 /* One decode step, LoomDecoder::Step's kappend, vappend, part_q, reduce (loom_decoder.hpp:253-268), in two dispatches
  * (arguments as yahkv_decode_step): seq_len[s] counts the step's own token, which goes to position seq_len[s] - 1.
  * The result is that of yahkv_kv8_append(n_new = 1) followed by yahkv_kv8_decode_attend, pools and output. Steps of a

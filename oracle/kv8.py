@@ -111,3 +111,24 @@ def dense(pools, table_row, n_tokens, as_f16=False):
     fn = lib().orc_kv8_dense_f16 if as_f16 else lib().orc_kv8_dense
     fn(C.byref(g), C.byref(st), _ptr(row), C.c_int32(n_tokens), _ptr(Kd), _ptr(Vd))
     return Kd.reshape(n_tokens, g.n_kv_heads, HD), Vd.reshape(n_tokens, g.n_kv_heads, HD)
+
+
+def pools_of_sequence(dev, table_row, n_tokens):
+    """The pages of one sequence, copied from device pools (an object with uint8 torch tensors kq, ks, km, vq, vs, vopen
+    and a geometry) into host pools of their own, numbered in logical order: (HostPools, identity table row)."""
+    g = dev.geom
+    H, W = g.n_kv_heads, g.n_kv_heads * HD
+    n_pg = max((n_tokens + PT - 1) // PT, 1)
+    import torch
+    pg = torch.as_tensor(np.asarray(table_row[:n_pg], np.int64), device=dev.kq.device)
+    hp = HostPools(geometry(g.n_q_heads, H, n_pg))
+    tiles = g.n_pages * 16
+    take = lambda t, shape: t.view(*shape)
+    hp.kq[:] = take(dev.kq, (g.n_pages, PT * W))[pg].cpu().numpy().view(np.uint32).reshape(n_pg * PT, W // 4)
+    hp.ks[:] = take(dev.ks, (g.n_pages, PT * (W // 128) * 4))[pg].cpu().numpy().view(np.uint32).reshape(n_pg * PT, W // 128)
+    hp.km[:] = take(dev.km, (g.n_pages, W * 4))[pg].cpu().numpy().view(np.float32).reshape(n_pg, W)
+    hp.vq[:] = take(dev.vq, (H, g.n_pages, 16 * HD * 16))[:, pg].cpu().numpy().view(np.uint32).reshape(H, n_pg * 16, HD, 4)
+    hp.vs[:] = take(dev.vs, (H, g.n_pages, 16 * HD * 4))[:, pg].cpu().numpy().view(np.uint32).reshape(H, n_pg * 16, HD)
+    hp.vo[:] = take(dev.vopen, (g.n_pages, W * 16 * 2))[pg].cpu().numpy().view(np.uint16).reshape(n_pg, W, 16)
+    del tiles
+    return hp, np.arange(n_pg, dtype=np.int32)

@@ -110,6 +110,9 @@ def _load():
     lib.yahkv_kv8_decode_workspace_bytes.argtypes = [G, i32, i32, O]
     lib.yahkv_kv8_decode_attend.argtypes = [G, K8, i32p, i32, i32p, i32, i32, vp, i32, C.c_float, vp, vp, vp, C.c_size_t,
                                             O, vp]
+    lib.yahkv_kv8_decode_part.argtypes = [G, K8, i32p, i32, i32p, i32, i32, vp, i32, C.c_float, vp, C.c_size_t, O, vp]
+    lib.yahkv_kv8_decode_reduce.argtypes = [G, K8, i32p, i32, i32p, i32, i32, vp, vp, i32, vp, i32, C.c_float, vp, vp,
+                                            vp, C.c_size_t, O, vp]
     lib.yahkv_kv8_prefill_workspace_bytes.restype = C.c_size_t
     lib.yahkv_kv8_prefill_workspace_bytes.argtypes = [G, i32, i32, i32]
     lib.yahkv_kv8_prefill_attend.argtypes = [G, K8, i32p, i32, i32p, i32, i32, i32, vp, C.c_float, vp, vp, i32, vp,
@@ -683,3 +686,22 @@ def kv8_prefill_attend(pools, table, prefix_len, max_prefix_len, q, scale, gate=
                                         max_prefix_len, chunk, _dp(q), scale, _dp(gate), _dp(out), _dtype_code(out),
                                         _dp(workspace), workspace.numel(), _stream()), "kv8_prefill_attend")
     return out
+
+
+def kv8_decode_part(pools, table, seq_len, max_seq_len, q, scale, workspace, opt=None):
+    g = pools.geom
+    st = pools.struct()
+    _check(lib.yahkv_kv8_decode_part(C.byref(g), C.byref(st), _dp(table), table.shape[1], _dp(seq_len), q.shape[0],
+                                     max_seq_len, _dp(q), _dtype_code(q), scale, _dp(workspace), workspace.numel(),
+                                     _op(opt), _stream()), "kv8_decode_part")
+
+
+def kv8_decode_reduce(pools, table, seq_len, max_seq_len, q, scale, out, workspace, k_new=None, v_new=None, gate=None,
+                      opt=None):
+    """The merge; with k_new / v_new [n_seqs][H][256] the step's (it appends that token and attends to it)."""
+    g = pools.geom
+    st = pools.struct()
+    _check(lib.yahkv_kv8_decode_reduce(C.byref(g), C.byref(st), _dp(table), table.shape[1], _dp(seq_len), q.shape[0],
+                                       max_seq_len, _dp(k_new), _dp(v_new), 0 if k_new is None else _dtype_code(k_new),
+                                       _dp(q), _dtype_code(q), scale, _dp(gate), _dp(out), _dp(workspace),
+                                       workspace.numel(), _op(opt), _stream()), "kv8_decode_reduce")

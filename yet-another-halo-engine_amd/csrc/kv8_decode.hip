@@ -522,35 +522,16 @@ __global__ __launch_bounds__(kReduceThreads) void Kv8Reduce(const DecodeArgs a, 
   }
 }
 
-int CheckArgs(const yahkv_geometry* g, const yahkv_kv8_pools* pools, const int32_t* page_table, const void* q, int32_t q_dtype,
-              const float* out) {
-  if (const int st = CheckKv8Pools(g, pools)) return st;
+int Fill(const yahkv_geometry* g, const yahkv_kv8_pools* pools, const int32_t* page_table, int32_t stride,
+         const int32_t* seq_len, int32_t n_seqs, int32_t max_seq_len, const void* q, int32_t q_dtype, float softmax_scale,
+         void* workspace, size_t workspace_bytes, const yahkv_decode_options* opt, DecodeArgs* a) {
+  if (const int rc = CheckKv8Pools(g, pools)) return rc;
   if (page_table == nullptr || q == nullptr || (reinterpret_cast<uintptr_t>(q) & 15)) return YAHKV_ERR_ARG;
   if (q_dtype != YAHKV_F32 && q_dtype != YAHKV_F16 && q_dtype != YAHKV_BF16) return YAHKV_ERR_ARG;
-  if (out == nullptr || (reinterpret_cast<uintptr_t>(out) & 15)) return YAHKV_ERR_ARG;
-  return YAHKV_OK;
-}
-
-int Launch(const yahkv_geometry* g, const yahkv_kv8_pools* pools, const int32_t* page_table, int32_t stride,
-           const int32_t* seq_len, int32_t n_seqs, int32_t max_seq_len, const StepRows& rows, const void* q, int32_t q_dtype,
-           float softmax_scale, const float* gate, float* out, void* workspace, size_t workspace_bytes,
-           const yahkv_decode_options* opt, hipStream_t st) {
-  if (const int rc = CheckArgs(g, pools, page_table, q, q_dtype, out)) return rc;
   if (MakeTuning(opt).one_launch) return YAHKV_ERR_ARG;
-  DecodeArgs a;
-  if (const int rc = Prepare(MakeGeom(*g), stride, seq_len, n_seqs, max_seq_len, workspace, workspace_bytes, opt, &a)) return rc;
-  a.table = page_table, a.q = q, a.q_dtype = q_dtype, a.scale = softmax_scale, a.gate = gate, a.out = out;
-  a.open_tile = 1;
-  const Kv8Pools p = MakeKv8Pools(*pools);
-  hipLaunchKernelGGL(Kv8Part<0>, dim3(static_cast<unsigned>(a.n_chunks)), dim3(64 * kWavesPerGroup), 0, st, a, p);
-  if (const int rc = LaunchStatus()) return rc;
-  int split = 1;
-  while (int64_t(a.g.n_q) * a.n_seqs * split < ComputeUnits() && a.g.hd / (2 * split) >= kReduceMinDims) split *= 2;
-  const int asked = MakeTuning(opt).reduce_split;
-  if (asked > 0) split = std::min(asked, a.g.hd / kReduceMinDims);
-  while (a.g.hd % split != 0 || (a.g.hd / split) % 4 != 0) --split;
-  hipLaunchKernelGGL(Kv8Reduce, dim3(a.g.n_q, a.n_seqs, split), dim3(kReduceThreads), 0, st, a, p, rows);
-  return LaunchStatus();
+  if (const int rc = Prepare(MakeGeom(*g), stride, seq_len, n_seqs, max_seq_len, workspace, workspace_bytes, opt, a)) return rc;
+  a->table = page_table, a->q = q, a->q_dtype = q_dtype, a->scale = softmax_scale, a->open_tile = 1;
+  return YAHKV_OK;
 }
 
 }  // namespace
@@ -564,13 +545,58 @@ extern "C" size_t yahkv_kv8_decode_workspace_bytes(const yahkv_geometry* g, int3
   return MakePlan(MakeGeom(*g), n_seqs, max_seq_len, MakeTuning(opt)).bytes;
 }
 
+extern "C" int yahkv_kv8_decode_part(const yahkv_geometry* g, const yahkv_kv8_pools* pools, const int32_t* page_table,
+                                     int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs,
+                                     int32_t max_seq_len, const void* q, int32_t q_dtype, float softmax_scale,
+                                     void* workspace, size_t workspace_bytes, const yahkv_decode_options* opt,
+                                     void* stream) {
+  DecodeArgs a;
+  if (const int rc = Fill(g, pools, page_table, page_table_stride, seq_len, n_seqs, max_seq_len, q, q_dtype, softmax_scale,
+                          workspace, workspace_bytes, opt, &a))
+    return rc;
+  hipLaunchKernelGGL(Kv8Part<0>, dim3(static_cast<unsigned>(a.n_chunks)), dim3(64 * kWavesPerGroup), 0,
+                     static_cast<hipStream_t>(stream), a, MakeKv8Pools(*pools));
+  return LaunchStatus();
+}
+
+extern "C" int yahkv_kv8_decode_reduce(const yahkv_geometry* g, const yahkv_kv8_pools* pools, const int32_t* page_table,
+                                       int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs,
+                                       int32_t max_seq_len, const void* k_new, const void* v_new, int32_t new_dtype,
+                                       const void* q, int32_t q_dtype, float softmax_scale, const float* gate,
+                                       float* out, void* workspace, size_t workspace_bytes,
+                                       const yahkv_decode_options* opt, void* stream) {
+  if (out == nullptr || (reinterpret_cast<uintptr_t>(out) & 15)) return YAHKV_ERR_ARG;
+  if ((k_new == nullptr) != (v_new == nullptr)) return YAHKV_ERR_ARG;
+  if (k_new != nullptr) {
+    if ((reinterpret_cast<uintptr_t>(k_new) | reinterpret_cast<uintptr_t>(v_new)) & 15) return YAHKV_ERR_ARG;
+    if (new_dtype != YAHKV_F32 && new_dtype != YAHKV_F16 && new_dtype != YAHKV_BF16) return YAHKV_ERR_ARG;
+  }
+  DecodeArgs a;
+  if (const int rc = Fill(g, pools, page_table, page_table_stride, seq_len, n_seqs, max_seq_len, q, q_dtype, softmax_scale,
+                          workspace, workspace_bytes, opt, &a))
+    return rc;
+  a.gate = gate, a.out = out;
+  int split = 1;
+  while (int64_t(a.g.n_q) * a.n_seqs * split < ComputeUnits() && a.g.hd / (2 * split) >= kReduceMinDims) split *= 2;
+  const int asked = MakeTuning(opt).reduce_split;
+  if (asked > 0) split = std::min(asked, a.g.hd / kReduceMinDims);
+  while (a.g.hd % split != 0 || (a.g.hd / split) % 4 != 0) --split;
+  hipLaunchKernelGGL(Kv8Reduce, dim3(a.g.n_q, a.n_seqs, split), dim3(kReduceThreads), 0, static_cast<hipStream_t>(stream), a,
+                     MakeKv8Pools(*pools), StepRows{k_new, v_new, new_dtype});
+  return LaunchStatus();
+}
+
 extern "C" int yahkv_kv8_decode_attend(const yahkv_geometry* g, const yahkv_kv8_pools* pools, const int32_t* page_table,
                                        int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs,
                                        int32_t max_seq_len, const void* q, int32_t q_dtype, float softmax_scale,
                                        const float* gate, float* out, void* workspace, size_t workspace_bytes,
                                        const yahkv_decode_options* opt, void* stream) {
-  return Launch(g, pools, page_table, page_table_stride, seq_len, n_seqs, max_seq_len, StepRows{nullptr, nullptr, 0}, q,
-                q_dtype, softmax_scale, gate, out, workspace, workspace_bytes, opt, static_cast<hipStream_t>(stream));
+  if (out == nullptr || (reinterpret_cast<uintptr_t>(out) & 15)) return YAHKV_ERR_ARG;  // before anything is launched
+  if (const int rc = yahkv_kv8_decode_part(g, pools, page_table, page_table_stride, seq_len, n_seqs, max_seq_len, q,
+                                           q_dtype, softmax_scale, workspace, workspace_bytes, opt, stream))
+    return rc;
+  return yahkv_kv8_decode_reduce(g, pools, page_table, page_table_stride, seq_len, n_seqs, max_seq_len, nullptr, nullptr,
+                                 0, q, q_dtype, softmax_scale, gate, out, workspace, workspace_bytes, opt, stream);
 }
 
 extern "C" int yahkv_kv8_decode_step(const yahkv_geometry* g, const yahkv_kv8_pools* pools, const int32_t* page_table,
@@ -579,9 +605,13 @@ extern "C" int yahkv_kv8_decode_step(const yahkv_geometry* g, const yahkv_kv8_po
                                      const void* q, int32_t q_dtype, float softmax_scale, const float* gate, float* out,
                                      void* workspace, size_t workspace_bytes, const yahkv_decode_options* opt,
                                      void* stream) {
+  if (out == nullptr || (reinterpret_cast<uintptr_t>(out) & 15)) return YAHKV_ERR_ARG;
   if (k_new == nullptr || v_new == nullptr) return YAHKV_ERR_ARG;
   if ((reinterpret_cast<uintptr_t>(k_new) | reinterpret_cast<uintptr_t>(v_new)) & 15) return YAHKV_ERR_ARG;
   if (new_dtype != YAHKV_F32 && new_dtype != YAHKV_F16 && new_dtype != YAHKV_BF16) return YAHKV_ERR_ARG;
-  return Launch(g, pools, page_table, page_table_stride, seq_len, n_seqs, max_seq_len, StepRows{k_new, v_new, new_dtype},
-                q, q_dtype, softmax_scale, gate, out, workspace, workspace_bytes, opt, static_cast<hipStream_t>(stream));
+  if (const int rc = yahkv_kv8_decode_part(g, pools, page_table, page_table_stride, seq_len, n_seqs, max_seq_len, q,
+                                           q_dtype, softmax_scale, workspace, workspace_bytes, opt, stream))
+    return rc;
+  return yahkv_kv8_decode_reduce(g, pools, page_table, page_table_stride, seq_len, n_seqs, max_seq_len, k_new, v_new,
+                                 new_dtype, q, q_dtype, softmax_scale, gate, out, workspace, workspace_bytes, opt, stream);
 }
