@@ -46,14 +46,23 @@ WORKLOADS = {
 MFMA_F16_PEAK_TFLOPS = 2500.0
 EVENT_EVERY = 4      # decode workloads: HIP events around the split-K kernel on every fourth timed step
 NQ, NKV, HD, PT = 24, 4, 256, 64
-# HBM bytes per launch of the split-K kernel from rocprofv3 counters (FETCH_SIZE + WRITE_SIZE, each scaled by what the
-# counter reads for a plain 1 GiB copy); a measurement made outside this script, recorded with its summary.
-TRAFFIC = {"ragged_b64_q8_0": (5.327e9, "profiles/decode_part_q8_0_ragged_b64.md"),
-           "b1_ctx32k_q8_0": (8.60e7, "profiles/decode_part_q8_0_b1_ctx32k.md"),
-           "b16_ctx128k_f16": (8.619e9, "profiles/decode_part_f16_b16_ctx128k.md"),
-           "b16_ctx128k_q4_0": (2.445e9, "profiles/decode_part_q4_0_b16_ctx128k.md"),
-           "prefill_b8_ctx16k_chunk2k_q8_0": (2.150e9, "profiles/prefill_attend_q8_0_b8_ctx16k_chunk2k.md")}
+# HBM bytes per launch of each workload's dominant kernel from rocprofv3 counters (FETCH_SIZE + WRITE_SIZE, each scaled
+# by what the counter reads for a plain 1 GiB copy): measurements made outside this script, kept in a tracked table that
+# names the commit each was taken at.
+def load_traffic():
+    table = {}
+    try:
+        with open(os.path.join(ROOT, "profiles", "hbm_traffic.md")) as f:
+            for line in f:
+                cols = [c.strip() for c in line.strip().strip("|").split("|")]
+                if len(cols) == 5 and cols[0] in WORKLOADS:
+                    table[cols[0]] = (float(cols[1]), "%s (kernel %s, measured at commit %s)" % (cols[4], cols[2], cols[3]))
+    except (OSError, ValueError):
+        pass
+    return table
 
+
+TRAFFIC = load_traffic()
 
 def fnv1a(b):
     h = 0xCBF29CE484222325
@@ -688,6 +697,8 @@ def run_decode(a, wl, torch, yahkv):
     ws = torch.empty(yahkv.decode_workspace_bytes(g, B, max_len, opt), dtype=torch.uint8, device="cuda")
     # set-up, as a server does once: the XCDs' relative read speeds on this batch (equal shares without it)
     xcd = yahkv.decode_calibrate(pools, t_table, len_rows[0], max_len, q, ws, opt, rounds=3) if not a.no_calibrate else None
+    if a.one_launch:
+        yahkv.decode_workspace_init(g, B, max_len, ws, opt)
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(a.steps)]
     separate = a.separate_append or a.one_launch
 
@@ -716,12 +727,13 @@ def run_decode(a, wl, torch, yahkv):
             if pair:
                 pair[1].record()
 
-    # parity before timing: first step, a few sequences against the float64 closed form
+    # parity before timing: first step; the shortest, a quartile, the median and the longest sequence (the ones that span
+    # the most chunks and XCD shares) against the float64 closed form
     step(0)
     torch.cuda.synchronize()
     first_hash = fnv1a(out.cpu().numpy().tobytes())
     order = np.argsort(lens)
-    rows = [int(order[0]), int(order[len(order) // 4])] if B > 1 else [0]
+    rows = sorted({int(order[0]), int(order[len(order) // 4]), int(order[len(order) // 2]), int(order[-1])})
     err = parity_check(yahkv, torch, g, pools, t_table, lens + 1, q, out, scale, rows)
     if not err < 2e-3:
         raise SystemExit(f"bench.py: parity check failed before timing: max relative error {err:.3e}")
@@ -825,7 +837,8 @@ def run_workload(a, torch, yahkv):
 
 
 # what the default run times besides its own workload: the other configurations of the benchmark that fill a GPU
-ALSO = ["b1_ctx32k_q8_0", "prefill_b8_ctx16k_chunk2k_q8_0", "b16_ctx128k_q4_0"]
+ALSO = ["b1_ctx32k_q8_0", "prefill_b8_ctx16k_chunk2k_q8_0", "b16_ctx128k_q4_0", "ragged_b64_kv8a16", "ragged_b64_f16",
+        "prefill_b8_ctx16k_chunk2k_q4_0"]
 
 
 def main():

@@ -163,7 +163,9 @@ typedef struct yahkv_decode_options {
   int32_t one_launch;       /* not 0: yahkv_decode_attend issues one dispatch instead of two: the workgroup that is last
                                to finish a pair's keys merges the pair's partials itself. Same results; measured slower
                                than the two dispatches on an MI355X (partials cross between XCDs through memory), so it
-                               is for callers to whom the number of dispatches matters more than the time */
+                               is for callers to whom the number of dispatches matters more than the time. Its arrival
+                               counts live in the workspace and must start at zero: call yahkv_decode_workspace_init
+                               once on a new workspace, and again when n_seqs, max_seq_len or the options change */
 } yahkv_decode_options;
 
 /* Decode attention: one query token per sequence against keys 0 .. seq_len[s] - 1.
@@ -177,6 +179,12 @@ typedef struct yahkv_decode_options {
  * Replaces yah_dattn_part_q + yah_dattn_reduce (gen_decode_attn.py:576-1040, 338-411). */
 size_t yahkv_decode_workspace_bytes(const yahkv_geometry* g, int32_t n_seqs, int32_t max_seq_len,
                                     const yahkv_decode_options* opt);
+/* Prepares a workspace for opt->one_launch: zeroes the per-(sequence, kv head) arrival counts that form keeps in it
+ * (every such launch leaves them at zero again, so once per workspace and shape is enough; a launch that was aborted
+ * half way needs it again). A small fill kernel on `stream`; harmless, and not needed, for the two-dispatch forms.
+ * No counterpart in the reference (its reduce is always a dispatch of its own, loom_decoder.hpp:268). */
+int yahkv_decode_workspace_init(const yahkv_geometry* g, int32_t n_seqs, int32_t max_seq_len,
+                                const yahkv_decode_options* opt, void* workspace, size_t workspace_bytes, void* stream);
 /* The two dispatches of a decode attention on their own, as LoomDecoder::Step issues its own (loom_decoder.hpp:259-268):
  * `part` cuts the batch into equal pieces of work from the device-resident lengths (the reference needs no cut: it
  * has one sequence and launches one workgroup per page in use) and leaves partials (M, l, acc) per piece in the
@@ -211,7 +219,9 @@ int yahkv_decode_step(const yahkv_geometry* g, const yahkv_pools* pools, const i
 /* The second dispatch of yahkv_decode_step on its own, for callers that issue the two themselves (a timer or other
  * work between them). The first is yahkv_decode_part with the lengths BEFORE the step (every seq_len one less; a
  * device array of its own, since lengths are read on the device) and otherwise the same arguments; this call takes
- * the lengths after the step, as yahkv_decode_step does. */
+ * the lengths after the step, as yahkv_decode_step does. The split form needs every seq_len[s] <= max_seq_len (the two
+ * calls clamp longer ones differently, each from the lengths it is given; yahkv_decode_step itself clamps
+ * consistently). */
 int yahkv_decode_step_reduce(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
                              int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs, int32_t max_seq_len,
                              const void* k_new, const void* v_new, int32_t new_dtype, const void* q, int32_t q_dtype,

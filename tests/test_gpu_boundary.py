@@ -85,7 +85,8 @@ def g_dev(yahkv, g):
 @pytest.mark.parametrize("fmt,n_q,n_kv,hd,pt", [(8, 24, 4, 256, 64), (4, 24, 4, 256, 64), (8, 8, 2, 128, 16), (4, 16, 2, 256, 32)])
 def test_one_launch_form_gives_the_two_dispatches_results(yahkv, torch_gpu, fmt, n_q, n_kv, hd, pt):
     """opt.one_launch: the workgroup that is last to finish a pair's keys merges the pair itself. Sequences that lie in
-    one chunk, that span many, that are empty; twice on one workspace (the tickets of the first call are left clean),
+    one chunk, that span many, that are empty; on a workspace of random bytes that went through yahkv_decode_workspace_init
+    once, twice in a row (the arrival counts of the first call are left at zero),
     then with the chunk count forced up so that every pair spans several chunks; with the deterministic pattern the
     one dispatch repeats bit for bit as well."""
     torch = torch_gpu
@@ -98,7 +99,8 @@ def test_one_launch_form_gives_the_two_dispatches_results(yahkv, torch_gpu, fmt,
     for opt in (yahkv.decode_options(one_launch=True), yahkv.decode_options(one_launch=True, n_chunks=1000, min_chunk_tiles=2),
                 yahkv.decode_options(one_launch=True, n_chunks=7)):
         ws = torch.empty(yahkv.decode_workspace_bytes(g_dev(yahkv, g), len(lens), max(lens), opt), dtype=torch.uint8, device="cuda")
-        ws.random_(0, 256)                                     # nothing in the workspace has to start at zero
+        ws.random_(0, 256)                                     # junk everywhere, the arrival counts included ...
+        yahkv.decode_workspace_init(g_dev(yahkv, g), len(lens), max(lens), ws, opt)   # ... which this call zeroes, once
         tq = torch.from_numpy(q).cuda().to(torch.bfloat16)
         tg = torch.from_numpy(gate).cuda()
         t_table = torch.from_numpy(table).cuda()

@@ -4,6 +4,11 @@ scrambled page table, pools filled with poison first, appended bytes bit-exact, 
 closed form over the dequantized blocks):
   config 2   one sequence of 32768 tokens, q8_0, 24 Q / 4 KV heads, head_dim 256, 64-token pages, a 1024-page pool
              of which a seeded permutation hands out 512 (+ 1 for the appended token), bf16 query
+  config 3   the headline: 64 sequences with lengths uniform in [1024, 65536], q8_0, one shared pool sized to fit exactly
+             through the page allocator and shuffled; the source rows of the shortest, the median, the longest sequence
+             and of one whose length is a multiple of 64 (its step's token opens a new page) are kept and their pool
+             blocks held to the oracle's quantizer bit for bit; then one decode step (append + attention), those
+             sequences against the closed form, and the new token not visible one step earlier
   config 5   q4_0, batch 16, the same heads, K with 8 seeded outlier channels per head scaled x 20; at 2048 tokens per
              sequence against the oracle, and at the full 131072 tokens per sequence against the closed form on the
              gathered blocks of two sequences; one token appended per sequence before the attention
@@ -70,6 +75,74 @@ def test_config2_one_sequence_of_32768_tokens(yahkv, torch_gpu):
     prev = yahkv.decode_attend(dev, t_table, lens - 1, n + 1, bf16_cuda(torch, q), scale).cpu().numpy()
     assert rel_err(prev[0], closed_from_blocks(yahkv, dev, t_table[0], n, q[0], scale, 8)) < TOL
     assert np.abs(prev - got).max() > 0
+
+
+def test_config3_ragged_batch_of_64_at_full_size(yahkv, torch_gpu):
+    torch = torch_gpu
+    rng = np.random.default_rng(4)
+    B = 64
+    lens = rng.integers(1024, 65537, B).astype(np.int32)
+    order = np.argsort(lens)
+    crossing = int(order[B // 3])
+    lens[crossing] = (int(lens[crossing]) // PT) * PT          # the step's token is this sequence's first on a new page
+    order = np.argsort(lens)
+    kept = sorted({int(order[0]), int(order[B // 2]), int(order[-1]), crossing})
+    pages = (lens + 1 + PT - 1) // PT
+    n_pages = int(pages.sum())                                 # the pool fits the job exactly
+    g = yahkv.geometry(8, NQ, NKV, HD, PT, n_pages)
+    alloc = yahkv.PagePool(n_pages)
+    alloc.shuffle(4)
+    table = np.zeros((B, int(pages.max())), np.int32)
+    for s_, n_ in enumerate(pages):
+        table[s_, :n_] = alloc.alloc(int(n_))
+    assert alloc.free_count == 0
+    yahkv.validate_page_table(g, table, lens + 1)
+    dev = yahkv.DevicePools(g, fill=0x7F)
+    t_table = torch.from_numpy(table).cuda()
+    gen = torch.Generator(device="cuda").manual_seed(4)
+    src = {}
+    for s_ in range(B):
+        ks, vs = [], []
+        for o in range(0, int(lens[s_]), 8192):
+            n_ = min(8192, int(lens[s_]) - o)
+            k = torch.randn((1, n_, NKV, HD), generator=gen, device="cuda").to(torch.bfloat16)
+            v = torch.randn((1, n_, NKV, HD), generator=gen, device="cuda").to(torch.bfloat16)
+            yahkv.append(dev, t_table[s_:s_ + 1], torch.tensor([o], dtype=torch.int32, device="cuda"), k, v)
+            if s_ in kept:
+                ks.append(k[0].float().cpu().numpy()), vs.append(v[0].float().cpu().numpy())
+        if s_ in kept:
+            src[s_] = (np.concatenate(ks), np.concatenate(vs))
+    knew = to_bf16_f32(rng.standard_normal((B, NKV, HD)))
+    vnew = to_bf16_f32(rng.standard_normal((B, NKV, HD)))
+    q = to_bf16_f32(rng.standard_normal((B, NQ, HD)))
+    scale = 1.0 / 16
+    t_lens = torch.from_numpy(lens).cuda()
+    max_len = int(lens.max()) + 1
+    opt = yahkv.decode_options()
+    ws = torch.empty(yahkv.decode_workspace_bytes(g, B, max_len, opt), dtype=torch.uint8, device="cuda")
+    yahkv.decode_calibrate(dev, t_table, t_lens, max_len, bf16_cuda(torch, q), ws, opt, rounds=2)   # unequal XCD shares, as the bench runs
+    before = yahkv.decode_attend(dev, t_table, t_lens, max_len, bf16_cuda(torch, q), scale, workspace=ws, opt=opt).cpu().numpy()
+    out = yahkv.decode_step(dev, t_table, t_lens + 1, max_len, bf16_cuda(torch, knew), bf16_cuda(torch, vnew),
+                            bf16_cuda(torch, q), scale, workspace=ws, opt=opt)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    assert np.all(np.isfinite(got))
+    for s_ in kept:
+        n_ = int(lens[s_])
+        k, v = yahkv.gather_blocks(dev, t_table[s_], n_ + 1)
+        kb, vb = k.cpu().numpy(), v.cpu().numpy()
+        # pool bytes of the whole sequence against the oracle's quantizer on the kept source rows, and the step's token
+        assert np.array_equal(kb[:n_].reshape(-1, 34), oracle.quantize_q8_0(src[s_][0])), f"sequence {s_}: K blocks"
+        assert np.array_equal(vb[:n_].reshape(-1, 34), oracle.quantize_q8_0(src[s_][1])), f"sequence {s_}: V blocks"
+        assert np.array_equal(kb[n_].reshape(-1, 34), oracle.quantize_q8_0(knew[s_])), f"sequence {s_}: the step's K"
+        assert np.array_equal(vb[n_].reshape(-1, 34), oracle.quantize_q8_0(vnew[s_])), f"sequence {s_}: the step's V"
+        Kd = oracle.dequantize_q8_0(kb.reshape(-1, 34)).reshape(n_ + 1, NKV, HD)
+        Vd = oracle.dequantize_q8_0(vb.reshape(-1, 34)).reshape(n_ + 1, NKV, HD)
+        err = rel_err(got[s_], closed_form(Kd, Vd, q[s_], scale))
+        assert err < TOL, (s_, n_, err)
+        assert rel_err(before[s_], closed_form(Kd[:n_], Vd[:n_], q[s_], scale)) < TOL, (s_, "one step earlier")
+        assert np.abs(before[s_] - got[s_]).max() > 0
+    assert int(lens[crossing]) % PT == 0 and pages[crossing] == int(lens[crossing]) // PT + 1   # the token's own page
 
 
 def outlier_scales(rng):

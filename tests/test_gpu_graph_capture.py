@@ -34,6 +34,8 @@ def test_decode_step_replays_from_a_graph(yahkv, torch_gpu, form):
             yahkv.decode_step(dev, t_table, seq_len, 701, k[:, 0], v[:, 0], q, 0.0625, out=out, workspace=ws, opt=opt)
             return
         yahkv.append(dev, t_table, pos, k, v)
+        if form == "one_launch":                      # its arrival counts start at zero: the fill kernel is captured too
+            yahkv.decode_workspace_init(dev.geom, 4, 701, ws, opt)
         yahkv.decode_attend(dev, t_table, seq_len, 701, q, 0.0625, out=out, workspace=ws, opt=opt)
 
     step()                                            # eager: also the one-time host set-up of the library

@@ -71,6 +71,7 @@ def _load():
     lib.yahkv_decode_workspace_bytes.restype = C.c_size_t
     O = C.POINTER(DecodeOptions)
     lib.yahkv_decode_workspace_bytes.argtypes = [G, i32, i32, O]
+    lib.yahkv_decode_workspace_init.argtypes = [G, i32, i32, O, vp, C.c_size_t, vp]
     lib.yahkv_decode_part.argtypes = [G, P, i32p, i32, i32p, i32, i32, vp, i32, C.c_float, vp, C.c_size_t, O, vp]
     lib.yahkv_decode_reduce.argtypes = [G, i32, i32p, i32, i32, vp, vp, vp, C.c_size_t, O, vp]
     lib.yahkv_decode_attend.argtypes = [G, P, i32p, i32, i32p, i32, i32, vp, i32, C.c_float, vp, vp, vp, C.c_size_t, O,
@@ -391,8 +392,15 @@ def decode_workspace_bytes(g, n_seqs, max_seq_len, opt=None):
     return lib.yahkv_decode_workspace_bytes(C.byref(g), n_seqs, max_seq_len, _op(opt))
 
 
+def decode_workspace_init(g, n_seqs, max_seq_len, workspace, opt=None):
+    """Zeroes the arrival counts the one-launch form keeps in the workspace (once per workspace and shape)."""
+    _check(lib.yahkv_decode_workspace_init(C.byref(g), n_seqs, max_seq_len, _op(opt), _dp(workspace), workspace.numel(),
+                                           _stream()), "decode_workspace_init")
+
+
 def decode_attend(pools, table, seq_len, max_seq_len, q, scale, gate=None, out=None, workspace=None, opt=None):
-    """q: [n_seqs][n_q_heads][D] f16 / bf16 / f32; returns out f32 of the same shape."""
+    """q: [n_seqs][n_q_heads][D] f16 / bf16 / f32; returns out f32 of the same shape. A workspace given by the caller
+    and used with opt.one_launch must have been through decode_workspace_init."""
     import torch
     g = pools.geom
     n_seqs = q.shape[0]
@@ -402,6 +410,8 @@ def decode_attend(pools, table, seq_len, max_seq_len, q, scale, gate=None, out=N
     need = decode_workspace_bytes(g, n_seqs, max_seq_len, opt)
     if workspace is None:
         workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
+        if opt is not None and opt.one_launch:
+            decode_workspace_init(g, n_seqs, max_seq_len, workspace, opt)
     st = pools.struct()
     _check(lib.yahkv_decode_attend(C.byref(g), C.byref(st), _dp(table), table.shape[1], _dp(seq_len), n_seqs,
                                    max_seq_len, _dp(q), _dtype_code(q), scale, _dp(gate), _dp(out), _dp(workspace),

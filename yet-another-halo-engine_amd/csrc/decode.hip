@@ -101,26 +101,16 @@ __device__ __forceinline__ h8v RawNibbles8(uint32_t w0, uint32_t w1) {
 
 
 // A workgroup announces that its partials of a pair are written; true for the one that is last of `n`, which then owns
-// the merge. The ticket word carries the launch's epoch above the count: a word with another epoch in it (memory that
-// was never used, or the zero the last arrival of an earlier launch left) counts as empty, so the workspace needs no
-// clearing, and the last arrival puts the zero back, so a graph replay, which repeats its epoch, starts clean too.
-// Only the first arrival of a launch has to replace the word (compare and swap); the others, who find the launch's
-// epoch in it, add one, which no number of simultaneous arrivals turns into retries.
-__device__ __forceinline__ int Arrive(unsigned long long* ticket, uint32_t epoch, uint32_t n) {
-  unsigned long long old = __hip_atomic_load(ticket, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  while (true) {
-    if (static_cast<uint32_t>(old >> 32) == epoch) {
-      old = __hip_atomic_fetch_add(ticket, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if (static_cast<uint32_t>(old) + 1 != n) return 0;
-      __hip_atomic_store(ticket, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // everybody has arrived
-      return 1;
-    }
-    const bool last = n == 1;
-    const unsigned long long next = last ? 0ull : (static_cast<unsigned long long>(epoch) << 32) | 1ull;
-    if (__hip_atomic_compare_exchange_strong(ticket, &old, next, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
-                                             __HIP_MEMORY_SCOPE_AGENT))
-      return last ? 1 : 0;
-  }
+// the merge. The ticket is a plain count that starts at zero: yahkv_decode_workspace_init zeroes the tickets once, and
+// the last arrival of every launch puts the zero back, so launch after launch and graph replay after graph replay find
+// it clean. (Relaxed atomics at device scope: the partials themselves travel by device-scope buffer accesses, written
+// through and waited for before the arrival, read past the L2 after it; a release / acquire pair here would write back
+// and invalidate whole L2s instead, which cost the kernel 12 % when measured.)
+__device__ __forceinline__ int Arrive(unsigned long long* ticket, uint32_t n) {
+  const unsigned long long old = __hip_atomic_fetch_add(ticket, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (static_cast<uint32_t>(old) + 1 != n) return 0;
+  __hip_atomic_store(ticket, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // everybody has arrived
+  return 1;
 }
 
 // One workgroup of eight waves per chunk, one workgroup per CU (two waves per SIMD). The waves share nothing but the
@@ -714,7 +704,7 @@ void DattnPart(const DecodeArgs a) {
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
     if (threadIdx.x == 0)
-      merge_flag = k0 == k1 ? 1 : Arrive(&a.tickets[s_ * H + h_], a.epoch, static_cast<uint32_t>(k1 - k0 + 1));
+      merge_flag = k0 == k1 ? 1 : Arrive(&a.tickets[s_ * H + h_], static_cast<uint32_t>(k1 - k0 + 1));
     __syncthreads();
     const bool mine = merge_flag != 0;
     __syncthreads();  // (the flag is free again)
@@ -1061,15 +1051,32 @@ extern "C" int yahkv_decode_step(const yahkv_geometry* g, const yahkv_pools* poo
                                   stream);
 }
 
+namespace yahkv {
 namespace {
-// A number no two launches of this process share (0 is what a ticket holds between launches).
-uint32_t NextEpoch() {
-  static std::atomic<uint32_t> counter{0};
-  uint32_t e = 0;
-  while (e == 0) e = counter.fetch_add(1, std::memory_order_relaxed) + 1;
-  return e;
+__global__ void ClearTickets(unsigned long long* tickets, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) tickets[i] = 0ull;
 }
 }  // namespace
+}  // namespace yahkv
+
+// The one-launch form counts arrivals per (sequence, kv head) in the workspace and leaves every count at zero when it
+// is done; this call puts the zeros there in the first place (a small fill kernel, so it may be captured into a graph).
+extern "C" int yahkv_decode_workspace_init(const yahkv_geometry* g, int32_t n_seqs, int32_t max_seq_len,
+                                           const yahkv_decode_options* opt, void* workspace, size_t workspace_bytes,
+                                           void* stream) {
+  if (const int st = CheckGeometry(g)) return st;
+  if (workspace == nullptr || (reinterpret_cast<uintptr_t>(workspace) & 15) || n_seqs <= 0 || max_seq_len <= 0)
+    return YAHKV_ERR_ARG;
+  if (n_seqs > kMaxSeqs) return YAHKV_ERR_SHAPE;
+  const Geom m = MakeGeom(*g);
+  const Plan p = MakePlan(m, n_seqs, max_seq_len, MakeTuning(opt));
+  if (workspace_bytes < p.bytes) return YAHKV_ERR_WORKSPACE;
+  const int n = n_seqs * m.n_kv;
+  hipLaunchKernelGGL(ClearTickets, dim3((n + 255) / 256), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     reinterpret_cast<unsigned long long*>(static_cast<char*>(workspace) + p.off_tickets), n);
+  return LaunchStatus();
+}
 
 // Two dispatches, partials and their merge; or, if the caller's options ask for it, one: the split-K kernel, whose
 // workgroups then also merge the pairs they are last to finish.
@@ -1092,7 +1099,7 @@ extern "C" int yahkv_decode_attend(const yahkv_geometry* g, const yahkv_pools* p
     return st;
   if (const int st = CheckPartArgs(g, pools, page_table, q, q_dtype)) return st;
   a.pools = MakePools(*pools), a.table = page_table, a.q = q, a.q_dtype = q_dtype, a.scale = softmax_scale;
-  a.gate = gate, a.out = out, a.fused = 1, a.epoch = NextEpoch();
+  a.gate = gate, a.out = out, a.fused = 1;
   return LaunchPart(a, static_cast<hipStream_t>(stream));
 }
 

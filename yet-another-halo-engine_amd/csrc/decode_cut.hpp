@@ -42,8 +42,7 @@ struct DecodeArgs {
   unsigned long long* stamps;  // calibration only: [2 * n_chunks] when each workgroup started, and when its last wave finished
   // one launch for part and merge: the workgroup that is last to finish a pair's tiles merges the pair's partials
   int32_t fused;                // (read by the host, which launches the kernel's one-launch instance)
-  uint32_t epoch;               // never 0, different in every launch (graph replays aside: see Arrive)
-  unsigned long long* tickets;  // [n_seqs * H] arrivals per pair: (epoch << 32) | workgroups that have arrived
+  unsigned long long* tickets;  // [n_seqs * H] workgroups that have arrived at a pair's merge; zero between launches
   // The step form (append + attention in two launches): seq_len counts the step's own token, which is not in the
   // pools yet. The part kernel then covers the len_bias = -1 shorter sequences already there, and the reduce
   // quantizes the token's rows, writes them to the pools and adds the token's term to the sums (StepRows).

@@ -1079,6 +1079,15 @@ extern "C" int yahkv_prefill_attend(const yahkv_geometry* g, const yahkv_pools* 
                                     const float* gate, void* out, int32_t out_dtype, void* workspace,
                                     size_t workspace_bytes, void* stream) {
   if (workspace != nullptr) {
+    {  // everything the second dispatch would refuse is refused here, before the first one is queued
+      PrefillArgs chk;
+      if (const int rc = PreparePrefill(g, pools, page_table, page_table_stride, prefix_len, n_seqs, max_prefix_len,
+                                        chunk_len, &chk))
+        return rc;
+      if (const int rc = PrepareQueries(q, softmax_scale, gate, out, out_dtype, &chk)) return rc;
+      if (int64_t(TilesPerPair(max_prefix_len, chunk_len)) * (2 * kKeys * chk.g.hd * 2) > 0x7fffffffLL) return YAHKV_ERR_SHAPE;
+      if (const int rc = CheckWorkspace(chk, workspace, workspace_bytes)) return rc;
+    }
     if (const int rc = yahkv_prefill_decode_tiles(g, pools, page_table, page_table_stride, prefix_len, n_seqs,
                                                   max_prefix_len, chunk_len, workspace, workspace_bytes, stream))
       return rc;
