@@ -19,6 +19,17 @@ def test_kv_cache_cpp_program():
 
 
 @pytest.mark.gpu
+def test_kv8_cache_cpp_program():
+    """Kv8Decoder / Kv8Prefill (the reference's own KV format): chunks, steps across tiles and a page, a sequence that
+    starts with steps, the contiguity rule of the open V tile; buffers bit for bit against the oracle of that format."""
+    exe = os.path.join(ROOT, "tests", "cpp", "kv8_cache_test")
+    assert os.path.exists(exe), "tests/cpp/kv8_cache_test is not built: run `python __graft_entry__.py build`"
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=100)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "kv8_cache_test: ok" in r.stdout
+
+
+@pytest.mark.gpu
 def test_kv_batcher_cpp_program():
     """Twelve requests through a pool too small for them: waiting, side by side, put back and started again; every
     attention row against the oracle, every finished request's blocks bit-exact, no page lost."""
