@@ -425,6 +425,8 @@ def run_kv8(a, wl, torch, yahkv):
     vnew = torch.randn((total, B, NKV, HD), generator=gen, device="cuda").to(torch.bfloat16)
     out = torch.empty((B, NQ, HD), dtype=torch.float32, device="cuda")
     opt = yahkv.decode_options(deterministic=a.deterministic, min_chunk_tiles=a.min_chunk_tiles)
+    if a.first_come:
+        opt.deterministic = -1
     ws = torch.empty(yahkv.lib.yahkv_kv8_decode_workspace_bytes(g, B, max_len, opt), dtype=torch.uint8, device="cuda")
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(a.steps)]
 
@@ -693,7 +695,9 @@ def run_decode(a, wl, torch, yahkv):
     vnew = torch.randn((total, B, 1, NKV, HD), generator=gen, device="cuda").to(torch.bfloat16)
     out = torch.empty((B, NQ, HD), dtype=torch.float32, device="cuda")
     opt = yahkv.decode_options(one_launch=a.one_launch, deterministic=a.deterministic,
-                               min_chunk_tiles=a.min_chunk_tiles)
+                               min_chunk_tiles=a.min_chunk_tiles, wg_partials=a.wg_partials)
+    if a.first_come:
+        opt.deterministic = -1
     ws = torch.empty(yahkv.decode_workspace_bytes(g, B, max_len, opt), dtype=torch.uint8, device="cuda")
     # set-up, as a server does once: the XCDs' relative read speeds on this batch (equal shares without it)
     xcd = yahkv.decode_calibrate(pools, t_table, len_rows[0], max_len, q, ws, opt, rounds=3) if not a.no_calibrate else None
@@ -852,14 +856,19 @@ def main():
     ap.add_argument("--no-also", action="store_true",
                     help="default workload only: do not time the other configurations for the line's `also` object")
     ap.add_argument("--no-calibrate", action="store_true", help="decode workloads: equal chunk shares for all XCDs")
-    ap.add_argument("--deterministic", action="store_true",
-                    help="decode workloads: opt.deterministic (fixed tile pattern per wave: same bytes in, same bits out)")
+    ap.add_argument("--deterministic", action="store_true", help="decode workloads: the default (fixed tile pattern per wave)")
+    ap.add_argument("--first-come", action="store_true",
+                    help="decode workloads: opt.deterministic = -1, a workgroup's tiles handed out first come, first served "
+                         "(results then differ in their last bits from run to run)")
     ap.add_argument("--one-launch", action="store_true",
                     help="decode workloads: yahkv_decode_attend with opt.one_launch instead of part + reduce")
     ap.add_argument("--one-pass", action="store_true",
                     help="quantized prefill workloads: no workspace, the attention kernel decodes its tiles itself")
     ap.add_argument("--min-chunk-tiles", type=int, default=0,
                     help="decode workloads: yahkv_decode_options::min_chunk_tiles (0: the library's default)")
+    ap.add_argument("--wg-partials", type=int, default=0, choices=[0, 1, 2],
+                    help="q8_0 / q4_0 decode workloads: yahkv_decode_options::wg_partials (1: one partial per workgroup for a "
+                         "chunk's last pair, 2: one per wave, 0: chosen from the batch's size)")
     ap.add_argument("--separate-append", action="store_true",
                     help="decode workloads: the step's token is appended by a dispatch of its own (three per step)")
     ap.add_argument("--clock-trace", action="store_true",

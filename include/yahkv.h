@@ -155,9 +155,11 @@ typedef struct yahkv_decode_options {
   int32_t min_chunk_tiles;  /* fewest 64-key tiles a piece gets (each piece costs a partial); 0: 16; at least 2 */
   int32_t pair_cost;        /* what a change of (sequence, kv head) costs a workgroup, in tiles; 0: 8; negative: none */
   int32_t reduce_split;     /* workgroups per (query head, sequence) of the merge; 0: chosen from the batch size */
-  int32_t deterministic;    /* not 0: the waves of a workgroup take its tiles in a fixed pattern, so two calls on the
-                               same bytes give the same bits (by default tiles go first come, first served, and
-                               results differ by about 1e-4 relative from run to run) */
+  int32_t deterministic;    /* 0 or positive (the default): the waves of a workgroup take its tiles in a fixed pattern, so
+                               two calls on the same bytes with the same options give the same bits (the two waves of a
+                               SIMD pace each other through their priorities, which costs nothing measurable against a
+                               first-come hand-out); negative: tiles go first come, first served, and results differ by
+                               about 1e-4 relative from run to run (kept for measurements) */
   int32_t xcd_weight[8];    /* relative read speeds of the eight XCDs, as yahkv_decode_calibrate measures them; the
                                chunks of a group of eight are sized by them; all 0: equal shares */
   int32_t one_launch;       /* not 0: yahkv_decode_attend issues one dispatch instead of two: the workgroup that is last
@@ -166,6 +168,9 @@ typedef struct yahkv_decode_options {
                                is for callers to whom the number of dispatches matters more than the time. Its arrival
                                counts live in the workspace and must start at zero: call yahkv_decode_workspace_init
                                once on a new workspace, and again when n_seqs, max_seq_len or the options change */
+  int32_t wg_partials;      /* what a workgroup leaves of the last (sequence, kv head) pair it worked on: 1: one partial,
+                               merged from its waves' in LDS; 2: one per wave; 0: chosen from the batch's size (one per
+                               workgroup when the whole batch is at most four 64-key tiles per wave) */
 } yahkv_decode_options;
 
 /* Decode attention: one query token per sequence against keys 0 .. seq_len[s] - 1.

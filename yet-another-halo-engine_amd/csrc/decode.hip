@@ -131,9 +131,13 @@ __device__ __forceinline__ int Arrive(unsigned long long* ticket, uint32_t n) {
 // for the whole wave).
 // FUSED: the one-launch form, whose merge follows the split-K work in the same kernel. It is a template argument and
 // not a field of the arguments because the merge's registers would otherwise be the plain kernel's too (spills).
-template <int FMT, int D, int PT, bool FUSED>
+// MODE 2: two dispatches as MODE 0, but what the waves have of the chunk's LAST pair meets in LDS and leaves as one
+// partial instead of eight (the in-LDS merge of the one-launch form, without its tickets). For a small batch, where a
+// chunk is a few tiles of a single pair, that is an eighth of the partials to write here and to read in the merge.
+template <int FMT, int D, int PT, int MODE>
 __global__ __launch_bounds__(64 * kWavesPerGroup) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void DattnPart(const DecodeArgs a) {
+  constexpr bool FUSED = MODE == 1, HOLD = MODE != 0;
   constexpr int NB = D / 32, NT = D / 16, PPT = kTile / PT;
   constexpr bool Q8 = FMT == 8;
   constexpr int KW = Q8 ? 4 : 2;             // dwords of K codes per lane and block
@@ -163,6 +167,7 @@ void DattnPart(const DecodeArgs a) {
   // half a tile of V codes on its way in (q8_0); at the kernel's end, either format: the waves' sums of a merge
   __shared__ __align__(16) uint8_t lvq_all[kWavesPerGroup][FMT == 8 ? NVB * 1024 : sizeof(float) * kMaxGroup * D];
   __shared__ int next_tile;
+  __shared__ int progress[kWavesPerGroup];  // tiles each wave is through with (fixed pattern only)
   __shared__ int wave_sum[kWavesPerGroup][2];
   __shared__ int4 chunk_rec;
   __shared__ long long chunk_tiles[4];  // [2], [3]: for the merge, see ChunkRecord
@@ -176,7 +181,11 @@ void DattnPart(const DecodeArgs a) {
 
   if (a.stamps != nullptr && threadIdx.x == 0) a.stamps[blockIdx.x] = wall_clock64();
   bool any_empty = false;
-  const int4 rec = ChunkRecord<64 * kWavesPerGroup>(a, blockIdx.x, wave_sum, &chunk_rec, chunk_tiles, &any_empty);
+  const int4 rec_v = a.n_seqs <= 64 ? ChunkRecordWave(a, blockIdx.x, wave, lane, &chunk_rec, chunk_tiles, &any_empty)
+                                    : ChunkRecord<64 * kWavesPerGroup>(a, blockIdx.x, wave_sum, &chunk_rec, chunk_tiles, &any_empty);
+  // (the record is the same in every lane: scalar registers for it and for everything derived from it)
+  const int4 rec = {__builtin_amdgcn_readfirstlane(rec_v.x), __builtin_amdgcn_readfirstlane(rec_v.y),
+                    __builtin_amdgcn_readfirstlane(rec_v.z), __builtin_amdgcn_readfirstlane(rec_v.w)};
   // One launch for part and merge: sequences without keys have no pair on the line and nobody merges them, so the
   // first workgroup writes their rows of zeros (its threads have just looked at a slice of the lengths each).
   if (FUSED && blockIdx.x == 0 && any_empty) {
@@ -191,11 +200,33 @@ void DattnPart(const DecodeArgs a) {
   }
   if (rec.x < 0) return;
   const int chunk_n = rec.w;
-  if (threadIdx.x == 0) next_tile = 0;
-  __syncthreads();
+  // (a chunk of at most one tile per wave needs no hand-out: wave w takes tile w, and the counter's barrier is saved)
+  const bool fixed_pattern = a.deterministic || chunk_n <= kWavesPerGroup;
+  if (!fixed_pattern) {
+    if (threadIdx.x == 0) next_tile = 0;
+    __syncthreads();
+  }
   int my_next = wave;
+  // With a fixed pattern nothing evens the waves out by itself: the two waves of a SIMD do not run equally fast (the
+  // older one wins the issue arbitration), the faster one runs out of tiles and leaves the SIMD to a lone wave. Each
+  // wave therefore tells its SIMD's other wave (wave ^ 4) how far it is, and whoever is behind raises its priority:
+  // which wave works on which tile stays fixed, and with it the bits of the result.
+  int done_tiles = 0;
+  if (lane == 0) progress[wave] = 0;
+  auto pace = [&]() {
+    if (!fixed_pattern) return;
+    ++done_tiles;
+    int other = 0;
+    if (lane == 0) {
+      __hip_atomic_store(&progress[wave], done_tiles, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      other = __hip_atomic_load(&progress[wave ^ 4], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+    other = __builtin_amdgcn_readfirstlane(other);
+    if (done_tiles < other) __builtin_amdgcn_s_setprio(2);
+    else __builtin_amdgcn_s_setprio(0);
+  };
   auto take = [&]() -> int {  // the next tile of the chunk nobody has taken yet (>= chunk_n: none left)
-    if (a.deterministic) {    // wave w takes tiles w, w + 8, ...: the same sums in the same order on every run
+    if (fixed_pattern) {      // wave w takes tiles w, w + 8, ...: the same sums in the same order on every run
       const int v = my_next;
       my_next += kWavesPerGroup;
       return v;
@@ -519,6 +550,7 @@ void DattnPart(const DecodeArgs a) {
       pv(0);
       if constexpr (!kLdsV) fetch_v(1, pgc);
       idx = nidx;
+      pace();
       if (!has_next) break;
       tile = ntile;
 #pragma unroll
@@ -528,7 +560,7 @@ void DattnPart(const DecodeArgs a) {
     pv(1);
     // One launch for part and merge: what a wave has of the chunk's last pair stays in its registers, and the waves'
     // shares of that pair meet in LDS below instead of travelling through memory one by one.
-    if (FUSED && cur.base + cur.n >= chunk_n) {
+    if (HOLD && cur.base + cur.n >= chunk_n) {
       held = true;
       break;
     }
@@ -538,12 +570,12 @@ void DattnPart(const DecodeArgs a) {
   // pairs of the chunk after this wave's last tile (of the last pair, a wave that holds nothing says so in LDS below)
   if (!held) {
     do {
-      if (!worked && !(FUSED && cur.base + cur.n >= chunk_n)) leave_empty();
+      if (!worked && !(HOLD && cur.base + cur.n >= chunk_n)) leave_empty();
       worked = false;
     } while (NextPair(a, chunk_n, &cur));
   }
   if (a.stamps != nullptr && lane == 0) atomicMax(&a.stamps[a.n_chunks + blockIdx.x], wall_clock64());
-  if (!FUSED) return;
+  if (!HOLD) return;
 
   // ---- the merge, in the same launch (gen_decode_attn.py:338-411 is the reference's separate dispatch). A pair's
   // partials come from the workgroups of every chunk its tiles lie in; each of them, when all its waves are done,
@@ -718,7 +750,7 @@ void DattnPart(const DecodeArgs a) {
     }
     const int s_ = mc.c.s, h_ = mc.c.h;
     const int k0 = ChunkOf(a, units_per_chunk, mc.line0), k1 = ChunkOf(a, units_per_chunk, mc.line0 + mc.ts - 1);
-    if (k0 == k1) {
+    if (FUSED && k0 == k1) {
       finish(s_, h_);
       __syncthreads();
     } else {
@@ -737,6 +769,7 @@ void DattnPart(const DecodeArgs a) {
           StoreDevice2(rml, (d * G + gi) * 8, merge_m[gi] * kLn2, d == 0 ? l : 0.0f);
         }
       }
+      if (!FUSED) return;  // MODE 2: the separate merge dispatch takes it from here
       arrive_and_merge(s_, h_, k0, k1);
     }
   }
@@ -925,8 +958,9 @@ int LaunchPart(const DecodeArgs& a, hipStream_t st) {
   const dim3 grid(static_cast<unsigned>(a.n_chunks));
 #define YAHKV_LAUNCH_PART(FF, DD, PP)                                                                          \
   do {                                                                                                         \
-    if (a.fused) hipLaunchKernelGGL((DattnPart<FF, DD, PP, true>), grid, dim3(64 * kWavesPerGroup), 0, st, a); \
-    else hipLaunchKernelGGL((DattnPart<FF, DD, PP, false>), grid, dim3(64 * kWavesPerGroup), 0, st, a);        \
+    if (a.fused) hipLaunchKernelGGL((DattnPart<FF, DD, PP, 1>), grid, dim3(64 * kWavesPerGroup), 0, st, a);           \
+    else if (a.wg_partials) hipLaunchKernelGGL((DattnPart<FF, DD, PP, 2>), grid, dim3(64 * kWavesPerGroup), 0, st, a); \
+    else hipLaunchKernelGGL((DattnPart<FF, DD, PP, 0>), grid, dim3(64 * kWavesPerGroup), 0, st, a);                    \
   } while (0)
 #define YAHKV_LAUNCH_FMT(FF)                                       \
   if (m.hd == 256 && m.pt == 64) YAHKV_LAUNCH_PART(FF, 256, 64);      \

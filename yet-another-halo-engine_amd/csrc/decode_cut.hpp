@@ -38,10 +38,11 @@ struct DecodeArgs {
   int32_t min_chunk_tiles;
   int32_t pair_cost;  // line units a (sequence, kv head) pair takes besides its tiles
   int32_t share[9];  // cumulative shares of the eight chunks of a group, in 1/8192 of the group (share[8] = 8192)
-  int32_t deterministic;  // waves take the chunk's tiles in a fixed pattern instead of first come, first served
+  int32_t deterministic;  // waves take the chunk's tiles in a fixed pattern (the default) instead of first come, first served
   unsigned long long* stamps;  // calibration only: [2 * n_chunks] when each workgroup started, and when its last wave finished
   // one launch for part and merge: the workgroup that is last to finish a pair's tiles merges the pair's partials
   int32_t fused;                // (read by the host, which launches the kernel's one-launch instance)
+  int32_t wg_partials;          // (host) the instance that leaves one partial per workgroup for a chunk's last pair
   unsigned long long* tickets;  // [n_seqs * H] workgroups that have arrived at a pair's merge; zero between launches
   // The step form (append + attention in two launches): seq_len counts the step's own token, which is not in the
   // pools yet. The part kernel then covers the len_bias = -1 shorter sequences already there, and the reduce
@@ -187,6 +188,53 @@ __device__ __forceinline__ int4 ChunkRecord(const DecodeArgs& a, int k, int (*wa
   int4 rec = *found;
   rec.w = static_cast<int>(tiles_at[1] - tiles_at[0]);
   if (rec.w <= 0) return int4{-1, 0, 0, 0};  // the chunk lies inside a pair's first units
+  return rec;
+}
+
+// The same record for a batch of at most 64 sequences, computed by every wave for itself (lane = sequence): no LDS,
+// no barrier, one load per lane and a handful of shuffles, where the general form costs two barriers and a loop per
+// thread. A small batch is where this matters: its part kernel runs some tens of microseconds, and the cut is a
+// dependent prologue in front of every wave's first load. The first wave of the workgroup leaves the record in LDS for
+// the merge at the kernel's end (which reads it behind a barrier).
+__device__ __forceinline__ int4 ChunkRecordWave(const DecodeArgs& a, int k, int wave, int lane, int4* found, long long* tiles_at,
+                                                bool* any_empty) {
+  const int H = a.g.n_kv, c = a.pair_cost;
+  const int ts = lane < a.n_seqs ? TilesOf(a, lane) : 0, units = UnitsOf(a, ts), cnt = ts > 0;
+  *any_empty = __builtin_amdgcn_ballot_w64(lane < a.n_seqs && ts == 0) != 0;
+  int incl = units, incl_cnt = cnt;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const int v = __shfl_up(incl, o, 64), vc = __shfl_up(incl_cnt, o, 64);
+    if (lane >= o) incl += v, incl_cnt += vc;
+  }
+  const int base = incl - units, base_cnt = incl_cnt - cnt;
+  const int total = __shfl(incl, 63, 64), total_cnt = __shfl(incl_cnt, 63, 64);
+  if (k == 0 && wave == 0) {
+    if (lane < a.n_seqs) a.tprefix[lane] = base;
+    if (lane == 0) a.tprefix[a.n_seqs] = total;
+  }
+  const long long line = static_cast<long long>(total) * H, A = ChunkUnits(a, line);
+  const long long start = ChunkStart(a, A, k), end = min(ChunkStart(a, A, k + 1), line);
+  if (start >= end) return int4{-1, 0, 0, 0};
+  // where line position x lies: the lane (sequence) whose stretch holds it works it out, the others take its answer
+  auto locate = [&](long long x, int* s_, int* h_, int* first_, long long* tiles, long long* line0) {
+    const bool mine = units > 0 && x >= static_cast<long long>(base) * H && x < static_cast<long long>(base + units) * H;
+    const int src = __builtin_ctzll(__builtin_amdgcn_ballot_w64(mine) | (1ull << 63));
+    const int r = static_cast<int>(x - static_cast<long long>(base) * H);
+    const int h = mine ? r / units : 0, first = mine ? max(r % units - c, 0) : 0;
+    const long long t = static_cast<long long>(base - c * base_cnt) * H + static_cast<long long>(h) * ts + first;
+    const long long l0 = static_cast<long long>(base) * H + static_cast<long long>(h) * units + c;
+    *s_ = src, *h_ = __shfl(h, src, 64), *first_ = __shfl(first, src, 64);
+    *tiles = __shfl(t, src, 64), *line0 = __shfl(l0, src, 64);
+  };
+  int s0, h0, f0, s1, h1, f1;
+  long long t0, t1, l0, l1;
+  locate(start, &s0, &h0, &f0, &t0, &l0);
+  if (end < line) locate(end, &s1, &h1, &f1, &t1, &l1);
+  else t1 = static_cast<long long>(total - c * total_cnt) * H;
+  int4 rec = {s0, h0, f0, static_cast<int>(t1 - t0)};
+  if (wave == 0 && lane == 0) *found = rec, tiles_at[0] = t0, tiles_at[1] = t1, tiles_at[2] = l0, tiles_at[3] = A;
+  if (rec.w <= 0) return int4{-1, 0, 0, 0};
   return rec;
 }
 
@@ -341,7 +389,7 @@ inline int ComputeUnits() {
 }
 // Tuning values of a call: the caller's options where given, else the defaults.
 struct Tuning {
-  int32_t n_chunks, min_chunk_tiles, pair_cost, reduce_split, deterministic, one_launch;
+  int32_t n_chunks, min_chunk_tiles, pair_cost, reduce_split, deterministic, one_launch, wg_partials;
   int32_t xcd_weight[8];
 };
 inline Tuning MakeTuning(const yahkv_decode_options* o) {
@@ -354,8 +402,9 @@ inline Tuning MakeTuning(const yahkv_decode_options* o) {
                                                              : 2 * kWavesPerGroup;
   t.pair_cost = o == nullptr || o->pair_cost == 0 ? 8 : std::min(std::max(o->pair_cost, 0), 1 << 10);
   t.reduce_split = o != nullptr ? std::max(o->reduce_split, 0) : 0;
-  t.deterministic = o != nullptr && o->deterministic != 0;
+  t.deterministic = o == nullptr || o->deterministic >= 0;  // (negative: tiles first come, first served)
   t.one_launch = o != nullptr && o->one_launch != 0;
+  t.wg_partials = o != nullptr ? o->wg_partials : 0;
   for (int j = 0; j < 8; ++j) t.xcd_weight[j] = o != nullptr ? std::max(o->xcd_weight[j], 0) : 0;
   return t;
 }
@@ -425,6 +474,9 @@ inline int Prepare(const Geom& m, int32_t page_table_stride, const int32_t* seq_
   a->acc = reinterpret_cast<float*>(ws + p.off_acc);
   a->n_chunks = p.n_chunks, a->wpc = p.wpc, a->min_chunk_tiles = p.min_chunk_tiles, a->pair_cost = p.pair_cost;
   a->deterministic = t.deterministic;
+  // One partial per workgroup for a chunk's last pair pays where chunks are short (a small batch: few tiles per wave, so
+  // a wave's partial is a large part of what it moves) and costs two barriers at the kernel's end where they are long.
+  a->wg_partials = t.wg_partials == 1 ? 1 : t.wg_partials == 2 ? 0 : (int64_t(p.max_len) + kTile - 1) / kTile * n_seqs * m.n_kv <= int64_t(p.n_chunks) * kWavesPerGroup * 4;
   std::copy(p.share, p.share + 9, a->share);
   return YAHKV_OK;
 }

@@ -47,6 +47,7 @@ void Kv8Part(const DecodeArgs a, const Kv8Pools pools) {
   __shared__ __align__(16) _Float16 lp_all[kWavesPerGroup][kMaxGroup][kTile];
   __shared__ __align__(16) uint8_t lk_all[kWavesPerGroup][32 * 256];  // 32 key rows, chunks swizzled by row
   __shared__ int next_tile;
+  __shared__ int progress[kWavesPerGroup];  // tiles each wave is through with (fixed pattern only)
   __shared__ int wave_sum[kWavesPerGroup][2];
   __shared__ int4 chunk_rec;
   __shared__ long long chunk_tiles[4];
@@ -57,14 +58,36 @@ void Kv8Part(const DecodeArgs a, const Kv8Pools pools) {
 
   if (a.stamps != nullptr && threadIdx.x == 0) a.stamps[blockIdx.x] = wall_clock64();
   bool any_empty = false;
-  const int4 rec = ChunkRecord<64 * kWavesPerGroup>(a, blockIdx.x, wave_sum, &chunk_rec, chunk_tiles, &any_empty);
+  const int4 rec_v = a.n_seqs <= 64 ? ChunkRecordWave(a, blockIdx.x, wave, lane, &chunk_rec, chunk_tiles, &any_empty)
+                                    : ChunkRecord<64 * kWavesPerGroup>(a, blockIdx.x, wave_sum, &chunk_rec, chunk_tiles, &any_empty);
+  // (the record is the same in every lane: scalar registers for it and for everything derived from it)
+  const int4 rec = {__builtin_amdgcn_readfirstlane(rec_v.x), __builtin_amdgcn_readfirstlane(rec_v.y),
+                    __builtin_amdgcn_readfirstlane(rec_v.z), __builtin_amdgcn_readfirstlane(rec_v.w)};
   if (rec.x < 0) return;
   const int chunk_n = rec.w;
-  if (threadIdx.x == 0) next_tile = 0;
-  __syncthreads();
+  const bool fixed_pattern = a.deterministic || chunk_n <= kWavesPerGroup;  // (at most one tile per wave: no hand-out)
+  if (!fixed_pattern) {
+    if (threadIdx.x == 0) next_tile = 0;
+    __syncthreads();
+  }
   int my_next = wave;
+  // (see decode.hip: with a fixed pattern the two waves of a SIMD pace each other through their priorities)
+  int done_tiles = 0;
+  if (lane == 0) progress[wave] = 0;
+  auto pace = [&]() {
+    if (!fixed_pattern) return;
+    ++done_tiles;
+    int other = 0;
+    if (lane == 0) {
+      __hip_atomic_store(&progress[wave], done_tiles, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      other = __hip_atomic_load(&progress[wave ^ 4], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+    other = __builtin_amdgcn_readfirstlane(other);
+    if (done_tiles < other) __builtin_amdgcn_s_setprio(2);
+    else __builtin_amdgcn_s_setprio(0);
+  };
   auto take = [&]() -> int {
-    if (a.deterministic) {
+    if (fixed_pattern) {
       const int v = my_next;
       my_next += kWavesPerGroup;
       return v;
@@ -294,6 +317,7 @@ void Kv8Part(const DecodeArgs a, const Kv8Pools pools) {
       fetch_v(tile, 1, pgc);
       idx = nidx;
       ptile = tile;
+      pace();
       if (!has_next) break;
       tile = ntile;
       pgc = pgn;
