@@ -651,14 +651,13 @@ constexpr int VmCnt(int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); }
 
 // Same work split as the fused kernel: 4 waves, 64 chunk positions x RB heads, RB row blocks of 16 queries per wave,
 // everything transposed (keys along MFMA rows, queries along lanes). LDS holds two tile images.
-template <int D, int RB>
+template <int D, int RB, int KP = 1, int VP = 6>
 __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, const char* img, int tiles_per_pair) {
   constexpr int KS = D / 32, NDT = D / 16, kHeadsPerGroup = RB;
   constexpr int KIMG = kKeys * D * 2, TIMG = TileImageBytes<D>();
   constexpr int kCopies = TIMG / 1024 / 4;  // 1 KB wave-wide copies per wave and tile
   // How far the operand reads run ahead of the products that use them, in steps of the first product (8 matrix
   // instructions each) and in 16-dim tiles of the second (4 each). Measured: 1 and 6 (2 and 2: 3 % slower).
-  constexpr int KP = 1, VP = 6;
   static_assert(kCopies == KS + NDT / 2, "one copy per step of the first product and per two of the second");
   const Geom g = a.g;
   const int G = g.group(), H = g.n_kv;
@@ -1061,12 +1060,14 @@ extern "C" int yahkv_prefill_attend_tiles(const yahkv_geometry* g, const yahkv_p
   if (const int rc = CheckWorkspace(a, workspace, workspace_bytes)) return rc;
   const char* img = static_cast<const char*>(workspace);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  // At head_dim 128, three row blocks per wave (three heads per workgroup) when the GQA group is a multiple of
-  // three: each tile image copied to LDS and each operand read from it then serves half as much arithmetic again.
-  // (At head_dim 256 three blocks' accumulators and query operands do not fit the register file: 140 spills.)
+  // Three row blocks per wave (three heads per workgroup) when the GQA group is a multiple of three: each tile image
+  // copied to LDS and each operand read from it then serves half as much arithmetic again. At head_dim 256 that is 504 of
+  // the wave's 512 registers (192 + 96 accumulation registers for O^T and two S^T, 96 for the queries' operands), no
+  // spills, and worth 2 - 3 % of the kernel's time against two row blocks.
 #define YAHKV_LAUNCH_ATT(DD, RR) \
   hipLaunchKernelGGL((PrefillAttendImg<DD, RR>), AttendGrid(a, RR), dim3(256), 0, st, a, img, tiles)
-  if (a.g.hd == 256) YAHKV_LAUNCH_ATT(256, 2);
+  if (a.g.hd == 256 && a.g.group() % 3 == 0) YAHKV_LAUNCH_ATT(256, 3);
+  else if (a.g.hd == 256) YAHKV_LAUNCH_ATT(256, 2);
   else if (a.g.group() % 3 == 0) YAHKV_LAUNCH_ATT(128, 3);
   else YAHKV_LAUNCH_ATT(128, 2);
 #undef YAHKV_LAUNCH_ATT
@@ -1179,7 +1180,8 @@ extern "C" int yahkv_f16_prefill_attend(const yahkv_geometry* g, const yahkv_f16
   const char* img = static_cast<const char*>(workspace);
 #define YAHKV_LAUNCH_ATT(DD, RR) \
   hipLaunchKernelGGL((PrefillAttendImg<DD, RR>), AttendGrid(a, RR), dim3(256), 0, st, a, img, tiles)
-  if (a.g.hd == 256) YAHKV_LAUNCH_ATT(256, 2);
+  if (a.g.hd == 256 && a.g.group() % 3 == 0) YAHKV_LAUNCH_ATT(256, 3);
+  else if (a.g.hd == 256) YAHKV_LAUNCH_ATT(256, 2);
   else if (a.g.group() % 3 == 0) YAHKV_LAUNCH_ATT(128, 3);
   else YAHKV_LAUNCH_ATT(128, 2);
 #undef YAHKV_LAUNCH_ATT
@@ -1220,7 +1222,9 @@ extern "C" int yahkv_kv8_prefill_attend(const yahkv_geometry* g, const yahkv_kv8
   hipLaunchKernelGGL(PrefillImagesKv8<0>, dim3(static_cast<unsigned>(tiles), static_cast<unsigned>(n_seqs * a.g.n_kv)),
                      dim3(256), 0, st, ia);
   if (const int rc = LaunchStatus()) return rc;
-  hipLaunchKernelGGL((PrefillAttendImg<256, 2>), AttendGrid(a, 2), dim3(256), 0, st, a,
-                     static_cast<const char*>(workspace), tiles);
+  if (a.g.group() % 3 == 0)
+    hipLaunchKernelGGL((PrefillAttendImg<256, 3>), AttendGrid(a, 3), dim3(256), 0, st, a, static_cast<const char*>(workspace), tiles);
+  else
+    hipLaunchKernelGGL((PrefillAttendImg<256, 2>), AttendGrid(a, 2), dim3(256), 0, st, a, static_cast<const char*>(workspace), tiles);
   return LaunchStatus();
 }
