@@ -42,6 +42,7 @@ WORKLOADS = {
     # the reference's own KV format (kv8a16: 2336 B per token, 256-token pages), the same ragged batch
     "ragged_b64_kv8a16": dict(fmt=816, batch=64, lo=1024, hi=65536, seed=4),
     "b1_ctx32k_kv8a16": dict(fmt=816, batch=1, lo=32768, hi=32768, seed=4, layers=8),
+    "prefill_b8_ctx16k_chunk2k_kv8a16": dict(fmt=816, batch=8, lo=16384, hi=16384, seed=4, chunk=2048, warmup=10),
 }
 MFMA_F16_PEAK_TFLOPS = 2500.0
 EVENT_EVERY = 4      # decode workloads: HIP events around the split-K kernel on every fourth timed step
@@ -487,6 +488,104 @@ def run_kv8(a, wl, torch, yahkv):
         "cpu_baseline": None}
 
 
+def run_prefill_kv8(a, wl, torch, yahkv):
+    """The prefill step on kv8a16 pools: quantize + scatter the chunk (K rows around the sequence's channel means, V in
+    16-key tiles), then one call that decodes prefix + chunk to f16 tile images and runs the causal attention."""
+    B, chunk, prefix, PG = wl["batch"], wl["chunk"], wl["lo"], 256
+    per_seq = (prefix + chunk + PG - 1) // PG
+    g = yahkv.kv8_geometry(NQ, NKV, B * per_seq)
+    alloc = yahkv.PagePool(g.n_pages)
+    alloc.shuffle(12345)
+    table = np.stack([alloc.alloc(per_seq) for _ in range(B)]).astype(np.int32)
+    pools = yahkv.Kv8Pools(g)
+    t_table = torch.from_numpy(table).cuda()
+    gen = torch.Generator(device="cuda").manual_seed(wl["seed"])
+    for s in range(B):
+        for o in range(0, prefix, 8192):
+            n = min(8192, prefix - o)
+            k = (torch.randn((1, n, NKV, HD), generator=gen, device="cuda") + 0.5).to(torch.bfloat16)
+            v = torch.randn((1, n, NKV, HD), generator=gen, device="cuda").to(torch.bfloat16)
+            if o == 0:
+                yahkv.kv8_kmean(pools, t_table[s:s + 1], k)
+            yahkv.kv8_append(pools, t_table[s:s + 1], torch.tensor([o], dtype=torch.int32, device="cuda"), k, v)
+    scale = 1.0 / float(np.sqrt(HD))
+    t_prefix = torch.full((B,), prefix, dtype=torch.int32, device="cuda")
+    q = torch.randn((B, chunk, NQ, HD), generator=gen, device="cuda").to(torch.bfloat16)
+    knew = (torch.randn((B, chunk, NKV, HD), generator=gen, device="cuda") + 0.5).to(torch.bfloat16)
+    vnew = torch.randn((B, chunk, NKV, HD), generator=gen, device="cuda").to(torch.bfloat16)
+    out = torch.empty(q.shape, dtype=torch.float16, device="cuda")
+    ws = torch.empty(yahkv.lib.yahkv_kv8_prefill_workspace_bytes(g, B, prefix, chunk), dtype=torch.uint8, device="cuda")
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(a.steps)]
+    ev_app = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(a.steps)]
+
+    def step(pair=None, app=None):
+        if app:
+            app[0].record()
+        yahkv.kv8_append(pools, t_table, t_prefix, knew, vnew)
+        if app:
+            app[1].record()
+        if pair:
+            pair[0].record()
+        yahkv.kv8_prefill_attend(pools, t_table, t_prefix, prefix, q, scale, out=out, workspace=ws)
+        if pair:
+            pair[1].record()
+
+    # parity before timing: float64 closed form over the oracle's model of what the prefill kernels decode (f16 values)
+    step()
+    torch.cuda.synchronize()
+    first_hash = fnv1a(out.view(torch.int16).cpu().numpy().tobytes())
+    from oracle import kv8 as okv8
+    n = prefix + chunk
+    err = 0.0
+    for s_ in (0, B - 1):
+        hp, row = okv8.pools_of_sequence(pools, table[s_], n)
+        Kd, Vd = okv8.dense(hp, row, n, as_f16=True)
+        for t in (0, 1, chunk // 3, chunk // 2, chunk - 65, chunk - 1):
+            for h in (0, 7, 13, NQ - 1):
+                kv = h // (NQ // NKV)
+                qv = q[s_, t, h].float().cpu().numpy().astype(np.float64)
+                sc = Kd[:prefix + t + 1, kv].astype(np.float64) @ qv * scale
+                p = np.exp(sc - sc.max())
+                want = (p / p.sum()) @ Vd[:prefix + t + 1, kv].astype(np.float64)
+                got = out[s_, t, h].float().cpu().numpy()
+                err = max(err, float(np.abs(got - want).max() / np.abs(want).max()))
+    if not err < 2e-3:
+        raise SystemExit(f"bench.py: parity check failed before timing: max relative error {err:.3e}")
+    for _ in range(a.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(a.steps):
+        step(ev[i], ev_app[i])
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / a.steps * 1e3
+    kern_ms = float(np.mean([p[0].elapsed_time(p[1]) for p in ev]))
+    app_ms = float(np.median([p[0].elapsed_time(p[1]) for p in ev_app]))
+    app_bytes = B * chunk * (2 * NKV * HD * 2 + NKV * 2336)      # bf16 rows in, codes + scales + stats out
+    flops = float(B) * NQ * chunk * (prefix + (chunk + 1) / 2) * HD * 4
+    return {
+        "metric": "chunked-prefill attention over paged kv8a16 KV, TFLOP/s (f16 MFMA) + tok/s",
+        "value": round(flops / (ms * 1e-3) / 1e12, 1), "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps,
+        "warmup": a.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": a.workload, "batch": B, "prefix": prefix, "chunk": chunk, "n_q_heads": NQ,
+                   "n_kv_heads": NKV, "head_dim": HD, "page_tokens": PG, "n_pages": g.n_pages, "kv_format": "kv8a16",
+                   "step": "append chunk (quantize + scatter) + decode tiles to f16 + causal attention"},
+        "tok_per_s": round(B * chunk / (ms * 1e-3), 1), "flops_per_step": int(flops),
+        "parity_max_rel_err": float(f"{err:.3e}"), "out_fnv1a": first_hash,
+        "append": {"kernel": "Kv8AppendRowsK + Kv8AppendTilesV", "ms": round(app_ms, 4), "bytes": int(app_bytes),
+                   "GB/s": round(app_bytes / (app_ms * 1e-3) / 1e9, 1),
+                   "frac_of_hbm_peak": round(app_bytes / (app_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                   "note": "quantize + scatter of the chunk, HIP events around the call (median)"},
+        "roofline": {"bound": "mfma", "achieved": round(flops / (kern_ms * 1e-3) / 1e12, 1),
+                     "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(flops / (kern_ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
+                     "traffic": TRAFFIC.get(a.workload, (None, None))[0],
+                     "traffic_source": TRAFFIC.get(a.workload, (None, None))[1],
+                     "kernel": "PrefillImagesKv8<0> + PrefillAttendImg<%d, 3>" % HD, "kernel_ms": round(kern_ms, 4)},
+        "cpu_baseline": None}
+
+
 def run_prefill(a, wl, torch, yahkv):
     """A step: quantize + scatter one chunk per sequence, decode prefix + chunk to f16 tiles, causal attention."""
     g, layers, lens, table, t_table, gen = build_state(yahkv, torch, wl, 0)
@@ -699,6 +798,11 @@ def run_decode(a, wl, torch, yahkv):
     if a.first_come:
         opt.deterministic = -1
     ws = torch.empty(yahkv.decode_workspace_bytes(g, B, max_len, opt), dtype=torch.uint8, device="cuda")
+    # which instance of the part kernel the library picks (its last template argument): 1 merges in the same launch,
+    # 2 leaves one partial per workgroup for a chunk's last pair (the library's rule for a batch with few tiles per wave)
+    chunks = torch.cuda.get_device_properties(0).multi_processor_count
+    few_tiles = -(-max_len // 64) * B * NKV <= chunks * 8 * 4
+    part_mode = 1 if a.one_launch else 2 if a.wg_partials == 1 or (a.wg_partials == 0 and few_tiles) else 0
     # set-up, as a server does once: the XCDs' relative read speeds on this batch (equal shares without it)
     xcd = yahkv.decode_calibrate(pools, t_table, len_rows[0], max_len, q, ws, opt, rounds=3) if not a.no_calibrate else None
     if a.one_launch:
@@ -781,7 +885,7 @@ def run_decode(a, wl, torch, yahkv):
         "roofline": {"bound": "hbm", "achieved": round(kgbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(kgbs / HBM_PEAK_GBS, 4), "traffic": TRAFFIC.get(a.workload, (None, None))[0],
                      "traffic_source": TRAFFIC.get(a.workload, (None, None))[1],
-                     "kernel": "DattnPart<%d, %d, %d, %s>" % (wl["fmt"], HD, PT, "true" if a.one_launch else "false"),
+                     "kernel": "DattnPart<%d, %d, %d, %d>" % (wl["fmt"], HD, PT, part_mode),
                      "kernel_ms": round(kern_ms, 4)},
     }
     # The same number of steps again, right after three idle seconds and without warm-up: what a server's first steps
@@ -831,6 +935,8 @@ def run_workload(a, torch, yahkv):
     wl = WORKLOADS[a.workload]
     if "chunk" in wl and wl["fmt"] == 16:
         return run_prefill_f16(a, wl, torch, yahkv)
+    if "chunk" in wl and wl["fmt"] == 816:
+        return run_prefill_kv8(a, wl, torch, yahkv)
     if "chunk" in wl:
         return run_prefill(a, wl, torch, yahkv)
     if wl["fmt"] == 16:
