@@ -484,7 +484,7 @@ def run_kv8(a, wl, torch, yahkv):
         "roofline": {"bound": "hbm", "achieved": round(kgbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(kgbs / HBM_PEAK_GBS, 4), "traffic": TRAFFIC.get(a.workload, (None, None))[0],
                      "traffic_source": TRAFFIC.get(a.workload, (None, None))[1],
-                     "kernel": "Kv8Part", "kernel_ms": round(kern_ms, 4)},
+                     "kernel": "Kv8Part<0>", "kernel_ms": round(kern_ms, 4)},
         "cpu_baseline": None}
 
 
@@ -582,7 +582,7 @@ def run_prefill_kv8(a, wl, torch, yahkv):
                      "frac": round(flops / (kern_ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
                      "traffic": TRAFFIC.get(a.workload, (None, None))[0],
                      "traffic_source": TRAFFIC.get(a.workload, (None, None))[1],
-                     "kernel": "PrefillImagesKv8<0> + PrefillAttendImg<%d, 3>" % HD, "kernel_ms": round(kern_ms, 4)},
+                     "kernel": "PrefillImagesKv8<0> + PrefillAttendImg<%d, 3, 1, 6>" % HD, "kernel_ms": round(kern_ms, 4)},
         "cpu_baseline": None}
 
 
@@ -681,7 +681,7 @@ def run_prefill(a, wl, torch, yahkv):
                      "traffic": None if a.one_pass else TRAFFIC.get(a.workload, (None, None))[0],
                      "traffic_source": None if a.one_pass else TRAFFIC.get(a.workload, (None, None))[1],
                      "kernel": ("PrefillAttendFused<%d, %d, %d>" % (wl["fmt"], HD, PT) if a.one_pass
-                                else "PrefillAttendImg<%d, 3>" % HD), "kernel_ms": round(kern_ms, 4)},
+                                else "PrefillAttendImg<%d, 3, 1, 6>" % HD), "kernel_ms": round(kern_ms, 4)},
     }
     if a.clock_trace:
         res["clock_trace"] = clock_trace(
@@ -770,7 +770,7 @@ def run_prefill_f16(a, wl, torch, yahkv):
                      "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(flops / (kern_ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
                      "traffic": None, "traffic_source": None,
-                     "kernel": "PrefillImagesF16<%d, %d> + PrefillAttendImg<%d, 3>" % (HD, PT, HD),
+                     "kernel": "PrefillImagesF16<%d, %d> + PrefillAttendImg<%d, 3, 1, 6>" % (HD, PT, HD),
                      "kernel_ms": round(kern_ms, 4)},
         "cpu_baseline": None}
 

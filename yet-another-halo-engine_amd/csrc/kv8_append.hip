@@ -88,7 +88,15 @@ __global__ __launch_bounds__(256) void Kv8Kmean(const Kv8AppendArgs a) {
   const int n = min(a.n_new, max(valid, 1));
   __shared__ float part[8][32];
   float acc = 0.0f;
-  for (int r = grp; r < n; r += 8) acc = acc + TruncF16(LoadSrc(a.k_src, (size_t(s) * a.n_new + r) * W + c, a.dtype));
+  int r = grp;
+  for (; r + 8 * 15 < n; r += 8 * 16) {  // sixteen loads in flight, added in the rows' order
+    float x[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) x[j] = LoadSrc(a.k_src, (size_t(s) * a.n_new + r + 8 * j) * W + c, a.dtype);
+#pragma unroll
+    for (int j = 0; j < 16; ++j) acc = acc + TruncF16(x[j]);
+  }
+  for (; r < n; r += 8) acc = acc + TruncF16(LoadSrc(a.k_src, (size_t(s) * a.n_new + r) * W + c, a.dtype));
   part[grp][cc] = acc;
   __syncthreads();
   if (grp == 0) {
