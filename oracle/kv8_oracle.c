@@ -117,6 +117,104 @@ void orc_kv8_deq_vtile(const uint32_t* dw, const uint16_t* st, int32_t n, float*
   }
 }
 
+/* ---- kv4a16 ----------------------------------------------------------------------------------------------------------- */
+
+void orc_kv4_hadamard256(float* x) {
+  for (int h = 1; h < 256; h <<= 1)
+    for (int i = 0; i < 256; ++i)
+      if (!(i & h)) {
+        const float a = x[i], b = x[i ^ h];
+        x[i] = a + b;
+        x[i ^ h] = a - b;
+      }
+}
+
+void orc_kv4_quant_k(const float* k, const float* mean, int32_t n_heads, uint32_t* dw, uint16_t* sc) {
+  for (int hd = 0; hd < n_heads; ++hd) {
+    float x[256];
+    for (int i = 0; i < 256; ++i) x[i] = trunc_f16(k[hd * 256 + i]) - mean[hd * 256 + i];
+    orc_kv4_hadamard256(x);
+    for (int i = 0; i < 256; ++i) x[i] = x[i] * 0.0625f; /* 1 / sqrt(256) */
+    for (int g = 0; g < 8; ++g) {
+      const float* xr = x + 32 * g;
+      float lo = xr[0], hi = xr[0];
+      for (int i = 1; i < 32; ++i) lo = fminf(lo, xr[i]), hi = fmaxf(hi, xr[i]);
+      const float s0 = (hi - lo) / 15.0f;
+      const float s = s0 > 0.0f ? s0 : 1.0f;
+      const float inv = 1.0f / s;
+      for (int c = 0; c < 4; ++c) {
+        uint32_t w = 0;
+        for (int i = 0; i < 8; ++i) {
+          const float r = fminf(fmaxf(rintf((xr[8 * c + i] - lo) * inv), 0.0f), 15.0f);
+          w |= (code_of(r) & 15u) << (4 * (i / 2) + (i % 2 ? 16 : 0));
+        }
+        dw[hd * 32 + g * 4 + c] = w;
+      }
+      const float S0 = s * 16.0f;
+      sc[2 * (hd * 8 + g)] = orc_f32_to_f16(S0);
+      sc[2 * (hd * 8 + g) + 1] = orc_f32_to_f16(lo - S0);
+    }
+  }
+}
+
+void orc_kv4_deq_k(const uint32_t* dw, const uint16_t* sc, int32_t n_heads, float* out) {
+  for (int g = 0; g < n_heads * 8; ++g) {
+    const float S = orc_f16_to_f32(sc[2 * g]), C = orc_f16_to_f32(sc[2 * g + 1]);
+    const float d = S / 16.0f, lo = C + S;
+    for (int c = 0; c < 4; ++c)
+      for (int i = 0; i < 8; ++i) {
+        const float u = (float)((dw[g * 4 + c] >> (4 * (i / 2) + (i % 2 ? 16 : 0))) & 15u);
+        out[g * 32 + 8 * c + i] = u * d + lo;
+      }
+  }
+}
+
+static int key_of_nibble4(int w, int p) { return 8 * w + (p < 4 ? 2 * p : 2 * (p - 4) + 1); }
+
+void orc_kv4_quant_vtile(const uint16_t* v, int32_t n, uint32_t* dw, uint16_t* st) {
+  for (int c = 0; c < n; ++c) {
+    float x[16], mx, mn;
+    for (int j = 0; j < 16; ++j) x[j] = orc_f16_to_f32(v[j * n + c]);
+    mx = mn = x[0];
+    for (int j = 1; j < 16; ++j) mx = fmaxf(mx, x[j]), mn = fminf(mn, x[j]);
+    const float cen = (mx + mn) * 0.5f;
+    const float s0 = (mx - mn) / 14.0f;
+    const float s = s0 > 0.0f ? s0 : 1.0f;
+    const float sf = trunc_f16(s), cf = trunc_f16(cen);
+    const float inv = 1.0f / sf;
+    for (int w = 0; w < 2; ++w) {
+      uint32_t word = 0;
+      for (int p = 0; p < 8; ++p) {
+        const float q = (x[key_of_nibble4(w, p)] - cf) * inv;
+        const float r = fminf(fmaxf(rintf(q) + 7.0f, 0.0f), 14.0f);
+        word |= (code_of(r) & 15u) << (4 * p);
+      }
+      dw[c * 2 + w] = word;
+    }
+    st[2 * c] = orc_f32_to_f16(sf * 16.0f);
+    st[2 * c + 1] = orc_f32_to_f16(cf + sf * -23.0f); /* sf * 23 is exact in f32 (sf has 11 bits) */
+  }
+}
+
+void orc_kv4_deq_vtile(const uint32_t* dw, const uint16_t* st, int32_t n, float* out) {
+  for (int c = 0; c < n; ++c) {
+    const float S = orc_f16_to_f32(st[2 * c]), Cp = orc_f16_to_f32(st[2 * c + 1]);
+    const float d = S / 16.0f;
+    for (int w = 0; w < 2; ++w)
+      for (int p = 0; p < 8; ++p) {
+        const float u = (float)((dw[c * 2 + w] >> (4 * p)) & 15u);
+        out[key_of_nibble4(w, p) * n + c] = (u * d + S) + Cp;
+      }
+  }
+}
+
+void orc_kv4_rotate_q(const float* q, float* out) {
+  float x[256];
+  memcpy(x, q, sizeof(x));
+  orc_kv4_hadamard256(x);
+  for (int i = 0; i < 256; ++i) out[i] = x[i] * 0.0625f;
+}
+
 void orc_kv8_kmean(const float* k, int32_t n_rows, int32_t W, float* mean) {
   for (int c = 0; c < W; ++c) {
     float grp[8];
@@ -131,6 +229,10 @@ void orc_kv8_kmean(const float* k, int32_t n_rows, int32_t W, float* mean) {
   }
 }
 
+static int kq_row_dwords(const orc_kv8_geometry* g) { return g->n_kv_heads * (g->k_bits == 4 ? 32 : 64); }
+static int ks_row_dwords(const orc_kv8_geometry* g) { return g->n_kv_heads * (g->k_bits == 4 ? 8 : 2); }
+static int vq_dwords(const orc_kv8_geometry* g) { return g->v_bits == 4 ? 2 : 4; } /* per (tile, dim) */
+
 static int page_of(const orc_kv8_geometry* g, const int32_t* row, int32_t pos) {
   int pg = row[pos / 256];
   if (pg < 0) pg = 0;
@@ -142,11 +244,13 @@ static int page_of(const orc_kv8_geometry* g, const int32_t* row, int32_t pos) {
 static void store_vtile(const orc_kv8_geometry* g, const orc_kv8_pools* p, const uint16_t* tile, int pt) {
   const int H = g->n_kv_heads, W = H * 256;
   const size_t tiles = (size_t)g->n_pages * 16;
+  const size_t nw = (size_t)vq_dwords(g);
   uint32_t* dw = (uint32_t*)malloc(sizeof(uint32_t) * (size_t)W * 4);
   uint16_t* st = (uint16_t*)malloc(sizeof(uint16_t) * (size_t)W * 2);
-  orc_kv8_quant_vtile(tile, W, dw, st);
+  if (g->v_bits == 4) orc_kv4_quant_vtile(tile, W, dw, st);
+  else orc_kv8_quant_vtile(tile, W, dw, st);
   for (int h = 0; h < H; ++h) {
-    memcpy(p->vq + (((size_t)h * tiles + (size_t)pt) * 256) * 4, dw + (size_t)h * 256 * 4, sizeof(uint32_t) * 256 * 4);
+    memcpy(p->vq + (((size_t)h * tiles + (size_t)pt) * 256) * nw, dw + (size_t)h * 256 * nw, sizeof(uint32_t) * 256 * nw);
     memcpy(p->vs + ((size_t)h * tiles + (size_t)pt) * 256, st + (size_t)h * 256 * 2, sizeof(uint32_t) * 256);
   }
   free(dw);
@@ -172,8 +276,10 @@ void orc_kv8_append(const orc_kv8_geometry* g, const orc_kv8_pools* p, const int
     const float* mean = p->km + (size_t)page_of(g, row, 0) * W;
     for (int64_t i = 0; i < nv; ++i) {
       const int64_t pos = p0 + i, r = (int64_t)page_of(g, row, (int32_t)pos) * 256 + pos % 256;
-      orc_kv8_quant_k(ks + (size_t)i * W, mean, W / 128, p->kq + (size_t)r * (W / 4),
-                      (uint16_t*)(p->ks + (size_t)r * (W / 128)));
+      uint32_t* dw = p->kq + (size_t)r * kq_row_dwords(g);
+      uint16_t* sc = (uint16_t*)(p->ks + (size_t)r * ks_row_dwords(g));
+      if (g->k_bits == 4) orc_kv4_quant_k(ks + (size_t)i * W, mean, H, dw, sc);
+      else orc_kv8_quant_k(ks + (size_t)i * W, mean, W / 128, dw, sc);
     }
     if (n_new == 1) { /* the decoder's vappend */
       const int pg = page_of(g, row, (int32_t)p0), key = (int)(p0 % 16);
@@ -220,10 +326,20 @@ static void dense(const orc_kv8_geometry* g, const orc_kv8_pools* p, const int32
   float out[16 * 256];
   for (int pos = 0; pos < n; ++pos) {
     const size_t r = (size_t)page_of(g, row, pos) * 256 + (size_t)(pos % 256);
-    const uint32_t* dw = p->kq + r * (W / 4);
-    const uint16_t* sc = (const uint16_t*)(p->ks + r * (W / 128));
-    if (!as_f16) {
+    const uint32_t* dw = p->kq + r * kq_row_dwords(g);
+    const uint16_t* sc = (const uint16_t*)(p->ks + r * ks_row_dwords(g));
+    if (!as_f16 && g->k_bits == 4) {
+      orc_kv4_deq_k(dw, sc, H, Kd + (size_t)pos * W);
+    } else if (!as_f16) {
       orc_kv8_deq_k(dw, sc, W / 128, Kd + (size_t)pos * W);
+    } else if (g->k_bits == 4) { /* yah_kdeq4: f16(1 + u / 16) * S + C, one f16 fma (gen_attn_fa.py:4652-4700) */
+      for (int i = 0; i < W / 8; ++i)
+        for (int e = 0; e < 8; ++e) {
+          const double f = 1.0 + (double)((dw[i] >> (4 * (e / 2) + (e % 2 ? 16 : 0))) & 15u) / 16.0;
+          const int gi = (8 * i) / 32;
+          const double v = fma(f, (double)orc_f16_to_f32(sc[2 * gi]), (double)orc_f16_to_f32(sc[2 * gi + 1]));
+          Kd[(size_t)pos * W + 8 * i + e] = orc_f16_to_f32(f64_to_f16(v));
+        }
     } else {
       for (int i = 0; i < W / 4; ++i)
         for (int b = 0; b < 4; ++b) {
@@ -244,10 +360,20 @@ static void dense(const orc_kv8_geometry* g, const orc_kv8_pools* p, const int32
           for (int c = 0; c < 256; ++c) Vd[(size_t)(16 * t + j) * W + h * 256 + c] = orc_f16_to_f32(vo[(size_t)c * 16 + j]);
         continue;
       }
-      const uint32_t* dw = p->vq + (((size_t)h * tiles + (size_t)pt) * 256) * 4;
+      const uint32_t* dw = p->vq + (((size_t)h * tiles + (size_t)pt) * 256) * (size_t)vq_dwords(g);
       const uint16_t* st = (const uint16_t*)(p->vs + ((size_t)h * tiles + (size_t)pt) * 256);
-      if (!as_f16) {
+      if (!as_f16 && g->v_bits == 4) {
+        orc_kv4_deq_vtile(dw, st, 256, out);
+      } else if (!as_f16) {
         orc_kv8_deq_vtile(dw, st, 256, out);
+      } else if (g->v_bits == 4) { /* yah_vdeq4: f16(1 + u / 16) * S + C' */
+        for (int c = 0; c < 256; ++c)
+          for (int w = 0; w < 2; ++w)
+            for (int pn = 0; pn < 8; ++pn) {
+              const double f = 1.0 + (double)((dw[c * 2 + w] >> (4 * pn)) & 15u) / 16.0;
+              const double v = fma(f, (double)orc_f16_to_f32(st[2 * c]), (double)orc_f16_to_f32(st[2 * c + 1]));
+              out[key_of_nibble4(w, pn) * 256 + c] = orc_f16_to_f32(f64_to_f16(v));
+            }
       } else {
         for (int c = 0; c < 256; ++c)
           for (int w = 0; w < 4; ++w)

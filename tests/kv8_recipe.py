@@ -15,17 +15,19 @@ def sha(a):
     return np.frombuffer(hashlib.sha256(np.ascontiguousarray(a).tobytes()).digest(), np.uint8)
 
 
-def golden():
-    return np.load(os.path.join(ROOT, "tests", "golden", "kv8a16_vectors.npz"), allow_pickle=False)
+def golden(bits=8):
+    return np.load(os.path.join(ROOT, "tests", "golden", "kv%da16_vectors.npz" % bits), allow_pickle=False)
 
 
 class Recipe:
     pass
 
 
-def load():
-    g = golden()
+def load(bits=8):
+    """bits = 4: the same draws (the checker's stream does not depend on the format) with kv4a16_vectors.npz's outputs"""
+    g = golden(bits)
     r = Recipe()
+    r.bits = bits
     r.g = g
     r.T, r.pos = int(g["rc_T"]), int(g["rc_pos"])
     rng = np.random.default_rng(5)
