@@ -65,7 +65,10 @@ typedef enum yahkv_format {
   YAHKV_Q4_0 = 4,
   YAHKV_Q8_0 = 8,
   YAHKV_KV_F16 = 16,   /* yahkv_f16_* functions only */
-  YAHKV_KV8A16 = 816   /* the reference's own format, "kv q 8 8": yahkv_kv8_* functions only */
+  YAHKV_KV8A16 = 816,  /* the reference's own format, "kv q 8 8": yahkv_kv8_* functions only */
+  YAHKV_KV4A16 = 416,  /* its 4-bit sibling, "kv q 4 4" (H256-rotated K, 16 levels; V 15 levels): yahkv_kv8_* functions */
+  YAHKV_K8V4A16 = 8416, /* "kv q 8 4": K as kv8a16, V as kv4a16 */
+  YAHKV_K4V8A16 = 4816  /* "kv q 4 8" */
 } yahkv_format;
 typedef enum yahkv_dtype { YAHKV_F32 = 0, YAHKV_F16 = 1, YAHKV_BF16 = 2 } yahkv_dtype;
 
@@ -410,7 +413,20 @@ int yahkv_f16_prefill_attend(const yahkv_geometry* g, const yahkv_f16_pools* poo
  *                                             gen_kvq.py:99-163); zero them for a sequence that starts with decode steps
  *   vopen  f16 [n_pages][W][16]               the open tile of the sequence whose NEWEST page this is: the keys of the
  *                                             sequence's last 16-key tile, unquantized (gen_decode_attn.py:436-573)
- * 2336 bytes per token (kq + ks + vq + vs; architecture.md:219). All buffers 16-byte aligned. */
+ * 2336 bytes per token (kq + ks + vq + vs; architecture.md:219). All buffers 16-byte aligned.
+ *
+ * kv4a16 (YAHKV_KV4A16, "kv q 4 4"; architecture.md:220, gen_kvq.py:288-463 and gen_vqt(4)) through the same functions:
+ *   kq     u32 [n_pages * 256][W / 8]         K - mean of a kv head rotated by the orthonormal 256-point Walsh-Hadamard
+ *                                             transform (f32 butterflies, stages 1 .. 128 in order, then / 16), 16 levels per
+ *                                             32-dim group: u = clamp(rne((x - lo) / s), 0, 15), s = (hi - lo) / 15; dims
+ *                                             2 j / 2 j + 1 of a dword's eight at bits 4 j / 16 + 4 j
+ *   ks     u32 [n_pages * 256][W / 32]        f16 pairs (16 s, lo - 16 s), index kv head * 8 + group
+ *   vq     u32 [H][n_pages * 16][256][2]      15 levels: u = clamp(rne((v - c) / s) + 7, 0, 14), s = range / 14; dword w
+ *                                             holds keys 8 w + (0, 2, 4, 6, 1, 3, 5, 7) at nibbles 0 .. 7
+ *   vs     u32 [H][n_pages * 16][256]         f16 pairs (16 s, c - 23 s)
+ * 1408 bytes per token. The attention rotates the queries the same way itself (yah_qrot / part_q's butterfly,
+ * gen_attn_fa.py:4541-4611, gen_decode_attn.py:655-683): callers pass plain queries. YAHKV_K8V4A16 and YAHKV_K4V8A16
+ * take K from one format and V from the other, as the reference's "kv q KB VB" allows (loom_decoder.hpp:4,76-79). */
 typedef struct yahkv_kv8_pools {
   void* kq;
   void* ks;

@@ -10,6 +10,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libyahkv.so")
 
 Q8_0, Q4_0, KV_F16, KV8A16 = 8, 4, 16, 816
+KV4A16, K8V4A16, K4V8A16 = 416, 8416, 4816
+_KV8_FORMATS = {(8, 8): KV8A16, (4, 4): KV4A16, (8, 4): K8V4A16, (4, 8): K4V8A16}
 F32, F16, BF16 = 0, 1, 2
 
 
@@ -583,10 +585,11 @@ def gather_blocks(pools, table_row, n_tokens):
 
 # ---- kv8a16: the reference's own KV format (yahkv_kv8_*) --------------------------------------------------------------
 
-def kv8_geometry(n_q_heads, n_kv_heads, n_pages):
-    g = Geometry(KV8A16, n_q_heads, n_kv_heads, 256, 256, n_pages)
+def kv8_geometry(n_q_heads, n_kv_heads, n_pages, k_bits=8, v_bits=8):
+    """The reference's own formats: kv8a16 (8, 8), kv4a16 (4, 4) and the mixes k8v4 / k4v8."""
+    g = Geometry(_KV8_FORMATS[(k_bits, v_bits)], n_q_heads, n_kv_heads, 256, 256, n_pages)
     if lib.yahkv_kv8_kq_bytes(C.byref(g)) == 0:
-        raise YahkvError(-2, "kv8a16 geometry")
+        raise YahkvError(-2, "kv8a16 / kv4a16 geometry")
     return g
 
 
@@ -598,8 +601,9 @@ class Kv8Pools:
 
     def __init__(self, g, fill=0, device="cuda:0"):
         import torch
-        assert g.format == KV8A16
+        assert g.format in _KV8_FORMATS.values()
         self.geom = g
+        self.k_bits, self.v_bits = next(kv for kv, f in _KV8_FORMATS.items() if f == g.format)
         for n in self.NAMES:
             nbytes = getattr(lib, f"yahkv_kv8_{n}_bytes")(C.byref(g))
             setattr(self, n, torch.full((nbytes,), fill, dtype=torch.uint8, device=device))
@@ -614,8 +618,10 @@ class Kv8Pools:
         g = self.geom
         H, P, W = g.n_kv_heads, g.n_pages, g.n_kv_heads * 256
         raw = {n: getattr(self, n).cpu().numpy() for n in self.NAMES}
-        return {"kq": raw["kq"].view(np.uint32).reshape(P * 256, W // 4), "ks": raw["ks"].view(np.uint32).reshape(P * 256, W // 128),
-                "km": raw["km"].view(np.float32).reshape(P, W), "vq": raw["vq"].view(np.uint32).reshape(H, P * 16, 256, 4),
+        kqw, ksw, vqw = (W // 8, W // 32) if self.k_bits == 4 else (W // 4, W // 128), None, 2 if self.v_bits == 4 else 4
+        kqw, ksw = kqw
+        return {"kq": raw["kq"].view(np.uint32).reshape(P * 256, kqw), "ks": raw["ks"].view(np.uint32).reshape(P * 256, ksw),
+                "km": raw["km"].view(np.float32).reshape(P, W), "vq": raw["vq"].view(np.uint32).reshape(H, P * 16, 256, vqw),
                 "vs": raw["vs"].view(np.uint32).reshape(H, P * 16, 256), "vo": raw["vopen"].view(np.uint16).reshape(P, W, 16)}
 
     def load(self, arrays):

@@ -79,7 +79,7 @@ namespace {
 int ValidateTable(const yahkv_geometry* g, const int32_t* table, int32_t page_table_stride, const int32_t* seq_len,
                   int32_t n_seqs, const std::vector<int32_t>* owners) {
   // (the reference's own format has its own geometry check: 256-token pages)
-  if (const int st = g != nullptr && g->format == YAHKV_KV8A16 ? yahkv::CheckKv8Geometry(g) : yahkv::CheckGeometry(g)) return st;
+  if (const int st = g != nullptr && yahkv::Kv8BitsK(g->format) != 0 ? yahkv::CheckKv8Geometry(g) : yahkv::CheckGeometry(g)) return st;
   if (table == nullptr || seq_len == nullptr || n_seqs <= 0 || page_table_stride <= 0) return YAHKV_ERR_ARG;
   std::vector<int32_t> used(static_cast<size_t>(g->n_pages), 0), row_of(static_cast<size_t>(g->n_pages), -1);
   for (int32_t s = 0; s < n_seqs; ++s) {

@@ -9,7 +9,7 @@ namespace yahkv {
 
 int CheckKv8Geometry(const yahkv_geometry* g) {
   if (g == nullptr) return YAHKV_ERR_ARG;
-  if (g->format != YAHKV_KV8A16) return YAHKV_ERR_SHAPE;
+  if (Kv8BitsK(g->format) == 0) return YAHKV_ERR_SHAPE;
   if (g->n_q_heads <= 0 || g->n_kv_heads <= 0 || g->n_pages <= 0) return YAHKV_ERR_ARG;
   if (g->n_q_heads % g->n_kv_heads != 0 || g->n_q_heads / g->n_kv_heads > 8) return YAHKV_ERR_SHAPE;
   if (g->head_dim != kKv8Dim || g->page_tokens != kKv8Page) return YAHKV_ERR_SHAPE;
@@ -77,6 +77,38 @@ __device__ __forceinline__ void Kv8StoreRowK(const Kv8Geom& g, const Kv8Pools& p
   p.kq[g.kq_row(row, h) + lane] = Kv8CodesK(c, inv);
   if (lane % 32 == 0) p.ks[g.ks_row(row, h) + lane / 32] = pair;
 }
+// the same for 4-bit K: rotated, 16 levels per 32-dim group (eight lanes), two lanes per dword
+__device__ __forceinline__ void Kv4StoreRowK(const Kv8Geom& g, const Kv8Pools& p, int page0, size_t row, int h, int lane,
+                                             float4 x) {
+#pragma clang fp contract(off)
+  const float4 m = *reinterpret_cast<const float4*>(p.km + g.km_head(page0, h) + 4 * lane);
+  const float4 c = {TruncF16(x.x) - m.x, TruncF16(x.y) - m.y, TruncF16(x.z) - m.z, TruncF16(x.w) - m.w};
+  uint32_t pair;
+  float4 deq;
+  uint32_t w = Kv4CodesK(c, lane, &pair, &deq);
+  w |= __shfl_xor(w, 1, 64);
+  if (lane % 2 == 0) p.kq[g.kq_row(row, h) + lane / 2] = w;
+  if (lane % 8 == 0) p.ks[g.ks_row(row, h) + lane / 8] = pair;
+}
+__device__ __forceinline__ void StoreRowK(const Kv8Geom& g, const Kv8Pools& p, int page0, size_t row, int h, int lane,
+                                          float4 x) {
+  if (g.kb == 4) Kv4StoreRowK(g, p, page0, row, h, lane, x);
+  else Kv8StoreRowK(g, p, page0, row, h, lane, x);
+}
+// a channel's 16 keys of a tile to their place among the codes and stats
+__device__ __forceinline__ void StoreTileV(const Kv8Geom& g, const Kv8Pools& p, int h, size_t pt, int d, const float (&x)[16]) {
+  uint32_t stats;
+  if (g.vb == 4) {
+    uint2 codes;
+    Kv4QuantTile(x, &codes, &stats);
+    *reinterpret_cast<uint2*>(p.vq + g.vq_tile(h, pt) + size_t(d) * 2) = codes;
+  } else {
+    uint4 codes;
+    Kv8QuantTile(x, &codes, &stats);
+    *reinterpret_cast<uint4*>(p.vq + g.vq_tile(h, pt) + size_t(d) * 4) = codes;
+  }
+  p.vs[g.vs_tile(h, pt) + d] = stats;
+}
 
 // yah_kmean: thread (row group, channel); eight row groups, each summing its rows in order, then the groups in order
 template <int DUMMY>
@@ -116,7 +148,7 @@ __global__ __launch_bounds__(64) void Kv8AppendToken(const Kv8AppendArgs a) {
   const int page = PageOf(a, s, pos), page0 = PageOf(a, s, 0);
   const size_t src = (size_t(s) * g.n_kv + h) * kKv8Dim + 4 * lane;
   const float4 k = Load4(a.k_src, src, a.dtype), v = Load4(a.v_src, src, a.dtype);
-  Kv8StoreRowK(g, a.p, page0, size_t(page) * kKv8Page + pos % kKv8Page, h, lane, k);
+  StoreRowK(g, a.p, page0, size_t(page) * kKv8Page + pos % kKv8Page, h, lane, k);
   // V: the token's key of the open tile; on the tile's 16th key the tile is quantized into its place
   const int key = pos % 16;
   uint16_t* vo = a.p.vo + g.vo_head(page, h) + size_t(4 * lane) * 16;
@@ -133,11 +165,7 @@ __global__ __launch_bounds__(64) void Kv8AppendToken(const Kv8AppendArgs a) {
 #pragma unroll
     for (int j = 0; j < 16; ++j) x[j] = WidenF16(static_cast<uint16_t>(w[j / 2] >> (16 * (j % 2))));
     x[15] = TruncF16(ve[e]);  // this lane's own store above
-    uint4 codes;
-    uint32_t stats;
-    Kv8QuantTile(x, &codes, &stats);
-    *reinterpret_cast<uint4*>(a.p.vq + g.vq_tile(h, pt) + size_t(4 * lane + e) * 4) = codes;
-    a.p.vs[g.vs_tile(h, pt) + 4 * lane + e] = stats;
+    StoreTileV(g, a.p, h, pt, 4 * lane + e, x);
   }
 }
 
@@ -150,7 +178,7 @@ __global__ __launch_bounds__(256) void Kv8AppendRowsK(const Kv8AppendArgs a) {
   const int pos = p0 + i, page = PageOf(a, s, pos), page0 = PageOf(a, s, 0);
   for (int h = wave; h < g.n_kv; h += 4) {
     const float4 k = Load4(a.k_src, ((size_t(s) * a.n_new + i) * g.n_kv + h) * kKv8Dim + 4 * lane, a.dtype);
-    Kv8StoreRowK(g, a.p, page0, size_t(page) * kKv8Page + pos % kKv8Page, h, lane, k);
+    StoreRowK(g, a.p, page0, size_t(page) * kKv8Page + pos % kKv8Page, h, lane, k);
   }
 }
 
@@ -182,12 +210,8 @@ __global__ __launch_bounds__(256) void Kv8AppendTilesV(const Kv8AppendArgs a) {
       x[j] = TruncF16(LoadSrc(a.v_src, ((size_t(s) * a.n_new + i) * g.n_kv + h) * kKv8Dim + d, a.dtype));
     }
   }
-  uint4 codes;
-  uint32_t stats;
-  Kv8QuantTile(x, &codes, &stats);
   const size_t pt = size_t(page) * 16 + t % 16;
-  *reinterpret_cast<uint4*>(a.p.vq + g.vq_tile(h, pt) + size_t(d) * 4) = codes;
-  a.p.vs[g.vs_tile(h, pt) + d] = stats;
+  StoreTileV(g, a.p, h, pt, d, x);
   if (t == last / 16) {  // yah_vseed: the newest tile stays open, keys past the last real token zero
     uint32_t w[8];
 #pragma unroll
@@ -221,15 +245,17 @@ using namespace yahkv;
 extern "C" {
 
 size_t yahkv_kv8_kq_bytes(const yahkv_geometry* g) {
-  return CheckKv8Geometry(g) ? 0 : size_t(g->n_pages) * kKv8Page * g->n_kv_heads * kKv8Dim;
+  return CheckKv8Geometry(g) ? 0 : size_t(g->n_pages) * kKv8Page * g->n_kv_heads * MakeKv8Geom(*g).kq_head() * 4;
 }
 size_t yahkv_kv8_ks_bytes(const yahkv_geometry* g) {
-  return CheckKv8Geometry(g) ? 0 : size_t(g->n_pages) * kKv8Page * g->n_kv_heads * 2 * 4;
+  return CheckKv8Geometry(g) ? 0 : size_t(g->n_pages) * kKv8Page * g->n_kv_heads * MakeKv8Geom(*g).ks_head() * 4;
 }
 size_t yahkv_kv8_km_bytes(const yahkv_geometry* g) {
   return CheckKv8Geometry(g) ? 0 : size_t(g->n_pages) * g->n_kv_heads * kKv8Dim * 4;
 }
-size_t yahkv_kv8_vq_bytes(const yahkv_geometry* g) { return yahkv_kv8_kq_bytes(g); }
+size_t yahkv_kv8_vq_bytes(const yahkv_geometry* g) {
+  return CheckKv8Geometry(g) ? 0 : size_t(g->n_pages) * 16 * g->n_kv_heads * kKv8Dim * MakeKv8Geom(*g).vq_dim() * 4;
+}
 size_t yahkv_kv8_vs_bytes(const yahkv_geometry* g) {
   return CheckKv8Geometry(g) ? 0 : size_t(g->n_pages) * 16 * g->n_kv_heads * kKv8Dim * 4;
 }

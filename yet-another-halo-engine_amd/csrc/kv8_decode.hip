@@ -550,6 +550,7 @@ int Fill(const yahkv_geometry* g, const yahkv_kv8_pools* pools, const int32_t* p
          const int32_t* seq_len, int32_t n_seqs, int32_t max_seq_len, const void* q, int32_t q_dtype, float softmax_scale,
          void* workspace, size_t workspace_bytes, const yahkv_decode_options* opt, DecodeArgs* a) {
   if (const int rc = CheckKv8Pools(g, pools)) return rc;
+  if (g->format != YAHKV_KV8A16) return YAHKV_ERR_SHAPE;
   if (page_table == nullptr || q == nullptr || (reinterpret_cast<uintptr_t>(q) & 15)) return YAHKV_ERR_ARG;
   if (q_dtype != YAHKV_F32 && q_dtype != YAHKV_F16 && q_dtype != YAHKV_BF16) return YAHKV_ERR_ARG;
   if (MakeTuning(opt).one_launch) return YAHKV_ERR_ARG;

@@ -1203,6 +1203,7 @@ extern "C" int yahkv_kv8_prefill_attend(const yahkv_geometry* g, const yahkv_kv8
                                         void* out, int32_t out_dtype, void* workspace, size_t workspace_bytes,
                                         void* stream) {
   if (const int rc = CheckKv8Pools(g, pools)) return rc;
+  if (g->format != YAHKV_KV8A16) return YAHKV_ERR_SHAPE;
   if (page_table == nullptr || prefix_len == nullptr) return YAHKV_ERR_ARG;
   if (n_seqs <= 0 || chunk_len <= 0 || max_prefix_len < 0 || page_table_stride <= 0) return YAHKV_ERR_ARG;
   PrefillArgs a{};
