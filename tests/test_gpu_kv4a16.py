@@ -159,3 +159,127 @@ def test_directed_rows_and_tiles_through_the_kernels(yahkv, torch_gpu):
                          torch.zeros_like(v[:, :1]), v[:, key:key + 1].contiguous())
     got3 = dp3.numpy()
     assert np.array_equal(got3["vq"][:, ::16], got2["vq"][:, ::16]) and np.array_equal(got3["vs"][:, ::16], got2["vs"][:, ::16])
+
+
+def attend(yahkv, torch, dp, table, lens, q, gate=None, **kw):
+    sl = torch.tensor(lens, dtype=torch.int32, device="cuda")
+    out = yahkv.kv8_decode_attend(dp, table, sl, int(max(lens)), torch.from_numpy(q).cuda(), 1.0 / 16.0,
+                                  None if gate is None else torch.from_numpy(gate).cuda(), **kw)
+    torch.cuda.synchronize()
+    return out.cpu().numpy()
+
+
+def model_attention(hp, table_row, n, q, gate=None):
+    """float64 closed form over the oracle's dequantized model; with 4-bit K against the rotated query rounded to f16, as
+    the kernels hold it (the rounding is part of the computation the result is held to 2e-3 for, not of the model)."""
+    Kd, Vd = kv8.dense(hp, table_row, n)
+    qx = kv8.rotate_q(q) if hp.geom.k_bits == 4 else q
+    return closed_form(Kd, Vd, qx, 1.0 / 16.0, gate)
+
+
+def test_recipe_attention_against_the_checkers_own_result(yahkv, torch_gpu, rc):
+    """part_q + reduce at pos 700 with a scrambled table and stale open-tile keys poisoned with 7.0, against the float64
+    result the checker itself compares with (dattn_q_check.py:193-208, K4 against the rotated query)."""
+    torch, g = torch_gpu, rc.g
+    dp, table = dev_pools(yahkv, torch, rc, rc.n)
+    arrs = dp.numpy()
+    arrs["vo"][rc.ptab[rc.pos // 256]][:, rc.nk:] = np.float16(7.0).view(np.uint16)
+    dp.load(arrs)
+    out = attend(yahkv, torch, dp, table, [rc.n], rc.q[None], rc.gate[None])[0]
+    err = rel_err(out, g["rc_ref"])
+    print(f"kv4a16 decode vs the checker's dequantized model: {err:.2e}; vs f16 KV {rel_err(out, g['rc_exact']):.2e}")
+    assert err < TOL
+    out2 = attend(yahkv, torch, dp, table, [rc.n], rc.q[None], None)[0]
+    assert rel_err(out2, model_attention(host_pools(rc, rc.n), rc.ptab, rc.n, rc.q)) < TOL
+
+
+@pytest.mark.parametrize("kb,vb", FORMATS)
+@pytest.mark.parametrize("n", [1, 15, 16, 17, 64, 65, 255, 256, 257, 300, 1023, 1024])
+def test_attention_at_tile_and_page_boundaries(yahkv, torch_gpu, rc, n, kb, vb):
+    torch = torch_gpu
+    dp, table = dev_pools(yahkv, torch, rc, n, kb=kb, vb=vb)
+    hp = host_pools(rc, n, kb=kb, vb=vb)
+    out = attend(yahkv, torch, dp, table, [n], rc.q[None])[0]
+    assert rel_err(out, model_attention(hp, rc.ptab, n, rc.q)) < TOL
+
+
+@pytest.mark.parametrize("kb,vb", FORMATS)
+def test_decode_steps_across_tiles_and_a_page(yahkv, torch_gpu, rc, kb, vb):
+    """Steps 240 .. 275 after a chunk of 240: every step's output, and the pools at the end, against a token-by-token
+    oracle. Crosses tile boundaries (a tile closes on 255, 271) and the page boundary at 256."""
+    torch = torch_gpu
+    n0, n1 = 240, 276
+    dp, table = dev_pools(yahkv, torch, rc, n0, fill=0x11, kb=kb, vb=vb)
+    hp = host_pools(rc, n0, fill=0x11, kb=kb, vb=vb)
+    worst = 0.0
+    for pos in range(n0, n1):
+        kn = torch.from_numpy(rc.K[pos].astype(np.float32).reshape(1, 4, 256)).cuda()
+        vn = torch.from_numpy(rc.V[pos].astype(np.float32).reshape(1, 4, 256)).cuda()
+        sl = torch.tensor([pos + 1], dtype=torch.int32, device="cuda")
+        out = yahkv.kv8_decode_step(dp, table, sl, pos + 1, kn, vn, torch.from_numpy(rc.q[None]).cuda(), 1.0 / 16.0)
+        kv8.append(hp, rc.ptab[None], [pos], None, rc.K[None, pos:pos + 1].astype(np.float32), rc.V[None, pos:pos + 1].astype(np.float32))
+        worst = max(worst, rel_err(out.cpu().numpy()[0], model_attention(hp, rc.ptab, pos + 1, rc.q)))
+    assert worst < TOL, worst
+    assert_pools_equal(dp, hp, "after 36 steps")
+
+
+@pytest.mark.parametrize("kb,vb", FORMATS)
+def test_ragged_batch_shared_pool(yahkv, torch_gpu, kb, vb):
+    """Several sequences of ragged lengths in one shuffled pool: chunk appends with padded chunks (n_valid), a chunk that
+    continues mid-tile, then attention with a gate; every row against the closed form, the pools against the oracle; the
+    default repeats bit for bit; then a step for every sequence at once."""
+    torch = torch_gpu
+    rng = np.random.default_rng(21)
+    lens = [5, 700, 16, 1300, 257, 2047, 1, 96]
+    n_q, H = 12, 2
+    pages = [(n + 40 + 255) // 256 for n in lens]
+    P = sum(pages) + 3
+    perm = rng.permutation(P).astype(np.int32)
+    stride = max(pages)
+    table = np.zeros((len(lens), stride), np.int32)
+    o = 0
+    for s, np_ in enumerate(pages):
+        table[s, :np_] = perm[o:o + np_]
+        o += np_
+    g = yahkv.kv8_geometry(n_q, H, P, kb, vb)
+    dp, hp = yahkv.Kv8Pools(g, 0x77), kv8.HostPools(kv8.geometry(n_q, H, P, kb, vb), 0x77)
+    cap = max(lens)
+    K = (rng.standard_normal((len(lens), cap, H, 256)) + 0.5 * rng.standard_normal((len(lens), 1, H, 256))).astype(np.float16)
+    V = rng.standard_normal((len(lens), cap, H, 256)).astype(np.float16)
+    t_table = torch.from_numpy(table).cuda()
+    nv = np.array(lens, np.int32)
+    Kt, Vt = torch.from_numpy(K).cuda(), torch.from_numpy(V).cuda()
+    yahkv.kv8_kmean(dp, t_table, Kt, torch.from_numpy(nv).cuda())
+    for s in range(len(lens)):
+        hp.km[table[s, 0]] = kv8.kmean(K[s, :lens[s]].astype(np.float32).reshape(lens[s], H * 256))
+    first = np.minimum(nv, 37).astype(np.int32)
+    zero = torch.zeros(len(lens), dtype=torch.int32, device="cuda")
+    yahkv.kv8_append(dp, t_table, zero, Kt[:, :37].contiguous(), Vt[:, :37].contiguous(), torch.from_numpy(first).cuda())
+    kv8.append(hp, table, np.zeros(len(lens), np.int32), first, K[:, :37].astype(np.float32).reshape(len(lens), 37, -1),
+               V[:, :37].astype(np.float32).reshape(len(lens), 37, -1))
+    rest = (nv - first).astype(np.int32)
+    yahkv.kv8_append(dp, t_table, torch.from_numpy(first).cuda(), Kt[:, 37:].contiguous(), Vt[:, 37:].contiguous(),
+                     torch.from_numpy(rest).cuda())
+    kv8.append(hp, table, first, rest, K[:, 37:].astype(np.float32).reshape(len(lens), cap - 37, -1),
+               V[:, 37:].astype(np.float32).reshape(len(lens), cap - 37, -1))
+    torch.cuda.synchronize()
+    assert_pools_equal(dp, hp, "ragged chunks")
+    q = rng.standard_normal((len(lens), n_q, 256)).astype(np.float32)
+    gate = rng.standard_normal((len(lens), n_q, 256)).astype(np.float32)
+    runs = []
+    for kw in ({}, {}, {"opt": yahkv.DecodeOptions(deterministic=-1)}):
+        out = attend(yahkv, torch, dp, t_table, lens, q, gate, **kw)
+        runs.append(out)
+        for s, n in enumerate(lens):
+            assert rel_err(out[s], model_attention(hp, table[s], n, q[s], gate[s])) < TOL, (s, n)
+    assert np.array_equal(runs[0].view(np.uint32), runs[1].view(np.uint32))
+    kn = rng.standard_normal((len(lens), H, 256)).astype(np.float32)
+    vn = rng.standard_normal((len(lens), H, 256)).astype(np.float32)
+    sl = torch.from_numpy(nv + 1).cuda()
+    out = yahkv.kv8_decode_step(dp, t_table, sl, int(max(lens)) + 1, torch.from_numpy(kn).cuda(), torch.from_numpy(vn).cuda(),
+                                torch.from_numpy(q).cuda().to(torch.bfloat16), 1.0 / 16.0).cpu().numpy()
+    kv8.append(hp, table, nv, None, kn.reshape(len(lens), 1, -1), vn.reshape(len(lens), 1, -1))
+    assert_pools_equal(dp, hp, "batched step")
+    qb = torch.from_numpy(q).to(torch.bfloat16).float().numpy()
+    for s, n in enumerate(lens):
+        assert rel_err(out[s], model_attention(hp, table[s], n + 1, qb[s])) < TOL, (s, n)

@@ -42,8 +42,8 @@ inline Kv8Pools MakeKv8Pools(const yahkv_kv8_pools& p) {
 }
 
 // bits of the K and of the V codes of a format of this family (0: not one of them)
-inline int Kv8BitsK(int format) { return format == YAHKV_KV8A16 || format == YAHKV_K8V4A16 ? 8 : format == YAHKV_KV4A16 || format == YAHKV_K4V8A16 ? 4 : 0; }
-inline int Kv8BitsV(int format) { return format == YAHKV_KV8A16 || format == YAHKV_K4V8A16 ? 8 : format == YAHKV_KV4A16 || format == YAHKV_K8V4A16 ? 4 : 0; }
+__host__ __device__ inline int Kv8BitsK(int format) { return format == YAHKV_KV8A16 || format == YAHKV_K8V4A16 ? 8 : format == YAHKV_KV4A16 || format == YAHKV_K4V8A16 ? 4 : 0; }
+__host__ __device__ inline int Kv8BitsV(int format) { return format == YAHKV_KV8A16 || format == YAHKV_K4V8A16 ? 8 : format == YAHKV_KV4A16 || format == YAHKV_K8V4A16 ? 4 : 0; }
 
 int CheckKv8Geometry(const yahkv_geometry* g);
 int CheckKv8Pools(const yahkv_geometry* g, const yahkv_kv8_pools* pools);

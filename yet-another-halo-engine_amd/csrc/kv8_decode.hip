@@ -28,7 +28,15 @@ namespace yahkv {
 namespace {
 
 // ---- the split-K kernel ---------------------------------------------------------------------------------------------
-template <int DUMMY>
+// KB / VB: bits of the K and of the V codes (8: kv8a16, 4: kv4a16; see kv8.hpp). What differs with 4 bits:
+//   K rows are 128 bytes (eight 16-byte chunks = the eight 32-dim groups of a head); a key's dword (eight dims) becomes
+//      the f16 values 1 + u / 16 by four shifts and masks, the two matrix instructions of a group sum (1 + u / 16) q'
+//      over its 32 dims, and with the group's pair (S, C) = (16 s, lo - 16 s) the group's share of the score is
+//      S * sum + C * (sum of the group's q'): the format's own `(1 + u / 16) * S + C`, exact in f32. q' = H256 q / 16
+//      is made by each wave when it starts on a pair (f32 butterflies in the reference's order, then f16).
+//   V codes are 8 bytes per (dim, tile); a dword's nibbles are keys (0, 2, 4, 6, 1, 3, 5, 7) of its eight, so the same
+//      shifts and masks give the key pairs in order, and one packed f16 fma with (16 s, c - 23 s) the values.
+template <int KB, int VB>
 __global__ __launch_bounds__(64 * kWavesPerGroup) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void Kv8Part(const DecodeArgs a, const Kv8Pools pools) {
   constexpr int D = kKv8Dim, NT = D / 16;
@@ -43,9 +51,9 @@ void Kv8Part(const DecodeArgs a, const Kv8Pools pools) {
   // Query A-operands [step m of 16][lane half][head row][8 dims]: step m = 2 j + sub covers, in lane half hf, the 8
   // bytes `sub` of the 16-byte chunk 2 j + hf of a key's row: dims 16 (2 j + hf) + 8 sub + (0, 2, 1, 3, 4, 6, 5, 7).
   __shared__ __align__(16) _Float16 lq_all[kWavesPerGroup][16][2][8][8];
-  __shared__ __align__(16) float lcorr_all[kWavesPerGroup][2][8];
+  __shared__ __align__(16) float lcorr_all[kWavesPerGroup][KB == 4 ? 8 : 2][8];
   __shared__ __align__(16) _Float16 lp_all[kWavesPerGroup][kMaxGroup][kTile];
-  __shared__ __align__(16) uint8_t lk_all[kWavesPerGroup][32 * 256];  // 32 key rows, chunks swizzled by row
+  __shared__ __align__(16) uint8_t lk_all[kWavesPerGroup][32 * (KB == 4 ? 128 : 256)];  // 32 key rows, chunks swizzled by row
   __shared__ int next_tile;
   __shared__ int progress[kWavesPerGroup];  // tiles each wave is through with (fixed pattern only)
   __shared__ int wave_sum[kWavesPerGroup][2];
@@ -98,7 +106,9 @@ void Kv8Part(const DecodeArgs a, const Kv8Pools pools) {
   };
 
   uint2 ksc;       // this lane's key: the two halves' scale pairs
-  uint4 vb[NT / 2];  // 16 keys of this lane's dim in this lane group's tile (one half of the dims at a time)
+  uint4 ksc4[2];   // 4-bit K: the eight groups' pairs
+  uint4 vb[VB == 4 ? 1 : NT / 2];  // 16 keys of this lane's dim in this lane group's tile (one half of the dims at a time)
+  uint2 vb4[VB == 4 ? NT / 2 : 1];
   uint32_t vst[NT / 2];
   float m[4], lsum[4], sc[2][4];
   f4v o[NT];
@@ -117,30 +127,89 @@ void Kv8Part(const DecodeArgs a, const Kv8Pools pools) {
   // (l % 16) ^ (row % 16) of row 4 i + l / 16 to LDS position 1024 i + 16 l
   auto load_k = [&](int tile, int tt, int page) {
     const size_t row0 = size_t(page) * kKv8Page + (tile % 4) * kTile + 32 * tt;
-    const auto rk = __builtin_amdgcn_make_buffer_rsrc(
-        reinterpret_cast<uint8_t*>(pools.kq) + (row0 * H + cur.h) * 256, 0, 0x7fffffff, 0x00020000);
-    const uint32_t r = lane / 16, c = lane % 16;
+    if constexpr (KB == 4) {
+      // eight rows per instruction; lane l of instruction i carries chunk (l % 8) ^ (row % 8) of row 8 i + l / 8
+      const auto rk4 = __builtin_amdgcn_make_buffer_rsrc(
+          reinterpret_cast<uint8_t*>(pools.kq) + (row0 * H + cur.h) * 128, 0, 0x7fffffff, 0x00020000);
+      const uint32_t r = lane / 8, c = lane % 8;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const uint32_t rr = 4 * i + r;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, (__attribute__((address_space(3))) void*)(&lk[i * 1024]), 16,
-                                               rr * (H * 256) + ((c ^ (rr & 15)) << 4), 0, 0, kStreamed);
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t rr = 8 * i + r;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rk4, (__attribute__((address_space(3))) void*)(&lk[i * 1024]), 16,
+                                                 rr * (H * 128) + ((c ^ (rr & 7)) << 4), 0, 0, kStreamed);
+      }
+      const uint32_t* sp4 = pools.ks + ((row0 + n32) * H + cur.h) * 8;
+      ksc4[0] = StreamLoad(reinterpret_cast<const uint4*>(sp4));
+      ksc4[1] = StreamLoad(reinterpret_cast<const uint4*>(sp4 + 4));
+    } else {
+      const auto rk = __builtin_amdgcn_make_buffer_rsrc(
+          reinterpret_cast<uint8_t*>(pools.kq) + (row0 * H + cur.h) * 256, 0, 0x7fffffff, 0x00020000);
+      const uint32_t r = lane / 16, c = lane % 16;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const uint32_t rr = 4 * i + r;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, (__attribute__((address_space(3))) void*)(&lk[i * 1024]), 16,
+                                                 rr * (H * 256) + ((c ^ (rr & 15)) << 4), 0, 0, kStreamed);
+      }
+      const uint32_t* sp = pools.ks + ((row0 + n32) * H + cur.h) * 2;
+      ksc = StreamLoad(reinterpret_cast<const uint2*>(sp));
     }
-    const uint32_t* sp = pools.ks + ((row0 + n32) * H + cur.h) * 2;
-    ksc = StreamLoad(reinterpret_cast<const uint2*>(sp));
   };
   auto fetch_v = [&](int tile, int hf, int page) {
     const size_t pt = size_t(page) * 16 + (tile % 4) * 4 + kg;
-    const uint32_t* vp = pools.vq + ((size_t(cur.h) * tiles16 + pt) * 256 + 128 * hf + n16) * 4;
+    const uint32_t* vp = pools.vq + ((size_t(cur.h) * tiles16 + pt) * 256 + 128 * hf + n16) * (VB == 4 ? 2 : 4);
     const uint32_t* sp = pools.vs + (size_t(cur.h) * tiles16 + pt) * 256 + 128 * hf + n16;
+    if constexpr (VB == 4) {
 #pragma unroll
-    for (int j = 0; j < NT / 2; ++j) vb[j] = StreamLoad(reinterpret_cast<const uint4*>(vp + 64 * j));
+      for (int j = 0; j < NT / 2; ++j) vb4[j] = StreamLoad(reinterpret_cast<const uint2*>(vp + 32 * j));
+    } else {
+#pragma unroll
+      for (int j = 0; j < NT / 2; ++j) vb[j] = StreamLoad(reinterpret_cast<const uint4*>(vp + 64 * j));
+    }
 #pragma unroll
     for (int j = 0; j < NT / 2; ++j) vst[j] = StreamLoad(sp + 16 * j);
   };
   // scores of the 32 keys in the LDS slot against all heads: the two 128-dim halves are two accumulator chains
+  // a dword of eight 4-bit codes (dims 2 j / 2 j + 1 at bits 4 j / 16 + 4 j) as the f16 values 1 + u / 16 in dim order
+  auto nibbles_f16 = [](uint32_t w) -> h8v {
+    const uint4 k = {((w << 6) & 0x03c003c0u) | 0x3c003c00u, ((w << 2) & 0x03c003c0u) | 0x3c003c00u,
+                     ((w >> 2) & 0x03c003c0u) | 0x3c003c00u, ((w >> 6) & 0x03c003c0u) | 0x3c003c00u};
+    return __builtin_bit_cast(h8v, k);
+  };
   auto scores = [&](int tt) {
     f16v c0 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}, c1 = c0;
+    if constexpr (KB == 4) {
+      // group c = chunk c of the key's row; lane half hf holds dwords 2 hf, 2 hf + 1 of it: steps 2 c and 2 c + 1
+      const uint32_t pr[8] = {ksc4[0].x, ksc4[0].y, ksc4[0].z, ksc4[0].w, ksc4[1].x, ksc4[1].y, ksc4[1].z, ksc4[1].w};
+      float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int c = 0; c < 8; c += 2) {
+        const uint2 w0 = *reinterpret_cast<const uint2*>(&lk[n32 * 128 + ((c ^ (n32 & 7)) << 4) + 8 * half]);
+        const uint2 w1 = *reinterpret_cast<const uint2*>(&lk[n32 * 128 + (((c + 1) ^ (n32 & 7)) << 4) + 8 * half]);
+        const h8v qa0 = *reinterpret_cast<const h8v*>(&lq[2 * c][half][n32 % 8][0]);
+        const h8v qa1 = *reinterpret_cast<const h8v*>(&lq[2 * c + 1][half][n32 % 8][0]);
+        const h8v qb0 = *reinterpret_cast<const h8v*>(&lq[2 * c + 2][half][n32 % 8][0]);
+        const h8v qb1 = *reinterpret_cast<const h8v*>(&lq[2 * c + 3][half][n32 % 8][0]);
+        const f16v z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        f16v g0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(qa0, nibbles_f16(w0.x), z, 0, 0, 0);
+        f16v g1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(qb0, nibbles_f16(w1.x), z, 0, 0, 0);
+        g0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(qa1, nibbles_f16(w0.y), g0, 0, 0, 0);
+        g1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(qb1, nibbles_f16(w1.y), g1, 0, 0, 0);
+        const float4 s0 = *reinterpret_cast<const float4*>(&lcorr[c][4 * half]);
+        const float4 s1 = *reinterpret_cast<const float4*>(&lcorr[c + 1][4 * half]);
+        const float S0 = WidenF16(static_cast<uint16_t>(pr[c] & 0xFFFF)), C0 = WidenF16(static_cast<uint16_t>(pr[c] >> 16));
+        const float S1 = WidenF16(static_cast<uint16_t>(pr[c + 1] & 0xFFFF)), C1 = WidenF16(static_cast<uint16_t>(pr[c + 1] >> 16));
+        const float q0[4] = {s0.x, s0.y, s0.z, s0.w}, q1[4] = {s1.x, s1.y, s1.z, s1.w};
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          acc[r] = __builtin_fmaf(S0, g0[r], __builtin_fmaf(C0, q0[r], acc[r]));
+          acc[r] = __builtin_fmaf(S1, g1[r], __builtin_fmaf(C1, q1[r], acc[r]));
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) sc[tt][r] = acc[r] * qk_scale;
+      return;
+    }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const uint4 w0 = *reinterpret_cast<const uint4*>(&lk[n32 * 256 + (((2 * j + half) ^ (n32 & 15)) << 4)]);
@@ -180,6 +249,17 @@ void Kv8Part(const DecodeArgs a, const Kv8Pools pools) {
       const uint32_t st = dead ? 0u : vst[j];
       const h2v sp = __builtin_bit_cast(h2v, st);
       const h2v S2 = {sp[0], sp[0]}, C2 = {sp[1], sp[1]};
+      if constexpr (VB == 4) {
+        // dword w holds keys 8 w + (0, 2, 4, 6 | 1, 3, 5, 7): the pairs (2 p, 2 p + 1) sit 16 bits apart
+        const h8v u0 = nibbles_f16(vb4[j].x), u1 = nibbles_f16(vb4[j].y);
+        const h8v S8 = {sp[0], sp[0], sp[0], sp[0], sp[0], sp[0], sp[0], sp[0]};
+        const h8v C8 = {sp[1], sp[1], sp[1], sp[1], sp[1], sp[1], sp[1], sp[1]};
+        const h8v v0 = __builtin_elementwise_fma(u0, S8, C8), v1 = __builtin_elementwise_fma(u1, S8, C8);
+        const int nt = hf * (NT / 2) + j;
+        o[nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa0, v0, o[nt], 0, 0, 0);
+        o[nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa1, v1, o[nt], 0, 0, 0);
+        continue;
+      }
       const uint32_t w[4] = {vb[j].x, vb[j].y, vb[j].z, vb[j].w};
       h2v f[8];
 #pragma unroll
@@ -238,7 +318,68 @@ void Kv8Part(const DecodeArgs a, const Kv8Pools pools) {
     int pgc = load_page(tile), pgn;
     load_k(tile, 0, pgc);
     fetch_v(tile, 1, pgc);  // not used: keeps the count of loads in flight at the loop's head the same on every pass
-    {
+    if constexpr (KB == 4) {
+      // Entry e of this lane: step mm = lane / 16 + 4 e, lane half hf = (lane / 8) % 2, head row rw = lane % 8, the eight
+      // dims 32 (mm / 2) + 8 (2 hf + mm % 2) + [0, 8) in their natural order. H256 over a head's 256 dims, stages in the
+      // reference's order: dims 1, 2, 4 apart inside an entry; 8 apart = lane ^ 16, 16 = lane ^ 8, 32 = lane ^ 32;
+      // 64 and 128 apart = entries e ^ 1 and e ^ 2.
+#pragma clang fp contract(off)
+      const int rw = lane % 8, hf = (lane / 8) % 2;
+      float x[4][8];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int mm = lane / 16 + 4 * e;
+        const int d0 = 32 * (mm / 2) + 8 * (2 * hf + mm % 2);
+        h8v qv = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (rw < G) qv = LoadQ8(a.q, (size_t(cur.s) * g.n_q + size_t(cur.h) * G + rw) * D + d0, a.q_dtype);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) x[e][k] = static_cast<float>(qv[k]);
+#pragma unroll
+        for (int st = 1; st < 8; st <<= 1)
+#pragma unroll
+          for (int k = 0; k < 8; ++k)
+            if (!(k & st)) {
+              const float lo = x[e][k], up = x[e][k | st];
+              x[e][k] = lo + up, x[e][k | st] = lo - up;
+            }
+      }
+      auto cross = [&](int xm) {
+        const bool upper = (lane & xm) != 0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+#pragma unroll
+          for (int k = 0; k < 8; ++k) {
+            const float o2 = __shfl_xor(x[e][k], xm, 64);
+            x[e][k] = upper ? o2 - x[e][k] : x[e][k] + o2;
+          }
+      };
+      cross(16), cross(8), cross(32);
+#pragma unroll
+      for (int st = 1; st < 4; st <<= 1)
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (!(e & st))
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+              const float lo = x[e][k], up = x[e | st][k];
+              x[e][k] = lo + up, x[e | st][k] = lo - up;
+            }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int mm = lane / 16 + 4 * e;
+        h8v qs;
+        float t = 0.0f;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+          qs[k] = static_cast<_Float16>(x[e][k] * 0.0625f);
+          t += static_cast<float>(qs[k]);
+        }
+        *reinterpret_cast<h8v*>(&lq[mm][hf][rw][0]) = qs;
+        // the group's sum of q': its four entries sit in the lanes that differ in bits 3 and 4
+        t += __shfl_xor(t, 8, 64), t += __shfl_xor(t, 16, 64);
+        if ((lane & 24) == 0) lcorr[2 * e + lane / 32][rw] = t;
+      }
+    } else {
       float hsum[2] = {0.0f, 0.0f};  // per (128-dim half, head row lane % 8): this lane's share
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
@@ -348,7 +489,8 @@ constexpr int kTail = 17;  // keys the merge adds itself: up to 16 of the open t
 // loom_decoder.hpp:254-261), and written to the pools by the workgroup of the group's first query head.
 __global__ __launch_bounds__(kReduceThreads) void Kv8Reduce(const DecodeArgs a, const Kv8Pools pools, const StepRows rows) {
   const Geom g = a.g;
-  const Kv8Geom kg8{g.n_q, g.n_kv, g.n_pages};
+  const Kv8Geom kg8{g.n_q, g.n_kv, g.n_pages, Kv8BitsK(g.format), Kv8BitsV(g.format)};
+  const bool k4 = kg8.kb == 4;
   constexpr int D = kKv8Dim;
   const int G = g.group(), H = g.n_kv;
   const int hq = blockIdx.x, s = blockIdx.y, t = threadIdx.x;
@@ -360,9 +502,25 @@ __global__ __launch_bounds__(kReduceThreads) void Kv8Reduce(const DecodeArgs a, 
   const int ts = TilesOf(a, s);
   __shared__ float tail_score[kTail];
   __shared__ __align__(16) float new_v[D];
+  __shared__ __align__(16) float qrot[D];  // 4-bit K: the head's rotated query, H256 q / 16 rounded to f16
   if (len <= 0) {
     for (int d = t; d < DZ; d += kReduceThreads) a.out[o + d] = 0.0f;
     return;
+  }
+  if (k4) {  // the butterfly of the part kernel's prologue, over LDS (gen_decode_attn.py:655-683)
+#pragma clang fp contract(off)
+    qrot[t] = static_cast<float>(SaturateToF16(LoadSrc(a.q, (size_t(s) * g.n_q + hq) * D + t, a.q_dtype)));
+    __syncthreads();
+    for (int st = 1; st < D; st <<= 1) {
+      if (t < D / 2) {
+        const int i = (t / st) * 2 * st + t % st;
+        const float lo = qrot[i], up = qrot[i + st];
+        qrot[i] = lo + up, qrot[i + st] = lo - up;
+      }
+      __syncthreads();
+    }
+    qrot[t] = static_cast<float>(static_cast<_Float16>(qrot[t] * 0.0625f));
+    __syncthreads();
   }
   const int closed = (len - 1) & ~15;           // keys the split-K kernel covered
   const int n_pool = step ? len - 1 : len;      // keys whose rows are in the pools
@@ -374,7 +532,20 @@ __global__ __launch_bounds__(kReduceThreads) void Kv8Reduce(const DecodeArgs a, 
   {
     const int j = t / 16, c = t % 16;
     float part = 0.0f;
-    if (j < n_tail) {
+    if (j < n_tail && k4) {  // 16 dims = two dwords of one group: u * (S / 16) + (C + S), gen_decode_attn.py:806-850
+      const size_t r = size_t(page) * kKv8Page + closed % kKv8Page + j;
+      const uint2 w = *reinterpret_cast<const uint2*>(pools.kq + kg8.kq_row(r, h) + 2 * c);
+      const uint32_t pair = pools.ks[kg8.ks_row(r, h) + c / 2];
+      const float S = WidenF16(static_cast<uint16_t>(pair & 0xFFFF)), C = WidenF16(static_cast<uint16_t>(pair >> 16));
+      const float d = S * 0.0625f, l0 = C + S;
+      const uint32_t ww[2] = {w.x, w.y};
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int e = i % 8;
+        const float u = static_cast<float>((ww[i / 8] >> (4 * (e / 2) + (e % 2 ? 16 : 0))) & 15u);
+        part += (u * d + l0) * qrot[16 * c + i];
+      }
+    } else if (j < n_tail) {
       const size_t r = size_t(page) * kKv8Page + closed % kKv8Page + j;
       const uint4 w = *reinterpret_cast<const uint4*>(pools.kq + kg8.kq_row(r, h) + 4 * c);
       const uint32_t pair = pools.ks[kg8.ks_row(r, h) + c / 8];
@@ -404,7 +575,25 @@ __global__ __launch_bounds__(kReduceThreads) void Kv8Reduce(const DecodeArgs a, 
     const int pos = len - 1;
     const int wpage = ClampPage(trow[min(pos / kKv8Page, a.stride - 1)], g.n_pages);
     const size_t src = (size_t(s) * H + h) * D + 4 * lane;
-    if (wave == 0) {
+    if (wave == 0 && k4) {
+#pragma clang fp contract(off)
+      const float4 x = Load4(rows.k, src, rows.dtype);
+      const float4 mean = *reinterpret_cast<const float4*>(pools.km + kg8.km_head(page0, h) + 4 * lane);
+      const float4 c = {TruncF16(x.x) - mean.x, TruncF16(x.y) - mean.y, TruncF16(x.z) - mean.z, TruncF16(x.w) - mean.w};
+      uint32_t pair;
+      float4 deq;
+      uint32_t w = Kv4CodesK(c, lane, &pair, &deq);
+      w |= __shfl_xor(w, 1, 64);
+      if (writes) {
+        const size_t r = size_t(wpage) * kKv8Page + pos % kKv8Page;
+        if (lane % 2 == 0) pools.kq[kg8.kq_row(r, h) + lane / 2] = w;
+        if (lane % 8 == 0) pools.ks[kg8.ks_row(r, h) + lane / 8] = pair;
+      }
+      const float4 q4 = *reinterpret_cast<const float4*>(&qrot[4 * lane]);
+      float dot = deq.x * q4.x + deq.y * q4.y + deq.z * q4.z + deq.w * q4.w;
+      dot = WaveSum(dot);
+      if (lane == 0) tail_score[n_tail] = dot * a.scale;
+    } else if (wave == 0) {
 #pragma clang fp contract(off)
       const float4 x = Load4(rows.k, src, rows.dtype);
       const float4 mean = *reinterpret_cast<const float4*>(pools.km + kg8.km_head(page0, h) + 4 * lane);
@@ -448,10 +637,16 @@ __global__ __launch_bounds__(kReduceThreads) void Kv8Reduce(const DecodeArgs a, 
 #pragma unroll
             for (int j = 0; j < 16; ++j) x[j] = WidenF16(static_cast<uint16_t>(w[j / 2] >> (16 * (j % 2))));
             x[15] = TruncF16(ve[e]);
-            uint4 codes;
             uint32_t stats;
-            Kv8QuantTile(x, &codes, &stats);
-            *reinterpret_cast<uint4*>(pools.vq + kg8.vq_tile(h, pt) + size_t(4 * lane + e) * 4) = codes;
+            if (kg8.vb == 4) {
+              uint2 codes;
+              Kv4QuantTile(x, &codes, &stats);
+              *reinterpret_cast<uint2*>(pools.vq + kg8.vq_tile(h, pt) + size_t(4 * lane + e) * 2) = codes;
+            } else {
+              uint4 codes;
+              Kv8QuantTile(x, &codes, &stats);
+              *reinterpret_cast<uint4*>(pools.vq + kg8.vq_tile(h, pt) + size_t(4 * lane + e) * 4) = codes;
+            }
             pools.vs[kg8.vs_tile(h, pt) + 4 * lane + e] = stats;
           }
         }
@@ -550,7 +745,6 @@ int Fill(const yahkv_geometry* g, const yahkv_kv8_pools* pools, const int32_t* p
          const int32_t* seq_len, int32_t n_seqs, int32_t max_seq_len, const void* q, int32_t q_dtype, float softmax_scale,
          void* workspace, size_t workspace_bytes, const yahkv_decode_options* opt, DecodeArgs* a) {
   if (const int rc = CheckKv8Pools(g, pools)) return rc;
-  if (g->format != YAHKV_KV8A16) return YAHKV_ERR_SHAPE;
   if (page_table == nullptr || q == nullptr || (reinterpret_cast<uintptr_t>(q) & 15)) return YAHKV_ERR_ARG;
   if (q_dtype != YAHKV_F32 && q_dtype != YAHKV_F16 && q_dtype != YAHKV_BF16) return YAHKV_ERR_ARG;
   if (MakeTuning(opt).one_launch) return YAHKV_ERR_ARG;
@@ -579,8 +773,15 @@ extern "C" int yahkv_kv8_decode_part(const yahkv_geometry* g, const yahkv_kv8_po
   if (const int rc = Fill(g, pools, page_table, page_table_stride, seq_len, n_seqs, max_seq_len, q, q_dtype, softmax_scale,
                           workspace, workspace_bytes, opt, &a))
     return rc;
-  hipLaunchKernelGGL(Kv8Part<0>, dim3(static_cast<unsigned>(a.n_chunks)), dim3(64 * kWavesPerGroup), 0,
-                     static_cast<hipStream_t>(stream), a, MakeKv8Pools(*pools));
+  const dim3 grid(static_cast<unsigned>(a.n_chunks)), block(64 * kWavesPerGroup);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const Kv8Pools p = MakeKv8Pools(*pools);
+  switch (g->format) {
+    case YAHKV_KV8A16: hipLaunchKernelGGL((Kv8Part<8, 8>), grid, block, 0, st, a, p); break;
+    case YAHKV_KV4A16: hipLaunchKernelGGL((Kv8Part<4, 4>), grid, block, 0, st, a, p); break;
+    case YAHKV_K8V4A16: hipLaunchKernelGGL((Kv8Part<8, 4>), grid, block, 0, st, a, p); break;
+    default: hipLaunchKernelGGL((Kv8Part<4, 8>), grid, block, 0, st, a, p); break;
+  }
   return LaunchStatus();
 }
 
