@@ -283,3 +283,74 @@ def test_ragged_batch_shared_pool(yahkv, torch_gpu, kb, vb):
     qb = torch.from_numpy(q).to(torch.bfloat16).float().numpy()
     for s, n in enumerate(lens):
         assert rel_err(out[s], model_attention(hp, table[s], n + 1, qb[s])) < TOL, (s, n)
+
+
+@pytest.mark.parametrize("kb,vb", FORMATS)
+def test_chunked_prefill_over_a_paged_prefix(yahkv, torch_gpu, kb, vb):
+    """Two sequences with prefixes of different lengths (one ending inside a tile), a chunk appended to each, then the
+    chunk's causal attention: against the closed form over the prefill-side decode (one f16 fma per element, every V
+    tile from codes; yah_kdeq4 / yah_vdeq4) with, for 4-bit K, the query rotated and rounded to f16 as yah_qrot leaves it."""
+    torch = torch_gpu
+    rng = np.random.default_rng(31)
+    n_q, H, chunk = 12, 2, 200
+    prefix = [300, 77]
+    pages = [(p + chunk + 255) // 256 for p in prefix]
+    P = sum(pages) + 2
+    perm = rng.permutation(P).astype(np.int32)
+    table = np.zeros((2, max(pages)), np.int32)
+    table[0, :pages[0]], table[1, :pages[1]] = perm[:pages[0]], perm[pages[0]:pages[0] + pages[1]]
+    g = yahkv.kv8_geometry(n_q, H, P, kb, vb)
+    dp, hp = yahkv.Kv8Pools(g, 0x21), kv8.HostPools(kv8.geometry(n_q, H, P, kb, vb), 0x21)
+    cap = max(prefix)
+    K = (rng.standard_normal((2, cap + chunk, H, 256)) + 0.7 * rng.standard_normal((2, 1, H, 256))).astype(np.float16)
+    V = rng.standard_normal((2, cap + chunk, H, 256)).astype(np.float16)
+    t_table = torch.from_numpy(table).cuda()
+    pl = torch.tensor(prefix, dtype=torch.int32, device="cuda")
+    Kp, Vp = torch.from_numpy(K[:, :cap].copy()).cuda(), torch.from_numpy(V[:, :cap].copy()).cuda()
+    yahkv.kv8_kmean(dp, t_table, Kp, pl)
+    yahkv.kv8_append(dp, t_table, torch.zeros(2, dtype=torch.int32, device="cuda"), Kp, Vp, pl)
+    Kc = np.stack([K[s, prefix[s]:prefix[s] + chunk] for s in range(2)])
+    Vc = np.stack([V[s, prefix[s]:prefix[s] + chunk] for s in range(2)])
+    yahkv.kv8_append(dp, t_table, pl, torch.from_numpy(Kc).cuda(), torch.from_numpy(Vc).cuda())
+    for s in range(2):
+        hp.km[table[s, 0]] = kv8.kmean(K[s, :prefix[s]].astype(np.float32).reshape(prefix[s], -1))
+    kv8.append(hp, table, [0, 0], prefix, K[:, :cap].astype(np.float32).reshape(2, cap, -1), V[:, :cap].astype(np.float32).reshape(2, cap, -1))
+    kv8.append(hp, table, prefix, None, Kc.astype(np.float32).reshape(2, chunk, -1), Vc.astype(np.float32).reshape(2, chunk, -1))
+    torch.cuda.synchronize()
+    assert_pools_equal(dp, hp, "prefix + chunk")
+    q = torch.from_numpy(rng.standard_normal((2, chunk, n_q, 256)).astype(np.float32)).cuda().to(torch.bfloat16)
+    gate = rng.standard_normal((2, chunk, n_q, 256)).astype(np.float32)
+    out = yahkv.kv8_prefill_attend(dp, t_table, pl, max(prefix), q, 1.0 / 16.0, torch.from_numpy(gate).cuda(),
+                                   out=torch.empty(q.shape, dtype=torch.float32, device="cuda")).cpu().numpy()
+    qf = q.float().cpu().numpy()
+    if kb == 4:
+        qf = kv8.rotate_q(qf).astype(np.float16).astype(np.float32)
+    worst = 0.0
+    for s in range(2):
+        n = prefix[s] + chunk
+        Kh, Vh = kv8.dense(hp, table[s], n, as_f16=True)
+        for t in (0, 1, 15, 16, 63, 64, 128, chunk - 1):
+            vis = prefix[s] + t + 1
+            worst = max(worst, rel_err(out[s, t], closed_form(Kh[:vis], Vh[:vis], qf[s, t], 1.0 / 16.0, gate[s, t])))
+    print(f"k{kb}v{vb} prefill vs the closed form over its own f16 decode: {worst:.2e}")
+    assert worst < TOL
+
+
+def test_refusals(yahkv, torch_gpu):
+    import ctypes as C
+    bad = yahkv.Geometry(yahkv.KV4A16, 24, 4, 128, 256, 2)
+    assert yahkv.lib.yahkv_kv8_kq_bytes(C.byref(bad)) == 0
+    g = yahkv.kv8_geometry(24, 4, 2, 4, 4)
+    assert yahkv.lib.yahkv_kv8_kq_bytes(C.byref(g)) == 2 * 256 * 512 and yahkv.lib.yahkv_kv8_ks_bytes(C.byref(g)) == 2 * 256 * 128
+    assert yahkv.lib.yahkv_kv8_vq_bytes(C.byref(g)) == 4 * 32 * 256 * 8 and yahkv.lib.yahkv_kv8_vs_bytes(C.byref(g)) == 4 * 32 * 256 * 4
+    dp = yahkv.Kv8Pools(yahkv.kv8_geometry(24, 4, 2, 8, 8))          # 8-bit pools are too short for... no: K is longer; V too
+    g84 = yahkv.kv8_geometry(24, 4, 2, 4, 4)
+    small = yahkv.Kv8Pools(g84)
+    table = torch_gpu.zeros((1, 2), dtype=torch_gpu.int32, device="cuda")
+    k = torch_gpu.zeros((1, 1, 4, 256), device="cuda")
+    st = small.struct()
+    g88 = yahkv.kv8_geometry(24, 4, 2, 8, 8)                         # 4-bit pools handed over with an 8-bit geometry
+    rc_ = yahkv.lib.yahkv_kv8_append(C.byref(g88), C.byref(st), table.data_ptr(), 2, table.data_ptr(), None, 1, 1,
+                                     k.data_ptr(), k.data_ptr(), 0, None)
+    assert rc_ == -1
+    del dp

@@ -47,6 +47,7 @@ struct PrefillArgs {
   const int32_t* prefix_len;
   int32_t n_seqs, max_prefix, chunk_len;
   const uint16_t* q;  // bf16 [n_seqs][chunk_len][n_q][D]
+  int32_t q_is_f16;   // q holds f16 values instead (the rotated queries of the 4-bit K format)
   float scale;
   const float* gate;
   void* out;
@@ -65,8 +66,9 @@ __device__ __forceinline__ uint32_t PackF16(float a, float b) {  // round to nea
 __device__ __forceinline__ float ClampF16(float x) { return __builtin_fminf(__builtin_fmaxf(x, -65504.0f), 65504.0f) + (x - x); }
 __device__ __forceinline__ uint32_t PackF16Sat(float a, float b) { return PackF16(ClampF16(a), ClampF16(b)); }
 // Eight bf16 query elements as f16.
-__device__ __forceinline__ h8v QueryF16(const uint16_t* p) {
+__device__ __forceinline__ h8v QueryF16(const uint16_t* p, bool is_f16 = false) {
   const uint4 w = *reinterpret_cast<const uint4*>(p);
+  if (is_f16) return __builtin_bit_cast(h8v, w);
   const uint32_t u[4] = {w.x, w.y, w.z, w.w};
   uint32_t o[4];
 #pragma unroll
@@ -583,11 +585,39 @@ __device__ __forceinline__ void Kv8DecodeDword(uint32_t w, uint32_t pair, uint32
   *lo = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(a, S, C));
   *hi = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(b, S, C));
 }
+// 4-bit codes (kv4a16): eight nibbles of a dword (elements 2 j / 2 j + 1 at bits 4 j / 16 + 4 j) become the f16 pairs
+// 1 + u / 16 in order by four shifts and masks, and the same fma gives the values (yah_kdeq4 / yah_vdeq4,
+// gen_attn_fa.py:4652-4700). `first`: the pair index of the first of the `n` pairs wanted.
+__device__ __forceinline__ void Kv4DecodePairs(uint32_t w, uint32_t pair, int first, int n, uint32_t* out) {
+  typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+  const h2 sp = __builtin_bit_cast(h2, pair);
+  const h2 S = {sp[0], sp[0]}, C = {sp[1], sp[1]};
+  for (int i = 0; i < n; ++i) {
+    const int sh = 6 - 4 * (first + i);  // pair 0: << 6, 1: << 2, 2: >> 2, 3: >> 6
+    const uint32_t x = sh >= 0 ? w << sh : w >> -sh;
+    const h2 f = __builtin_bit_cast(h2, (x & 0x03c003c0u) | 0x3c003c00u);
+    out[i] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(f, S, C));
+  }
+}
+// The queries of a chunk rotated for 4-bit K: f16(H256 q / 16) per head (yah_qrot, gen_attn_fa.py:4541-4611; the
+// softmax scale stays a separate factor here). One wave per (token, head) row, four dims per lane.
+__global__ __launch_bounds__(256) void Kv4RotateQ(const uint16_t* q, uint16_t* out, int64_t n_rows) {
+#pragma clang fp contract(off)
+  const int64_t r = int64_t(blockIdx.x) * 4 + threadIdx.x / 64;
+  const int lane = threadIdx.x % 64;
+  if (r >= n_rows) return;
+  const uint2 w = *reinterpret_cast<const uint2*>(q + r * kKv8Dim + 4 * lane);
+  const float4 x = {ClampF16(WidenBf16(static_cast<uint16_t>(w.x & 0xFFFF))), ClampF16(WidenBf16(static_cast<uint16_t>(w.x >> 16))),
+                    ClampF16(WidenBf16(static_cast<uint16_t>(w.y & 0xFFFF))), ClampF16(WidenBf16(static_cast<uint16_t>(w.y >> 16)))};
+  const float4 h = WaveHadamard256(x, lane);
+  *reinterpret_cast<uint2*>(out + r * kKv8Dim + 4 * lane) =
+      uint2{PackF16(h.x * 0.0625f, h.y * 0.0625f), PackF16(h.z * 0.0625f, h.w * 0.0625f)};
+}
 template <int DUMMY>
 __global__ __launch_bounds__(256) void PrefillImagesKv8(const ImageArgs a) {
   constexpr int D = kKv8Dim, PT = kKv8Page, CPR = D / 8;
   const Geom g = a.g;
-  const Kv8Geom kg{g.n_q, g.n_kv, g.n_pages};
+  const Kv8Geom kg{g.n_q, g.n_kv, g.n_pages, Kv8BitsK(g.format), Kv8BitsV(g.format)};
   const int H = g.n_kv, tile = blockIdx.x, pair = blockIdx.y, s = pair / H, h = pair % H, tid = threadIdx.x;
   const int n_keys = ClampPrefix(a.prefix_len, s, a.max_prefix, a.stride, PT, a.chunk_len) + a.chunk_len;
   if (tile * kKeys >= n_keys) return;
@@ -600,10 +630,14 @@ __global__ __launch_bounds__(256) void PrefillImagesKv8(const ImageArgs a) {
     uint32_t o[4] = {0u, 0u, 0u, 0u};
     if (kk < n_keys) {
       const size_t r = size_t(page) * PT + kk % PT;
-      const uint2 w = StreamLoad(reinterpret_cast<const uint2*>(a.kv8.kq + kg.kq_row(r, h) + 2 * c));
-      const uint32_t sc = a.kv8.ks[kg.ks_row(r, h) + c / 16];
-      Kv8DecodeDword(w.x, sc, &o[0], &o[1]);
-      Kv8DecodeDword(w.y, sc, &o[2], &o[3]);
+      if (kg.kb == 4) {  // the chunk's eight dims are one dword of codes, in the 32-dim group c / 4
+        Kv4DecodePairs(StreamLoad(a.kv8.kq + kg.kq_row(r, h) + c), a.kv8.ks[kg.ks_row(r, h) + c / 4], 0, 4, o);
+      } else {
+        const uint2 w = StreamLoad(reinterpret_cast<const uint2*>(a.kv8.kq + kg.kq_row(r, h) + 2 * c));
+        const uint32_t sc = a.kv8.ks[kg.ks_row(r, h) + c / 16];
+        Kv8DecodeDword(w.x, sc, &o[0], &o[1]);
+        Kv8DecodeDword(w.y, sc, &o[2], &o[3]);
+      }
     }
     *reinterpret_cast<uint4*>(kimg + size_t(p) * 16) = uint4{o[0], o[1], o[2], o[3]};
   }
@@ -614,10 +648,14 @@ __global__ __launch_bounds__(256) void PrefillImagesKv8(const ImageArgs a) {
     for (int hf = 0; hf < 2; ++hf) {
       const int kk = tile * kKeys + 32 * s2 + 16 * hf + 4 * jg;  // four keys: dword (kk % 16) / 4 of their 16-key tile
       const size_t pt = size_t(page) * 16 + (kk / 16) % 16;
-      const uint32_t w = StreamLoad(a.kv8.vq + kg.vq_tile(h, pt) + size_t(dim) * 4 + (kk % 16) / 4);
       const uint32_t st = a.kv8.vs[kg.vs_tile(h, pt) + dim];
       uint32_t u[2];
-      Kv8DecodeDword(w, st, &u[0], &u[1]);
+      if (kg.vb == 4) {  // keys (kk % 16) .. + 3 of the tile: pairs (kk % 8) / 2 and the next of dword (kk % 16) / 8
+        Kv4DecodePairs(StreamLoad(a.kv8.vq + kg.vq_tile(h, pt) + size_t(dim) * 2 + (kk % 16) / 8), st, (kk % 8) / 2, 2, u);
+      } else {
+        const uint32_t w = StreamLoad(a.kv8.vq + kg.vq_tile(h, pt) + size_t(dim) * 4 + (kk % 16) / 4);
+        Kv8DecodeDword(w, st, &u[0], &u[1]);
+      }
 #pragma unroll
       for (int e = 0; e < 4; ++e)  // keys at or past the end are zero in the image
         if (kk + e >= n_keys) u[e / 2] &= e % 2 ? 0x0000FFFFu : 0xFFFF0000u;
@@ -688,7 +726,7 @@ __global__ __launch_bounds__(256) void PrefillAttendImg(const PrefillArgs a, con
     const int t = min(qpos[i], a.chunk_len - 1), hd = min(head[i], G - 1);
     const uint16_t* qp = a.q + ((size_t(s) * a.chunk_len + t) * g.n_q + size_t(h) * G + hd) * D;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) qb[i][ks] = QueryF16(qp + 32 * ks + 8 * jg);
+    for (int ks = 0; ks < KS; ++ks) qb[i][ks] = QueryF16(qp + 32 * ks + 8 * jg, a.q_is_f16 != 0);
   }
   f4v o[RB][NDT];
   float m[RB];
@@ -1191,7 +1229,9 @@ extern "C" int yahkv_f16_prefill_attend(const yahkv_geometry* g, const yahkv_f16
 extern "C" size_t yahkv_kv8_prefill_workspace_bytes(const yahkv_geometry* g, int32_t n_seqs, int32_t max_prefix_len,
                                                     int32_t chunk_len) {
   if (CheckKv8Geometry(g) || n_seqs <= 0 || max_prefix_len < 0 || chunk_len <= 0) return 0;
-  return ImageBytes(MakeGeom(*g), n_seqs, max_prefix_len, chunk_len);
+  // 4-bit K: the chunk's rotated queries (f16) lie behind the images
+  const size_t rotated = Kv8BitsK(g->format) == 4 ? size_t(n_seqs) * chunk_len * g->n_q_heads * kKv8Dim * 2 : 0;
+  return ImageBytes(MakeGeom(*g), n_seqs, max_prefix_len, chunk_len) + rotated;
 }
 
 // Chunked-prefill attention over kv8a16 pools: the keys' f16 tile images are decoded from the pools with the reference's
@@ -1203,7 +1243,6 @@ extern "C" int yahkv_kv8_prefill_attend(const yahkv_geometry* g, const yahkv_kv8
                                         void* out, int32_t out_dtype, void* workspace, size_t workspace_bytes,
                                         void* stream) {
   if (const int rc = CheckKv8Pools(g, pools)) return rc;
-  if (g->format != YAHKV_KV8A16) return YAHKV_ERR_SHAPE;
   if (page_table == nullptr || prefix_len == nullptr) return YAHKV_ERR_ARG;
   if (n_seqs <= 0 || chunk_len <= 0 || max_prefix_len < 0 || page_table_stride <= 0) return YAHKV_ERR_ARG;
   PrefillArgs a{};
@@ -1215,11 +1254,19 @@ extern "C" int yahkv_kv8_prefill_attend(const yahkv_geometry* g, const yahkv_kv8
   const int tiles = TilesPerPair(max_prefix_len, chunk_len);
   if (int64_t(tiles) * (2 * kKeys * a.g.hd * 2) > 0x7fffffffLL) return YAHKV_ERR_SHAPE;
   if (const int rc = CheckWorkspace(a, workspace, workspace_bytes)) return rc;
+  if (workspace_bytes < yahkv_kv8_prefill_workspace_bytes(g, n_seqs, max_prefix_len, chunk_len)) return YAHKV_ERR_WORKSPACE;
   ImageArgs ia{};
   ia.g = a.g, ia.table = page_table, ia.stride = page_table_stride, ia.prefix_len = prefix_len, ia.n_seqs = n_seqs;
   ia.max_prefix = max_prefix_len, ia.chunk_len = chunk_len, ia.img = static_cast<char*>(workspace);
   ia.tiles_per_pair = tiles, ia.kv8 = MakeKv8Pools(*pools);
   hipStream_t st = static_cast<hipStream_t>(stream);
+  if (Kv8BitsK(g->format) == 4) {
+    uint16_t* rotated = reinterpret_cast<uint16_t*>(static_cast<char*>(workspace) + ImageBytes(a.g, n_seqs, max_prefix_len, chunk_len));
+    const int64_t rows = int64_t(n_seqs) * chunk_len * a.g.n_q;
+    hipLaunchKernelGGL(Kv4RotateQ, dim3(static_cast<unsigned>((rows + 3) / 4)), dim3(256), 0, st, a.q, rotated, rows);
+    if (const int rc = LaunchStatus()) return rc;
+    a.q = rotated, a.q_is_f16 = 1;
+  }
   hipLaunchKernelGGL(PrefillImagesKv8<0>, dim3(static_cast<unsigned>(tiles), static_cast<unsigned>(n_seqs * a.g.n_kv)),
                      dim3(256), 0, st, ia);
   if (const int rc = LaunchStatus()) return rc;
