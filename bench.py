@@ -43,6 +43,10 @@ WORKLOADS = {
     "ragged_b64_kv8a16": dict(fmt=816, batch=64, lo=1024, hi=65536, seed=4),
     "b1_ctx32k_kv8a16": dict(fmt=816, batch=1, lo=32768, hi=32768, seed=4, layers=8),
     "prefill_b8_ctx16k_chunk2k_kv8a16": dict(fmt=816, batch=8, lo=16384, hi=16384, seed=4, chunk=2048, warmup=10),
+    # ... and in its 4-bit sibling, kv4a16 (H256-rotated K in 16 levels per 32-dim group, V in 15 levels per tile)
+    "ragged_b64_kv4a16": dict(fmt=416, batch=64, lo=1024, hi=65536, seed=4),
+    "b16_ctx128k_kv4a16": dict(fmt=416, batch=16, lo=131072, hi=131072, seed=4, warmup=40),
+    "prefill_b8_ctx16k_chunk2k_kv4a16": dict(fmt=416, batch=8, lo=16384, hi=16384, seed=4, chunk=2048, warmup=10),
 }
 MFMA_F16_PEAK_TFLOPS = 2500.0
 EVENT_EVERY = 4      # decode workloads: HIP events around the split-K kernel on every fourth timed step
@@ -399,7 +403,8 @@ def run_kv8(a, wl, torch, yahkv):
     pages = (lens + total + PG - 1) // PG
     n_layers = wl.get("layers", 1)
     n_pages = int(pages.sum())                       # the pool fits the job exactly
-    g = yahkv.kv8_geometry(NQ, NKV, n_pages)
+    bits = 4 if wl["fmt"] == 416 else 8
+    g = yahkv.kv8_geometry(NQ, NKV, n_pages, bits, bits)
     alloc = yahkv.PagePool(n_pages)
     alloc.shuffle(12345)
     table = np.zeros((B, int(pages.max())), np.int32)
@@ -454,7 +459,10 @@ def run_kv8(a, wl, torch, yahkv):
         n = int(lens[s]) + 1
         hp, row = okv8.pools_of_sequence(layers[0], table[s], n)
         Kd, Vd = okv8.dense(hp, row, n)
-        err = max(err, closed_form_err(Kd, Vd, q[s].float().cpu().numpy(), scale, out[s].cpu().numpy()))
+        qs = q[s].float().cpu().numpy()
+        if bits == 4:                                # 4-bit K is stored rotated: the scores are taken against H256 q / 16
+            qs = okv8.rotate_q(qs)
+        err = max(err, closed_form_err(Kd, Vd, qs, scale, out[s].cpu().numpy()))
     if not err < 2e-3:
         raise SystemExit(f"bench.py: parity check failed before timing: max relative error {err:.3e}")
     for i in range(a.warmup):
@@ -466,17 +474,17 @@ def run_kv8(a, wl, torch, yahkv):
     torch.cuda.synchronize()
     ms = (time.perf_counter() - t0) / a.steps * 1e3
     kern_ms = float(np.mean([p[0].elapsed_time(p[1]) for p in ev[::EVENT_EVERY]]))
-    bpt = 2336                                           # kq 1024 + ks 32 + vq 1024 + vs 256 (architecture.md:219)
+    bpt = 2336 if bits == 8 else 1408                    # kq 1024 + ks 32 + vq 1024 + vs 256; 512 + 128 + 512 + 256 (architecture.md:219-220)
     tokens = [int(lens.sum()) + B * (2 + a.warmup + i) for i in range(a.steps)]
     kv_bytes = float(np.mean(tokens)) * bpt
     gbs, kgbs = kv_bytes / (ms * 1e-3) / 1e9, kv_bytes / (kern_ms * 1e-3) / 1e9
     return {
-        "metric": "paged kv8a16 KV decode-attn HBM GB/s (% of peak) + tok/s", "value": round(gbs, 1), "unit": "GB/s",
+        "metric": "paged kv%da16 KV decode-attn HBM GB/s (%% of peak) + tok/s" % bits, "value": round(gbs, 1), "unit": "GB/s",
         "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
         "config": {"workload": a.workload, "batch": B, "ctx_min": int(lens.min()), "ctx_max": int(lens.max()),
                    "ctx_sum": int(lens.sum()), "n_q_heads": NQ, "n_kv_heads": NKV, "head_dim": HD, "page_tokens": PG,
-                   "n_pages": n_pages, "layers_rotated": n_layers, "kv_format": "kv8a16",
+                   "n_pages": n_pages, "layers_rotated": n_layers, "kv_format": "kv%da16" % bits,
                    "step": "append 1 token/seq + paged decode attention (part, reduce with the open tile and the append in it)"},
         "pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2), "tok_per_s": round(B / (ms * 1e-3), 1),
         "kv_bytes_per_step": int(kv_bytes), "parity_max_rel_err": float(f"{err:.3e}"), "parity_rows": rows,
@@ -484,7 +492,7 @@ def run_kv8(a, wl, torch, yahkv):
         "roofline": {"bound": "hbm", "achieved": round(kgbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(kgbs / HBM_PEAK_GBS, 4), "traffic": TRAFFIC.get(a.workload, (None, None))[0],
                      "traffic_source": TRAFFIC.get(a.workload, (None, None))[1],
-                     "kernel": "Kv8Part<0>", "kernel_ms": round(kern_ms, 4)},
+                     "kernel": "Kv8Part<%d, %d>" % (bits, bits), "kernel_ms": round(kern_ms, 4)},
         "cpu_baseline": None}
 
 
@@ -493,7 +501,8 @@ def run_prefill_kv8(a, wl, torch, yahkv):
     16-key tiles), then one call that decodes prefix + chunk to f16 tile images and runs the causal attention."""
     B, chunk, prefix, PG = wl["batch"], wl["chunk"], wl["lo"], 256
     per_seq = (prefix + chunk + PG - 1) // PG
-    g = yahkv.kv8_geometry(NQ, NKV, B * per_seq)
+    bits = 4 if wl["fmt"] == 416 else 8
+    g = yahkv.kv8_geometry(NQ, NKV, B * per_seq, bits, bits)
     alloc = yahkv.PagePool(g.n_pages)
     alloc.shuffle(12345)
     table = np.stack([alloc.alloc(per_seq) for _ in range(B)]).astype(np.int32)
@@ -543,7 +552,10 @@ def run_prefill_kv8(a, wl, torch, yahkv):
         for t in (0, 1, chunk // 3, chunk // 2, chunk - 65, chunk - 1):
             for h in (0, 7, 13, NQ - 1):
                 kv = h // (NQ // NKV)
-                qv = q[s_, t, h].float().cpu().numpy().astype(np.float64)
+                qv = q[s_, t, h].float().cpu().numpy()
+                if bits == 4:                        # as the rotation kernel leaves it: H256 q / 16 rounded to f16
+                    qv = okv8.rotate_q(qv).astype(np.float16)
+                qv = qv.astype(np.float64)
                 sc = Kd[:prefix + t + 1, kv].astype(np.float64) @ qv * scale
                 p = np.exp(sc - sc.max())
                 want = (p / p.sum()) @ Vd[:prefix + t + 1, kv].astype(np.float64)
@@ -561,15 +573,15 @@ def run_prefill_kv8(a, wl, torch, yahkv):
     ms = (time.perf_counter() - t0) / a.steps * 1e3
     kern_ms = float(np.mean([p[0].elapsed_time(p[1]) for p in ev]))
     app_ms = float(np.median([p[0].elapsed_time(p[1]) for p in ev_app]))
-    app_bytes = B * chunk * (2 * NKV * HD * 2 + NKV * 2336)      # bf16 rows in, codes + scales + stats out
+    app_bytes = B * chunk * (2 * NKV * HD * 2 + (2336 if bits == 8 else 1408))   # bf16 rows in, codes + scales + stats out
     flops = float(B) * NQ * chunk * (prefix + (chunk + 1) / 2) * HD * 4
     return {
-        "metric": "chunked-prefill attention over paged kv8a16 KV, TFLOP/s (f16 MFMA) + tok/s",
+        "metric": "chunked-prefill attention over paged kv%da16 KV, TFLOP/s (f16 MFMA) + tok/s" % bits,
         "value": round(flops / (ms * 1e-3) / 1e12, 1), "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps,
         "warmup": a.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f16", "data": "synthetic",
         "config": {"workload": a.workload, "batch": B, "prefix": prefix, "chunk": chunk, "n_q_heads": NQ,
-                   "n_kv_heads": NKV, "head_dim": HD, "page_tokens": PG, "n_pages": g.n_pages, "kv_format": "kv8a16",
+                   "n_kv_heads": NKV, "head_dim": HD, "page_tokens": PG, "n_pages": g.n_pages, "kv_format": "kv%da16" % bits,
                    "step": "append chunk (quantize + scatter) + decode tiles to f16 + causal attention"},
         "tok_per_s": round(B * chunk / (ms * 1e-3), 1), "flops_per_step": int(flops),
         "parity_max_rel_err": float(f"{err:.3e}"), "out_fnv1a": first_hash,
@@ -582,7 +594,8 @@ def run_prefill_kv8(a, wl, torch, yahkv):
                      "frac": round(flops / (kern_ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
                      "traffic": TRAFFIC.get(a.workload, (None, None))[0],
                      "traffic_source": TRAFFIC.get(a.workload, (None, None))[1],
-                     "kernel": "PrefillImagesKv8<0> + PrefillAttendImg<%d, 3, 1, 6>" % HD, "kernel_ms": round(kern_ms, 4)},
+                     "kernel": ("Kv4RotateQ + " if bits == 4 else "") + "PrefillImagesKv8<0> + PrefillAttendImg<%d, 3, 1, 6>" % HD,
+                     "kernel_ms": round(kern_ms, 4)},
         "cpu_baseline": None}
 
 
@@ -935,13 +948,13 @@ def run_workload(a, torch, yahkv):
     wl = WORKLOADS[a.workload]
     if "chunk" in wl and wl["fmt"] == 16:
         return run_prefill_f16(a, wl, torch, yahkv)
-    if "chunk" in wl and wl["fmt"] == 816:
+    if "chunk" in wl and wl["fmt"] in (816, 416):
         return run_prefill_kv8(a, wl, torch, yahkv)
     if "chunk" in wl:
         return run_prefill(a, wl, torch, yahkv)
     if wl["fmt"] == 16:
         return run_f16(a, wl, torch, yahkv)
-    if wl["fmt"] == 816:
+    if wl["fmt"] in (816, 416):
         return run_kv8(a, wl, torch, yahkv)
     return run_decode(a, wl, torch, yahkv)
 

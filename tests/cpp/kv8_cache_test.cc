@@ -1,5 +1,5 @@
-// GPU test of the C++ host classes for the reference's own KV format (csrc/kv8_cache.hpp) against the CPU oracle of that
-// format (oracle/kv8_oracle.c): two prefill chunks of two sequences (the second chunk starts inside a 16-key tile), then
+// GPU test of the C++ host classes for the reference's own KV formats (csrc/kv8_cache.hpp; kv8a16, then kv4a16) against
+// the CPU oracle of those formats (oracle/kv8_oracle.c): two prefill chunks of two sequences (the second chunk starts inside a 16-key tile), then
 // decode steps that close tiles and cross a page, a third sequence that starts with decode steps; buffers bit-exact,
 // attention within 2e-3 of the float64 closed form over the oracle's dequantized model; and the host checks that throw
 // where the reference's LoomDecoder throws (engine/model/loom_decoder.hpp:186-203, 229-235).
@@ -55,6 +55,17 @@ void Closed(const std::vector<float>& Kd, const std::vector<float>& Vd, int n, c
     }
   }
 }
+// what the attention over 4-bit K scores against: H256 q / 16 per head, the prefill's rounded to f16 (yah_qrot)
+std::vector<float> Rotated(const float* q, int kb, bool to_f16) {
+  std::vector<float> out(q, q + size_t(NQ) * D);
+  if (kb != 4) return out;
+  for (int hq = 0; hq < NQ; ++hq) {
+    orc_kv4_rotate_q(q + hq * D, out.data() + hq * D);
+    if (to_f16)
+      for (int i = 0; i < D; ++i) out[size_t(hq) * D + i] = orc_f16_to_f32(orc_f32_to_f16(out[size_t(hq) * D + i]));
+  }
+  return out;
+}
 double RelErr(const float* got, const double* want, size_t n) {
   double d = 0, m = 0;
   for (size_t i = 0; i < n; ++i) d = std::max(d, std::fabs(got[i] - want[i])), m = std::max(m, std::fabs(want[i]));
@@ -65,16 +76,18 @@ struct HostPools {
   std::vector<uint32_t> kq, ks, vq, vs;
   std::vector<float> km;
   std::vector<uint16_t> vo;
-  HostPools()
-      : kq(size_t(P) * 256 * W / 4), ks(size_t(P) * 256 * W / 128), vq(size_t(H) * P * 16 * 256 * 4), vs(size_t(H) * P * 16 * 256),
+  HostPools(int kb, int vb)
+      : kq(size_t(P) * 256 * W / (kb == 4 ? 8 : 4)), ks(size_t(P) * 256 * W / (kb == 4 ? 32 : 128)),
+        vq(size_t(H) * P * 16 * 256 * (vb == 4 ? 2 : 4)), vs(size_t(H) * P * 16 * 256),
         km(size_t(P) * W), vo(size_t(P) * W * 16) {}
   orc_kv8_pools view() { return orc_kv8_pools{kq.data(), ks.data(), km.data(), vq.data(), vs.data(), vo.data()}; }
 };
 
-int RunTest() {
+int RunTest(int kb, int vb) {
   try {
-    const yahkv_geometry g{YAHKV_KV8A16, NQ, H, D, 256, P};
-    const orc_kv8_geometry og{NQ, H, P};
+    Stage(kb == 8 ? "kv8a16" : "kv4a16");
+    const yahkv_geometry g{kb == 8 ? YAHKV_KV8A16 : YAHKV_KV4A16, NQ, H, D, 256, P};
+    const orc_kv8_geometry og{NQ, H, P, kb, vb};
     const int B = 2, T = 600, chunk0 = 100, chunk1 = 150, steps = 30;
     std::mt19937 rng(11);
     std::normal_distribution<float> nd;
@@ -103,10 +116,10 @@ int RunTest() {
       ExpectThrow([&] { dec.Bind(small); }, "Bind must reject a missing buffer");
     }
     dec.Bind(st);
-    Expect(dec.KqBytes() == size_t(P) * 256 * W && dec.VsBytes() == size_t(P) * 16 * W * 4, "pool byte formulas");
+    Expect(dec.KqBytes() == size_t(P) * 256 * W / (kb == 4 ? 2 : 1) && dec.VsBytes() == size_t(P) * 16 * W * 4, "pool byte formulas");
     for (const BufferRef* r : {&st.kq, &st.ks, &st.vq, &st.vs, &st.vopen})  // poison: what is not written stays
       CheckHip(hipMemset(r->ptr, 0x5A, r->length), "poison");
-    HostPools hp;
+    HostPools hp(kb, vb);
     std::memset(hp.kq.data(), 0x5A, hp.kq.size() * 4), std::memset(hp.ks.data(), 0x5A, hp.ks.size() * 4);
     std::memset(hp.vq.data(), 0x5A, hp.vq.size() * 4), std::memset(hp.vs.data(), 0x5A, hp.vs.size() * 4);
     std::memset(hp.vo.data(), 0x5A, hp.vo.size() * 2);
@@ -162,7 +175,7 @@ int RunTest() {
         for (int t : {0, 17, chunk - 1}) {
           std::vector<double> want(size_t(NQ) * D);
           const size_t qo = (size_t(s) * chunk + t) * NQ * D;
-          Closed(Kd, Vd, prefix[size_t(s)] + t + 1, qf.data() + qo, want.data());
+          Closed(Kd, Vd, prefix[size_t(s)] + t + 1, Rotated(qf.data() + qo, kb, true).data(), want.data());
           worst_prefill = std::max(worst_prefill, RelErr(got.data() + qo, want.data(), want.size()));
         }
         prefix[size_t(s)] = n;
@@ -193,7 +206,7 @@ int RunTest() {
         std::vector<float> Kd(size_t(n) * W), Vd(size_t(n) * W);
         orc_kv8_dense(&og, &op, table.data() + size_t(s) * stride, n, Kd.data(), Vd.data());
         std::vector<double> want(size_t(NQ) * D);
-        Closed(Kd, Vd, n, q1.data() + size_t(s) * NQ * D, want.data());
+        Closed(Kd, Vd, n, Rotated(q1.data() + size_t(s) * NQ * D, kb, false).data(), want.data());
         worst_decode = std::max(worst_decode, RelErr(got.data() + size_t(s) * NQ * D, want.data(), want.size()));
       }
     }
@@ -204,7 +217,7 @@ int RunTest() {
                 "a step inside a tile the open tile does not cover must throw");
     dec.Release(0), dec.Release(1), dec.Release(2);
     Expect(dec.free_pages() == P, "every page back in the pool");
-    std::printf("kv8_cache_test: ok (prefill %.2e, decode %.2e)\n", worst_prefill, worst_decode);
+    std::printf("kv8_cache_test: ok, kv%da16 (prefill %.2e, decode %.2e)\n", kb, worst_prefill, worst_decode);
     return 0;
   } catch (const std::exception& e) {
     std::printf("kv8_cache_test: FAILED: %s\n", e.what());
@@ -213,4 +226,7 @@ int RunTest() {
 }
 }  // namespace
 
-int main() { return RunTest(); }
+int main() {
+  if (const int rc = RunTest(8, 8)) return rc;
+  return RunTest(4, 4);
+}

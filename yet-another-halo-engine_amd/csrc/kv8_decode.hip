@@ -65,9 +65,15 @@ void Kv8Part(const DecodeArgs a, const Kv8Pools pools) {
   auto& lk = lk_all[wave];
 
   if (a.stamps != nullptr && threadIdx.x == 0) a.stamps[blockIdx.x] = wall_clock64();
+  // Which chunk of the line this workgroup takes. Workgroup k runs on XCD k % 8; with chunk k the kv heads of a sequence,
+  // neighbours on the line, would read the same rows of `ks` (a token's scale pairs of all kv heads share a 32- or
+  // 128-byte row) through four different L2 caches at about the same time. Neighbouring chunks therefore go to the same
+  // XCD: XCD x takes chunks x n / 8 .. (x + 1) n / 8 - 1.
+  const int chunk_id = a.n_chunks % 8 == 0 ? static_cast<int>(blockIdx.x % 8) * (a.n_chunks / 8) + static_cast<int>(blockIdx.x / 8)
+                                           : static_cast<int>(blockIdx.x);
   bool any_empty = false;
-  const int4 rec_v = a.n_seqs <= 64 ? ChunkRecordWave(a, blockIdx.x, wave, lane, &chunk_rec, chunk_tiles, &any_empty)
-                                    : ChunkRecord<64 * kWavesPerGroup>(a, blockIdx.x, wave_sum, &chunk_rec, chunk_tiles, &any_empty);
+  const int4 rec_v = a.n_seqs <= 64 ? ChunkRecordWave(a, chunk_id, wave, lane, &chunk_rec, chunk_tiles, &any_empty)
+                                    : ChunkRecord<64 * kWavesPerGroup>(a, chunk_id, wave_sum, &chunk_rec, chunk_tiles, &any_empty);
   // (the record is the same in every lane: scalar registers for it and for everything derived from it)
   const int4 rec = {__builtin_amdgcn_readfirstlane(rec_v.x), __builtin_amdgcn_readfirstlane(rec_v.y),
                     __builtin_amdgcn_readfirstlane(rec_v.z), __builtin_amdgcn_readfirstlane(rec_v.w)};
@@ -277,11 +283,11 @@ void Kv8Part(const DecodeArgs a, const Kv8Pools pools) {
     }
   };
   auto leave_empty = [&]() {
-    const size_t part = PartialIndex(a, blockIdx.x, wave, cur) * G;
+    const size_t part = PartialIndex(a, chunk_id, wave, cur) * G;
     if (lane < G) StoreDevice2(DeviceBuffer(a.ml + part * 2), lane * 8, kNegMax, 0.0f);
   };
   auto leave_partial = [&]() {
-    const size_t part = PartialIndex(a, blockIdx.x, wave, cur) * G;
+    const size_t part = PartialIndex(a, chunk_id, wave, cur) * G;
     const auto rml = DeviceBuffer(a.ml + part * 2), racc = DeviceBuffer(a.acc + part * D);
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
