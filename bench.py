@@ -960,8 +960,8 @@ def run_workload(a, torch, yahkv):
 
 
 # what the default run times besides its own workload: the other configurations of the benchmark that fill a GPU
-ALSO = ["b1_ctx32k_q8_0", "prefill_b8_ctx16k_chunk2k_q8_0", "b16_ctx128k_q4_0", "ragged_b64_kv8a16", "ragged_b64_f16",
-        "prefill_b8_ctx16k_chunk2k_q4_0"]
+ALSO = ["b1_ctx32k_q8_0", "prefill_b8_ctx16k_chunk2k_q8_0", "b16_ctx128k_q4_0", "ragged_b64_kv8a16", "ragged_b64_kv4a16",
+        "ragged_b64_f16", "prefill_b8_ctx16k_chunk2k_q4_0"]
 
 
 def main():

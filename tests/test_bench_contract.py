@@ -48,7 +48,7 @@ def test_decode_line_has_the_fields_a_driver_reads():
     assert d["parity_max_rel_err"] < 2e-3
     # the other configurations that fill a GPU are timed by the same run, into one object of the same line
     assert sorted(d["also"]) == ["b16_ctx128k_q4_0", "b1_ctx32k_q8_0", "prefill_b8_ctx16k_chunk2k_q4_0",
-                                 "prefill_b8_ctx16k_chunk2k_q8_0", "ragged_b64_f16", "ragged_b64_kv8a16"]
+                                 "prefill_b8_ctx16k_chunk2k_q8_0", "ragged_b64_f16", "ragged_b64_kv4a16", "ragged_b64_kv8a16"]
     for name, r in d["also"].items():
         assert r["value"] > 0 and r["ms_per_step"] > 0 and r["parity_max_rel_err"] < 2e-3, name
         assert 0.0 < r["roofline"]["frac"] < 1.0 and r["roofline"]["bound"] == ("mfma" if "prefill" in name else "hbm")
