@@ -502,6 +502,30 @@ int yahkv_kv8_decode_step(const yahkv_geometry* g, const yahkv_kv8_pools* pools,
                           const void* k_new, const void* v_new, int32_t new_dtype, const void* q, int32_t q_dtype,
                           float softmax_scale, const float* gate, float* out, void* workspace, size_t workspace_bytes,
                           const yahkv_decode_options* opt, void* stream);
+/* The reference's own slot files ("YAHSLOT1": LoomPrefill::SaveState / LoadState, engine/model/loom_prefill.hpp:976-1024):
+ * five u64 {magic, T, B, chunks, nbufs = 10}, then per buffer a u64 byte count and the raw bytes, in the order page
+ * table, kq, ks, km, vq, vs, f16 K pool, f16 V^T pool, convolution rings, DeltaNet states (StateBuffers(), :1027-1030);
+ * the KV buffers hold all full-attention layers one after the other, in the layouts above. parse validates a file held
+ * in host memory (magic, counts, truncation, sizes that fit one of the four quantized formats with four kv heads, page
+ * table entries in range) and reports what it holds; load_layer copies one layer's pages covering chunks * B tokens,
+ * through the slot's page table, into pages[0 .. n) of the caller's pools (host int32, logical order; any free pages),
+ * and the layer's channel means to km of pages[0]. The stream is synchronized before it returns. The recurrent states in
+ * the file are skipped: they are not part of this library. */
+typedef struct yahkv_refslot_info {
+  uint64_t context;     /* T: the context the set was built for */
+  uint64_t chunk;       /* B: its chunk size */
+  uint64_t chunks;      /* chunks the slot covers: chunks * B tokens */
+  int32_t n_pages;      /* entries of the slot's page table = 256-token pages of its pools */
+  int32_t n_layers;     /* full-attention layers in the file */
+  int32_t n_kv_heads;   /* 4 */
+  int32_t format;       /* YAHKV_KV8A16, YAHKV_KV4A16, YAHKV_K8V4A16 or YAHKV_K4V8A16 */
+  uint64_t offset[10];  /* where each buffer's bytes start in the file, and how many there are */
+  uint64_t size[10];
+} yahkv_refslot_info;
+int yahkv_refslot_parse(const void* file, size_t file_bytes, yahkv_refslot_info* info);
+int yahkv_refslot_load_layer(const yahkv_geometry* g, const yahkv_kv8_pools* pools, const void* file, size_t file_bytes,
+                             int32_t layer, const int32_t* pages, int32_t n_pages, void* stream);
+
 /* Chunked-prefill attention over kv8a16 pools after the chunk has been appended (arguments as yahkv_prefill_attend;
  * the workspace is required): keys 0 .. prefix_len[s] + chunk_len are decoded once into f16 tiles with the
  * reference's own decode, one f16 fma f16(1 + u / 256) * S + C' per element, every V tile from codes (yah_kdeq8 /

@@ -632,6 +632,32 @@ class Kv8Pools:
             getattr(self, n).copy_(torch.from_numpy(np.ascontiguousarray(a).view(np.uint8).reshape(-1)))
 
 
+class RefSlotInfo(C.Structure):
+    _fields_ = [("context", C.c_uint64), ("chunk", C.c_uint64), ("chunks", C.c_uint64), ("n_pages", C.c_int32),
+                ("n_layers", C.c_int32), ("n_kv_heads", C.c_int32), ("format", C.c_int32), ("offset", C.c_uint64 * 10),
+                ("size", C.c_uint64 * 10)]
+
+
+def refslot_parse(file_bytes):
+    """Validates a slot file of the reference ("YAHSLOT1", loom_prefill.hpp:976-1024) held in a bytes-like object or a
+    uint8 numpy array and says what it holds. Host only."""
+    import numpy as np
+    buf = np.frombuffer(file_bytes, np.uint8) if not isinstance(file_bytes, np.ndarray) else file_bytes
+    info = RefSlotInfo()
+    _check(lib.yahkv_refslot_parse(C.c_void_p(buf.ctypes.data), C.c_size_t(buf.size), C.byref(info)), "refslot_parse")
+    return info
+
+
+def refslot_load_layer(pools, file_bytes, layer, pages):
+    """One layer's pages of a reference slot file into pages[...] (logical order) of kv8a16 / kv4a16 pools."""
+    import numpy as np
+    buf = np.frombuffer(file_bytes, np.uint8) if not isinstance(file_bytes, np.ndarray) else file_bytes
+    pg = np.ascontiguousarray(pages, np.int32)
+    g, st = pools.geom, pools.struct()
+    _check(lib.yahkv_refslot_load_layer(C.byref(g), C.byref(st), C.c_void_p(buf.ctypes.data), C.c_size_t(buf.size),
+                                        int(layer), C.c_void_p(pg.ctypes.data), int(pg.size), _stream()), "refslot_load_layer")
+
+
 def kv8_kmean(pools, table, k_src, n_valid=None):
     """Channel means of each sequence's first chunk k_src [n_seqs][n_rows][H][256], written to km of its first page."""
     g = pools.geom

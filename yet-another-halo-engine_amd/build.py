@@ -7,7 +7,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 LIB = os.path.join(HERE, "libyahkv.so")
 SOURCES = ["host.cpp", "append.hip", "decode.hip", "prefill.hip", "slots.hip", "f16kv.hip", "kv8_append.hip",
-           "kv8_decode.hip"]
+           "kv8_decode.hip", "refslot.cpp"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wextra",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",   # no packed-FP32 VALU forms
