@@ -52,7 +52,13 @@ struct DecodeArgs {
   // closed tiles only, keys 0 .. 16 * ((len - 1) / 16) - 1 whether or not len counts a token still to be appended, and
   // the merge adds the open tile's keys.
   int32_t open_tile;
+  // Pools in which the kv heads of a token share rows (the reference's own formats: a token's K scale pairs of all kv
+  // heads lie in one row): tile_mult = H cuts the line by (sequence, tile) with the kv heads of a tile next to each
+  // other, so that the waves of a workgroup read a row's heads at the same time. A sequence is then one pair of
+  // H x tiles items, item j = (tile j / H, kv head j % H). 0 or 1: the line is cut by (sequence, kv head).
+  int32_t tile_mult;
 };
+__device__ __forceinline__ int CutHeads(const DecodeArgs& a) { return a.tile_mult > 1 ? 1 : a.g.n_kv; }
 // The step's own token for the reduce kernel: K / V rows [n_seqs][H][D] of `dtype`, or null pointers.
 struct StepRows {
   const void* k;
@@ -108,7 +114,9 @@ __device__ __forceinline__ int ChunkOf(const DecodeArgs& a, long long A, long lo
 // leaves a partial and fetches new queries: about eight tiles' worth per workgroup, measured), then one unit per
 // tile. Cutting this line evenly gives chunks of equal time rather than of equal tiles: without it the workgroups
 // finish up to 50 us apart, by the number of pairs their chunks hold.
-__device__ __forceinline__ int TilesOf(const DecodeArgs& a, int s) { return (ClampLen(a, s) + kTile - 1) / kTile; }
+__device__ __forceinline__ int TilesOf(const DecodeArgs& a, int s) {
+  return (ClampLen(a, s) + kTile - 1) / kTile * max(a.tile_mult, 1);
+}
 __device__ __forceinline__ int UnitsOf(const DecodeArgs& a, int ts) { return ts > 0 ? ts + a.pair_cost : 0; }
 // (Divisions of line coordinates: 64-bit divisions by run-time values are long sequences of scalar instructions, which
 // every wave of the merge kernel would repeat; a line below 2^31 units, any real one, takes the 32-bit form.)
@@ -130,7 +138,7 @@ __device__ __forceinline__ long long ChunkUnits(const DecodeArgs& a, long long l
 template <int NT>
 __device__ __forceinline__ int4 ChunkRecord(const DecodeArgs& a, int k, int (*wave_sum)[2], int4* found, long long* tiles_at,
                                             bool* any_empty) {
-  const int t = threadIdx.x, H = a.g.n_kv, c = a.pair_cost;
+  const int t = threadIdx.x, H = CutHeads(a), c = a.pair_cost;
   const int per = (a.n_seqs + NT - 1) / NT;
   const int s0 = min(t * per, a.n_seqs), s1 = min(s0 + per, a.n_seqs);
   int sum = 0, cnt = 0;  // units of the slice, and sequences in it that are not empty
@@ -198,7 +206,7 @@ __device__ __forceinline__ int4 ChunkRecord(const DecodeArgs& a, int k, int (*wa
 // the merge at the kernel's end (which reads it behind a barrier).
 __device__ __forceinline__ int4 ChunkRecordWave(const DecodeArgs& a, int k, int wave, int lane, int4* found, long long* tiles_at,
                                                 bool* any_empty) {
-  const int H = a.g.n_kv, c = a.pair_cost;
+  const int H = CutHeads(a), c = a.pair_cost;
   const int ts = lane < a.n_seqs ? TilesOf(a, lane) : 0, units = UnitsOf(a, ts), cnt = ts > 0;
   *any_empty = __builtin_amdgcn_ballot_w64(lane < a.n_seqs && ts == 0) != 0;
   int incl = units, incl_cnt = cnt;
@@ -253,10 +261,10 @@ __device__ __forceinline__ bool NextPair(const DecodeArgs& a, int chunk_n, PairC
   c->base += c->n, c->first = 0;
   int ts = 0;
   do {  // empty sequences have no tiles on the line
-    if (++c->h == a.g.n_kv) c->h = 0, ++c->s;
+    if (++c->h == CutHeads(a)) c->h = 0, ++c->s;
     if (c->s >= a.n_seqs) return false;
     ts = TilesOf(a, c->s);
-    if (ts == 0) c->h = a.g.n_kv - 1;
+    if (ts == 0) c->h = CutHeads(a) - 1;
   } while (ts == 0);
   c->n = min(ts, chunk_n - c->base), c->len = ClampLen(a, c->s);
   return true;
@@ -442,7 +450,9 @@ inline Plan MakePlan(const Geom& g, int32_t n_seqs, int32_t max_seq_len, const T
   // rounding leaves a few 8192ths over or short: the last chunks take them, none going below its bound
   for (int j = 8, over = p.share[8] - 8192; j >= 1; --j) p.share[j] = std::min(p.share[j] - over, 8192 - 512 * (8 - j));
   p.share[8] = 8192;
-  const size_t parts = (size_t(p.n_chunks) + size_t(n_seqs) * g.n_kv) * p.wpc;
+  // (the formats whose line is cut by (sequence, tile), DecodeArgs::tile_mult, keep a row of places per kv head)
+  const bool by_tile = g.format > 16 && g.n_kv > 1 && kWavesPerGroup % g.n_kv == 0;
+  const size_t parts = (by_tile ? (size_t(p.n_chunks) + size_t(n_seqs)) * g.n_kv : size_t(p.n_chunks) + size_t(n_seqs) * g.n_kv) * p.wpc;
   p.off_tprefix = 0;
   p.off_tickets = Align(sizeof(int32_t) * (size_t(n_seqs) + 1));
   p.off_ml = Align(p.off_tickets + sizeof(unsigned long long) * size_t(n_seqs) * g.n_kv);

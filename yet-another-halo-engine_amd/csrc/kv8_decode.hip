@@ -65,12 +65,7 @@ void Kv8Part(const DecodeArgs a, const Kv8Pools pools) {
   auto& lk = lk_all[wave];
 
   if (a.stamps != nullptr && threadIdx.x == 0) a.stamps[blockIdx.x] = wall_clock64();
-  // Which chunk of the line this workgroup takes. Workgroup k runs on XCD k % 8; with chunk k the kv heads of a sequence,
-  // neighbours on the line, would read the same rows of `ks` (a token's scale pairs of all kv heads share a 32- or
-  // 128-byte row) through four different L2 caches at about the same time. Neighbouring chunks therefore go to the same
-  // XCD: XCD x takes chunks x n / 8 .. (x + 1) n / 8 - 1.
-  const int chunk_id = a.n_chunks % 8 == 0 ? static_cast<int>(blockIdx.x % 8) * (a.n_chunks / 8) + static_cast<int>(blockIdx.x / 8)
-                                           : static_cast<int>(blockIdx.x);
+  const int chunk_id = static_cast<int>(blockIdx.x);
   bool any_empty = false;
   const int4 rec_v = a.n_seqs <= 64 ? ChunkRecordWave(a, chunk_id, wave, lane, &chunk_rec, chunk_tiles, &any_empty)
                                     : ChunkRecord<64 * kWavesPerGroup>(a, chunk_id, wave_sum, &chunk_rec, chunk_tiles, &any_empty);
@@ -79,7 +74,12 @@ void Kv8Part(const DecodeArgs a, const Kv8Pools pools) {
                     __builtin_amdgcn_readfirstlane(rec_v.z), __builtin_amdgcn_readfirstlane(rec_v.w)};
   if (rec.x < 0) return;
   const int chunk_n = rec.w;
-  const bool fixed_pattern = a.deterministic || chunk_n <= kWavesPerGroup;  // (at most one tile per wave: no hand-out)
+  // The line's items: tiles of a (sequence, kv head) pair, or, with a.tile_mult = H, the H kv heads of a sequence's tiles
+  // one after the other. There wave w of the fixed pattern keeps its kv head as long as it stays with a sequence (its
+  // items are eight apart and H divides eight), and the waves of a workgroup take the heads of a tile side by side:
+  // the row of `ks` that holds a token's scale pairs of all heads is fetched once instead of once per head.
+  const int lg_mult = a.tile_mult > 1 ? __builtin_ctz(static_cast<unsigned>(a.tile_mult)) : 0;
+  const bool fixed_pattern = a.deterministic || chunk_n <= kWavesPerGroup || lg_mult > 0;  // (one tile per wave: no hand-out)
   if (!fixed_pattern) {
     if (threadIdx.x == 0) next_tile = 0;
     __syncthreads();
@@ -122,6 +122,7 @@ void Kv8Part(const DecodeArgs a, const Kv8Pools pools) {
   const int prow = n16 < 4 ? n16 : (n16 >= 8 && n16 < 12 ? n16 - 4 : 0);
 
   PairCursor cur = FirstPair(a, rec);
+  int head = 0;  // the kv head of the wave's current items
   const int32_t* row = nullptr;
   typedef const int32_t __attribute__((address_space(4))) * ConstRow;
   // a 64-key tile lies inside one 256-token page
@@ -136,7 +137,7 @@ void Kv8Part(const DecodeArgs a, const Kv8Pools pools) {
     if constexpr (KB == 4) {
       // eight rows per instruction; lane l of instruction i carries chunk (l % 8) ^ (row % 8) of row 8 i + l / 8
       const auto rk4 = __builtin_amdgcn_make_buffer_rsrc(
-          reinterpret_cast<uint8_t*>(pools.kq) + (row0 * H + cur.h) * 128, 0, 0x7fffffff, 0x00020000);
+          reinterpret_cast<uint8_t*>(pools.kq) + (row0 * H + head) * 128, 0, 0x7fffffff, 0x00020000);
       const uint32_t r = lane / 8, c = lane % 8;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
@@ -144,12 +145,12 @@ void Kv8Part(const DecodeArgs a, const Kv8Pools pools) {
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rk4, (__attribute__((address_space(3))) void*)(&lk[i * 1024]), 16,
                                                  rr * (H * 128) + ((c ^ (rr & 7)) << 4), 0, 0, kStreamed);
       }
-      const uint32_t* sp4 = pools.ks + ((row0 + n32) * H + cur.h) * 8;
+      const uint32_t* sp4 = pools.ks + ((row0 + n32) * H + head) * 8;
       ksc4[0] = StreamLoad(reinterpret_cast<const uint4*>(sp4));
       ksc4[1] = StreamLoad(reinterpret_cast<const uint4*>(sp4 + 4));
     } else {
       const auto rk = __builtin_amdgcn_make_buffer_rsrc(
-          reinterpret_cast<uint8_t*>(pools.kq) + (row0 * H + cur.h) * 256, 0, 0x7fffffff, 0x00020000);
+          reinterpret_cast<uint8_t*>(pools.kq) + (row0 * H + head) * 256, 0, 0x7fffffff, 0x00020000);
       const uint32_t r = lane / 16, c = lane % 16;
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
@@ -157,14 +158,14 @@ void Kv8Part(const DecodeArgs a, const Kv8Pools pools) {
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, (__attribute__((address_space(3))) void*)(&lk[i * 1024]), 16,
                                                  rr * (H * 256) + ((c ^ (rr & 15)) << 4), 0, 0, kStreamed);
       }
-      const uint32_t* sp = pools.ks + ((row0 + n32) * H + cur.h) * 2;
+      const uint32_t* sp = pools.ks + ((row0 + n32) * H + head) * 2;
       ksc = StreamLoad(reinterpret_cast<const uint2*>(sp));
     }
   };
   auto fetch_v = [&](int tile, int hf, int page) {
     const size_t pt = size_t(page) * 16 + (tile % 4) * 4 + kg;
-    const uint32_t* vp = pools.vq + ((size_t(cur.h) * tiles16 + pt) * 256 + 128 * hf + n16) * (VB == 4 ? 2 : 4);
-    const uint32_t* sp = pools.vs + (size_t(cur.h) * tiles16 + pt) * 256 + 128 * hf + n16;
+    const uint32_t* vp = pools.vq + ((size_t(head) * tiles16 + pt) * 256 + 128 * hf + n16) * (VB == 4 ? 2 : 4);
+    const uint32_t* sp = pools.vs + (size_t(head) * tiles16 + pt) * 256 + 128 * hf + n16;
     if constexpr (VB == 4) {
 #pragma unroll
       for (int j = 0; j < NT / 2; ++j) vb4[j] = StreamLoad(reinterpret_cast<const uint2*>(vp + 32 * j));
@@ -176,10 +177,19 @@ void Kv8Part(const DecodeArgs a, const Kv8Pools pools) {
     for (int j = 0; j < NT / 2; ++j) vst[j] = StreamLoad(sp + 16 * j);
   };
   // scores of the 32 keys in the LDS slot against all heads: the two 128-dim halves are two accumulator chains
+  // `(x & mask) | one` is one instruction (v_and_or_b32) only if neither constant is a literal, which that encoding does
+  // not take: the mask is handed to the compiler in a scalar register and the f16 pair (1.0, 1.0) in a vector register,
+  // both behind an empty asm it cannot see through (with literals it emits an `and` and an `or`: a third more
+  // instructions for every pair of codes).
+  // (8-bit codes keep the literals: that kernel is bound by memory, and the register this takes costs it spills.)
+  uint32_t one2 = 0x3c003c00u, mask4 = 0x03c003c0u;
+  if constexpr (KB == 4 || VB == 4) {
+    asm volatile("" : "+v"(one2));
+    asm volatile("" : "+s"(mask4));
+  }
   // a dword of eight 4-bit codes (dims 2 j / 2 j + 1 at bits 4 j / 16 + 4 j) as the f16 values 1 + u / 16 in dim order
-  auto nibbles_f16 = [](uint32_t w) -> h8v {
-    const uint4 k = {((w << 6) & 0x03c003c0u) | 0x3c003c00u, ((w << 2) & 0x03c003c0u) | 0x3c003c00u,
-                     ((w >> 2) & 0x03c003c0u) | 0x3c003c00u, ((w >> 6) & 0x03c003c0u) | 0x3c003c00u};
+  auto nibbles_f16 = [&](uint32_t w) -> h8v {
+    const uint4 k = {((w << 6) & mask4) | one2, ((w << 2) & mask4) | one2, ((w >> 2) & mask4) | one2, ((w >> 6) & mask4) | one2};
     return __builtin_bit_cast(h8v, k);
   };
   auto scores = [&](int tt) {
@@ -282,12 +292,27 @@ void Kv8Part(const DecodeArgs a, const Kv8Pools pools) {
       o[nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa1, v1, o[nt], 0, 0, 0);
     }
   };
+  // partial of (this chunk, this wave, the current sequence, kv head h)
+  // (chunk + pair counts a wave's places along the line without collisions as long as pairs follow each other on it;
+  // with a sequence as the pair, every kv head has a row of places of its own)
+  auto part_of = [&](int h) -> size_t {
+    if (lg_mult > 0) return ((size_t(h) * (a.n_chunks + a.n_seqs) + chunk_id + cur.s) * a.wpc + wave) * G;
+    return ((size_t(chunk_id) + size_t(cur.s) * H + h) * a.wpc + wave) * G;
+  };
+  auto empty_at = [&](int h) {
+    if (lane < G) StoreDevice2(DeviceBuffer(a.ml + part_of(h) * 2), lane * 8, kNegMax, 0.0f);
+  };
+  // (with the heads of a tile dealt to the waves, a wave's partial belongs to one head of the sequence; the merge of
+  // another head finds this wave's place for that head empty)
   auto leave_empty = [&]() {
-    const size_t part = PartialIndex(a, chunk_id, wave, cur) * G;
-    if (lane < G) StoreDevice2(DeviceBuffer(a.ml + part * 2), lane * 8, kNegMax, 0.0f);
+    if (lg_mult == 0) return empty_at(cur.h);
+    for (int h = 0; h < H; ++h) empty_at(h);
   };
   auto leave_partial = [&]() {
-    const size_t part = PartialIndex(a, chunk_id, wave, cur) * G;
+    if (lg_mult > 0)
+      for (int h = 0; h < H; ++h)
+        if (h != head) empty_at(h);
+    const size_t part = part_of(lg_mult > 0 ? head : cur.h);
     const auto rml = DeviceBuffer(a.ml + part * 2), racc = DeviceBuffer(a.acc + part * D);
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
@@ -320,7 +345,9 @@ void Kv8Part(const DecodeArgs a, const Kv8Pools pools) {
     // ---- first tile of this wave in the pair: query operands, the constants' shares, empty state, first loads
     row = a.table + int64_t(cur.s) * a.stride;
     const int live16 = cur.len / 16;  // closed 16-key tiles of the pair (cur.len is a multiple of 16)
-    int tile = cur.first + (idx - cur.base);
+    const int item = cur.first + (idx - cur.base);
+    head = lg_mult > 0 ? item & (a.tile_mult - 1) : cur.h;
+    int tile = item >> lg_mult;
     int pgc = load_page(tile), pgn;
     load_k(tile, 0, pgc);
     fetch_v(tile, 1, pgc);  // not used: keeps the count of loads in flight at the loop's head the same on every pass
@@ -337,7 +364,7 @@ void Kv8Part(const DecodeArgs a, const Kv8Pools pools) {
         const int mm = lane / 16 + 4 * e;
         const int d0 = 32 * (mm / 2) + 8 * (2 * hf + mm % 2);
         h8v qv = {0, 0, 0, 0, 0, 0, 0, 0};
-        if (rw < G) qv = LoadQ8(a.q, (size_t(cur.s) * g.n_q + size_t(cur.h) * G + rw) * D + d0, a.q_dtype);
+        if (rw < G) qv = LoadQ8(a.q, (size_t(cur.s) * g.n_q + size_t(head) * G + rw) * D + d0, a.q_dtype);
 #pragma unroll
         for (int k = 0; k < 8; ++k) x[e][k] = static_cast<float>(qv[k]);
 #pragma unroll
@@ -393,7 +420,7 @@ void Kv8Part(const DecodeArgs a, const Kv8Pools pools) {
         const int i = lane + 64 * e, mm = i / 16, hf = (i / 8) % 2, rw = i % 8;
         const int d0 = 16 * (2 * (mm / 2) + hf) + 8 * (mm % 2);
         h8v qv = {0, 0, 0, 0, 0, 0, 0, 0};
-        if (rw < G) qv = LoadQ8(a.q, (size_t(cur.s) * g.n_q + size_t(cur.h) * G + rw) * D + d0, a.q_dtype);
+        if (rw < G) qv = LoadQ8(a.q, (size_t(cur.s) * g.n_q + size_t(head) * G + rw) * D + d0, a.q_dtype);
         float t = 0.0f;
 #pragma unroll
         for (int k = 0; k < 8; ++k) t += static_cast<float>(qv[k]);
@@ -418,7 +445,7 @@ void Kv8Part(const DecodeArgs a, const Kv8Pools pools) {
     while (true) {
       const int nidx = take();
       const bool has_next = nidx < cur.base + cur.n;
-      const int ntile = cur.first + (nidx - cur.base);
+      const int ntile = (cur.first + (nidx - cur.base)) >> lg_mult;
       pgn = load_page(has_next ? ntile : tile);
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
@@ -662,12 +689,19 @@ __global__ __launch_bounds__(kReduceThreads) void Kv8Reduce(const DecodeArgs a, 
   const int n_extra = n_tail + (step ? 1 : 0);  // 1 .. 17
   size_t p0 = 0, p1 = 0;
   if (ts > 0) {
-    const long long A_ = ChunkUnits(a, static_cast<long long>(a.tprefix[a.n_seqs]) * H);
+    // (with the kv heads dealt to the waves the sequence is one pair on the line, and this head's partials lie among
+    // those of all the chunks that hold a piece of the sequence)
+    const int Hc = CutHeads(a);
+    const long long A_ = ChunkUnits(a, static_cast<long long>(a.tprefix[a.n_seqs]) * Hc);
     const int pair = s * H + h;
-    const long long first =
-        static_cast<long long>(a.tprefix[s]) * H + static_cast<long long>(h) * UnitsOf(a, ts) + a.pair_cost;
+    const long long first = static_cast<long long>(a.tprefix[s]) * Hc +
+                            static_cast<long long>(Hc == 1 ? 0 : h) * UnitsOf(a, ts) + a.pair_cost;
     const int k0 = ChunkOf(a, A_, first), k1 = ChunkOf(a, A_, first + ts - 1);
     p0 = size_t(k0 + pair) * a.wpc, p1 = size_t(k1 + pair + 1) * a.wpc;
+    if (Hc == 1 && H > 1) {
+      const size_t row = size_t(h) * (a.n_chunks + a.n_seqs) + s;
+      p0 = (row + k0) * a.wpc, p1 = (row + k1 + 1) * a.wpc;
+    }
   }
   constexpr int NW = kReduceThreads / 64;
   __shared__ float wgt[kReduceThreads], wl[kReduceThreads];
@@ -756,6 +790,7 @@ int Fill(const yahkv_geometry* g, const yahkv_kv8_pools* pools, const int32_t* p
   if (MakeTuning(opt).one_launch) return YAHKV_ERR_ARG;
   if (const int rc = Prepare(MakeGeom(*g), stride, seq_len, n_seqs, max_seq_len, workspace, workspace_bytes, opt, a)) return rc;
   a->table = page_table, a->q = q, a->q_dtype = q_dtype, a->scale = softmax_scale, a->open_tile = 1;
+  if (g->n_kv_heads > 1 && kWavesPerGroup % g->n_kv_heads == 0) a->tile_mult = g->n_kv_heads;
   return YAHKV_OK;
 }
 
