@@ -146,8 +146,10 @@ void Kv8Part(const DecodeArgs a, const Kv8Pools pools) {
                                                  rr * (H * 128) + ((c ^ (rr & 7)) << 4), 0, 0, kStreamed);
       }
       const uint32_t* sp4 = pools.ks + ((row0 + n32) * H + head) * 8;
-      ksc4[0] = StreamLoad(reinterpret_cast<const uint4*>(sp4));
-      ksc4[1] = StreamLoad(reinterpret_cast<const uint4*>(sp4 + 4));
+      // (plain loads: the row's other quarters are wanted by the waves next to this one, and a streaming read leaves
+      // nothing in the L2 for them)
+      ksc4[0] = *reinterpret_cast<const uint4*>(sp4);
+      ksc4[1] = *reinterpret_cast<const uint4*>(sp4 + 4);
     } else {
       const auto rk = __builtin_amdgcn_make_buffer_rsrc(
           reinterpret_cast<uint8_t*>(pools.kq) + (row0 * H + head) * 256, 0, 0x7fffffff, 0x00020000);
@@ -159,7 +161,7 @@ void Kv8Part(const DecodeArgs a, const Kv8Pools pools) {
                                                  rr * (H * 256) + ((c ^ (rr & 15)) << 4), 0, 0, kStreamed);
       }
       const uint32_t* sp = pools.ks + ((row0 + n32) * H + head) * 2;
-      ksc = StreamLoad(reinterpret_cast<const uint2*>(sp));
+      ksc = *reinterpret_cast<const uint2*>(sp);  // (a plain load, as for the 4-bit rows)
     }
   };
   auto fetch_v = [&](int tile, int hf, int page) {
