@@ -807,7 +807,7 @@ def run_decode(a, wl, torch, yahkv):
     vnew = torch.randn((total, B, 1, NKV, HD), generator=gen, device="cuda").to(torch.bfloat16)
     out = torch.empty((B, NQ, HD), dtype=torch.float32, device="cuda")
     opt = yahkv.decode_options(one_launch=a.one_launch, deterministic=a.deterministic,
-                               min_chunk_tiles=a.min_chunk_tiles, wg_partials=a.wg_partials)
+                               min_chunk_tiles=a.min_chunk_tiles, wg_partials=a.wg_partials, cut=a.cut)
     if a.first_come:
         opt.deterministic = -1
     ws = torch.empty(yahkv.decode_workspace_bytes(g, B, max_len, opt), dtype=torch.uint8, device="cuda")
@@ -988,6 +988,9 @@ def main():
     ap.add_argument("--wg-partials", type=int, default=0, choices=[0, 1, 2],
                     help="q8_0 / q4_0 decode workloads: yahkv_decode_options::wg_partials (1: one partial per workgroup for a "
                          "chunk's last pair, 2: one per wave, 0: chosen from the batch's size)")
+    ap.add_argument("--cut", type=int, default=0, choices=[0, 1, 2],
+                    help="q8_0 / q4_0 decode workloads: yahkv_decode_options::cut (1: by (sequence, kv head), 2: by "
+                         "(sequence, tile) with the kv heads of a tile on neighbouring waves, 0: the library's choice)")
     ap.add_argument("--separate-append", action="store_true",
                     help="decode workloads: the step's token is appended by a dispatch of its own (three per step)")
     ap.add_argument("--clock-trace", action="store_true",

@@ -174,6 +174,13 @@ typedef struct yahkv_decode_options {
   int32_t wg_partials;      /* what a workgroup leaves of the last (sequence, kv head) pair it worked on: 1: one partial,
                                merged from its waves' in LDS; 2: one per wave; 0: chosen from the batch's size (one per
                                workgroup when the whole batch is at most four 64-key tiles per wave) */
+  int32_t cut;              /* how the work is cut among the waves: 1: by (sequence, kv head), each wave a stretch of one
+                               head's tiles; 2: by (sequence, tile), the kv heads of a tile dealt to neighbouring waves
+                               (kv head counts that divide 8; not with one_launch or one partial per workgroup: those
+                               cut by head), which reads a page's kv heads together: 2 - 3 % faster, and the workspace
+                               holds (chunks + n_seqs) * kv heads places for partials instead of chunks + n_seqs * kv
+                               heads; 0: by tile where that is possible. The kv8a16 / kv4a16 functions always cut by
+                               tile where the head count allows */
 } yahkv_decode_options;
 
 /* Decode attention: one query token per sequence against keys 0 .. seq_len[s] - 1.

@@ -121,3 +121,28 @@ def test_one_launch_form_gives_the_two_dispatches_results(yahkv, torch_gpu, fmt,
     runs = [gpu_attend(yahkv, torch, dev, table, lens, q, scale, opt=det) for _ in range(3)]
     assert np.array_equal(runs[0].view(np.uint32), runs[1].view(np.uint32))
     assert np.array_equal(runs[0].view(np.uint32), runs[2].view(np.uint32))
+
+
+@pytest.mark.parametrize("fmt,n_q,n_kv", [(8, 24, 4), (4, 16, 2), (8, 24, 8), (8, 18, 3)])
+def test_cut_by_tile_and_by_head_agree(yahkv, torch_gpu, fmt, n_q, n_kv):
+    """opt.cut: by (sequence, tile) with the kv heads of a tile on neighbouring waves (the default where the head count
+    divides 8) and by (sequence, kv head) give the oracle's result, each bit for bit the same on a second call; with
+    three kv heads both are the cut by head. Ragged lengths incl. empty and one-key sequences, with a gate; then the
+    step form, pools byte for byte."""
+    torch = torch_gpu
+    lens = [1, 0, 63, 64, 65, 700, 5000, 31, 12000, 129, 2500, 0, 64 * 40, 33000]
+    g, table, host, dev, rng = setup(yahkv, torch, fmt, n_q, n_kv, 256, 64, lens, seed=fmt + n_kv, fill=0x3C)
+    q = to_bf16_f32(rng.standard_normal((len(lens), n_q, 256)))
+    gate = rng.standard_normal(q.shape).astype(np.float32)
+    want = oracle.decode_attend(host, table, lens, q, 0.0625, gate)
+    outs = {}
+    for cut in (1, 2, 0):
+        opt = yahkv.decode_options(cut=cut)
+        a = gpu_attend(yahkv, torch, dev, table, lens, q, 0.0625, opt=opt, gate=gate)
+        b = gpu_attend(yahkv, torch, dev, table, lens, q, 0.0625, opt=opt, gate=gate)
+        assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), cut
+        assert rel_err(a, want) < TOL, cut
+        assert not a[1].any() and not a[11].any()
+        outs[cut] = a
+    assert np.array_equal(outs[0].view(np.uint32), outs[2 if 8 % n_kv == 0 else 1].view(np.uint32))
+    assert rel_err(outs[1], outs[2]) < 5e-4

@@ -43,7 +43,7 @@ class DecodeOptions(C.Structure):
     """yahkv_decode_options: zero fields are the defaults."""
     _fields_ = [("n_chunks", C.c_int32), ("min_chunk_tiles", C.c_int32), ("pair_cost", C.c_int32),
                 ("reduce_split", C.c_int32), ("deterministic", C.c_int32), ("xcd_weight", C.c_int32 * 8),
-                ("one_launch", C.c_int32), ("wg_partials", C.c_int32)]
+                ("one_launch", C.c_int32), ("wg_partials", C.c_int32), ("cut", C.c_int32)]
 
 
 class Rope(C.Structure):
@@ -377,11 +377,12 @@ def append_rope(pools, table, start_pos, k_src, v_src, theta, eps, rotary_dim, k
 
 
 def decode_options(n_chunks=0, min_chunk_tiles=0, pair_cost=0, reduce_split=0, deterministic=False, xcd_weight=None,
-                   one_launch=False, wg_partials=0):
+                   one_launch=False, wg_partials=0, cut=0):
     """yahkv_decode_options; zero / None fields are the defaults."""
     o = DecodeOptions(n_chunks, min_chunk_tiles, pair_cost, reduce_split, 1 if deterministic else 0)
     o.one_launch = 1 if one_launch else 0
     o.wg_partials = int(wg_partials)
+    o.cut = int(cut)
     for j, w in enumerate(xcd_weight or ()):
         o.xcd_weight[j] = int(w)
     return o

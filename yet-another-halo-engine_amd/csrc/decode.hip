@@ -201,7 +201,11 @@ void DattnPart(const DecodeArgs a) {
   if (rec.x < 0) return;
   const int chunk_n = rec.w;
   // (a chunk of at most one tile per wave needs no hand-out: wave w takes tile w, and the counter's barrier is saved)
-  const bool fixed_pattern = a.deterministic || chunk_n <= kWavesPerGroup;
+  // (cut by (sequence, tile), DecodeArgs::tile_mult: item j of a sequence is tile j / H of kv head j % H, a wave of
+  // the fixed pattern keeps its head, and neighbouring waves read the heads of the same tokens side by side)
+  const int lg_mult = MODE == 0 && a.tile_mult > 1 ? __builtin_ctz(static_cast<unsigned>(a.tile_mult)) : 0;
+  const bool fixed_pattern = a.deterministic || chunk_n <= kWavesPerGroup || lg_mult > 0;
+  int head = 0;  // the kv head of the wave's current items
   if (!fixed_pattern) {
     if (threadIdx.x == 0) next_tile = 0;
     __syncthreads();
@@ -262,7 +266,7 @@ void DattnPart(const DecodeArgs a) {
     int p = pg[0];
 #pragma unroll
     for (int j = 1; j < PPT; ++j) p = tok_in_tile / PT == j ? pg[j] : p;
-    return size_t(p) * H + cur.h;
+    return size_t(p) * H + head;
   };
   // Addresses are a base per (page, kv head), which is the same for the whole wave when a tile is one page, plus a
   // 32-bit offset per lane: the form the scalar-base addressing mode of the global loads takes.
@@ -310,7 +314,7 @@ void DattnPart(const DecodeArgs a) {
 #pragma unroll
       for (int j = 0; j < NVB; ++j) vb[j] = StreamLoad(reinterpret_cast<const uint4*>(vp + (16 * (hf * NVB + j) * PT + off)));
     } else if constexpr (PPT == 1) {
-      const size_t ph = size_t(pg[0]) * H + cur.h;
+      const size_t ph = size_t(pg[0]) * H + head;
       const auto rv = __builtin_amdgcn_make_buffer_rsrc(
           const_cast<uint8_t*>(a.pools.vq) + ph * (Q8 ? D * PT : NB * 16 * PT), 0, 0x7fffffff, 0x00020000);
 #pragma unroll
@@ -404,13 +408,24 @@ void DattnPart(const DecodeArgs a) {
     }
   };
   // l = 0 for a pair this wave got no tile of (the reduce then skips it)
+  // partial of (this chunk, this wave, the current sequence, kv head h); cut by tile, every head has a row of places
+  auto part_of = [&](int h) -> size_t {
+    if (lg_mult > 0) return ((size_t(h) * (a.n_chunks + a.n_seqs) + blockIdx.x + cur.s) * a.wpc + wave) * G;
+    return PartialIndex(a, blockIdx.x, wave, cur) * G;
+  };
+  auto empty_at = [&](int h) {
+    if (lane < G) StoreDevice2(DeviceBuffer(a.ml + part_of(h) * 2), lane * 8, kNegMax, 0.0f);
+  };
   auto leave_empty = [&]() {
-    const size_t part = PartialIndex(a, blockIdx.x, wave, cur) * G;
-    if (lane < G) StoreDevice2(DeviceBuffer(a.ml + part * 2), lane * 8, kNegMax, 0.0f);
+    if (lg_mult == 0) return empty_at(cur.h);
+    for (int h = 0; h < H; ++h) empty_at(h);
   };
   // the pair's partial, straight from registers (natural-log units, as the reduce expects)
   auto leave_partial = [&]() {
-    const size_t part = PartialIndex(a, blockIdx.x, wave, cur) * G;
+    if (lg_mult > 0)
+      for (int h = 0; h < H; ++h)
+        if (h != head) empty_at(h);
+    const size_t part = part_of(lg_mult > 0 ? head : cur.h);
     const auto rml = DeviceBuffer(a.ml + part * 2), racc = DeviceBuffer(a.acc + part * D);
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
@@ -445,16 +460,18 @@ void DattnPart(const DecodeArgs a) {
     // ---- first tile of this wave in the pair: query rows, empty state, first loads
     constexpr int QE = NB * 32 / 64;  // lq entries per lane
     h8v qreg[QE];
+    const int item = cur.first + (idx - cur.base);
+    head = lg_mult > 0 ? item & (a.tile_mult - 1) : cur.h;
 #pragma unroll
     for (int e = 0; e < QE; ++e) {
       const int i = lane + 64 * e, b = i / 32, sub = (i / 16) % 2, hf = (i / 8) % 2, rw = i % 8;
       qreg[e] = h8v{0, 0, 0, 0, 0, 0, 0, 0};
       if (rw < G)
-        qreg[e] = LoadQ8(a.q, (size_t(cur.s) * g.n_q + size_t(cur.h) * G + rw) * D + b * 32 +
+        qreg[e] = LoadQ8(a.q, (size_t(cur.s) * g.n_q + size_t(head) * G + rw) * D + b * 32 +
                                    (Q8 ? 16 * hf + 8 * sub : 16 * sub + 8 * hf), a.q_dtype);
     }
     row = a.table + int64_t(cur.s) * a.stride;
-    int tile = cur.first + (idx - cur.base);
+    int tile = item >> lg_mult;
     int pgc[PPT], pgn[PPT];
     load_pages(tile, pgc);
     load_k(0, pgc);
@@ -487,7 +504,7 @@ void DattnPart(const DecodeArgs a) {
     while (true) {
       const int nidx = take();
       const bool has_next = nidx < cur.base + cur.n;  // the wave's next tile is in the same pair
-      const int ntile = cur.first + (nidx - cur.base);
+      const int ntile = (cur.first + (nidx - cur.base)) >> lg_mult;
       // Every pass issues the same loads whether or not the wave has a next tile in this pair (without one it
       // reads the first half of this tile's K again and drops it): the compiler counts outstanding loads along
       // every path into a wait and takes the smallest, so a load issued on one path only turns the waits after the
@@ -872,12 +889,18 @@ __global__ __launch_bounds__(kReduceThreads) void DattnReduce(const DecodeArgs a
   // line units of the sequences before this one and of the whole line; the pair's tiles follow its first units
   size_t p0 = 0, p1 = 0;  // (a sequence that has nothing but its new token has no partials)
   if (ts > 0) {
-    const long long A_ = ChunkUnits(a, static_cast<long long>(a.tprefix[a.n_seqs]) * H);
+    // (cut by tile, the sequence is one pair on the line and every head has a row of places of its own)
+    const int Hc = CutHeads(a);
+    const long long A_ = ChunkUnits(a, static_cast<long long>(a.tprefix[a.n_seqs]) * Hc);
     const int pair = s * H + h;
-    const long long first =
-        static_cast<long long>(a.tprefix[s]) * H + static_cast<long long>(h) * UnitsOf(a, ts) + a.pair_cost;
+    const long long first = static_cast<long long>(a.tprefix[s]) * Hc +
+                            static_cast<long long>(Hc == 1 ? 0 : h) * UnitsOf(a, ts) + a.pair_cost;
     const int k0 = ChunkOf(a, A_, first), k1 = ChunkOf(a, A_, first + ts - 1);
     p0 = size_t(k0 + pair) * a.wpc, p1 = size_t(k1 + pair + 1) * a.wpc;
+    if (Hc == 1 && H > 1) {
+      const size_t row = size_t(h) * (a.n_chunks + a.n_seqs) + s;
+      p0 = (row + k0) * a.wpc, p1 = (row + k1 + 1) * a.wpc;
+    }
   }
   constexpr int NW = kReduceThreads / 64;
   __shared__ float wgt[kReduceThreads], wl[kReduceThreads];
@@ -1254,10 +1277,12 @@ extern "C" int yahkv_decode_attend_static(const yahkv_geometry* g, const yahkv_p
   if (const int st = CheckPools(g, pools)) return st;
   if (n_seqs <= 0 || max_seq_len <= 0) return YAHKV_ERR_ARG;
   // the partials of this batch must fit the array: nothing is launched otherwise
-  if (MakePlan(MakeGeom(*g), n_seqs, max_seq_len, MakeTuning(nullptr)).bytes > kStaticScratchBytes)
+  yahkv_decode_options o{};
+  o.cut = 1;  // by (sequence, kv head): the cut with the fewest places for partials, so the array holds larger batches
+  if (MakePlan(MakeGeom(*g), n_seqs, max_seq_len, MakeTuning(&o)).bytes > kStaticScratchBytes)
     return YAHKV_ERR_WORKSPACE;
   void* ws = nullptr;
   if (const int st = StaticScratch(&ws)) return st;
   return yahkv_decode_attend(g, pools, page_table, page_table_stride, seq_len, n_seqs, max_seq_len, q, q_dtype,
-                             softmax_scale, gate, out, ws, kStaticScratchBytes, nullptr, stream);
+                             softmax_scale, gate, out, ws, kStaticScratchBytes, &o, stream);
 }

@@ -397,7 +397,7 @@ inline int ComputeUnits() {
 }
 // Tuning values of a call: the caller's options where given, else the defaults.
 struct Tuning {
-  int32_t n_chunks, min_chunk_tiles, pair_cost, reduce_split, deterministic, one_launch, wg_partials;
+  int32_t n_chunks, min_chunk_tiles, pair_cost, reduce_split, deterministic, one_launch, wg_partials, cut;
   int32_t xcd_weight[8];
 };
 inline Tuning MakeTuning(const yahkv_decode_options* o) {
@@ -413,8 +413,15 @@ inline Tuning MakeTuning(const yahkv_decode_options* o) {
   t.deterministic = o == nullptr || o->deterministic >= 0;  // (negative: tiles first come, first served)
   t.one_launch = o != nullptr && o->one_launch != 0;
   t.wg_partials = o != nullptr ? o->wg_partials : 0;
+  t.cut = o != nullptr ? o->cut : 0;
   for (int j = 0; j < 8; ++j) t.xcd_weight[j] = o != nullptr ? std::max(o->xcd_weight[j], 0) : 0;
   return t;
+}
+// Whether the line is cut by (sequence, tile), DecodeArgs::tile_mult: the reference's own formats wherever the kv head
+// count allows it, the block formats when the options ask for it.
+inline bool CutByTile(const Geom& g, const Tuning& t) {
+  if (g.n_kv <= 1 || kWavesPerGroup % g.n_kv != 0) return false;
+  return g.format > 16 || (t.cut != 1 && !t.one_launch && t.wg_partials != 1);
 }
 inline Plan MakePlan(const Geom& g, int32_t n_seqs, int32_t max_seq_len, const Tuning& t) {
   Plan p;
@@ -451,7 +458,7 @@ inline Plan MakePlan(const Geom& g, int32_t n_seqs, int32_t max_seq_len, const T
   for (int j = 8, over = p.share[8] - 8192; j >= 1; --j) p.share[j] = std::min(p.share[j] - over, 8192 - 512 * (8 - j));
   p.share[8] = 8192;
   // (the formats whose line is cut by (sequence, tile), DecodeArgs::tile_mult, keep a row of places per kv head)
-  const bool by_tile = g.format > 16 && g.n_kv > 1 && kWavesPerGroup % g.n_kv == 0;
+  const bool by_tile = CutByTile(g, t);
   const size_t parts = (by_tile ? (size_t(p.n_chunks) + size_t(n_seqs)) * g.n_kv : size_t(p.n_chunks) + size_t(n_seqs) * g.n_kv) * p.wpc;
   p.off_tprefix = 0;
   p.off_tickets = Align(sizeof(int32_t) * (size_t(n_seqs) + 1));
@@ -487,6 +494,7 @@ inline int Prepare(const Geom& m, int32_t page_table_stride, const int32_t* seq_
   // One partial per workgroup for a chunk's last pair pays where chunks are short (a small batch: few tiles per wave, so
   // a wave's partial is a large part of what it moves) and costs two barriers at the kernel's end where they are long.
   a->wg_partials = t.wg_partials == 1 ? 1 : t.wg_partials == 2 ? 0 : (int64_t(p.max_len) + kTile - 1) / kTile * n_seqs * m.n_kv <= int64_t(p.n_chunks) * kWavesPerGroup * 4;
+  if (m.format <= 16 && CutByTile(m, t) && !a->wg_partials) a->tile_mult = m.n_kv;
   std::copy(p.share, p.share + 9, a->share);
   return YAHKV_OK;
 }
