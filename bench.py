@@ -434,6 +434,8 @@ def run_kv8(a, wl, torch, yahkv):
     if a.first_come:
         opt.deterministic = -1
     ws = torch.empty(yahkv.lib.yahkv_kv8_decode_workspace_bytes(g, B, max_len, opt), dtype=torch.uint8, device="cuda")
+    xcd = (yahkv.kv8_decode_calibrate(layers[0], t_table, len_rows[0], max_len, q, ws, opt, rounds=3)
+           if not a.no_calibrate else None)            # set-up, as a server does once (equal shares without it)
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(a.steps)]
 
     def step(i, pair=None):
@@ -484,7 +486,7 @@ def run_kv8(a, wl, torch, yahkv):
         "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
         "config": {"workload": a.workload, "batch": B, "ctx_min": int(lens.min()), "ctx_max": int(lens.max()),
                    "ctx_sum": int(lens.sum()), "n_q_heads": NQ, "n_kv_heads": NKV, "head_dim": HD, "page_tokens": PG,
-                   "n_pages": n_pages, "layers_rotated": n_layers, "kv_format": "kv%da16" % bits,
+                   "n_pages": n_pages, "layers_rotated": n_layers, "kv_format": "kv%da16" % bits, "xcd_weight": xcd,
                    "step": "append 1 token/seq + paged decode attention (part, reduce with the open tile and the append in it)"},
         "pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2), "tok_per_s": round(B / (ms * 1e-3), 1),
         "kv_bytes_per_step": int(kv_bytes), "parity_max_rel_err": float(f"{err:.3e}"), "parity_rows": rows,

@@ -486,6 +486,12 @@ int yahkv_kv8_decode_attend(const yahkv_geometry* g, const yahkv_kv8_pools* pool
                             int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs, int32_t max_seq_len,
                             const void* q, int32_t q_dtype, float softmax_scale, const float* gate, float* out,
                             void* workspace, size_t workspace_bytes, const yahkv_decode_options* opt, void* stream);
+/* yahkv_decode_calibrate for these formats: the XCDs' relative read speeds on the caller's own batch into
+ * opt->xcd_weight (a set-up call: synchronizes the stream, overwrites the workspace). No counterpart in the reference. */
+int yahkv_kv8_decode_calibrate(const yahkv_geometry* g, const yahkv_kv8_pools* pools, const int32_t* page_table,
+                               int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs, int32_t max_seq_len,
+                               const void* q, int32_t q_dtype, void* workspace, size_t workspace_bytes,
+                               yahkv_decode_options* opt, int32_t rounds, void* stream);
 /* The two dispatches of yahkv_kv8_decode_attend and yahkv_kv8_decode_step on their own, as LoomDecoder::Step issues
  * its own (loom_decoder.hpp:259-268); both take the same lengths (whether or not they count a token still to be
  * appended, the split-K dispatch covers the 16-key tiles that are closed once it is). With k_new / v_new the merge is

@@ -376,3 +376,36 @@ def test_refusals(yahkv, torch_gpu):
     with pytest.raises(yahkv.YahkvError):
         yahkv.kv8_decode_attend(dp, table, torch.ones(1, dtype=torch.int32, device="cuda"), 1,
                                 torch.zeros((1, 24, 256), device="cuda"), 0.0625, opt=yahkv.DecodeOptions(one_launch=1))
+
+
+def test_xcd_calibration_for_these_formats(yahkv, torch_gpu):
+    """yahkv_kv8_decode_calibrate returns shares of the XCDs' speeds that leave the results where they were."""
+    torch = torch_gpu
+    rng = np.random.default_rng(41)
+    lens = [int(x) for x in rng.integers(3000, 20000, 24)]
+    n_q, H = 24, 4
+    pages = [(n + 255) // 256 for n in lens]
+    P = sum(pages)
+    table = np.zeros((len(lens), max(pages)), np.int32)
+    perm, o = rng.permutation(P).astype(np.int32), 0
+    for s, np_ in enumerate(pages):
+        table[s, :np_] = perm[o:o + np_]
+        o += np_
+    g = yahkv.kv8_geometry(n_q, H, P)
+    dp = yahkv.Kv8Pools(g)
+    t_table = torch.from_numpy(table).cuda()
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    for s, n in enumerate(lens):
+        k = torch.randn((1, n, H, 256), generator=gen, device="cuda").to(torch.bfloat16)
+        v = torch.randn((1, n, H, 256), generator=gen, device="cuda").to(torch.bfloat16)
+        yahkv.kv8_kmean(dp, t_table[s:s + 1], k)
+        yahkv.kv8_append(dp, t_table[s:s + 1], torch.zeros(1, dtype=torch.int32, device="cuda"), k, v)
+    q = torch.randn((len(lens), n_q, 256), generator=gen, device="cuda")
+    sl = torch.tensor(lens, dtype=torch.int32, device="cuda")
+    before = yahkv.kv8_decode_attend(dp, t_table, sl, max(lens), q, 0.0625).cpu().numpy()
+    opt = yahkv.decode_options()
+    ws = torch.empty(yahkv.lib.yahkv_kv8_decode_workspace_bytes(g, len(lens), max(lens), opt), dtype=torch.uint8, device="cuda")
+    w = yahkv.kv8_decode_calibrate(dp, t_table, sl, max(lens), q, ws, opt, rounds=2)
+    assert len(w) == 8 and max(w) == 10000 and min(w) >= 5000, w
+    after = yahkv.kv8_decode_attend(dp, t_table, sl, max(lens), q, 0.0625, workspace=ws, opt=opt).cpu().numpy()
+    assert rel_err(after, before) < 5e-4

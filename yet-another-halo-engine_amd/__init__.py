@@ -732,6 +732,15 @@ def kv8_prefill_attend(pools, table, prefix_len, max_prefix_len, q, scale, gate=
     return out
 
 
+def kv8_decode_calibrate(pools, table, seq_len, max_seq_len, q, workspace, opt, rounds=2):
+    """Measures the XCDs' relative read speeds on this batch into opt.xcd_weight; returns them as a list."""
+    g, st = pools.geom, pools.struct()
+    _check(lib.yahkv_kv8_decode_calibrate(C.byref(g), C.byref(st), _dp(table), table.shape[1], _dp(seq_len), q.shape[0],
+                                          max_seq_len, _dp(q), _dtype_code(q), _dp(workspace), C.c_size_t(workspace.numel()),
+                                          C.byref(opt), int(rounds), _stream()), "kv8_decode_calibrate")
+    return list(opt.xcd_weight)
+
+
 def kv8_decode_part(pools, table, seq_len, max_seq_len, q, scale, workspace, opt=None):
     g = pools.geom
     st = pools.struct()

@@ -1160,58 +1160,22 @@ extern "C" int yahkv_decode_attend(const yahkv_geometry* g, const yahkv_pools* p
   return LaunchPart(a, static_cast<hipStream_t>(stream));
 }
 
-constexpr int kCalibrationLaunches = 8;  // measured launches per round of yahkv_decode_calibrate
-
-// Relative read speeds of the eight XCDs on the caller's own batch. Workgroup k of a dispatch runs on XCD k % 8, and the
-// XCDs of one GPU do not read memory equally fast (up to 10 % apart, measured); chunk shares that follow their speeds
-// let all workgroups finish together. Each round runs the part kernel nine times with the current shares (the first
-// launch warms caches and clocks), reads when each workgroup's last wave finished, and sets every XCD's weight to its
-// share divided by its mean time over the eight measured launches. Synchronizes the stream: a set-up call, not part of a step.
 extern "C" int yahkv_decode_calibrate(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
                                       int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs,
                                       int32_t max_seq_len, const void* q, int32_t q_dtype, void* workspace,
                                       size_t workspace_bytes, yahkv_decode_options* opt, int32_t rounds,
                                       void* stream) {
-  if (opt == nullptr || rounds <= 0) return YAHKV_ERR_ARG;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  for (int32_t r = 0; r < rounds; ++r) {
-    DecodeArgs a;
+  auto prepare = [&](DecodeArgs* a) -> int {
     if (const int rc = CheckGeometry(g)) return rc;
-    if (const int rc = Prepare(MakeGeom(*g), page_table_stride, seq_len, n_seqs, max_seq_len, workspace, workspace_bytes, opt, &a))
+    if (const int rc = Prepare(MakeGeom(*g), page_table_stride, seq_len, n_seqs, max_seq_len, workspace, workspace_bytes, opt, a))
       return rc;
     if (const int rc = CheckPartArgs(g, pools, page_table, q, q_dtype)) return rc;
-    if (a.n_chunks % 8 != 0) return YAHKV_OK;  // a batch too small for whole groups is cut into equal shares anyway
-    a.pools = MakePools(*pools), a.table = page_table, a.q = q, a.q_dtype = q_dtype, a.scale = 1.0f;
-    const Plan p = MakePlan(a.g, n_seqs, max_seq_len, MakeTuning(opt));
-    a.stamps = reinterpret_cast<unsigned long long*>(static_cast<char*>(workspace) + p.off_stamps);
-    const size_t n = 2 * size_t(a.n_chunks);  // [0, n_chunks): start of each workgroup, [n_chunks, ..): its end
-    std::vector<unsigned long long> stamps(n);
-    double t[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    int cnt[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    for (int pass = 0; pass < 1 + kCalibrationLaunches; ++pass) {  // the first launch warms caches and clocks
-      if (hipMemsetAsync(a.stamps, 0, n * sizeof(unsigned long long), st) != hipSuccess) return YAHKV_ERR_LAUNCH;
-      if (const int rc = LaunchPart(a, st)) return rc;
-      if (pass == 0) continue;
-      if (hipMemcpyAsync(stamps.data(), a.stamps, n * sizeof(unsigned long long), hipMemcpyDeviceToHost, st) != hipSuccess ||
-          hipStreamSynchronize(st) != hipSuccess)
-        return YAHKV_ERR_LAUNCH;
-      unsigned long long start = ~0ull;
-      for (int k = 0; k < a.n_chunks; ++k)
-        if (stamps[size_t(k)] != 0) start = std::min(start, stamps[size_t(k)]);
-      for (int k = 0; k < a.n_chunks; ++k) {
-        const unsigned long long end = stamps[size_t(a.n_chunks) + size_t(k)];
-        if (end > start) t[k % 8] += double(end - start), ++cnt[k % 8];
-      }
-    }
-    double speed[8], top = 0;
-    for (int j = 0; j < 8; ++j) {
-      if (cnt[j] == 0 || t[j] <= 0) return YAHKV_OK;  // an XCD without work: nothing to learn from this batch
-      speed[j] = double(a.share[j + 1] - a.share[j]) / (t[j] / cnt[j]);
-      top = std::max(top, speed[j]);
-    }
-    for (int j = 0; j < 8; ++j) opt->xcd_weight[j] = std::max(1, static_cast<int32_t>(speed[j] / top * 10000.0 + 0.5));
-  }
-  return YAHKV_OK;
+    a->pools = MakePools(*pools), a->table = page_table, a->q = q, a->q_dtype = q_dtype, a->scale = 1.0f;
+    return YAHKV_OK;
+  };
+  return CalibrateXcds(prepare, [&](const DecodeArgs& a) { return LaunchPart(a, st); }, workspace, n_seqs, max_seq_len, opt,
+                       rounds, st);
 }
 
 // ---- the shader clock, as a kernel sees it -----------------------------------------------------------------------------------

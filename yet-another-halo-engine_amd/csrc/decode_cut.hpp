@@ -6,6 +6,7 @@
 
 #include <algorithm>
 #include <cstdint>
+#include <vector>
 
 #include "common.hpp"
 
@@ -496,6 +497,56 @@ inline int Prepare(const Geom& m, int32_t page_table_stride, const int32_t* seq_
   a->wg_partials = t.wg_partials == 1 ? 1 : t.wg_partials == 2 ? 0 : (int64_t(p.max_len) + kTile - 1) / kTile * n_seqs * m.n_kv <= int64_t(p.n_chunks) * kWavesPerGroup * 4;
   if (m.format <= 16 && CutByTile(m, t) && !a->wg_partials) a->tile_mult = m.n_kv;
   std::copy(p.share, p.share + 9, a->share);
+  return YAHKV_OK;
+}
+
+// ---- XCD calibration -----------------------------------------------------------------------------------------------------
+
+constexpr int kCalibrationLaunches = 8;  // measured launches per round
+
+// Relative read speeds of the eight XCDs on the caller's own batch. Workgroup k of a dispatch runs on XCD k % 8, and the
+// XCDs of one GPU do not read memory equally fast (up to 10 % apart, measured); chunk shares that follow their speeds
+// let all workgroups finish together. Each round runs the part kernel nine times with the current shares (the first
+// launch warms caches and clocks), reads when each workgroup's last wave finished, and sets every XCD's weight to its
+// share divided by its mean time over the eight measured launches. Synchronizes the stream: a set-up call, not part of
+// a step. `prepare` fills the launch arguments from the caller's (and validates them), `launch` runs the part kernel.
+template <typename PrepareFn, typename LaunchFn>
+inline int CalibrateXcds(PrepareFn prepare, LaunchFn launch, void* workspace, int32_t n_seqs, int32_t max_seq_len,
+                         yahkv_decode_options* opt, int32_t rounds, hipStream_t st) {
+  if (opt == nullptr || rounds <= 0) return YAHKV_ERR_ARG;
+  for (int32_t r = 0; r < rounds; ++r) {
+    DecodeArgs a;
+    if (const int rc = prepare(&a)) return rc;
+    if (a.n_chunks % 8 != 0) return YAHKV_OK;  // a batch too small for whole groups is cut into equal shares anyway
+    const Plan p = MakePlan(a.g, n_seqs, max_seq_len, MakeTuning(opt));
+    a.stamps = reinterpret_cast<unsigned long long*>(static_cast<char*>(workspace) + p.off_stamps);
+    const size_t n = 2 * size_t(a.n_chunks);  // [0, n_chunks): start of each workgroup, [n_chunks, ..): its end
+    std::vector<unsigned long long> stamps(n);
+    double t[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    int cnt[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int pass = 0; pass < 1 + kCalibrationLaunches; ++pass) {  // the first launch warms caches and clocks
+      if (hipMemsetAsync(a.stamps, 0, n * sizeof(unsigned long long), st) != hipSuccess) return YAHKV_ERR_LAUNCH;
+      if (const int rc = launch(a)) return rc;
+      if (pass == 0) continue;
+      if (hipMemcpyAsync(stamps.data(), a.stamps, n * sizeof(unsigned long long), hipMemcpyDeviceToHost, st) != hipSuccess ||
+          hipStreamSynchronize(st) != hipSuccess)
+        return YAHKV_ERR_LAUNCH;
+      unsigned long long start = ~0ull;
+      for (int k = 0; k < a.n_chunks; ++k)
+        if (stamps[size_t(k)] != 0) start = std::min(start, stamps[size_t(k)]);
+      for (int k = 0; k < a.n_chunks; ++k) {
+        const unsigned long long end = stamps[size_t(a.n_chunks) + size_t(k)];
+        if (end > start) t[k % 8] += double(end - start), ++cnt[k % 8];
+      }
+    }
+    double speed[8], top = 0;
+    for (int j = 0; j < 8; ++j) {
+      if (cnt[j] == 0 || t[j] <= 0) return YAHKV_OK;  // an XCD without work: nothing to learn from this batch
+      speed[j] = double(a.share[j + 1] - a.share[j]) / (t[j] / cnt[j]);
+      top = std::max(top, speed[j]);
+    }
+    for (int j = 0; j < 8; ++j) opt->xcd_weight[j] = std::max(1, static_cast<int32_t>(speed[j] / top * 10000.0 + 0.5));
+  }
   return YAHKV_OK;
 }
 

@@ -801,6 +801,18 @@ int Fill(const yahkv_geometry* g, const yahkv_kv8_pools* pools, const int32_t* p
 
 using namespace yahkv;
 
+static int LaunchKv8Part(const yahkv_geometry* g, const yahkv_kv8_pools* pools, const DecodeArgs& a, hipStream_t st) {
+  const dim3 grid(static_cast<unsigned>(a.n_chunks)), block(64 * kWavesPerGroup);
+  const Kv8Pools p = MakeKv8Pools(*pools);
+  switch (g->format) {
+    case YAHKV_KV8A16: hipLaunchKernelGGL((Kv8Part<8, 8>), grid, block, 0, st, a, p); break;
+    case YAHKV_KV4A16: hipLaunchKernelGGL((Kv8Part<4, 4>), grid, block, 0, st, a, p); break;
+    case YAHKV_K8V4A16: hipLaunchKernelGGL((Kv8Part<8, 4>), grid, block, 0, st, a, p); break;
+    default: hipLaunchKernelGGL((Kv8Part<4, 8>), grid, block, 0, st, a, p); break;
+  }
+  return LaunchStatus();
+}
+
 extern "C" size_t yahkv_kv8_decode_workspace_bytes(const yahkv_geometry* g, int32_t n_seqs, int32_t max_seq_len,
                                                    const yahkv_decode_options* opt) {
   if (CheckKv8Geometry(g) || n_seqs <= 0 || max_seq_len <= 0) return 0;
@@ -816,16 +828,21 @@ extern "C" int yahkv_kv8_decode_part(const yahkv_geometry* g, const yahkv_kv8_po
   if (const int rc = Fill(g, pools, page_table, page_table_stride, seq_len, n_seqs, max_seq_len, q, q_dtype, softmax_scale,
                           workspace, workspace_bytes, opt, &a))
     return rc;
-  const dim3 grid(static_cast<unsigned>(a.n_chunks)), block(64 * kWavesPerGroup);
+  return LaunchKv8Part(g, pools, a, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int yahkv_kv8_decode_calibrate(const yahkv_geometry* g, const yahkv_kv8_pools* pools, const int32_t* page_table,
+                                          int32_t page_table_stride, const int32_t* seq_len, int32_t n_seqs,
+                                          int32_t max_seq_len, const void* q, int32_t q_dtype, void* workspace,
+                                          size_t workspace_bytes, yahkv_decode_options* opt, int32_t rounds,
+                                          void* stream) {
   hipStream_t st = static_cast<hipStream_t>(stream);
-  const Kv8Pools p = MakeKv8Pools(*pools);
-  switch (g->format) {
-    case YAHKV_KV8A16: hipLaunchKernelGGL((Kv8Part<8, 8>), grid, block, 0, st, a, p); break;
-    case YAHKV_KV4A16: hipLaunchKernelGGL((Kv8Part<4, 4>), grid, block, 0, st, a, p); break;
-    case YAHKV_K8V4A16: hipLaunchKernelGGL((Kv8Part<8, 4>), grid, block, 0, st, a, p); break;
-    default: hipLaunchKernelGGL((Kv8Part<4, 8>), grid, block, 0, st, a, p); break;
-  }
-  return LaunchStatus();
+  auto prepare = [&](DecodeArgs* a) -> int {
+    return Fill(g, pools, page_table, page_table_stride, seq_len, n_seqs, max_seq_len, q, q_dtype, 1.0f, workspace,
+                workspace_bytes, opt, a);
+  };
+  auto launch = [&](const DecodeArgs& a) -> int { return LaunchKv8Part(g, pools, a, st); };
+  return CalibrateXcds(prepare, launch, workspace, n_seqs, max_seq_len, opt, rounds, st);
 }
 
 extern "C" int yahkv_kv8_decode_reduce(const yahkv_geometry* g, const yahkv_kv8_pools* pools, const int32_t* page_table,
