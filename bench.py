@@ -44,8 +44,8 @@ WORKLOADS = {
     "b1_ctx32k_kv8a16": dict(fmt=816, batch=1, lo=32768, hi=32768, seed=4, layers=8),
     "prefill_b8_ctx16k_chunk2k_kv8a16": dict(fmt=816, batch=8, lo=16384, hi=16384, seed=4, chunk=2048, warmup=10),
     # ... and in its 4-bit sibling, kv4a16 (H256-rotated K in 16 levels per 32-dim group, V in 15 levels per tile)
-    "ragged_b64_kv4a16": dict(fmt=416, batch=64, lo=1024, hi=65536, seed=4),
-    "b16_ctx128k_kv4a16": dict(fmt=416, batch=16, lo=131072, hi=131072, seed=4, warmup=40),
+    "ragged_b64_kv4a16": dict(fmt=416, batch=64, lo=1024, hi=65536, seed=4, warmup=80),
+    "b16_ctx128k_kv4a16": dict(fmt=416, batch=16, lo=131072, hi=131072, seed=4, warmup=80),
     "prefill_b8_ctx16k_chunk2k_kv4a16": dict(fmt=416, batch=8, lo=16384, hi=16384, seed=4, chunk=2048, warmup=10),
 }
 MFMA_F16_PEAK_TFLOPS = 2500.0
@@ -480,7 +480,7 @@ def run_kv8(a, wl, torch, yahkv):
     tokens = [int(lens.sum()) + B * (2 + a.warmup + i) for i in range(a.steps)]
     kv_bytes = float(np.mean(tokens)) * bpt
     gbs, kgbs = kv_bytes / (ms * 1e-3) / 1e9, kv_bytes / (kern_ms * 1e-3) / 1e9
-    return {
+    res = {
         "metric": "paged kv%da16 KV decode-attn HBM GB/s (%% of peak) + tok/s" % bits, "value": round(gbs, 1), "unit": "GB/s",
         "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
@@ -496,6 +496,16 @@ def run_kv8(a, wl, torch, yahkv):
                      "traffic_source": TRAFFIC.get(a.workload, (None, None))[1],
                      "kernel": "Kv8Part<%d, %d>" % (bits, bits), "kernel_ms": round(kern_ms, 4)},
         "cpu_baseline": None}
+    # the same number of steps again right after three idle seconds, without warm-up (see run_decode): an extra figure
+    time.sleep(3.0)
+    t0 = time.perf_counter()
+    for i in range(a.steps):
+        step(1 + i)
+    torch.cuda.synchronize()
+    cold_ms = (time.perf_counter() - t0) / a.steps * 1e3
+    res["after_idle"] = {"ms_per_step": round(cold_ms, 4), "GB/s": round(kv_bytes / (cold_ms * 1e-3) / 1e9, 1),
+                         "note": "%d steps right after 3 idle seconds, no warm-up" % a.steps}
+    return res
 
 
 def run_prefill_kv8(a, wl, torch, yahkv):
