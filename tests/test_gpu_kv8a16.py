@@ -409,3 +409,50 @@ def test_xcd_calibration_for_these_formats(yahkv, torch_gpu):
     assert len(w) == 8 and max(w) == 10000 and min(w) >= 5000, w
     after = yahkv.kv8_decode_attend(dp, t_table, sl, max(lens), q, 0.0625, workspace=ws, opt=opt).cpu().numpy()
     assert rel_err(after, before) < 5e-4
+
+
+@pytest.mark.parametrize("n_q,H,kb", [(4, 1, 8), (6, 3, 8), (16, 8, 8), (16, 8, 4), (6, 3, 4)])
+def test_other_kv_head_counts(yahkv, torch_gpu, n_q, H, kb):
+    """The split-K kernel deals the kv heads of a tile to a workgroup's eight waves where the head count divides 8 (one,
+    two, four, eight heads) and cuts the work by (sequence, kv head) otherwise (three): both against the oracle, on ragged
+    lengths with a step."""
+    torch = torch_gpu
+    rng = np.random.default_rng(50 + H + kb)
+    lens = [300, 1, 2100, 17, 700]
+    pages = [(n + 1 + 255) // 256 for n in lens]
+    P = sum(pages) + 1
+    perm, o = rng.permutation(P).astype(np.int32), 0
+    table = np.zeros((len(lens), max(pages)), np.int32)
+    for s, np_ in enumerate(pages):
+        table[s, :np_] = perm[o:o + np_]
+        o += np_
+    g = yahkv.kv8_geometry(n_q, H, P, kb, kb)
+    dp, hp = yahkv.Kv8Pools(g, 0x42), kv8.HostPools(kv8.geometry(n_q, H, P, kb, kb), 0x42)
+    cap = max(lens)
+    K = (rng.standard_normal((len(lens), cap, H, 256)) + 0.4).astype(np.float16)
+    V = rng.standard_normal((len(lens), cap, H, 256)).astype(np.float16)
+    t_table = torch.from_numpy(table).cuda()
+    nv = np.array(lens, np.int32)
+    yahkv.kv8_kmean(dp, t_table, torch.from_numpy(K).cuda(), torch.from_numpy(nv).cuda())
+    for s in range(len(lens)):
+        hp.km[table[s, 0]] = kv8.kmean(K[s, :lens[s]].astype(np.float32).reshape(lens[s], H * 256))
+    yahkv.kv8_append(dp, t_table, torch.zeros(len(lens), dtype=torch.int32, device="cuda"), torch.from_numpy(K).cuda(),
+                     torch.from_numpy(V).cuda(), torch.from_numpy(nv).cuda())
+    kv8.append(hp, table, np.zeros(len(lens), np.int32), nv, K.astype(np.float32).reshape(len(lens), cap, -1),
+               V.astype(np.float32).reshape(len(lens), cap, -1))
+    assert_pools_equal(dp, hp, f"{H} kv heads")
+    q = rng.standard_normal((len(lens), n_q, 256)).astype(np.float32)
+    out = attend(yahkv, torch, dp, t_table, lens, q)
+    rot = (lambda x: kv8.rotate_q(x)) if kb == 4 else (lambda x: x)
+    for s, n in enumerate(lens):
+        Kd, Vd = kv8.dense(hp, table[s], n)
+        assert rel_err(out[s], closed_form(Kd, Vd, rot(q[s]), 1.0 / 16.0)) < TOL, (s, n)
+    kn = rng.standard_normal((len(lens), H, 256)).astype(np.float32)
+    vn = rng.standard_normal((len(lens), H, 256)).astype(np.float32)
+    out = yahkv.kv8_decode_step(dp, t_table, torch.from_numpy(nv + 1).cuda(), cap + 1, torch.from_numpy(kn).cuda(),
+                                torch.from_numpy(vn).cuda(), torch.from_numpy(q).cuda(), 1.0 / 16.0).cpu().numpy()
+    kv8.append(hp, table, nv, None, kn.reshape(len(lens), 1, -1), vn.reshape(len(lens), 1, -1))
+    assert_pools_equal(dp, hp, "step")
+    for s, n in enumerate(lens):
+        Kd, Vd = kv8.dense(hp, table[s], n + 1)
+        assert rel_err(out[s], closed_form(Kd, Vd, rot(q[s]), 1.0 / 16.0)) < TOL, (s, n)
