@@ -271,12 +271,14 @@ void DattnPart(const DecodeArgs a) {
   // Addresses are a base per (page, kv head), which is the same for the whole wave when a tile is one page, plus a
   // 32-bit offset per lane: the form the scalar-base addressing mode of the global loads takes.
   constexpr uint32_t KB = Q8 ? 32 : 16;  // bytes of K codes per key and block
-  auto load_k = [&](int tt, const int (&pg)[PPT]) {
+  // `live` false: a load whose result nobody uses (it keeps the count of loads in flight the same on every path, see the
+  // loop): every lane then reads the start of its piece, a few lines for the whole wave instead of the piece itself.
+  auto load_k = [&](int tt, const int (&pg)[PPT], bool live = true) {
     const int tk = 32 * tt + n32;
     const size_t ph = page_head(pg, tk);
-    const uint32_t t = tk % PT;
+    const uint32_t t = live ? tk % PT : 0u;
     const uint8_t* kp = a.pools.kq + ph * (NB * PT * KB);
-    const uint32_t off = t * KB + (KB / 2) * half;
+    const uint32_t off = live ? t * KB + (KB / 2) * half : 0u;
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
       if constexpr (Q8) {
@@ -306,8 +308,8 @@ void DattnPart(const DecodeArgs a) {
   // q4_0 keeps the plain register loads: that kernel is bound by instruction issue, and the detour costs it more
   // instructions than the earlier request saves.
   constexpr bool kLdsV = Q8;
-  auto fetch_v = [&](int hf, const int (&pg)[PPT]) {
-    const uint32_t off = n16 * PT + (16 * kg) % PT;
+  auto fetch_v = [&](int hf, const int (&pg)[PPT], bool live = true) {
+    const uint32_t off = live ? n16 * PT + (16 * kg) % PT : 0u;
     if constexpr (!kLdsV) {
       const size_t ph = page_head(pg, 16 * kg);
       const uint8_t* vp = a.pools.vq + ph * (Q8 ? D * PT : NB * 16 * PT);
@@ -334,7 +336,7 @@ void DattnPart(const DecodeArgs a) {
       const int b = lane / 8, chunk = lane % 8;
       if (b < NB) {
         const size_t ps = page_head(pg, 8 * chunk);
-        const uint32_t soff = (b * PT + (8 * chunk) % PT) * 2;
+        const uint32_t soff = live ? (b * PT + (8 * chunk) % PT) * 2 : 0u;
         vsr = StreamLoad(reinterpret_cast<const uint4*>(reinterpret_cast<const uint8_t*>(a.pools.vs) + ps * (NB * PT * 2) + soff));
       }
     }
@@ -475,8 +477,8 @@ void DattnPart(const DecodeArgs a) {
     int pgc[PPT], pgn[PPT];
     load_pages(tile, pgc);
     load_k(0, pgc);
-    fetch_v(1, pgc);  // not used (the first pass has no previous tile): it keeps the count of loads in flight at the
-                      // head of the loop the same as on the way round, see below
+    fetch_v(1, pgc, false);  // not used (the first pass has no previous tile): it keeps the count of loads in flight at
+                             // the head of the loop the same as on the way round, see below
 #pragma unroll
     for (int e = 0; e < QE; ++e) {
       const int i = lane + 64 * e, sub = (i / 16) % 2;
@@ -520,7 +522,7 @@ void DattnPart(const DecodeArgs a) {
       if constexpr (!kLdsV) fetch_v(0, pgc);
       first = false;
       scores(1);
-      load_k(0, pgn);
+      load_k(0, pgn, has_next);
       // ---- online softmax (base 2); keys at or past len are masked by select, so stale scales cannot leak
       float alpha[4];
 #pragma unroll

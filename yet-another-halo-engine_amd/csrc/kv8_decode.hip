@@ -132,7 +132,9 @@ void Kv8Part(const DecodeArgs a, const Kv8Pools pools) {
   };
   // K: the 32 rows of half tile tt to the LDS slot, four rows per instruction; lane l of instruction i carries chunk
   // (l % 16) ^ (row % 16) of row 4 i + l / 16 to LDS position 1024 i + 16 l
-  auto load_k = [&](int tile, int tt, int page) {
+  // `live` false: a load whose result nobody uses (it keeps the count of loads in flight the same on every path):
+  // every lane reads the start of the piece, a few lines for the whole wave instead of the piece itself.
+  auto load_k = [&](int tile, int tt, int page, bool live = true) {
     const size_t row0 = size_t(page) * kKv8Page + (tile % 4) * kTile + 32 * tt;
     if constexpr (KB == 4) {
       // eight rows per instruction; lane l of instruction i carries chunk (l % 8) ^ (row % 8) of row 8 i + l / 8
@@ -143,9 +145,9 @@ void Kv8Part(const DecodeArgs a, const Kv8Pools pools) {
       for (int i = 0; i < 4; ++i) {
         const uint32_t rr = 8 * i + r;
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rk4, (__attribute__((address_space(3))) void*)(&lk[i * 1024]), 16,
-                                                 rr * (H * 128) + ((c ^ (rr & 7)) << 4), 0, 0, kStreamed);
+                                                 live ? rr * (H * 128) + ((c ^ (rr & 7)) << 4) : 0u, 0, 0, kStreamed);
       }
-      const uint32_t* sp4 = pools.ks + ((row0 + n32) * H + head) * 8;
+      const uint32_t* sp4 = pools.ks + ((row0 + (live ? n32 : 0)) * H + head) * 8;
       // (plain loads: the row's other quarters are wanted by the waves next to this one, and a streaming read leaves
       // nothing in the L2 for them)
       ksc4[0] = *reinterpret_cast<const uint4*>(sp4);
@@ -158,16 +160,17 @@ void Kv8Part(const DecodeArgs a, const Kv8Pools pools) {
       for (int i = 0; i < 8; ++i) {
         const uint32_t rr = 4 * i + r;
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, (__attribute__((address_space(3))) void*)(&lk[i * 1024]), 16,
-                                                 rr * (H * 256) + ((c ^ (rr & 15)) << 4), 0, 0, kStreamed);
+                                                 live ? rr * (H * 256) + ((c ^ (rr & 15)) << 4) : 0u, 0, 0, kStreamed);
       }
-      const uint32_t* sp = pools.ks + ((row0 + n32) * H + head) * 2;
+      const uint32_t* sp = pools.ks + ((row0 + (live ? n32 : 0)) * H + head) * 2;
       ksc = *reinterpret_cast<const uint2*>(sp);  // (a plain load, as for the 4-bit rows)
     }
   };
-  auto fetch_v = [&](int tile, int hf, int page) {
-    const size_t pt = size_t(page) * 16 + (tile % 4) * 4 + kg;
-    const uint32_t* vp = pools.vq + ((size_t(head) * tiles16 + pt) * 256 + 128 * hf + n16) * (VB == 4 ? 2 : 4);
-    const uint32_t* sp = pools.vs + (size_t(head) * tiles16 + pt) * 256 + 128 * hf + n16;
+  auto fetch_v = [&](int tile, int hf, int page, bool live = true) {
+    const size_t pt = size_t(page) * 16 + (tile % 4) * 4 + (live ? kg : 0);
+    const int dim = 128 * hf + (live ? n16 : 0);
+    const uint32_t* vp = pools.vq + ((size_t(head) * tiles16 + pt) * 256 + dim) * (VB == 4 ? 2 : 4);
+    const uint32_t* sp = pools.vs + (size_t(head) * tiles16 + pt) * 256 + dim;
     if constexpr (VB == 4) {
 #pragma unroll
       for (int j = 0; j < NT / 2; ++j) vb4[j] = StreamLoad(reinterpret_cast<const uint2*>(vp + 32 * j));
@@ -352,7 +355,7 @@ void Kv8Part(const DecodeArgs a, const Kv8Pools pools) {
     int tile = item >> lg_mult;
     int pgc = load_page(tile), pgn;
     load_k(tile, 0, pgc);
-    fetch_v(tile, 1, pgc);  // not used: keeps the count of loads in flight at the loop's head the same on every pass
+    fetch_v(tile, 1, pgc, false);  // not used: keeps the count of loads in flight at the loop's head the same on every pass
     if constexpr (KB == 4) {
       // Entry e of this lane: step mm = lane / 16 + 4 e, lane half hf = (lane / 8) % 2, head row rw = lane % 8, the eight
       // dims 32 (mm / 2) + 8 (2 hf + mm % 2) + [0, 8) in their natural order. H256 over a head's 256 dims, stages in the
@@ -462,7 +465,7 @@ void Kv8Part(const DecodeArgs a, const Kv8Pools pools) {
       scores(1);
       __builtin_amdgcn_s_waitcnt(0xC07F);
       __builtin_amdgcn_sched_barrier(0);
-      load_k(has_next ? ntile : tile, 0, pgn);
+      load_k(has_next ? ntile : tile, 0, pgn, has_next);
       float alpha[4];
 #pragma unroll
       for (int tt = 0; tt < 2; ++tt) {
