@@ -1029,6 +1029,8 @@ def main():
     asked_warmup = a.warmup
     headline = a.workload
     a.warmup = asked_warmup if asked_warmup is not None else WORKLOADS[headline].get("warmup", 3)
+    if headline == "ragged_b64_q8_0" and not a.no_also:
+        a.graph_replay = True   # the default run also says what its steps take as one HIP graph (an extra figure)
     res = run_workload(a, torch, yahkv)
     if headline == "ragged_b64_q8_0" and not a.no_also:
         # the other configurations, timed by the same run with their own default warm-up, a short record each

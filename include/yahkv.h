@@ -515,6 +515,20 @@ int yahkv_kv8_decode_step(const yahkv_geometry* g, const yahkv_kv8_pools* pools,
                           const void* k_new, const void* v_new, int32_t new_dtype, const void* q, int32_t q_dtype,
                           float softmax_scale, const float* gate, float* out, void* workspace, size_t workspace_bytes,
                           const yahkv_decode_options* opt, void* stream);
+/* yahkv_copy_pages and the slots (above) for these formats: a page's share of all six buffers (its rows of kq / ks, its
+ * channel means, its open tile, and per kv head its 16 tiles of vq / vs) moves together. A slot's body is a set of pools
+ * of the slot's own page count with the identity page table, in the layouts above (kq, ks, km, vq, vs, vopen one after
+ * the other), behind the same 64-byte header (6 buffers, head_dim 256, 256-token pages). */
+int yahkv_kv8_copy_pages(const yahkv_geometry* g, const yahkv_kv8_pools* pools, const int32_t* src_pages,
+                         const int32_t* dst_pages, int32_t n, void* stream);
+size_t yahkv_kv8_slot_bytes(const yahkv_geometry* g, int32_t n_pages);
+int yahkv_kv8_slot_pack(const yahkv_geometry* g, const yahkv_kv8_pools* pools, const int32_t* table_row, int32_t n_pages,
+                        int32_t n_tokens, void* slot, void* stream);
+int yahkv_kv8_slot_check(const yahkv_geometry* g, const void* header, size_t slot_bytes, int32_t* n_pages,
+                         int32_t* n_tokens);
+int yahkv_kv8_slot_unpack(const yahkv_geometry* g, const yahkv_kv8_pools* pools, const int32_t* table_row,
+                          int32_t n_pages, const void* slot, void* stream);
+
 /* The reference's own slot files ("YAHSLOT1": LoomPrefill::SaveState / LoadState, engine/model/loom_prefill.hpp:976-1024):
  * five u64 {magic, T, B, chunks, nbufs = 10}, then per buffer a u64 byte count and the raw bytes, in the order page
  * table, kq, ks, km, vq, vs, f16 K pool, f16 V^T pool, convolution rings, DeltaNet states (StateBuffers(), :1027-1030);

@@ -456,3 +456,55 @@ def test_other_kv_head_counts(yahkv, torch_gpu, n_q, H, kb):
     for s, n in enumerate(lens):
         Kd, Vd = kv8.dense(hp, table[s], n + 1)
         assert rel_err(out[s], closed_form(Kd, Vd, rot(q[s]), 1.0 / 16.0)) < TOL, (s, n)
+
+
+@pytest.mark.parametrize("kb,vb", [(8, 8), (4, 4)])
+def test_page_copies_and_slots(yahkv, torch_gpu, rc, kb, vb):
+    """yahkv_kv8_copy_pages moves a page's share of all six buffers; a slot's body is the sequence's pools with the identity
+    page table (the oracle's pools_of_sequence, buffer after buffer); it unpacks into other pages of another pool, where
+    the attention gives the same bits; headers of another geometry are refused."""
+    torch = torch_gpu
+    n = 700
+    g = yahkv.kv8_geometry(24, 4, rc.T // 256, kb, vb)
+    dp = yahkv.Kv8Pools(g, 0x5A)
+    arrs = dp.numpy()
+    arrs["km"][rc.ptab[0]] = rc.m
+    dp.load(arrs)
+    table = torch.from_numpy(rc.ptab[None].copy()).cuda()
+    yahkv.kv8_append(dp, table, torch.zeros(1, dtype=torch.int32, device="cuda"),
+                     torch.from_numpy(rc.K[None, :n].reshape(1, n, 4, 256)).cuda(), torch.from_numpy(rc.V[None, :n].reshape(1, n, 4, 256)).cuda())
+    q = torch.from_numpy(rc.q[None]).cuda()
+    sl = torch.tensor([n], dtype=torch.int32, device="cuda")
+    want = yahkv.kv8_decode_attend(dp, table, sl, n, q, 0.0625).cpu().numpy()
+    # the slot: header, then pools of three pages with the identity table
+    slot = yahkv.kv8_slot_pack(dp, table[0], 3, n)
+    host = slot.cpu().numpy()
+    assert yahkv.kv8_slot_check(g, host) == (3, n)
+    hp, _ = kv8.pools_of_sequence(dp, rc.ptab, n)
+    body = b"".join(np.ascontiguousarray(getattr(hp, name)).tobytes() for name in ("kq", "ks", "km", "vq", "vs", "vo"))
+    assert host[64:].tobytes() == body
+    other = yahkv.kv8_geometry(16, 2, rc.T // 256, kb, vb)
+    with pytest.raises(yahkv.YahkvError):
+        yahkv.kv8_slot_check(other, host)
+    with pytest.raises(yahkv.YahkvError):
+        yahkv.kv8_slot_check(g, host[:-16])
+    # into pages (6, 1, 4) of a pool of seven pages
+    g7 = yahkv.kv8_geometry(24, 4, 7, kb, vb)
+    dp7 = yahkv.Kv8Pools(g7, 0x33)
+    row = torch.tensor([6, 1, 4], dtype=torch.int32, device="cuda")
+    yahkv.kv8_slot_unpack(dp7, row, 3, slot)
+    got = yahkv.kv8_decode_attend(dp7, row[None], sl, n, q, 0.0625).cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    a7 = dp7.numpy()
+    for untouched in (0, 2, 3, 5):
+        assert np.all(a7["kq"][untouched * 256:untouched * 256 + 256] == 0x33333333)
+        assert np.all(a7["vq"][:, untouched * 16:untouched * 16 + 16] == 0x33333333) and np.all(a7["vo"][untouched] == 0x3333)
+    # a page copied inside the pools carries all six buffers' shares
+    yahkv.kv8_copy_pages(dp7, torch.tensor([4], dtype=torch.int32, device="cuda"), torch.tensor([0], dtype=torch.int32, device="cuda"))
+    b7 = dp7.numpy()
+    for name in ("kq", "ks"):
+        assert np.array_equal(b7[name][0:256], a7[name][4 * 256:5 * 256]), name
+    assert np.array_equal(b7["vq"][:, 0:16], a7["vq"][:, 64:80]) and np.array_equal(b7["vs"][:, 0:16], a7["vs"][:, 64:80])
+    assert np.array_equal(b7["vo"][0], a7["vo"][4]) and np.array_equal(b7["km"][0].view(np.uint32), a7["km"][4].view(np.uint32))
+    got2 = yahkv.kv8_decode_attend(dp7, torch.tensor([[6, 1, 0]], dtype=torch.int32, device="cuda"), sl, n, q, 0.0625).cpu().numpy()
+    assert np.array_equal(got2.view(np.uint32), want.view(np.uint32))

@@ -116,6 +116,8 @@ def _load():
     lib.yahkv_kv8_decode_part.argtypes = [G, K8, i32p, i32, i32p, i32, i32, vp, i32, C.c_float, vp, C.c_size_t, O, vp]
     lib.yahkv_kv8_decode_reduce.argtypes = [G, K8, i32p, i32, i32p, i32, i32, vp, vp, i32, vp, i32, C.c_float, vp, vp,
                                             vp, C.c_size_t, O, vp]
+    lib.yahkv_kv8_slot_bytes.restype = C.c_size_t
+    lib.yahkv_kv8_slot_bytes.argtypes = [G, i32]
     lib.yahkv_kv8_prefill_workspace_bytes.restype = C.c_size_t
     lib.yahkv_kv8_prefill_workspace_bytes.argtypes = [G, i32, i32, i32]
     lib.yahkv_kv8_prefill_attend.argtypes = [G, K8, i32p, i32, i32p, i32, i32, i32, vp, C.c_float, vp, vp, i32, vp,
@@ -631,6 +633,36 @@ class Kv8Pools:
         for n in self.NAMES:
             a = arrays["vo" if n == "vopen" else n]
             getattr(self, n).copy_(torch.from_numpy(np.ascontiguousarray(a).view(np.uint8).reshape(-1)))
+
+
+def kv8_copy_pages(pools, src_pages, dst_pages):
+    """Whole pages src_pages[i] -> dst_pages[i] (int32 cuda tensors) in all six buffers."""
+    g, st = pools.geom, pools.struct()
+    _check(lib.yahkv_kv8_copy_pages(C.byref(g), C.byref(st), _dp(src_pages), _dp(dst_pages), src_pages.numel(), _stream()),
+           "kv8_copy_pages")
+
+
+def kv8_slot_pack(pools, table_row, n_pages, n_tokens):
+    """The sequence's pages (device int32 row) as one uint8 cuda tensor: header + pools of n_pages pages, identity table."""
+    import torch
+    g, st = pools.geom, pools.struct()
+    slot = torch.empty(lib.yahkv_kv8_slot_bytes(C.byref(g), n_pages), dtype=torch.uint8, device=table_row.device)
+    _check(lib.yahkv_kv8_slot_pack(C.byref(g), C.byref(st), _dp(table_row), n_pages, n_tokens, _dp(slot), _stream()),
+           "kv8_slot_pack")
+    return slot
+
+
+def kv8_slot_check(g, slot_host):
+    """(n_pages, n_tokens) of a slot held in a uint8 numpy array; raises where the geometry does not match."""
+    np_, nt = C.c_int32(0), C.c_int32(0)
+    _check(lib.yahkv_kv8_slot_check(C.byref(g), C.c_void_p(slot_host.ctypes.data), C.c_size_t(slot_host.size), C.byref(np_),
+                                    C.byref(nt)), "kv8_slot_check")
+    return np_.value, nt.value
+
+
+def kv8_slot_unpack(pools, table_row, n_pages, slot):
+    g, st = pools.geom, pools.struct()
+    _check(lib.yahkv_kv8_slot_unpack(C.byref(g), C.byref(st), _dp(table_row), n_pages, _dp(slot), _stream()), "kv8_slot_unpack")
 
 
 class RefSlotInfo(C.Structure):
