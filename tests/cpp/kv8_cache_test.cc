@@ -7,6 +7,7 @@
 #include <cstdio>
 #include <cstring>
 #include <random>
+#include <string>
 #include <vector>
 
 #include "kv8_cache.hpp"
@@ -152,7 +153,7 @@ int RunTest(int kb, int vb) {
     const float scale = 0.0625f;
     Kv8Prefill pre(dec);
     std::vector<int32_t> prefix(B, 0);
-    double worst_prefill = 0, worst_decode = 0;
+    double worst_prefill = 0, worst_decode = 0, worst_twin = 0;
     for (int round = 0; round < 2; ++round) {
       Stage(round == 0 ? "first chunk (channel means, chunk append, attention)" : "second chunk (starts inside a tile)");
       const int chunk = round == 0 ? chunk0 : chunk1;
@@ -213,11 +214,81 @@ int RunTest(int kb, int vb) {
     pools_equal("after the decode steps");
     Expect(worst_decode < 2e-3, "decode attention differs from the closed form");
     Expect(dec.length(0) == chunk0 + chunk1 + steps && dec.pages(0).size() == 2 && dec.length(2) == steps, "lengths after the steps");
+    Stage("fork and slots (sequence 1 becomes a copy of sequence 0, then is loaded from its slot)");
+    {
+      auto read_file = [](const std::string& path) {
+        std::vector<uint8_t> b;
+        FILE* f = std::fopen(path.c_str(), "rb");
+        if (f == nullptr) throw Fail("a slot file is missing");
+        uint8_t buf[1 << 16];
+        for (size_t n; (n = std::fread(buf, 1, sizeof buf, f)) > 0;) b.insert(b.end(), buf, buf + n);
+        std::fclose(f);
+        return b;
+      };
+      // both sequences take the same rows: the outputs agree up to where the cut places the sequences' tiles (each
+      // part rounds its weights to f16 against its own running maximum), and what the steps write is the same byte
+      // for byte
+      auto twin_steps = [&](int n, const char* what) {
+        for (int i = 0; i < n; ++i) {
+          std::vector<float> k1 = randn(W, 0.6f), v1 = randn(W, 0.0f), q1 = randn(size_t(NQ) * D, 0.0f);
+          k1.insert(k1.end(), k1.begin(), k1.begin() + W), v1.insert(v1.end(), v1.begin(), v1.begin() + W);
+          q1.insert(q1.end(), q1.begin(), q1.begin() + size_t(NQ) * D);
+          DeviceBuffer dk = to_dev_bf16(k1), dv = to_dev_bf16(v1), dq = to_dev_bf16(q1), dout(q1.size() * 4);
+          dec.Step(2, dk.get(), dv.get(), YAHKV_BF16, dq.get(), YAHKV_BF16, scale, nullptr, static_cast<float*>(dout.get()));
+          std::vector<float> got(q1.size());
+          CheckHip(hipMemcpy(got.data(), dout.get(), got.size() * 4, hipMemcpyDeviceToHost), "d2h");
+          double d = 0, m = 0;
+          for (size_t j = 0; j < size_t(NQ) * D; ++j)
+            d = std::max(d, double(std::fabs(got[j] - got[size_t(NQ) * D + j]))), m = std::max(m, double(std::fabs(got[j])));
+          worst_twin = std::max(worst_twin, d / m);
+          if (!(d <= 1e-3 * m)) throw Fail((std::string(what) + ": the copy attends differently").c_str());
+        }
+      };
+      const std::string a = "/tmp/yahkv_kv8_cache_test_a.slot", b = "/tmp/yahkv_kv8_cache_test_b.slot";
+      auto slots_equal = [&](const char* what) {
+        dec.SaveSlot(0, a), dec.SaveSlot(1, b);
+        const std::vector<uint8_t> fa = read_file(a), fb = read_file(b);
+        if (fa.size() != yahkv_kv8_slot_bytes(&g, int32_t(dec.pages(0).size())) || fa != fb)
+          throw Fail((std::string(what) + ": the two sequences' slots differ").c_str());
+      };
+      ExpectThrow([&] { dec.Fork(0, 1); }, "a fork into a sequence that holds pages must throw");
+      dec.Release(1);
+      const int32_t free_before = dec.free_pages(), len0 = dec.length(0);
+      dec.Fork(0, 1);  // 280 tokens: the first page shared, the second copied with its open tile
+      Expect(dec.length(1) == len0 && dec.pages(1).size() == 2 && dec.pages(1)[0] == dec.pages(0)[0] &&
+                 dec.pages(1)[1] != dec.pages(0)[1] && dec.free_pages() == free_before - 1, "pages after the fork");
+      twin_steps(10, "after the fork");  // to 290: two tiles close
+      slots_equal("after the fork");
+      dec.Release(1);
+      Expect(dec.free_pages() == free_before, "a released fork gives back its own page only");
+      ExpectThrow([&] { dec.LoadSlot(0, a); }, "a slot loads into an empty sequence only");
+      Expect(dec.LoadSlot(1, a) == len0 + 10 && dec.length(1) == len0 + 10 && dec.pages(1).size() == 2 &&
+                 dec.pages(1)[0] != dec.pages(0)[0], "a loaded slot's length and pages");
+      twin_steps(250, "after the load");  // past the next page boundary (512)
+      slots_equal("after the load");
+      Expect(dec.pages(1).size() == 3, "pages after the steps");
+      {
+        const yahkv_geometry other{kb == 8 ? YAHKV_KV4A16 : YAHKV_KV8A16, NQ, H, D, 256, P};
+        Kv8Decoder wrong(other, 1, T);
+        wrong.Bind(wrong.OwnState());
+        ExpectThrow([&] { wrong.LoadSlot(0, a); }, "a slot of another format must be refused");
+        std::vector<uint8_t> cut = read_file(a);
+        cut.resize(cut.size() - 1);
+        FILE* f = std::fopen(b.c_str(), "wb");
+        std::fwrite(cut.data(), 1, cut.size(), f), std::fclose(f);
+        dec.Release(1);
+        ExpectThrow([&] { dec.LoadSlot(1, b); }, "a truncated slot must be refused");
+        Expect(dec.pages(1).empty(), "a refused slot leaves the sequence empty");
+      }
+      std::remove(a.c_str()), std::remove(b.c_str());
+      dec.ResumeAt(1, 0);
+    }
     ExpectThrow([&] { dec.ResumeAt(1, 100); dec.Step(2, nullptr, nullptr, YAHKV_BF16, nullptr, YAHKV_BF16, 1.0f, nullptr, nullptr); },
                 "a step inside a tile the open tile does not cover must throw");
     dec.Release(0), dec.Release(1), dec.Release(2);
     Expect(dec.free_pages() == P, "every page back in the pool");
-    std::printf("kv8_cache_test: ok, kv%da16 (prefill %.2e, decode %.2e)\n", kb, worst_prefill, worst_decode);
+    std::printf("kv8_cache_test: ok, kv%da16 (prefill %.2e, decode %.2e, a copy against its source %.2e)\n", kb,
+                worst_prefill, worst_decode, worst_twin);
     return 0;
   } catch (const std::exception& e) {
     std::printf("kv8_cache_test: FAILED: %s\n", e.what());

@@ -51,7 +51,14 @@ class Kv8Decoder {
   }
 
   int32_t context() const { return T_; }
-  std::pair<uint32_t, uint32_t> kv_bits() const { return {8u, 8u}; }
+  std::pair<uint32_t, uint32_t> kv_bits() const {
+    switch (g_.format) {
+      case YAHKV_KV4A16: return {4u, 4u};
+      case YAHKV_K8V4A16: return {8u, 4u};
+      case YAHKV_K4V8A16: return {4u, 8u};
+      default: return {8u, 8u};
+    }
+  }
   bool quant() const { return true; }
   size_t KqBytes() const { return yahkv_kv8_kq_bytes(&g_); }
   size_t KsBytes() const { return yahkv_kv8_ks_bytes(&g_); }
@@ -123,6 +130,87 @@ class Kv8Decoder {
     len_[size_t(seq)] = 0, open_at_[size_t(seq)] = 0;
   }
 
+  // Sequence `dst` (empty) becomes a copy of `src` that shares its full pages; the last, partly filled page is copied
+  // with its open tile (and, where it is also the first page, the channel means), so both can go on appending. The
+  // means of a longer sequence stay with the shared first page: they are written by the first chunk only.
+  void Fork(int32_t src, int32_t dst) {
+    if (!bound_) throw KvError("kv8 decoder: no state bound");
+    if (src == dst || !pages_.at(size_t(dst)).empty()) throw KvError("kv8 decoder: fork needs an empty target sequence");
+    const auto& from = pages_.at(size_t(src));
+    const int32_t len = len_[size_t(src)], full = len / g_.page_tokens;
+    std::vector<int32_t> shared(from.begin(), from.begin() + full);
+    pool_->Retain(shared);
+    auto& to = pages_[size_t(dst)];
+    to = shared;
+    if (len % g_.page_tokens != 0) {
+      const std::vector<int32_t> own = pool_->Alloc(1);
+      const int32_t pair[2] = {from[size_t(full)], own[0]};
+      DeviceBuffer ids(sizeof pair);
+      CheckHip(hipMemcpyAsync(ids.get(), pair, sizeof pair, hipMemcpyHostToDevice, stream_), "fork");
+      const yahkv_kv8_pools pools = PoolsOf(st_);
+      Check(yahkv_kv8_copy_pages(&g_, &pools, static_cast<const int32_t*>(ids.get()),
+                                 static_cast<const int32_t*>(ids.get()) + 1, 1, stream_), "kv8_copy_pages");
+      CheckHip(hipStreamSynchronize(stream_), "fork");  // `ids` and `pair` go out of scope
+      to.push_back(own[0]);
+    }
+    for (size_t i = 0; i < to.size(); ++i) table_[size_t(dst) * stride_ + i] = to[i];
+    len_[size_t(dst)] = len;
+    open_at_[size_t(dst)] = open_at_[size_t(src)];
+    table_dirty_ = true;
+  }
+
+  // A sequence's state as a slot file: the 64-byte header and the sequence's share of the six buffers, raw
+  // (yahkv_kv8_slot_pack); LoadSlot puts it into free pages of this decoder and returns the tokens it covers, so the
+  // caller continues at that position, open tile included (SaveState / LoadState, loom_prefill.hpp:979-1019).
+  void SaveSlot(int32_t seq, const std::string& path) {
+    if (!bound_) throw KvError("kv8 decoder: no state bound");
+    const int32_t len = len_.at(size_t(seq)), np = (len + g_.page_tokens - 1) / g_.page_tokens;
+    if (np <= 0) throw KvError("kv8 decoder: nothing to save");
+    if (len % 16 != 0 && len != open_at_[size_t(seq)]) throw KvError("kv8 decoder: the open tile does not reach the length");
+    Upload();
+    const size_t bytes = yahkv_kv8_slot_bytes(&g_, np);
+    DeviceBuffer slot(bytes);
+    const yahkv_kv8_pools pools = PoolsOf(st_);
+    Check(yahkv_kv8_slot_pack(&g_, &pools, static_cast<const int32_t*>(st_.ptab.ptr) + size_t(seq) * stride_, np, len,
+                              slot.get(), stream_), "kv8_slot_pack");
+    std::vector<uint8_t> host(bytes);
+    CheckHip(hipMemcpyAsync(host.data(), slot.get(), bytes, hipMemcpyDeviceToHost, stream_), "slot");
+    CheckHip(hipStreamSynchronize(stream_), "slot");
+    FILE* f = std::fopen(path.c_str(), "wb");
+    if (f == nullptr) throw KvError("kv8 decoder: cannot write the slot " + path);
+    const bool ok = std::fwrite(host.data(), 1, bytes, f) == bytes;
+    if (std::fclose(f) != 0 || !ok) throw KvError("kv8 decoder: short write to the slot " + path);
+  }
+  int32_t LoadSlot(int32_t seq, const std::string& path) {
+    if (!bound_) throw KvError("kv8 decoder: no state bound");
+    if (!pages_.at(size_t(seq)).empty()) throw KvError("kv8 decoder: a slot loads into an empty sequence");
+    FILE* f = std::fopen(path.c_str(), "rb");
+    if (f == nullptr) throw KvError("kv8 decoder: cannot open the slot " + path);
+    std::vector<uint8_t> host;
+    uint8_t buf[1 << 16];
+    for (size_t n; (n = std::fread(buf, 1, sizeof buf, f)) > 0;) host.insert(host.end(), buf, buf + n);
+    std::fclose(f);
+    int32_t np = 0, len = 0;
+    if (yahkv_kv8_slot_check(&g_, host.data(), host.size(), &np, &len) != YAHKV_OK)
+      throw KvError("kv8 decoder: the slot " + path + " does not match this geometry");
+    // the header's page count is the one the tokens need, and the sequence's row holds exactly those pages: a slot
+    // never reaches pages the sequence does not own
+    if (np != (len + g_.page_tokens - 1) / g_.page_tokens || np > stride_)
+      throw KvError("kv8 decoder: the slot " + path + " names more pages than its tokens fill");
+    Reserve(seq, len);
+    if (int32_t(pages_[size_t(seq)].size()) != np) throw KvError("kv8 decoder: the slot " + path + " does not fit the sequence");
+    Upload();
+    DeviceBuffer slot(host.size());
+    CheckHip(hipMemcpyAsync(slot.get(), host.data(), host.size(), hipMemcpyHostToDevice, stream_), "slot");
+    const yahkv_kv8_pools pools = PoolsOf(st_);
+    Check(yahkv_kv8_slot_unpack(&g_, &pools, static_cast<const int32_t*>(st_.ptab.ptr) + size_t(seq) * stride_, np,
+                                slot.get(), stream_), "kv8_slot_unpack");
+    CheckHip(hipStreamSynchronize(stream_), "slot");
+    len_[size_t(seq)] = len;
+    open_at_[size_t(seq)] = len;
+    return len;
+  }
+
   // The next Step of `seq` writes position pos. With quantized V the open tile must hold the keys since the last 16-key
   // boundary: pos is such a boundary, or the position the open tile was last written up to (by a Step, or seeded by the
   // prefill: SeedOpenTile, loom_prefill.hpp:944-947) (loom_decoder.hpp:233-235).
@@ -174,7 +262,9 @@ class Kv8Decoder {
     if (!table_dirty_) return;
     std::vector<int32_t> owned(static_cast<size_t>(max_seqs_), 0);
     for (int32_t s = 0; s < max_seqs_; ++s) owned[size_t(s)] = int32_t(pages_[size_t(s)].size()) * g_.page_tokens;
-    Check(yahkv_validate_page_table(&g_, table_.data(), stride_, owned.data(), max_seqs_), "page table");
+    // forked sequences share their full pages: a page may appear as often as the allocator has it retained
+    Check(yahkv_validate_shared_page_table(&g_, pool_->handle(), table_.data(), stride_, owned.data(), max_seqs_),
+          "page table");
     CheckHip(hipMemcpyAsync(st_.ptab.ptr, table_.data(), sizeof(int32_t) * table_.size(), hipMemcpyHostToDevice, stream_),
              "page table upload");
     CheckHip(hipStreamSynchronize(stream_), "page table upload");
