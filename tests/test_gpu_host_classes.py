@@ -48,3 +48,15 @@ def test_kv_cache_header_is_host_only_cxx():
                         "-I", os.path.join(ROOT, "include"), "-I", os.path.join(ROOT, "yet-another-halo-engine_amd", "csrc"),
                         "-I", "/opt/rocm/include", "-"], input=src, capture_output=True, text=True, timeout=120)
     assert r.returncode == 0, r.stderr
+
+
+@pytest.mark.gpu
+def test_kv8_batcher_cpp_program():
+    """The same driver over pools in the reference's own formats (kv8a16, then kv4a16): ten requests through five
+    pages, chunks that start inside tiles and pages, first and later chunks in one step; all six buffers of both layers
+    bit for bit against the oracle after every step, attention rows against the closed form."""
+    exe = os.path.join(ROOT, "tests", "cpp", "kv8_batcher_test")
+    assert os.path.exists(exe), "tests/cpp/kv8_batcher_test is not built: run `python __graft_entry__.py build`"
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=200)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert r.stdout.count("kv8_batcher_test: ok") == 2

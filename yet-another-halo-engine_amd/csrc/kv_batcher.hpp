@@ -239,53 +239,36 @@ class BatchScheduler {
   bool planned_ = false;
 };
 
-class KvBatcher {
+// The planned step's page-table rows and columns on the device: rows of the plan's prompt chunks, then of its decode
+// tokens, and per row the prefix, valid, position and length columns. Shared by the batchers of both format families.
+class StepStage {
  public:
-  // g.n_pages pages per layer; the layers share the page table.
-  KvBatcher(const yahkv_geometry& g, int32_t n_layers, int32_t max_running, int32_t context, int32_t chunk,
-            int32_t max_prefill, hipStream_t stream = nullptr, uint64_t shuffle_seed = 0)
-      : g_(g), stream_(stream),
-        sched_(g.n_pages, g.page_tokens, max_running, context, chunk, max_prefill, shuffle_seed) {
-    Check(yahkv_check_geometry(&g_), "batcher");
-    if (n_layers <= 0) throw KvError("batcher: bad sizes");
+  StepStage(const yahkv_geometry& g, int32_t max_running, int32_t max_prefill, int32_t context, hipStream_t stream)
+      : g_(g), stream_(stream) {
     stride_ = (context + g_.page_tokens - 1) / g_.page_tokens;
-    for (int32_t l = 0; l < n_layers; ++l) {
-      layers_.emplace_back();
-      Layer& L = layers_.back();
-      L.kq = DeviceBuffer(yahkv_kq_bytes(&g_)), L.ks = DeviceBuffer(yahkv_ks_bytes(&g_));
-      L.vq = DeviceBuffer(yahkv_vq_bytes(&g_)), L.vs = DeviceBuffer(yahkv_vs_bytes(&g_));
-    }
-    workspace_ = DeviceBuffer(yahkv_decode_workspace_bytes(&g_, max_running, context, nullptr));
-    // per step: table rows of the planned requests, then prefix, valid, position and length columns
     rows_ = size_t(max_running) + size_t(max_prefill);
-    stage_ints_ = rows_ * size_t(stride_) + 4 * rows_;
-    stage_dev_ = DeviceBuffer(sizeof(int32_t) * stage_ints_);
-    CheckHip(hipHostMalloc(reinterpret_cast<void**>(&stage_), sizeof(int32_t) * stage_ints_), "hipHostMalloc");
+    ints_ = rows_ * size_t(stride_) + 4 * rows_;
+    dev_ = DeviceBuffer(sizeof(int32_t) * ints_);
+    CheckHip(hipHostMalloc(reinterpret_cast<void**>(&host_), sizeof(int32_t) * ints_), "hipHostMalloc");
   }
-  KvBatcher(const KvBatcher&) = delete;
-  KvBatcher& operator=(const KvBatcher&) = delete;
-  ~KvBatcher() {
-    if (stage_ != nullptr) (void)hipHostFree(stage_);
+  StepStage(const StepStage&) = delete;
+  StepStage& operator=(const StepStage&) = delete;
+  ~StepStage() {
+    if (host_ != nullptr) (void)hipHostFree(host_);
   }
 
-  void Submit(int64_t id, int32_t prompt_len, int32_t max_new) { sched_.Submit(id, prompt_len, max_new); }
-  void Stop(int64_t id) { sched_.Stop(id); }
-  std::vector<int64_t> TakeFinished() { return sched_.TakeFinished(); }
-
-  // Plans the step (BatchScheduler::Schedule), checks the page table it implies and sends it to the device.
-  const BatchPlan& Schedule() {
-    const BatchPlan& plan = sched_.Schedule();
+  // Checks the page table the plan implies and sends it to the device.
+  void Upload(const BatchScheduler& sched, const BatchPlan& plan) {
     const int32_t np = int32_t(plan.prefill.size()), nd = int32_t(plan.decode.size());
-    if (np + nd == 0) return plan;
     CheckHip(hipStreamSynchronize(stream_), "batcher");  // the last step has read the staging buffer
-    int32_t* table = stage_;
-    int32_t* prefix = stage_ + rows_ * size_t(stride_);
+    int32_t* table = host_;
+    int32_t* prefix = host_ + rows_ * size_t(stride_);
     int32_t *valid = prefix + rows_, *pos = valid + rows_, *len = pos + rows_;
     std::vector<int32_t> owned(size_t(np + nd));
     max_prefix_ = 0;
     for (int32_t i = 0; i < np + nd; ++i) {
       const BatchWork& w = i < np ? plan.prefill[size_t(i)] : plan.decode[size_t(i - np)];
-      const std::vector<int32_t>& pages = sched_.pages(w.id);
+      const std::vector<int32_t>& pages = sched.pages(w.id);
       std::fill(table + size_t(i) * stride_, table + size_t(i + 1) * stride_, 0);
       std::copy(pages.begin(), pages.end(), table + size_t(i) * stride_);
       owned[size_t(i)] = int32_t(pages.size()) * g_.page_tokens;
@@ -296,10 +279,59 @@ class KvBatcher {
         pos[i - np] = w.pos, len[i - np] = w.pos + 1;
       }
     }
-    Check(yahkv_validate_shared_page_table(&g_, sched_.pool().handle(), table, stride_, owned.data(), np + nd),
+    Check(yahkv_validate_shared_page_table(&g_, sched.pool().handle(), table, stride_, owned.data(), np + nd),
           "page table");
-    CheckHip(hipMemcpyAsync(stage_dev_.get(), stage_, sizeof(int32_t) * stage_ints_, hipMemcpyHostToDevice, stream_),
-             "batcher upload");
+    CheckHip(hipMemcpyAsync(dev_.get(), host_, sizeof(int32_t) * ints_, hipMemcpyHostToDevice, stream_), "batcher upload");
+  }
+
+  int32_t stride() const { return stride_; }
+  int32_t max_prefix() const { return max_prefix_; }
+  // device pointers: the table's rows (prompt chunks first), the chunks' prefix lengths and valid rows, the decode
+  // rows' positions and lengths
+  const int32_t* table() const { return static_cast<const int32_t*>(dev_.get()); }
+  const int32_t* prefix() const { return table() + rows_ * size_t(stride_); }
+  const int32_t* valid() const { return prefix() + rows_; }
+  const int32_t* pos() const { return valid() + rows_; }
+  const int32_t* len() const { return pos() + rows_; }
+
+ private:
+  yahkv_geometry g_;
+  hipStream_t stream_;
+  int32_t stride_ = 0, max_prefix_ = 0;
+  size_t rows_ = 0, ints_ = 0;
+  DeviceBuffer dev_;
+  int32_t* host_ = nullptr;
+};
+
+class KvBatcher {
+ public:
+  // g.n_pages pages per layer; the layers share the page table.
+  KvBatcher(const yahkv_geometry& g, int32_t n_layers, int32_t max_running, int32_t context, int32_t chunk,
+            int32_t max_prefill, hipStream_t stream = nullptr, uint64_t shuffle_seed = 0)
+      : g_(g), stream_(stream),
+        sched_(g.n_pages, g.page_tokens, max_running, context, chunk, max_prefill, shuffle_seed),
+        stage_(g, max_running, max_prefill, context, stream) {
+    Check(yahkv_check_geometry(&g_), "batcher");
+    if (n_layers <= 0) throw KvError("batcher: bad sizes");
+    for (int32_t l = 0; l < n_layers; ++l) {
+      layers_.emplace_back();
+      Layer& L = layers_.back();
+      L.kq = DeviceBuffer(yahkv_kq_bytes(&g_)), L.ks = DeviceBuffer(yahkv_ks_bytes(&g_));
+      L.vq = DeviceBuffer(yahkv_vq_bytes(&g_)), L.vs = DeviceBuffer(yahkv_vs_bytes(&g_));
+    }
+    workspace_ = DeviceBuffer(yahkv_decode_workspace_bytes(&g_, max_running, context, nullptr));
+  }
+  KvBatcher(const KvBatcher&) = delete;
+  KvBatcher& operator=(const KvBatcher&) = delete;
+
+  void Submit(int64_t id, int32_t prompt_len, int32_t max_new) { sched_.Submit(id, prompt_len, max_new); }
+  void Stop(int64_t id) { sched_.Stop(id); }
+  std::vector<int64_t> TakeFinished() { return sched_.TakeFinished(); }
+
+  // Plans the step (BatchScheduler::Schedule), checks the page table it implies and sends it to the device.
+  const BatchPlan& Schedule() {
+    const BatchPlan& plan = sched_.Schedule();
+    if (!plan.empty()) stage_.Upload(sched_, plan);
     return plan;
   }
 
@@ -317,9 +349,8 @@ class KvBatcher {
     const BatchPlan& plan = sched_.plan();
     const int32_t np = int32_t(plan.prefill.size()), nd = int32_t(plan.decode.size());
     if (np + nd == 0) return;
-    const int32_t* d = static_cast<const int32_t*>(stage_dev_.get());
-    const int32_t* d_prefix = d + rows_ * size_t(stride_);
-    const int32_t *d_valid = d_prefix + rows_, *d_len = d_valid + 2 * size_t(rows_);  // (between them: the decode rows' positions)
+    const int32_t *d = stage_.table(), *d_prefix = stage_.prefix(), *d_valid = stage_.valid(), *d_len = stage_.len();
+    const int32_t stride_ = stage_.stride(), max_prefix_ = stage_.max_prefix();
     const yahkv_pools pools = this->pools(layer);
     const int32_t chunk = sched_.chunk(), T = sched_.context();
     if (np > 0) {
@@ -349,7 +380,7 @@ class KvBatcher {
   int32_t queued() const { return sched_.queued(); }
   int32_t free_pages() const { return sched_.free_pages(); }
   int32_t n_layers() const { return int32_t(layers_.size()); }
-  int32_t page_table_stride() const { return stride_; }
+  int32_t page_table_stride() const { return stage_.stride(); }
   const BatchStats& stats() const { return sched_.stats(); }
   const yahkv_geometry& geometry() const { return g_; }
   yahkv_pools pools(int32_t layer) const {
@@ -366,11 +397,9 @@ class KvBatcher {
   yahkv_geometry g_;
   hipStream_t stream_;
   BatchScheduler sched_;
-  int32_t stride_ = 0, max_prefix_ = 0;
+  StepStage stage_;
   std::vector<Layer> layers_;
-  DeviceBuffer workspace_, images_, stage_dev_;
-  int32_t* stage_ = nullptr;
-  size_t rows_ = 0, stage_ints_ = 0;
+  DeviceBuffer workspace_, images_;
 };
 
 }  // namespace yahkv_host
