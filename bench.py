@@ -826,8 +826,11 @@ def run_decode(a, wl, torch, yahkv):
     # which instance of the part kernel the library picks (its last template argument): 1 merges in the same launch,
     # 2 leaves one partial per workgroup for a chunk's last pair (the library's rule for a batch with few tiles per wave)
     chunks = torch.cuda.get_device_properties(0).multi_processor_count
-    few_tiles = -(-max_len // 64) * B * NKV <= chunks * 8 * 4
-    part_mode = 1 if a.one_launch else 2 if a.wg_partials == 1 or (a.wg_partials == 0 and few_tiles) else 0
+    line = -(-max_len // 64) * B * NKV
+    few_tiles = line <= chunks * 8 * 4
+    # 3: the kernel of its own for q8_0 with at most two tiles per wave (DattnPartWhole: a wave asks for a whole tile at once)
+    whole = a.wg_partials in (0, 3) and g.format == 8 and not a.one_launch and line <= chunks * 8 * 2
+    part_mode = 1 if a.one_launch else 3 if whole else 2 if a.wg_partials in (1, 3) or (a.wg_partials == 0 and few_tiles) else 0
     # set-up, as a server does once: the XCDs' relative read speeds on this batch (equal shares without it)
     xcd = yahkv.decode_calibrate(pools, t_table, len_rows[0], max_len, q, ws, opt, rounds=3) if not a.no_calibrate else None
     if a.one_launch:
@@ -910,7 +913,7 @@ def run_decode(a, wl, torch, yahkv):
         "roofline": {"bound": "hbm", "achieved": round(kgbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(kgbs / HBM_PEAK_GBS, 4), "traffic": TRAFFIC.get(a.workload, (None, None))[0],
                      "traffic_source": TRAFFIC.get(a.workload, (None, None))[1],
-                     "kernel": "DattnPart<%d, %d, %d, %d>" % (wl["fmt"], HD, PT, part_mode),
+                     "kernel": "DattnPartWhole" if part_mode == 3 else "DattnPart<%d, %d, %d, %d>" % (wl["fmt"], HD, PT, part_mode),
                      "kernel_ms": round(kern_ms, 4)},
     }
     # The same number of steps again, right after three idle seconds and without warm-up: what a server's first steps
@@ -997,9 +1000,10 @@ def main():
                     help="quantized prefill workloads: no workspace, the attention kernel decodes its tiles itself")
     ap.add_argument("--min-chunk-tiles", type=int, default=0,
                     help="decode workloads: yahkv_decode_options::min_chunk_tiles (0: the library's default)")
-    ap.add_argument("--wg-partials", type=int, default=0, choices=[0, 1, 2],
+    ap.add_argument("--wg-partials", type=int, default=0, choices=[0, 1, 2, 3],
                     help="q8_0 / q4_0 decode workloads: yahkv_decode_options::wg_partials (1: one partial per workgroup for a "
-                         "chunk's last pair, 2: one per wave, 0: chosen from the batch's size)")
+                         "chunk's last pair, 2: one per wave, 3: one per workgroup from waves that ask for whole tiles, "
+                         "0: chosen from the batch's size)")
     ap.add_argument("--cut", type=int, default=0, choices=[0, 1, 2],
                     help="q8_0 / q4_0 decode workloads: yahkv_decode_options::cut (1: by (sequence, kv head), 2: by "
                          "(sequence, tile) with the kv heads of a tile on neighbouring waves, 0: the library's choice)")

@@ -172,8 +172,12 @@ typedef struct yahkv_decode_options {
                                counts live in the workspace and must start at zero: call yahkv_decode_workspace_init
                                once on a new workspace, and again when n_seqs, max_seq_len or the options change */
   int32_t wg_partials;      /* what a workgroup leaves of the last (sequence, kv head) pair it worked on: 1: one partial,
-                               merged from its waves' in LDS; 2: one per wave; 0: chosen from the batch's size (one per
-                               workgroup when the whole batch is at most four 64-key tiles per wave) */
+                               merged from its waves' in LDS; 2: one per wave; 3: one per workgroup, from waves that ask
+                               for a whole tile at once instead of half a tile ahead of the arithmetic (q8_0, head_dim
+                               256, 64-token pages and at most two tiles per wave with a workgroup on every CU; else as
+                               1): with about one tile per wave there is nothing to run ahead of, and the step of one
+                               32K sequence is 5 us shorter; 0: chosen from the batch's size (3 where it applies, else 1
+                               when the whole batch is at most four 64-key tiles per wave, else 2) */
   int32_t cut;              /* how the work is cut among the waves: 1: by (sequence, kv head), each wave a stretch of one
                                head's tiles; 2: by (sequence, tile), the kv heads of a tile dealt to neighbouring waves
                                (kv head counts that divide 8; not with one_launch or one partial per workgroup: those

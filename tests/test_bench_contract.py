@@ -77,4 +77,4 @@ def test_clock_trace_and_step_options():
     assert len(ct["kernel_ms"]) == len(ct["shader_mhz"]) == 60
     assert all(300 < m < 3500 for m in ct["shader_mhz"]) and 300 < ct["under_load"]["shader_mhz_median"] < 3500
     assert d["graph_replay"]["ms_per_step"] > 0 and "append, part, reduce" in d["config"]["step"]
-    assert d["roofline"]["kernel"] == "DattnPart<8, 256, 64, 2>"   # a batch of one: one partial per workgroup
+    assert d["roofline"]["kernel"] == "DattnPartWhole"   # a batch of one: whole tiles, one partial per workgroup

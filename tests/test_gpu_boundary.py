@@ -146,3 +146,35 @@ def test_cut_by_tile_and_by_head_agree(yahkv, torch_gpu, fmt, n_q, n_kv):
         outs[cut] = a
     assert np.array_equal(outs[0].view(np.uint32), outs[2 if 8 % n_kv == 0 else 1].view(np.uint32))
     assert rel_err(outs[1], outs[2]) < 5e-4
+
+
+@pytest.mark.parametrize("lens", [
+    [32769],                                   # one long sequence: 513 tiles per kv head, chunks of nine tiles (a wave takes two)
+    [32000],                                   # ... of eight: one tile per wave
+    [1], [63], [65],
+    [1, 0, 63, 64, 65, 700, 129, 0, 31],       # pairs that end inside a chunk: most waves' shares go to memory one by one
+    [3000, 5, 2000, 0, 1, 4100, 64],
+    [9000, 8000, 7000, 6000],                  # the largest batches the whole-tile instance takes (two tiles per wave)
+])
+def test_small_batches_whole_tiles(yahkv, torch_gpu, lens):
+    """A batch small enough for about a tile per wave (q8_0, head_dim 256, 64-token pages) goes to the instance of the
+    part kernel that asks for a wave's whole tile at once (opt.wg_partials = 0 picks it by the batch's size, 3 asks for
+    it). It gives the oracle's result, the same bits on a second call, and agrees with the rotating instances
+    (wg_partials = 1: one partial per workgroup, 2: one per wave) to rounding; with a gate."""
+    torch = torch_gpu
+    g, table, host, dev, rng = setup(yahkv, torch, 8, 24, 4, 256, 64, lens, seed=len(lens) + lens[0], fill=0x3C)
+    q = to_bf16_f32(rng.standard_normal((len(lens), 24, 256)))
+    gate = rng.standard_normal(q.shape).astype(np.float32)
+    want = oracle.decode_attend(host, table, lens, q, 0.0625, gate)
+    outs = {}
+    for mode in (0, 3, 1, 2):
+        opt = yahkv.decode_options(wg_partials=mode)
+        a = gpu_attend(yahkv, torch, dev, table, lens, q, 0.0625, opt=opt, gate=gate)
+        b = gpu_attend(yahkv, torch, dev, table, lens, q, 0.0625, opt=opt, gate=gate)
+        assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), mode
+        assert rel_err(a, want) < TOL, mode
+        for s, n in enumerate(lens):
+            assert n > 0 or not a[s].any()
+        outs[mode] = a
+    assert np.array_equal(outs[0].view(np.uint32), outs[3].view(np.uint32))
+    assert rel_err(outs[3], outs[1]) < 5e-4 and rel_err(outs[3], outs[2]) < 5e-4

@@ -802,6 +802,293 @@ void DattnPart(const DecodeArgs a) {
   }
 }
 
+// The part kernel for a batch of about one tile per wave (one long sequence, a few short ones): q8_0, head_dim 256,
+// 64-token pages, so a tile is one page. The cut of the line, the partials and what the separate merge expects are
+// DattnPart's in its MODE 2 (one partial per workgroup for the chunk's last pair); what differs is how a wave goes
+// through a tile. With a single tile there is nothing for the rotation above to run ahead of, and its four requests,
+// half a tile of K or V each, are four trips to memory one behind the other. Here a wave asks for both halves of its
+// tile's K at once, next to its query rows (which it only looks at once those requests are out), and for V into the
+// registers the K codes leave. Its result for the pair goes to the wave's LDS slot (V does not pass through LDS
+// here), where a second tile of the same pair joins it and where the workgroup's merge finds it, so nothing but the
+// tile in hand occupies registers. Wave w takes tiles w, w + 8, ... of the chunk: the same sums in the same order on
+// every run.
+__global__ __launch_bounds__(64 * kWavesPerGroup) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void DattnPartWhole(const DecodeArgs a) {
+  constexpr int D = 256, PT = kTile, NB = D / 32, NT = D / 16, NVB = NT / 2, QE = NB * 32 / 64;
+  constexpr int NTH = 64 * kWavesPerGroup;
+  constexpr float kLog2e = 1.4426950408889634f, kLn2 = 0.6931471805599453f;
+  const Geom g = a.g;
+  const int G = g.group(), H = g.n_kv;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64), lane = threadIdx.x % 64;
+  const int n32 = lane % 32, half = lane / 32;  // score layout: lane = key (mod 32), registers = heads 4 * half + r
+  const int n16 = lane % 16, kg = lane / 16;    // P.V layout: lane = dim (mod 16), 16 keys per lane group
+  // (query operands, their constants' sums, weights and V scales: the layouts of DattnPart<8, 256, 64, .>)
+  __shared__ __align__(16) _Float16 lq_all[kWavesPerGroup][NB][2][2][8][8];
+  __shared__ __align__(16) float lcorr_all[kWavesPerGroup][NB][8];
+  __shared__ __align__(16) _Float16 lp_all[kWavesPerGroup][kMaxGroup][kTile];
+  __shared__ __align__(16) _Float16 lvs_all[kWavesPerGroup][NB][kTile];
+  __shared__ __align__(16) float share_all[kWavesPerGroup][kMaxGroup][D];  // a wave's sums for its current pair
+  __shared__ float share_m[kWavesPerGroup][kMaxGroup], share_l[kWavesPerGroup][kMaxGroup];  // their maxima (log2) and weights
+  __shared__ int4 chunk_rec;
+  __shared__ long long chunk_tiles[4];
+  __shared__ int wave_sum[kWavesPerGroup][2];
+  auto& lq = lq_all[wave];
+  auto& lcorr = lcorr_all[wave];
+  auto& lp = lp_all[wave];
+  auto& lvs = lvs_all[wave];
+  float* const share = &share_all[wave][0][0];
+
+  if (a.stamps != nullptr && threadIdx.x == 0) a.stamps[blockIdx.x] = wall_clock64();
+  bool any_empty = false;
+  const int4 rec_v = a.n_seqs <= 64 ? ChunkRecordWave(a, blockIdx.x, wave, lane, &chunk_rec, chunk_tiles, &any_empty)
+                                    : ChunkRecord<NTH>(a, blockIdx.x, wave_sum, &chunk_rec, chunk_tiles, &any_empty);
+  const int4 rec = {__builtin_amdgcn_readfirstlane(rec_v.x), __builtin_amdgcn_readfirstlane(rec_v.y),
+                    __builtin_amdgcn_readfirstlane(rec_v.z), __builtin_amdgcn_readfirstlane(rec_v.w)};
+  if (rec.x < 0) return;
+  const int chunk_n = rec.w;
+
+  uint32_t kb[2][NB][4];  // [half of the tile][block]: 16 codes of this lane's key
+  uint4 ksc[2];           // that key's NB block scales (f16)
+  uint4 vb[2][NVB];       // [half of the dims]: 16 keys of this lane's dim
+  uint4 vsr;              // staging of the tile's V scales: 8 keys of one block per lane
+  float m[4], lsum[4], sc[2][4];
+  f4v o[NT];
+  const float qk_scale = a.scale * kLog2e;  // softmax in base 2
+  const int prow = n16 < 4 ? n16 : (n16 >= 8 && n16 < 12 ? n16 - 4 : 0);  // P rows as A-matrix rows, see DattnPart
+
+  PairCursor cur = FirstPair(a, rec);
+  typedef const int32_t __attribute__((address_space(4))) * ConstRow;  // (scalar loads, see DattnPart)
+  auto load_page = [&](int tile) -> int {
+    const ConstRow crow = (ConstRow)(reinterpret_cast<uintptr_t>(a.table + int64_t(cur.s) * a.stride));
+    return ClampPage(crow[min(tile, a.stride - 1)], g.n_pages);
+  };
+  auto load_k = [&](int tt, size_t ph) {
+    const uint8_t* kp = a.pools.kq + ph * (NB * PT * 32);
+    const uint32_t off = (32 * tt + n32) * 32 + 16 * half;
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      const uint4 v = StreamLoad(reinterpret_cast<const uint4*>(kp + (b * PT * 32 + off)));
+      kb[tt][b][0] = v.x, kb[tt][b][1] = v.y, kb[tt][b][2] = v.z, kb[tt][b][3] = v.w;
+    }
+    ksc[tt] = StreamLoad(reinterpret_cast<const uint4*>(reinterpret_cast<const uint8_t*>(a.pools.ks) + ph * (PT * NB * 2) +
+                                                        (32 * tt + n32) * (NB * 2)));
+  };
+  auto load_v = [&](int hf, size_t ph) {
+    const uint8_t* vp = a.pools.vq + ph * (D * PT);
+    const uint32_t off = n16 * PT + 16 * kg;
+#pragma unroll
+    for (int j = 0; j < NVB; ++j) vb[hf][j] = StreamLoad(reinterpret_cast<const uint4*>(vp + (16 * (hf * NVB + j) * PT + off)));
+  };
+  auto load_vs = [&](size_t ph) {  // lane = (block, 8 keys)
+    const int b = lane / 8, chunk = lane % 8;
+    vsr = StreamLoad(reinterpret_cast<const uint4*>(reinterpret_cast<const uint8_t*>(a.pools.vs) + ph * (NB * PT * 2) +
+                                                    (b * PT + 8 * chunk) * 2));
+  };
+  // scores of the 32 keys of half tt against all heads: two blocks (two accumulator chains) at a time
+  auto scores = [&](int tt) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) sc[tt][r] = 0.0f;
+#pragma unroll
+    for (int b = 0; b < NB; b += 2) {
+      const h8v qa0 = *reinterpret_cast<const h8v*>(&lq[b][0][half][n32 % 8][0]);
+      const h8v qa1 = *reinterpret_cast<const h8v*>(&lq[b][1][half][n32 % 8][0]);
+      const h8v qb0 = *reinterpret_cast<const h8v*>(&lq[b + 1][0][half][n32 % 8][0]);
+      const h8v qb1 = *reinterpret_cast<const h8v*>(&lq[b + 1][1][half][n32 % 8][0]);
+      const float4 k0 = *reinterpret_cast<const float4*>(&lcorr[b][4 * half]);
+      const float4 k1 = *reinterpret_cast<const float4*>(&lcorr[b + 1][4 * half]);
+      const float kc0[4] = {k0.x, k0.y, k0.z, k0.w}, kc1[4] = {k1.x, k1.y, k1.z, k1.w};
+      f16v c0 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}, c1 = c0;
+      c0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(qa0, RawCodes8(kb[tt][b][0], kb[tt][b][1]), c0, 0, 0, 0);
+      c1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(qb0, RawCodes8(kb[tt][b + 1][0], kb[tt][b + 1][1]), c1, 0, 0, 0);
+      c0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(qa1, RawCodes8(kb[tt][b][2], kb[tt][b][3]), c0, 0, 0, 0);
+      c1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(qb1, RawCodes8(kb[tt][b + 1][2], kb[tt][b + 1][3]), c1, 0, 0, 0);
+      const uint32_t w = b < 2 ? ksc[tt].x : b < 4 ? ksc[tt].y : b < 6 ? ksc[tt].z : ksc[tt].w;  // scales of blocks b, b + 1
+      const float d0 = WidenF16(static_cast<uint16_t>(w & 0xFFFF)) * qk_scale;
+      const float d1 = WidenF16(static_cast<uint16_t>(w >> 16)) * qk_scale;
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        sc[tt][r] = __builtin_fmaf(c1[r] - kc1[r], d1, __builtin_fmaf(c0[r] - kc0[r], d0, sc[tt][r]));
+      // (the accumulators die before the next pair of blocks starts, see DattnPart)
+      asm volatile("" : "+v"(sc[tt][0]), "+v"(sc[tt][1]), "+v"(sc[tt][2]), "+v"(sc[tt][3]));
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  // P.V for one half of the dims, from vb, lp and lvs
+  auto pv = [&](int hf) {
+    const h8v pa0 = *reinterpret_cast<const h8v*>(&lp[prow][16 * kg]);
+    const h8v pa1 = *reinterpret_cast<const h8v*>(&lp[prow][16 * kg + 8]);
+#pragma unroll
+    for (int bb = 0; bb < NB / 2; ++bb) {
+      const int b = hf * (NB / 2) + bb;
+      const h8v s0 = *reinterpret_cast<const h8v*>(&lvs[b][16 * kg]);
+      const h8v s1 = *reinterpret_cast<const h8v*>(&lvs[b][16 * kg + 8]);
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {  // output tile 2 b + j: dims 32 b + 16 j + 0..15
+        const uint4 w = vb[hf][2 * bb + j];
+        const int nt = 2 * b + j;
+        o[nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa0, Codes8(w.x, w.y) * s0, o[nt], 0, 0, 0);
+        o[nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa1, Codes8(w.z, w.w) * s1, o[nt], 0, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  auto leave_empty = [&]() {  // l = 0 for a pair this wave got no tile of (the merge then skips it)
+    if (lane < G) StoreDevice2(DeviceBuffer(a.ml + PartialIndex(a, blockIdx.x, wave, cur) * G * 2), lane * 8, kNegMax, 0.0f);
+  };
+  // the wave is through with pair `cur`, which ends inside the chunk: its share goes to memory as the wave's partial
+  auto flush = [&]() {
+    const size_t part = PartialIndex(a, blockIdx.x, wave, cur) * G;
+    const auto rml = DeviceBuffer(a.ml + part * 2), racc = DeviceBuffer(a.acc + part * D);
+    if (lane < G) StoreDevice2(rml, lane * 8, share_m[wave][lane] * kLn2, share_l[wave][lane]);
+    for (int i = lane; i < G * D; i += 64) StoreDevice(racc, i * 4, share[i]);
+    __builtin_amdgcn_wave_barrier();  // (the slot is rewritten for the next pair)
+  };
+
+  bool live = false;  // the wave has a share of pair `cur` in its slot
+  for (int idx = wave;; idx += kWavesPerGroup) {
+    bool more = idx < chunk_n;
+    while (more && idx >= cur.base + cur.n) {  // (a pair left behind by a later tile is not the chunk's last)
+      if (live) flush();
+      else leave_empty();
+      live = false;
+      more = NextPair(a, chunk_n, &cur);
+    }
+    if (!more) break;
+    const int tile = cur.first + (idx - cur.base);
+    // ---- requests: the query rows (a second tile of the same pair finds them in LDS), then K and the V scales
+    RawQ8 qraw[QE];
+    if (!live) {
+#pragma unroll
+      for (int e = 0; e < QE; ++e) {
+        const int i = lane + 64 * e, b = i / 32, sub = (i / 16) % 2, hf = (i / 8) % 2, rw = i % 8;
+        qraw[e] = RawQ8{uint4{0u, 0u, 0u, 0u}, uint4{0u, 0u, 0u, 0u}};  // (zero bits are zero in every query type)
+        if (rw < G)
+          qraw[e] = LoadRawQ8(a.q, (size_t(cur.s) * g.n_q + size_t(cur.h) * G + rw) * D + b * 32 + 16 * hf + 8 * sub, a.q_dtype);
+      }
+    }
+    const size_t ph = size_t(load_page(tile)) * H + cur.h;
+    load_k(0, ph), load_k(1, ph), load_vs(ph);
+    if (!live) {
+#pragma unroll
+      for (int e = 0; e < QE; ++e) {
+        const int i = lane + 64 * e, sub = (i / 16) % 2;
+        const h8v qv = ConvertQ8(qraw[e], a.q_dtype);
+        // what the codes' constants add to the block's product for head i % 8: the four entries of a (block, head)
+        // lie in lanes 8 apart
+        float t = 0.0f;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) t += static_cast<float>(qv[k]);
+        t *= 1152.0f;
+        t += __shfl_xor(t, 8, 64);
+        t += __shfl_xor(t, 16, 64);
+        if (lane % 32 < 8) lcorr[i / 32][i % 8] = t;
+        *reinterpret_cast<h8v*>(&lq[i / 32][sub][(i / 8) % 2][i % 8][0]) = qv;
+      }
+    }
+    // ---- scores; V is asked for into the registers the K codes leave
+    scores(0);
+    load_v(0, ph);
+    scores(1);
+    load_v(1, ph);
+    // ---- softmax (base 2) of the tile by itself; keys at or past len are masked by select
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt) {
+      const bool valid = tile * kTile + 32 * tt + n32 < cur.len;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) sc[tt][r] = valid ? sc[tt][r] : kNegMax;
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      m[r] = HalfMax32(fmaxf(sc[0][r], sc[1][r]));
+      const float p0 = __builtin_amdgcn_exp2f(sc[0][r] - m[r]), p1 = __builtin_amdgcn_exp2f(sc[1][r] - m[r]);
+      lsum[r] = HalfSum32(p0 + p1);
+      lp[4 * half + r][n32] = static_cast<_Float16>(p0);
+      lp[4 * half + r][32 + n32] = static_cast<_Float16>(p1);
+    }
+    {  // V scales of the tile to LDS; scales of keys at or past len become 0, which makes their V rows 0
+      const int b = lane / 8, chunk = lane % 8;
+      uint32_t w[4] = {vsr.x, vsr.y, vsr.z, vsr.w};
+      const int k0 = tile * kTile + 8 * chunk;
+      if (k0 + 8 > cur.len) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          if (k0 + j >= cur.len) w[j / 2] &= j % 2 ? 0x0000FFFFu : 0xFFFF0000u;
+      }
+      *reinterpret_cast<uint4*>(&lvs[b][8 * chunk]) = uint4{w[0], w[1], w[2], w[3]};
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) o[nt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
+    pv(0), pv(1);
+    // ---- the tile's result joins the wave's share of the pair
+    float fo[4], fn[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      fo[r] = 0.0f, fn[r] = 1.0f;
+      if (live) {
+        const float mo = share_m[wave][4 * half + r], mn = fmaxf(mo, m[r]);
+        fo[r] = __builtin_amdgcn_exp2f(mo - mn), fn[r] = __builtin_amdgcn_exp2f(m[r] - mn);
+        lsum[r] = __builtin_fmaf(share_l[wave][4 * half + r], fo[r], lsum[r] * fn[r]);
+        m[r] = mn;
+      }
+    }
+    __builtin_amdgcn_wave_barrier();  // (every lane has read the share's maxima and weights)
+    if (n32 == 0) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) share_m[wave][4 * half + r] = m[r], share_l[wave][4 * half + r] = lsum[r];
+    }
+    if (kg == 0 || kg == 2) {  // (these lanes' output rows are heads 2 kg + r)
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+          float* const at = &share[(2 * kg + r) * D + 16 * nt + n16];
+          *at = live ? __builtin_fmaf(*at, fo[r], o[nt][r] * fn[r]) : o[nt][r];
+        }
+    }
+    live = true;
+    __builtin_amdgcn_wave_barrier();  // lq, lp and lvs are rewritten for the next tile
+  }
+  // the pair of the wave's last tile and the pairs after it; the share of the chunk's last pair stays in the slot
+  bool held = false;
+  do {
+    if (cur.base + cur.n >= chunk_n) held = live;
+    else if (live) flush();
+    else leave_empty();
+    live = false;
+  } while (NextPair(a, chunk_n, &cur));
+  if (a.stamps != nullptr && lane == 0) atomicMax(&a.stamps[a.n_chunks + blockIdx.x], wall_clock64());
+
+  // ---- the chunk's last pair (every wave's cursor has come to rest on it): one barrier and one sweep over the row
+  // leave the workgroup's partial of it, slot 0 of its eight; the other seven stay empty
+  if (!held && n32 == 0) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) share_m[wave][4 * half + r] = kNegMax;
+  }
+  __syncthreads();
+  const size_t part = (size_t(blockIdx.x) + size_t(cur.s) * H + cur.h) * a.wpc * G;
+  const auto rml = DeviceBuffer(a.ml + part * 2), racc = DeviceBuffer(a.acc + part * D);
+  for (int i = threadIdx.x; i < G * D; i += NTH) {
+    const int gi = i / D, d = i % D;
+    float M = kNegMax;
+#pragma unroll
+    for (int w = 0; w < kWavesPerGroup; ++w) M = fmaxf(M, share_m[w][gi]);
+    float v = 0.0f, l = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kWavesPerGroup; ++w) {
+      const float mw = share_m[w][gi];
+      if (mw > kNegMax) {  // (the slot of a wave without a share holds anything)
+        const float f = __builtin_amdgcn_exp2f(mw - M);
+        v = __builtin_fmaf(share_all[w][gi][d], f, v), l = __builtin_fmaf(share_l[w][gi], f, l);
+      }
+    }
+    StoreDevice(racc, i * 4, v);
+    if (d < a.wpc) StoreDevice2(rml, (d * G + gi) * 8, M * kLn2, d == 0 ? l : 0.0f);
+  }
+}
+
 // ---- reduce -------------------------------------------------------------------------------------------------------------
 
 // One workgroup per (query head, sequence) (gen_decode_attn.py:338-411). The pair's partials are those of the waves
@@ -981,6 +1268,10 @@ __global__ __launch_bounds__(kReduceThreads) void DattnReduce(const DecodeArgs a
 int LaunchPart(const DecodeArgs& a, hipStream_t st) {
   const Geom& m = a.g;
   const dim3 grid(static_cast<unsigned>(a.n_chunks));
+  if (a.whole_tiles) {  // (Prepare sets it for q8_0, head_dim 256, 64-token pages and a small batch only)
+    hipLaunchKernelGGL(DattnPartWhole, grid, dim3(64 * kWavesPerGroup), 0, st, a);
+    return LaunchStatus();
+  }
 #define YAHKV_LAUNCH_PART(FF, DD, PP)                                                                          \
   do {                                                                                                         \
     if (a.fused) hipLaunchKernelGGL((DattnPart<FF, DD, PP, 1>), grid, dim3(64 * kWavesPerGroup), 0, st, a);           \

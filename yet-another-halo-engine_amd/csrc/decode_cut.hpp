@@ -44,6 +44,7 @@ struct DecodeArgs {
   // one launch for part and merge: the workgroup that is last to finish a pair's tiles merges the pair's partials
   int32_t fused;                // (read by the host, which launches the kernel's one-launch instance)
   int32_t wg_partials;          // (host) the instance that leaves one partial per workgroup for a chunk's last pair
+  int32_t whole_tiles;          // (host) ... and asks for a wave's whole tile at once (chunks of about a tile per wave)
   unsigned long long* tickets;  // [n_seqs * H] workgroups that have arrived at a pair's merge; zero between launches
   // The step form (append + attention in two launches): seq_len counts the step's own token, which is not in the
   // pools yet. The part kernel then covers the len_bias = -1 shorter sequences already there, and the reduce
@@ -320,17 +321,30 @@ typedef float f16v __attribute__((ext_vector_type(16)));
 __device__ __forceinline__ _Float16 SaturateToF16(float x) {
   return static_cast<_Float16>(__builtin_fminf(__builtin_fmaxf(x, -65504.0f), 65504.0f) + (x - x));  // x - x: 0, or NaN
 }
-__device__ __forceinline__ h8v LoadQ8(const void* q, size_t i, int dt) {
+// Eight query elements in two steps, so that a kernel can ask for them, ask for other things, and only then wait: the
+// bytes as they lie in memory (f32: 32 of them, f16 / bf16: 16), and their f16 values.
+struct RawQ8 {
+  uint4 a, b;
+};
+__device__ __forceinline__ RawQ8 LoadRawQ8(const void* q, size_t i, int dt) {
+  RawQ8 r;
+  if (dt == YAHKV_F32) {
+    r.a = *reinterpret_cast<const uint4*>(static_cast<const float*>(q) + i);
+    r.b = *reinterpret_cast<const uint4*>(static_cast<const float*>(q) + i + 4);
+  } else {
+    r.a = *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(q) + i);
+    r.b = uint4{0u, 0u, 0u, 0u};
+  }
+  return r;
+}
+__device__ __forceinline__ h8v ConvertQ8(const RawQ8& raw, int dt) {
   h8v r;
   if (dt == YAHKV_F32) {
-    const float4 a = *reinterpret_cast<const float4*>(static_cast<const float*>(q) + i);
-    const float4 b = *reinterpret_cast<const float4*>(static_cast<const float*>(q) + i + 4);
-    const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+    const uint32_t v[8] = {raw.a.x, raw.a.y, raw.a.z, raw.a.w, raw.b.x, raw.b.y, raw.b.z, raw.b.w};
 #pragma unroll
-    for (int j = 0; j < 8; ++j) r[j] = SaturateToF16(v[j]);
+    for (int j = 0; j < 8; ++j) r[j] = SaturateToF16(__builtin_bit_cast(float, v[j]));
   } else {
-    const uint4 a = *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(q) + i);
-    const uint32_t w[4] = {a.x, a.y, a.z, a.w};
+    const uint32_t w[4] = {raw.a.x, raw.a.y, raw.a.z, raw.a.w};
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const uint16_t hbits = static_cast<uint16_t>(w[j / 2] >> (16 * (j % 2)));
@@ -339,6 +353,7 @@ __device__ __forceinline__ h8v LoadQ8(const void* q, size_t i, int dt) {
   }
   return r;
 }
+__device__ __forceinline__ h8v LoadQ8(const void* q, size_t i, int dt) { return ConvertQ8(LoadRawQ8(q, i, dt), dt); }
 
 // Partials travel between workgroups on different XCDs, whose L2 caches do not see each other's lines: they are
 // written through to memory and read past the L2 (cache policy sc1, device scope) by these buffer accesses. Fences of
@@ -399,6 +414,7 @@ inline int ComputeUnits() {
 // Tuning values of a call: the caller's options where given, else the defaults.
 struct Tuning {
   int32_t n_chunks, min_chunk_tiles, pair_cost, reduce_split, deterministic, one_launch, wg_partials, cut;
+  bool min_chunk_given, pair_cost_given;
   int32_t xcd_weight[8];
 };
 inline Tuning MakeTuning(const yahkv_decode_options* o) {
@@ -409,6 +425,8 @@ inline Tuning MakeTuning(const yahkv_decode_options* o) {
   // counts on every chunk inside a pair's stretch of the line having left partials
   t.min_chunk_tiles = o != nullptr && o->min_chunk_tiles > 0 ? std::min(std::max(o->min_chunk_tiles, 2), 1 << 20)
                                                              : 2 * kWavesPerGroup;
+  t.min_chunk_given = o != nullptr && o->min_chunk_tiles > 0;
+  t.pair_cost_given = o != nullptr && o->pair_cost != 0;
   t.pair_cost = o == nullptr || o->pair_cost == 0 ? 8 : std::min(std::max(o->pair_cost, 0), 1 << 10);
   t.reduce_split = o != nullptr ? std::max(o->reduce_split, 0) : 0;
   t.deterministic = o == nullptr || o->deterministic >= 0;  // (negative: tiles first come, first served)
@@ -424,6 +442,12 @@ inline bool CutByTile(const Geom& g, const Tuning& t) {
   if (g.n_kv <= 1 || kWavesPerGroup % g.n_kv != 0) return false;
   return g.format > 16 || (t.cut != 1 && !t.one_launch && t.wg_partials != 1);
 }
+// Whether a batch is small enough for whole-tile requests (DattnPart's MODE 3: q8_0, head_dim 256, a tile = a page): at
+// most two tiles per wave when every CU has a workgroup. Such a batch is cut into chunks of one tile per wave.
+inline bool WholeTiles(const Geom& g, const Tuning& t, int64_t line_max) {
+  return g.format == 8 && g.hd == 256 && g.pt == kTile && !t.one_launch && (t.wg_partials == 0 || t.wg_partials == 3) &&
+         line_max <= int64_t(t.n_chunks) * kWavesPerGroup * 2;
+}
 inline Plan MakePlan(const Geom& g, int32_t n_seqs, int32_t max_seq_len, const Tuning& t) {
   Plan p;
   p.max_len = std::max(max_seq_len, 1);
@@ -431,6 +455,10 @@ inline Plan MakePlan(const Geom& g, int32_t n_seqs, int32_t max_seq_len, const T
   const int64_t line_max = max_tiles * n_seqs * g.n_kv;
   p.wpc = kWavesPerGroup;
   p.min_chunk_tiles = t.min_chunk_tiles, p.pair_cost = t.pair_cost;
+  if (WholeTiles(g, t, line_max)) {  // one tile per wave wherever the line allows it: a pair costs nothing besides
+    if (!t.min_chunk_given) p.min_chunk_tiles = kWavesPerGroup;
+    if (!t.pair_cost_given) p.pair_cost = 0;
+  }
   p.n_chunks =
       static_cast<int32_t>(std::min<int64_t>(t.n_chunks, (line_max + p.min_chunk_tiles - 1) / p.min_chunk_tiles));
   // Shares of the eight chunks of a group: proportional to the caller's relative XCD speeds (yahkv_decode_calibrate
@@ -494,7 +522,8 @@ inline int Prepare(const Geom& m, int32_t page_table_stride, const int32_t* seq_
   a->deterministic = t.deterministic;
   // One partial per workgroup for a chunk's last pair pays where chunks are short (a small batch: few tiles per wave, so
   // a wave's partial is a large part of what it moves) and costs two barriers at the kernel's end where they are long.
-  a->wg_partials = t.wg_partials == 1 ? 1 : t.wg_partials == 2 ? 0 : (int64_t(p.max_len) + kTile - 1) / kTile * n_seqs * m.n_kv <= int64_t(p.n_chunks) * kWavesPerGroup * 4;
+  a->wg_partials = t.wg_partials == 1 || t.wg_partials == 3 ? 1 : t.wg_partials == 2 ? 0 : (int64_t(p.max_len) + kTile - 1) / kTile * n_seqs * m.n_kv <= int64_t(p.n_chunks) * kWavesPerGroup * 4;
+  a->whole_tiles = a->wg_partials && WholeTiles(m, t, (int64_t(p.max_len) + kTile - 1) / kTile * n_seqs * m.n_kv);
   if (m.format <= 16 && CutByTile(m, t) && !a->wg_partials) a->tile_mult = m.n_kv;
   std::copy(p.share, p.share + 9, a->share);
   return YAHKV_OK;
