@@ -1153,10 +1153,12 @@ __device__ __forceinline__ void StepToken(const DecodeArgs& a, const StepRows& r
   if (lane == 0) *score = dot * a.scale;
 }
 
-constexpr int kReduceThreads = 256;  // also the number of partial slots weighed at a time
+constexpr int kReduceThreads = 256;  // also the number of partial slots weighed at a time (RT below)
+constexpr int kReduceThreadsWide = 512;  // ... where a pair has more than that many places for partials
 constexpr int kReduceDepth = 4;      // partials a group loads together
 constexpr int kReduceMinDims = 32;   // fewest dims of a head one workgroup sums
-__global__ __launch_bounds__(kReduceThreads) void DattnReduce(const DecodeArgs a, const StepRows rows) {
+template <int RT>
+__global__ __launch_bounds__(RT) void DattnReduce(const DecodeArgs a, const StepRows rows) {
   const Geom g = a.g;
   const int G = g.group(), H = g.n_kv, D = g.hd;
   const int hq = blockIdx.x, s = blockIdx.y, t = threadIdx.x;
@@ -1170,11 +1172,6 @@ __global__ __launch_bounds__(kReduceThreads) void DattnReduce(const DecodeArgs a
   const bool has_new = stores_new && StepSeesNewToken(a, a.seq_len[s]);
   __shared__ float new_score;
   __shared__ __align__(16) float new_v[256];
-  if (stores_new && t < 128) StepToken(a, rows, s, h, hq, t / 64, t % 64, gi == 0 && blockIdx.z == 0, &new_score, new_v);
-  if (ts <= 0 && !has_new) {  // nothing to attend to
-    for (int d = t; d < DZ; d += kReduceThreads) a.out[o + d] = 0.0f;
-    return;
-  }
   // line units of the sequences before this one and of the whole line; the pair's tiles follow its first units
   size_t p0 = 0, p1 = 0;  // (a sequence that has nothing but its new token has no partials)
   if (ts > 0) {
@@ -1191,16 +1188,25 @@ __global__ __launch_bounds__(kReduceThreads) void DattnReduce(const DecodeArgs a
       p0 = (row + k0) * a.wpc, p1 = (row + k1 + 1) * a.wpc;
     }
   }
-  constexpr int NW = kReduceThreads / 64;
-  __shared__ float wgt[kReduceThreads], wl[kReduceThreads];
-  __shared__ int slot[kReduceThreads];
+  // The first RT places' (maximum, sum) entries are asked for before the new token's rows are worked on, so the two
+  // waits overlap, and stay in registers for the sweep below (a small batch has no more places than that).
+  float2 first_ml = {kNegMax, 0.0f};
+  if (p0 + t < p1) first_ml = *reinterpret_cast<const float2*>(&a.ml[((p0 + t) * G + gi) * 2]);
+  if (stores_new && t < 128) StepToken(a, rows, s, h, hq, t / 64, t % 64, gi == 0 && blockIdx.z == 0, &new_score, new_v);
+  if (ts <= 0 && !has_new) {  // nothing to attend to
+    for (int d = t; d < DZ; d += RT) a.out[o + d] = 0.0f;
+    return;
+  }
+  constexpr int NW = RT / 64;
+  __shared__ float wgt[RT], wl[RT];
+  __shared__ int slot[RT];
   __shared__ float red[NW];
   __shared__ int wave_n[NW];
-  __shared__ __align__(16) float sums[kReduceThreads * 4];  // [group][DZ]
-  __shared__ float lsums[kReduceThreads / (kReduceMinDims / 4)];
+  __shared__ __align__(16) float sums[RT * 4];  // [group][DZ]
+  __shared__ float lsums[RT / (kReduceMinDims / 4)];
   // waves that got no tile of this pair left l = 0 (and no acc): they weigh nothing
-  float M = kNegMax;
-  for (size_t p = p0 + t; p < p1; p += kReduceThreads)
+  float M = first_ml.y > 0.0f ? first_ml.x : kNegMax;
+  for (size_t p = p0 + t + RT; p < p1; p += RT)
     if (a.ml[(p * G + gi) * 2 + 1] > 0.0f) M = fmaxf(M, a.ml[(p * G + gi) * 2]);
   M = WaveMax(M);
   if (t % 64 == 0) red[t / 64] = M;
@@ -1209,13 +1215,14 @@ __global__ __launch_bounds__(kReduceThreads) void DattnReduce(const DecodeArgs a
   for (int w = 1; w < NW; ++w) M = fmaxf(M, red[w]);
   if (has_new) M = fmaxf(M, new_score);
   const int lg_lanes = __builtin_ctz(static_cast<unsigned>(DZ)) - 2;  // four dims a lane
-  const int lanes = 1 << lg_lanes, n_groups = kReduceThreads >> lg_lanes, grp = t >> lg_lanes, dl = t & (lanes - 1);
+  const int lanes = 1 << lg_lanes, n_groups = RT >> lg_lanes, grp = t >> lg_lanes, dl = t & (lanes - 1);
   float L = 0.0f;
   float4 A = {0.0f, 0.0f, 0.0f, 0.0f};
-  for (size_t b0 = p0; b0 < p1; b0 += kReduceThreads) {
-    const int nb = static_cast<int>(min(p1 - b0, size_t(kReduceThreads)));
+  for (size_t b0 = p0; b0 < p1; b0 += RT) {
+    const int nb = static_cast<int>(min(p1 - b0, size_t(RT)));
     float l = 0.0f, m = 0.0f;
-    if (t < nb) l = a.ml[((b0 + t) * G + gi) * 2 + 1], m = a.ml[((b0 + t) * G + gi) * 2];
+    if (b0 == p0) l = first_ml.y, m = first_ml.x;
+    else if (t < nb) l = a.ml[((b0 + t) * G + gi) * 2 + 1], m = a.ml[((b0 + t) * G + gi) * 2];
     const unsigned long long mask = __ballot(l > 0.0f);
     __syncthreads();  // the previous batch's lists have been read
     if (t % 64 == 0) wave_n[t / 64] = __popcll(mask);
@@ -1249,7 +1256,7 @@ __global__ __launch_bounds__(kReduceThreads) void DattnReduce(const DecodeArgs a
   *reinterpret_cast<float4*>(&sums[grp * DZ + 4 * dl]) = A;
   if (dl == 0) lsums[grp] = L;
   __syncthreads();
-  for (int d = t; d < DZ; d += kReduceThreads) {
+  for (int d = t; d < DZ; d += RT) {
     float v = 0.0f, lt = 0.0f;
     for (int q = 0; q < n_groups; ++q) v += sums[q * DZ + d], lt += lsums[q];
     if (has_new) {
@@ -1302,7 +1309,13 @@ int LaunchReduce(const DecodeArgs& a, const StepRows& rows, const yahkv_decode_o
   const int asked = MakeTuning(opt).reduce_split;
   if (asked > 0) split = std::min(asked, a.g.hd / kReduceMinDims);
   while (a.g.hd % split != 0 || (a.g.hd / split) % 4 != 0) --split;
-  hipLaunchKernelGGL(DattnReduce, dim3(a.g.n_q, a.n_seqs, split), dim3(kReduceThreads), 0, st, a, rows);
+  // (a small batch cut into many chunks: a pair's places for partials, eight per chunk its tiles lie in, are weighed in
+  // one sweep of a wider workgroup instead of two)
+  const int64_t places = int64_t(a.n_chunks) * a.wpc / std::max<int64_t>(int64_t(a.n_seqs) * a.g.n_kv, 1) + a.wpc;
+  if (a.wg_partials && places > kReduceThreads)
+    hipLaunchKernelGGL(DattnReduce<kReduceThreadsWide>, dim3(a.g.n_q, a.n_seqs, split), dim3(kReduceThreadsWide), 0, st, a, rows);
+  else
+    hipLaunchKernelGGL(DattnReduce<kReduceThreads>, dim3(a.g.n_q, a.n_seqs, split), dim3(kReduceThreads), 0, st, a, rows);
   return LaunchStatus();
 }
 
