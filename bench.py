@@ -9,6 +9,7 @@ measured with HIP events on the launch stream; `cpu_baseline` is the CPU oracle'
 sample of the same sequences, on this box's host cores.
 """
 import argparse
+import ctypes
 import importlib
 import json
 import os
@@ -838,17 +839,24 @@ def run_decode(a, wl, torch, yahkv):
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(a.steps)]
     separate = a.separate_append or a.one_launch
 
-    def step(i, pair=None):
+    # The step's two calls with their arguments marshalled once per step index, before anything is timed: the timed loop
+    # then pays for the C calls alone, as a C++ caller does (building ctypes arguments from tensors costs Python about as
+    # much as a small batch's whole step takes on the GPU).
+    calls = None if separate else [
+        yahkv.decode_step_calls(layers[i % len(layers)], t_table, len_rows[i], len_rows[i + 1], max_len, knew[i][:, 0],
+                                vnew[i][:, 0], q, scale, out, ws, opt=opt) for i in range(total)]
+
+    def step(i, pair=None, on=None):        # on: the handle of the stream a graph is being captured on
         seq_len = len_rows[i + 1]
         pools = layers[i % len(layers)]     # (with several layers a layer sees every n-th token; the others stay zero blocks)
         if not separate:
+            part, merge = calls[i]
             if pair:
                 pair[0].record()
-            yahkv.decode_part(pools, t_table, len_rows[i], max_len, q, scale, ws, opt=opt)   # the tokens before the step
+            part(on) if on else part()      # the tokens before the step
             if pair:
                 pair[1].record()
-            yahkv.decode_step_reduce(pools, t_table, seq_len, max_len, knew[i][:, 0], vnew[i][:, 0], q, scale, out, ws,
-                                     opt=opt)
+            merge(on) if on else merge()    # the step's own token, the partials' merge
             return
         yahkv.append(pools, t_table, len_rows[i], knew[i], vnew[i])    # position = current length (device-resident)
         if pair:
@@ -882,6 +890,7 @@ def run_decode(a, wl, torch, yahkv):
         # (the kernel's own duration is taken on every fourth timed step: a pair of event records costs the stream a few
         # microseconds, which the other steps are spared)
         step(1 + a.warmup + i, ev[i] if i % EVENT_EVERY == 0 else None)
+    t_issued = time.perf_counter()          # (what the host took to queue the steps: below the step's time, or its bound)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
 
@@ -900,6 +909,7 @@ def run_decode(a, wl, torch, yahkv):
                    "paged q%d KV decode-attn HBM GB/s (%% of peak) + tok/s" % wl["fmt"]),
         "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "host_issue_ms_per_step": round((t_issued - t0) / a.steps * 1e3, 4),
         "dtype": "u8" if wl["fmt"] == 8 else "u4", "data": "synthetic",
         "config": {"workload": a.workload, "batch": B, "ctx_min": int(lens.min()), "ctx_max": int(lens.max()),
                    "ctx_sum": int(lens.sum()), "n_q_heads": NQ, "n_kv_heads": NKV, "head_dim": HD, "page_tokens": PT,
@@ -939,8 +949,9 @@ def run_decode(a, wl, torch, yahkv):
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.stream(side):
             with torch.cuda.graph(graph, stream=side):
+                on = ctypes.c_void_p(side.cuda_stream)
                 for i in range(a.steps):
-                    step(1 + a.warmup + i)
+                    step(1 + a.warmup + i, on=on)
         torch.cuda.synchronize()
         graph.replay()
         torch.cuda.synchronize()

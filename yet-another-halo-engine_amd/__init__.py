@@ -481,6 +481,37 @@ def decode_part(pools, table, seq_len, max_seq_len, q, scale, workspace, opt=Non
                                  _op(opt), _stream()), "decode_part")
 
 
+def decode_step_calls(pools, table, seq_len_before, seq_len, max_seq_len, k_new, v_new, q, scale, out, workspace,
+                      gate=None, opt=None):
+    """The two calls of one decode step (decode_part on the lengths before the step, decode_step_reduce on the lengths
+    with it) with their arguments marshalled once: returns (part, reduce), two functions of no arguments. A loop that
+    issues many steps (a benchmark, a server) then pays for the two C calls alone, as a C++ caller does, and not for
+    building ctypes arguments from tensors on every step. The tensors must stay alive and in place; the stream is the
+    one current now unless a call names another."""
+    g = pools.geom
+    st = pools.struct()
+    stream = _stream()
+    common = (C.byref(g), C.byref(st), _dp(table), table.shape[1])
+    part_args = common + (_dp(seq_len_before), q.shape[0], max_seq_len, _dp(q), _dtype_code(q), scale, _dp(workspace),
+                          workspace.numel(), _op(opt))
+    reduce_args = common + (_dp(seq_len), q.shape[0], max_seq_len, _dp(k_new), _dp(v_new), _dtype_code(k_new), _dp(q),
+                            _dtype_code(q), scale, _dp(gate), _dp(out), _dp(workspace), workspace.numel(), _op(opt))
+    keep = (g, st, table, seq_len_before, seq_len, k_new, v_new, q, out, workspace, gate, opt)
+    fp, fr = lib.yahkv_decode_part, lib.yahkv_decode_step_reduce
+
+    def part(on=stream, _keep=keep):  # on: another stream's handle (a ctypes void pointer), e.g. one that is being captured
+        rc = fp(*part_args, on)
+        if rc:
+            _check(rc, "decode_part")
+
+    def reduce(on=stream, _keep=keep):
+        rc = fr(*reduce_args, on)
+        if rc:
+            _check(rc, "decode_step_reduce")
+
+    return part, reduce
+
+
 def decode_reduce(g, table_stride, seq_len, n_seqs, max_seq_len, out, workspace, gate=None, opt=None):
     """Second dispatch of decode_attend: merge the partials into out."""
     _check(lib.yahkv_decode_reduce(C.byref(g), table_stride, _dp(seq_len), n_seqs, max_seq_len, _dp(gate), _dp(out),
