@@ -155,8 +155,10 @@ int yahkv_append_rope(const yahkv_geometry* g, const yahkv_pools* pools, const i
 typedef struct yahkv_decode_options {
   int32_t n_chunks;         /* pieces the batch's keys are cut into = workgroups of the split-K kernel; 0: one per
                                compute unit (f16 pools: workgroups aimed at in all; 0: sixteen per compute unit) */
-  int32_t min_chunk_tiles;  /* fewest 64-key tiles a piece gets (each piece costs a partial); 0: 16; at least 2 */
-  int32_t pair_cost;        /* what a change of (sequence, kv head) costs a workgroup, in tiles; 0: 8; negative: none */
+  int32_t min_chunk_tiles;  /* fewest 64-key tiles a piece gets (each piece costs a partial); 0: 16 (8 where the
+                               whole-tile kernel of wg_partials runs: one tile per wave); at least 2 */
+  int32_t pair_cost;        /* what a change of (sequence, kv head) costs a workgroup, in tiles; 0: 8 (none where the
+                               whole-tile kernel runs); negative: none */
   int32_t reduce_split;     /* workgroups per (query head, sequence) of the merge; 0: chosen from the batch size */
   int32_t deterministic;    /* 0 or positive (the default): the waves of a workgroup take its tiles in a fixed pattern, so
                                two calls on the same bytes with the same options give the same bits (the two waves of a
