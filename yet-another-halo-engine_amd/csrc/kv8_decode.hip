@@ -545,6 +545,26 @@ __global__ __launch_bounds__(kReduceThreads) void Kv8Reduce(const DecodeArgs a, 
     for (int d = t; d < DZ; d += kReduceThreads) a.out[o + d] = 0.0f;
     return;
   }
+  size_t p0 = 0, p1 = 0;
+  if (ts > 0) {
+    // (with the kv heads dealt to the waves the sequence is one pair on the line, and this head's partials lie among
+    // those of all the chunks that hold a piece of the sequence)
+    const int Hc = CutHeads(a);
+    const long long A_ = ChunkUnits(a, static_cast<long long>(a.tprefix[a.n_seqs]) * Hc);
+    const int pair = s * H + h;
+    const long long first = static_cast<long long>(a.tprefix[s]) * Hc +
+                            static_cast<long long>(Hc == 1 ? 0 : h) * UnitsOf(a, ts) + a.pair_cost;
+    const int k0 = ChunkOf(a, A_, first), k1 = ChunkOf(a, A_, first + ts - 1);
+    p0 = size_t(k0 + pair) * a.wpc, p1 = size_t(k1 + pair + 1) * a.wpc;
+    if (Hc == 1 && H > 1) {
+      const size_t row = size_t(h) * (a.n_chunks + a.n_seqs) + s;
+      p0 = (row + k0) * a.wpc, p1 = (row + k1 + 1) * a.wpc;
+    }
+  }
+  // The first places' (maximum, sum) entries are asked for here, before the open tile and the step's token are worked on,
+  // so that their way from memory overlaps that work; they stay in registers for the sweep below.
+  float2 first_ml = {kNegMax, 0.0f};
+  if (p0 + t < p1) first_ml = *reinterpret_cast<const float2*>(&a.ml[((p0 + t) * G + gi) * 2]);
   if (k4) {  // the butterfly of the part kernel's prologue, over LDS (gen_decode_attn.py:655-683)
 #pragma clang fp contract(off)
     qrot[t] = static_cast<float>(SaturateToF16(LoadSrc(a.q, (size_t(s) * g.n_q + hq) * D + t, a.q_dtype)));
@@ -566,6 +586,12 @@ __global__ __launch_bounds__(kReduceThreads) void Kv8Reduce(const DecodeArgs a, 
   const int32_t* trow = a.table + int64_t(s) * a.stride;
   const int page = ClampPage(trow[min(closed / kKv8Page, a.stride - 1)], g.n_pages);
   const int page0 = ClampPage(trow[0], g.n_pages);
+  // the open tile's V values of this thread's dim (the last loop below has one pass: DZ <= 256 threads), asked for now
+  uint4 vo_lo = {0u, 0u, 0u, 0u}, vo_hi = vo_lo;
+  if (n_tail > 0 && t < DZ) {
+    const uint16_t* vo = pools.vo + kg8.vo_head(page, h) + size_t(d0 + t) * 16;
+    vo_lo = *reinterpret_cast<const uint4*>(vo), vo_hi = *reinterpret_cast<const uint4*>(vo + 8);
+  }
   // ---- scores of the open tile's keys: thread = (key t / 16, 16 dims of the head)
   {
     const int j = t / 16, c = t % 16;
@@ -692,22 +718,6 @@ __global__ __launch_bounds__(kReduceThreads) void Kv8Reduce(const DecodeArgs a, 
     }
   }
   const int n_extra = n_tail + (step ? 1 : 0);  // 1 .. 17
-  size_t p0 = 0, p1 = 0;
-  if (ts > 0) {
-    // (with the kv heads dealt to the waves the sequence is one pair on the line, and this head's partials lie among
-    // those of all the chunks that hold a piece of the sequence)
-    const int Hc = CutHeads(a);
-    const long long A_ = ChunkUnits(a, static_cast<long long>(a.tprefix[a.n_seqs]) * Hc);
-    const int pair = s * H + h;
-    const long long first = static_cast<long long>(a.tprefix[s]) * Hc +
-                            static_cast<long long>(Hc == 1 ? 0 : h) * UnitsOf(a, ts) + a.pair_cost;
-    const int k0 = ChunkOf(a, A_, first), k1 = ChunkOf(a, A_, first + ts - 1);
-    p0 = size_t(k0 + pair) * a.wpc, p1 = size_t(k1 + pair + 1) * a.wpc;
-    if (Hc == 1 && H > 1) {
-      const size_t row = size_t(h) * (a.n_chunks + a.n_seqs) + s;
-      p0 = (row + k0) * a.wpc, p1 = (row + k1 + 1) * a.wpc;
-    }
-  }
   constexpr int NW = kReduceThreads / 64;
   __shared__ float wgt[kReduceThreads], wl[kReduceThreads];
   __shared__ int slot[kReduceThreads];
@@ -715,8 +725,8 @@ __global__ __launch_bounds__(kReduceThreads) void Kv8Reduce(const DecodeArgs a, 
   __shared__ int wave_n[NW];
   __shared__ __align__(16) float sums[kReduceThreads * 4];
   __shared__ float lsums[kReduceThreads / (kReduceMinDims / 4)];
-  float M = kNegMax;
-  for (size_t p = p0 + t; p < p1; p += kReduceThreads)
+  float M = first_ml.y > 0.0f ? first_ml.x : kNegMax;
+  for (size_t p = p0 + t + kReduceThreads; p < p1; p += kReduceThreads)
     if (a.ml[(p * G + gi) * 2 + 1] > 0.0f) M = fmaxf(M, a.ml[(p * G + gi) * 2]);
   M = WaveMax(M);
   if (t % 64 == 0) red[t / 64] = M;
@@ -731,7 +741,8 @@ __global__ __launch_bounds__(kReduceThreads) void Kv8Reduce(const DecodeArgs a, 
   for (size_t b0 = p0; b0 < p1; b0 += kReduceThreads) {
     const int nb = static_cast<int>(min(p1 - b0, size_t(kReduceThreads)));
     float l = 0.0f, mm = 0.0f;
-    if (t < nb) l = a.ml[((b0 + t) * G + gi) * 2 + 1], mm = a.ml[((b0 + t) * G + gi) * 2];
+    if (b0 == p0) l = first_ml.y, mm = first_ml.x;
+    else if (t < nb) l = a.ml[((b0 + t) * G + gi) * 2 + 1], mm = a.ml[((b0 + t) * G + gi) * 2];
     const unsigned long long mask = __ballot(l > 0.0f);
     __syncthreads();
     if (t % 64 == 0) wave_n[t / 64] = __popcll(mask);
@@ -769,12 +780,7 @@ __global__ __launch_bounds__(kReduceThreads) void Kv8Reduce(const DecodeArgs a, 
     float v = 0.0f, lt = 0.0f;
     for (int q = 0; q < n_groups; ++q) v += sums[q * DZ + d], lt += lsums[q];
     // the open tile's keys, as partials of one key each: V from the open f16 tile, the step's token from its source row
-    const uint16_t* vo = pools.vo + kg8.vo_head(page, h) + size_t(d0 + d) * 16;
-    uint32_t w[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    if (n_tail > 0) {
-      const uint4 lo = *reinterpret_cast<const uint4*>(vo), hi = *reinterpret_cast<const uint4*>(vo + 8);
-      w[0] = lo.x, w[1] = lo.y, w[2] = lo.z, w[3] = lo.w, w[4] = hi.x, w[5] = hi.y, w[6] = hi.z, w[7] = hi.w;
-    }
+    const uint32_t w[8] = {vo_lo.x, vo_lo.y, vo_lo.z, vo_lo.w, vo_hi.x, vo_hi.y, vo_hi.z, vo_hi.w};  // (d == t)
     for (int j = 0; j < n_extra; ++j) {
       const float wj = __expf(tail_score[j] - M);
       const float x = j < n_tail ? WidenF16(static_cast<uint16_t>(w[j / 2] >> (16 * (j % 2)))) : new_v[d0 + d];
