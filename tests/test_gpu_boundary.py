@@ -155,6 +155,8 @@ def test_cut_by_tile_and_by_head_agree(yahkv, torch_gpu, fmt, n_q, n_kv):
     [1, 0, 63, 64, 65, 700, 129, 0, 31],       # pairs that end inside a chunk: most waves' shares go to memory one by one
     [3000, 5, 2000, 0, 1, 4100, 64],
     [9000, 8000, 7000, 6000],                  # the largest batches the whole-tile instance takes (two tiles per wave)
+    [(i * 37) % 500 + (i % 7 != 0) for i in range(100)],   # a hundred short sequences, some empty: many pairs per chunk, and
+                                                           # the cut by the whole workgroup (more than 64 sequences)
 ])
 def test_small_batches_whole_tiles(yahkv, torch_gpu, lens):
     """A batch small enough for about a tile per wave (q8_0, head_dim 256, 64-token pages) goes to the instance of the
