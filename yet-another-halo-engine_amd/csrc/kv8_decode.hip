@@ -515,8 +515,7 @@ void Kv8Part(const DecodeArgs a, const Kv8Pools pools) {
 
 // ---- the merge, with the open tile and the step's token -----------------------------------------------------------------
 
-constexpr int kReduceThreads = 256;
-constexpr int kReduceDepth = 4;
+constexpr int kReduceDepth = 4;  // (the merge's width is its template argument: 256, 512 or 1024 threads)
 constexpr int kReduceMinDims = 32;
 constexpr int kTail = 17;  // keys the merge adds itself: up to 16 of the open tile, one of them the step's new token
 
@@ -525,7 +524,8 @@ constexpr int kTail = 17;  // keys the merge adds itself: up to 16 of the open t
 // open f16 tile; in the step form the newest of them is the step's own token, which is quantized here with the append
 // kernels' functions, scored from its codes as the reference's part_q would (the K append runs first there,
 // loom_decoder.hpp:254-261), and written to the pools by the workgroup of the group's first query head.
-__global__ __launch_bounds__(kReduceThreads) void Kv8Reduce(const DecodeArgs a, const Kv8Pools pools, const StepRows rows) {
+template <int RT>
+__global__ __launch_bounds__(RT) void Kv8Reduce(const DecodeArgs a, const Kv8Pools pools, const StepRows rows) {
   const Geom g = a.g;
   const Kv8Geom kg8{g.n_q, g.n_kv, g.n_pages, Kv8BitsK(g.format), Kv8BitsV(g.format)};
   const bool k4 = kg8.kb == 4;
@@ -542,7 +542,7 @@ __global__ __launch_bounds__(kReduceThreads) void Kv8Reduce(const DecodeArgs a, 
   __shared__ __align__(16) float new_v[D];
   __shared__ __align__(16) float qrot[D];  // 4-bit K: the head's rotated query, H256 q / 16 rounded to f16
   if (len <= 0) {
-    for (int d = t; d < DZ; d += kReduceThreads) a.out[o + d] = 0.0f;
+    for (int d = t; d < DZ; d += RT) a.out[o + d] = 0.0f;
     return;
   }
   size_t p0 = 0, p1 = 0;
@@ -567,7 +567,7 @@ __global__ __launch_bounds__(kReduceThreads) void Kv8Reduce(const DecodeArgs a, 
   if (p0 + t < p1) first_ml = *reinterpret_cast<const float2*>(&a.ml[((p0 + t) * G + gi) * 2]);
   if (k4) {  // the butterfly of the part kernel's prologue, over LDS (gen_decode_attn.py:655-683)
 #pragma clang fp contract(off)
-    qrot[t] = static_cast<float>(SaturateToF16(LoadSrc(a.q, (size_t(s) * g.n_q + hq) * D + t, a.q_dtype)));
+    if (t < D) qrot[t] = static_cast<float>(SaturateToF16(LoadSrc(a.q, (size_t(s) * g.n_q + hq) * D + t, a.q_dtype)));
     __syncthreads();
     for (int st = 1; st < D; st <<= 1) {
       if (t < D / 2) {
@@ -577,7 +577,7 @@ __global__ __launch_bounds__(kReduceThreads) void Kv8Reduce(const DecodeArgs a, 
       }
       __syncthreads();
     }
-    qrot[t] = static_cast<float>(static_cast<_Float16>(qrot[t] * 0.0625f));
+    if (t < D) qrot[t] = static_cast<float>(static_cast<_Float16>(qrot[t] * 0.0625f));
     __syncthreads();
   }
   const int closed = (len - 1) & ~15;           // keys the split-K kernel covered
@@ -718,15 +718,15 @@ __global__ __launch_bounds__(kReduceThreads) void Kv8Reduce(const DecodeArgs a, 
     }
   }
   const int n_extra = n_tail + (step ? 1 : 0);  // 1 .. 17
-  constexpr int NW = kReduceThreads / 64;
-  __shared__ float wgt[kReduceThreads], wl[kReduceThreads];
-  __shared__ int slot[kReduceThreads];
+  constexpr int NW = RT / 64;
+  __shared__ float wgt[RT], wl[RT];
+  __shared__ int slot[RT];
   __shared__ float red[NW];
   __shared__ int wave_n[NW];
-  __shared__ __align__(16) float sums[kReduceThreads * 4];
-  __shared__ float lsums[kReduceThreads / (kReduceMinDims / 4)];
+  __shared__ __align__(16) float sums[RT * 4];
+  __shared__ float lsums[RT / (kReduceMinDims / 4)];
   float M = first_ml.y > 0.0f ? first_ml.x : kNegMax;
-  for (size_t p = p0 + t + kReduceThreads; p < p1; p += kReduceThreads)
+  for (size_t p = p0 + t + RT; p < p1; p += RT)
     if (a.ml[(p * G + gi) * 2 + 1] > 0.0f) M = fmaxf(M, a.ml[(p * G + gi) * 2]);
   M = WaveMax(M);
   if (t % 64 == 0) red[t / 64] = M;
@@ -735,11 +735,11 @@ __global__ __launch_bounds__(kReduceThreads) void Kv8Reduce(const DecodeArgs a, 
   for (int w = 1; w < NW; ++w) M = fmaxf(M, red[w]);
   for (int j = 0; j < n_extra; ++j) M = fmaxf(M, tail_score[j]);
   const int lg_lanes = __builtin_ctz(static_cast<unsigned>(DZ)) - 2;
-  const int lanes = 1 << lg_lanes, n_groups = kReduceThreads >> lg_lanes, grp = t >> lg_lanes, dl = t & (lanes - 1);
+  const int lanes = 1 << lg_lanes, n_groups = RT >> lg_lanes, grp = t >> lg_lanes, dl = t & (lanes - 1);
   float L = 0.0f;
   float4 A = {0.0f, 0.0f, 0.0f, 0.0f};
-  for (size_t b0 = p0; b0 < p1; b0 += kReduceThreads) {
-    const int nb = static_cast<int>(min(p1 - b0, size_t(kReduceThreads)));
+  for (size_t b0 = p0; b0 < p1; b0 += RT) {
+    const int nb = static_cast<int>(min(p1 - b0, size_t(RT)));
     float l = 0.0f, mm = 0.0f;
     if (b0 == p0) l = first_ml.y, mm = first_ml.x;
     else if (t < nb) l = a.ml[((b0 + t) * G + gi) * 2 + 1], mm = a.ml[((b0 + t) * G + gi) * 2];
@@ -776,7 +776,7 @@ __global__ __launch_bounds__(kReduceThreads) void Kv8Reduce(const DecodeArgs a, 
   *reinterpret_cast<float4*>(&sums[grp * DZ + 4 * dl]) = A;
   if (dl == 0) lsums[grp] = L;
   __syncthreads();
-  for (int d = t; d < DZ; d += kReduceThreads) {
+  for (int d = t; d < DZ; d += RT) {
     float v = 0.0f, lt = 0.0f;
     for (int q = 0; q < n_groups; ++q) v += sums[q * DZ + d], lt += lsums[q];
     // the open tile's keys, as partials of one key each: V from the open f16 tile, the step's token from its source row
@@ -876,8 +876,16 @@ extern "C" int yahkv_kv8_decode_reduce(const yahkv_geometry* g, const yahkv_kv8_
   const int asked = MakeTuning(opt).reduce_split;
   if (asked > 0) split = std::min(asked, a.g.hd / kReduceMinDims);
   while (a.g.hd % split != 0 || (a.g.hd / split) % 4 != 0) --split;
-  hipLaunchKernelGGL(Kv8Reduce, dim3(a.g.n_q, a.n_seqs, split), dim3(kReduceThreads), 0, static_cast<hipStream_t>(stream), a,
-                     MakeKv8Pools(*pools), StepRows{k_new, v_new, new_dtype});
+  // A pair's places for partials are eight per chunk its tiles lie in, and with the kv heads dealt to the waves a
+  // sequence's tiles lie in every chunk of its stretch: a small batch (few sequences over many chunks) has up to a
+  // thousand places per pair, which a wider workgroup weighs in one sweep instead of four.
+  const int64_t places = int64_t(a.n_chunks) * a.wpc / std::max(a.n_seqs, 1) + a.wpc;
+  const dim3 grid(a.g.n_q, a.n_seqs, split);
+  const Kv8Pools kp = MakeKv8Pools(*pools);
+  const StepRows rows{k_new, v_new, new_dtype};
+  if (places > 512) hipLaunchKernelGGL(Kv8Reduce<1024>, grid, dim3(1024), 0, static_cast<hipStream_t>(stream), a, kp, rows);
+  else if (places > 256) hipLaunchKernelGGL(Kv8Reduce<512>, grid, dim3(512), 0, static_cast<hipStream_t>(stream), a, kp, rows);
+  else hipLaunchKernelGGL(Kv8Reduce<256>, grid, dim3(256), 0, static_cast<hipStream_t>(stream), a, kp, rows);
   return LaunchStatus();
 }
 
