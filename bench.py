@@ -196,6 +196,21 @@ def parity_check(yahkv, torch, g, pools, t_table, lens, q, out, scale, rows):
 
 
 CPU_REPS = 5
+APPEND_REPS = 20
+
+
+def time_repeated(torch, fn, reps=APPEND_REPS):
+    """ms per call of a short, repeatable piece of GPU work: `reps` calls back to back between one pair of HIP events
+    (a pair of events around a single call adds about 6 us of its own, a third of what a chunk append takes)."""
+    fn()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(reps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / reps
 
 
 def median_time(fn, reps=CPU_REPS):
@@ -538,14 +553,9 @@ def run_prefill_kv8(a, wl, torch, yahkv):
     out = torch.empty(q.shape, dtype=torch.float16, device="cuda")
     ws = torch.empty(yahkv.lib.yahkv_kv8_prefill_workspace_bytes(g, B, prefix, chunk), dtype=torch.uint8, device="cuda")
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(a.steps)]
-    ev_app = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(a.steps)]
 
-    def step(pair=None, app=None):
-        if app:
-            app[0].record()
+    def step(pair=None):
         yahkv.kv8_append(pools, t_table, t_prefix, knew, vnew)
-        if app:
-            app[1].record()
         if pair:
             pair[0].record()
         yahkv.kv8_prefill_attend(pools, t_table, t_prefix, prefix, q, scale, out=out, workspace=ws)
@@ -581,11 +591,12 @@ def run_prefill_kv8(a, wl, torch, yahkv):
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(a.steps):
-        step(ev[i], ev_app[i])
+        step(ev[i])
     torch.cuda.synchronize()
     ms = (time.perf_counter() - t0) / a.steps * 1e3
     kern_ms = float(np.mean([p[0].elapsed_time(p[1]) for p in ev]))
-    app_ms = float(np.median([p[0].elapsed_time(p[1]) for p in ev_app]))
+    # (the chunk's rows go to the same places again: the pools stay as they are)
+    app_ms = time_repeated(torch, lambda: yahkv.kv8_append(pools, t_table, t_prefix, knew, vnew))
     app_bytes = B * chunk * (2 * NKV * HD * 2 + (2336 if bits == 8 else 1408))   # bf16 rows in, codes + scales + stats out
     flops = float(B) * NQ * chunk * (prefix + (chunk + 1) / 2) * HD * 4
     return {
@@ -601,7 +612,7 @@ def run_prefill_kv8(a, wl, torch, yahkv):
         "append": {"kernel": "Kv8AppendRowsK + Kv8AppendTilesV", "ms": round(app_ms, 4), "bytes": int(app_bytes),
                    "GB/s": round(app_bytes / (app_ms * 1e-3) / 1e9, 1),
                    "frac_of_hbm_peak": round(app_bytes / (app_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-                   "note": "quantize + scatter of the chunk, HIP events around the call (median)"},
+                   "note": "quantize + scatter of the chunk: %d calls back to back between one pair of HIP events" % APPEND_REPS},
         "roofline": {"bound": "mfma", "achieved": round(flops / (kern_ms * 1e-3) / 1e12, 1),
                      "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(flops / (kern_ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
@@ -625,16 +636,9 @@ def run_prefill(a, wl, torch, yahkv):
     out = torch.empty(q.shape, dtype=torch.float16, device="cuda")   # the reference's kernel writes f16 (gen_attn_fa.py:1589-1595)
     ws = torch.empty(yahkv.prefill_workspace_bytes(g, B, prefix, chunk), dtype=torch.uint8, device="cuda")
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(a.steps)]
-    ev_app = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(a.steps)]
-    it = iter(ev_app)
 
     def step(pair=None):
-        app = next(it) if pair else None
-        if app:
-            app[0].record()
         yahkv.append(pools, t_table, t_prefix, knew, vnew)
-        if app:
-            app[1].record()
         if a.one_pass:                      # no workspace: the kernel that decodes each tile while staging it
             if pair:
                 pair[0].record()
@@ -682,7 +686,8 @@ def run_prefill(a, wl, torch, yahkv):
     dt = time.perf_counter() - t0
     ms = dt / a.steps * 1e3
     kern_ms = float(np.mean([p[0].elapsed_time(p[1]) for p in ev]))
-    app_ms = float(np.median([p[0].elapsed_time(p[1]) for p in ev_app]))
+    # (the chunk's rows go to the same places again: the pools stay as they are)
+    app_ms = time_repeated(torch, lambda: yahkv.append(pools, t_table, t_prefix, knew, vnew))
     app_bytes = B * chunk * (2 * NKV * HD * 2 + 2 * NKV * (HD // 32) * (34 if wl["fmt"] == 8 else 18))   # bf16 rows in, blocks out
     flops = float(B) * NQ * chunk * (prefix + (chunk + 1) / 2) * HD * 4   # both products, causal part counted once
     res = {
@@ -700,7 +705,7 @@ def run_prefill(a, wl, torch, yahkv):
         "append": {"kernel": "AppendPages<%d, 2>" % wl["fmt"], "ms": round(app_ms, 4), "bytes": int(app_bytes),
                    "GB/s": round(app_bytes / (app_ms * 1e-3) / 1e9, 1),
                    "frac_of_hbm_peak": round(app_bytes / (app_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-                   "note": "quantize + scatter of the chunk, HIP events around the call (median)"},
+                   "note": "quantize + scatter of the chunk: %d calls back to back between one pair of HIP events" % APPEND_REPS},
         "roofline": {"bound": "mfma", "achieved": round(flops / (kern_ms * 1e-3) / 1e12, 1),
                      "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(flops / (kern_ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
