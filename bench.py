@@ -622,7 +622,7 @@ def run_prefill_kv8(a, wl, torch, yahkv):
                    "step": "append chunk (quantize + scatter) + decode tiles to f16 + causal attention"},
         "tok_per_s": round(B * chunk / (ms * 1e-3), 1), "flops_per_step": int(flops),
         "parity_max_rel_err": float(f"{err:.3e}"), "out_fnv1a": first_hash,
-        "append": {"kernel": "Kv8AppendRowsK + Kv8AppendTilesV", "ms": round(app_ms, 4), "bytes": int(app_bytes),
+        "append": {"kernel": "Kv8AppendChunk", "ms": round(app_ms, 4), "bytes": int(app_bytes),
                    "GB/s": round(app_bytes / (app_ms * 1e-3) / 1e9, 1),
                    "frac_of_hbm_peak": round(app_bytes / (app_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                    "note": "quantize + scatter of the chunk: %d calls back to back between one pair of HIP events" % APPEND_REPS},

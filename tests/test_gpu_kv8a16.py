@@ -357,6 +357,45 @@ def test_chunked_prefill_over_a_paged_prefix(yahkv, torch_gpu):
     assert worst < TOL
 
 
+@pytest.mark.parametrize("bits", [8, 4])
+def test_chunks_that_start_inside_a_tile_and_end_in_its_page(yahkv, torch_gpu, bits):
+    """The chunk's first tile takes its earlier keys from the page's open tile, and the chunk's newest tile is written
+    there: with first and newest tile in one page these are the same bytes, read and written inside one launch. Many
+    sequences with such chunks (and some that start on a tile, end on one, or cross into the next page), three chunks
+    one after the other, every buffer against the oracle after each."""
+    torch = torch_gpu
+    rng = np.random.default_rng(77)
+    n_q, H, S = 8, 4, 96
+    g = yahkv.kv8_geometry(n_q, H, 2 * S, bits, bits)
+    dp, hp = yahkv.Kv8Pools(g, 0x33), kv8.HostPools(kv8.geometry(n_q, H, 2 * S, bits, bits), 0x33)
+    table = rng.permutation(2 * S).astype(np.int32).reshape(S, 2)
+    t_table = torch.from_numpy(table).cuda()
+    pos = rng.integers(0, 40, S).astype(np.int32)
+    pos[:4] = (0, 16, 5, 250)
+    first = np.maximum(pos, 1)
+    K0 = rng.standard_normal((S, 256, H, 256)).astype(np.float16)
+    V0 = rng.standard_normal((S, 256, H, 256)).astype(np.float16)
+    nv = torch.from_numpy(first).cuda()
+    yahkv.kv8_kmean(dp, t_table, torch.from_numpy(K0).cuda(), nv)
+    for s in range(S):
+        hp.km[table[s, 0]] = kv8.kmean(K0[s, :first[s]].astype(np.float32).reshape(first[s], -1))
+    # the keys before the first chunk, so that there is an open tile to read
+    yahkv.kv8_append(dp, t_table, torch.zeros(S, dtype=torch.int32, device="cuda"), torch.from_numpy(K0).cuda(),
+                     torch.from_numpy(V0).cuda(), torch.from_numpy(pos).cuda())
+    kv8.append(hp, table, [0] * S, pos.tolist(), K0.astype(np.float32).reshape(S, 256, -1), V0.astype(np.float32).reshape(S, 256, -1))
+    for step, chunk in enumerate((37, 64, 50)):
+        n = rng.integers(2, chunk + 1, S).astype(np.int32)
+        n[:3] = chunk
+        K = rng.standard_normal((S, chunk, H, 256)).astype(np.float16)
+        V = rng.standard_normal((S, chunk, H, 256)).astype(np.float16)
+        yahkv.kv8_append(dp, t_table, torch.from_numpy(pos).cuda(), torch.from_numpy(K).cuda(), torch.from_numpy(V).cuda(),
+                         torch.from_numpy(n).cuda())
+        kv8.append(hp, table, pos.tolist(), n.tolist(), K.astype(np.float32).reshape(S, chunk, -1), V.astype(np.float32).reshape(S, chunk, -1))
+        torch.cuda.synchronize()
+        assert_pools_equal(dp, hp, f"chunk {step} of {chunk} rows")
+        pos = pos + n
+
+
 def test_refusals(yahkv, torch_gpu):
     torch = torch_gpu
     g = yahkv.kv8_geometry(24, 4, 2)

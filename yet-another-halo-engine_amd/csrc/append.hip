@@ -41,21 +41,6 @@ struct RopeArgs {
   float* k_out;       // [n_seqs][n_new][H][D] f32 or null: the rotated K rows, for callers that want them
 };
 
-// The same in two steps, for loads that stay in flight while other work is done: the raw bytes, widened later.
-__device__ __forceinline__ uint4 LoadRaw4(const void* src, size_t i, int dtype) {
-  if (dtype == YAHKV_F32) return *reinterpret_cast<const uint4*>(static_cast<const float*>(src) + i);
-  const uint2 w = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(src) + i);
-  return uint4{w.x, w.y, 0u, 0u};
-}
-__device__ __forceinline__ float4 Widen4(uint4 w, int dtype) {
-  if (dtype == YAHKV_F32)
-    return float4{__builtin_bit_cast(float, w.x), __builtin_bit_cast(float, w.y), __builtin_bit_cast(float, w.z),
-                  __builtin_bit_cast(float, w.w)};
-  const uint16_t h[4] = {static_cast<uint16_t>(w.x & 0xFFFF), static_cast<uint16_t>(w.x >> 16),
-                         static_cast<uint16_t>(w.y & 0xFFFF), static_cast<uint16_t>(w.y >> 16)};
-  if (dtype == YAHKV_F16) return float4{WidenF16(h[0]), WidenF16(h[1]), WidenF16(h[2]), WidenF16(h[3])};
-  return float4{WidenBf16(h[0]), WidenBf16(h[1]), WidenBf16(h[2]), WidenBf16(h[3])};
-}
 __device__ __forceinline__ void Store4(void* dst, size_t i, int dtype, float4 v) {
   if (dtype == YAHKV_F32) {
     *reinterpret_cast<float4*>(static_cast<float*>(dst) + i) = v;

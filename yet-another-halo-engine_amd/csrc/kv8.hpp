@@ -22,7 +22,10 @@
 #ifndef YAHKV_KV8_HPP_
 #define YAHKV_KV8_HPP_
 
+#include <type_traits>
+
 #include "common.hpp"
+#include "quant.hpp"
 
 namespace yahkv {
 
@@ -116,15 +119,17 @@ __device__ __forceinline__ float4 WaveHadamard256(float4 x, int lane) {
 #pragma clang fp contract(off)
   const float a0 = x.x + x.y, a1 = x.x - x.y, a2 = x.z + x.w, a3 = x.z - x.w;
   float v[4] = {a0 + a2, a1 + a3, a0 - a2, a1 - a3};
-#pragma unroll
-  for (int k = 1; k < 64; k <<= 1) {
+  auto stage = [&](auto kc) {
+    constexpr int k = decltype(kc)::value;
     const bool upper = (lane & k) != 0;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      const float o = __shfl_xor(v[e], k, 64);
+      const float o = LaneXor<k>(v[e]);
       v[e] = upper ? o - v[e] : v[e] + o;
     }
-  }
+  };
+  stage(std::integral_constant<int, 1>{}), stage(std::integral_constant<int, 2>{}), stage(std::integral_constant<int, 4>{});
+  stage(std::integral_constant<int, 8>{}), stage(std::integral_constant<int, 16>{}), stage(std::integral_constant<int, 32>{});
   return float4{v[0], v[1], v[2], v[3]};
 }
 
@@ -137,8 +142,9 @@ __device__ __forceinline__ uint32_t Kv4CodesK(float4 centred, int lane, uint32_t
   const float4 h = WaveHadamard256(centred, lane);
   const float xr[4] = {h.x * 0.0625f, h.y * 0.0625f, h.z * 0.0625f, h.w * 0.0625f};
   float lo = fminf(fminf(xr[0], xr[1]), fminf(xr[2], xr[3])), hi = fmaxf(fmaxf(xr[0], xr[1]), fmaxf(xr[2], xr[3]));
-#pragma unroll
-  for (int k = 1; k < 8; k <<= 1) lo = fminf(lo, __shfl_xor(lo, k, 64)), hi = fmaxf(hi, __shfl_xor(hi, k, 64));
+  lo = fminf(lo, LaneXor<1>(lo)), hi = fmaxf(hi, LaneXor<1>(hi));  // over the group's eight lanes
+  lo = fminf(lo, LaneXor<2>(lo)), hi = fmaxf(hi, LaneXor<2>(hi));
+  lo = fminf(lo, LaneXor<4>(lo)), hi = fmaxf(hi, LaneXor<4>(hi));
   const float s0 = (hi - lo) / 15.0f;
   const float s = s0 > 0.0f ? s0 : 1.0f;
   const float inv = 1.0f / s;

@@ -47,10 +47,16 @@ struct Kv8AppendArgs {
   int32_t dtype;
 };
 
+// The positions, counts and page table are read through the constant address space: nothing writes them while the
+// kernel runs, and only then does the compiler use scalar loads, several of which go out together (as ordinary global
+// loads each one waited for the one before, with a branch between).
+typedef const int32_t __attribute__((address_space(4))) * ConstInts;
+__device__ __forceinline__ ConstInts AsConst(const int32_t* p) { return (ConstInts)(reinterpret_cast<uintptr_t>(p)); }
+
 // first position and number of real tokens of sequence s that lie inside the table; count 0: nothing to write
 __device__ __forceinline__ int RealTokens(const Kv8AppendArgs& a, int s, int* p0) {
-  const int start = a.start_pos[s];
-  int nv = a.n_valid != nullptr ? min(a.n_valid[s], a.n_new) : a.n_new;
+  const int start = AsConst(a.start_pos)[s];
+  int nv = a.n_valid != nullptr ? min(AsConst(a.n_valid)[s], a.n_new) : a.n_new;
   *p0 = start;
   if (start < 0) return 0;
   const long long cap = static_cast<long long>(a.stride) * kKv8Page;
@@ -58,19 +64,18 @@ __device__ __forceinline__ int RealTokens(const Kv8AppendArgs& a, int s, int* p0
   return max(nv, 0);
 }
 __device__ __forceinline__ int PageOf(const Kv8AppendArgs& a, int s, int pos) {
-  return ClampPage(a.table[int64_t(s) * a.stride + pos / kKv8Page], a.g.n_pages);
+  return ClampPage(AsConst(a.table)[int64_t(s) * a.stride + pos / kKv8Page], a.g.n_pages);
 }
 
 // One K row of one kv head across a wave, four consecutive dims per lane: centre, scale per 128-dim half (32 lanes),
 // codes, stores. `x`: the lane's four source values.
-__device__ __forceinline__ void Kv8StoreRowK(const Kv8Geom& g, const Kv8Pools& p, int page0, size_t row, int h, int lane,
+__device__ __forceinline__ void Kv8StoreRowK(const Kv8Geom& g, const Kv8Pools& p, float4 m, size_t row, int h, int lane,
                                              float4 x) {
 #pragma clang fp contract(off)
-  const float4 m = *reinterpret_cast<const float4*>(p.km + g.km_head(page0, h) + 4 * lane);
   const float4 c = {TruncF16(x.x) - m.x, TruncF16(x.y) - m.y, TruncF16(x.z) - m.z, TruncF16(x.w) - m.w};
   float amax = fmaxf(fmaxf(fabsf(c.x), fabsf(c.y)), fmaxf(fabsf(c.z), fabsf(c.w)));
-#pragma unroll
-  for (int o = 16; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));  // over the half's 32 lanes
+  amax = fmaxf(amax, LaneXor<1>(amax)), amax = fmaxf(amax, LaneXor<2>(amax)), amax = fmaxf(amax, LaneXor<4>(amax));
+  amax = fmaxf(amax, LaneXor<8>(amax)), amax = fmaxf(amax, LaneXor<16>(amax));  // over the half's 32 lanes
   float inv;
   uint32_t pair;
   Kv8ScaleK(amax, &inv, &pair);
@@ -78,22 +83,25 @@ __device__ __forceinline__ void Kv8StoreRowK(const Kv8Geom& g, const Kv8Pools& p
   if (lane % 32 == 0) p.ks[g.ks_row(row, h) + lane / 32] = pair;
 }
 // the same for 4-bit K: rotated, 16 levels per 32-dim group (eight lanes), two lanes per dword
-__device__ __forceinline__ void Kv4StoreRowK(const Kv8Geom& g, const Kv8Pools& p, int page0, size_t row, int h, int lane,
+__device__ __forceinline__ void Kv4StoreRowK(const Kv8Geom& g, const Kv8Pools& p, float4 m, size_t row, int h, int lane,
                                              float4 x) {
 #pragma clang fp contract(off)
-  const float4 m = *reinterpret_cast<const float4*>(p.km + g.km_head(page0, h) + 4 * lane);
   const float4 c = {TruncF16(x.x) - m.x, TruncF16(x.y) - m.y, TruncF16(x.z) - m.z, TruncF16(x.w) - m.w};
   uint32_t pair;
   float4 deq;
   uint32_t w = Kv4CodesK(c, lane, &pair, &deq);
-  w |= __shfl_xor(w, 1, 64);
+  w |= LaneXorBits<1>(w);
   if (lane % 2 == 0) p.kq[g.kq_row(row, h) + lane / 2] = w;
   if (lane % 8 == 0) p.ks[g.ks_row(row, h) + lane / 8] = pair;
 }
-__device__ __forceinline__ void StoreRowK(const Kv8Geom& g, const Kv8Pools& p, int page0, size_t row, int h, int lane,
+// `m`: the lane's four channel means (MeansK)
+__device__ __forceinline__ void StoreRowK(const Kv8Geom& g, const Kv8Pools& p, float4 m, size_t row, int h, int lane,
                                           float4 x) {
-  if (g.kb == 4) Kv4StoreRowK(g, p, page0, row, h, lane, x);
-  else Kv8StoreRowK(g, p, page0, row, h, lane, x);
+  if (g.kb == 4) Kv4StoreRowK(g, p, m, row, h, lane, x);
+  else Kv8StoreRowK(g, p, m, row, h, lane, x);
+}
+__device__ __forceinline__ float4 MeansK(const Kv8Geom& g, const Kv8Pools& p, int page0, int h, int lane) {
+  return *reinterpret_cast<const float4*>(p.km + g.km_head(page0, h) + 4 * lane);
 }
 // a channel's 16 keys of a tile to their place among the codes and stats
 __device__ __forceinline__ void StoreTileV(const Kv8Geom& g, const Kv8Pools& p, int h, size_t pt, int d, const float (&x)[16]) {
@@ -110,25 +118,28 @@ __device__ __forceinline__ void StoreTileV(const Kv8Geom& g, const Kv8Pools& p, 
   p.vs[g.vs_tile(h, pt) + d] = stats;
 }
 
-// yah_kmean: thread (row group, channel); eight row groups, each summing its rows in order, then the groups in order
-template <int DUMMY>
+// yah_kmean: thread (row group, channel); eight row groups, each summing its rows in order, then the groups in order.
+// SRC: the source rows' type, known when compiling: as a run-time value it put a branch behind every load, and the
+// loads then went out one at a time, each waiting for the one before (2048 rows: 325 us; this way 32 are in flight).
+template <int SRC>
 __global__ __launch_bounds__(256) void Kv8Kmean(const Kv8AppendArgs a) {
 #pragma clang fp contract(off)
+  constexpr int kAhead = 32;
   const int s = blockIdx.y, t = threadIdx.x, cc = t % 32, grp = t / 32, W = a.g.W();
   const int c = blockIdx.x * 32 + cc;
-  const int valid = a.n_valid != nullptr ? a.n_valid[s] : a.n_new;
+  const int valid = a.n_valid != nullptr ? AsConst(a.n_valid)[s] : a.n_new;
   const int n = min(a.n_new, max(valid, 1));
   __shared__ float part[8][32];
   float acc = 0.0f;
   int r = grp;
-  for (; r + 8 * 15 < n; r += 8 * 16) {  // sixteen loads in flight, added in the rows' order
-    float x[16];
+  for (; r + 8 * (kAhead - 1) < n; r += 8 * kAhead) {  // added in the rows' order
+    uint32_t x[kAhead];
 #pragma unroll
-    for (int j = 0; j < 16; ++j) x[j] = LoadSrc(a.k_src, (size_t(s) * a.n_new + r + 8 * j) * W + c, a.dtype);
+    for (int j = 0; j < kAhead; ++j) x[j] = LoadRaw1(a.k_src, (size_t(s) * a.n_new + r + 8 * j) * W + c, SRC);
 #pragma unroll
-    for (int j = 0; j < 16; ++j) acc = acc + TruncF16(x[j]);
+    for (int j = 0; j < kAhead; ++j) acc = acc + TruncF16(Widen1(x[j], SRC));
   }
-  for (; r < n; r += 8) acc = acc + TruncF16(LoadSrc(a.k_src, (size_t(s) * a.n_new + r) * W + c, a.dtype));
+  for (; r < n; r += 8) acc = acc + TruncF16(Widen1(LoadRaw1(a.k_src, (size_t(s) * a.n_new + r) * W + c, SRC), SRC));
   part[grp][cc] = acc;
   __syncthreads();
   if (grp == 0) {
@@ -148,7 +159,7 @@ __global__ __launch_bounds__(64) void Kv8AppendToken(const Kv8AppendArgs a) {
   const int page = PageOf(a, s, pos), page0 = PageOf(a, s, 0);
   const size_t src = (size_t(s) * g.n_kv + h) * kKv8Dim + 4 * lane;
   const float4 k = Load4(a.k_src, src, a.dtype), v = Load4(a.v_src, src, a.dtype);
-  StoreRowK(g, a.p, page0, size_t(page) * kKv8Page + pos % kKv8Page, h, lane, k);
+  StoreRowK(g, a.p, MeansK(g, a.p, page0, h, lane), size_t(page) * kKv8Page + pos % kKv8Page, h, lane, k);
   // V: the token's key of the open tile; on the tile's 16th key the tile is quantized into its place
   const int key = pos % 16;
   uint16_t* vo = a.p.vo + g.vo_head(page, h) + size_t(4 * lane) * 16;
@@ -169,60 +180,138 @@ __global__ __launch_bounds__(64) void Kv8AppendToken(const Kv8AppendArgs a) {
   }
 }
 
-// The prefill's K rows: one workgroup of four waves per (token, sequence), the kv heads dealt to the waves.
-__global__ __launch_bounds__(256) void Kv8AppendRowsK(const Kv8AppendArgs a) {
-  const int i = blockIdx.x, s = blockIdx.y, wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+// The prefill's K rows: a workgroup of four waves takes kRowsPerGroup consecutive tokens of a sequence, the kv heads dealt
+// to the waves; a wave asks for all its rows of a head, and for the head's means, before it works on the first (a row is
+// a few round trips and 40 instructions: one row per workgroup left the memory system mostly waiting).
+constexpr int kRowsPerGroup = 8;
+static_assert(kRowsPerGroup <= kKv8Page, "a group's rows lie in at most two pages");
+template <int SRC>
+__device__ __forceinline__ void AppendRowsK(const Kv8AppendArgs& a, int i0, int s) {
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   int p0;
-  if (i >= RealTokens(a, s, &p0)) return;
+  const int nv = RealTokens(a, s, &p0);
+  if (i0 >= nv) return;
   const Kv8Geom& g = a.g;
-  const int pos = p0 + i, page = PageOf(a, s, pos), page0 = PageOf(a, s, 0);
+  // (the group's rows lie in at most two pages: both numbers now, not one per row between the rows' work)
+  const int pos_a = p0 + i0, pos_b = p0 + min(i0 + kRowsPerGroup, nv) - 1;
+  const int page0 = PageOf(a, s, 0), page_a = PageOf(a, s, pos_a), page_b = PageOf(a, s, pos_b);
   for (int h = wave; h < g.n_kv; h += 4) {
-    const float4 k = Load4(a.k_src, ((size_t(s) * a.n_new + i) * g.n_kv + h) * kKv8Dim + 4 * lane, a.dtype);
-    StoreRowK(g, a.p, page0, size_t(page) * kKv8Page + pos % kKv8Page, h, lane, k);
+    uint4 raw[kRowsPerGroup];
+#pragma unroll
+    for (int r = 0; r < kRowsPerGroup; ++r) {
+      const int i = min(i0 + r, nv - 1);
+      raw[r] = LoadRaw4(a.k_src, ((size_t(s) * a.n_new + i) * g.n_kv + h) * kKv8Dim + 4 * lane, SRC);
+    }
+    const float4 m = MeansK(g, a.p, page0, h, lane);
+#pragma unroll
+    for (int r = 0; r < kRowsPerGroup; ++r) {
+      if (i0 + r >= nv) break;
+      const int pos = p0 + i0 + r, page = pos / kKv8Page == pos_a / kKv8Page ? page_a : page_b;
+      StoreRowK(g, a.p, m, size_t(page) * kKv8Page + pos % kKv8Page, h, lane, Widen4(raw[r], SRC));
+    }
   }
 }
 
-// The prefill's V tiles: one workgroup per (16-key tile the chunk touches, sequence, kv head), thread = channel.
-// Keys of the tile before the chunk's first are in the open tile; keys past the chunk's last real token repeat it.
-__global__ __launch_bounds__(256) void Kv8AppendTilesV(const Kv8AppendArgs a) {
-  const int s = blockIdx.y, h = blockIdx.z, d = threadIdx.x;
+// The prefill's V tiles: one wave per (16-key tile the chunk touches, kv head), four channels per lane (a row of the
+// source is then 8 or 16 bytes per lane; with a lane per channel the 2-byte loads kept the address units busier than
+// the memory). Keys of the tile before the chunk's first are in the open tile; keys past the chunk's last real token
+// repeat it.
+__device__ __forceinline__ float Component(const float4& v, int e) { return e == 0 ? v.x : e == 1 ? v.y : e == 2 ? v.z : v.w; }
+template <int SRC>
+__device__ __forceinline__ void AppendTileV(const Kv8AppendArgs& a, int item, int s) {
+  const Kv8Geom& g = a.g;
+  const int tile = item / g.n_kv, h = item % g.n_kv, d0 = 4 * (threadIdx.x % 64);
   int p0;
   const int nv = RealTokens(a, s, &p0);
   if (nv < 1) return;
-  const Kv8Geom& g = a.g;
-  const int last = p0 + nv - 1, t = p0 / 16 + blockIdx.x;
+  const int last = p0 + nv - 1, t = p0 / 16 + tile;
   if (16 * t > last) return;
-  const int page = PageOf(a, s, 16 * t);
-  uint16_t* vo = a.p.vo + g.vo_head(page, h) + size_t(d) * 16;
-  float x[16];
-  uint32_t open[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-  if (16 * t < p0) {
-    const uint4 lo = *reinterpret_cast<const uint4*>(vo), hi = *reinterpret_cast<const uint4*>(vo + 8);
-    open[0] = lo.x, open[1] = lo.y, open[2] = lo.z, open[3] = lo.w, open[4] = hi.x, open[5] = hi.y, open[6] = hi.z, open[7] = hi.w;
-  }
+  const int t_first = p0 / 16, t_last = last / 16;
+  const bool reads_open = 16 * t_first < p0;
+  const int page = PageOf(a, s, 16 * t), page_last = PageOf(a, s, 16 * t_last);
+  uint16_t* vo = a.p.vo + g.vo_head(page, h) + size_t(d0) * 16;
+  // all sixteen rows asked for at once (a key before the chunk's first asks for the first: its value is not used)
+  uint4 raw[16];
+  auto request = [&](int tt) {
 #pragma unroll
-  for (int j = 0; j < 16; ++j) {
-    const int pos = 16 * t + j;
-    if (pos < p0) {
-      x[j] = WidenF16(static_cast<uint16_t>(open[j / 2] >> (16 * (j % 2))));
+    for (int j = 0; j < 16; ++j) {
+      const size_t i = static_cast<size_t>(min(max(16 * tt + j, p0), last) - p0);
+      raw[j] = LoadRaw4(a.v_src, ((size_t(s) * a.n_new + i) * g.n_kv + h) * kKv8Dim + d0, SRC);
+    }
+  };
+  request(t);
+  uint4 open[4][2] = {};
+  if (16 * t < p0) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      open[e][0] = *reinterpret_cast<const uint4*>(vo + e * 16), open[e][1] = *reinterpret_cast<const uint4*>(vo + e * 16 + 8);
+  }
+  auto open_word = [&](int e, int w) -> uint32_t {  // keys 2 w, 2 w + 1 of channel d0 + e
+    const uint4& q = open[e][w / 4];
+    return w % 4 == 0 ? q.x : w % 4 == 1 ? q.y : w % 4 == 2 ? q.z : q.w;
+  };
+  // yah_vseed: the newest tile stays open, keys past the last real token zero. The open tile of a page is also what
+  // the chunk's first tile reads when the chunk starts inside a tile, and first and newest tile can lie in one page: the
+  // wave that reads the open tile is then also the one that writes it (each lane reads and writes its own channels'
+  // bytes, in that order); left to the newest tile's wave the write could come before the read.
+  const bool seeds = t == (reads_open ? t_first : t_last);
+  const size_t pt = size_t(page) * 16 + t % 16;
+  uint32_t stats[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {  // channel d0 + e
+    float x[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      const float from_open = WidenF16(static_cast<uint16_t>(open_word(e, j / 2) >> (16 * (j % 2))));
+      x[j] = 16 * t + j < p0 ? from_open : TruncF16(Component(Widen4(raw[j], SRC), e));
+    }
+    if (g.vb == 4) {
+      uint2 codes;
+      Kv4QuantTile(x, &codes, &stats[e]);
+      *reinterpret_cast<uint2*>(a.p.vq + g.vq_tile(h, pt) + size_t(d0 + e) * 2) = codes;
     } else {
-      const size_t i = static_cast<size_t>(min(pos, last) - p0);
-      x[j] = TruncF16(LoadSrc(a.v_src, ((size_t(s) * a.n_new + i) * g.n_kv + h) * kKv8Dim + d, a.dtype));
+      uint4 codes;
+      Kv8QuantTile(x, &codes, &stats[e]);
+      *reinterpret_cast<uint4*>(a.p.vq + g.vq_tile(h, pt) + size_t(d0 + e) * 4) = codes;
+    }
+    if (seeds && t == t_last) {
+      uint32_t w[8];
+#pragma unroll
+      for (int j = 0; j < 16; j += 2) {
+        const uint32_t b0 = 16 * t + j < p0 ? open_word(e, j / 2) & 0xFFFFu : (16 * t + j <= last ? F16Bits(x[j]) : 0u);
+        const uint32_t b1 = 16 * t + j + 1 < p0 ? open_word(e, j / 2) >> 16 : (16 * t + j + 1 <= last ? F16Bits(x[j + 1]) : 0u);
+        w[j / 2] = b0 | (b1 << 16);
+      }
+      *reinterpret_cast<uint4*>(vo + e * 16) = uint4{w[0], w[1], w[2], w[3]};
+      *reinterpret_cast<uint4*>(vo + e * 16 + 8) = uint4{w[4], w[5], w[6], w[7]};
     }
   }
-  const size_t pt = size_t(page) * 16 + t % 16;
-  StoreTileV(g, a.p, h, pt, d, x);
-  if (t == last / 16) {  // yah_vseed: the newest tile stays open, keys past the last real token zero
+  *reinterpret_cast<uint4*>(a.p.vs + g.vs_tile(h, pt) + d0) = uint4{stats[0], stats[1], stats[2], stats[3]};
+  if (!seeds || t == t_last) return;
+  // the newest tile lies wholly inside the chunk: its rows once more
+  request(t_last);
+  vo = a.p.vo + g.vo_head(page_last, h) + size_t(d0) * 16;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
     uint32_t w[8];
 #pragma unroll
     for (int j = 0; j < 16; j += 2) {
-      const uint32_t b0 = 16 * t + j < p0 ? open[j / 2] & 0xFFFFu : (16 * t + j <= last ? F16Bits(x[j]) : 0u);
-      const uint32_t b1 = 16 * t + j + 1 < p0 ? open[j / 2] >> 16 : (16 * t + j + 1 <= last ? F16Bits(x[j + 1]) : 0u);
+      const uint32_t b0 = 16 * t_last + j <= last ? F16Bits(TruncF16(Component(Widen4(raw[j], SRC), e))) : 0u;
+      const uint32_t b1 = 16 * t_last + j + 1 <= last ? F16Bits(TruncF16(Component(Widen4(raw[j + 1], SRC), e))) : 0u;
       w[j / 2] = b0 | (b1 << 16);
     }
-    *reinterpret_cast<uint4*>(vo) = uint4{w[0], w[1], w[2], w[3]};
-    *reinterpret_cast<uint4*>(vo + 8) = uint4{w[4], w[5], w[6], w[7]};
+    *reinterpret_cast<uint4*>(vo + e * 16) = uint4{w[0], w[1], w[2], w[3]};
+    *reinterpret_cast<uint4*>(vo + e * 16 + 8) = uint4{w[4], w[5], w[6], w[7]};
   }
+}
+
+// A chunk's K rows and V tiles in one launch (they are independent): blocks [0, k_groups) take the K rows, the waves of
+// the rest one (tile, kv head) each, kv head fastest. SRC: the source rows' type (see Kv8Kmean).
+template <int SRC>
+__global__ __launch_bounds__(256) void Kv8AppendChunk(const Kv8AppendArgs a, int k_groups) {
+  const int b = blockIdx.x, s = blockIdx.y;
+  if (b < k_groups) AppendRowsK<SRC>(a, b * kRowsPerGroup, s);
+  else AppendTileV<SRC>(a, (b - k_groups) * 4 + static_cast<int>(threadIdx.x / 64), s);
 }
 
 int FillArgs(const yahkv_geometry* g, const yahkv_kv8_pools* pools, const int32_t* page_table, int32_t stride,
@@ -270,7 +359,11 @@ int yahkv_kv8_kmean(const yahkv_geometry* g, const yahkv_kv8_pools* pools, const
   if (const int st = FillArgs(g, pools, page_table, page_table_stride, nullptr, n_valid, n_seqs, n_rows, k_src, k_src,
                               src_dtype, &a))
     return st;
-  hipLaunchKernelGGL(Kv8Kmean<0>, dim3(a.g.W() / 32, n_seqs), dim3(256), 0, static_cast<hipStream_t>(stream), a);
+  const dim3 grid(a.g.W() / 32, n_seqs);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (src_dtype == YAHKV_F32) hipLaunchKernelGGL(Kv8Kmean<YAHKV_F32>, grid, dim3(256), 0, st, a);
+  else if (src_dtype == YAHKV_F16) hipLaunchKernelGGL(Kv8Kmean<YAHKV_F16>, grid, dim3(256), 0, st, a);
+  else hipLaunchKernelGGL(Kv8Kmean<YAHKV_BF16>, grid, dim3(256), 0, st, a);
   return LaunchStatus();
 }
 
@@ -287,10 +380,14 @@ int yahkv_kv8_append(const yahkv_geometry* g, const yahkv_kv8_pools* pools, cons
     hipLaunchKernelGGL(Kv8AppendToken, dim3(g->n_kv_heads, n_seqs), dim3(64), 0, st, a);
     return LaunchStatus();
   }
-  hipLaunchKernelGGL(Kv8AppendRowsK, dim3(n_new, n_seqs), dim3(256), 0, st, a);
-  if (const int rc = LaunchStatus()) return rc;
   // a chunk that starts inside a tile touches one tile more than its length says
-  hipLaunchKernelGGL(Kv8AppendTilesV, dim3((n_new + 15) / 16 + 1, n_seqs, g->n_kv_heads), dim3(256), 0, st, a);
+  const int k_groups = (n_new + kRowsPerGroup - 1) / kRowsPerGroup;
+  const long long blocks = k_groups + (static_cast<long long>((n_new + 15) / 16 + 1) * g->n_kv_heads + 3) / 4;
+  if (blocks > 0x7fffffffll) return YAHKV_ERR_SHAPE;
+  const dim3 grid(static_cast<unsigned>(blocks), n_seqs);
+  if (src_dtype == YAHKV_F32) hipLaunchKernelGGL(Kv8AppendChunk<YAHKV_F32>, grid, dim3(256), 0, st, a, k_groups);
+  else if (src_dtype == YAHKV_F16) hipLaunchKernelGGL(Kv8AppendChunk<YAHKV_F16>, grid, dim3(256), 0, st, a, k_groups);
+  else hipLaunchKernelGGL(Kv8AppendChunk<YAHKV_BF16>, grid, dim3(256), 0, st, a, k_groups);
   return LaunchStatus();
 }
 

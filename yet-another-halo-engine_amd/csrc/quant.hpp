@@ -31,6 +31,34 @@ template <int CTRL>
 __device__ __forceinline__ int DppI(int x) { return __builtin_amdgcn_update_dpp(0, x, CTRL, 0xF, 0xF, false); }
 constexpr int kQuadSwap1 = 0xB1, kQuadSwap2 = 0x4E, kHalfMirror = 0x141, kRowMirror = 0x140;
 
+// The value of lane (l ^ K) of the wave, K a power of two: what `__shfl_xor(x, K, 64)` returns, without its round trip
+// through LDS. Inside a row of 16 lanes DPP controls do it (l ^ 4 is a half mirror, l ^ 7, then a reversed quad,
+// l ^ 3; l ^ 8 a row mirror, l ^ 15, then a half mirror); across rows the two row-swapping instructions of gfx950,
+// each of which leaves the lane's own value in one result and its partner's in the other.
+constexpr int kQuadReverse = 0x1B;
+template <int K>
+__device__ __forceinline__ uint32_t LaneXorBits(uint32_t u) {
+  static_assert(K == 1 || K == 2 || K == 4 || K == 8 || K == 16 || K == 32, "one bit of the lane number");
+  const int i = static_cast<int>(u);
+  if constexpr (K == 1) return static_cast<uint32_t>(DppI<kQuadSwap1>(i));
+  else if constexpr (K == 2) return static_cast<uint32_t>(DppI<kQuadSwap2>(i));
+  else if constexpr (K == 4) return static_cast<uint32_t>(DppI<kQuadReverse>(DppI<kHalfMirror>(i)));
+  else if constexpr (K == 8) return static_cast<uint32_t>(DppI<kHalfMirror>(DppI<kRowMirror>(i)));
+  else if constexpr (K == 16) {
+    const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    const uint32_t r0 = r[0], r1 = r[1];
+    return r0 != u ? r0 : r1;
+  } else {
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    const uint32_t r0 = r[0], r1 = r[1];
+    return r0 != u ? r0 : r1;
+  }
+}
+template <int K>
+__device__ __forceinline__ float LaneXor(float x) {
+  return __builtin_bit_cast(float, LaneXorBits<K>(__builtin_bit_cast(uint32_t, x)));
+}
+
 // Sum over the 64 lanes, in every lane: four DPP steps inside each row of 16 lanes, then the two row-swapping
 // instructions of gfx950 across the rows (no LDS round trips).
 __device__ __forceinline__ float WaveSum(float v) {
@@ -119,6 +147,31 @@ __device__ __forceinline__ float4 Load4(const void* src, size_t i, int dtype) {
                          static_cast<uint16_t>(w.y & 0xFFFF), static_cast<uint16_t>(w.y >> 16)};
   if (dtype == YAHKV_F16) return float4{WidenF16(h[0]), WidenF16(h[1]), WidenF16(h[2]), WidenF16(h[3])};
   return float4{WidenBf16(h[0]), WidenBf16(h[1]), WidenBf16(h[2]), WidenBf16(h[3])};
+}
+
+// The same in two steps, for loads that stay in flight while other work is done: the raw bytes, widened later.
+__device__ __forceinline__ uint4 LoadRaw4(const void* src, size_t i, int dtype) {
+  if (dtype == YAHKV_F32) return *reinterpret_cast<const uint4*>(static_cast<const float*>(src) + i);
+  const uint2 w = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(src) + i);
+  return uint4{w.x, w.y, 0u, 0u};
+}
+__device__ __forceinline__ float4 Widen4(uint4 w, int dtype) {
+  if (dtype == YAHKV_F32)
+    return float4{__builtin_bit_cast(float, w.x), __builtin_bit_cast(float, w.y), __builtin_bit_cast(float, w.z),
+                  __builtin_bit_cast(float, w.w)};
+  const uint16_t h[4] = {static_cast<uint16_t>(w.x & 0xFFFF), static_cast<uint16_t>(w.x >> 16),
+                         static_cast<uint16_t>(w.y & 0xFFFF), static_cast<uint16_t>(w.y >> 16)};
+  if (dtype == YAHKV_F16) return float4{WidenF16(h[0]), WidenF16(h[1]), WidenF16(h[2]), WidenF16(h[3])};
+  return float4{WidenBf16(h[0]), WidenBf16(h[1]), WidenBf16(h[2]), WidenBf16(h[3])};
+}
+// One element the same way: the raw bits (the low 16 for f16 / bf16), widened later.
+__device__ __forceinline__ uint32_t LoadRaw1(const void* src, size_t i, int dtype) {
+  if (dtype == YAHKV_F32) return static_cast<const uint32_t*>(src)[i];
+  return static_cast<const uint16_t*>(src)[i];
+}
+__device__ __forceinline__ float Widen1(uint32_t w, int dtype) {
+  if (dtype == YAHKV_F32) return __builtin_bit_cast(float, w);
+  return dtype == YAHKV_F16 ? WidenF16(static_cast<uint16_t>(w)) : WidenBf16(static_cast<uint16_t>(w));
 }
 
 // Where a quantized row goes. A row of head_dim values lies across a wavefront, four consecutive dims per lane (lanes
