@@ -130,6 +130,20 @@ void Kv8Part(const DecodeArgs a, const Kv8Pools pools) {
     const ConstRow crow = (ConstRow)(reinterpret_cast<uintptr_t>(row));
     return ClampPage(crow[min(tile / 4, a.stride - 1)], g.n_pages);
   };
+  // A pair's query entries of this lane, four pieces of eight dims of head row `rw` (first dim of piece e: dim0(e)): all
+  // four asked for together, under one branch on the type. With the type looked at load by load each piece's load sat in
+  // a branch of its own and went out when the one before had come back. A row past the group's asks for the last one;
+  // the caller zeroes it.
+  auto load_queries = [&](RawQ8 (&rq)[4], auto dim0, int rw) {
+    const size_t row = (size_t(cur.s) * g.n_q + size_t(head) * G + min(rw, G - 1)) * D;
+    if (a.q_dtype == YAHKV_F32) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) rq[e] = LoadRawQ8(a.q, row + dim0(e), YAHKV_F32);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) rq[e] = LoadRawQ8(a.q, row + dim0(e), YAHKV_F16);  // (16 bytes for bf16 as well)
+    }
+  };
   // K: the 32 rows of half tile tt to the LDS slot, four rows per instruction; lane l of instruction i carries chunk
   // (l % 16) ^ (row % 16) of row 4 i + l / 16 to LDS position 1024 i + 16 l
   // `live` false: a load whose result nobody uses (it keeps the count of loads in flight the same on every path):
@@ -364,12 +378,15 @@ void Kv8Part(const DecodeArgs a, const Kv8Pools pools) {
 #pragma clang fp contract(off)
       const int rw = lane % 8, hf = (lane / 8) % 2;
       float x[4][8];
+      RawQ8 rq[4];
+      load_queries(rq, [&](int e) {
+        const int mm = lane / 16 + 4 * e;
+        return 32 * (mm / 2) + 8 * (2 * hf + mm % 2);
+      }, rw);
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const int mm = lane / 16 + 4 * e;
-        const int d0 = 32 * (mm / 2) + 8 * (2 * hf + mm % 2);
-        h8v qv = {0, 0, 0, 0, 0, 0, 0, 0};
-        if (rw < G) qv = LoadQ8(a.q, (size_t(cur.s) * g.n_q + size_t(head) * G + rw) * D + d0, a.q_dtype);
+        h8v qv = ConvertQ8(rq[e], a.q_dtype);
+        if (rw >= G) qv = h8v{0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
         for (int k = 0; k < 8; ++k) x[e][k] = static_cast<float>(qv[k]);
 #pragma unroll
@@ -419,13 +436,17 @@ void Kv8Part(const DecodeArgs a, const Kv8Pools pools) {
       }
     } else {
       float hsum[2] = {0.0f, 0.0f};  // per (128-dim half, head row lane % 8): this lane's share
+      // entry i = lane + 64 e: step m = i / 16, lane half hf = (i / 8) % 2, head row rw = i % 8
+      RawQ8 rq[4];
+      load_queries(rq, [&](int e) {
+        const int i = lane + 64 * e, mm = i / 16, hf = (i / 8) % 2;
+        return 16 * (2 * (mm / 2) + hf) + 8 * (mm % 2);
+      }, lane % 8);
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        // entry i = lane + 64 e: step m = i / 16, lane half hf = (i / 8) % 2, head row rw = i % 8
         const int i = lane + 64 * e, mm = i / 16, hf = (i / 8) % 2, rw = i % 8;
-        const int d0 = 16 * (2 * (mm / 2) + hf) + 8 * (mm % 2);
-        h8v qv = {0, 0, 0, 0, 0, 0, 0, 0};
-        if (rw < G) qv = LoadQ8(a.q, (size_t(cur.s) * g.n_q + size_t(head) * G + rw) * D + d0, a.q_dtype);
+        h8v qv = ConvertQ8(rq[e], a.q_dtype);
+        if (rw >= G) qv = h8v{0, 0, 0, 0, 0, 0, 0, 0};
         float t = 0.0f;
 #pragma unroll
         for (int k = 0; k < 8; ++k) t += static_cast<float>(qv[k]);
