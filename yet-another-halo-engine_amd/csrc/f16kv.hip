@@ -12,11 +12,11 @@
 #include <cstdlib>
 
 #include "common.hpp"
+#include "decode_cut.hpp"
 
 namespace yahkv {
 namespace {
 
-typedef _Float16 h8v __attribute__((ext_vector_type(8)));
 typedef float f4v __attribute__((ext_vector_type(4)));
 typedef float f16v __attribute__((ext_vector_type(16)));
 
@@ -182,13 +182,10 @@ __device__ __forceinline__ float HalfSum(float v) {
   for (int o = 16; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
   return v;
 }
-// Eight consecutive query elements as f16 (bf16 and f16 sources convert exactly in the normal f16 range).
-__device__ __forceinline__ h8v Query8(const void* q, size_t i, int dt) {
-  h8v r;
-#pragma unroll
-  for (int j = 0; j < 8; ++j) r[j] = static_cast<_Float16>(LoadSrc(q, i + j, dt));
-  return r;
-}
+// Eight consecutive query elements as f16, one 16- or 32-byte read (LoadQ8: bf16 and f16 sources convert exactly in the
+// normal f16 range, finite values beyond it saturate). Element by element, with the type looked at for each, the
+// eight loads went out one after the other.
+__device__ __forceinline__ h8v Query8(const void* q, size_t i, int dt) { return LoadQ8(q, i, dt); }
 
 // One workgroup per (stretch of keys, kv head, sequence); its four waves take the stretch's 32-key tiles in turn, each
 // with its own online softmax, and merge through LDS into one partial (m, l, acc) per query head (gen_decode_attn.py:
@@ -495,7 +492,7 @@ extern "C" int yahkv_f16_decode_attend(const yahkv_geometry* g, const yahkv_f16_
     return YAHKV_ERR_ARG;
   if (n_seqs <= 0 || max_seq_len <= 0 || page_table_stride <= 0) return YAHKV_ERR_ARG;
   if (q_dtype != YAHKV_F32 && q_dtype != YAHKV_F16 && q_dtype != YAHKV_BF16) return YAHKV_ERR_ARG;
-  if (reinterpret_cast<uintptr_t>(workspace) & 15) return YAHKV_ERR_ARG;
+  if ((reinterpret_cast<uintptr_t>(workspace) | reinterpret_cast<uintptr_t>(q)) & 15) return YAHKV_ERR_ARG;
   if (n_seqs > 65535) return YAHKV_ERR_SHAPE;
   F16Args a{};
   a.g = MakeGeom(*g);

@@ -636,9 +636,17 @@ __global__ __launch_bounds__(RT) void Kv8Reduce(const DecodeArgs a, const Kv8Poo
       const uint32_t pair = pools.ks[kg8.ks_row(r, h) + c / 8];
       const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
       const size_t qi = (size_t(s) * g.n_q + hq) * D + 16 * c;
+      uint4 rq[4];  // the sixteen query values, asked for together under one branch on the type
+      if (a.q_dtype == YAHKV_F32) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) rq[i] = LoadRaw4(a.q, qi + 4 * i, YAHKV_F32);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) rq[i] = LoadRaw4(a.q, qi + 4 * i, YAHKV_F16);  // (8 bytes for bf16 as well)
+      }
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float4 q4 = Load4(a.q, qi + 4 * i, a.q_dtype);
+        const float4 q4 = Widen4(rq[i], a.q_dtype);
         const float qe[4] = {static_cast<float>(SaturateToF16(q4.x)), static_cast<float>(SaturateToF16(q4.y)),
                              static_cast<float>(SaturateToF16(q4.z)), static_cast<float>(SaturateToF16(q4.w))};
         // byte slots (d0, d2, d1, d3)
