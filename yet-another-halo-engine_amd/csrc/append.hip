@@ -65,9 +65,11 @@ __device__ __forceinline__ void Store4(void* dst, size_t i, int dtype, float4 v)
 // query heads) are dealt to the wavefronts in turn; a row lies across a wavefront, four consecutive dims per lane, so
 // every load and store is 16 (or 8) bytes per lane, the sum of squares and the block maxima are DPP reductions, and
 // the partner of a rotated pair comes through one lane shuffle: rows never go through LDS. A wavefront issues the
-// loads of all its rows (up to eight at a time) before it works on the first.
+// loads of all its rows (up to eight at a time) before it works on the first; for that the loads must not sit behind
+// branches, so the source rows' type SRC is known when compiling (as in AppendPages: with the type a run-time value
+// each load waited for the one before) and a row or lane that has nothing to load asks for an address that exists.
 constexpr int kRopeWaves = 4, kRowsInFlight = 8;
-template <int FMT, bool ROPE>
+template <int FMT, bool ROPE, int SRC>
 __global__ __launch_bounds__(64 * kRopeWaves) void AppendRows(const RopeArgs a) {
 #pragma clang fp contract(off)
   const Geom g = a.g;
@@ -122,24 +124,21 @@ __global__ __launch_bounds__(64 * kRopeWaves) void AppendRows(const RopeArgs a) 
     else *src = a.q_src, *off = (tok * g.n_q + (row - 2 * H)) * D;
   };
   for (int first_row = wave; first_row < rows_per_token; first_row += kRopeWaves * kRowsInFlight) {
-    float4 x[kRowsInFlight];
+    uint4 raw[kRowsInFlight];
 #pragma unroll
     for (int j = 0; j < kRowsInFlight; ++j) {
-      const int row = first_row + kRopeWaves * j;
-      x[j] = float4{0.0f, 0.0f, 0.0f, 0.0f};
-      if (row < rows_per_token && has) {
-        const void* src;
-        size_t off;
-        source(row, &src, &off);
-        x[j] = Load4(src, off + d0, a.src_dtype);
-      }
+      const void* src;
+      size_t off;
+      source(min(first_row + kRopeWaves * j, rows_per_token - 1), &src, &off);
+      raw[j] = LoadRaw4(src, off + (has ? d0 : 0), SRC);
     }
 #pragma unroll
     for (int j = 0; j < kRowsInFlight; ++j) {
       const int row = first_row + kRopeWaves * j;
       if (row >= rows_per_token) break;
       const bool is_v = row >= H && row < 2 * H, is_q = row >= 2 * H;
-      float4 v = x[j];
+      float4 v = Widen4(raw[j], SRC);
+      if (!has) v = float4{0.0f, 0.0f, 0.0f, 0.0f};
       if (ROPE && !is_v) {
         const float ss = WaveSum(v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w);
         const float inv_rms = 1.0f / sqrtf(ss / static_cast<float>(D) + a.eps);
@@ -381,6 +380,23 @@ int CheckAppend(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t
 }
 }  // namespace
 
+namespace {
+// AppendRows for the pools' format and the source rows' type (the kernel is compiled for each pair)
+template <bool ROPE>
+void LaunchRows(int32_t format, int32_t src_dtype, dim3 grid, hipStream_t st, const RopeArgs& a) {
+  const dim3 block(64 * kRopeWaves);
+  if (format == YAHKV_Q8_0) {
+    if (src_dtype == YAHKV_F32) hipLaunchKernelGGL((AppendRows<8, ROPE, YAHKV_F32>), grid, block, 0, st, a);
+    else if (src_dtype == YAHKV_F16) hipLaunchKernelGGL((AppendRows<8, ROPE, YAHKV_F16>), grid, block, 0, st, a);
+    else hipLaunchKernelGGL((AppendRows<8, ROPE, YAHKV_BF16>), grid, block, 0, st, a);
+  } else {
+    if (src_dtype == YAHKV_F32) hipLaunchKernelGGL((AppendRows<4, ROPE, YAHKV_F32>), grid, block, 0, st, a);
+    else if (src_dtype == YAHKV_F16) hipLaunchKernelGGL((AppendRows<4, ROPE, YAHKV_F16>), grid, block, 0, st, a);
+    else hipLaunchKernelGGL((AppendRows<4, ROPE, YAHKV_BF16>), grid, block, 0, st, a);
+  }
+}
+}  // namespace
+
 extern "C" int yahkv_append(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t* page_table,
                             int32_t page_table_stride, const int32_t* start_pos, const int32_t* n_valid,
                             int32_t n_seqs, int32_t n_new, const void* k_src, const void* v_src, int32_t src_dtype,
@@ -411,10 +427,7 @@ extern "C" int yahkv_append(const yahkv_geometry* g, const yahkv_pools* pools, c
     return LaunchStatus();
   }
   const dim3 grid(static_cast<unsigned>(n_seqs) * static_cast<unsigned>(n_new));
-  if (g->format == YAHKV_Q8_0)
-    hipLaunchKernelGGL((AppendRows<8, false>), grid, dim3(64 * kRopeWaves), 0, st, a);
-  else
-    hipLaunchKernelGGL((AppendRows<4, false>), grid, dim3(64 * kRopeWaves), 0, st, a);
+  LaunchRows<false>(g->format, src_dtype, grid, st, a);
   return LaunchStatus();
 }
 
@@ -441,10 +454,7 @@ extern "C" int yahkv_append_rope(const yahkv_geometry* g, const yahkv_pools* poo
   const int64_t tokens = int64_t(n_seqs) * n_new;
   if (tokens > 0x7FFFFFFF) return YAHKV_ERR_SHAPE;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (g->format == YAHKV_Q8_0)
-    hipLaunchKernelGGL((AppendRows<8, true>), dim3(static_cast<unsigned>(tokens)), dim3(64 * kRopeWaves), 0, st, a);
-  else
-    hipLaunchKernelGGL((AppendRows<4, true>), dim3(static_cast<unsigned>(tokens)), dim3(64 * kRopeWaves), 0, st, a);
+  LaunchRows<true>(g->format, src_dtype, dim3(static_cast<unsigned>(tokens)), st, a);
   return LaunchStatus();
 }
 
