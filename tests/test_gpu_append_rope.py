@@ -14,15 +14,17 @@ pytestmark = pytest.mark.gpu
 TOL = 1e-3
 
 
-@pytest.mark.parametrize("fmt,n_q,n_kv,hd,pt,rot,theta", [
-    (8, 24, 4, 256, 64, 256, 1e7), (8, 8, 2, 128, 16, 128, 1e4), (8, 24, 4, 256, 64, 64, 1e6),
-    (4, 24, 4, 256, 64, 256, 1e7), (4, 8, 2, 128, 32, 64, 1e4),
+@pytest.mark.parametrize("fmt,n_q,n_kv,hd,pt,rot,theta,n_new", [
+    (8, 24, 4, 256, 64, 256, 1e7, 21), (8, 8, 2, 128, 16, 128, 1e4, 21), (8, 24, 4, 256, 64, 64, 1e6, 21),
+    (4, 24, 4, 256, 64, 256, 1e7, 21), (4, 8, 2, 128, 32, 64, 1e4, 21),
+    # chunks of eight pages or more: a page's tokens go to the workgroups of one XCD, in another order than the rows'
+    (8, 24, 4, 256, 64, 64, 1e6, 600), (4, 8, 2, 128, 16, 128, 1e4, 131), (8, 8, 2, 128, 32, 64, 1e4, 256),
 ])
-def test_fused_append_matches_oracle(yahkv, torch_gpu, fmt, n_q, n_kv, hd, pt, rot, theta):
+def test_fused_append_matches_oracle(yahkv, torch_gpu, fmt, n_q, n_kv, hd, pt, rot, theta, n_new):
     torch = torch_gpu
-    rng = np.random.default_rng(fmt * 100 + hd + rot)
-    starts, n_new = [0, 37, 1000], 21
-    n_valid = [21, 5, 21]
+    rng = np.random.default_rng(fmt * 100 + hd + rot + n_new)
+    starts = [0, 37, 1000]
+    n_valid = [n_new, 5 if n_new == 21 else n_new - 77, n_new]
     pages = [(s + n_new + pt - 1) // pt for s in starts]
     g = oracle.geometry(fmt, n_q, n_kv, hd, pt, sum(pages) + 1)
     table = make_tables(rng, pages, g.n_pages)

@@ -39,6 +39,7 @@ struct RopeArgs {
   void* q_out;        // same shape, of q_out_dtype
   int32_t q_out_dtype;
   float* k_out;       // [n_seqs][n_new][H][D] f32 or null: the rotated K rows, for callers that want them
+  int32_t per_xcd;    // AppendRows: tokens per XCD and sequence (a multiple of the page), or 0: tokens in order
 };
 
 __device__ __forceinline__ void Store4(void* dst, size_t i, int dtype, float4 v) {
@@ -76,7 +77,16 @@ __global__ __launch_bounds__(64 * kRopeWaves) void AppendRows(const RopeArgs a) 
   const int H = g.n_kv, PT = g.pt, D = g.hd, NQ = a.q_src != nullptr ? g.n_q : 0;
   const int rows_per_token = 2 * H + NQ;
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
-  const int i = int(blockIdx.x % a.n_new), s = int(blockIdx.x / a.n_new);
+  // Token i of sequence s. Workgroup b of a dispatch runs on XCD b % 8, and V's codes are single bytes of the
+  // transposed page: with a long chunk's tokens dealt to the workgroups in order, every line of a page would be put
+  // together from bytes in eight L2 caches, each of which writes its part back on its own. a.per_xcd > 0: workgroups
+  // b, b + 8, ... take per_xcd consecutive tokens (whole pages), so a page's bytes meet in one L2.
+  int i = int(blockIdx.x % a.n_new), s = int(blockIdx.x / a.n_new);
+  if (a.per_xcd > 0) {
+    const int span = 8 * a.per_xcd, r = int(blockIdx.x % span);
+    s = int(blockIdx.x / span), i = (r % 8) * a.per_xcd + r / 8;
+    if (i >= a.n_new) return;
+  }
   if (a.n_valid != nullptr && i >= a.n_valid[s]) return;  // padding row of a short chunk
   const int pos_raw = a.start_pos[s] + i;
   const int pos = min(max(pos_raw, 0), a.stride * PT - 1);
@@ -454,7 +464,13 @@ extern "C" int yahkv_append_rope(const yahkv_geometry* g, const yahkv_pools* poo
   const int64_t tokens = int64_t(n_seqs) * n_new;
   if (tokens > 0x7FFFFFFF) return YAHKV_ERR_SHAPE;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  LaunchRows<true>(g->format, src_dtype, dim3(static_cast<unsigned>(tokens)), st, a);
+  int64_t blocks = tokens;
+  if (n_new >= 8 * m.pt) {  // a long chunk: a page's tokens to one XCD (see AppendRows)
+    a.per_xcd = ((n_new + 7) / 8 + m.pt - 1) / m.pt * m.pt;
+    blocks = int64_t(n_seqs) * 8 * a.per_xcd;
+    if (blocks > 0x7FFFFFFF) return YAHKV_ERR_SHAPE;
+  }
+  LaunchRows<true>(g->format, src_dtype, dim3(static_cast<unsigned>(blocks)), st, a);
   return LaunchStatus();
 }
 
