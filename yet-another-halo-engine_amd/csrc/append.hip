@@ -40,6 +40,8 @@ struct RopeArgs {
   int32_t q_out_dtype;
   float* k_out;       // [n_seqs][n_new][H][D] f32 or null: the rotated K rows, for callers that want them
   int32_t per_xcd;    // AppendRows: tokens per XCD and sequence (a multiple of the page), or 0: tokens in order
+  int32_t skip_v;     // AppendRows: the V rows are left to another launch (AppendPages with skip_k)
+  int32_t skip_k;     // AppendPages: V only
 };
 
 __device__ __forceinline__ void Store4(void* dst, size_t i, int dtype, float4 v) {
@@ -75,7 +77,9 @@ __global__ __launch_bounds__(64 * kRopeWaves) void AppendRows(const RopeArgs a) 
 #pragma clang fp contract(off)
   const Geom g = a.g;
   const int H = g.n_kv, PT = g.pt, D = g.hd, NQ = a.q_src != nullptr ? g.n_q : 0;
-  const int rows_per_token = 2 * H + NQ;
+  // (with a.skip_v the token's rows are its K heads and its query heads: row numbers H .. 2 H - 1 are passed over)
+  const int rows_per_token = (a.skip_v ? H : 2 * H) + NQ;
+  auto row_of = [&](int r) -> int { return a.skip_v && r >= H ? r + H : r; };
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   // Token i of sequence s. Workgroup b of a dispatch runs on XCD b % 8, and V's codes are single bytes of the
   // transposed page: with a long chunk's tokens dealt to the workgroups in order, every line of a page would be put
@@ -139,13 +143,13 @@ __global__ __launch_bounds__(64 * kRopeWaves) void AppendRows(const RopeArgs a) 
     for (int j = 0; j < kRowsInFlight; ++j) {
       const void* src;
       size_t off;
-      source(min(first_row + kRopeWaves * j, rows_per_token - 1), &src, &off);
+      source(row_of(min(first_row + kRopeWaves * j, rows_per_token - 1)), &src, &off);
       raw[j] = LoadRaw4(src, off + (has ? d0 : 0), SRC);
     }
 #pragma unroll
     for (int j = 0; j < kRowsInFlight; ++j) {
-      const int row = first_row + kRopeWaves * j;
-      if (row >= rows_per_token) break;
+      if (first_row + kRopeWaves * j >= rows_per_token) break;
+      const int row = row_of(first_row + kRopeWaves * j);
       const bool is_v = row >= H && row < 2 * H, is_q = row >= 2 * H;
       float4 v = Widen4(raw[j], SRC);
       if (!has) v = float4{0.0f, 0.0f, 0.0f, 0.0f};
@@ -232,7 +236,8 @@ __global__ __launch_bounds__(64 * kPageWaves) void AppendPages(const RopeArgs a)
       rk[j] = rv[j] = uint4{0u, 0u, 0u, 0u};  // reads as 0.0 in every source type
       if (t >= t_lo && t < t_hi && has) {
         const size_t row = ((size_t(s) * a.n_new + token_at(pi * PT + t)) * H + h) * D;
-        rk[j] = LoadRaw4(a.k_src, row + d0, SRC), rv[j] = LoadRaw4(a.v_src, row + d0, SRC);
+        rv[j] = LoadRaw4(a.v_src, row + d0, SRC);
+        if (!a.skip_k) rk[j] = LoadRaw4(a.k_src, row + d0, SRC);
       }
     }
   };
@@ -297,7 +302,7 @@ __global__ __launch_bounds__(64 * kPageWaves) void AppendPages(const RopeArgs a)
   const size_t ph = size_t(page) * H + h;
   const int n_t = t_hi - t_lo, tid = threadIdx.x, NT = 64 * kPageWaves;
   const int lg_pt = __builtin_ctz(static_cast<unsigned>(PT));  // pages are 16, 32 or 64 tokens
-  {  // K codes: per block the tokens' pieces are contiguous
+  if (!a.skip_k) {  // K codes: per block the tokens' pieces are contiguous
     uint8_t* dst = a.pools.kq + ph * (size_t(NB) * PT * KB);
     if (n_t == PT) {  // a whole page (most of a chunk's): the region as it lies, no division by a run-time value
       for (int u = tid; u < (NB * KB / 16) << lg_pt; u += NT)
@@ -310,7 +315,7 @@ __global__ __launch_bounds__(64 * kPageWaves) void AppendPages(const RopeArgs a)
       }
     }
   }
-  {  // K scales: [token][block], 8 bytes at a time
+  if (!a.skip_k) {  // K scales: [token][block], 8 bytes at a time
     uint8_t* dst = reinterpret_cast<uint8_t*>(a.pools.ks) + ph * (size_t(PT) * NB * 2);
     for (int u = tid; u < n_t * NB / 4; u += NT) {
       const int off = t_lo * NB * 2 + u * 8;
@@ -392,6 +397,21 @@ int CheckAppend(const yahkv_geometry* g, const yahkv_pools* pools, const int32_t
 
 namespace {
 // AppendRows for the pools' format and the source rows' type (the kernel is compiled for each pair)
+// AppendPages likewise: one workgroup per (page the chunk touches, kv head, sequence)
+void LaunchPages(int32_t format, int32_t src_dtype, int32_t n_seqs, int32_t n_new, hipStream_t st, const RopeArgs& a) {
+  const dim3 grid(static_cast<unsigned>((n_new + a.g.pt - 2) / a.g.pt + 1), static_cast<unsigned>(a.g.n_kv),
+                  static_cast<unsigned>(n_seqs));
+  const dim3 block(64 * kPageWaves);
+  if (format == YAHKV_Q8_0) {
+    if (src_dtype == YAHKV_F32) hipLaunchKernelGGL((AppendPages<8, YAHKV_F32>), grid, block, 0, st, a);
+    else if (src_dtype == YAHKV_F16) hipLaunchKernelGGL((AppendPages<8, YAHKV_F16>), grid, block, 0, st, a);
+    else hipLaunchKernelGGL((AppendPages<8, YAHKV_BF16>), grid, block, 0, st, a);
+  } else {
+    if (src_dtype == YAHKV_F32) hipLaunchKernelGGL((AppendPages<4, YAHKV_F32>), grid, block, 0, st, a);
+    else if (src_dtype == YAHKV_F16) hipLaunchKernelGGL((AppendPages<4, YAHKV_F16>), grid, block, 0, st, a);
+    else hipLaunchKernelGGL((AppendPages<4, YAHKV_BF16>), grid, block, 0, st, a);
+  }
+}
 template <bool ROPE>
 void LaunchRows(int32_t format, int32_t src_dtype, dim3 grid, hipStream_t st, const RopeArgs& a) {
   const dim3 block(64 * kRopeWaves);
@@ -420,20 +440,7 @@ extern "C" int yahkv_append(const yahkv_geometry* g, const yahkv_pools* pools, c
   a.src_dtype = src_dtype, a.rotary_dim = 8, a.theta = 1.0f;
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (n_new >= kPageAppendMin && n_seqs <= 65535) {  // a chunk: page by page (the grid's z extent is the batch)
-    const dim3 grid(static_cast<unsigned>((n_new + a.g.pt - 2) / a.g.pt + 1), static_cast<unsigned>(a.g.n_kv),
-                    static_cast<unsigned>(n_seqs));
-#define YAHKV_LAUNCH_PAGES(FF, SS) hipLaunchKernelGGL((AppendPages<FF, SS>), grid, dim3(64 * kPageWaves), 0, st, a)
-#define YAHKV_LAUNCH_PAGES_FMT(FF)                                   \
-  if (src_dtype == YAHKV_F32) YAHKV_LAUNCH_PAGES(FF, YAHKV_F32);     \
-  else if (src_dtype == YAHKV_F16) YAHKV_LAUNCH_PAGES(FF, YAHKV_F16); \
-  else YAHKV_LAUNCH_PAGES(FF, YAHKV_BF16)
-    if (g->format == YAHKV_Q8_0) {
-      YAHKV_LAUNCH_PAGES_FMT(8);
-    } else {
-      YAHKV_LAUNCH_PAGES_FMT(4);
-    }
-#undef YAHKV_LAUNCH_PAGES_FMT
-#undef YAHKV_LAUNCH_PAGES
+    LaunchPages(g->format, src_dtype, n_seqs, n_new, st, a);
     return LaunchStatus();
   }
   const dim3 grid(static_cast<unsigned>(n_seqs) * static_cast<unsigned>(n_new));
@@ -464,6 +471,15 @@ extern "C" int yahkv_append_rope(const yahkv_geometry* g, const yahkv_pools* poo
   const int64_t tokens = int64_t(n_seqs) * n_new;
   if (tokens > 0x7FFFFFFF) return YAHKV_ERR_SHAPE;
   hipStream_t st = static_cast<hipStream_t>(stream);
+  if (n_new >= kPageAppendMin && n_seqs <= 65535) {
+    // A chunk: V page by page, as the plain append takes it (whole lines from an image of the page, where the
+    // token's workgroup would store V's codes byte by byte into the transposed page), K and the query rows by token.
+    RopeArgs v = a;
+    v.skip_k = 1;
+    LaunchPages(g->format, src_dtype, n_seqs, n_new, st, v);
+    if (const int rc = LaunchStatus()) return rc;
+    a.skip_v = 1;
+  }
   int64_t blocks = tokens;
   if (n_new >= 8 * m.pt) {  // a long chunk: a page's tokens to one XCD (see AppendRows)
     a.per_xcd = ((n_new + 7) / 8 + m.pt - 1) / m.pt * m.pt;
