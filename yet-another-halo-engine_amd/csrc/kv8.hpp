@@ -121,12 +121,9 @@ __device__ __forceinline__ float4 WaveHadamard256(float4 x, int lane) {
   float v[4] = {a0 + a2, a1 + a3, a0 - a2, a1 - a3};
   auto stage = [&](auto kc) {
     constexpr int k = decltype(kc)::value;
-    const bool upper = (lane & k) != 0;
+    const float sign = (lane & k) != 0 ? -1.0f : 1.0f;  // upper' = partner - own, lower' = own + partner
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const float o = LaneXor<k>(v[e]);
-      v[e] = upper ? o - v[e] : v[e] + o;
-    }
+    for (int e = 0; e < 4; ++e) v[e] = __builtin_fmaf(v[e], sign, LaneXor<k>(v[e]));  // (+-1 * x is exact: one rounding, the sum's)
   };
   stage(std::integral_constant<int, 1>{}), stage(std::integral_constant<int, 2>{}), stage(std::integral_constant<int, 4>{});
   stage(std::integral_constant<int, 8>{}), stage(std::integral_constant<int, 16>{}), stage(std::integral_constant<int, 32>{});
