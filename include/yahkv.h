@@ -390,9 +390,9 @@ size_t yahkv_f16_pool_bytes(const yahkv_geometry* g);
 int yahkv_f16_append(const yahkv_geometry* g, const yahkv_f16_pools* pools, const int32_t* page_table,
                      int32_t page_table_stride, const int32_t* start_pos, const int32_t* n_valid, int32_t n_seqs,
                      int32_t n_new, const void* k_src, const void* v_src, int32_t src_dtype, void* stream);
-/* Decode attention over keys 0 .. seq_len[s] - 1 (arguments as yahkv_decode_attend): two dispatches, partials of
- * fixed stretches of every sequence, then their merge with the optional sigmoid gate. Of the options only n_chunks is
- * used. */
+/* Decode attention over keys 0 .. seq_len[s] - 1 (arguments as yahkv_decode_attend, q 16-byte aligned as there): two
+ * dispatches, partials of fixed stretches of every sequence, then their merge with the optional sigmoid gate. Of the
+ * options only n_chunks is used. */
 size_t yahkv_f16_decode_workspace_bytes(const yahkv_geometry* g, int32_t n_seqs, int32_t max_seq_len,
                                         const yahkv_decode_options* opt);
 int yahkv_f16_decode_attend(const yahkv_geometry* g, const yahkv_f16_pools* pools, const int32_t* page_table,
