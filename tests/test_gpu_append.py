@@ -139,19 +139,21 @@ def test_append_rejects_bad_arguments(yahkv, torch_gpu):
     assert rc == -1
 
 
-@pytest.mark.parametrize("fmt,pt", [(8, 64), (4, 16), (8, 32)])
-def test_chunk_positions_clamp_like_a_loop_over_the_tokens(yahkv, torch_gpu, fmt, pt):
+@pytest.mark.parametrize("fmt,pt,n_new", [(8, 64, 40), (4, 16, 40), (8, 32, 40), (8, 64, 6), (4, 32, 7)])
+def test_chunk_positions_clamp_like_a_loop_over_the_tokens(yahkv, torch_gpu, fmt, pt, n_new):
     """A chunk that runs past the table's last position, and one that starts before position 0: every token goes to
-    its clamped position, and where several clamp to the same slot the last one stays, as in the oracle's loop."""
+    its clamped position, and where several clamp to the same slot the last one stays, as in the oracle's loop (chunks
+    of 40 tokens go page by page, those of 6 or 7 token by token)."""
     torch = torch_gpu
-    rng = np.random.default_rng(fmt + pt)
-    n_kv, hd, stride, n_new = 2, 128, 3, 40
+    rng = np.random.default_rng(fmt + pt + n_new)
+    n_kv, hd, stride = 2, 128, 3
     g = oracle.geometry(fmt, n_kv, n_kv, hd, pt, 3 * stride + 1)
     table = make_tables(rng, [stride] * 3, g.n_pages)
     host = oracle.HostPools(g, fill=0x3C)
     dev = yahkv.DevicePools(yahkv.geometry(fmt, n_kv, n_kv, hd, pt, g.n_pages), fill=0x3C)
-    start = np.array([stride * pt - 25, -7, stride * pt + 100], np.int32)    # over the end, before 0, all past the end
-    valid = np.array([n_new, 33, 12], np.int32)
+    over = 25 if n_new == 40 else 3
+    start = np.array([stride * pt - over, -7 if n_new == 40 else -3, stride * pt + 100], np.int32)    # over the end, before 0, all past the end
+    valid = np.array([n_new, 33, 12] if n_new == 40 else [n_new, n_new - 1, 4], np.int32)
     K = to_bf16_f32(rng.standard_normal((3, n_new, n_kv, hd)))
     V = to_bf16_f32(rng.standard_normal((3, n_new, n_kv, hd)))
     oracle.append(host, table, start, valid, K, V)

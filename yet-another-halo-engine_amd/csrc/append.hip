@@ -91,9 +91,13 @@ __global__ __launch_bounds__(64 * kRopeWaves) void AppendRows(const RopeArgs a) 
     s = int(blockIdx.x / span), i = (r % 8) * a.per_xcd + r / 8;
     if (i >= a.n_new) return;
   }
-  if (a.n_valid != nullptr && i >= a.n_valid[s]) return;  // padding row of a short chunk
-  const int pos_raw = a.start_pos[s] + i;
-  const int pos = min(max(pos_raw, 0), a.stride * PT - 1);
+  const int nv = a.n_valid != nullptr ? min(a.n_valid[s], a.n_new) : a.n_new;
+  if (i >= nv) return;  // padding row of a short chunk
+  const int start = a.start_pos[s], pos_raw = start + i, last_pos = a.stride * PT - 1;
+  const int pos = min(max(pos_raw, 0), last_pos);
+  // Where several tokens of the call clamp to the table's first or last slot, the one a loop over the tokens would
+  // leave there writes it (AppendPages' token_at); the others only produce their query rows and rotated K rows.
+  const bool owns_slot = pos_raw >= last_pos ? i == nv - 1 : (pos_raw <= 0 ? i == min(nv - 1, -start) : true);
   const int page = ClampPage(a.table[int64_t(s) * a.stride + pos / PT], g.n_pages);
   const int t = pos % PT;
 
@@ -176,7 +180,7 @@ __global__ __launch_bounds__(64 * kRopeWaves) void AppendRows(const RopeArgs a) 
       const int h = is_v ? row - H : row, lb = lane % 8;
       uint16_t scale;
       const uint32_t codes = FMT == 8 ? QuantizeLanesQ8(v, &scale) : QuantizeLanesQ4(v, lb, &scale);
-      if (!has) continue;
+      if (!has || !owns_slot) continue;
       if (!is_v)
         StoreRowK<FMT>(a.pools, g, page, h, t, lane, codes, scale);
       else
