@@ -396,6 +396,48 @@ def test_chunks_that_start_inside_a_tile_and_end_in_its_page(yahkv, torch_gpu, b
         pos = pos + n
 
 
+@pytest.mark.parametrize("seed,bits", [(1, 8), (2, 8), (3, 4), (4, 4)])
+def test_random_appends_against_the_oracle(yahkv, torch_gpu, seed, bits):
+    """Sequences that grow by calls of random length (one token, a few, several tiles, across pages), some rows of a
+    call padding, f16 or bf16 or f32 rows: after every call all six buffers are the oracle's, byte for byte."""
+    torch = torch_gpu
+    rng = np.random.default_rng(1000 + seed)
+    n_q, H = 8, 2
+    S = int(rng.integers(3, 40))
+    pages_each = 4
+    g = yahkv.kv8_geometry(n_q, H, S * pages_each + 1, bits, bits)
+    dp, hp = yahkv.Kv8Pools(g, 0x17), kv8.HostPools(kv8.geometry(n_q, H, S * pages_each + 1, bits, bits), 0x17)
+    table = rng.permutation(S * pages_each + 1)[:S * pages_each].astype(np.int32).reshape(S, pages_each)
+    t_table = torch.from_numpy(table).cuda()
+    pos = np.zeros(S, np.int32)
+    cap = pages_each * 256
+    first = True
+    for call in range(9):
+        n_new = int(rng.choice([1, 1, 2, 5, 16, 33, 100, 257, 300]))
+        n = rng.integers(0 if not first else 1, n_new + 1, S).astype(np.int32)
+        n = np.minimum(n, cap - pos).astype(np.int32)
+        n[0] = min(n_new, cap - pos[0])
+        dt = [np.float16, "bf16", np.float32][call % 3]
+        K = (rng.standard_normal((S, n_new, H, 256)) + 0.3).astype(np.float32)
+        V = rng.standard_normal((S, n_new, H, 256)).astype(np.float32)
+        if dt == "bf16":
+            tk, tv = torch.from_numpy(K).cuda().to(torch.bfloat16), torch.from_numpy(V).cuda().to(torch.bfloat16)
+            K, V = tk.float().cpu().numpy(), tv.float().cpu().numpy()
+        else:
+            K, V = K.astype(dt), V.astype(dt)
+            tk, tv = torch.from_numpy(K).cuda(), torch.from_numpy(V).cuda()
+        if first:                                      # the channel means from each sequence's first rows
+            yahkv.kv8_kmean(dp, t_table, tk, torch.from_numpy(n).cuda())
+            for s in range(S):
+                hp.km[table[s, 0]] = kv8.kmean(K[s, :max(n[s], 1)].astype(np.float32).reshape(max(n[s], 1), -1))
+            first = False
+        yahkv.kv8_append(dp, t_table, torch.from_numpy(pos).cuda(), tk, tv, torch.from_numpy(n).cuda())
+        kv8.append(hp, table, pos.tolist(), n.tolist(), K.astype(np.float32).reshape(S, n_new, -1), V.astype(np.float32).reshape(S, n_new, -1))
+        torch.cuda.synchronize()
+        assert_pools_equal(dp, hp, f"seed {seed}, call {call}: {n_new} rows of {dt}")
+        pos = pos + n
+
+
 def test_refusals(yahkv, torch_gpu):
     torch = torch_gpu
     g = yahkv.kv8_geometry(24, 4, 2)
