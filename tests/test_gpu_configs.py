@@ -143,6 +143,18 @@ def test_config3_ragged_batch_of_64_at_full_size(yahkv, torch_gpu):
         assert rel_err(before[s_], closed_form(Kd[:n_], Vd[:n_], q[s_], scale)) < TOL, (s_, "one step earlier")
         assert np.abs(before[s_] - got[s_]).max() > 0
     assert int(lens[crossing]) % PT == 0 and pages[crossing] == int(lens[crossing]) // PT + 1   # the token's own page
+    # every other row of the batch: the step's attention against the closed form over that sequence's own blocks
+    worst = 0.0
+    for s_ in range(B):
+        if s_ in kept:
+            continue
+        n_ = int(lens[s_]) + 1
+        k, v = yahkv.gather_blocks(dev, t_table[s_], n_)
+        Kd = oracle.dequantize_q8_0(k.cpu().numpy().reshape(-1, 34)).reshape(n_, NKV, HD)
+        Vd = oracle.dequantize_q8_0(v.cpu().numpy().reshape(-1, 34)).reshape(n_, NKV, HD)
+        worst = max(worst, rel_err(got[s_], closed_form(Kd, Vd, q[s_], scale)))
+    print(f"config 3, the other {B - len(kept)} rows against the closed form: {worst:.2e}")
+    assert worst < TOL
 
 
 def outlier_scales(rng):
